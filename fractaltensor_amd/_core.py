@@ -1,0 +1,239 @@
+"""ctypes binding of libftkernels.so, the C ABI declared in include/ftk.h.
+
+This is the only place the package touches native code.  The library is
+required: importing this module without a built libftkernels.so raises, and
+no function here has a CPU or PyTorch fallback.
+"""
+from __future__ import annotations
+
+import ctypes
+import os
+from typing import Optional, Sequence, Tuple
+
+import torch
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, 'libftkernels.so')
+
+# every symbol include/ftk.h declares; checked at load time
+EXPORTS = (
+    'ftk_version', 'ftk_last_error', 'ftk_device_info_query',
+    'ftk_lstm_cell_f32', 'ftk_lstm_elementwise_f32',
+    'ftk_stacked_lstm_workspace_bytes', 'ftk_stacked_lstm_f32', 'ftk_dilated_lstm_f32',
+    'ftk_stacked_lstm_wavefront_f32',
+    'ftk_b2b_gemm_f16', 'ftk_flash_attn_f16', 'ftk_online_softmax_f32',
+)
+
+
+class FtkError(RuntimeError):
+    """A non-zero return from the C ABI; carries the code and ftk_last_error()."""
+
+    def __init__(self, code: int, message: str):
+        super().__init__(f'libftkernels error {code}: {message}')
+        self.code = code
+
+
+class DeviceInfo(ctypes.Structure):
+    _fields_ = [('compute_units', ctypes.c_int), ('lds_bytes_per_block', ctypes.c_int),
+                ('clock_khz', ctypes.c_int), ('wavefront_size', ctypes.c_int),
+                ('persistent_slots', ctypes.c_int), ('arch', ctypes.c_char * 32)]
+
+
+def _load() -> ctypes.CDLL:
+    if not os.path.exists(LIB_PATH):
+        raise ImportError(
+            f'{LIB_PATH} is missing: build it with `make -C fractaltensor_amd/csrc` '
+            '(or __graft_entry__.build()); there is no fallback path')
+    lib = ctypes.CDLL(LIB_PATH)
+    for name in EXPORTS:
+        if not hasattr(lib, name):
+            raise ImportError(f'{LIB_PATH} does not export {name}')
+    lib.ftk_version.restype = ctypes.c_int
+    lib.ftk_last_error.restype = ctypes.c_char_p
+    lib.ftk_stacked_lstm_workspace_bytes.restype = ctypes.c_size_t
+    lib.ftk_stacked_lstm_workspace_bytes.argtypes = [ctypes.c_int] * 4
+    for name in EXPORTS:
+        if name not in ('ftk_last_error', 'ftk_stacked_lstm_workspace_bytes'):
+            getattr(lib, name).restype = ctypes.c_int
+    return lib
+
+
+lib = _load()
+
+
+def _check(rc: int) -> None:
+    if rc != 0:
+        raise FtkError(rc, lib.ftk_last_error().decode('utf-8', 'replace'))
+
+
+def _ptr(t: Optional[torch.Tensor]):
+    return ctypes.c_void_p(0 if t is None else t.data_ptr())
+
+
+def _stream():
+    return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def _req(t: torch.Tensor, dtype, name: str) -> torch.Tensor:
+    if not isinstance(t, torch.Tensor):
+        raise TypeError(f'{name} must be a torch.Tensor')
+    if not t.is_cuda:
+        raise RuntimeError(f'{name} must live on the GPU (got {t.device}); there is no CPU path')
+    if t.dtype != dtype:
+        raise TypeError(f'{name} must be {dtype}, got {t.dtype}')
+    if not t.is_contiguous():
+        raise ValueError(f'{name} must be contiguous')
+    return t
+
+
+def version() -> int:
+    return lib.ftk_version()
+
+
+def device_info() -> DeviceInfo:
+    info = DeviceInfo()
+    _check(lib.ftk_device_info_query(ctypes.byref(info)))
+    return info
+
+
+def lstm_cell(x, h_prev, c_prev, WU, bias=None) -> Tuple[torch.Tensor, torch.Tensor]:
+    """Fused cell: x [B,I], h_prev/c_prev [B,H] or None, WU [(I+H),4H], bias [4H] or None."""
+    f32 = torch.float32
+    _req(x, f32, 'x'); _req(WU, f32, 'WU')
+    B, I = x.shape
+    H = WU.shape[1] // 4
+    if WU.shape != (I + H, 4 * H):
+        raise ValueError(f'WU must be [(I+H), 4H] = [{I + H}, {4 * H}], got {tuple(WU.shape)}')
+    for t, n in ((h_prev, 'h_prev'), (c_prev, 'c_prev')):
+        if t is not None and _req(t, f32, n).shape != (B, H):
+            raise ValueError(f'{n} must be [{B}, {H}]')
+    if bias is not None and _req(bias, f32, 'bias').numel() != 4 * H:
+        raise ValueError('bias must have 4H elements')
+    h = torch.empty((B, H), dtype=f32, device=x.device)
+    c = torch.empty((B, H), dtype=f32, device=x.device)
+    _check(lib.ftk_lstm_cell_f32(_ptr(x), _ptr(h_prev), _ptr(c_prev), _ptr(WU), _ptr(bias), _ptr(h), _ptr(c),
+                                 ctypes.c_int(B), ctypes.c_int(I), ctypes.c_int(H), _stream()))
+    return h, c
+
+
+def lstm_elementwise(gates, bias, c_prev) -> Tuple[torch.Tensor, torch.Tensor]:
+    """State update on pre-activation gates [B,4H] (the unfused baseline's second kernel)."""
+    f32 = torch.float32
+    _req(gates, f32, 'gates')
+    B, H4 = gates.shape
+    H = H4 // 4
+    if bias is not None:
+        _req(bias, f32, 'bias')
+    if c_prev is not None:
+        _req(c_prev, f32, 'c_prev')
+    h = torch.empty((B, H), dtype=f32, device=gates.device)
+    c = torch.empty((B, H), dtype=f32, device=gates.device)
+    _check(lib.ftk_lstm_elementwise_f32(_ptr(gates), _ptr(bias), _ptr(c_prev), _ptr(h), _ptr(c),
+                                        ctypes.c_int(B), ctypes.c_int(H), _stream()))
+    return h, c
+
+
+def stacked_lstm_workspace_bytes(L: int, T: int, B: int, H: int) -> int:
+    return int(lib.ftk_stacked_lstm_workspace_bytes(L, T, B, H))
+
+
+def stacked_lstm(xs, WU, bias=None, dilations: Optional[Sequence[int]] = None, schedule: str = 'auto',
+                 out: Optional[Tuple[torch.Tensor, torch.Tensor]] = None,
+                 workspace: Optional[torch.Tensor] = None) -> Tuple[torch.Tensor, torch.Tensor]:
+    """xs [T,B,H], WU [L,2H,4H], bias [L,4H] or None -> hsss, csss [L,T,B,H].
+
+    schedule: 'auto' (persistent kernel when the shape allows, else per-stage
+    launches) or 'wavefront' (always per-stage launches).
+    """
+    f32 = torch.float32
+    _req(xs, f32, 'xs'); _req(WU, f32, 'WU')
+    T, B, H = xs.shape
+    L = WU.shape[0]
+    if WU.shape != (L, 2 * H, 4 * H):
+        raise ValueError(f'WU must be [L, 2H, 4H] = [{L}, {2 * H}, {4 * H}], got {tuple(WU.shape)}')
+    if bias is not None and _req(bias, f32, 'bias').shape != (L, 4 * H):
+        raise ValueError('bias must be [L, 4H]')
+    if out is None:
+        hsss = torch.empty((L, T, B, H), dtype=f32, device=xs.device)
+        csss = torch.empty((L, T, B, H), dtype=f32, device=xs.device)
+    else:
+        hsss, csss = out
+        _req(hsss, f32, 'hsss'); _req(csss, f32, 'csss')
+    dil = None
+    if dilations is not None:
+        if len(dilations) != L:
+            raise ValueError('dilations must have one entry per layer')
+        dil = (ctypes.c_int * L)(*[int(d) for d in dilations])
+    ci = ctypes.c_int
+    if schedule == 'wavefront':
+        _check(lib.ftk_stacked_lstm_wavefront_f32(_ptr(xs), _ptr(WU), _ptr(bias), dil, _ptr(hsss), _ptr(csss),
+                                                  ci(L), ci(T), ci(B), ci(H), _stream()))
+        return hsss, csss
+    if schedule != 'auto':
+        raise ValueError("schedule must be 'auto' or 'wavefront'")
+    need = stacked_lstm_workspace_bytes(L, T, B, H)
+    if workspace is None:
+        workspace = torch.empty(need, dtype=torch.uint8, device=xs.device)
+    ws_bytes = ctypes.c_size_t(workspace.numel() * workspace.element_size())
+    if dil is None:
+        _check(lib.ftk_stacked_lstm_f32(_ptr(xs), _ptr(WU), _ptr(bias), _ptr(hsss), _ptr(csss),
+                                        ci(L), ci(T), ci(B), ci(H), _ptr(workspace), ws_bytes, _stream()))
+    else:
+        _check(lib.ftk_dilated_lstm_f32(_ptr(xs), _ptr(WU), _ptr(bias), dil, _ptr(hsss), _ptr(csss),
+                                        ci(L), ci(T), ci(B), ci(H), _ptr(workspace), ws_bytes, _stream()))
+    return hsss, csss
+
+
+def persistent_status(workspace: torch.Tensor) -> int:
+    """Error word a persistent stacked-LSTM launch left in its workspace (synchronises).
+
+    0 = every bounded wait completed; 1 = a wait ran out of polls and the launch drained early.
+    """
+    torch.cuda.synchronize()
+    return int(workspace[:4].view(torch.int32).item())
+
+
+def b2b_gemm(A, B_nk, C_pn, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """D = (A @ B) @ C.  A [G,M,K]; B_nk [G,N,K] (B stored column-major); C_pn [G,P,N]; D [G,M,P]; fp16."""
+    f16 = torch.float16
+    _req(A, f16, 'A'); _req(B_nk, f16, 'B_nk'); _req(C_pn, f16, 'C_pn')
+    squeeze = A.dim() == 2
+    if squeeze:
+        A, B_nk, C_pn = A[None], B_nk[None], C_pn[None]
+    G, M, K = A.shape
+    N = B_nk.shape[1]
+    P = C_pn.shape[1]
+    if B_nk.shape != (G, N, K) or C_pn.shape != (G, P, N):
+        raise ValueError(f'shape mismatch: A {tuple(A.shape)}, B_nk {tuple(B_nk.shape)}, C_pn {tuple(C_pn.shape)}')
+    D = out if out is not None else torch.empty((G, M, P), dtype=f16, device=A.device)
+    _req(D, f16, 'D')
+    ci = ctypes.c_int
+    _check(lib.ftk_b2b_gemm_f16(_ptr(A), _ptr(B_nk), _ptr(C_pn), _ptr(D), ci(G), ci(M), ci(N), ci(K), ci(P), _stream()))
+    return D[0] if squeeze and out is None else D
+
+
+def flash_attention(Q, K, V, scale: Optional[float] = None, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """O = softmax(Q K^T scale) V.  Q [B,Hd,Sq,D], K/V [B,Hd,Skv,D], fp16, non-causal."""
+    f16 = torch.float16
+    _req(Q, f16, 'Q'); _req(K, f16, 'K'); _req(V, f16, 'V')
+    B, Hd, Sq, D = Q.shape
+    Skv = K.shape[2]
+    if K.shape != (B, Hd, Skv, D) or V.shape != (B, Hd, Skv, D):
+        raise ValueError(f'shape mismatch: Q {tuple(Q.shape)}, K {tuple(K.shape)}, V {tuple(V.shape)}')
+    if scale is None:
+        scale = D ** -0.5
+    O = out if out is not None else torch.empty_like(Q)
+    _req(O, f16, 'O')
+    ci = ctypes.c_int
+    _check(lib.ftk_flash_attn_f16(_ptr(Q), _ptr(K), _ptr(V), _ptr(O), ci(B), ci(Hd), ci(Sq), ci(Skv), ci(D),
+                                  ctypes.c_float(scale), _stream()))
+    return O
+
+
+def online_softmax(x) -> torch.Tensor:
+    """Row softmax of x [rows, cols], fp32."""
+    _req(x, torch.float32, 'x')
+    rows, cols = x.shape
+    y = torch.empty_like(x)
+    _check(lib.ftk_online_softmax_f32(_ptr(x), _ptr(y), ctypes.c_int(rows), ctypes.c_int(cols), _stream()))
+    return y

@@ -1,0 +1,302 @@
+// Non-causal flash attention for gfx950: fp16 Q/K/V/O, fp32 accumulation on
+// v_mfma_f32_32x32x16_f16, online softmax (running max and sum) in registers.
+//
+// Both contractions are computed transposed so that a lane owns one query row:
+//   S^T[key, q] = sum_d Ks[key][d] * Q[q][d]     MFMA A-operand = K rows (LDS),
+//                                                B-operand = Q row fragments (registers)
+//   O^T[d, q]  += sum_key Vt[d][key] * P[q][key]  A-operand = V^T rows (LDS),
+//                                                B-operand = exp'd scores, fp16 (registers)
+// The 32x32 accumulator of lane (q = lane%32, half = lane/32) holds, for that
+// one query, keys 8g + 4*half + r (g = reg/4, r = reg%4) of a 32-key subtile.
+// Row max / row sum are therefore a reduction over the lane's own registers
+// plus one exchange with lane^32; the rescale factor of O^T is lane-local; and
+// the exp'd scores already are a valid MFMA B-operand if the PV product
+// contracts keys in the order the lane holds them (step s of a subtile takes
+// keys {16s + 4*half + r} U {16s + 8 + 4*half + r}), which only changes which
+// two 8-byte pieces of a V^T row the A-operand reads.  P never touches LDS.
+//
+// A workgroup is 4 waves; each wave owns 32*QT query rows, the workgroup
+// streams K/V in 64-key tiles: K as stored ([key][d], padded rows), V
+// transposed on the way into LDS ([d][key]) by 4x4 register transposes.  Tiles
+// are double buffered with register prefetch of the next tile.
+#include <algorithm>
+#include <type_traits>
+
+#include "ftk_common.h"
+
+namespace ftk {
+
+// Compile-time loop: the body sees its index as a constant expression, so
+// register arrays indexed by it are promoted to registers even when the body
+// sits under a runtime condition.
+template <int N, typename F>
+__device__ __forceinline__ void static_for(F&& f) {
+  if constexpr (N > 0) {
+    static_for<N - 1>(f);
+    f(std::integral_constant<int, N - 1>{});
+  }
+}
+
+constexpr int FA_KT = 64;          // keys per tile
+constexpr int FA_VLD = FA_KT + 4;  // padded V^T row (halfs)
+
+template <int D, int QT>
+__global__ __launch_bounds__(256) void flash_attn_kernel(const _Float16* __restrict__ Q,
+                                                         const _Float16* __restrict__ K,
+                                                         const _Float16* __restrict__ V,
+                                                         _Float16* __restrict__ O, int Sq, int Skv,
+                                                         float scale_log2e) {
+  constexpr int KLD = D + 8;   // padded K row (halfs)
+  constexpr int DS = D / 16;   // k steps of S^T
+  constexpr int DT = D / 32;   // d tiles of O^T
+  constexpr int KSZ = FA_KT * KLD;
+  constexpr int VSZ = D * FA_VLD;
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+  _Float16* Ks = reinterpret_cast<_Float16*>(smem);  // [2][64][KLD]
+  _Float16* Vt = Ks + 2 * KSZ;                       // [2][D][VLD]
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = tid >> 6;
+  const int j = lane & 31;
+  const int hh = lane >> 5;
+  const int bh = blockIdx.y;
+  const int q_base = blockIdx.x * (128 * QT) + wave * (32 * QT);
+
+  const _Float16* Qg = Q + (size_t)bh * Sq * D;
+  const _Float16* Kg = K + (size_t)bh * Skv * D;
+  const _Float16* Vg = V + (size_t)bh * Skv * D;
+  _Float16* Og = O + (size_t)bh * Sq * D;
+
+  // ---- Q row fragments, resident for the whole kernel
+  v8h qf[QT][DS];
+#pragma unroll
+  for (int qt = 0; qt < QT; ++qt) {
+    const int row = min(q_base + 32 * qt + j, Sq - 1);
+#pragma unroll
+    for (int s = 0; s < DS; ++s) {
+      const uint4 v = *reinterpret_cast<const uint4*>(Qg + (size_t)row * D + 16 * s + 8 * hh);
+      qf[qt][s] = *reinterpret_cast<const v8h*>(&v);
+    }
+  }
+
+  v16f oacc[QT][DT];
+  float m_run[QT], l_run[QT];
+#pragma unroll
+  for (int qt = 0; qt < QT; ++qt) {
+    m_run[qt] = -INFINITY;
+    l_run[qt] = 0.0f;
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) oacc[qt][dt][r] = 0.0f;
+  }
+
+  // ---- staging assignments
+  constexpr int KN = D / 32;  // 16-byte K loads per thread per tile
+  constexpr int VN = D / 64;  // 4x4 V blocks per thread per tile
+  static_assert(D % 64 == 0, "head dim must be a multiple of 64");
+  v4u kreg[KN];
+  v2u vreg[VN][4];
+
+  auto load_tile = [&](int kt) __attribute__((always_inline)) {
+    const int key0 = kt * FA_KT;
+    static_for<KN>([&](auto nc) __attribute__((always_inline)) {
+      constexpr int n = decltype(nc)::value;
+      const int idx = tid + 256 * n;
+      const int key = min(key0 + idx / (D / 8), Skv - 1);
+      const int c8 = idx % (D / 8);
+      kreg[n] = *reinterpret_cast<const v4u*>(Kg + (size_t)key * D + 8 * c8);
+    });
+    static_for<VN * 4>([&](auto nc) __attribute__((always_inline)) {
+      constexpr int n = decltype(nc)::value / 4;
+      constexpr int nn = decltype(nc)::value % 4;
+      const int u = tid + 256 * n;
+      const int dg = u % (D / 4);
+      const int kq = u / (D / 4);
+      const int key = min(key0 + 4 * kq + nn, Skv - 1);
+      vreg[n][nn] = *reinterpret_cast<const v2u*>(Vg + (size_t)key * D + 4 * dg);
+    });
+  };
+  auto store_tile = [&](int buf) __attribute__((always_inline)) {
+    _Float16* ks = Ks + buf * KSZ;
+    _Float16* vt = Vt + buf * VSZ;
+    static_for<KN>([&](auto nc) __attribute__((always_inline)) {
+      constexpr int n = decltype(nc)::value;
+      const int idx = tid + 256 * n;
+      const int key = idx / (D / 8);
+      const int c8 = idx % (D / 8);
+      *reinterpret_cast<v4u*>(ks + key * KLD + 8 * c8) = kreg[n];
+    });
+    static_for<VN>([&](auto nc) __attribute__((always_inline)) {
+      constexpr int n = decltype(nc)::value;
+      const int u = tid + 256 * n;
+      const int dg = u % (D / 4);
+      const int kq = u / (D / 4);
+      const v2u r0 = vreg[n][0], r1 = vreg[n][1], r2 = vreg[n][2], r3 = vreg[n][3];
+      // 4x4 transpose of halfs: row e of the result = element e of keys 0..3
+      v2u c0, c1, c2, c3;
+      c0.x = __builtin_amdgcn_perm(r1.x, r0.x, 0x05040100u);
+      c0.y = __builtin_amdgcn_perm(r3.x, r2.x, 0x05040100u);
+      c1.x = __builtin_amdgcn_perm(r1.x, r0.x, 0x07060302u);
+      c1.y = __builtin_amdgcn_perm(r3.x, r2.x, 0x07060302u);
+      c2.x = __builtin_amdgcn_perm(r1.y, r0.y, 0x05040100u);
+      c2.y = __builtin_amdgcn_perm(r3.y, r2.y, 0x05040100u);
+      c3.x = __builtin_amdgcn_perm(r1.y, r0.y, 0x07060302u);
+      c3.y = __builtin_amdgcn_perm(r3.y, r2.y, 0x07060302u);
+      _Float16* dst = vt + (4 * dg) * FA_VLD + 4 * kq;
+      *reinterpret_cast<v2u*>(dst) = c0;
+      *reinterpret_cast<v2u*>(dst + FA_VLD) = c1;
+      *reinterpret_cast<v2u*>(dst + 2 * FA_VLD) = c2;
+      *reinterpret_cast<v2u*>(dst + 3 * FA_VLD) = c3;
+    });
+  };
+
+  const int ntiles = (Skv + FA_KT - 1) / FA_KT;
+  load_tile(0);
+  store_tile(0);
+  __syncthreads();
+
+  for (int kt = 0; kt < ntiles; ++kt) {
+    const int buf = kt & 1;
+    if (kt + 1 < ntiles) load_tile(kt + 1);
+    const _Float16* ks = Ks + buf * KSZ;
+    const _Float16* vt = Vt + buf * VSZ;
+
+    // ---- S^T = K Q^T for two 32-key subtiles
+    v16f sacc[QT][2];
+#pragma unroll
+    for (int qt = 0; qt < QT; ++qt)
+#pragma unroll
+      for (int k2 = 0; k2 < 2; ++k2)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) sacc[qt][k2][r] = 0.0f;
+#pragma unroll
+    for (int k2 = 0; k2 < 2; ++k2) {
+      const _Float16* krow = ks + (32 * k2 + j) * KLD + 8 * hh;
+#pragma unroll
+      for (int s = 0; s < DS; ++s) {
+        const v8h kf = *reinterpret_cast<const v8h*>(krow + 16 * s);
+#pragma unroll
+        for (int qt = 0; qt < QT; ++qt)
+          sacc[qt][k2] = __builtin_amdgcn_mfma_f32_32x32x16_f16(kf, qf[qt][s], sacc[qt][k2], 0, 0, 0);
+      }
+    }
+
+    // ---- online softmax, one query row per lane (two lanes share a row)
+    const bool ragged = (kt + 1 == ntiles) && (Skv % FA_KT != 0);
+    v8h pf[QT][2][2];
+#pragma unroll
+    for (int qt = 0; qt < QT; ++qt) {
+      float mx = -INFINITY;
+#pragma unroll
+      for (int k2 = 0; k2 < 2; ++k2)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          float s2 = sacc[qt][k2][r] * scale_log2e;
+          if (ragged) {
+            const int key = kt * FA_KT + 32 * k2 + 8 * (r >> 2) + 4 * hh + (r & 3);
+            if (key >= Skv) s2 = -INFINITY;
+          }
+          sacc[qt][k2][r] = s2;
+          mx = fmaxf(mx, s2);
+        }
+      mx = fmaxf(mx, __shfl_xor(mx, 32));
+      const float m_new = fmaxf(m_run[qt], mx);
+      const float alpha = __builtin_amdgcn_exp2f(m_run[qt] - m_new);
+      m_run[qt] = m_new;
+      float psum = 0.0f;
+#pragma unroll
+      for (int k2 = 0; k2 < 2; ++k2)
+#pragma unroll
+        for (int s = 0; s < 2; ++s)
+#pragma unroll
+          for (int e = 0; e < 8; ++e) {
+            const float p = __builtin_amdgcn_exp2f(sacc[qt][k2][8 * s + e] - m_new);
+            psum += p;
+            pf[qt][k2][s][e] = (_Float16)p;
+          }
+      l_run[qt] = l_run[qt] * alpha + psum;  // this lane's half of the row sum
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) oacc[qt][dt][r] *= alpha;
+    }
+
+    // ---- O^T += V^T P^T
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) {
+      const _Float16* vrow = vt + (32 * dt + j) * FA_VLD + 4 * hh;
+#pragma unroll
+      for (int k2 = 0; k2 < 2; ++k2)
+#pragma unroll
+        for (int s = 0; s < 2; ++s) {
+          const v4h v0 = *reinterpret_cast<const v4h*>(vrow + 32 * k2 + 16 * s);
+          const v4h v1 = *reinterpret_cast<const v4h*>(vrow + 32 * k2 + 16 * s + 8);
+          const v8h vf = {v0[0], v0[1], v0[2], v0[3], v1[0], v1[1], v1[2], v1[3]};
+#pragma unroll
+          for (int qt = 0; qt < QT; ++qt)
+            oacc[qt][dt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(vf, pf[qt][k2][s], oacc[qt][dt], 0, 0, 0);
+        }
+    }
+
+    if (kt + 1 < ntiles) store_tile(buf ^ 1);
+    __syncthreads();
+  }
+
+  // ---- normalise and store: lane holds d = 32dt + 8g + 4*half + r of its row
+#pragma unroll
+  for (int qt = 0; qt < QT; ++qt) {
+    const float l = l_run[qt] + __shfl_xor(l_run[qt], 32);
+    const float inv = 1.0f / l;
+    const int row = q_base + 32 * qt + j;
+    if (row < Sq) {
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+          const v4h o = {(_Float16)(oacc[qt][dt][4 * g + 0] * inv), (_Float16)(oacc[qt][dt][4 * g + 1] * inv),
+                         (_Float16)(oacc[qt][dt][4 * g + 2] * inv), (_Float16)(oacc[qt][dt][4 * g + 3] * inv)};
+          *reinterpret_cast<v4h*>(Og + (size_t)row * D + 32 * dt + 8 * g + 4 * hh) = o;
+        }
+    }
+  }
+}
+
+template <int D, int QT>
+static int launch_fa(const void* Q, const void* K, const void* V, void* O, int BH, int Sq, int Skv, float scale,
+                     int lds_max, hipStream_t s) {
+  const size_t lds = (size_t)2 * (FA_KT * (D + 8) + D * FA_VLD) * 2;
+  if ((int)lds > lds_max) return fail(FTK_ERR_UNSUPPORTED_SHAPE, "ftk_flash_attn_f16: needs %zu bytes of LDS", lds);
+  const void* fn = (const void*)flash_attn_kernel<D, QT>;
+  FTK_HIP(hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+  dim3 grid((Sq + 128 * QT - 1) / (128 * QT), BH);
+  hipLaunchKernelGGL((flash_attn_kernel<D, QT>), grid, dim3(256), lds, s, (const _Float16*)Q, (const _Float16*)K,
+                     (const _Float16*)V, (_Float16*)O, Sq, Skv, scale * 1.4426950408889634f);
+  return check_launch("flash_attn_kernel");
+}
+
+}  // namespace ftk
+
+extern "C" int ftk_flash_attn_f16(const void* Q, const void* K, const void* V, void* O, int B, int Hd, int Sq, int Skv,
+                                  int D, float scale, ftk_stream_t stream) {
+  using namespace ftk;
+  if (!Q || !K || !V || !O) return fail(FTK_ERR_INVALID_ARGUMENT, "ftk_flash_attn_f16: Q, K, V, O must be non-NULL");
+  if (B <= 0 || Hd <= 0 || Sq <= 0 || Skv <= 0 || D <= 0)
+    return fail(FTK_ERR_INVALID_ARGUMENT, "ftk_flash_attn_f16: B, Hd, Sq, Skv, D must be positive");
+  if (D != 64 && D != 128) return fail(FTK_ERR_UNSUPPORTED_SHAPE, "ftk_flash_attn_f16: D=%d must be 64 or 128", D);
+  const long long bh = (long long)B * Hd;
+  if (bh > 65535) return fail(FTK_ERR_UNSUPPORTED_SHAPE, "ftk_flash_attn_f16: B*Hd=%lld above 65535", bh);
+  const DeviceProps* dp = nullptr;
+  int rc = device_props(&dp);
+  if (rc) return rc;
+  hipStream_t s = (hipStream_t)stream;
+  // 64 query rows per wave halve the LDS operand traffic per flop; use them once
+  // there are enough 256-row blocks to occupy the chip
+  const bool big = (long long)((Sq + 255) / 256) * bh >= dp->cus;
+  if (D == 128)
+    return big ? launch_fa<128, 2>(Q, K, V, O, (int)bh, Sq, Skv, scale, dp->lds_optin, s)
+               : launch_fa<128, 1>(Q, K, V, O, (int)bh, Sq, Skv, scale, dp->lds_optin, s);
+  return big ? launch_fa<64, 2>(Q, K, V, O, (int)bh, Sq, Skv, scale, dp->lds_optin, s)
+             : launch_fa<64, 1>(Q, K, V, O, (int)bh, Sq, Skv, scale, dp->lds_optin, s);
+}

@@ -1,0 +1,81 @@
+// Shared helpers for the gfx950 kernels behind include/ftk.h.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdarg.h>
+#include <stdint.h>
+#include <stdio.h>
+
+#include "../../include/ftk.h"
+
+namespace ftk {
+
+// ---- error reporting ------------------------------------------------------
+// One message buffer per host thread; entry points return a code and leave the
+// text here.  Kernel launch failures are turned into FTK_ERR_LAUNCH.
+char* last_error_buffer();
+constexpr int kErrLen = 512;
+
+inline int fail(int code, const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(last_error_buffer(), kErrLen, fmt, ap);
+  va_end(ap);
+  return code;
+}
+
+inline int check_launch(const char* what) {
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess)
+    return fail(FTK_ERR_LAUNCH, "%s: %s", what, hipGetErrorString(e));
+  return FTK_OK;
+}
+
+#define FTK_HIP(call)                                                        \
+  do {                                                                       \
+    hipError_t e_ = (call);                                                  \
+    if (e_ != hipSuccess)                                                    \
+      return ::ftk::fail(FTK_ERR_LAUNCH, "%s: %s", #call, hipGetErrorString(e_)); \
+  } while (0)
+
+// Device properties, queried once per device id.
+struct DeviceProps {
+  int cus = 0;
+  int lds_optin = 0;
+  int clock_khz = 0;
+  int wave = 0;
+  char arch[32] = {0};
+};
+int device_props(const DeviceProps** out);
+
+// ---- vector types for MFMA operands ----------------------------------------
+typedef float v4f __attribute__((ext_vector_type(4)));
+typedef float v16f __attribute__((ext_vector_type(16)));
+typedef unsigned v2u __attribute__((ext_vector_type(2)));
+typedef unsigned v4u __attribute__((ext_vector_type(4)));
+typedef _Float16 v4h __attribute__((ext_vector_type(4)));
+typedef _Float16 v8h __attribute__((ext_vector_type(8)));
+
+// ---- device math ------------------------------------------------------------
+// exp through the hardware base-2 exponential (about 1 ulp), reciprocal through
+// v_rcp_f32 (1 ulp).  sigmoid is accurate to a few 1e-7 relative everywhere.
+__device__ __forceinline__ float fast_exp(float x) {
+  return __builtin_amdgcn_exp2f(x * 1.4426950408889634f);
+}
+
+__device__ __forceinline__ float sigmoid_f(float x) {
+  return __builtin_amdgcn_rcpf(1.0f + fast_exp(-x));
+}
+
+// tanh(x) = 1 - 2/(1+e^{2x}) loses relative accuracy near 0 (the result is the
+// difference of two numbers close to 1), so small arguments use the odd Taylor
+// polynomial instead; the switch point keeps both branches below 2e-7 relative.
+__device__ __forceinline__ float tanh_f(float x) {
+  const float big = 1.0f - 2.0f * __builtin_amdgcn_rcpf(1.0f + fast_exp(2.0f * x));
+  const float x2 = x * x;
+  const float small =
+      x * (1.0f + x2 * (-0.33333333333f + x2 * (0.13333333333f + x2 * (-0.05396825397f + x2 * 0.02186948854f))));
+  return fabsf(x) < 0.25f ? small : big;
+}
+
+}  // namespace ftk

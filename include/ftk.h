@@ -1,0 +1,177 @@
+/*
+ * ftk.h -- C ABI of libftkernels.so: MI355X (gfx950) kernels for the
+ * FractalTensor hot path (fused LSTM cell scan, stacked / dilated LSTM,
+ * back-to-back fp16 GEMM, flash attention with online softmax).
+ *
+ * Conventions (all entry points):
+ *   - plain C, no C++/torch types; every pointer argument is a DEVICE pointer
+ *     owned by the caller unless its comment says "host";
+ *   - `stream` is a hipStream_t passed as void* (NULL = the default stream);
+ *     calls are stream-ordered and asynchronous, nothing synchronises;
+ *   - the return value is 0 on success and a negative FTK_ERR_* code on
+ *     failure; ftk_last_error() returns a thread-local description of the
+ *     last failure.  Nothing exits, aborts or throws;
+ *   - no entry point allocates device memory: kernels that need scratch take
+ *     a caller-provided workspace whose size the matching
+ *     *_workspace_bytes() function reports;
+ *   - matrices are dense row-major with the last index contiguous.
+ *
+ * The reference (microsoft/FractalTensor) has no C ABI of its own: its
+ * kernels are compile-time-shaped C++ functors called from gtest/benchmark
+ * binaries, and its Python frontend never reaches them.  Each declaration
+ * below names the reference functor or Python function it stands in for.
+ */
+#ifndef FTK_H_
+#define FTK_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define FTK_OK 0
+#define FTK_ERR_INVALID_ARGUMENT (-1) /* null pointer, non-positive size          */
+#define FTK_ERR_UNSUPPORTED_SHAPE (-2) /* shape outside what the kernels tile for */
+#define FTK_ERR_WORKSPACE (-3)        /* workspace missing or too small           */
+#define FTK_ERR_LAUNCH (-4)           /* HIP reported an error at launch          */
+#define FTK_ERR_DEVICE (-5)           /* device query failed / not a gfx950 part  */
+
+typedef void* ftk_stream_t;
+
+typedef struct ftk_device_info {
+  int compute_units;       /* multiProcessorCount                               */
+  int lds_bytes_per_block; /* sharedMemPerBlock opt-in maximum                  */
+  int clock_khz;           /* engine clock                                      */
+  int wavefront_size;      /* 64 on CDNA                                        */
+  int persistent_slots;    /* co-resident 256-thread, full-register workgroups  */
+  char arch[32];           /* gcnArchName, e.g. "gfx950:sramecc+:xnack-"        */
+} ftk_device_info;
+
+/* Library version, major*10000 + minor*100 + patch. */
+int ftk_version(void);
+
+/* Thread-local text for the most recent non-zero return on this thread. */
+const char* ftk_last_error(void);
+
+/* Properties of the current HIP device.
+ * Stands in for GPUContext / GetGPUComputeCapability
+ * (kaleido/core/device/gpu_context.h:11-64, kaleido/core/device/cuda_info.h). */
+int ftk_device_info_query(ftk_device_info* out);
+
+/* ---------------------------------------------------------------- LSTM -- */
+
+/*
+ * One batched LSTM cell, gate GEMM and state update fused in one launch:
+ *   g = [x, h_prev] @ WU + bias,  column blocks of g: i | f | o | c~
+ *   c = sigmoid(f)*c_prev + sigmoid(i)*tanh(c~);  h = sigmoid(o)*tanh(c)
+ * x [B,I], h_prev/c_prev [B,H] (both NULL = zero state), WU [(I+H),4H],
+ * bias [4H] or NULL, outputs h/c [B,H].  fp32.  Needs I%32==0, H%32==0.
+ * Replaces CuteLSTMCell::operator() (kaleido/core/device/kernels/lstm.h:253-348:
+ * KeCuteLSTMGate lstm_kernels.h:25-126 + KeLSTMElementWise lstm/inner.h:595-662)
+ * and the Python lstm_cell (examples/stacked_rnn/stacked_rnn.py:23-36).
+ */
+int ftk_lstm_cell_f32(const float* x, const float* h_prev, const float* c_prev,
+                      const float* WU, const float* bias, float* h, float* c,
+                      int B, int I, int H, ftk_stream_t stream);
+
+/*
+ * The state-update half alone, for the unfused baseline: gates [B,4H] already
+ * holds x@W + h@U (pre-activation, blocks i|f|o|c~); bias [4H] or NULL;
+ * c_prev [B,H] or NULL.  Replaces ElementwiseLstmAct
+ * (kaleido/core/device/kernels/elementwise.h:141-155) as used by
+ * benchmarks/rnn/fractaltensor/utils.h:439-495.
+ */
+int ftk_lstm_elementwise_f32(const float* gates, const float* bias,
+                             const float* c_prev, float* h, float* c, int B,
+                             int H, ftk_stream_t stream);
+
+/* Bytes of workspace ftk_stacked_lstm_f32 / ftk_dilated_lstm_f32 need. */
+size_t ftk_stacked_lstm_workspace_bytes(int L, int T, int B, int H);
+
+/*
+ * L stacked LSTM layers over T steps; layer l reads layer l-1's hidden
+ * sequence; zero initial state.  xs [T,B,H], WU [L,2H,4H], bias [L,4H] or
+ * NULL, outputs hsss/csss [L,T,B,H] (every layer's h and c at every step).
+ * One persistent launch walks the (layer,time) wavefront with each layer's
+ * weights held in registers; shapes it is not specialised for fall back to
+ * one fused-cell launch per wavefront diagonal.
+ * Replaces StackedLstmRegion1/2/3
+ * (kaleido/core/device/kernels/lstm/stacked_lstm/region1.h:11-43,
+ * region2.h:15-70, region3.h:18-140) and the Python stacked_lstm
+ * (examples/stacked_rnn/stacked_rnn.py:54-79).
+ */
+int ftk_stacked_lstm_f32(const float* xs, const float* WU, const float* bias,
+                         float* hsss, float* csss, int L, int T, int B, int H,
+                         void* workspace, size_t workspace_bytes,
+                         ftk_stream_t stream);
+
+/*
+ * Same with a per-layer dilation: layer l takes its state from step
+ * t - dilations[l] (zero state for t < dilations[l]).  `dilations` is a HOST
+ * array of L positive ints.  Replaces DilatedLstmRegion1/2
+ * (kaleido/core/device/kernels/lstm/dilated_lstm/region1.h:13-29,
+ * region2.h:12-82) and dilated_layer/model of
+ * examples/dilated_rnn/dilated_rnn.py:16-41.
+ */
+int ftk_dilated_lstm_f32(const float* xs, const float* WU, const float* bias,
+                         const int* dilations, float* hsss, float* csss, int L,
+                         int T, int B, int H, void* workspace,
+                         size_t workspace_bytes, ftk_stream_t stream);
+
+/*
+ * The same stack evaluated as one batched fused-cell launch per wavefront
+ * diagonal (no persistent kernel, no workspace); any H%32==0.  This is the
+ * launch structure of StackedLstmRegion3 (region3.h:50-103) and the fallback
+ * of the two entry points above.  dilations: host array or NULL (all 1).
+ */
+int ftk_stacked_lstm_wavefront_f32(const float* xs, const float* WU,
+                                   const float* bias, const int* dilations,
+                                   float* hsss, float* csss, int L, int T,
+                                   int B, int H, ftk_stream_t stream);
+
+/* ------------------------------------------------------------ B2B GEMM -- */
+
+/*
+ * G independent problems D = (A @ B) @ C, fp16 storage, fp32 accumulation,
+ * intermediate A@B rounded to fp16 in registers between the two products.
+ * A [G,M,K] row-major; B stored [G,N,K] (= K x N column-major); C stored
+ * [G,P,N] (= N x P column-major); D [G,M,P] row-major -- the layouts of
+ * kaleido/core/operators/tests/b2b_gemm_test_utils.h:3-9.
+ * Needs K%32==0, N%32==0, P%32==0, K<=256, P<=256.
+ * Replaces B2BGemm::operator() (kaleido/core/device/kernels/gemm.h:235-269,
+ * KeBack2BackGemm cutlass_wmma.h:441-540); the reference has no batch
+ * dimension, G maps to independent workgroups.
+ */
+int ftk_b2b_gemm_f16(const void* A, const void* B, const void* C, void* D,
+                     int G, int M, int N, int K, int P, ftk_stream_t stream);
+
+/* ------------------------------------------------------ flash attention -- */
+
+/*
+ * O = softmax(Q K^T * scale) V per (batch, head), non-causal, fp16 storage,
+ * fp32 accumulation, online softmax (running max / sum) in registers.
+ * Q,O [B,Hd,Sq,D]; K,V [B,Hd,Skv,D].  Needs D==128 or D==64, Sq%64==0... see
+ * ftk_last_error() for the exact constraint that failed.
+ * Replaces the map/reduce program flash_attention
+ * (examples/flash_attention/flash_attention.py:14-91); the reference has no
+ * device kernel for it.
+ */
+int ftk_flash_attn_f16(const void* Q, const void* K, const void* V, void* O,
+                       int B, int Hd, int Sq, int Skv, int D, float scale,
+                       ftk_stream_t stream);
+
+/*
+ * Row softmax through an online (max, denominator) scan, fp32, [rows, cols].
+ * Replaces OnlineNormalizedSoftmaxOp
+ * (kaleido/core/operators/online_softmax_op.cu:14-36,
+ * KeOnlineNormalizedSoftMax kaleido/core/device/kernels/online_softmax.h:176-183).
+ */
+int ftk_online_softmax_f32(const float* x, float* y, int rows, int cols,
+                           ftk_stream_t stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* FTK_H_ */

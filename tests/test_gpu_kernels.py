@@ -1,0 +1,305 @@
+"""Parity of the HIP kernels (through the C ABI) against the CPU oracle.
+
+Tolerances: fp32 LSTM max relative error <= 1e-4; fp16 GEMM / attention <= 1e-2
+against an fp32/fp64-accumulated reference (the oracle).  "Relative" is the
+maximum absolute difference over the maximum absolute reference value; LSTM
+tests additionally bound the element-wise relative error with a 1e-3 floor.
+"""
+import numpy as np
+import pytest
+import torch
+
+from oracle import c_oracle
+from oracle import kaleido_oracle as ko
+
+pytestmark = pytest.mark.gpu
+
+LSTM_TOL = 1e-4
+F16_TOL = 1e-2
+
+
+@pytest.fixture(scope='module')
+def core():
+    import fractaltensor_amd._core as c
+    return c
+
+
+def dev(a, dtype=None):
+    t = torch.from_numpy(np.ascontiguousarray(a))
+    if dtype is not None:
+        t = t.to(dtype)
+    return t.cuda()
+
+
+def lstm_inputs(seed, L, T, B, H, scale, bias=True):
+    rng = np.random.default_rng(seed)
+    xs = rng.standard_normal((T, B, H)).astype(np.float32)
+    WU = rng.uniform(-scale, scale, (L, 2 * H, 4 * H)).astype(np.float32)
+    bs = rng.uniform(-scale, scale, (L, 4 * H)).astype(np.float32) if bias else None
+    return xs, WU, bs
+
+
+def assert_lstm_close(got, ref, what):
+    got = got.detach().cpu().numpy()
+    e1 = ko.max_rel_err(got, ref)
+    e2 = ko.max_elem_rel_err(got, ref, floor=1e-3)
+    assert e1 <= LSTM_TOL, f'{what}: max rel err {e1:.3e}'
+    assert e2 <= 10 * LSTM_TOL, f'{what}: element-wise rel err (floor 1e-3) {e2:.3e}'
+
+
+# ------------------------------------------------------------------ LSTM cell
+
+@pytest.mark.parametrize('B,I,H,prev,bias', [
+    (64, 256, 256, True, False),    # config 1 per-step shape
+    (64, 256, 256, False, True),
+    (50, 64, 128, True, True),      # ragged batch, I != H
+    (1, 32, 32, True, True),        # one sample, smallest tile
+    (256, 256, 256, True, True),    # config 4 per-cell shape
+])
+def test_lstm_cell(core, B, I, H, prev, bias):
+    rng = np.random.default_rng(7)
+    x = rng.standard_normal((B, I)).astype(np.float32)
+    hp = rng.uniform(-1, 1, (B, H)).astype(np.float32) if prev else None
+    cp = rng.standard_normal((B, H)).astype(np.float32) if prev else None
+    WU = rng.uniform(-0.1, 0.1, (I + H, 4 * H)).astype(np.float32)
+    b = rng.uniform(-0.5, 0.5, 4 * H).astype(np.float32) if bias else None
+    h, c = core.lstm_cell(dev(x), None if hp is None else dev(hp), None if cp is None else dev(cp), dev(WU),
+                          None if b is None else dev(b))
+    zero = np.zeros((B, H))
+    hr, cr = ko.lstm_cell(x, zero if hp is None else hp, zero if cp is None else cp, WU, b)
+    assert_lstm_close(h, hr, 'h'); assert_lstm_close(c, cr, 'c')
+
+
+def test_lstm_cell_closed_forms(core):
+    """Zero weights: c = 0.5 c_prev, h = 0.5 tanh(c); saturated forget gate carries c."""
+    B, H = 32, 64
+    rng = np.random.default_rng(3)
+    x = dev(rng.standard_normal((B, H)).astype(np.float32))
+    hp = dev(rng.standard_normal((B, H)).astype(np.float32))
+    cp_np = rng.standard_normal((B, H)).astype(np.float32)
+    WU = torch.zeros((2 * H, 4 * H), device='cuda')
+    h, c = core.lstm_cell(x, hp, dev(cp_np), WU)
+    np.testing.assert_allclose(c.cpu().numpy(), 0.5 * cp_np, rtol=1e-6, atol=1e-7)
+    np.testing.assert_allclose(h.cpu().numpy(), 0.5 * np.tanh(0.5 * cp_np), rtol=2e-6, atol=1e-7)
+    bias = np.zeros(4 * H, np.float32); bias[H:2 * H] = 50; bias[:H] = -50
+    h, c = core.lstm_cell(x, hp, dev(cp_np), WU, dev(bias))
+    np.testing.assert_allclose(c.cpu().numpy(), cp_np, rtol=1e-6, atol=1e-7)
+
+
+def test_lstm_elementwise(core):
+    B, H = 70, 128
+    rng = np.random.default_rng(11)
+    g = (rng.standard_normal((B, 4 * H)) * 3).astype(np.float32)
+    b = rng.standard_normal(4 * H).astype(np.float32)
+    cp = rng.standard_normal((B, H)).astype(np.float32)
+    h, c = core.lstm_elementwise(dev(g), dev(b), dev(cp))
+    gg = g.astype(np.float64) + b
+    i, f, o, cand = (gg[:, k * H:(k + 1) * H] for k in range(4))
+    cr = ko.sigmoid(f) * cp + ko.sigmoid(i) * np.tanh(cand)
+    hr = ko.sigmoid(o) * np.tanh(cr)
+    assert_lstm_close(h, hr, 'h'); assert_lstm_close(c, cr, 'c')
+
+
+# ------------------------------------------------------- stacked / dilated LSTM
+
+@pytest.mark.parametrize('L,T,B,H,dil', [
+    (3, 5, 40, 64, None),
+    (3, 9, 33, 32, [1, 2, 4]),
+    (2, 4, 64, 256, None),
+])
+def test_stacked_lstm_wavefront_launches(core, L, T, B, H, dil):
+    xs, WU, bs = lstm_inputs(21, L, T, B, H, 0.1)
+    hsss, csss = core.stacked_lstm(dev(xs), dev(WU), dev(bs), dilations=dil, schedule='wavefront')
+    hr, cr = ko.stacked_lstm(xs, WU, bs, dilations=dil)
+    assert_lstm_close(hsss, hr, 'hsss'); assert_lstm_close(csss, cr, 'csss')
+
+
+@pytest.mark.parametrize('L,T,B,dil,bias', [
+    (1, 16, 64, None, False),          # config 1: single layer scan, B 64, T 16, H 256
+    (2, 4, 64, None, True),
+    (3, 6, 100, None, True),           # ragged batch
+    (4, 9, 32, [1, 2, 4, 8], True),    # dilated, one 32-row block
+    (6, 12, 256, [1, 2, 4, 8, 16, 32], False),  # config 5 layer structure, short sequence
+])
+def test_stacked_lstm_persistent(core, L, T, B, dil, bias):
+    H = 256
+    xs, WU, bs = lstm_inputs(5, L, T, B, H, 1.0 / 16, bias)
+    ws = torch.empty(core.stacked_lstm_workspace_bytes(L, T, B, H), dtype=torch.uint8, device='cuda')
+    hsss, csss = core.stacked_lstm(dev(xs), dev(WU), None if bs is None else dev(bs), dilations=dil, workspace=ws)
+    assert core.persistent_status(ws) == 0, 'a dependency wait timed out'
+    hr, cr = c_oracle.stacked_lstm(xs, WU, bs, dil)
+    assert_lstm_close(hsss, hr, 'hsss'); assert_lstm_close(csss, cr, 'csss')
+
+
+def test_stacked_lstm_config4_full_size(core):
+    """L 32, B 256, T 64, H 256: persistent kernel vs per-stage launches on the GPU, and
+    vs the oracle on a subset of batch rows (rows never interact)."""
+    L, T, B, H = 32, 64, 256, 256
+    xs, WU, _ = lstm_inputs(1234, L, T, B, H, 1.0 / 16, bias=False)
+    dx, dW = dev(xs), dev(WU)
+    h1, c1 = core.stacked_lstm(dx, dW)
+    h2, c2 = core.stacked_lstm(dx, dW, schedule='wavefront')
+    torch.cuda.synchronize()
+    assert torch.equal(h1, h2) or ko.max_rel_err(h1.cpu().numpy(), h2.cpu().numpy()) < 1e-6
+    rows = [0, 31, 32, 100, 255]
+    hr, cr = ko.stacked_lstm(xs[:, rows], WU, None)
+    assert_lstm_close(h1[:, :, rows], hr, 'hsss rows'); assert_lstm_close(c1[:, :, rows], cr, 'csss rows')
+    # second call reuses nothing stale: same answer
+    h3, _ = core.stacked_lstm(dx, dW)
+    assert torch.equal(h1, h3)
+
+
+def test_stacked_lstm_rejects_bad_arguments(core):
+    xs = torch.zeros((4, 8, 48), device='cuda')
+    WU = torch.zeros((2, 96, 192), device='cuda')
+    with pytest.raises(core.FtkError) as e:
+        core.stacked_lstm(xs, WU)                       # H = 48 is not a multiple of 32
+    assert e.value.code == -2
+    xs = torch.zeros((4, 8, 64), device='cuda'); WU = torch.zeros((2, 128, 256), device='cuda')
+    with pytest.raises(core.FtkError) as e:
+        core.stacked_lstm(xs, WU, dilations=[1, 0])
+    assert e.value.code == -1
+    with pytest.raises(RuntimeError):
+        core.stacked_lstm(xs.cpu(), WU)                 # no CPU path
+
+
+# -------------------------------------------------------------------- B2B GEMM
+
+def b2b_inputs(seed, G, M, N, K, P):
+    rng = np.random.default_rng(seed)
+    A = (rng.standard_normal((G, M, K)) / np.sqrt(K)).astype(np.float16)
+    Bn = (rng.standard_normal((G, N, K)) / np.sqrt(K)).astype(np.float16)
+    Cp = (rng.standard_normal((G, P, N)) / np.sqrt(N)).astype(np.float16)
+    return A, Bn, Cp
+
+
+@pytest.mark.parametrize('G,M,N,K,P', [
+    (1, 32, 32, 32, 32),
+    (2, 100, 64, 32, 64),       # ragged M
+    (3, 256, 96, 96, 160),      # P spans two workgroup tiles, odd tile counts
+    (1, 8192, 256, 64, 64),     # reference benchmark shape (fused_two_hgemms.cu:152-175)
+    (1, 1024, 512, 64, 64),
+])
+def test_b2b_gemm(core, G, M, N, K, P):
+    A, Bn, Cp = b2b_inputs(9, G, M, N, K, P)
+    D = core.b2b_gemm(dev(A), dev(Bn), dev(Cp)).cpu().numpy().astype(np.float64)
+    for g in range(G):
+        ref = ko.b2b_gemm(A[g], Bn[g], Cp[g])
+        assert ko.max_rel_err(D[g], ref) <= F16_TOL
+        # against the variant that rounds the intermediate like the kernel does: only the
+        # final fp16 rounding of D and accumulation order remain
+        ref_r = ko.b2b_gemm(A[g], Bn[g], Cp[g], round_intermediate=True)
+        assert ko.max_rel_err(D[g], ref_r) <= 2e-3
+
+
+def test_b2b_identity_and_permutation(core):
+    M, K = 64, 32
+    rng = np.random.default_rng(2)
+    A = rng.standard_normal((1, M, K)).astype(np.float16)
+    eye = np.eye(K, dtype=np.float16)[None]
+    D = core.b2b_gemm(dev(A), dev(eye), dev(eye)).cpu().numpy()
+    assert np.array_equal(D, A)
+    perm = np.eye(K, dtype=np.float16)[rng.permutation(K)]       # B[k,n]
+    D = core.b2b_gemm(dev(A), dev(perm.T[None].copy()), dev(eye)).cpu().numpy()
+    assert np.array_equal(D[0], (A[0].astype(np.float32) @ perm.astype(np.float32)).astype(np.float16))
+
+
+def test_b2b_config2_full_size(core):
+    G, M, N, K, P = 32, 4096, 128, 128, 128
+    A, Bn, Cp = b2b_inputs(1234, G, M, N, K, P)
+    D = core.b2b_gemm(dev(A), dev(Bn), dev(Cp)).cpu().numpy()
+    worst = 0.0
+    for g in range(G):
+        worst = max(worst, ko.max_rel_err(D[g], ko.b2b_gemm(A[g], Bn[g], Cp[g], dtype=np.float32)))
+    assert worst <= F16_TOL
+    Dc = c_oracle.b2b_gemm(A[5:6, :256], Bn[5:6], Cp[5:6], round_intermediate=True)
+    assert ko.max_rel_err(D[5, :256], Dc[0]) <= 2e-3
+
+
+def test_b2b_rejects_bad_shapes(core):
+    z = lambda *s: torch.zeros(s, dtype=torch.float16, device='cuda')
+    with pytest.raises(core.FtkError) as e:
+        core.b2b_gemm(z(1, 64, 100), z(1, 64, 100), z(1, 64, 64))      # K = 100
+    assert e.value.code == -2
+    with pytest.raises(core.FtkError) as e:
+        core.b2b_gemm(z(1, 64, 64), z(1, 48, 64), z(1, 64, 48))        # N = 48
+    assert e.value.code == -2
+
+
+# ------------------------------------------------------------- flash attention
+
+def fa_inputs(seed, B, Hd, Sq, Skv, D):
+    rng = np.random.default_rng(seed)
+    return tuple(rng.standard_normal(s).astype(np.float16)
+                 for s in ((B, Hd, Sq, D), (B, Hd, Skv, D), (B, Hd, Skv, D)))
+
+
+@pytest.mark.parametrize('B,Hd,Sq,Skv,D', [
+    (1, 2, 64, 64, 64),
+    (1, 2, 100, 77, 64),       # ragged queries and keys
+    (2, 3, 256, 256, 128),
+    (1, 1, 300, 1000, 128),    # ragged, many tiles
+    (2, 8, 1024, 1024, 64),    # the example's sizes, batch 2, 8 heads (flash_attention.py:96-110) at D 64
+])
+def test_flash_attention(core, B, Hd, Sq, Skv, D):
+    Q, K, V = fa_inputs(4, B, Hd, Sq, Skv, D)
+    scale = 1.0 / np.sqrt(D)
+    O = core.flash_attention(dev(Q), dev(K), dev(V), scale).cpu().numpy()
+    ref = ko.attention(Q, K, V, scale, dtype=np.float32)
+    assert ko.max_rel_err(O, ref) <= F16_TOL
+    if Sq * Skv <= 100 * 100:
+        Oc = c_oracle.flash_attention(Q.reshape(-1, Sq, D), K.reshape(-1, Skv, D), V.reshape(-1, Skv, D), scale)
+        assert ko.max_rel_err(O.reshape(-1, Sq, D), Oc) <= F16_TOL
+
+
+def test_flash_attention_uniform_keys_give_mean_of_values(core):
+    B, Hd, S, D = 1, 2, 192, 128
+    rng = np.random.default_rng(8)
+    Q = rng.standard_normal((B, Hd, S, D)).astype(np.float16)
+    K = np.tile(rng.standard_normal((B, Hd, 1, D)), (1, 1, S, 1)).astype(np.float16)
+    V = rng.standard_normal((B, Hd, S, D)).astype(np.float16)
+    O = core.flash_attention(dev(Q), dev(K), dev(V), 1.0).cpu().numpy().astype(np.float32)
+    ref = np.broadcast_to(V.astype(np.float32).mean(axis=2, keepdims=True), O.shape)
+    assert np.max(np.abs(O - ref)) <= 2e-3
+
+
+def test_flash_attention_config3_full_size(core):
+    B, Hd, S, D = 8, 16, 2048, 128
+    g = torch.Generator().manual_seed(1234)
+    Q, K, V = (torch.randn((B, Hd, S, D), generator=g).half() for _ in range(3))
+    scale = 1.0 / np.sqrt(D)
+    O = core.flash_attention(Q.cuda(), K.cuda(), V.cuda(), scale)
+    torch.cuda.synchronize()
+    # oracle on a sample of (batch, head) pairs
+    for (b, h) in [(0, 0), (3, 7), (7, 15)]:
+        ref = ko.attention(Q[b, h].numpy(), K[b, h].numpy(), V[b, h].numpy(), scale, dtype=np.float32)
+        assert ko.max_rel_err(O[b, h].cpu().numpy(), ref) <= F16_TOL
+    # every head against the library routine in fp32
+    ref_all = torch.nn.functional.scaled_dot_product_attention(Q.cuda().float(), K.cuda().float(), V.cuda().float(),
+                                                               scale=scale)
+    err = (O.float() - ref_all).abs().max().item() / ref_all.abs().max().item()
+    assert err <= F16_TOL
+    # rows of softmax sum to one: with V = 1 the output is 1
+    ones = torch.ones_like(V).cuda()
+    O1 = core.flash_attention(Q.cuda(), K.cuda(), ones, scale)
+    assert (O1.float() - 1).abs().max().item() <= 2e-3
+
+
+def test_flash_attention_rejects_bad_shapes(core):
+    z = lambda *s: torch.zeros(s, dtype=torch.float16, device='cuda')
+    with pytest.raises(core.FtkError) as e:
+        core.flash_attention(z(1, 1, 64, 48), z(1, 1, 64, 48), z(1, 1, 64, 48))
+    assert e.value.code == -2
+
+
+# -------------------------------------------------------------- online softmax
+
+@pytest.mark.parametrize('cols', [1, 7, 517, 1027, 4096])   # 7/517/1027: test_softmax.cc:77-87
+def test_online_softmax(core, cols):
+    rng = np.random.default_rng(13)
+    x = (rng.standard_normal((37, cols)) * 6).astype(np.float32)
+    y = core.online_softmax(dev(x)).cpu().numpy()
+    ref = ko.online_softmax_rows(x, chunk=64)
+    np.testing.assert_allclose(y, ref, rtol=2e-5, atol=1e-7)
+    np.testing.assert_allclose(y.sum(-1), 1.0, atol=1e-5)
+    np.testing.assert_allclose(y, c_oracle.online_softmax(x), rtol=2e-5, atol=1e-7)
