@@ -15,104 +15,165 @@
 // lane already holds, and two 8-byte LDS reads of Cs for the other operand.
 // No shuffle, no LDS round trip for P.
 //
-// A workgroup (8 waves) stages one problem's B and C in LDS once and then
-// walks row tiles of that problem; the grid is (workgroups per problem, P
-// tiles of 128, G).  D tiles go through an LDS transpose so global stores are
-// full 16-byte-per-lane row segments.
+// A workgroup stages one problem's B and C in LDS once and then walks row tiles
+// of that problem, each wave 64 rows at a time (two 32-row tiles sharing every
+// B and C fragment read).  The A rows of a wave's first tile are requested
+// before the staging starts, so the HBM latency of A hides behind it.  The
+// grid is one-dimensional and remapped so that the workgroups of one problem
+// share an XCD (and with it the L2 copy of B and C).  D tiles go through an
+// LDS transpose so global stores are full 16-byte-per-lane row segments.
 #include <algorithm>
 
 #include "ftk_common.h"
 
 namespace ftk {
 
-constexpr int B2B_WAVES = 8;
-constexpr int B2B_THREADS = B2B_WAVES * 64;
 constexpr int B2B_PTILE = 128;  // p columns per workgroup
-constexpr int B2B_DLD = B2B_PTILE + 4;  // padded D staging row (halfs)
 
-__device__ __forceinline__ uint4 ldg16(const void* p) { return *reinterpret_cast<const uint4*>(p); }
+__device__ __forceinline__ v4u ldg16(const void* p) { return *reinterpret_cast<const v4u*>(p); }
+
+struct B2BGrid {
+  int per_problem;  // workgroups sharing one (problem, p tile)
+  int ptiles;
+  int total;        // per_problem * ptiles * G
+};
 
 template <int KS>  // K = 16 * KS
-__global__ __launch_bounds__(B2B_THREADS) void b2b_gemm_kernel(const _Float16* __restrict__ A,
-                                                               const _Float16* __restrict__ Bm,
-                                                               const _Float16* __restrict__ Cm,
-                                                               _Float16* __restrict__ D, int M, int N, int P) {
+__global__ __launch_bounds__(512) void b2b_gemm_kernel(const _Float16* __restrict__ A,
+                                                       const _Float16* __restrict__ Bm,
+                                                       const _Float16* __restrict__ Cm, _Float16* __restrict__ D,
+                                                       int M, int N, int P, B2BGrid gr) {
   constexpr int K = 16 * KS;
   constexpr int BLD = K + 8;  // padded Bs row (halfs)
   const int CLD = N + 4;      // padded Cs row (halfs)
+  const int threads = blockDim.x;
+  const int waves = threads >> 6;
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
-  _Float16* Bs = reinterpret_cast<_Float16*>(smem);  // [N][BLD]
-  _Float16* Cs = Bs + N * BLD;                       // [PTILE][CLD]
-  _Float16* Ds = Cs + B2B_PTILE * CLD;               // [waves][32][DLD]
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = tid >> 6;
   const int j = lane & 31;
   const int hh = lane >> 5;
-  const int g = blockIdx.z;
-  const int p0 = blockIdx.y * B2B_PTILE;
-  const int np_tiles = min(B2B_PTILE, P - p0) / 32;  // p tiles handled here (1..4)
+
+  // consecutive logical ids land on one XCD (hardware deals workgroups round-robin over 8 XCDs)
+  int id = blockIdx.x;
+  if ((gr.total & 7) == 0) id = (blockIdx.x & 7) * (gr.total >> 3) + (blockIdx.x >> 3);
+  const int part = id % gr.per_problem;
+  const int pt_idx = (id / gr.per_problem) % gr.ptiles;
+  const int g = id / (gr.per_problem * gr.ptiles);
+
+  const int p0 = pt_idx * B2B_PTILE;
+  const int pw = min(B2B_PTILE, P - p0);  // p columns handled here
+  const int np_tiles = pw / 32;           // 1..4
+  const int DLD = pw + 4;                 // padded D staging row (halfs)
+
+  _Float16* Bs = reinterpret_cast<_Float16*>(smem);  // [N][BLD]
+  _Float16* Cs = Bs + N * BLD;                       // [pw][CLD]
+  _Float16* Ds = Cs + pw * CLD;                      // [waves][32][DLD]
+  _Float16* Dw = Ds + wave * 32 * DLD;
 
   const _Float16* Ag = A + (size_t)g * M * K;
   const _Float16* Bg = Bm + (size_t)g * N * K;
-  const _Float16* Cg = Cm + (size_t)g * P * N;
-  _Float16* Dg = D + (size_t)g * M * P;
-  _Float16* Dw = Ds + wave * 32 * B2B_DLD;
+  const _Float16* Cg = Cm + (size_t)g * P * N + (size_t)p0 * N;
+  _Float16* Dg = D + (size_t)g * M * P + p0;
 
-  // ---- stage this problem's Bs[n][k] and Cs[p][n] once per workgroup
-  for (int idx = tid; idx < N * (K / 8); idx += B2B_THREADS) {
-    const int n = idx / (K / 8);
-    const int k8 = idx - n * (K / 8);
-    *reinterpret_cast<uint4*>(Bs + n * BLD + 8 * k8) = ldg16(Bg + (size_t)n * K + 8 * k8);
-  }
-  for (int idx = tid; idx < np_tiles * 32 * (N / 8); idx += B2B_THREADS) {
-    const int p = idx / (N / 8);
-    const int n8 = idx - p * (N / 8);
-    const uint4 v = ldg16(Cg + (size_t)(p0 + p) * N + 8 * n8);
-    // CLD is not a multiple of 8 halfs: write as two 8-byte pieces
-    *reinterpret_cast<uint2*>(Cs + p * CLD + 8 * n8) = make_uint2(v.x, v.y);
-    *reinterpret_cast<uint2*>(Cs + p * CLD + 8 * n8 + 4) = make_uint2(v.z, v.w);
+  const int row_pairs = (M + 63) / 64;  // units of 64 rows
+  const int wave_stride = gr.per_problem * waves;
+  int pair = part * waves + wave;
+
+  // ---- A row fragments: step s contracts k in [8s, 8s+8) (lanes 0-31) and
+  //      [K/2 + 8s, K/2 + 8s + 8) (lanes 32-63): 16*KS contiguous bytes per lane
+  v8h afrag[2][KS];
+  auto load_a = [&](int pr_) __attribute__((always_inline)) {
+#pragma unroll
+    for (int rt = 0; rt < 2; ++rt) {
+      const int row_c = min(pr_ * 64 + 32 * rt + j, M - 1);
+      const _Float16* arow = Ag + (size_t)row_c * K + hh * (K / 2);
+#pragma unroll
+      for (int s = 0; s < KS; ++s) {
+        const v4u v = ldg16(arow + 8 * s);
+        afrag[rt][s] = *reinterpret_cast<const v8h*>(&v);
+      }
+    }
+  };
+  if (pair < row_pairs) load_a(pair);
+
+  // ---- stage this problem's Bs[n][k] and Cs[p][n]: loads in batches of four
+  {
+    const int nb = N * (K / 8);
+    for (int base = 0; base < nb; base += 4 * threads) {
+      v4u v[4];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const int idx = base + u * threads + tid;
+        if (idx < nb) v[u] = ldg16(Bg + (size_t)idx * 8);
+      }
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const int idx = base + u * threads + tid;
+        if (idx < nb) {
+          const int n = idx / (K / 8);
+          const int k8 = idx - n * (K / 8);
+          *reinterpret_cast<v4u*>(Bs + n * BLD + 8 * k8) = v[u];
+        }
+      }
+    }
+    const int n8s = N / 8;
+    const int ncq = pw * n8s;
+    for (int base = 0; base < ncq; base += 4 * threads) {
+      v4u v[4];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const int idx = base + u * threads + tid;
+        if (idx < ncq) v[u] = ldg16(Cg + (size_t)idx * 8);
+      }
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const int idx = base + u * threads + tid;
+        if (idx < ncq) {
+          const int p = idx / n8s;
+          const int n8 = idx - p * n8s;
+          // CLD is not a multiple of 8 halfs: two 8-byte pieces
+          *reinterpret_cast<v2u*>(Cs + p * CLD + 8 * n8) = v2u{v[u][0], v[u][1]};
+          *reinterpret_cast<v2u*>(Cs + p * CLD + 8 * n8 + 4) = v2u{v[u][2], v[u][3]};
+        }
+      }
+    }
   }
   __syncthreads();
 
-  const int row_tiles = (M + 31) / 32;
-  const int wave_stride = gridDim.x * B2B_WAVES;
-  for (int tile = blockIdx.x * B2B_WAVES + wave; tile < row_tiles; tile += wave_stride) {
-    const int row_c = min(tile * 32 + j, M - 1);
-    // ---- A row fragments: step s contracts k in [8s, 8s+8) (lanes 0-31) and
-    //      [K/2 + 8s, K/2 + 8s + 8) (lanes 32-63): 16*KS contiguous bytes per lane
-    v8h afrag[KS];
-    const _Float16* arow = Ag + (size_t)row_c * K + hh * (K / 2);
+  for (; pair < row_pairs; pair += wave_stride) {
+    v16f dacc[2][4];
 #pragma unroll
-    for (int s = 0; s < KS; ++s) {
-      const uint4 v = ldg16(arow + 8 * s);
-      afrag[s] = *reinterpret_cast<const v8h*>(&v);
-    }
-
-    v16f dacc[4];
+    for (int rt = 0; rt < 2; ++rt)
 #pragma unroll
-    for (int pt = 0; pt < 4; ++pt)
+      for (int pt = 0; pt < 4; ++pt)
 #pragma unroll
-      for (int r = 0; r < 16; ++r) dacc[pt][r] = 0.0f;
+        for (int r = 0; r < 16; ++r) dacc[rt][pt][r] = 0.0f;
 
     for (int nt = 0; nt < N / 32; ++nt) {
-      // GEMM1: P^T tile [32 n, 32 rows]
-      v16f pacc;
+      // GEMM1: P^T tiles [32 n, 32 rows] for both row tiles
+      v16f pacc[2];
 #pragma unroll
-      for (int r = 0; r < 16; ++r) pacc[r] = 0.0f;
+      for (int rt = 0; rt < 2; ++rt)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) pacc[rt][r] = 0.0f;
       const _Float16* brow = Bs + (nt * 32 + j) * BLD + hh * (K / 2);
 #pragma unroll
       for (int s = 0; s < KS; ++s) {
         const v8h bfrag = *reinterpret_cast<const v8h*>(brow + 8 * s);
-        pacc = __builtin_amdgcn_mfma_f32_32x32x16_f16(bfrag, afrag[s], pacc, 0, 0, 0);
+        pacc[0] = __builtin_amdgcn_mfma_f32_32x32x16_f16(bfrag, afrag[0][s], pacc[0], 0, 0, 0);
+        pacc[1] = __builtin_amdgcn_mfma_f32_32x32x16_f16(bfrag, afrag[1][s], pacc[1], 0, 0, 0);
       }
-      // round to fp16: the two B-operands of GEMM2 for this n tile
-      v8h pf[2];
+      // round to fp16: the B-operands of GEMM2 for this n tile
+      v8h pf[2][2];
 #pragma unroll
-      for (int s = 0; s < 2; ++s)
+      for (int rt = 0; rt < 2; ++rt)
 #pragma unroll
-        for (int e = 0; e < 8; ++e) pf[s][e] = (_Float16)pacc[8 * s + e];
+        for (int s = 0; s < 2; ++s)
+#pragma unroll
+          for (int e = 0; e < 8; ++e) pf[rt][s][e] = (_Float16)pacc[rt][8 * s + e];
       // GEMM2: D^T[p tile] += Cs[p][n] * P
 #pragma unroll
       for (int pt = 0; pt < 4; ++pt) {
@@ -123,62 +184,83 @@ __global__ __launch_bounds__(B2B_THREADS) void b2b_gemm_kernel(const _Float16* _
             const v4h c0 = *reinterpret_cast<const v4h*>(crow + 16 * s);
             const v4h c1 = *reinterpret_cast<const v4h*>(crow + 16 * s + 8);
             const v8h cfrag = {c0[0], c0[1], c0[2], c0[3], c1[0], c1[1], c1[2], c1[3]};
-            dacc[pt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(cfrag, pf[s], dacc[pt], 0, 0, 0);
+            dacc[0][pt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(cfrag, pf[0][s], dacc[0][pt], 0, 0, 0);
+            dacc[1][pt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(cfrag, pf[1][s], dacc[1][pt], 0, 0, 0);
           }
         }
       }
     }
 
+    // next pair's A rows go into flight while this pair's D drains
+    const int this_pair = pair;
+    if (pair + wave_stride < row_pairs) load_a(pair + wave_stride);
+
     // ---- epilogue: D^T accumulators -> LDS [row][p] -> 16-byte row segments.
     // A wave reads back only what it wrote itself and LDS operations of one
     // wave complete in order, so no workgroup barrier is needed.
 #pragma unroll
-    for (int pt = 0; pt < 4; ++pt) {
-      if (pt < np_tiles) {
+    for (int rt = 0; rt < 2; ++rt) {
 #pragma unroll
-        for (int gq = 0; gq < 4; ++gq) {
-          const v4h o = {(_Float16)dacc[pt][4 * gq + 0], (_Float16)dacc[pt][4 * gq + 1],
-                         (_Float16)dacc[pt][4 * gq + 2], (_Float16)dacc[pt][4 * gq + 3]};
-          *reinterpret_cast<v4h*>(Dw + j * B2B_DLD + pt * 32 + 8 * gq + 4 * hh) = o;
+      for (int pt = 0; pt < 4; ++pt) {
+        if (pt < np_tiles) {
+#pragma unroll
+          for (int gq = 0; gq < 4; ++gq) {
+            const v4h o = {(_Float16)dacc[rt][pt][4 * gq + 0], (_Float16)dacc[rt][pt][4 * gq + 1],
+                           (_Float16)dacc[rt][pt][4 * gq + 2], (_Float16)dacc[rt][pt][4 * gq + 3]};
+            *reinterpret_cast<v4h*>(Dw + j * DLD + pt * 32 + 8 * gq + 4 * hh) = o;
+          }
         }
       }
-    }
-    const int segs = np_tiles * 4;  // 16-byte segments per row
-    for (int idx = lane; idx < 32 * segs; idx += 64) {
-      const int r = idx / segs;
-      const int sg = idx - r * segs;
-      const int grow = tile * 32 + r;
-      if (grow < M) {
-        const uint2 lo = *reinterpret_cast<const uint2*>(Dw + r * B2B_DLD + 8 * sg);
-        const uint2 hi = *reinterpret_cast<const uint2*>(Dw + r * B2B_DLD + 8 * sg + 4);
-        *reinterpret_cast<uint4*>(Dg + (size_t)grow * P + p0 + 8 * sg) = make_uint4(lo.x, lo.y, hi.x, hi.y);
+      const int segs = np_tiles * 4;  // 16-byte segments per row
+      for (int idx = lane; idx < 32 * segs; idx += 64) {
+        const int r = idx / segs;
+        const int sg = idx - r * segs;
+        const int grow = this_pair * 64 + 32 * rt + r;
+        if (grow < M) {
+          const v2u lo = *reinterpret_cast<const v2u*>(Dw + r * DLD + 8 * sg);
+          const v2u hi = *reinterpret_cast<const v2u*>(Dw + r * DLD + 8 * sg + 4);
+          *reinterpret_cast<v4u*>(Dg + (size_t)grow * P + 8 * sg) = v4u{lo[0], lo[1], hi[0], hi[1]};
+        }
       }
     }
   }
 }
 
-static size_t b2b_lds_bytes(int N, int K) {
-  return (size_t)(N * (K + 8) + B2B_PTILE * (N + 4) + B2B_WAVES * 32 * B2B_DLD) * 2;
+static size_t b2b_lds_bytes(int N, int K, int pw, int waves) {
+  return (size_t)(N * (K + 8) + pw * (N + 4) + waves * 32 * (pw + 4)) * 2;
 }
 
 template <int KS>
 static int launch_b2b(const void* A, const void* B, const void* C, void* D, int G, int M, int N, int P, int cus,
                       int lds_max, hipStream_t s) {
   constexpr int K = 16 * KS;
-  const size_t lds = b2b_lds_bytes(N, K);
+  const int pw = std::min(P, B2B_PTILE);
+  int waves = 8;
+  while (waves > 1 && (int)b2b_lds_bytes(N, K, pw, waves) > lds_max) waves >>= 1;
+  const size_t lds = b2b_lds_bytes(N, K, pw, waves);
   if ((int)lds > lds_max)
     return fail(FTK_ERR_UNSUPPORTED_SHAPE,
-                "ftk_b2b_gemm_f16: B and C tiles for N=%d K=%d need %zu bytes of LDS, the device has %d", N, K, lds,
-                lds_max);
-  const int ptiles = (P + B2B_PTILE - 1) / B2B_PTILE;
-  const int row_tiles = (M + 31) / 32;
-  // enough workgroups per problem to fill the chip once; each walks its share of the row tiles
-  int per_problem = (cus + G * ptiles - 1) / (G * ptiles);
-  per_problem = std::max(1, std::min(per_problem, (row_tiles + B2B_WAVES - 1) / B2B_WAVES));
+                "ftk_b2b_gemm_f16: B and C tiles for N=%d K=%d P=%d need %zu bytes of LDS, the device has %d", N, K, P,
+                lds, lds_max);
+  B2BGrid gr;
+  gr.ptiles = (P + B2B_PTILE - 1) / B2B_PTILE;
+  const int row_pairs = (M + 63) / 64;
+  const long long units = (long long)G * gr.ptiles;
+  // enough workgroups per (problem, p tile) to fill the chip once; each walks its share of the rows
+  long long per = (cus + units - 1) / units;
+  per = std::max(1LL, std::min(per, (long long)(row_pairs + waves - 1) / waves));
+  gr.per_problem = (int)per;
+  const long long total = units * per;
+  if (total > 0x7fffffffLL) return fail(FTK_ERR_UNSUPPORTED_SHAPE, "ftk_b2b_gemm_f16: grid too large");
+  gr.total = (int)total;
   const void* fn = (const void*)b2b_gemm_kernel<KS>;
-  FTK_HIP(hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-  hipLaunchKernelGGL(b2b_gemm_kernel<KS>, dim3(per_problem, ptiles, G), dim3(B2B_THREADS), lds, s,
-                     (const _Float16*)A, (const _Float16*)B, (const _Float16*)C, (_Float16*)D, M, N, P);
+  static int attr_lds = 0;
+  if ((int)lds > attr_lds) {
+    FTK_HIP(hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+    attr_lds = (int)lds;
+  }
+  hipLaunchKernelGGL(b2b_gemm_kernel<KS>, dim3(gr.total), dim3(waves * 64), lds, s, (const _Float16*)A,
+                     (const _Float16*)B, (const _Float16*)C, (_Float16*)D, M, N, P, gr);
   return check_launch("b2b_gemm_kernel");
 }
 
@@ -191,7 +273,8 @@ extern "C" int ftk_b2b_gemm_f16(const void* A, const void* B, const void* C, voi
   if (G <= 0 || M <= 0 || N <= 0 || K <= 0 || P <= 0)
     return fail(FTK_ERR_INVALID_ARGUMENT, "ftk_b2b_gemm_f16: G, M, N, K, P must be positive");
   if (N % 32 || P % 32) return fail(FTK_ERR_UNSUPPORTED_SHAPE, "ftk_b2b_gemm_f16: N=%d and P=%d must be multiples of 32", N, P);
-  if (G > 65535) return fail(FTK_ERR_UNSUPPORTED_SHAPE, "ftk_b2b_gemm_f16: G=%d above 65535", G);
+  if (K != 32 && K != 64 && K != 96 && K != 128)
+    return fail(FTK_ERR_UNSUPPORTED_SHAPE, "ftk_b2b_gemm_f16: K=%d must be one of 32, 64, 96, 128", K);
   const DeviceProps* dp = nullptr;
   int rc = device_props(&dp);
   if (rc) return rc;
@@ -200,8 +283,6 @@ extern "C" int ftk_b2b_gemm_f16(const void* A, const void* B, const void* C, voi
     case 32: return launch_b2b<2>(A, B, C, D, G, M, N, P, dp->cus, dp->lds_optin, s);
     case 64: return launch_b2b<4>(A, B, C, D, G, M, N, P, dp->cus, dp->lds_optin, s);
     case 96: return launch_b2b<6>(A, B, C, D, G, M, N, P, dp->cus, dp->lds_optin, s);
-    case 128: return launch_b2b<8>(A, B, C, D, G, M, N, P, dp->cus, dp->lds_optin, s);
-    default:
-      return fail(FTK_ERR_UNSUPPORTED_SHAPE, "ftk_b2b_gemm_f16: K=%d must be one of 32, 64, 96, 128", K);
+    default: return launch_b2b<8>(A, B, C, D, G, M, N, P, dp->cus, dp->lds_optin, s);
   }
 }

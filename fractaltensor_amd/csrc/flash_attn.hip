@@ -19,6 +19,8 @@
 // streams K/V in 64-key tiles: K as stored ([key][d], padded rows), V
 // transposed on the way into LDS ([d][key]) by 4x4 register transposes.  Tiles
 // are double buffered with register prefetch of the next tile.
+#include <stdlib.h>
+
 #include <algorithm>
 #include <type_traits>
 
@@ -39,9 +41,10 @@ __device__ __forceinline__ void static_for(F&& f) {
 
 constexpr int FA_KT = 64;          // keys per tile
 constexpr int FA_VLD = FA_KT + 4;  // padded V^T row (halfs)
+constexpr float FA_TAU = 8.0f;     // slack (in powers of two) before the running maximum is moved
 
-template <int D, int QT>
-__global__ __launch_bounds__(256) void flash_attn_kernel(const _Float16* __restrict__ Q,
+template <int D, int QT, int WAVES>
+__global__ __launch_bounds__(WAVES * 64) void flash_attn_kernel(const _Float16* __restrict__ Q,
                                                          const _Float16* __restrict__ K,
                                                          const _Float16* __restrict__ V,
                                                          _Float16* __restrict__ O, int Sq, int Skv,
@@ -61,7 +64,8 @@ __global__ __launch_bounds__(256) void flash_attn_kernel(const _Float16* __restr
   const int j = lane & 31;
   const int hh = lane >> 5;
   const int bh = blockIdx.y;
-  const int q_base = blockIdx.x * (128 * QT) + wave * (32 * QT);
+  constexpr int NT = WAVES * 64;  // threads
+  const int q_base = blockIdx.x * (WAVES * 32 * QT) + wave * (32 * QT);
 
   const _Float16* Qg = Q + (size_t)bh * Sq * D;
   const _Float16* Kg = K + (size_t)bh * Skv * D;
@@ -93,9 +97,9 @@ __global__ __launch_bounds__(256) void flash_attn_kernel(const _Float16* __restr
   }
 
   // ---- staging assignments
-  constexpr int KN = D / 32;  // 16-byte K loads per thread per tile
-  constexpr int VN = D / 64;  // 4x4 V blocks per thread per tile
-  static_assert(D % 64 == 0, "head dim must be a multiple of 64");
+  constexpr int KN = FA_KT * (D / 8) / NT;   // 16-byte K loads per thread per tile
+  constexpr int VN = (FA_KT / 4) * (D / 4) / NT;  // 4x4 V blocks per thread per tile
+  static_assert(KN >= 1 && VN >= 1, "tile too small for this many threads");
   v4u kreg[KN];
   v2u vreg[VN][4];
 
@@ -103,7 +107,7 @@ __global__ __launch_bounds__(256) void flash_attn_kernel(const _Float16* __restr
     const int key0 = kt * FA_KT;
     static_for<KN>([&](auto nc) __attribute__((always_inline)) {
       constexpr int n = decltype(nc)::value;
-      const int idx = tid + 256 * n;
+      const int idx = tid + NT * n;
       const int key = min(key0 + idx / (D / 8), Skv - 1);
       const int c8 = idx % (D / 8);
       kreg[n] = *reinterpret_cast<const v4u*>(Kg + (size_t)key * D + 8 * c8);
@@ -111,7 +115,7 @@ __global__ __launch_bounds__(256) void flash_attn_kernel(const _Float16* __restr
     static_for<VN * 4>([&](auto nc) __attribute__((always_inline)) {
       constexpr int n = decltype(nc)::value / 4;
       constexpr int nn = decltype(nc)::value % 4;
-      const int u = tid + 256 * n;
+      const int u = tid + NT * n;
       const int dg = u % (D / 4);
       const int kq = u / (D / 4);
       const int key = min(key0 + 4 * kq + nn, Skv - 1);
@@ -123,14 +127,14 @@ __global__ __launch_bounds__(256) void flash_attn_kernel(const _Float16* __restr
     _Float16* vt = Vt + buf * VSZ;
     static_for<KN>([&](auto nc) __attribute__((always_inline)) {
       constexpr int n = decltype(nc)::value;
-      const int idx = tid + 256 * n;
+      const int idx = tid + NT * n;
       const int key = idx / (D / 8);
       const int c8 = idx % (D / 8);
       *reinterpret_cast<v4u*>(ks + key * KLD + 8 * c8) = kreg[n];
     });
     static_for<VN>([&](auto nc) __attribute__((always_inline)) {
       constexpr int n = decltype(nc)::value;
-      const int u = tid + 256 * n;
+      const int u = tid + NT * n;
       const int dg = u % (D / 4);
       const int kq = u / (D / 4);
       const v2u r0 = vreg[n][0], r1 = vreg[n][1], r2 = vreg[n][2], r3 = vreg[n][3];
@@ -153,6 +157,7 @@ __global__ __launch_bounds__(256) void flash_attn_kernel(const _Float16* __restr
   };
 
   const int ntiles = (Skv + FA_KT - 1) / FA_KT;
+  const float tau_raw = FA_TAU / scale_log2e;
   load_tile(0);
   store_tile(0);
   __syncthreads();
@@ -183,28 +188,43 @@ __global__ __launch_bounds__(256) void flash_attn_kernel(const _Float16* __restr
       }
     }
 
-    // ---- online softmax, one query row per lane (two lanes share a row)
+    // ---- online softmax, one query row per lane (two lanes share a row).
+    // Scores stay in raw units; p = exp2(s*c - m_ref*c) with c = scale*log2(e)
+    // is one fused multiply-add and one exponential per score.  m_ref is a
+    // reference maximum that is only moved (and O, l rescaled) when the true
+    // row maximum has run ahead of it by more than FA_TAU in exponent units:
+    // any m_ref gives the same O = acc/l, p merely ranges up to 2^FA_TAU.
     const bool ragged = (kt + 1 == ntiles) && (Skv % FA_KT != 0);
     v8h pf[QT][2][2];
 #pragma unroll
     for (int qt = 0; qt < QT; ++qt) {
-      float mx = -INFINITY;
+      if (ragged) {
+#pragma unroll
+        for (int k2 = 0; k2 < 2; ++k2)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) {
+            const int key = kt * FA_KT + 32 * k2 + 8 * (r >> 2) + 4 * hh + (r & 3);
+            if (key >= Skv) sacc[qt][k2][r] = -INFINITY;
+          }
+      }
+      float mx = sacc[qt][0][0];
 #pragma unroll
       for (int k2 = 0; k2 < 2; ++k2)
 #pragma unroll
-        for (int r = 0; r < 16; ++r) {
-          float s2 = sacc[qt][k2][r] * scale_log2e;
-          if (ragged) {
-            const int key = kt * FA_KT + 32 * k2 + 8 * (r >> 2) + 4 * hh + (r & 3);
-            if (key >= Skv) s2 = -INFINITY;
-          }
-          sacc[qt][k2][r] = s2;
-          mx = fmaxf(mx, s2);
-        }
+        for (int r = 0; r < 16; ++r) mx = fmaxf(mx, sacc[qt][k2][r]);
       mx = fmaxf(mx, __shfl_xor(mx, 32));
-      const float m_new = fmaxf(m_run[qt], mx);
-      const float alpha = __builtin_amdgcn_exp2f(m_run[qt] - m_new);
-      m_run[qt] = m_new;
+      const bool need = mx > m_run[qt] + tau_raw;
+      if (__builtin_amdgcn_ballot_w64(need) != 0) {
+        const float m_new = need ? mx : m_run[qt];
+        const float alpha = __builtin_amdgcn_exp2f((m_run[qt] - m_new) * scale_log2e);
+        m_run[qt] = m_new;
+        l_run[qt] *= alpha;
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) oacc[qt][dt][r] *= alpha;
+      }
+      const float mc = -m_run[qt] * scale_log2e;
       float psum = 0.0f;
 #pragma unroll
       for (int k2 = 0; k2 < 2; ++k2)
@@ -212,15 +232,11 @@ __global__ __launch_bounds__(256) void flash_attn_kernel(const _Float16* __restr
         for (int s = 0; s < 2; ++s)
 #pragma unroll
           for (int e = 0; e < 8; ++e) {
-            const float p = __builtin_amdgcn_exp2f(sacc[qt][k2][8 * s + e] - m_new);
+            const float p = __builtin_amdgcn_exp2f(__builtin_fmaf(sacc[qt][k2][8 * s + e], scale_log2e, mc));
             psum += p;
             pf[qt][k2][s][e] = (_Float16)p;
           }
-      l_run[qt] = l_run[qt] * alpha + psum;  // this lane's half of the row sum
-#pragma unroll
-      for (int dt = 0; dt < DT; ++dt)
-#pragma unroll
-        for (int r = 0; r < 16; ++r) oacc[qt][dt][r] *= alpha;
+      l_run[qt] += psum;  // this lane's half of the row sum
     }
 
     // ---- O^T += V^T P^T
@@ -263,17 +279,33 @@ __global__ __launch_bounds__(256) void flash_attn_kernel(const _Float16* __restr
   }
 }
 
-template <int D, int QT>
+template <int D, int QT, int WAVES>
 static int launch_fa(const void* Q, const void* K, const void* V, void* O, int BH, int Sq, int Skv, float scale,
                      int lds_max, hipStream_t s) {
   const size_t lds = (size_t)2 * (FA_KT * (D + 8) + D * FA_VLD) * 2;
   if ((int)lds > lds_max) return fail(FTK_ERR_UNSUPPORTED_SHAPE, "ftk_flash_attn_f16: needs %zu bytes of LDS", lds);
-  const void* fn = (const void*)flash_attn_kernel<D, QT>;
-  FTK_HIP(hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-  dim3 grid((Sq + 128 * QT - 1) / (128 * QT), BH);
-  hipLaunchKernelGGL((flash_attn_kernel<D, QT>), grid, dim3(256), lds, s, (const _Float16*)Q, (const _Float16*)K,
+  const void* fn = (const void*)flash_attn_kernel<D, QT, WAVES>;
+  static bool attr_set = false;
+  if (!attr_set) {
+    FTK_HIP(hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+    attr_set = true;
+  }
+  constexpr int ROWS = WAVES * 32 * QT;
+  dim3 grid((Sq + ROWS - 1) / ROWS, BH);
+  hipLaunchKernelGGL((flash_attn_kernel<D, QT, WAVES>), grid, dim3(WAVES * 64), lds, s, (const _Float16*)Q, (const _Float16*)K,
                      (const _Float16*)V, (_Float16*)O, Sq, Skv, scale * 1.4426950408889634f);
   return check_launch("flash_attn_kernel");
+}
+
+// Tuning hook: FTK_FA_VARIANT=1|2|3 pins the tiling variant (read once).
+static int fa_variant_override() {
+  static int v = -1;
+  if (v < 0) {
+    const char* e = getenv("FTK_FA_VARIANT");
+    v = e ? atoi(e) : 0;
+    if (v < 0 || v > 3) v = 0;
+  }
+  return v;
 }
 
 }  // namespace ftk
@@ -291,12 +323,21 @@ extern "C" int ftk_flash_attn_f16(const void* Q, const void* K, const void* V, v
   int rc = device_props(&dp);
   if (rc) return rc;
   hipStream_t s = (hipStream_t)stream;
-  // 64 query rows per wave halve the LDS operand traffic per flop; use them once
-  // there are enough 256-row blocks to occupy the chip
-  const bool big = (long long)((Sq + 255) / 256) * bh >= dp->cus;
-  if (D == 128)
-    return big ? launch_fa<128, 2>(Q, K, V, O, (int)bh, Sq, Skv, scale, dp->lds_optin, s)
-               : launch_fa<128, 1>(Q, K, V, O, (int)bh, Sq, Skv, scale, dp->lds_optin, s);
-  return big ? launch_fa<64, 2>(Q, K, V, O, (int)bh, Sq, Skv, scale, dp->lds_optin, s)
-             : launch_fa<64, 1>(Q, K, V, O, (int)bh, Sq, Skv, scale, dp->lds_optin, s);
+  // Variant: 0 = choose by problem size, 1 = 4 waves x 32 rows, 2 = 4 waves x 64 rows, 3 = 8 waves x 32 rows.
+  int variant = fa_variant_override();
+  if (variant == 0) variant = ((long long)((Sq + 255) / 256) * bh >= dp->cus) ? 2 : 1;
+  const int lds = dp->lds_optin;
+  if (D == 128) {
+    switch (variant) {
+      case 1: return launch_fa<128, 1, 4>(Q, K, V, O, (int)bh, Sq, Skv, scale, lds, s);
+      case 3: return launch_fa<128, 1, 8>(Q, K, V, O, (int)bh, Sq, Skv, scale, lds, s);
+      default: return launch_fa<128, 2, 4>(Q, K, V, O, (int)bh, Sq, Skv, scale, lds, s);
+    }
+  }
+  switch (variant) {
+    case 1: return launch_fa<64, 1, 4>(Q, K, V, O, (int)bh, Sq, Skv, scale, lds, s);
+    case 3:  // a 64-key tile of 64-wide heads has too little to stage for 8 waves
+    default: return launch_fa<64, 2, 4>(Q, K, V, O, (int)bh, Sq, Skv, scale, lds, s);
+  }
 }
+

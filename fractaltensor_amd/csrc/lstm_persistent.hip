@@ -7,23 +7,34 @@
 // {i,f,o,c~}), each of its four waves 32 of them as 256 VGPRs per lane, the
 // MFMA "A" operands of v_mfma_f32_32x32x2_f32.  Eight such column slices make
 // a layer; with spare compute units a layer gets several row slices as well,
-// each handling its own subset of the batch's row blocks.
+// each handling its own subset of the batch's 32-row blocks.
 //
 // Work item = (t, row block).  For an item the workgroup stages the activation
-// tile [rows, 512] = [x_t | h_{t-d}] in LDS, runs the K = 512 product against
+// tile [32, 512] = [x_t | h_{t-d}] in LDS, runs the K = 512 product against
 // the resident weights, applies bias, sigmoid/tanh and the state update in
 // registers (all four gates of a (row, unit) pair land in one lane, see
 // lstm_cell.hip) and writes h, c.  Batch rows never interact, so dependencies
 // are per row block: item (l, t, rb) needs h[l-1][t][rb] from the layer below
-// and h[l][t-d][rb] from all eight column slices of its own layer.  Producers
-// publish a row block with a release fence and an atomic increment of
-// flags[l][t][rb]; consumers spin (bounded) until the count reaches 8.
-// Layer l therefore trails layer l-1 by one item: the wavefront of the
+// and h[l][t-d][rb] from all eight column slices of its own layer.  Layer l
+// therefore trails layer l-1 by an item or two: the wavefront of the
 // reference's region schedule, without launches, device syncs or scatter.
 //
-// All workgroups must be co-resident: the host launches cooperatively with
-// one workgroup per compute unit (each uses the whole register file of its
-// CU).  Every wait is bounded by spin_limit polls; on expiry the kernel
+// Hand-off between compute units (which may sit on different XCDs, whose L2
+// caches are not coherent with each other) uses no cache-wide fences: h is
+// written with agent-scope write-through stores and read with agent-scope
+// loads, the producer waits for its stores to be acknowledged, then one thread
+// per workgroup increments flags[l][t][rb]; consumers poll that count with
+// agent-scope loads until it reaches 8.  c is only ever re-read by the
+// workgroup that wrote it and goes through the cache normally.
+//
+// The activation tile is double buffered: while item n is on the matrix cores
+// the next item's tile is already in flight into registers (if its producers
+// are done; otherwise the wave waits for them after its own MFMAs).  One
+// workgroup barrier per item.
+//
+// All workgroups must be co-resident: the host launches cooperatively with at
+// most one workgroup per compute unit (each uses the whole register file of
+// its CU).  Every wait is bounded by spin_limit polls; on expiry the kernel
 // records an error word and every workgroup drains.
 #include <algorithm>
 
@@ -54,35 +65,54 @@ struct PersistArgs {
   int pr;          // row slices per layer
   int groups;      // workgroups that take part (= L * PC * pr)
   int xcd_remap;   // 1: grid is a multiple of 8, map workgroups so a layer shares an XCD
+  int serial;      // 1: some workgroup's next item depends on its current one (no prefetch)
   int spin_limit;
   int dil[kMaxLayers];
 };
 
-__device__ __forceinline__ bool wait_count(int* flag, int target, int* status, int spin_limit) {
+typedef unsigned long long u64;
+
+__device__ __forceinline__ int flag_load(const int* flag) {
+  return __hip_atomic_load(flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+// Bounded wait until *flag >= target.  Every lane polls the same word, so the
+// result is wave-uniform.
+__device__ __forceinline__ bool wait_count(const int* flag, int target, int* status, int spin_limit) {
   int n = 0;
-  while (__hip_atomic_load(flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) < target) {
+  while (flag_load(flag) < target) {
     __builtin_amdgcn_s_sleep(1);
     if (++n >= spin_limit) {
       __hip_atomic_store(status, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       return false;
     }
-    if ((n & 1023) == 0 && __hip_atomic_load(status, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0) return false;
+    if ((n & 1023) == 0 && flag_load(status) != 0) return false;
   }
   return true;
 }
 
-template <int RT>
+// 8-byte agent-scope accesses: they bypass whatever a non-coherent cache level
+// may hold, with no ordering side effects of their own.
+__device__ __forceinline__ u64 coherent_load8(const float* p) {
+  return __hip_atomic_load(reinterpret_cast<const u64*>(p), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ void coherent_store8(float* p, float a, float b) {
+  u64 v = (u64)__float_as_uint(a) | ((u64)__float_as_uint(b) << 32);
+  __hip_atomic_store(reinterpret_cast<u64*>(p), v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+constexpr int P_TILE = 32 * P_LD;  // floats per LDS buffer
+constexpr int P_PF = 32;           // 8-byte prefetch registers per thread (8 rows x 512 floats per wave)
+
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1)))
 void lstm_persistent_kernel(PersistArgs a) {
-  extern __shared__ __attribute__((aligned(16))) float tile[];  // [32*RT][P_LD]
-  __shared__ int ok_s;
+  extern __shared__ __attribute__((aligned(16))) float tile[];  // [2][32][P_LD]
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = tid >> 6;
   const int j = lane & 31;
   const int hh = lane >> 5;
-  constexpr int ROWS = 32 * RT;
 
   int q = blockIdx.x;
   if (a.xcd_remap) q = (blockIdx.x & 7) * (gridDim.x >> 3) + (blockIdx.x >> 3);
@@ -95,6 +125,8 @@ void lstm_persistent_kernel(PersistArgs a) {
   const int d = a.dil[l];
   const int T = a.T, B = a.B;
   const size_t cell = (size_t)B * PH;
+  const int my_rbs = (a.nrb - prs + a.pr - 1) / a.pr;  // row blocks this workgroup walks per time step
+  const int n_items = T * my_rbs;
 
   // Resident weights: lane (i = j, half hh) of wave w holds, for MFMA step
   // s = 4q + c, WU[l][k = 8q + 4hh + c][gate(i)*H + 32pc + 8w + i%8].
@@ -119,104 +151,153 @@ void lstm_persistent_kernel(PersistArgs a) {
     }
   }
 
-  const int ld_c4 = tid & 63;   // float4 column within a 256-float half row
-  const int ld_r0 = tid >> 6;   // first row this thread stages
+  // Staging: wave w moves rows 8w..8w+7 of the tile; a row is 256 floats of x
+  // and 256 of h_prev, 128 eight-byte pieces each; lane handles pieces
+  // lane and lane+64 of either half.
+  u64 pf[P_PF];
+  bool alive = true;
 
-  for (int t = 0; t < T; ++t) {
-    const bool has_prev = t >= d;
+  auto item_t = [&](int n) { return n / my_rbs; };
+  auto item_rb = [&](int n) { return prs + a.pr * (n % my_rbs); };
+
+  // inputs of item n complete?  (blocking: bounded spin; otherwise one poll)
+  auto deps_ready = [&](int n, bool blocking) __attribute__((always_inline)) -> bool {
+    const int t = item_t(n), rb = item_rb(n);
+    bool ok = true;
+    if (l > 0) {
+      const int* f = a.flags + ((size_t)(l - 1) * T + t) * a.nrb + rb;
+      ok = blocking ? wait_count(f, PC, a.status, a.spin_limit) : (flag_load(f) >= PC);
+    }
+    if (ok && t >= d) {
+      const int* f = a.flags + ((size_t)l * T + (t - d)) * a.nrb + rb;
+      ok = blocking ? wait_count(f, PC, a.status, a.spin_limit) : (flag_load(f) >= PC);
+    }
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");  // data loads stay behind the flag reads
+    return ok;
+  };
+  auto issue_loads = [&](int n) __attribute__((always_inline)) {
+    const int t = item_t(n), rb = item_rb(n);
     const float* xsrc = (l == 0) ? a.xs + (size_t)t * cell : a.hsss + ((size_t)(l - 1) * T + t) * cell;
-    const float* hsrc = has_prev ? a.hsss + ((size_t)l * T + (t - d)) * cell : nullptr;
-    const float* csrc = has_prev ? a.csss + ((size_t)l * T + (t - d)) * cell : nullptr;
+    const bool has_prev = t >= d;
+    const float* hsrc = a.hsss + ((size_t)l * T + (has_prev ? t - d : 0)) * cell;
+#pragma unroll
+    for (int r = 0; r < 8; ++r) {
+      const int rg = min(rb * 32 + 8 * wave + r, B - 1);
+      pf[4 * r + 0] = coherent_load8(xsrc + (size_t)rg * PH + 2 * lane);
+      pf[4 * r + 1] = coherent_load8(xsrc + (size_t)rg * PH + 128 + 2 * lane);
+      if (has_prev) {
+        pf[4 * r + 2] = coherent_load8(hsrc + (size_t)rg * PH + 2 * lane);
+        pf[4 * r + 3] = coherent_load8(hsrc + (size_t)rg * PH + 128 + 2 * lane);
+      }
+    }
+  };
+  auto write_tile = [&](int n, int buf) __attribute__((always_inline)) {
+    const bool has_prev = item_t(n) >= d;
+    float* dst = tile + buf * P_TILE + (8 * wave) * P_LD + 2 * lane;
+#pragma unroll
+    for (int r = 0; r < 8; ++r) {
+      *reinterpret_cast<u64*>(dst + r * P_LD) = pf[4 * r + 0];
+      *reinterpret_cast<u64*>(dst + r * P_LD + 128) = pf[4 * r + 1];
+      if (has_prev) {
+        *reinterpret_cast<u64*>(dst + r * P_LD + 256) = pf[4 * r + 2];
+        *reinterpret_cast<u64*>(dst + r * P_LD + 384) = pf[4 * r + 3];
+      }
+    }
+  };
+
+  // prologue: first tile
+  alive = deps_ready(0, true);
+  if (alive) issue_loads(0);
+  if (alive) write_tile(0, 0);
+  __syncthreads();
+
+  for (int n = 0; n < n_items; ++n) {
+    const int buf = n & 1;
+    const int t = item_t(n), rb = item_rb(n);
+    const bool has_prev = t >= d;
+    const bool more = n + 1 < n_items;
     float* hdst = a.hsss + ((size_t)l * T + t) * cell;
     float* cdst = a.csss + ((size_t)l * T + t) * cell;
+    const int rg = rb * 32 + j;
+    const int rgc = min(rg, B - 1);
 
-    for (int rb = prs; rb < a.nrb; rb += a.pr) {
-      // ---- wait for the producers of this item's inputs
-      if (tid == 0) {
-        bool ok = true;
-        if (l > 0) ok = wait_count(a.flags + ((size_t)(l - 1) * T + t) * a.nrb + rb, PC, a.status, a.spin_limit);
-        if (ok && has_prev) ok = wait_count(a.flags + ((size_t)l * T + (t - d)) * a.nrb + rb, PC, a.status, a.spin_limit);
-        ok_s = ok ? 1 : 0;
+    // the next tile goes into flight now if its producers are already done;
+    // in serial mode (next item depends on this one) it can only start later
+    bool early = false;
+    if (alive && more && !a.serial) early = deps_ready(n + 1, false);
+    if (early) issue_loads(n + 1);
+
+    float4 cp = make_float4(0.f, 0.f, 0.f, 0.f);
+    if (alive && has_prev)
+      cp = *reinterpret_cast<const float4*>(a.csss + ((size_t)l * T + (t - d)) * cell + (size_t)rgc * PH + u0);
+
+    // ---- gates^T = WU^T * act^T on the matrix cores
+    v16f acc;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) acc[r] = 0.0f;
+    const float* arow = tile + buf * P_TILE + j * P_LD + 4 * hh;
+#pragma unroll
+    for (int qq = 0; qq < PH / 8; ++qq) {
+      const v4f b = *reinterpret_cast<const v4f*>(arow + 8 * qq);
+      acc = __builtin_amdgcn_mfma_f32_32x32x2f32(wr[4 * qq + 0], b[0], acc, 0, 0, 0);
+      acc = __builtin_amdgcn_mfma_f32_32x32x2f32(wr[4 * qq + 1], b[1], acc, 0, 0, 0);
+      acc = __builtin_amdgcn_mfma_f32_32x32x2f32(wr[4 * qq + 2], b[2], acc, 0, 0, 0);
+      acc = __builtin_amdgcn_mfma_f32_32x32x2f32(wr[4 * qq + 3], b[3], acc, 0, 0, 0);
+    }
+    if (has_prev) {
+#pragma unroll
+      for (int qq = PH / 8; qq < PK / 8; ++qq) {
+        const v4f b = *reinterpret_cast<const v4f*>(arow + 8 * qq);
+        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(wr[4 * qq + 0], b[0], acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(wr[4 * qq + 1], b[1], acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(wr[4 * qq + 2], b[2], acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(wr[4 * qq + 3], b[3], acc, 0, 0, 0);
       }
-      __syncthreads();  // also: every wave is done reading the previous tile
-      if (!ok_s) return;
-      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+    }
 
-      // ---- stage [x | h_prev] rows into LDS
-      const int row0 = rb * ROWS;
-#pragma unroll 4
-      for (int r = ld_r0; r < ROWS; r += 4) {
-        const int rg = min(row0 + r, B - 1);
-        const float4 xv = *reinterpret_cast<const float4*>(xsrc + (size_t)rg * PH + 4 * ld_c4);
-        *reinterpret_cast<float4*>(&tile[r * P_LD + 4 * ld_c4]) = xv;
-        if (has_prev) {
-          const float4 hv = *reinterpret_cast<const float4*>(hsrc + (size_t)rg * PH + 4 * ld_c4);
-          *reinterpret_cast<float4*>(&tile[r * P_LD + PH + 4 * ld_c4]) = hv;
-        }
+    // ---- state update, lane-local; h leaves through write-through stores
+    if (alive && rg < B) {
+      const float cpv[4] = {cp.x, cp.y, cp.z, cp.w};
+      float hv[4], cv[4];
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const float ig = sigmoid_f(acc[r] + bi[r]);
+        const float fg = sigmoid_f(acc[4 + r] + bf[r]);
+        const float og = sigmoid_f(acc[8 + r] + bo[r]);
+        const float cand = tanh_f(acc[12 + r] + bg[r]);
+        cv[r] = fg * cpv[r] + ig * cand;
+        hv[r] = og * tanh_f(cv[r]);
+      }
+      *reinterpret_cast<float4*>(cdst + (size_t)rg * PH + u0) = make_float4(cv[0], cv[1], cv[2], cv[3]);
+      coherent_store8(hdst + (size_t)rg * PH + u0, hv[0], hv[1]);
+      coherent_store8(hdst + (size_t)rg * PH + u0 + 2, hv[2], hv[3]);
+    }
+
+    if (!a.serial) {
+      // late start of the next tile: wait for its producers (never this item), then load
+      if (alive && more && !early) {
+        alive = deps_ready(n + 1, true);
+        if (alive) issue_loads(n + 1);
+      }
+      if (alive && more) write_tile(n + 1, buf ^ 1);
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+      __builtin_amdgcn_s_waitcnt(0);  // this wave's h stores are acknowledged
+      __syncthreads();
+      if (tid == 0 && alive)
+        __hip_atomic_fetch_add(a.flags + ((size_t)l * T + t) * a.nrb + rb, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    } else {
+      // the next item needs this one: publish first, then fetch
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+      __builtin_amdgcn_s_waitcnt(0);
+      __syncthreads();
+      if (tid == 0 && alive)
+        __hip_atomic_fetch_add(a.flags + ((size_t)l * T + t) * a.nrb + rb, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      if (alive && more) {
+        alive = deps_ready(n + 1, true);
+        if (alive) issue_loads(n + 1);
+        if (alive) write_tile(n + 1, buf ^ 1);
       }
       __syncthreads();
-
-      // ---- gates^T = WU^T * act^T on the matrix cores
-      v16f acc[RT];
-#pragma unroll
-      for (int rt = 0; rt < RT; ++rt)
-#pragma unroll
-        for (int r = 0; r < 16; ++r) acc[rt][r] = 0.0f;
-
-      const float* arow = &tile[j * P_LD + 4 * hh];
-#pragma unroll
-      for (int qq = 0; qq < PH / 8; ++qq) {
-#pragma unroll
-        for (int rt = 0; rt < RT; ++rt) {
-          const float4 b = *reinterpret_cast<const float4*>(arow + rt * 32 * P_LD + 8 * qq);
-          acc[rt] = __builtin_amdgcn_mfma_f32_32x32x2f32(wr[4 * qq + 0], b.x, acc[rt], 0, 0, 0);
-          acc[rt] = __builtin_amdgcn_mfma_f32_32x32x2f32(wr[4 * qq + 1], b.y, acc[rt], 0, 0, 0);
-          acc[rt] = __builtin_amdgcn_mfma_f32_32x32x2f32(wr[4 * qq + 2], b.z, acc[rt], 0, 0, 0);
-          acc[rt] = __builtin_amdgcn_mfma_f32_32x32x2f32(wr[4 * qq + 3], b.w, acc[rt], 0, 0, 0);
-        }
-      }
-      if (has_prev) {
-#pragma unroll
-        for (int qq = PH / 8; qq < PK / 8; ++qq) {
-#pragma unroll
-          for (int rt = 0; rt < RT; ++rt) {
-            const float4 b = *reinterpret_cast<const float4*>(arow + rt * 32 * P_LD + 8 * qq);
-            acc[rt] = __builtin_amdgcn_mfma_f32_32x32x2f32(wr[4 * qq + 0], b.x, acc[rt], 0, 0, 0);
-            acc[rt] = __builtin_amdgcn_mfma_f32_32x32x2f32(wr[4 * qq + 1], b.y, acc[rt], 0, 0, 0);
-            acc[rt] = __builtin_amdgcn_mfma_f32_32x32x2f32(wr[4 * qq + 2], b.z, acc[rt], 0, 0, 0);
-            acc[rt] = __builtin_amdgcn_mfma_f32_32x32x2f32(wr[4 * qq + 3], b.w, acc[rt], 0, 0, 0);
-          }
-        }
-      }
-
-      // ---- state update, lane-local
-#pragma unroll
-      for (int rt = 0; rt < RT; ++rt) {
-        const int rg = row0 + 32 * rt + j;
-        if (rg < B) {
-          float4 cp = make_float4(0.f, 0.f, 0.f, 0.f);
-          if (has_prev) cp = *reinterpret_cast<const float4*>(csrc + (size_t)rg * PH + u0);
-          const float cpv[4] = {cp.x, cp.y, cp.z, cp.w};
-          float hv[4], cv[4];
-#pragma unroll
-          for (int r = 0; r < 4; ++r) {
-            const float ig = sigmoid_f(acc[rt][r] + bi[r]);
-            const float fg = sigmoid_f(acc[rt][4 + r] + bf[r]);
-            const float og = sigmoid_f(acc[rt][8 + r] + bo[r]);
-            const float cand = tanh_f(acc[rt][12 + r] + bg[r]);
-            cv[r] = fg * cpv[r] + ig * cand;
-            hv[r] = og * tanh_f(cv[r]);
-          }
-          *reinterpret_cast<float4*>(cdst + (size_t)rg * PH + u0) = make_float4(cv[0], cv[1], cv[2], cv[3]);
-          *reinterpret_cast<float4*>(hdst + (size_t)rg * PH + u0) = make_float4(hv[0], hv[1], hv[2], hv[3]);
-        }
-      }
-
-      // ---- publish: every thread's stores first, then one count per workgroup
-      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
-      __syncthreads();
-      if (tid == 0)
-        __hip_atomic_fetch_add(a.flags + ((size_t)l * T + t) * a.nrb + rb, 1, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
     }
   }
 }
@@ -225,13 +306,8 @@ __global__ void fill_zero_kernel(int* p, size_t n) {
   for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x) p[i] = 0;
 }
 
-// Rows per item: 64 halves the per-item synchronisation cost, 32 gives a finer
-// pipeline (shorter fill) and double the items to spread over row slices.
-static int pick_rt(int B) { return B >= 64 ? 2 : 1; }
-
 static size_t flag_count(int L, int T, int B) {
-  const int rt = pick_rt(B);
-  const int nrb = (B + 32 * rt - 1) / (32 * rt);
+  const int nrb = (B + 31) / 32;
   return (size_t)L * T * nrb;
 }
 
@@ -242,11 +318,18 @@ static int run_persistent(const float* xs, const float* WU, const float* bias, c
   const DeviceProps* dp = nullptr;
   int rc = device_props(&dp);
   if (rc) return rc;
-  const int slots = dp->cus;
-  if (L > kMaxLayers || L * PC > slots) return FTK_OK;  // not enough compute units to pin every layer: fall back
-  const int rt = pick_rt(B);
-  const size_t lds = (size_t)32 * rt * P_LD * sizeof(float);
+  const size_t lds = (size_t)2 * P_TILE * sizeof(float);
   if ((int)lds > dp->lds_optin) return FTK_OK;
+  const void* fn = (const void*)lstm_persistent_kernel;
+  static bool attr_set = false;
+  if (!attr_set) {
+    FTK_HIP(hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+    attr_set = true;
+  }
+  int per_cu = 0;
+  FTK_HIP(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, fn, 256, lds));
+  const int slots = per_cu * dp->cus;
+  if (L > kMaxLayers || L * PC > slots) return FTK_OK;  // cannot pin every layer on its own compute units: fall back
 
   const size_t nflags = flag_count(L, T, B);
   const size_t need = (nflags + 64) * sizeof(int);
@@ -258,22 +341,26 @@ static int run_persistent(const float* xs, const float* WU, const float* bias, c
   a.status = reinterpret_cast<int*>(ws);
   a.flags = a.status + 64;
   a.L = L; a.T = T; a.B = B;
-  a.nrb = (B + 32 * rt - 1) / (32 * rt);
-  a.pr = std::max(1, std::min(slots / (L * PC), a.nrb));
+  a.nrb = (B + 31) / 32;
+  // spare compute units become row slices, but a workgroup keeps at least two
+  // row blocks when it can so that the next tile never depends on the current item
+  a.pr = std::max(1, std::min(slots / (L * PC), std::max(1, a.nrb / 2)));
   a.groups = L * PC * a.pr;
   a.spin_limit = 1 << 22;
-  for (int l = 0; l < kMaxLayers; ++l) a.dil[l] = (l < L && dil) ? dil[l] : 1;
-  int grid = a.groups;
-  a.xcd_remap = 0;
-  if (grid % 8 == 0) a.xcd_remap = 1;
+  const int min_rbs = a.nrb / a.pr;
+  a.serial = 0;
+  for (int l = 0; l < kMaxLayers; ++l) {
+    a.dil[l] = (l < L && dil) ? dil[l] : 1;
+    if (l < L && (long long)a.dil[l] * min_rbs < 2) a.serial = 1;
+  }
+  const int grid = a.groups;
+  a.xcd_remap = (grid % 8 == 0) ? 1 : 0;
 
   hipLaunchKernelGGL(fill_zero_kernel, dim3(64), dim3(256), 0, s, a.status, nflags + 64);
   rc = check_launch("fill_zero_kernel");
   if (rc) return rc;
 
   void* kargs[] = {&a};
-  const void* fn = rt == 2 ? (const void*)lstm_persistent_kernel<2> : (const void*)lstm_persistent_kernel<1>;
-  FTK_HIP(hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
   FTK_HIP(hipLaunchCooperativeKernel(fn, dim3(grid), dim3(256), kargs, (unsigned)lds, s));
   *handled = true;
   return FTK_OK;
