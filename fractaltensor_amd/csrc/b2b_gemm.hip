@@ -17,16 +17,28 @@
 //
 // A workgroup stages one problem's B and C in LDS once and then walks row tiles
 // of that problem, each wave 64 rows at a time (two 32-row tiles sharing every
-// B and C fragment read).  The A rows of a wave's first tile are requested
-// before the staging starts, so the HBM latency of A hides behind it.  The
-// grid is one-dimensional and remapped so that the workgroups of one problem
-// share an XCD (and with it the L2 copy of B and C).  D tiles go through an
-// LDS transpose so global stores are full 16-byte-per-lane row segments.
+// B and C fragment read).  A rows are fetched with fully coalesced 16-byte
+// loads (64 lanes = 4 whole rows), parked in a wave-private LDS region and read
+// back as fragments; the fetch for the wave's next 64 rows is issued before the
+// current rows go to the matrix cores, so reads, MFMAs and the D stores of
+// successive row groups overlap.  D tiles leave through the same wave-private
+// region so global stores are full 16-byte-per-lane row segments.  The grid is
+// one-dimensional and remapped so that the workgroups of one problem share an
+// XCD (and with it the L2 copy of B and C).
 #include <algorithm>
+#include <type_traits>
 
 #include "ftk_common.h"
 
 namespace ftk {
+
+template <int N, typename F>
+__device__ __forceinline__ void static_for(F&& f) {
+  if constexpr (N > 0) {
+    static_for<N - 1>(f);
+    f(std::integral_constant<int, N - 1>{});
+  }
+}
 
 constexpr int B2B_PTILE = 128;  // p columns per workgroup
 
@@ -36,15 +48,17 @@ struct B2BGrid {
   int per_problem;  // workgroups sharing one (problem, p tile)
   int ptiles;
   int total;        // per_problem * ptiles * G
+  int wave_region;  // halfs of wave-private LDS (A rows in, D rows out)
 };
 
-template <int KS>  // K = 16 * KS
-__global__ __launch_bounds__(512) void b2b_gemm_kernel(const _Float16* __restrict__ A,
+template <int KS, int PT>  // K = 16 * KS, 32 * PT columns of D per workgroup
+__global__ __launch_bounds__(256) void b2b_gemm_kernel(const _Float16* __restrict__ A,
                                                        const _Float16* __restrict__ Bm,
                                                        const _Float16* __restrict__ Cm, _Float16* __restrict__ D,
-                                                       int M, int N, int P, B2BGrid gr) {
+                                                       int M, int N, int P, int p_base, B2BGrid gr) {
   constexpr int K = 16 * KS;
-  constexpr int BLD = K + 8;  // padded Bs row (halfs)
+  constexpr int BLD = K + 8;  // padded Bs / A-staging row (halfs)
+  constexpr int AN = 2 * KS;  // 16-byte A loads per lane for 64 rows (64 rows * K/8 chunks over 64 lanes)
   const int CLD = N + 4;      // padded Cs row (halfs)
   const int threads = blockDim.x;
   const int waves = threads >> 6;
@@ -63,15 +77,14 @@ __global__ __launch_bounds__(512) void b2b_gemm_kernel(const _Float16* __restric
   const int pt_idx = (id / gr.per_problem) % gr.ptiles;
   const int g = id / (gr.per_problem * gr.ptiles);
 
-  const int p0 = pt_idx * B2B_PTILE;
-  const int pw = min(B2B_PTILE, P - p0);  // p columns handled here
-  const int np_tiles = pw / 32;           // 1..4
-  const int DLD = pw + 4;                 // padded D staging row (halfs)
+  constexpr int pw = 32 * PT;             // p columns handled here
+  constexpr int DLD = pw + 4;             // padded D staging row (halfs)
+  const int p0 = p_base + pt_idx * pw;
 
   _Float16* Bs = reinterpret_cast<_Float16*>(smem);  // [N][BLD]
   _Float16* Cs = Bs + N * BLD;                       // [pw][CLD]
-  _Float16* Ds = Cs + pw * CLD;                      // [waves][32][DLD]
-  _Float16* Dw = Ds + wave * 32 * DLD;
+  _Float16* Wa = Cs + pw * CLD + wave * gr.wave_region;  // wave-private: A rows in, [32][BLD]
+  _Float16* Ws = Wa + 32 * BLD;                          // wave-private: D rows out, [32][DLD]
 
   const _Float16* Ag = A + (size_t)g * M * K;
   const _Float16* Bg = Bm + (size_t)g * N * K;
@@ -82,22 +95,35 @@ __global__ __launch_bounds__(512) void b2b_gemm_kernel(const _Float16* __restric
   const int wave_stride = gr.per_problem * waves;
   int pair = part * waves + wave;
 
-  // ---- A row fragments: step s contracts k in [8s, 8s+8) (lanes 0-31) and
-  //      [K/2 + 8s, K/2 + 8s + 8) (lanes 32-63): 16*KS contiguous bytes per lane
-  v8h afrag[2][KS];
-  auto load_a = [&](int pr_) __attribute__((always_inline)) {
-#pragma unroll
-    for (int rt = 0; rt < 2; ++rt) {
-      const int row_c = min(pr_ * 64 + 32 * rt + j, M - 1);
-      const _Float16* arow = Ag + (size_t)row_c * K + hh * (K / 2);
-#pragma unroll
-      for (int s = 0; s < KS; ++s) {
-        const v4u v = ldg16(arow + 8 * s);
-        afrag[rt][s] = *reinterpret_cast<const v8h*>(&v);
-      }
-    }
+  // ---- coalesced fetch of 64 A rows: load u covers 16-byte chunks u*64 + lane of the row group
+  constexpr int CPR = K / 8;  // 16-byte chunks per row
+  v4u areg[AN];
+  auto fetch_a = [&](int pr_) __attribute__((always_inline)) {
+    static_for<AN>([&](auto uc) __attribute__((always_inline)) {
+      constexpr int u = decltype(uc)::value;
+      const int chunk = u * 64 + lane;
+      const int row = min(pr_ * 64 + chunk / CPR, M - 1);
+      areg[u] = ldg16(Ag + (size_t)row * K + 8 * (chunk % CPR));
+    });
   };
-  if (pair < row_pairs) load_a(pair);
+  // park them in the wave's LDS region, then pull the MFMA fragments: step s
+  // contracts k in [8s, 8s+8) (lanes 0-31) and [K/2 + 8s, K/2 + 8s + 8) (lanes 32-63)
+  v8h afrag[2][KS];
+  auto park_a = [&]() __attribute__((always_inline)) {
+    // 32 rows at a time through the same region; LDS operations of a wave complete in order
+    static_for<2>([&](auto rtc) __attribute__((always_inline)) {
+      constexpr int rt = decltype(rtc)::value;
+      static_for<AN / 2>([&](auto uc) __attribute__((always_inline)) {
+        constexpr int u = decltype(uc)::value;
+        const int chunk = u * 64 + lane;  // chunk within this 32-row half
+        *reinterpret_cast<v4u*>(Wa + (chunk / CPR) * BLD + 8 * (chunk % CPR)) = areg[rt * (AN / 2) + u];
+      });
+#pragma unroll
+      for (int s = 0; s < KS; ++s)
+        afrag[rt][s] = *reinterpret_cast<const v8h*>(Wa + j * BLD + hh * (K / 2) + 8 * s);
+    });
+  };
+  if (pair < row_pairs) fetch_a(pair);
 
   // ---- stage this problem's Bs[n][k] and Cs[p][n]: loads in batches of four
   {
@@ -143,12 +169,19 @@ __global__ __launch_bounds__(512) void b2b_gemm_kernel(const _Float16* __restric
   }
   __syncthreads();
 
+  // Software pipeline per wave: the fragments of row group n+1 are parked and
+  // the fetch of group n+2 issued between the arithmetic of group n and its D
+  // stores, so every load and store has a whole arithmetic phase to complete.
+  if (pair < row_pairs) {
+    park_a();
+    if (pair + wave_stride < row_pairs) fetch_a(pair + wave_stride);
+  }
   for (; pair < row_pairs; pair += wave_stride) {
-    v16f dacc[2][4];
+    v16f dacc[2][PT];
 #pragma unroll
     for (int rt = 0; rt < 2; ++rt)
 #pragma unroll
-      for (int pt = 0; pt < 4; ++pt)
+      for (int pt = 0; pt < PT; ++pt)
 #pragma unroll
         for (int r = 0; r < 16; ++r) dacc[rt][pt][r] = 0.0f;
 
@@ -176,49 +209,47 @@ __global__ __launch_bounds__(512) void b2b_gemm_kernel(const _Float16* __restric
           for (int e = 0; e < 8; ++e) pf[rt][s][e] = (_Float16)pacc[rt][8 * s + e];
       // GEMM2: D^T[p tile] += Cs[p][n] * P
 #pragma unroll
-      for (int pt = 0; pt < 4; ++pt) {
-        if (pt < np_tiles) {
-          const _Float16* crow = Cs + (pt * 32 + j) * CLD + nt * 32 + 4 * hh;
+      for (int pt = 0; pt < PT; ++pt) {
+        const _Float16* crow = Cs + (pt * 32 + j) * CLD + nt * 32 + 4 * hh;
 #pragma unroll
-          for (int s = 0; s < 2; ++s) {
-            const v4h c0 = *reinterpret_cast<const v4h*>(crow + 16 * s);
-            const v4h c1 = *reinterpret_cast<const v4h*>(crow + 16 * s + 8);
-            const v8h cfrag = {c0[0], c0[1], c0[2], c0[3], c1[0], c1[1], c1[2], c1[3]};
-            dacc[0][pt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(cfrag, pf[0][s], dacc[0][pt], 0, 0, 0);
-            dacc[1][pt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(cfrag, pf[1][s], dacc[1][pt], 0, 0, 0);
-          }
+        for (int s = 0; s < 2; ++s) {
+          const v4h c0 = *reinterpret_cast<const v4h*>(crow + 16 * s);
+          const v4h c1 = *reinterpret_cast<const v4h*>(crow + 16 * s + 8);
+          const v8h cfrag = {c0[0], c0[1], c0[2], c0[3], c1[0], c1[1], c1[2], c1[3]};
+          dacc[0][pt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(cfrag, pf[0][s], dacc[0][pt], 0, 0, 0);
+          dacc[1][pt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(cfrag, pf[1][s], dacc[1][pt], 0, 0, 0);
         }
       }
     }
 
-    // next pair's A rows go into flight while this pair's D drains
-    const int this_pair = pair;
-    if (pair + wave_stride < row_pairs) load_a(pair + wave_stride);
+    if (pair + wave_stride < row_pairs) {
+      park_a();
+      if (pair + 2 * wave_stride < row_pairs) fetch_a(pair + 2 * wave_stride);
+    }
 
-    // ---- epilogue: D^T accumulators -> LDS [row][p] -> 16-byte row segments.
-    // A wave reads back only what it wrote itself and LDS operations of one
-    // wave complete in order, so no workgroup barrier is needed.
+    // ---- epilogue: D^T accumulators -> wave-private LDS [row][p] -> 16-byte
+    // row segments.  A wave reads back only what it wrote itself and LDS
+    // operations of one wave complete in order, so no barrier is needed.
 #pragma unroll
     for (int rt = 0; rt < 2; ++rt) {
 #pragma unroll
-      for (int pt = 0; pt < 4; ++pt) {
-        if (pt < np_tiles) {
+      for (int pt = 0; pt < PT; ++pt) {
 #pragma unroll
-          for (int gq = 0; gq < 4; ++gq) {
-            const v4h o = {(_Float16)dacc[rt][pt][4 * gq + 0], (_Float16)dacc[rt][pt][4 * gq + 1],
-                           (_Float16)dacc[rt][pt][4 * gq + 2], (_Float16)dacc[rt][pt][4 * gq + 3]};
-            *reinterpret_cast<v4h*>(Dw + j * DLD + pt * 32 + 8 * gq + 4 * hh) = o;
-          }
+        for (int gq = 0; gq < 4; ++gq) {
+          const v4h o = {(_Float16)dacc[rt][pt][4 * gq + 0], (_Float16)dacc[rt][pt][4 * gq + 1],
+                         (_Float16)dacc[rt][pt][4 * gq + 2], (_Float16)dacc[rt][pt][4 * gq + 3]};
+          *reinterpret_cast<v4h*>(Ws + j * DLD + pt * 32 + 8 * gq + 4 * hh) = o;
         }
       }
-      const int segs = np_tiles * 4;  // 16-byte segments per row
+      constexpr int segs = PT * 4;  // 16-byte segments per row
+#pragma unroll
       for (int idx = lane; idx < 32 * segs; idx += 64) {
         const int r = idx / segs;
         const int sg = idx - r * segs;
-        const int grow = this_pair * 64 + 32 * rt + r;
+        const int grow = pair * 64 + 32 * rt + r;
         if (grow < M) {
-          const v2u lo = *reinterpret_cast<const v2u*>(Dw + r * DLD + 8 * sg);
-          const v2u hi = *reinterpret_cast<const v2u*>(Dw + r * DLD + 8 * sg + 4);
+          const v2u lo = *reinterpret_cast<const v2u*>(Ws + r * DLD + 8 * sg);
+          const v2u hi = *reinterpret_cast<const v2u*>(Ws + r * DLD + 8 * sg + 4);
           *reinterpret_cast<v4u*>(Dg + (size_t)grow * P + 8 * sg) = v4u{lo[0], lo[1], hi[0], hi[1]};
         }
       }
@@ -226,16 +257,18 @@ __global__ __launch_bounds__(512) void b2b_gemm_kernel(const _Float16* __restric
   }
 }
 
+static int b2b_wave_region(int K, int pw) { return 32 * (K + 8) + 32 * (pw + 4); }
+
 static size_t b2b_lds_bytes(int N, int K, int pw, int waves) {
-  return (size_t)(N * (K + 8) + pw * (N + 4) + waves * 32 * (pw + 4)) * 2;
+  return (size_t)(N * (K + 8) + pw * (N + 4) + waves * b2b_wave_region(K, pw)) * 2;
 }
 
-template <int KS>
-static int launch_b2b(const void* A, const void* B, const void* C, void* D, int G, int M, int N, int P, int cus,
-                      int lds_max, hipStream_t s) {
+template <int KS, int PT>
+static int launch_b2b_cols(const void* A, const void* B, const void* C, void* D, int G, int M, int N, int P,
+                           int p_base, int ptiles, int cus, int lds_max, hipStream_t s) {
   constexpr int K = 16 * KS;
-  const int pw = std::min(P, B2B_PTILE);
-  int waves = 8;
+  constexpr int pw = 32 * PT;
+  int waves = 4;
   while (waves > 1 && (int)b2b_lds_bytes(N, K, pw, waves) > lds_max) waves >>= 1;
   const size_t lds = b2b_lds_bytes(N, K, pw, waves);
   if ((int)lds > lds_max)
@@ -243,7 +276,8 @@ static int launch_b2b(const void* A, const void* B, const void* C, void* D, int 
                 "ftk_b2b_gemm_f16: B and C tiles for N=%d K=%d P=%d need %zu bytes of LDS, the device has %d", N, K, P,
                 lds, lds_max);
   B2BGrid gr;
-  gr.ptiles = (P + B2B_PTILE - 1) / B2B_PTILE;
+  gr.ptiles = ptiles;
+  gr.wave_region = b2b_wave_region(K, pw);
   const int row_pairs = (M + 63) / 64;
   const long long units = (long long)G * gr.ptiles;
   // enough workgroups per (problem, p tile) to fill the chip once; each walks its share of the rows
@@ -253,15 +287,34 @@ static int launch_b2b(const void* A, const void* B, const void* C, void* D, int 
   const long long total = units * per;
   if (total > 0x7fffffffLL) return fail(FTK_ERR_UNSUPPORTED_SHAPE, "ftk_b2b_gemm_f16: grid too large");
   gr.total = (int)total;
-  const void* fn = (const void*)b2b_gemm_kernel<KS>;
+  const void* fn = (const void*)b2b_gemm_kernel<KS, PT>;
   static int attr_lds = 0;
   if ((int)lds > attr_lds) {
     FTK_HIP(hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
     attr_lds = (int)lds;
   }
-  hipLaunchKernelGGL(b2b_gemm_kernel<KS>, dim3(gr.total), dim3(waves * 64), lds, s, (const _Float16*)A,
-                     (const _Float16*)B, (const _Float16*)C, (_Float16*)D, M, N, P, gr);
+  hipLaunchKernelGGL((b2b_gemm_kernel<KS, PT>), dim3(gr.total), dim3(waves * 64), lds, s, (const _Float16*)A,
+                     (const _Float16*)B, (const _Float16*)C, (_Float16*)D, M, N, P, p_base, gr);
   return check_launch("b2b_gemm_kernel");
+}
+
+// Columns of D go out in workgroup tiles of 128; a remainder of 32, 64 or 96
+// columns is a second launch of the narrower instantiation.
+template <int KS>
+static int launch_b2b(const void* A, const void* B, const void* C, void* D, int G, int M, int N, int P, int cus,
+                      int lds_max, hipStream_t s) {
+  const int full = P / B2B_PTILE;
+  const int rem = (P % B2B_PTILE) / 32;
+  int rc = FTK_OK;
+  if (full > 0) rc = launch_b2b_cols<KS, 4>(A, B, C, D, G, M, N, P, 0, full, cus, lds_max, s);
+  if (rc) return rc;
+  const int pb = full * B2B_PTILE;
+  switch (rem) {
+    case 1: return launch_b2b_cols<KS, 1>(A, B, C, D, G, M, N, P, pb, 1, cus, lds_max, s);
+    case 2: return launch_b2b_cols<KS, 2>(A, B, C, D, G, M, N, P, pb, 1, cus, lds_max, s);
+    case 3: return launch_b2b_cols<KS, 3>(A, B, C, D, G, M, N, P, pb, 1, cus, lds_max, s);
+    default: return FTK_OK;
+  }
 }
 
 }  // namespace ftk

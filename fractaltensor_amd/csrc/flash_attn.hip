@@ -162,7 +162,8 @@ __global__ __launch_bounds__(WAVES * 64) void flash_attn_kernel(const _Float16* 
   store_tile(0);
   __syncthreads();
 
-  for (int kt = 0; kt < ntiles; ++kt) {
+  auto process_tile = [&](int kt, auto ragged_c) __attribute__((always_inline)) {
+    constexpr bool ragged = decltype(ragged_c)::value;
     const int buf = kt & 1;
     if (kt + 1 < ntiles) load_tile(kt + 1);
     const _Float16* ks = Ks + buf * KSZ;
@@ -194,11 +195,10 @@ __global__ __launch_bounds__(WAVES * 64) void flash_attn_kernel(const _Float16* 
     // reference maximum that is only moved (and O, l rescaled) when the true
     // row maximum has run ahead of it by more than FA_TAU in exponent units:
     // any m_ref gives the same O = acc/l, p merely ranges up to 2^FA_TAU.
-    const bool ragged = (kt + 1 == ntiles) && (Skv % FA_KT != 0);
     v8h pf[QT][2][2];
 #pragma unroll
     for (int qt = 0; qt < QT; ++qt) {
-      if (ragged) {
+      if constexpr (ragged) {
 #pragma unroll
         for (int k2 = 0; k2 < 2; ++k2)
 #pragma unroll
@@ -231,10 +231,14 @@ __global__ __launch_bounds__(WAVES * 64) void flash_attn_kernel(const _Float16* 
 #pragma unroll
         for (int s = 0; s < 2; ++s)
 #pragma unroll
-          for (int e = 0; e < 8; ++e) {
-            const float p = __builtin_amdgcn_exp2f(__builtin_fmaf(sacc[qt][k2][8 * s + e], scale_log2e, mc));
-            psum += p;
-            pf[qt][k2][s][e] = (_Float16)p;
+          for (int e = 0; e < 8; e += 2) {
+            const float p0 = __builtin_amdgcn_exp2f(__builtin_fmaf(sacc[qt][k2][8 * s + e], scale_log2e, mc));
+            const float p1 = __builtin_amdgcn_exp2f(__builtin_fmaf(sacc[qt][k2][8 * s + e + 1], scale_log2e, mc));
+            const v2h pp = {(_Float16)p0, (_Float16)p1};
+            pf[qt][k2][s][e] = pp[0];
+            pf[qt][k2][s][e + 1] = pp[1];
+            // row sum over the rounded values that enter the PV product, two per instruction
+            psum = __builtin_amdgcn_fdot2(pp, v2h{(_Float16)1.0f, (_Float16)1.0f}, psum, false);
           }
       l_run[qt] += psum;  // this lane's half of the row sum
     }
@@ -258,7 +262,12 @@ __global__ __launch_bounds__(WAVES * 64) void flash_attn_kernel(const _Float16* 
 
     if (kt + 1 < ntiles) store_tile(buf ^ 1);
     __syncthreads();
-  }
+  };
+
+  const bool has_ragged = (Skv % FA_KT) != 0;
+  const int nfull = has_ragged ? ntiles - 1 : ntiles;
+  for (int kt = 0; kt < nfull; ++kt) process_tile(kt, std::false_type{});
+  if (has_ragged) process_tile(ntiles - 1, std::true_type{});
 
   // ---- normalise and store: lane holds d = 32dt + 8g + 4*half + r of its row
 #pragma unroll

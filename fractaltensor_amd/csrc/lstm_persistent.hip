@@ -36,6 +36,8 @@
 // most one workgroup per compute unit (each uses the whole register file of
 // its CU).  Every wait is bounded by spin_limit polls; on expiry the kernel
 // records an error word and every workgroup drains.
+#include <stdlib.h>
+
 #include <algorithm>
 
 #include "ftk_common.h"
@@ -67,6 +69,8 @@ struct PersistArgs {
   int xcd_remap;   // 1: grid is a multiple of 8, map workgroups so a layer shares an XCD
   int serial;      // 1: some workgroup's next item depends on its current one (no prefetch)
   int spin_limit;
+  int trace_q;            // logical workgroup whose item timeline is recorded, or -1
+  long long* trace;       // [items][5] 100 MHz clock stamps of that workgroup
   int dil[kMaxLayers];
 };
 
@@ -211,8 +215,10 @@ void lstm_persistent_kernel(PersistArgs a) {
   if (alive) write_tile(0, 0);
   __syncthreads();
 
+  const bool tracing = (q == a.trace_q) && tid == 0;
   for (int n = 0; n < n_items; ++n) {
     const int buf = n & 1;
+    if (tracing) a.trace[5 * n + 0] = wall_clock64();
     const int t = item_t(n), rb = item_rb(n);
     const bool has_prev = t >= d;
     const bool more = n + 1 < n_items;
@@ -221,39 +227,59 @@ void lstm_persistent_kernel(PersistArgs a) {
     const int rg = rb * 32 + j;
     const int rgc = min(rg, B - 1);
 
-    // the next tile goes into flight now if its producers are already done;
-    // in serial mode (next item depends on this one) it can only start later
-    bool early = false;
-    if (alive && more && !a.serial) early = deps_ready(n + 1, false);
-    if (early) issue_loads(n + 1);
-
     float4 cp = make_float4(0.f, 0.f, 0.f, 0.f);
     if (alive && has_prev)
       cp = *reinterpret_cast<const float4*>(a.csss + ((size_t)l * T + (t - d)) * cell + (size_t)rgc * PH + u0);
 
-    // ---- gates^T = WU^T * act^T on the matrix cores
-    v16f acc;
+    // the next item's flags are requested now and looked at half way through
+    // the item, so their round trip to memory is off the critical path
+    int f_below = PC, f_own = PC;
+    if (more && !a.serial) {
+      const int t1 = item_t(n + 1), rb1 = item_rb(n + 1);
+      if (l > 0) f_below = flag_load(a.flags + ((size_t)(l - 1) * T + t1) * a.nrb + rb1);
+      if (t1 >= d) f_own = flag_load(a.flags + ((size_t)l * T + (t1 - d)) * a.nrb + rb1);
+    }
+
+    // ---- gates^T = WU^T * act^T on the matrix cores; two accumulators so
+    // that consecutive MFMAs never wait on each other's result
+    v16f acc0, acc1;
 #pragma unroll
-    for (int r = 0; r < 16; ++r) acc[r] = 0.0f;
+    for (int r = 0; r < 16; ++r) { acc0[r] = 0.0f; acc1[r] = 0.0f; }
     const float* arow = tile + buf * P_TILE + j * P_LD + 4 * hh;
 #pragma unroll
     for (int qq = 0; qq < PH / 8; ++qq) {
       const v4f b = *reinterpret_cast<const v4f*>(arow + 8 * qq);
-      acc = __builtin_amdgcn_mfma_f32_32x32x2f32(wr[4 * qq + 0], b[0], acc, 0, 0, 0);
-      acc = __builtin_amdgcn_mfma_f32_32x32x2f32(wr[4 * qq + 1], b[1], acc, 0, 0, 0);
-      acc = __builtin_amdgcn_mfma_f32_32x32x2f32(wr[4 * qq + 2], b[2], acc, 0, 0, 0);
-      acc = __builtin_amdgcn_mfma_f32_32x32x2f32(wr[4 * qq + 3], b[3], acc, 0, 0, 0);
+      acc0 = __builtin_amdgcn_mfma_f32_32x32x2f32(wr[4 * qq + 0], b[0], acc0, 0, 0, 0);
+      acc1 = __builtin_amdgcn_mfma_f32_32x32x2f32(wr[4 * qq + 1], b[1], acc1, 0, 0, 0);
+      acc0 = __builtin_amdgcn_mfma_f32_32x32x2f32(wr[4 * qq + 2], b[2], acc0, 0, 0, 0);
+      acc1 = __builtin_amdgcn_mfma_f32_32x32x2f32(wr[4 * qq + 3], b[3], acc1, 0, 0, 0);
     }
+    if (tracing) a.trace[5 * n + 1] = wall_clock64();
+
+    // Half way through the item, fetch the next tile: wait (bounded) for its
+    // producers, then put its loads in flight behind the rest of the MFMAs.
+    // Waiting here rather than at the end of the item makes each layer settle
+    // about one and a half items behind the layer below, which is what lets
+    // the loads overlap the arithmetic in steady state.
+    if (alive && more && !a.serial) {
+      if (f_below < PC || f_own < PC) alive = deps_ready(n + 1, true);
+      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+      if (alive) issue_loads(n + 1);
+    }
+
     if (has_prev) {
 #pragma unroll
       for (int qq = PH / 8; qq < PK / 8; ++qq) {
         const v4f b = *reinterpret_cast<const v4f*>(arow + 8 * qq);
-        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(wr[4 * qq + 0], b[0], acc, 0, 0, 0);
-        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(wr[4 * qq + 1], b[1], acc, 0, 0, 0);
-        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(wr[4 * qq + 2], b[2], acc, 0, 0, 0);
-        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(wr[4 * qq + 3], b[3], acc, 0, 0, 0);
+        acc0 = __builtin_amdgcn_mfma_f32_32x32x2f32(wr[4 * qq + 0], b[0], acc0, 0, 0, 0);
+        acc1 = __builtin_amdgcn_mfma_f32_32x32x2f32(wr[4 * qq + 1], b[1], acc1, 0, 0, 0);
+        acc0 = __builtin_amdgcn_mfma_f32_32x32x2f32(wr[4 * qq + 2], b[2], acc0, 0, 0, 0);
+        acc1 = __builtin_amdgcn_mfma_f32_32x32x2f32(wr[4 * qq + 3], b[3], acc1, 0, 0, 0);
       }
     }
+    v16f acc;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) acc[r] = acc0[r] + acc1[r];
 
     // ---- state update, lane-local; h leaves through write-through stores
     if (alive && rg < B) {
@@ -273,16 +299,14 @@ void lstm_persistent_kernel(PersistArgs a) {
       coherent_store8(hdst + (size_t)rg * PH + u0 + 2, hv[2], hv[3]);
     }
 
+    if (tracing) a.trace[5 * n + 2] = wall_clock64();
     if (!a.serial) {
-      // late start of the next tile: wait for its producers (never this item), then load
-      if (alive && more && !early) {
-        alive = deps_ready(n + 1, true);
-        if (alive) issue_loads(n + 1);
-      }
       if (alive && more) write_tile(n + 1, buf ^ 1);
       __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
       __builtin_amdgcn_s_waitcnt(0);  // this wave's h stores are acknowledged
+      if (tracing) a.trace[5 * n + 3] = wall_clock64();
       __syncthreads();
+      if (tracing) a.trace[5 * n + 4] = wall_clock64();
       if (tid == 0 && alive)
         __hip_atomic_fetch_add(a.flags + ((size_t)l * T + t) * a.nrb + rb, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     } else {
@@ -311,6 +335,22 @@ static size_t flag_count(int L, int T, int B) {
   return (size_t)L * T * nrb;
 }
 
+// Workspace layout: [64 ints: status][flags][trace: T*nrb*5 stamps of 8 bytes].
+static size_t trace_offset_bytes(int L, int T, int B) { return ((flag_count(L, T, B) + 64) * sizeof(int) + 15) / 16 * 16; }
+static size_t workspace_need(int L, int T, int B) {
+  return trace_offset_bytes(L, T, B) + (size_t)T * ((B + 31) / 32) * 5 * sizeof(long long);
+}
+
+// Tuning hook: FTK_LSTM_TRACE=<logical workgroup> records that workgroup's per-item timeline.
+static int trace_workgroup() {
+  static int v = -2;
+  if (v == -2) {
+    const char* e = getenv("FTK_LSTM_TRACE");
+    v = e ? atoi(e) : -1;
+  }
+  return v;
+}
+
 static int run_persistent(const float* xs, const float* WU, const float* bias, const int* dil, float* hsss,
                           float* csss, int L, int T, int B, void* ws, size_t ws_bytes, hipStream_t s,
                           bool* handled) {
@@ -332,7 +372,7 @@ static int run_persistent(const float* xs, const float* WU, const float* bias, c
   if (L > kMaxLayers || L * PC > slots) return FTK_OK;  // cannot pin every layer on its own compute units: fall back
 
   const size_t nflags = flag_count(L, T, B);
-  const size_t need = (nflags + 64) * sizeof(int);
+  const size_t need = workspace_need(L, T, B);
   if (!ws || ws_bytes < need)
     return fail(FTK_ERR_WORKSPACE, "stacked LSTM needs a %zu-byte workspace, got %zu", need, ws_bytes);
 
@@ -347,6 +387,8 @@ static int run_persistent(const float* xs, const float* WU, const float* bias, c
   a.pr = std::max(1, std::min(slots / (L * PC), std::max(1, a.nrb / 2)));
   a.groups = L * PC * a.pr;
   a.spin_limit = 1 << 22;
+  a.trace_q = trace_workgroup();
+  a.trace = reinterpret_cast<long long*>(reinterpret_cast<char*>(ws) + trace_offset_bytes(L, T, B));
   const int min_rbs = a.nrb / a.pr;
   a.serial = 0;
   for (int l = 0; l < kMaxLayers; ++l) {
@@ -396,7 +438,7 @@ extern "C" {
 
 size_t ftk_stacked_lstm_workspace_bytes(int L, int T, int B, int H) {
   if (L <= 0 || T <= 0 || B <= 0 || H <= 0) return 0;
-  return (ftk::flag_count(L, T, B) + 64) * sizeof(int);
+  return ftk::workspace_need(L, T, B);
 }
 
 int ftk_stacked_lstm_f32(const float* xs, const float* WU, const float* bias, float* hsss, float* csss, int L, int T,

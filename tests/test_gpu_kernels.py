@@ -140,7 +140,9 @@ def test_stacked_lstm_config4_full_size(core):
     h1, c1 = core.stacked_lstm(dx, dW)
     h2, c2 = core.stacked_lstm(dx, dW, schedule='wavefront')
     torch.cuda.synchronize()
-    assert torch.equal(h1, h2) or ko.max_rel_err(h1.cpu().numpy(), h2.cpu().numpy()) < 1e-6
+    # two GPU schedules with different fp32 summation orders: equal to well inside the tolerance
+    e12 = ko.max_rel_err(h1.cpu().numpy(), h2.cpu().numpy())
+    assert e12 <= LSTM_TOL / 4, f'persistent vs per-stage launches: {e12:.3e}'
     rows = [0, 31, 32, 100, 255]
     hr, cr = ko.stacked_lstm(xs[:, rows], WU, None)
     assert_lstm_close(h1[:, :, rows], hr, 'hsss rows'); assert_lstm_close(c1[:, :, rows], cr, 'csss rows')
