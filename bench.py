@@ -1,0 +1,309 @@
+#!/usr/bin/env python3
+"""Benchmark of the FractalTensor hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload b2b|attention|stacked_lstm|dilated_lstm]
+                    [--no-extras] [--no-cpu]
+
+Prints ONE JSON line.  The headline workload is BASELINE.json configs[1], the
+fused back-to-back fp16 GEMM (32 problems of [4096,128]x[128,128]x[128,128]);
+the other single-GPU configurations (flash attention, stacked LSTM, dilated
+LSTM) are measured the same way and reported under "other_workloads" unless
+--no-extras is given.  A step is one pass of the kernel over one batch of
+synthetic input that is already resident in HBM.  For the B2B GEMM the timed
+steps walk a ring of input sets larger than the 256 MB memory-side cache, so
+the figure is an HBM figure; the same-buffers figure is reported next to it.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+# MI355X published peaks (dense)
+PEAK_HBM_GBS = 8000.0
+PEAK_F16_TFLOPS = 2500.0
+PEAK_F32_MATRIX_TFLOPS = 157.3
+
+# HBM traffic per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
+# (profiles/*_pmc.txt name the commands); None = not measured for that kernel.
+MEASURED_TRAFFIC_BYTES = {}
+try:
+    with open(os.path.join(ROOT, 'profiles', 'traffic.json')) as _f:
+        MEASURED_TRAFFIC_BYTES = json.load(_f)
+except Exception:
+    pass
+
+
+def _events_ms(torch, fn, steps, warmup):
+    """Average duration of fn over `steps` launches, HIP events on the launch stream."""
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    start = torch.cuda.Event(enable_timing=True)
+    end = torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    start.record()
+    for _ in range(steps):
+        fn()
+    end.record()
+    torch.cuda.synchronize()
+    wall = (time.perf_counter() - t0) * 1e3 / steps
+    return start.elapsed_time(end) / steps, wall
+
+
+def bench_b2b(torch, core, steps, warmup, cpu):
+    G, M, N, K, P = 32, 4096, 128, 128, 128
+    flop = 2.0 * G * M * N * (K + P)
+    nbytes = 2.0 * G * (M * K + N * K + P * N + M * P)
+    gen = torch.Generator(device='cpu').manual_seed(1234)
+    ring = 8   # 8 x 69 MB of operands and results: larger than the 256 MB memory-side cache
+    sets = []
+    for _ in range(ring):
+        A = (torch.randn((G, M, K), generator=gen) / K ** 0.5).half().cuda()
+        Bn = (torch.randn((G, N, K), generator=gen) / K ** 0.5).half().cuda()
+        Cp = (torch.randn((G, P, N), generator=gen) / N ** 0.5).half().cuda()
+        D = torch.empty((G, M, P), dtype=torch.float16, device='cuda')
+        sets.append((A, Bn, Cp, D))
+    state = {'i': 0}
+
+    def step_ring():
+        A, Bn, Cp, D = sets[state['i'] % ring]
+        state['i'] += 1
+        core.b2b_gemm(A, Bn, Cp, out=D)
+
+    def step_same():
+        A, Bn, Cp, D = sets[0]
+        core.b2b_gemm(A, Bn, Cp, out=D)
+
+    ms, wall = _events_ms(torch, step_ring, steps, warmup)
+    ms_same, _ = _events_ms(torch, step_same, steps, warmup)
+    res = {
+        'metric': 'TFLOP/s + % MFMA peak (B2B GEMM)',
+        'value': flop / ms / 1e9, 'unit': 'TFLOP/s', 'ms_per_step': ms, 'dtype': 'f16',
+        'config': {'workload': 'fused back-to-back GEMM D=(A@B)@C, BASELINE.json configs[1]',
+                   'problems': G, 'M': M, 'N': N, 'K': K, 'P': P, 'accumulate': 'f32',
+                   'inputs': 'ring of 8 operand sets (553 MB) so steps read HBM, not the memory-side cache'},
+        'pct_f16_mfma_peak': 100.0 * flop / ms / 1e9 / PEAK_F16_TFLOPS,
+        'same_buffers': {'ms_per_step': ms_same, 'tflops': flop / ms_same / 1e9, 'gbs': nbytes / ms_same / 1e6},
+        'host_wall_ms_per_step': wall,
+        'roofline': {'bound': 'hbm', 'achieved': nbytes / ms / 1e6, 'peak': PEAK_HBM_GBS, 'unit': 'GB/s',
+                     'frac': nbytes / ms / 1e6 / PEAK_HBM_GBS,
+                     'traffic': MEASURED_TRAFFIC_BYTES.get('b2b_gemm_kernel'),
+                     'kernel': 'b2b_gemm_kernel<8,4>', 'algorithmic_bytes_per_launch': nbytes},
+    }
+    if cpu:
+        from oracle import c_oracle
+        sample = 12   # problems of the 32
+        A, Bn, Cp, _ = sets[0]
+        a, b, c = (x[:sample].cpu().numpy() for x in (A, Bn, Cp))
+        t0 = time.perf_counter()
+        c_oracle.b2b_gemm(a, b, c, round_intermediate=True)
+        dt = time.perf_counter() - t0
+        res['cpu_baseline'] = {'value': flop * sample / G / dt / 1e12, 'unit': 'TFLOP/s', 'cores': 1, 'kind': 'port',
+                               'sample': f'{sample} of the {G} problems through oracle/oracle.c (scalar C, one thread), '
+                                         f'{dt:.1f} s'}
+    return res
+
+
+def bench_attention(torch, core, steps, warmup, cpu):
+    B, Hd, S, D = 8, 16, 2048, 128
+    flop = 4.0 * B * Hd * S * S * D
+    gen = torch.Generator(device='cpu').manual_seed(1234)
+    Q, K, V = (torch.randn((B, Hd, S, D), generator=gen).half().cuda() for _ in range(3))
+    O = torch.empty_like(Q)
+    scale = D ** -0.5
+    ms, wall = _events_ms(torch, lambda: core.flash_attention(Q, K, V, scale, out=O), steps, warmup)
+    res = {
+        'metric': 'TFLOP/s + % MFMA peak (attention)', 'value': flop / ms / 1e9, 'unit': 'TFLOP/s',
+        'ms_per_step': ms, 'dtype': 'f16',
+        'config': {'workload': 'flash attention, non-causal, BASELINE.json configs[2]', 'batch': B, 'heads': Hd,
+                   'seq': S, 'head_dim': D, 'accumulate': 'f32'},
+        'pct_f16_mfma_peak': 100.0 * flop / ms / 1e9 / PEAK_F16_TFLOPS,
+        'roofline': {'bound': 'mfma', 'achieved': flop / ms / 1e9, 'peak': PEAK_F16_TFLOPS, 'unit': 'TFLOP/s',
+                     'frac': flop / ms / 1e9 / PEAK_F16_TFLOPS,
+                     'traffic': MEASURED_TRAFFIC_BYTES.get('flash_attn_kernel'), 'kernel': 'flash_attn_kernel'},
+    }
+    if cpu:
+        from oracle import c_oracle
+        heads = 1
+        q, k, v = (x[0, :heads].cpu().numpy() for x in (Q, K, V))
+        t0 = time.perf_counter()
+        c_oracle.flash_attention(q, k, v, scale, block_kv=64)
+        dt = time.perf_counter() - t0
+        res['cpu_baseline'] = {'value': flop * heads / (B * Hd) / dt / 1e12, 'unit': 'TFLOP/s', 'cores': 1,
+                               'kind': 'port', 'sample': f'{heads} of {B * Hd} (batch, head) pairs through '
+                                                         f'oracle/oracle.c, {dt:.1f} s'}
+    return res
+
+
+def _unfused_lstm_baseline(torch, core, xs, WU, hs, cs, dil=None):
+    """Per-step GEMM (rocBLAS/hipBLASLt through torch) + one elementwise kernel, layer-major:
+    the structure of benchmarks/rnn/fractaltensor/stacked_lstm (utils.h:559-625).  Returns a
+    callable that replays the whole forward pass as one HIP graph, and the eager callable."""
+    L, T, B, H = hs.shape
+    W = WU[:, :H].contiguous()
+    U = WU[:, H:].contiguous()
+    xw = torch.empty((T * B, 4 * H), device='cuda')
+    gates = torch.empty((B, 4 * H), device='cuda')
+
+    def forward():
+        inp = xs
+        for l in range(L):
+            d = 1 if dil is None else dil[l]
+            torch.mm(inp.reshape(T * B, H), W[l], out=xw)        # x@W for all steps in one GEMM
+            for t in range(T):
+                g = xw[t * B:(t + 1) * B]
+                if t >= d:
+                    torch.addmm(g, hs[l, t - d], U[l], out=gates)  # per-step h@U
+                    core.lstm_elementwise(gates, None, cs[l, t - d], out=(hs[l, t], cs[l, t]))
+                else:
+                    core.lstm_elementwise(g, None, None, out=(hs[l, t], cs[l, t]))
+            inp = hs[l]
+
+    forward()
+    torch.cuda.synchronize()
+    graph = None
+    try:
+        s = torch.cuda.Stream()
+        s.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(s):
+            forward()
+        torch.cuda.current_stream().wait_stream(s)
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            forward()
+    except Exception as e:  # graph capture is an optimisation of the baseline, not a requirement
+        print(f'# baseline graph capture unavailable: {e}', file=sys.stderr)
+        graph = None
+    return forward, graph
+
+
+def bench_lstm(torch, core, steps, warmup, cpu, dilated):
+    if dilated:
+        L, T, B, H = 6, 128, 256, 256
+        dil = [1, 2, 4, 8, 16, 32]
+        name = 'dilated LSTM, BASELINE.json configs[4]'
+    else:
+        L, T, B, H = 32, 64, 256, 256
+        dil = None
+        name = 'stacked LSTM, BASELINE.json configs[3]'
+    flop = 2.0 * L * T * B * (2 * H) * (4 * H)
+    gen = torch.Generator(device='cpu').manual_seed(1234)
+    xs = torch.randn((T, B, H), generator=gen).cuda()
+    WU = ((torch.rand((L, 2 * H, 4 * H), generator=gen) - 0.5) / 8).cuda()   # U(-1/16, 1/16)
+    hs = torch.empty((L, T, B, H), device='cuda')
+    cs = torch.empty_like(hs)
+    ws = torch.empty(core.stacked_lstm_workspace_bytes(L, T, B, H), dtype=torch.uint8, device='cuda')
+    fused = lambda: core.stacked_lstm(xs, WU, dilations=dil, out=(hs, cs), workspace=ws)
+    ms, wall = _events_ms(torch, fused, steps, warmup)
+    status = core.persistent_status(ws)
+    ref_h = hs.clone()
+
+    # per-stage launches of the fused cell (no persistent kernel)
+    ms_wave, _ = _events_ms(torch, lambda: core.stacked_lstm(xs, WU, dilations=dil, out=(hs, cs), schedule='wavefront'),
+                            max(2, steps // 4), 1)
+    # unfused GPU baseline
+    hs_b = torch.empty_like(hs)
+    cs_b = torch.empty_like(cs)
+    eager, graph = _unfused_lstm_baseline(torch, core, xs, WU, hs_b, cs_b, dil)
+    nb = max(2, steps // 4)
+    ms_eager, _ = _events_ms(torch, eager, nb, 1)
+    ms_graph = None
+    if graph is not None:
+        hs_b.zero_()
+        ms_graph, _ = _events_ms(torch, graph.replay, nb, 2)
+    base_err = float((hs_b - ref_h).abs().max() / ref_h.abs().max())
+    ms_base = ms_graph if ms_graph is not None else ms_eager
+
+    res = {
+        'metric': 'stacked-LSTM sequences/s', 'value': B / ms * 1e3, 'unit': 'sequences/s', 'ms_per_step': ms,
+        'dtype': 'f32',
+        'config': {'workload': name, 'layers': L, 'batch': B, 'seq_len': T, 'hidden': H,
+                   'dilations': dil, 'outputs': 'h and c of every layer at every step'},
+        'tflops': flop / ms / 1e9,
+        'persistent_status': status,
+        'per_stage_launches': {'ms_per_step': ms_wave, 'sequences_per_s': B / ms_wave * 1e3},
+        'unfused_gpu_baseline': {'ms_per_step_hip_graph': ms_graph, 'ms_per_step_eager': ms_eager,
+                                 'sequences_per_s': B / ms_base * 1e3, 'speedup_of_fused': ms_base / ms,
+                                 'max_rel_diff_vs_fused': base_err,
+                                 'what': 'one x@W GEMM per layer + per-step h@U GEMM (torch/rocBLAS) + one '
+                                         'elementwise kernel per step, layer-major'},
+        'roofline': {'bound': 'mfma', 'achieved': flop / ms / 1e9, 'peak': PEAK_F32_MATRIX_TFLOPS, 'unit': 'TFLOP/s',
+                     'frac': flop / ms / 1e9 / PEAK_F32_MATRIX_TFLOPS,
+                     'traffic': MEASURED_TRAFFIC_BYTES.get('lstm_persistent_kernel'), 'kernel': 'lstm_persistent_kernel'},
+    }
+    if cpu:
+        from oracle import c_oracle
+        Ls, Ts, Bs = (2, 4, 64) if not dilated else (2, 8, 32)
+        x = xs[:Ts, :Bs].cpu().numpy()
+        w = WU[:Ls].cpu().numpy()
+        t0 = time.perf_counter()
+        c_oracle.stacked_lstm(x, w, None, None if dil is None else dil[:Ls])
+        dt = time.perf_counter() - t0
+        cells = Ls * Ts
+        # sequences/s of the full configuration extrapolated from the per-(cell,row) cost of the sample
+        full_seconds = dt * (L * T * B) / (cells * Bs)
+        res['cpu_baseline'] = {'value': B / full_seconds, 'unit': 'sequences/s', 'cores': 1, 'kind': 'port',
+                               'sample': f'{Ls} layers x {Ts} steps x {Bs} rows through oracle/oracle.c in {dt:.1f} s, '
+                                         f'scaled by cell-rows to the full configuration'}
+    return res
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument('--gpus', type=int, default=1)
+    ap.add_argument('--steps', type=int, default=50)
+    ap.add_argument('--warmup', type=int, default=10)
+    ap.add_argument('--workload', default='b2b', choices=['b2b', 'attention', 'stacked_lstm', 'dilated_lstm'])
+    ap.add_argument('--no-extras', action='store_true', help='measure only the chosen workload')
+    ap.add_argument('--no-cpu', action='store_true', help='skip the CPU baseline leg')
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print('bench.py measures one GPU: every workload here is a single-device kernel '
+              '(independent problems / heads / batch rows; no collectives). Run with --gpus 1.', file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+    import fractaltensor_amd._core as core   # raises if libftkernels.so is missing: no fallback
+    if not torch.cuda.is_available():
+        print('bench.py needs a GPU', file=sys.stderr)
+        sys.exit(2)
+    torch.cuda.set_device(0)
+    cpu = not args.no_cpu
+
+    runners = {
+        'b2b': lambda s, w, c: bench_b2b(torch, core, s, w, c),
+        'attention': lambda s, w, c: bench_attention(torch, core, s, w, c),
+        'stacked_lstm': lambda s, w, c: bench_lstm(torch, core, max(3, s // 5), max(1, w // 5), c, False),
+        'dilated_lstm': lambda s, w, c: bench_lstm(torch, core, max(3, s // 5), max(1, w // 5), c, True),
+    }
+    res = runners[args.workload](args.steps, args.warmup, cpu)
+    line = {
+        'metric': res.pop('metric'), 'value': res.pop('value'), 'unit': res.pop('unit'),
+        'n_gpus': 1, 'steps': args.steps, 'warmup': args.warmup, 'ms_per_step': res.pop('ms_per_step'),
+        'higher_is_better': True, 'scaling': 'weak', 'vs_baseline': None,
+        'dtype': res.pop('dtype'), 'data': 'synthetic', 'config': res.pop('config'),
+        'roofline': res.pop('roofline'), 'cpu_baseline': res.pop('cpu_baseline', None),
+    }
+    line.update(res)
+    info = core.device_info()
+    line['device'] = {'arch': info.arch.decode(), 'compute_units': info.compute_units,
+                      'host_cpus': os.cpu_count(), 'torch': torch.__version__}
+    if not args.no_extras:
+        others = {}
+        for name in runners:
+            if name == args.workload:
+                continue
+            try:
+                others[name] = runners[name](max(5, args.steps // 2), max(2, args.warmup // 2), cpu)
+            except Exception as e:   # an extra must not take the headline down with it
+                others[name] = {'error': repr(e)}
+        line['other_workloads'] = others
+    print(json.dumps(line))
+
+
+if __name__ == '__main__':
+    main()

@@ -116,7 +116,8 @@ def lstm_cell(x, h_prev, c_prev, WU, bias=None) -> Tuple[torch.Tensor, torch.Ten
     return h, c
 
 
-def lstm_elementwise(gates, bias, c_prev) -> Tuple[torch.Tensor, torch.Tensor]:
+def lstm_elementwise(gates, bias, c_prev, out: Optional[Tuple[torch.Tensor, torch.Tensor]] = None
+                     ) -> Tuple[torch.Tensor, torch.Tensor]:
     """State update on pre-activation gates [B,4H] (the unfused baseline's second kernel)."""
     f32 = torch.float32
     _req(gates, f32, 'gates')
@@ -126,8 +127,12 @@ def lstm_elementwise(gates, bias, c_prev) -> Tuple[torch.Tensor, torch.Tensor]:
         _req(bias, f32, 'bias')
     if c_prev is not None:
         _req(c_prev, f32, 'c_prev')
-    h = torch.empty((B, H), dtype=f32, device=gates.device)
-    c = torch.empty((B, H), dtype=f32, device=gates.device)
+    if out is None:
+        h = torch.empty((B, H), dtype=f32, device=gates.device)
+        c = torch.empty((B, H), dtype=f32, device=gates.device)
+    else:
+        h, c = out
+        _req(h, f32, 'h'); _req(c, f32, 'c')
     _check(lib.ftk_lstm_elementwise_f32(_ptr(gates), _ptr(bias), _ptr(c_prev), _ptr(h), _ptr(c),
                                         ctypes.c_int(B), ctypes.c_int(H), _stream()))
     return h, c

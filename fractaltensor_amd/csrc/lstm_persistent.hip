@@ -22,15 +22,15 @@
 // Hand-off between compute units (which may sit on different XCDs, whose L2
 // caches are not coherent with each other) uses no cache-wide fences: h is
 // written with agent-scope write-through stores and read with agent-scope
-// loads, the producer waits for its stores to be acknowledged, then one thread
-// per workgroup increments flags[l][t][rb]; consumers poll that count with
-// agent-scope loads until it reaches 8.  c is only ever re-read by the
+// loads, every producer wave waits for its own stores to be acknowledged and
+// then increments flags[l][t][rb]; consumers poll that count with agent-scope
+// loads until it reaches 32 (8 column slices x 4 waves).  c is only ever re-read by the
 // workgroup that wrote it and goes through the cache normally.
 //
-// The activation tile is double buffered: while item n is on the matrix cores
-// the next item's tile is already in flight into registers (if its producers
-// are done; otherwise the wave waits for them after its own MFMAs).  One
-// workgroup barrier per item.
+// The activation tile is double buffered and the item loop is software
+// pipelined: the loads of tile n+1 are issued half way through item n, and the
+// activations / state update / stores of item n-1 run in the shadow of item
+// n's first MFMAs.  One workgroup barrier per item.
 //
 // All workgroups must be co-resident: the host launches cooperatively with at
 // most one workgroup per compute unit (each uses the whole register file of
@@ -39,6 +39,7 @@
 #include <stdlib.h>
 
 #include <algorithm>
+#include <type_traits>
 
 #include "ftk_common.h"
 
@@ -67,10 +68,9 @@ struct PersistArgs {
   int pr;          // row slices per layer
   int groups;      // workgroups that take part (= L * PC * pr)
   int xcd_remap;   // 1: grid is a multiple of 8, map workgroups so a layer shares an XCD
-  int serial;      // 1: some workgroup's next item depends on its current one (no prefetch)
   int spin_limit;
   int trace_q;            // logical workgroup whose item timeline is recorded, or -1
-  long long* trace;       // [items][5] 100 MHz clock stamps of that workgroup
+  long long* trace;       // [items][8] 100 MHz clock stamps of that workgroup
   int dil[kMaxLayers];
 };
 
@@ -105,8 +105,16 @@ __device__ __forceinline__ void coherent_store8(float* p, float a, float b) {
   __hip_atomic_store(reinterpret_cast<u64*>(p), v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
+// 16 bytes per lane from global memory straight into LDS at lds_base + 16*lane
+// (lds_base must be wave-uniform), agent scope.
+__device__ __forceinline__ void lds_dma16(const float* gsrc, float* lds_base) {
+  __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)gsrc,
+                                   (__attribute__((address_space(3))) void*)lds_base, 16, 0, /*sc1*/ 16);
+}
+
 constexpr int P_TILE = 32 * P_LD;  // floats per LDS buffer
-constexpr int P_PF = 32;           // 8-byte prefetch registers per thread (8 rows x 512 floats per wave)
+constexpr int FLAG_TARGET = PC * 4;  // one count per wave of each of the 8 column slices
+constexpr int TS = 8;              // trace stamps per item
 
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1)))
 void lstm_persistent_kernel(PersistArgs a) {
@@ -155,175 +163,266 @@ void lstm_persistent_kernel(PersistArgs a) {
     }
   }
 
-  // Staging: wave w moves rows 8w..8w+7 of the tile; a row is 256 floats of x
-  // and 256 of h_prev, 128 eight-byte pieces each; lane handles pieces
-  // lane and lane+64 of either half.
-  u64 pf[P_PF];
   bool alive = true;
 
   auto item_t = [&](int n) { return n / my_rbs; };
   auto item_rb = [&](int n) { return prs + a.pr * (n % my_rbs); };
+  auto flag_of = [&](int ll, int t, int rb) { return a.flags + ((size_t)ll * T + t) * a.nrb + rb; };
 
-  // inputs of item n complete?  (blocking: bounded spin; otherwise one poll)
-  auto deps_ready = [&](int n, bool blocking) __attribute__((always_inline)) -> bool {
+  // inputs of item n complete?  Bounded spin on the two counters.
+  auto wait_deps = [&](int n) __attribute__((always_inline)) -> bool {
     const int t = item_t(n), rb = item_rb(n);
     bool ok = true;
-    if (l > 0) {
-      const int* f = a.flags + ((size_t)(l - 1) * T + t) * a.nrb + rb;
-      ok = blocking ? wait_count(f, PC, a.status, a.spin_limit) : (flag_load(f) >= PC);
-    }
-    if (ok && t >= d) {
-      const int* f = a.flags + ((size_t)l * T + (t - d)) * a.nrb + rb;
-      ok = blocking ? wait_count(f, PC, a.status, a.spin_limit) : (flag_load(f) >= PC);
-    }
-    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");  // data loads stay behind the flag reads
+    if (l > 0) ok = wait_count(flag_of(l - 1, t, rb), FLAG_TARGET, a.status, a.spin_limit);
+    if (ok && t >= d) ok = wait_count(flag_of(l, t - d, rb), FLAG_TARGET, a.status, a.spin_limit);
+    // The data loads must stay behind the flag reads.  The hardware issues and
+    // returns loads in order, so a compiler barrier is all it takes; a fence
+    // instruction here would also wait for this wave's outstanding stores.
+    asm volatile("" ::: "memory");
     return ok;
   };
-  auto issue_loads = [&](int n) __attribute__((always_inline)) {
+  // request / test the two counters of item n without waiting
+  struct Flags { int below, own; };
+  auto request_flags = [&](int n) __attribute__((always_inline)) -> Flags {
+    Flags f{FLAG_TARGET, FLAG_TARGET};
+    const int t = item_t(n), rb = item_rb(n);
+    if (l > 0) f.below = flag_load(flag_of(l - 1, t, rb));
+    if (t >= d) f.own = flag_load(flag_of(l, t - d, rb));
+    return f;
+  };
+  auto flags_ready = [](const Flags& f) { return f.below >= FLAG_TARGET && f.own >= FLAG_TARGET; };
+
+  // Tile n into LDS buffer buf, global -> LDS directly: wave w moves rows
+  // 8w..8w+7; one instruction carries half a row (256 floats = 64 lanes x 16
+  // bytes, consecutive lanes to consecutive LDS addresses), agent-scope so it
+  // sees what other compute units published.
+  auto issue_tile = [&](int n, int buf) __attribute__((always_inline)) {
     const int t = item_t(n), rb = item_rb(n);
     const float* xsrc = (l == 0) ? a.xs + (size_t)t * cell : a.hsss + ((size_t)(l - 1) * T + t) * cell;
     const bool has_prev = t >= d;
     const float* hsrc = a.hsss + ((size_t)l * T + (has_prev ? t - d : 0)) * cell;
+    float* dst = tile + buf * P_TILE + (8 * wave) * P_LD;
 #pragma unroll
     for (int r = 0; r < 8; ++r) {
       const int rg = min(rb * 32 + 8 * wave + r, B - 1);
-      pf[4 * r + 0] = coherent_load8(xsrc + (size_t)rg * PH + 2 * lane);
-      pf[4 * r + 1] = coherent_load8(xsrc + (size_t)rg * PH + 128 + 2 * lane);
-      if (has_prev) {
-        pf[4 * r + 2] = coherent_load8(hsrc + (size_t)rg * PH + 2 * lane);
-        pf[4 * r + 3] = coherent_load8(hsrc + (size_t)rg * PH + 128 + 2 * lane);
-      }
+      lds_dma16(xsrc + (size_t)rg * PH + 4 * lane, dst + r * P_LD);
+      if (has_prev) lds_dma16(hsrc + (size_t)rg * PH + 4 * lane, dst + r * P_LD + PH);
     }
   };
-  auto write_tile = [&](int n, int buf) __attribute__((always_inline)) {
-    const bool has_prev = item_t(n) >= d;
-    float* dst = tile + buf * P_TILE + (8 * wave) * P_LD + 2 * lane;
-#pragma unroll
-    for (int r = 0; r < 8; ++r) {
-      *reinterpret_cast<u64*>(dst + r * P_LD) = pf[4 * r + 0];
-      *reinterpret_cast<u64*>(dst + r * P_LD + 128) = pf[4 * r + 1];
-      if (has_prev) {
-        *reinterpret_cast<u64*>(dst + r * P_LD + 256) = pf[4 * r + 2];
-        *reinterpret_cast<u64*>(dst + r * P_LD + 384) = pf[4 * r + 3];
-      }
-    }
-  };
-
-  // prologue: first tile
-  alive = deps_ready(0, true);
-  if (alive) issue_loads(0);
-  if (alive) write_tile(0, 0);
-  __syncthreads();
-
-  const bool tracing = (q == a.trace_q) && tid == 0;
-  for (int n = 0; n < n_items; ++n) {
-    const int buf = n & 1;
-    if (tracing) a.trace[5 * n + 0] = wall_clock64();
-    const int t = item_t(n), rb = item_rb(n);
-    const bool has_prev = t >= d;
-    const bool more = n + 1 < n_items;
-    float* hdst = a.hsss + ((size_t)l * T + t) * cell;
-    float* cdst = a.csss + ((size_t)l * T + t) * cell;
-    const int rg = rb * 32 + j;
-    const int rgc = min(rg, B - 1);
-
-    float4 cp = make_float4(0.f, 0.f, 0.f, 0.f);
-    if (alive && has_prev)
-      cp = *reinterpret_cast<const float4*>(a.csss + ((size_t)l * T + (t - d)) * cell + (size_t)rgc * PH + u0);
-
-    // the next item's flags are requested now and looked at half way through
-    // the item, so their round trip to memory is off the critical path
-    int f_below = PC, f_own = PC;
-    if (more && !a.serial) {
-      const int t1 = item_t(n + 1), rb1 = item_rb(n + 1);
-      if (l > 0) f_below = flag_load(a.flags + ((size_t)(l - 1) * T + t1) * a.nrb + rb1);
-      if (t1 >= d) f_own = flag_load(a.flags + ((size_t)l * T + (t1 - d)) * a.nrb + rb1);
-    }
-
-    // ---- gates^T = WU^T * act^T on the matrix cores; two accumulators so
-    // that consecutive MFMAs never wait on each other's result
-    v16f acc0, acc1;
-#pragma unroll
-    for (int r = 0; r < 16; ++r) { acc0[r] = 0.0f; acc1[r] = 0.0f; }
+  // steps [q0, q1) of the K loop (steps 0..31: x rows of WU, 32..63: h rows)
+  // into two accumulators so that consecutive MFMAs never wait on each other's
+  // result; the LDS read for step q+1 is issued before the MFMAs of step q
+  auto mfma_part = [&](int buf, auto q0c, auto q1c, v16f& acc0, v16f& acc1) __attribute__((always_inline)) {
+    constexpr int q0 = decltype(q0c)::value;
+    constexpr int q1 = decltype(q1c)::value;
     const float* arow = tile + buf * P_TILE + j * P_LD + 4 * hh;
+    v4f b = *reinterpret_cast<const v4f*>(arow + 8 * q0);
 #pragma unroll
-    for (int qq = 0; qq < PH / 8; ++qq) {
-      const v4f b = *reinterpret_cast<const v4f*>(arow + 8 * qq);
+    for (int qq = q0; qq < q1; ++qq) {
+      v4f bn = b;
+      if (qq + 1 < q1) bn = *reinterpret_cast<const v4f*>(arow + 8 * (qq + 1));
       acc0 = __builtin_amdgcn_mfma_f32_32x32x2f32(wr[4 * qq + 0], b[0], acc0, 0, 0, 0);
       acc1 = __builtin_amdgcn_mfma_f32_32x32x2f32(wr[4 * qq + 1], b[1], acc1, 0, 0, 0);
       acc0 = __builtin_amdgcn_mfma_f32_32x32x2f32(wr[4 * qq + 2], b[2], acc0, 0, 0, 0);
       acc1 = __builtin_amdgcn_mfma_f32_32x32x2f32(wr[4 * qq + 3], b[3], acc1, 0, 0, 0);
+      b = bn;
     }
-    if (tracing) a.trace[5 * n + 1] = wall_clock64();
-
-    // Half way through the item, fetch the next tile: wait (bounded) for its
-    // producers, then put its loads in flight behind the rest of the MFMAs.
-    // Waiting here rather than at the end of the item makes each layer settle
-    // about one and a half items behind the layer below, which is what lets
-    // the loads overlap the arithmetic in steady state.
-    if (alive && more && !a.serial) {
-      if (f_below < PC || f_own < PC) alive = deps_ready(n + 1, true);
-      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
-      if (alive) issue_loads(n + 1);
-    }
-
-    if (has_prev) {
+    __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
 #pragma unroll
-      for (int qq = PH / 8; qq < PK / 8; ++qq) {
-        const v4f b = *reinterpret_cast<const v4f*>(arow + 8 * qq);
-        acc0 = __builtin_amdgcn_mfma_f32_32x32x2f32(wr[4 * qq + 0], b[0], acc0, 0, 0, 0);
-        acc1 = __builtin_amdgcn_mfma_f32_32x32x2f32(wr[4 * qq + 1], b[1], acc1, 0, 0, 0);
-        acc0 = __builtin_amdgcn_mfma_f32_32x32x2f32(wr[4 * qq + 2], b[2], acc0, 0, 0, 0);
-        acc1 = __builtin_amdgcn_mfma_f32_32x32x2f32(wr[4 * qq + 3], b[3], acc1, 0, 0, 0);
-      }
+    for (int g4 = q0; g4 < q1; ++g4) {
+      __builtin_amdgcn_sched_group_barrier(0x008, 4, 0);
+      __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
     }
-    v16f acc;
+  };
+  // bias, activations and state update of an item: lane-local and branch-free,
+  // so the scheduler can slot it between MFMAs of the next item
+  auto epilogue_math = [&](const v16f& acc, const float4& cp, float (&hv)[4], float (&cv)[4]) __attribute__((always_inline)) {
+    const float cpv[4] = {cp.x, cp.y, cp.z, cp.w};
 #pragma unroll
-    for (int r = 0; r < 16; ++r) acc[r] = acc0[r] + acc1[r];
-
-    // ---- state update, lane-local; h leaves through write-through stores
+    for (int r = 0; r < 4; ++r) {
+      const float ig = sigmoid_f(acc[r] + bi[r]);
+      const float fg = sigmoid_f(acc[4 + r] + bf[r]);
+      const float og = sigmoid_f(acc[8 + r] + bo[r]);
+      const float cand = tanh_f(acc[12 + r] + bg[r]);
+      cv[r] = fg * cpv[r] + ig * cand;
+      hv[r] = og * tanh_f(cv[r]);
+    }
+  };
+  // h leaves through write-through stores, c through the cache
+  auto epilogue_store = [&](int n, const float (&hv)[4], const float (&cv)[4]) __attribute__((always_inline)) {
+    const int t = item_t(n), rb = item_rb(n);
+    const int rg = rb * 32 + j;
     if (alive && rg < B) {
-      const float cpv[4] = {cp.x, cp.y, cp.z, cp.w};
-      float hv[4], cv[4];
-#pragma unroll
-      for (int r = 0; r < 4; ++r) {
-        const float ig = sigmoid_f(acc[r] + bi[r]);
-        const float fg = sigmoid_f(acc[4 + r] + bf[r]);
-        const float og = sigmoid_f(acc[8 + r] + bo[r]);
-        const float cand = tanh_f(acc[12 + r] + bg[r]);
-        cv[r] = fg * cpv[r] + ig * cand;
-        hv[r] = og * tanh_f(cv[r]);
-      }
-      *reinterpret_cast<float4*>(cdst + (size_t)rg * PH + u0) = make_float4(cv[0], cv[1], cv[2], cv[3]);
-      coherent_store8(hdst + (size_t)rg * PH + u0, hv[0], hv[1]);
-      coherent_store8(hdst + (size_t)rg * PH + u0 + 2, hv[2], hv[3]);
+      float* hdst = a.hsss + ((size_t)l * T + t) * cell + (size_t)rg * PH + u0;
+      float* cdst = a.csss + ((size_t)l * T + t) * cell + (size_t)rg * PH + u0;
+      *reinterpret_cast<float4*>(cdst) = make_float4(cv[0], cv[1], cv[2], cv[3]);
+      coherent_store8(hdst, hv[0], hv[1]);
+      coherent_store8(hdst + 2, hv[2], hv[3]);
     }
+  };
+  auto epilogue = [&](int n, const v16f& acc, const float4& cp) __attribute__((always_inline)) {
+    float hv[4], cv[4];
+    epilogue_math(acc, cp, hv, cv);
+    epilogue_store(n, hv, cv);
+  };
+  auto load_cprev = [&](int n) __attribute__((always_inline)) -> float4 {
+    const int t = item_t(n), rb = item_rb(n);
+    float4 cp = make_float4(0.f, 0.f, 0.f, 0.f);
+    if (alive && t >= d) {
+      const int rgc = min(rb * 32 + j, B - 1);
+      cp = *reinterpret_cast<const float4*>(a.csss + ((size_t)l * T + (t - d)) * cell + (size_t)rgc * PH + u0);
+    }
+    return cp;
+  };
+  // every wave publishes its own part of an item: its stores acknowledged, then one count
+  auto publish = [&](int n) __attribute__((always_inline)) {
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+    __builtin_amdgcn_s_waitcnt(0);
+    if (lane == 0 && alive)
+      __hip_atomic_fetch_add(flag_of(l, item_t(n), item_rb(n)), 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  };
 
-    if (tracing) a.trace[5 * n + 2] = wall_clock64();
-    if (!a.serial) {
-      if (alive && more) write_tile(n + 1, buf ^ 1);
-      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
-      __builtin_amdgcn_s_waitcnt(0);  // this wave's h stores are acknowledged
-      if (tracing) a.trace[5 * n + 3] = wall_clock64();
-      __syncthreads();
-      if (tracing) a.trace[5 * n + 4] = wall_clock64();
-      if (tid == 0 && alive)
-        __hip_atomic_fetch_add(a.flags + ((size_t)l * T + t) * a.nrb + rb, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    } else {
-      // the next item needs this one: publish first, then fetch
-      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+  const bool tracing = (q == a.trace_q) && tid == 0;
+  v16f acc0, acc1;
+
+  // How far apart an item and the item that needs it are in this workgroup's
+  // own sequence decides the schedule: distance 1 (one row block, dilation 1)
+  // leaves nothing to overlap; distance 2 means item n-1 must be published
+  // before the wait for item n+1 can end.
+  const long long own_distance = (long long)d * my_rbs;
+  const bool serial = own_distance < 2;
+  const bool publish_mid = own_distance < 3;
+
+  if (serial) {
+    for (int n = 0; n < n_items; ++n) {
+      if (tracing) a.trace[TS * n + 0] = wall_clock64();
+      if (alive) alive = wait_deps(n);
+      if (alive) issue_tile(n, 0);
+      const float4 cp = load_cprev(n);
       __builtin_amdgcn_s_waitcnt(0);
       __syncthreads();
-      if (tid == 0 && alive)
-        __hip_atomic_fetch_add(a.flags + ((size_t)l * T + t) * a.nrb + rb, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      if (alive && more) {
-        alive = deps_ready(n + 1, true);
-        if (alive) issue_loads(n + 1);
-        if (alive) write_tile(n + 1, buf ^ 1);
-      }
-      __syncthreads();
+#pragma unroll
+      for (int r = 0; r < 16; ++r) { acc0[r] = 0.0f; acc1[r] = 0.0f; }
+      mfma_part(0, std::integral_constant<int, 0>{}, std::integral_constant<int, PH / 8>{}, acc0, acc1);
+      if (item_t(n) >= d) mfma_part(0, std::integral_constant<int, PH / 8>{}, std::integral_constant<int, PK / 8>{}, acc0, acc1);
+      v16f acc;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[r] = acc0[r] + acc1[r];
+      epilogue(n, acc, cp);
+      publish(n);
+      __syncthreads();  // the tile is rewritten by the next item
+      if (tracing) a.trace[TS * n + 7] = wall_clock64();
     }
+    return;
   }
+
+  // ---- pipelined schedule.  Per item n:
+  //   x half of the MFMAs;
+  //   activations, state update and stores of item n-1;
+  //   h half of the MFMAs;
+  //   publish item n-1 (its stores went out half an item ago, so waiting for
+  //     their acknowledgement is free; with own_distance 2 the publish moves
+  //     up to the middle of the item);
+  //   one workgroup barrier.
+  // Tile n+1 goes into the other LDS buffer as soon as its producers are seen
+  // to be done.  The counters are requested a stretch of MFMAs before each of
+  // several look-at points, so looking costs nothing; only if every look fails
+  // does the wave wait at the end of the item, and then it also backs off once
+  // so that from then on it trails its producers by enough for an early look
+  // to succeed.
+  alive = wait_deps(0);
+  if (alive) issue_tile(0, 0);
+  Flags fl = (n_items > 1) ? request_flags(1) : Flags{FLAG_TARGET, FLAG_TARGET};
+  __builtin_amdgcn_s_waitcnt(0);
+  __syncthreads();
+
+  v16f acc_prev;
+  float4 cp_prev = make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll
+  for (int r = 0; r < 16; ++r) acc_prev[r] = 0.0f;
+
+  for (int n = 0; n < n_items; ++n) {
+    const int buf = n & 1;
+    if (tracing) a.trace[TS * n + 0] = wall_clock64();
+    const bool has_prev = item_t(n) >= d;
+    const bool more = n + 1 < n_items;
+    bool pending = alive && more;  // tile n+1 still to be requested
+    int looks = 0;                 // looks taken before the request went out (for the trace)
+
+    auto look = [&]() __attribute__((always_inline)) {
+      if (pending) {
+        ++looks;
+        if (flags_ready(fl)) {
+          asm volatile("" ::: "memory");
+          issue_tile(n + 1, buf ^ 1);
+          pending = false;
+        } else {
+          fl = request_flags(n + 1);
+        }
+      }
+    };
+
+    look();  // counters requested in the middle of item n-1
+    const bool first_look_failed = pending;
+    const float4 cp = load_cprev(n);
+#pragma unroll
+    for (int r = 0; r < 16; ++r) { acc0[r] = 0.0f; acc1[r] = 0.0f; }
+    mfma_part(buf, std::integral_constant<int, 0>{}, std::integral_constant<int, PH / 8>{}, acc0, acc1);
+    // the counters are consumed before the stores go out, so that waiting for
+    // those (old) loads never waits for the stores
+    const bool ready2 = pending && flags_ready(fl);
+    if (tracing) a.trace[TS * n + 1] = wall_clock64();
+    if (n > 0) epilogue(n - 1, acc_prev, cp_prev);
+    if (tracing) a.trace[TS * n + 2] = wall_clock64();
+    if (publish_mid && n > 0) publish(n - 1);
+    if (pending) {
+      ++looks;
+      if (ready2) {
+        asm volatile("" ::: "memory");
+        issue_tile(n + 1, buf ^ 1);
+        pending = false;
+      }
+    }
+    // counters of item n+2 for the first look of the next item (in
+    // publish-in-the-middle mode: of item n+1, for the wait at the end)
+    if (publish_mid) {
+      if (pending) fl = request_flags(n + 1);
+    } else if (!pending && n + 2 < n_items) {
+      fl = request_flags(n + 2);
+    }
+    if (tracing) a.trace[TS * n + 3] = wall_clock64();
+
+    if (has_prev) mfma_part(buf, std::integral_constant<int, PH / 8>{}, std::integral_constant<int, PK / 8>{}, acc0, acc1);
+#pragma unroll
+    for (int r = 0; r < 16; ++r) acc_prev[r] = acc0[r] + acc1[r];
+    cp_prev = cp;
+    if (tracing) a.trace[TS * n + 4] = wall_clock64() | ((long long)(pending ? 7 : looks) << 60);
+
+    if (!publish_mid && n > 0) publish(n - 1);
+    if (tracing) a.trace[TS * n + 5] = wall_clock64();
+    // last resort: wait for the producers here
+    if (pending) {
+      if (publish_mid && flags_ready(fl)) {
+        asm volatile("" ::: "memory");
+      } else {
+        alive = wait_deps(n + 1);
+      }
+      if (alive) issue_tile(n + 1, buf ^ 1);
+      if (n + 2 < n_items) fl = request_flags(n + 2);
+    } else if (publish_mid && n + 2 < n_items) {
+      fl = request_flags(n + 2);
+    }
+    // Back off a little whenever the first look failed: the wave then trails
+    // its producers by a bit more, until the first look always succeeds and
+    // the tile has the whole item to arrive.
+    if (first_look_failed && !publish_mid) __builtin_amdgcn_s_sleep(80);
+    __builtin_amdgcn_s_waitcnt(0);  // tile n+1 has landed in LDS
+    if (tracing) a.trace[TS * n + 6] = wall_clock64();
+    __syncthreads();
+    if (tracing) a.trace[TS * n + 7] = wall_clock64();
+  }
+  epilogue(n_items - 1, acc_prev, cp_prev);
+  publish(n_items - 1);
 }
 
 __global__ void fill_zero_kernel(int* p, size_t n) {
@@ -335,10 +434,10 @@ static size_t flag_count(int L, int T, int B) {
   return (size_t)L * T * nrb;
 }
 
-// Workspace layout: [64 ints: status][flags][trace: T*nrb*5 stamps of 8 bytes].
+// Workspace layout: [64 ints: status][flags][trace: T*nrb*8 stamps of 8 bytes].
 static size_t trace_offset_bytes(int L, int T, int B) { return ((flag_count(L, T, B) + 64) * sizeof(int) + 15) / 16 * 16; }
 static size_t workspace_need(int L, int T, int B) {
-  return trace_offset_bytes(L, T, B) + (size_t)T * ((B + 31) / 32) * 5 * sizeof(long long);
+  return trace_offset_bytes(L, T, B) + (size_t)T * ((B + 31) / 32) * 8 * sizeof(long long);
 }
 
 // Tuning hook: FTK_LSTM_TRACE=<logical workgroup> records that workgroup's per-item timeline.
@@ -389,12 +488,7 @@ static int run_persistent(const float* xs, const float* WU, const float* bias, c
   a.spin_limit = 1 << 22;
   a.trace_q = trace_workgroup();
   a.trace = reinterpret_cast<long long*>(reinterpret_cast<char*>(ws) + trace_offset_bytes(L, T, B));
-  const int min_rbs = a.nrb / a.pr;
-  a.serial = 0;
-  for (int l = 0; l < kMaxLayers; ++l) {
-    a.dil[l] = (l < L && dil) ? dil[l] : 1;
-    if (l < L && (long long)a.dil[l] * min_rbs < 2) a.serial = 1;
-  }
+  for (int l = 0; l < kMaxLayers; ++l) a.dil[l] = (l < L && dil) ? dil[l] : 1;
   const int grid = a.groups;
   a.xcd_remap = (grid % 8 == 0) ? 1 : 0;
 
