@@ -96,7 +96,7 @@ def bench_b2b(torch, core, steps, warmup, cpu):
     }
     if cpu:
         from oracle import c_oracle
-        sample = 12   # problems of the 32
+        sample = 32   # all problems: about ten seconds of scalar C
         A, Bn, Cp, _ = sets[0]
         a, b, c = (x[:sample].cpu().numpy() for x in (A, Bn, Cp))
         t0 = time.perf_counter()
@@ -106,6 +106,18 @@ def bench_b2b(torch, core, steps, warmup, cpu):
                                'sample': f'{sample} of the {G} problems through oracle/oracle.c (scalar C, one thread), '
                                          f'{dt:.1f} s'}
     return res
+
+
+def bench_copy(torch, core, steps, warmup, cpu):
+    """Plain device copy of a known size: the calibration kernel for the FETCH_SIZE / WRITE_SIZE counters."""
+    n = 64 << 20   # 64 MiB read + 64 MiB written per launch
+    src = torch.empty(n, dtype=torch.uint8, device='cuda').random_()
+    dst = torch.empty_like(src)
+    ms, _ = _events_ms(torch, lambda: dst.copy_(src), steps, warmup)
+    return {'metric': 'copy GB/s (counter calibration)', 'value': 2.0 * n / ms / 1e6, 'unit': 'GB/s', 'ms_per_step': ms,
+            'dtype': 'u8', 'config': {'workload': 'torch copy_ of 64 MiB (reads 64 MiB, writes 64 MiB per launch)'},
+            'roofline': {'bound': 'hbm', 'achieved': 2.0 * n / ms / 1e6, 'peak': PEAK_HBM_GBS, 'unit': 'GB/s',
+                         'frac': 2.0 * n / ms / 1e6 / PEAK_HBM_GBS, 'traffic': None}}
 
 
 def bench_attention(torch, core, steps, warmup, cpu):
@@ -128,7 +140,7 @@ def bench_attention(torch, core, steps, warmup, cpu):
     }
     if cpu:
         from oracle import c_oracle
-        heads = 1
+        heads = 24
         q, k, v = (x[0, :heads].cpu().numpy() for x in (Q, K, V))
         t0 = time.perf_counter()
         c_oracle.flash_attention(q, k, v, scale, block_kv=64)
@@ -237,7 +249,7 @@ def bench_lstm(torch, core, steps, warmup, cpu, dilated):
     }
     if cpu:
         from oracle import c_oracle
-        Ls, Ts, Bs = (2, 4, 64) if not dilated else (2, 8, 32)
+        Ls, Ts, Bs = (8, 64, 256) if not dilated else (6, 32, 256)
         x = xs[:Ts, :Bs].cpu().numpy()
         w = WU[:Ls].cpu().numpy()
         t0 = time.perf_counter()
@@ -257,7 +269,7 @@ def main():
     ap.add_argument('--gpus', type=int, default=1)
     ap.add_argument('--steps', type=int, default=50)
     ap.add_argument('--warmup', type=int, default=10)
-    ap.add_argument('--workload', default='b2b', choices=['b2b', 'attention', 'stacked_lstm', 'dilated_lstm'])
+    ap.add_argument('--workload', default='b2b', choices=['b2b', 'attention', 'stacked_lstm', 'dilated_lstm', 'copy'])
     ap.add_argument('--no-extras', action='store_true', help='measure only the chosen workload')
     ap.add_argument('--no-cpu', action='store_true', help='skip the CPU baseline leg')
     args = ap.parse_args()
@@ -280,6 +292,9 @@ def main():
         'stacked_lstm': lambda s, w, c: bench_lstm(torch, core, max(3, s // 5), max(1, w // 5), c, False),
         'dilated_lstm': lambda s, w, c: bench_lstm(torch, core, max(3, s // 5), max(1, w // 5), c, True),
     }
+    if args.workload == 'copy':
+        runners = {'copy': lambda s, w, c: bench_copy(torch, core, s, w, c)}
+        args.no_extras = True
     res = runners[args.workload](args.steps, args.warmup, cpu)
     line = {
         'metric': res.pop('metric'), 'value': res.pop('value'), 'unit': res.pop('unit'),

@@ -48,7 +48,7 @@ __global__ __launch_bounds__(WAVES * 64) void flash_attn_kernel(const _Float16* 
                                                          const _Float16* __restrict__ K,
                                                          const _Float16* __restrict__ V,
                                                          _Float16* __restrict__ O, int Sq, int Skv,
-                                                         float scale_log2e) {
+                                                         float scale_log2e, int nqb) {
   constexpr int KLD = D + 8;   // padded K row (halfs)
   constexpr int DS = D / 16;   // k steps of S^T
   constexpr int DT = D / 32;   // d tiles of O^T
@@ -63,9 +63,16 @@ __global__ __launch_bounds__(WAVES * 64) void flash_attn_kernel(const _Float16* 
   const int wave = tid >> 6;
   const int j = lane & 31;
   const int hh = lane >> 5;
-  const int bh = blockIdx.y;
+  // One-dimensional grid of nqb query blocks x (batch*heads).  The hardware
+  // deals workgroups round-robin over the 8 XCDs; remap so that the query
+  // blocks of one head run on one XCD and share its L2 copy of K and V.
+  int id = blockIdx.x;
+  const int total = gridDim.x;
+  if ((total & 7) == 0) id = (blockIdx.x & 7) * (total >> 3) + (blockIdx.x >> 3);
+  const int bh = id / nqb;
+  const int qb = id - bh * nqb;
   constexpr int NT = WAVES * 64;  // threads
-  const int q_base = blockIdx.x * (WAVES * 32 * QT) + wave * (32 * QT);
+  const int q_base = qb * (WAVES * 32 * QT) + wave * (32 * QT);
 
   const _Float16* Qg = Q + (size_t)bh * Sq * D;
   const _Float16* Kg = K + (size_t)bh * Skv * D;
@@ -300,9 +307,12 @@ static int launch_fa(const void* Q, const void* K, const void* V, void* O, int B
     attr_set = true;
   }
   constexpr int ROWS = WAVES * 32 * QT;
-  dim3 grid((Sq + ROWS - 1) / ROWS, BH);
-  hipLaunchKernelGGL((flash_attn_kernel<D, QT, WAVES>), grid, dim3(WAVES * 64), lds, s, (const _Float16*)Q, (const _Float16*)K,
-                     (const _Float16*)V, (_Float16*)O, Sq, Skv, scale * 1.4426950408889634f);
+  const int nqb = (Sq + ROWS - 1) / ROWS;
+  const long long total = (long long)nqb * BH;
+  if (total > 0x7fffffffLL) return fail(FTK_ERR_UNSUPPORTED_SHAPE, "ftk_flash_attn_f16: grid too large");
+  hipLaunchKernelGGL((flash_attn_kernel<D, QT, WAVES>), dim3((unsigned)total), dim3(WAVES * 64), lds, s,
+                     (const _Float16*)Q, (const _Float16*)K, (const _Float16*)V, (_Float16*)O, Sq, Skv,
+                     scale * 1.4426950408889634f, nqb);
   return check_launch("flash_attn_kernel");
 }
 
@@ -327,14 +337,19 @@ extern "C" int ftk_flash_attn_f16(const void* Q, const void* K, const void* V, v
     return fail(FTK_ERR_INVALID_ARGUMENT, "ftk_flash_attn_f16: B, Hd, Sq, Skv, D must be positive");
   if (D != 64 && D != 128) return fail(FTK_ERR_UNSUPPORTED_SHAPE, "ftk_flash_attn_f16: D=%d must be 64 or 128", D);
   const long long bh = (long long)B * Hd;
-  if (bh > 65535) return fail(FTK_ERR_UNSUPPORTED_SHAPE, "ftk_flash_attn_f16: B*Hd=%lld above 65535", bh);
+  if (bh > (1LL << 24)) return fail(FTK_ERR_UNSUPPORTED_SHAPE, "ftk_flash_attn_f16: B*Hd=%lld too large", bh);
   const DeviceProps* dp = nullptr;
   int rc = device_props(&dp);
   if (rc) return rc;
   hipStream_t s = (hipStream_t)stream;
   // Variant: 0 = choose by problem size, 1 = 4 waves x 32 rows, 2 = 4 waves x 64 rows, 3 = 8 waves x 32 rows.
   int variant = fa_variant_override();
-  if (variant == 0) variant = ((long long)((Sq + 255) / 256) * bh >= dp->cus) ? 2 : 1;
+  // measured on MI355X at B8 H16 S2048 D128: 8 waves x 32 rows (two waves per SIMD, softmax of one
+  // overlapping the MFMAs of the other) beats 4 waves x 64 rows, which beats 4 waves x 32 rows
+  if (variant == 0) {
+    const bool big = (long long)((Sq + 255) / 256) * bh >= dp->cus;
+    variant = big ? (D == 128 ? 3 : 2) : 1;
+  }
   const int lds = dp->lds_optin;
   if (D == 128) {
     switch (variant) {

@@ -440,6 +440,20 @@ static size_t workspace_need(int L, int T, int B) {
   return trace_offset_bytes(L, T, B) + (size_t)T * ((B + 31) / 32) * 8 * sizeof(long long);
 }
 
+// Profiling hook: FTK_LSTM_PLAIN_LAUNCH=1 launches without the cooperative
+// co-residency check (counter collection tools that cannot follow cooperative
+// launches).  The grid never exceeds one workgroup per compute unit, so on an
+// otherwise idle device the workgroups are co-resident all the same; if they
+// are not, the bounded waits end the launch with the error word set.
+static bool plain_launch() {
+  static int v = -1;
+  if (v < 0) {
+    const char* e = getenv("FTK_LSTM_PLAIN_LAUNCH");
+    v = (e && atoi(e) != 0) ? 1 : 0;
+  }
+  return v == 1;
+}
+
 // Tuning hook: FTK_LSTM_TRACE=<logical workgroup> records that workgroup's per-item timeline.
 static int trace_workgroup() {
   static int v = -2;
@@ -497,7 +511,13 @@ static int run_persistent(const float* xs, const float* WU, const float* bias, c
   if (rc) return rc;
 
   void* kargs[] = {&a};
-  FTK_HIP(hipLaunchCooperativeKernel(fn, dim3(grid), dim3(256), kargs, (unsigned)lds, s));
+  if (plain_launch()) {
+    hipLaunchKernelGGL(lstm_persistent_kernel, dim3(grid), dim3(256), lds, s, a);
+    rc = check_launch("lstm_persistent_kernel");
+    if (rc) return rc;
+  } else {
+    FTK_HIP(hipLaunchCooperativeKernel(fn, dim3(grid), dim3(256), kargs, (unsigned)lds, s));
+  }
   *handled = true;
   return FTK_OK;
 }
