@@ -1,0 +1,164 @@
+"""GPU fast paths: the three hot-path programs of the reference as single
+kernel calls on FractalTensors that live on the GPU.
+
+  stacked_lstm   the fold-over-layers / scan-over-time / map-over-batch program of
+                 examples/stacked_rnn/stacked_rnn.py:23-79
+  dilated_lstm   the dilated_map program of examples/dilated_rnn/dilated_rnn.py:16-41
+  flash_attention  the map / reduce program of examples/flash_attention/flash_attention.py:14-91
+  b2b_gemm       (a @ b) @ c, the computation of benchmarks/fused_two_hgemms
+
+A regular (non-ragged) FractalTensor already is a dense row-major tensor in
+its flat buffer, so inputs are handed to the kernels as views and outputs are
+wrapped back without copies.  Everything here runs through the C ABI in
+fractaltensor_amd._core; there is no CPU or PyTorch fallback: CPU inputs are
+rejected, and a missing library is an ImportError.
+"""
+from __future__ import annotations
+
+from typing import Optional, Sequence
+
+import torch
+
+from ..fractal_tensor import FractalTensor
+from ..tensor import Tensor
+
+__all__ = ['pack_lstm_weights', 'stacked_lstm', 'dilated_lstm', 'lstm_cell', 'flash_attention', 'b2b_gemm',
+           'online_softmax']
+
+
+def _core():
+    from ... import _core
+    return _core
+
+
+def _dense_gpu(ft: FractalTensor, name: str, depth: int) -> torch.Tensor:
+    if not isinstance(ft, FractalTensor):
+        raise TypeError(f'{name} should be a FractalTensor.')
+    if ft.depth != depth:
+        raise ValueError(f'{name} should have depth {depth}, got {ft.depth}.')
+    if not ft.is_regular():
+        raise ValueError(f'{name} is ragged; the fused kernels take regular batches.')
+    t = ft.as_dense()
+    if not t.is_cuda:
+        raise RuntimeError(f'{name} lives on {t.device}; the fused kernels run on the GPU only.')
+    return t
+
+
+def pack_lstm_weights(Wss: FractalTensor, Uss: FractalTensor, bss: Optional[FractalTensor] = None):
+    """Per-gate parameters -> the fused layout of the kernels.
+
+    Wss, Uss: depth-2 [L][4] of [H, H] (gate order i, f, o, candidate, as in
+    examples/stacked_rnn/rnn_utils.py:28-36); bss: depth-2 [L][4] of [1, H].
+    Returns WU [L, 2H, 4H] with column blocks i|f|o|c~ (x rows, then h rows)
+    and bias [L, 4H] or None."""
+    W = _dense_gpu(Wss, 'Wss', 2)   # [L, 4, H, H]
+    U = _dense_gpu(Uss, 'Uss', 2)
+    L, G, H, H2 = W.shape
+    if G != 4 or H != H2 or U.shape != W.shape:
+        raise ValueError('Wss and Uss should be [L][4] of [H, H].')
+    WU = torch.cat([W.permute(0, 2, 1, 3).reshape(L, H, 4 * H), U.permute(0, 2, 1, 3).reshape(L, H, 4 * H)], dim=1)
+    bias = None
+    if bss is not None:
+        b = _dense_gpu(bss, 'bss', 2)   # [L, 4, 1, H]
+        bias = b.reshape(L, 4 * H).contiguous()
+    return WU.contiguous(), bias
+
+
+def _run_stack(xss, Wss, Uss, bss, dilations, return_all_layers):
+    core = _core()
+    xs = _dense_gpu(xss, 'xss', 2)   # [T, B, 1, H]
+    T, B = xs.shape[0], xs.shape[1]
+    H = xs.shape[-1]
+    xs = xs.reshape(T, B, H)
+    WU, bias = pack_lstm_weights(Wss, Uss, bss)
+    hsss, csss = core.stacked_lstm(xs.float(), WU.float(), None if bias is None else bias.float(), dilations=dilations)
+    L = WU.shape[0]
+    if return_all_layers:
+        return (FractalTensor.from_dense(hsss.view(L, T, B, 1, H), 3), FractalTensor.from_dense(csss.view(L, T, B, 1, H), 3))
+    return FractalTensor.from_dense(hsss[L - 1].reshape(T, B, 1, H), 2)
+
+
+def stacked_lstm(xss: FractalTensor, Wss: FractalTensor, Uss: FractalTensor, bss: Optional[FractalTensor] = None,
+                 return_all_layers: bool = False):
+    """Stacked LSTM over a time-major batch.
+
+    xss: depth-2 [T][B] of [1, H] (what stacked_rnn.py's `embs` is for equal-length
+    sequences).  Returns the last layer's hidden sequence as depth-2 [T][B] of
+    [1, H], which is what the reference's stacked_lstm returns; with
+    return_all_layers the (h, c) of every layer as depth-3 [L][T][B]."""
+    return _run_stack(xss, Wss, Uss, bss, None, return_all_layers)
+
+
+def dilated_lstm(xss: FractalTensor, Wss: FractalTensor, Uss: FractalTensor, bss: Optional[FractalTensor] = None,
+                 dilations: Optional[Sequence[int]] = None, return_all_layers: bool = False):
+    """Dilated stack: layer k takes its state from step t - dilations[k]
+    (default 2**k, the reference's choice, dilated_rnn.py:26).  xss as in stacked_lstm."""
+    L = len(Wss)
+    if dilations is None:
+        dilations = [2 ** k for k in range(L)]
+    return _run_stack(xss, Wss, Uss, bss, list(dilations), return_all_layers)
+
+
+def lstm_cell(hs_prev: FractalTensor, cs_prev: FractalTensor, xs: FractalTensor, ws: FractalTensor,
+              us: FractalTensor, bs: Optional[FractalTensor] = None):
+    """One batched cell: the `batched_cell` of stacked_rnn.py:40-50 as one launch.
+    hs_prev, cs_prev, xs: depth-1 [B] of [1, H]; ws, us: depth-1 [4] of [H, H]; bs: [4] of [1, H]."""
+    core = _core()
+    x = _dense_gpu(xs, 'xs', 1)
+    B, H = x.shape[0], x.shape[-1]
+    hp = _dense_gpu(hs_prev, 'hs_prev', 1).reshape(-1, H)[:B].contiguous()
+    cp = _dense_gpu(cs_prev, 'cs_prev', 1).reshape(-1, H)[:B].contiguous()
+    W = _dense_gpu(ws, 'ws', 1)
+    U = _dense_gpu(us, 'us', 1)
+    WU = torch.cat([W.permute(1, 0, 2).reshape(W.shape[1], 4 * H), U.permute(1, 0, 2).reshape(H, 4 * H)], dim=0).contiguous()
+    bias = None if bs is None else _dense_gpu(bs, 'bs', 1).reshape(4 * H).contiguous()
+    h, c = core.lstm_cell(x.reshape(B, -1).contiguous(), hp, cp, WU, bias)
+    return FractalTensor.from_dense(h.view(B, 1, H), 1), FractalTensor.from_dense(c.view(B, 1, H), 1)
+
+
+def flash_attention(qsss: FractalTensor, ksss: FractalTensor, vsss: FractalTensor, scale: Optional[float] = None):
+    """Blockwise attention.  qsss, ksss, vsss: depth-3 [batch][head][block] of
+    [block_rows, head_dim], the layout flash_attention_utils.create_input builds.
+    The result has the structure of qsss.  fp32 inputs are converted to fp16 for
+    the kernel (which accumulates in fp32) and the result converted back; `scale`
+    defaults to 1/sqrt(head_dim) (the reference program applies none: pass 1.0
+    for its exact maths)."""
+    core = _core()
+    q = _dense_gpu(qsss, 'qsss', 3)   # [B, Hd, nb, rows, D]
+    k = _dense_gpu(ksss, 'ksss', 3)
+    v = _dense_gpu(vsss, 'vsss', 3)
+    B, Hd, nbq, rq, D = q.shape
+    to4 = lambda t: t.reshape(t.shape[0], t.shape[1], t.shape[2] * t.shape[3], t.shape[4])
+    in_dtype = q.dtype
+    O = core.flash_attention(to4(q).half().contiguous(), to4(k).half().contiguous(), to4(v).half().contiguous(),
+                             D ** -0.5 if scale is None else float(scale))
+    return FractalTensor.from_dense(O.to(in_dtype).view(B, Hd, nbq, rq, D), 3)
+
+
+def b2b_gemm(a, b, c):
+    """(a @ b) @ c in one kernel.  a [M,K], b [K,N], c [N,P] Tensors, or
+    depth-1 FractalTensors of them (independent problems).  fp16 on the GPU."""
+    core = _core()
+
+    def dense(x, name):
+        if isinstance(x, FractalTensor):
+            return _dense_gpu(x, name, 1)
+        if isinstance(x, Tensor):
+            if not x.data.is_cuda:
+                raise RuntimeError(f'{name} lives on {x.data.device}; the fused kernels run on the GPU only.')
+            return x.data.unsqueeze(0)
+        raise TypeError(f'{name} should be a Tensor or a FractalTensor.')
+
+    A, Bm, Cm = dense(a, 'a'), dense(b, 'b'), dense(c, 'c')
+    in_dtype = A.dtype
+    # the kernel takes B and C with the contraction index contiguous
+    D = core.b2b_gemm(A.half().contiguous(), Bm.half().transpose(1, 2).contiguous(),
+                      Cm.half().transpose(1, 2).contiguous()).to(in_dtype)
+    if isinstance(a, Tensor):
+        return Tensor.from_tensor(D[0])
+    return FractalTensor.from_dense(D, 1)
+
+
+def online_softmax(x: Tensor) -> Tensor:
+    """Row softmax of a [rows, cols] fp32 Tensor through the online (max, sum) kernel."""
+    return Tensor.from_tensor(_core().online_softmax(x.data.contiguous()))

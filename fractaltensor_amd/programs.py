@@ -1,0 +1,122 @@
+"""The three hot-path model programs written against the kaleido operator API.
+
+These are the eager counterparts of the reference's example programs: every
+cell is a handful of torch calls on one sample and map / scan / fold are
+Python loops.  They serve as (1) the operator-level statement of what the
+fused kernels compute, used by the parity tests, and (2) the "CPU eager path"
+baseline that bench.py times on configuration 1.
+
+  stacked LSTM     examples/stacked_rnn/stacked_rnn.py:13-79 (time-major batch)
+  dilated LSTM     examples/dilated_rnn/dilated_rnn.py:16-41 (here over a time-major batch)
+  flash attention  examples/flash_attention/flash_attention.py:14-91, with the state
+                   initialised as the README's maths requires (max -inf, sum 0, o 0;
+                   the example seeds (sum, max, o) into a (max, sum, o) signature) and
+                   an explicit score scale
+"""
+from __future__ import annotations
+
+import torch
+
+from . import kaleido
+from .kaleido import FractalTensor, Tensor
+from .kaleido import operations as ops
+
+
+# ---- parameters and inputs ----------------------------------------------------
+
+def make_lstm_params(layers: int, hidden: int, scale: float, seed: int, device: str = 'cpu', bias: bool = True):
+    """Wss, Uss: depth-2 [layers][4] of [hidden, hidden] ~ U(-scale, scale); bss: [layers][4] of [1, hidden]."""
+    gen = torch.Generator().manual_seed(seed)
+    W = (torch.rand((layers, 4, hidden, hidden), generator=gen) * 2 - 1) * scale
+    U = (torch.rand((layers, 4, hidden, hidden), generator=gen) * 2 - 1) * scale
+    b = (torch.rand((layers, 4, 1, hidden), generator=gen) * 2 - 1) * scale if bias else torch.zeros((layers, 4, 1, hidden))
+    to = lambda t: FractalTensor.from_dense(t.to(device), 2)
+    return to(W), to(U), to(b)
+
+
+def make_sequence_batch(seq_len: int, batch: int, hidden: int, seed: int, device: str = 'cpu') -> FractalTensor:
+    """Time-major batch: depth-2 [seq_len][batch] of [1, hidden] ~ N(0, 1)."""
+    gen = torch.Generator().manual_seed(seed)
+    return FractalTensor.from_dense(torch.randn((seq_len, batch, 1, hidden), generator=gen).to(device), 2)
+
+
+def make_attention_input(batch: int, heads: int, seq_len: int, block: int, head_dim: int, seed: int,
+                         device: str = 'cpu', dtype=torch.float32) -> FractalTensor:
+    """depth-3 [batch][heads][seq_len/block] of [block, head_dim]."""
+    gen = torch.Generator().manual_seed(seed)
+    t = torch.randn((batch, heads, seq_len // block, block, head_dim), generator=gen)
+    return FractalTensor.from_dense(t.to(device=device, dtype=dtype), 3)
+
+
+# ---- LSTM ------------------------------------------------------------------------
+
+def lstm_cell(h_prev: Tensor, c_prev: Tensor, x: Tensor, ws: FractalTensor, us: FractalTensor, bs: FractalTensor):
+    """One sample, one step: four separate gate projections, gate order i, f, o, candidate."""
+    pre = ops.map(lambda p: x @ p[0] + h_prev @ p[1] + p[2], ops.zip(ws, us, bs))
+    i, f, o = (ops.sigmoid(pre[k]) for k in range(3))
+    c = f * c_prev + i * ops.tanh(pre[3])
+    h = o * ops.tanh(c)
+    return h, c
+
+
+def batched_cell(hs_prev, cs_prev, xs, ws, us, bs):
+    n = xs.length
+    return ops.map(lambda s: lstm_cell(s[0], s[1], s[2], ws, us, bs), ops.zip(hs_prev[0:n], cs_prev[0:n], xs))
+
+
+def lstm_layer(xss: FractalTensor, ws, us, bs, dilation: int = 1) -> FractalTensor:
+    hidden = xss.element_shape[-1]
+    zero = ops.repeat(ops.zeros(shape=(1, hidden), device=xss.device), xss[0].length)
+
+    def scan_time(seq):
+        hss, css = ops.scan(lambda state, xs: batched_cell(state[0], state[1], xs, ws, us, bs), seq,
+                            initializer=(zero, zero))
+        return hss, css
+
+    if dilation == 1:
+        return scan_time(xss)[0]
+    hss, _ = ops.dilated_map(scan_time, xss, dilation=dilation)
+    return hss
+
+
+def stacked_lstm(xss: FractalTensor, Wss, Uss, bss) -> FractalTensor:
+    """Layer l reads layer l-1's hidden sequence; returns the last layer's."""
+    return ops.fold(lambda seq, p: lstm_layer(seq, p[0], p[1], p[2]), ops.zip(Wss, Uss, bss), initializer=xss)
+
+
+def dilated_lstm(xss: FractalTensor, Wss, Uss, bss) -> FractalTensor:
+    """Layer k uses dilation 2**k."""
+    layers = ops.enumerate(Wss, Uss, bss)
+    return ops.fold(lambda seq, p: lstm_layer(seq, p[1], p[2], p[3], dilation=2 ** int(p[0].data.item())), layers,
+                    initializer=xss)
+
+
+# ---- attention -----------------------------------------------------------------------
+
+def _attend_block(state, q: Tensor, k: Tensor, v: Tensor, scale: float):
+    m_prev, l_prev, o_prev = state
+    w = ops.scale(q @ k.T, Tensor.from_tensor(torch.tensor([scale], dtype=q.data.dtype, device=q.data.device)))
+    m_cur = ops.max(w, dim=-1, keepdim=True)
+    e = ops.exp(w - m_cur)
+    ev = e @ v
+    l_cur = ops.sum(e, dim=-1, keepdim=True)
+    m_new = ops.maximum(m_cur, m_prev)
+    r_prev = ops.exp(m_prev - m_new)
+    r_cur = ops.exp(m_cur - m_new)
+    l_new = r_prev * l_prev + r_cur * l_cur
+    o = (o_prev * l_prev * r_prev + r_cur * ev) / l_new
+    return m_new, l_new, o
+
+
+def _attend_query_block(q: Tensor, ks: FractalTensor, vs: FractalTensor, scale: float) -> Tensor:
+    rows, dim = q.shape
+    dev = q.device
+    init = (ops.full(shape=(rows, 1), fill_value=float('-inf'), device=dev), ops.zeros(shape=(rows, 1), device=dev),
+            ops.zeros(shape=(rows, dim), device=dev))
+    _, _, o = ops.reduce(lambda st, kv: _attend_block(st, q, kv[0], kv[1], scale), ops.zip(ks, vs), initializer=init)
+    return o
+
+
+def flash_attention(qsss: FractalTensor, ksss: FractalTensor, vsss: FractalTensor, scale: float) -> FractalTensor:
+    per_head = lambda qkv: ops.map(lambda q: _attend_query_block(q, qkv[1], qkv[2], scale), qkv[0])
+    return ops.map(lambda sample: ops.map(per_head, ops.zip(*sample)), ops.zip(qsss, ksss, vsss))

@@ -1,0 +1,355 @@
+"""The kaleido-compatible frontend on the CPU: the known answers the reference's own
+frontend tests hold, restated, and the eager model programs against the oracle."""
+import itertools
+import operator
+import random
+
+import numpy as np
+import pytest
+import torch
+
+import fractaltensor_amd.kaleido as kaleido
+from fractaltensor_amd import programs
+from fractaltensor_amd.kaleido import FractalTensor, Iterative, Tensor, TensorStorage, FractalTensorStorage
+from fractaltensor_amd.kaleido import operations as ops
+from oracle import kaleido_oracle as ko
+
+
+# ---- containers (kaleido/frontend/tests/test_fractaltensor_creation.py) ----------------
+
+@pytest.mark.parametrize('shape', [[13], [3, 7], [7, 11, 3], [3, 7, 2, 11, 5]])
+def test_row_major_strides(shape):                      # :14-46
+    t = Tensor(shape, kaleido.float32, device='cpu')
+    n = int(np.prod(shape))
+    t.initialize(torch.arange, n, dtype=torch.float32)
+    t.data = t.data.view(shape)
+    assert t.data.ndim == t.ndim
+    rnd = random.Random(1)
+    idx = [rnd.randint(0, s - 1) for s in shape]
+    off = sum(i * s for i, s in zip(idx, t.strides))
+    assert t.data.reshape(-1)[off] == off
+
+
+def test_from_tensors_keeps_shapes():                   # :55-70
+    ts = []
+    for _ in range(5):
+        t = Tensor([3, 7, 5], kaleido.float32, device='cpu')
+        t.initialize(torch.rand, *t.shape)
+        ts.append(t)
+    ft = FractalTensor.from_tensors(*ts)
+    assert ft.depth == 1 and len(ft) == 5
+    for i, t in enumerate(ft):
+        assert tuple(t.shape) == (3, 7, 5) and torch.equal(t.data, ts[i].data)
+
+
+def test_nested_from_uninitialised_children():          # :72-106
+    mk = lambda: FractalTensor(TensorStorage((3, 4), kaleido.float32, device='cpu', order='row'))
+    x = FractalTensor.from_fractaltensors(mk(), mk(), mk())
+    y = FractalTensor.from_fractaltensors(mk(), mk())
+    z = FractalTensor.from_fractaltensors(x, y)
+    z.indices = [[list(range(7)), list(range(11)), list(range(2))], [list(range(9)), list(range(1))]]
+    assert z.depth == 3 and z.numel == 30 and z.flatten_shape == (30, 3, 4)
+    z.initialize(torch.rand, *z.flatten_shape)
+    assert tuple(z[0][1][10].shape) == (3, 4)
+    assert torch.equal(z[1][0][0].data, z.data.view(30, 3, 4)[20])
+
+
+def test_from_pylist_flat():                            # :108-116
+    x = FractalTensor.from_pylist(list(range(13)))
+    assert x.depth == 1
+    for i in range(len(x)):
+        assert x[i].data == i
+
+
+def test_from_pylist_ragged_depth3():                   # :118-140
+    rnd = random.Random(12345)
+    data, start = [], 0
+    for _ in range(rnd.randint(1, 23)):
+        row = []
+        for _ in range(rnd.randint(1, 23)):
+            end = start + rnd.randint(1, 23)
+            row.append(list(range(start, end)))
+            start = end
+        data.append(row)
+    x = FractalTensor.from_pylist(data)
+    assert x.depth == 3
+    v = 0
+    for i in range(len(x)):
+        for j in range(len(x[i])):
+            for k in range(len(x[i][j])):
+                assert x[i][j][k].data[0] == v
+                v += 1
+
+
+def test_width_by_depth_literals():                     # :142-172
+    x = FractalTensor.from_pylist([[0, 1, 2], [3, 4], [5, 6, 7, 8]])
+    assert x.depth == 2
+    assert x.width_by_depth(-1) == [3]
+    assert x.width_by_depth(-2) == [3, 2, 4]
+    with pytest.raises(ValueError):
+        x.width_by_depth(-3)
+    x = FractalTensor.from_pylist([[[0, 1], [2, 3, 4], [5]], [[6, 7, 8, 9]], [[10]]])
+    assert x.depth == 3
+    assert x.width_by_depth(-1) == [3]
+    assert x.width_by_depth(-2) == [3, 1, 1]
+    assert x.width_by_depth(-3) == [2, 3, 1, 4, 1]
+    with pytest.raises(ValueError):
+        x.width_by_depth(-4)
+
+
+def test_type_equivalence():                            # tests/test_type_equivalence.py:17-43
+    from fractaltensor_amd.kaleido import Real, Int, Bool
+    assert not Real(64).is_equal_type(Int(32))
+    assert not Real(64).is_equal_type(Real(32))
+    assert not Bool().is_equal_type(Real(16))
+    assert Real(64).is_equal_type(Real(64)) and Int(16).is_equal_type(Int(16))
+    x = TensorStorage((2, 64), kaleido.float32, device='cpu')
+    assert x.is_equal_type(x)
+    assert not x.is_equal_type(TensorStorage((1, 3), kaleido.float32, 'cpu'))
+    y = FractalTensorStorage(TensorStorage((2, 64), kaleido.float32, device='cpu'))
+    assert y.is_equal_type(FractalTensorStorage(TensorStorage((2, 64), kaleido.float32, device='cpu')))
+    assert not y.is_equal_type(FractalTensorStorage(TensorStorage((4, 7), kaleido.float32, device='cpu')))
+
+
+def test_dense_view_is_zero_copy_and_ragged_has_none():
+    t = torch.arange(2 * 3 * 4 * 5, dtype=torch.float32).view(2, 3, 4, 5)
+    ft = FractalTensor.from_dense(t, 2)
+    assert ft.depth == 2 and ft.dense_shape() == (2, 3) and ft.element_shape == (4, 5)
+    assert ft.as_dense().data_ptr() == ft.data.data_ptr()
+    assert torch.equal(ft[1][2].data, t[1, 2])
+    ragged = FractalTensor.from_pylist([[0, 1, 2], [3, 4]])
+    assert not ragged.is_regular()
+    with pytest.raises(ValueError):
+        ragged.as_dense()
+
+
+# ---- parallel functions (operations/tests/test_aggregate.py, test_apply_to_each.py) -------
+
+def _ints(n=17, seed=12345):
+    rnd = random.Random(seed)
+    data = [rnd.randint(0, 193) for _ in range(n)]
+    return data, FractalTensor.from_pylist(data)
+
+
+def test_scan_is_accumulate():                          # test_aggregate.py:27-47
+    data, xs = _ints()
+    ys = ops.scan(lambda s, x: ops.add(s, x), xs)
+    assert isinstance(ys, FractalTensor) and len(ys) == len(xs)
+    assert [y.data.item() for y in ys] == list(itertools.accumulate(data, operator.add))
+    init = Tensor((1,), kaleido.int32)
+    init.data = torch.LongTensor([5])
+    ys = ops.scan(lambda s, x: ops.add(s, x), xs, init)
+    expected = list(itertools.accumulate([5] + data, operator.add))
+    assert [y.data.item() for y in ys] == expected[1:]
+    assert ops.fold(lambda s, x: ops.add(s, x), xs, init).data.item() == expected[-1]
+    assert ops.reduce(lambda s, x: ops.add(s, x), xs, init).data.item() == expected[-1]
+
+
+def test_scan_with_two_outputs():                       # test_aggregate.py:49-57
+    data, xs = _ints()
+    init = Tensor((1,), kaleido.int32)
+    init.data = torch.LongTensor([5])
+    ys, zs = ops.scan(lambda s, x: (x, x), xs, init)
+    for x, y, z in ops.zip(xs, ys, zs):
+        assert y.data.item() == x.data.item() == z.data.item()
+
+
+def test_functional_rejects_python_lists():             # test_apply_to_each.py:19-29
+    for fn in (ops.map, ops.fold, ops.scan, ops.reduce, ops.filter, ops.dilated_map):
+        with pytest.raises(TypeError):
+            fn(lambda x: x, [1, 2, 3])
+
+
+def test_nested_map_and_multiple_outputs():             # test_apply_to_each.py:31-54
+    xss = FractalTensor.from_pylist([[0, 1, 2], [3, 4], [5, 6, 7, 8]])
+    yss = ops.map(lambda xs: ops.map(lambda x: x, xs), xss)
+    a, b = ops.map(lambda xs: ops.map(lambda x: (x, x), xs), xss)
+    for i, row in enumerate(xss):
+        for j, x in enumerate(row):
+            assert x.data == yss[i][j].data == a[i][j].data == b[i][j].data
+
+
+def test_map_over_zip():                                # test_apply_to_each.py:56-77
+    xs1 = FractalTensor.from_pylist(list(range(7)))
+    xs2 = FractalTensor.from_pylist(list(range(7, 14)))
+    ys, zs = ops.map(lambda p: (p[0], p[1]), ops.zip(xs1, xs2))
+    for y, z, x1, x2 in ops.zip(ys, zs, xs1, xs2):
+        assert y.data.eq(x1.data).all() and z.data.eq(x2.data).all()
+
+
+def test_map_returning_iterative():                     # test_apply_to_each.py:79-91
+    xss = FractalTensor.from_pylist([[0, 1, 2], [3, 4], [5, 6, 7, 8]])
+
+    def f(xs):
+        v1, v2 = ops.map(lambda x: (x, x), xs)
+        return ops.zip(v1, v2)
+
+    yss, zss = ops.map(f, xss)
+    for i, ys in enumerate(yss):
+        for j, _ in enumerate(ys):
+            assert yss[i][j].data.item() == zss[i][j].data.item() == xss[i][j].data.item()
+
+
+def test_filter():
+    xs = FractalTensor.from_pylist(list(range(10)))
+    even = ops.filter(lambda x: x.data.item() % 2 == 0, xs)
+    assert [e.data.item() for e in even] == [0, 2, 4, 6, 8]
+    assert ops.filter(lambda x: False, xs) is None
+
+
+# ---- access and conversion (test_zip.py, test_product.py, test_join.py, test_flatten.py, test_constants.py)
+
+def test_zip_and_nested_zip():                          # test_zip.py:22-36
+    xs1 = FractalTensor.from_pylist(list(range(7)))
+    xs2 = FractalTensor.from_pylist(list(range(7, 14)))
+    z = ops.zip(xs1, xs2)
+    assert isinstance(z, Iterative)
+    for a, b in z:
+        assert b.data - a.data == 7
+    for ab, c in ops.zip(ops.zip(xs1, xs2), xs1):
+        a, b = ab
+        assert b.data - a.data == 7 and b.data - c.data == 7
+    assert ops.zip(xs1) is xs1
+    with pytest.raises(ValueError):
+        ops.zip(xs1, FractalTensor.from_pylist([1, 2]))
+
+
+def test_product():                                     # test_product.py:21-29
+    x = FractalTensor.from_pylist(list(range(11)))
+    y = FractalTensor.from_pylist(list(range(7)))
+    xss, yss = ops.product(x, y)
+    assert isinstance(xss, FractalTensor) and isinstance(yss, FractalTensor)
+    for i, (xs, ys) in enumerate(ops.zip(xss, yss)):
+        for j, (a, b) in enumerate(ops.zip(xs, ys)):
+            assert a.data.item() == j and b.data.item() == i
+
+
+def _rand_ft(depth, length, rnd):
+    elem = TensorStorage([3, 7], kaleido.float32, device='cpu')
+    if depth == 1:
+        ft = FractalTensor(elem)
+        ft.indices = list(range(length))
+    else:
+        ft = FractalTensor(FractalTensorStorage(elem))
+        ft.indices = [list(range(rnd.randint(5, 17))) for _ in range(length)]
+    ft.initialize(torch.rand, *ft.flatten_shape)
+    return ft
+
+
+def test_join():                                        # test_join.py:36-54
+    rnd = random.Random(12345)
+    for depth, (n1, n2) in ((1, (19, 3)), (2, (11, 7))):
+        a, b = _rand_ft(depth, n1, rnd), _rand_ft(depth, n2, rnd)
+        c = ops.join(a, b)
+        assert isinstance(c, FractalTensor) and c.depth == a.depth
+        assert len(c) == len(a) + len(b) and c.numel == a.numel + b.numel
+        assert torch.equal(c[len(a)].data if depth == 1 else c[len(a)][0].data, b[0].data if depth == 1 else b[0][0].data)
+
+
+@pytest.mark.parametrize('dim', [0, 1])
+def test_flatten_shapes(dim):                           # test_flatten.py:39-59
+    rnd = random.Random(5)
+    x = _rand_ft(2, 5, rnd)
+    count = x.numel
+    y = ops.flatten(x, dim)
+    assert isinstance(y, Tensor)
+    expect = [3, 7]
+    expect[dim] *= count
+    assert list(y.shape) == expect
+    if dim == 0:
+        assert torch.equal(y.data[3:6], x[0][1].data)
+
+
+def test_arange_slices_and_constants():                 # test_constants.py:16-34
+    for args in ((11,), (5, 7), (5, 24, 3)):
+        ft = ops.slices(ops.arange(*args), dim=0)
+        assert isinstance(ft, FractalTensor)
+        assert isinstance(ft.element_type.dtype, kaleido.Int)
+        assert [x.data.item() for x in ft] == list(range(*args))
+    z = ops.zeros(shape=(3, 7), dtype='float', device='cpu')
+    o = ops.ones(shape=(3, 7), dtype='float', device='cpu')
+    assert z.data.sum() == 0 and o.data.sum() == 21
+    rows = ops.slices(Tensor.from_tensor(torch.arange(12.).view(3, 4)), dim=0)
+    assert rows[1].shape == (1, 4)      # a row of a matrix stays a row vector
+    rep = ops.repeat(ops.zeros(shape=(1, 8), device='cpu'), 5)
+    assert rep.depth == 1 and len(rep) == 5 and rep.element_shape == (1, 8)
+
+
+def test_tensor_operators():
+    a = Tensor.from_tensor(torch.tensor([[1., 2.], [3., 4.]]))
+    b = Tensor.from_tensor(torch.tensor([[5., 6.], [7., 8.]]))
+    assert torch.equal((a + b).data, a.data + b.data)
+    assert torch.equal((a - b).data, a.data - b.data)
+    assert torch.equal((a * b).data, a.data * b.data)
+    assert torch.equal((a @ b).data, a.data @ b.data)
+    assert torch.equal((a / b).data, a.data / b.data)
+    assert torch.equal((a * 2.0).data, a.data * 2)
+    assert torch.equal(a.T.data, a.data.t())
+    with pytest.raises(ValueError):
+        ops.add(a, Tensor.from_tensor(torch.zeros(3, 3)))
+    with pytest.raises(TypeError):
+        ops.add(a, 3)
+
+
+def test_decorators_are_pass_through():
+    ctx = kaleido.Context()
+
+    @kaleido.function(ctx)
+    def f(x: Tensor['1, 4', float, 'cpu']) -> Tensor['1, 4', float, 'cpu']:
+        return x + x
+
+    out = f(Tensor.from_tensor(torch.ones(1, 4)))
+    assert out.data.sum() == 8
+    ctx[-1].ir_block.propagate_storage()
+    kaleido.PlotProgram().plot(ctx[-1].ir_block)
+
+
+# ---- eager model programs against the oracle -----------------------------------------------
+
+def _np_params(Wss, Uss, bss):
+    W = Wss.as_dense().numpy(); U = Uss.as_dense().numpy(); b = bss.as_dense().numpy()
+    L, _, H, _ = W.shape
+    WU = np.stack([ko.fuse_gate_weights(W[l], U[l]) for l in range(L)])
+    return WU, b.reshape(L, 4 * H)
+
+
+def test_eager_stacked_lstm_matches_oracle():
+    L, T, B, H = 2, 4, 3, 16
+    Wss, Uss, bss = programs.make_lstm_params(L, H, 0.3, seed=1)
+    xss = programs.make_sequence_batch(T, B, H, seed=2)
+    out = programs.stacked_lstm(xss, Wss, Uss, bss)
+    assert out.depth == 2 and out.dense_shape() == (T, B)
+    WU, bias = _np_params(Wss, Uss, bss)
+    hs, _ = ko.stacked_lstm(xss.as_dense().numpy().reshape(T, B, H), WU, bias, dtype=np.float32)
+    np.testing.assert_allclose(out.as_dense().numpy().reshape(T, B, H), hs[-1], atol=2e-6)
+
+
+def test_eager_dilated_lstm_matches_oracle():
+    L, T, B, H = 3, 9, 2, 8
+    Wss, Uss, bss = programs.make_lstm_params(L, H, 0.3, seed=3)
+    xss = programs.make_sequence_batch(T, B, H, seed=4)
+    out = programs.dilated_lstm(xss, Wss, Uss, bss)
+    WU, bias = _np_params(Wss, Uss, bss)
+    hs, _ = ko.stacked_lstm(xss.as_dense().numpy().reshape(T, B, H), WU, bias, dilations=[1, 2, 4], dtype=np.float32)
+    np.testing.assert_allclose(out.as_dense().numpy().reshape(T, B, H), hs[-1], atol=2e-6)
+
+
+def test_eager_flash_attention_matches_oracle():
+    B, Hd, S, blk, D = 1, 2, 32, 8, 16
+    q, k, v = (programs.make_attention_input(B, Hd, S, blk, D, seed=s) for s in (5, 6, 7))
+    scale = D ** -0.5
+    out = programs.flash_attention(q, k, v, scale)
+    assert out.depth == 3 and out.dense_shape() == (B, Hd, S // blk)
+    dense = lambda ft: ft.as_dense().numpy().reshape(B, Hd, S, D)
+    ref = ko.attention(dense(q), dense(k), dense(v), scale, dtype=np.float32)
+    np.testing.assert_allclose(dense(out), ref, atol=2e-6)
+
+
+def test_fused_paths_refuse_cpu_inputs():
+    Wss, Uss, bss = programs.make_lstm_params(1, 32, 0.1, seed=1)
+    xss = programs.make_sequence_batch(2, 2, 32, seed=2)
+    with pytest.raises(RuntimeError, match='GPU only'):
+        ops.fused.stacked_lstm(xss, Wss, Uss, bss)
+    q = programs.make_attention_input(1, 1, 64, 64, 64, seed=1)
+    with pytest.raises(RuntimeError, match='GPU only'):
+        ops.fused.flash_attention(q, q, q)

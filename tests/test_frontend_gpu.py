@@ -1,0 +1,101 @@
+"""Fused fast paths behind the kaleido operator API, on the GPU: each against the eager
+operator program it replaces (same FractalTensor inputs, on the GPU) and against the oracle."""
+import numpy as np
+import pytest
+import torch
+
+from fractaltensor_amd import programs
+from fractaltensor_amd.kaleido import FractalTensor, Tensor
+from fractaltensor_amd.kaleido import operations as ops
+from oracle import kaleido_oracle as ko
+
+pytestmark = pytest.mark.gpu
+
+
+def _np_params(Wss, Uss, bss):
+    W = Wss.as_dense().cpu().numpy(); U = Uss.as_dense().cpu().numpy(); b = bss.as_dense().cpu().numpy()
+    L, _, H, _ = W.shape
+    return np.stack([ko.fuse_gate_weights(W[l], U[l]) for l in range(L)]), b.reshape(L, 4 * H)
+
+
+@pytest.mark.parametrize('L,T,B,H', [(2, 3, 4, 32), (3, 4, 33, 256)])
+def test_fused_stacked_lstm_equals_eager_program(L, T, B, H):
+    Wss, Uss, bss = programs.make_lstm_params(L, H, 1 / 16, seed=1, device='cuda')
+    xss = programs.make_sequence_batch(T, B, H, seed=2, device='cuda')
+    fused = ops.fused.stacked_lstm(xss, Wss, Uss, bss)
+    assert isinstance(fused, FractalTensor) and fused.depth == 2 and fused.dense_shape() == (T, B)
+    assert fused.element_shape == (1, H)
+    got = fused.as_dense().cpu().numpy().reshape(T, B, H)
+    WU, bias = _np_params(Wss, Uss, bss)
+    ref, _ = ko.stacked_lstm(xss.as_dense().cpu().numpy().reshape(T, B, H), WU, bias)
+    assert ko.max_rel_err(got, ref[-1]) <= 1e-4
+    if B <= 4:   # the eager program is L*T*B Python cell calls
+        eager = programs.stacked_lstm(xss, Wss, Uss, bss)
+        assert ko.max_rel_err(got, eager.as_dense().cpu().numpy().reshape(T, B, H)) <= 1e-4
+    hsss, csss = ops.fused.stacked_lstm(xss, Wss, Uss, bss, return_all_layers=True)
+    assert hsss.depth == 3 and hsss.dense_shape() == (L, T, B)
+    assert ko.max_rel_err(hsss.as_dense().cpu().numpy().reshape(L, T, B, H), ref) <= 1e-4
+
+
+def test_fused_dilated_lstm_equals_eager_program():
+    L, T, B, H = 3, 9, 2, 32
+    Wss, Uss, bss = programs.make_lstm_params(L, H, 1 / 16, seed=3, device='cuda')
+    xss = programs.make_sequence_batch(T, B, H, seed=4, device='cuda')
+    fused = ops.fused.dilated_lstm(xss, Wss, Uss, bss).as_dense().cpu().numpy().reshape(T, B, H)
+    eager = programs.dilated_lstm(xss, Wss, Uss, bss).as_dense().cpu().numpy().reshape(T, B, H)
+    WU, bias = _np_params(Wss, Uss, bss)
+    ref, _ = ko.stacked_lstm(xss.as_dense().cpu().numpy().reshape(T, B, H), WU, bias, dilations=[1, 2, 4])
+    assert ko.max_rel_err(fused, ref[-1]) <= 1e-4
+    assert ko.max_rel_err(fused, eager) <= 1e-4
+
+
+def test_fused_lstm_cell_equals_eager_batched_cell():
+    B, H = 5, 64
+    Wss, Uss, bss = programs.make_lstm_params(1, H, 0.1, seed=5, device='cuda')
+    ws, us, bs = Wss[0], Uss[0], bss[0]
+    g = torch.Generator().manual_seed(6)
+    mk = lambda: FractalTensor.from_dense(torch.randn((B, 1, H), generator=g).cuda(), 1)
+    hs, cs, xs = mk(), mk(), mk()
+    h1, c1 = ops.fused.lstm_cell(hs, cs, xs, ws, us, bs)
+    h2, c2 = programs.batched_cell(hs, cs, xs, ws, us, bs)
+    assert ko.max_rel_err(h1.as_dense().cpu().numpy(), h2.as_dense().cpu().numpy()) <= 1e-4
+    assert ko.max_rel_err(c1.as_dense().cpu().numpy(), c2.as_dense().cpu().numpy()) <= 1e-4
+
+
+def test_fused_flash_attention_equals_eager_program():
+    B, Hd, S, blk, D = 1, 2, 256, 64, 64          # the example's block size (flash_attention.py:96-110)
+    q, k, v = (programs.make_attention_input(B, Hd, S, blk, D, seed=s, device='cuda') for s in (5, 6, 7))
+    scale = D ** -0.5
+    fused = ops.fused.flash_attention(q, k, v, scale)
+    assert fused.depth == 3 and fused.dense_shape() == (B, Hd, S // blk) and fused.element_shape == (blk, D)
+    dense = lambda ft: ft.as_dense().cpu().numpy().reshape(B, Hd, S, D)
+    eager = programs.flash_attention(q, k, v, scale)
+    ref = ko.attention(dense(q), dense(k), dense(v), scale)
+    assert ko.max_rel_err(dense(fused), ref) <= 1e-2          # fp16 kernel vs fp64 reference
+    assert ko.max_rel_err(dense(eager), ref) <= 1e-5          # fp32 eager program
+    assert ko.max_rel_err(dense(fused), dense(eager)) <= 1e-2
+
+
+def test_fused_b2b_gemm_equals_operator_expression():
+    M, K, N, P = 128, 64, 96, 32
+    g = torch.Generator().manual_seed(8)
+    a = Tensor.from_tensor((torch.randn((M, K), generator=g) / K ** 0.5).half().cuda())
+    b = Tensor.from_tensor((torch.randn((K, N), generator=g) / K ** 0.5).half().cuda())
+    c = Tensor.from_tensor((torch.randn((N, P), generator=g) / N ** 0.5).half().cuda())
+    fused = ops.fused.b2b_gemm(a, b, c)
+    eager = (a @ b) @ c
+    ref = ko.b2b_gemm(a.data.cpu().numpy(), b.data.t().cpu().numpy(), c.data.t().cpu().numpy())
+    assert ko.max_rel_err(fused.data.cpu().numpy(), ref) <= 1e-2
+    assert ko.max_rel_err(fused.data.cpu().numpy(), eager.data.float().cpu().numpy()) <= 1e-2
+    batch = FractalTensor.from_tensors(a, a)
+    out = ops.fused.b2b_gemm(batch, FractalTensor.from_tensors(b, b), FractalTensor.from_tensors(c, c))
+    assert out.depth == 1 and len(out) == 2 and torch.equal(out[1].data, fused.data)
+
+
+def test_fused_paths_reject_ragged_input():
+    Wss, Uss, bss = programs.make_lstm_params(1, 32, 0.1, seed=1, device='cuda')
+    t = torch.randn(5, 1, 32).cuda()
+    row = lambda n: FractalTensor.from_dense(t[:n].contiguous(), 1)
+    ragged = FractalTensor.from_fractaltensors(row(3), row(2))
+    with pytest.raises(ValueError, match='ragged'):
+        ops.fused.stacked_lstm(ragged, Wss, Uss, bss)
