@@ -22,6 +22,7 @@ EXPORTS = (
     'ftk_stacked_lstm_workspace_bytes', 'ftk_stacked_lstm_f32', 'ftk_dilated_lstm_f32',
     'ftk_stacked_lstm_wavefront_f32',
     'ftk_b2b_gemm_f16', 'ftk_flash_attn_f16', 'ftk_online_softmax_f32',
+    'ftk_debug_read_fa_trace',
 )
 
 
@@ -233,6 +234,14 @@ def flash_attention(Q, K, V, scale: Optional[float] = None, out: Optional[torch.
     _check(lib.ftk_flash_attn_f16(_ptr(Q), _ptr(K), _ptr(V), _ptr(O), ci(B), ci(Hd), ci(Sq), ci(Skv), ci(D),
                                   ctypes.c_float(scale), _stream()))
     return O
+
+
+def read_fa_trace(tiles: int):
+    """Timeline of one wave of workgroup 0 of the last flash-attention launch (needs FTK_FA_TRACE=1+wave): [tiles, 6] in us."""
+    import numpy as np
+    buf = (ctypes.c_longlong * (tiles * 6))()
+    _check(lib.ftk_debug_read_fa_trace(buf, ctypes.c_int(tiles * 6)))
+    return np.frombuffer(buf, dtype=np.int64).reshape(tiles, 6).astype(np.float64) / 100.0
 
 
 def online_softmax(x) -> torch.Tensor:

@@ -2,23 +2,40 @@
 // v_mfma_f32_32x32x16_f16, online softmax (running max and sum) in registers.
 //
 // Both contractions are computed transposed so that a lane owns one query row:
-//   S^T[key, q] = sum_d Ks[key][d] * Q[q][d]     MFMA A-operand = K rows (LDS),
+//   S^T[key, q] = sum_d K[key][d] * Q[q][d]      MFMA A-operand = K rows (LDS),
 //                                                B-operand = Q row fragments (registers)
-//   O^T[d, q]  += sum_key Vt[d][key] * P[q][key]  A-operand = V^T rows (LDS),
+//   O^T[d, q]  += sum_key V[key][d] * P[q][key]   A-operand = V columns (LDS, transposing read),
 //                                                B-operand = exp'd scores, fp16 (registers)
 // The 32x32 accumulator of lane (q = lane%32, half = lane/32) holds, for that
-// one query, keys 8g + 4*half + r (g = reg/4, r = reg%4) of a 32-key subtile.
+// one query, keys 8g + 4*half + r (g = reg/4, r = reg%4) of a 32-key half tile.
 // Row max / row sum are therefore a reduction over the lane's own registers
 // plus one exchange with lane^32; the rescale factor of O^T is lane-local; and
 // the exp'd scores already are a valid MFMA B-operand if the PV product
-// contracts keys in the order the lane holds them (step s of a subtile takes
-// keys {16s + 4*half + r} U {16s + 8 + 4*half + r}), which only changes which
-// two 8-byte pieces of a V^T row the A-operand reads.  P never touches LDS.
+// contracts keys in the order the lane holds them (step s of a half tile takes
+// keys {16s + 4*half + r} U {16s + 8 + 4*half + r}).  P never touches LDS.
 //
-// A workgroup is 4 waves; each wave owns 32*QT query rows, the workgroup
-// streams K/V in 64-key tiles: K as stored ([key][d], padded rows), V
-// transposed on the way into LDS ([d][key]) by 4x4 register transposes.  Tiles
-// are double buffered with register prefetch of the next tile.
+// K and V tiles of 64 keys go from global memory straight into LDS
+// (global_load_lds_dwordx4, 1 KB per wave instruction), both row-major as in
+// memory, so staging costs no registers, no vector instructions and no LDS
+// stores.  Each lane picks the 16 global bytes that land in its fixed LDS
+// slot, so the LDS rows can carry padding (FaLayout) that makes fragment reads
+// bank-conflict free at plain immediate offsets: no address arithmetic in the
+// loop.  The A-operand of the PV product is read with ds_read_b64_tr_b16,
+// where 16 lanes hand in the addresses of a 4-key x 16-column block (lane
+// 4a+b: key a, columns 4b..4b+3) and lane i receives column i of the four
+// keys, so V needs no transposed copy.  K is triple buffered (the scores of
+// tile kt+1 are started during tile kt), V double buffered; one barrier per
+// tile publishes the copies.
+//
+// What the loop is built around, measured on MI355X with two waves per SIMD:
+// vector instructions do not hide behind MFMAs the way loads do -- a handful
+// per MFMA are free, every further one costs issue time -- and dot-product
+// instructions (v_dot2*) run on the matrix pipeline and stall it outright.
+// So the per-score work is cut to one exponential, one add and half a pack:
+// Q is pre-multiplied by scale*log2(e), the reference maximum is subtracted by
+// the matrix unit itself (score accumulators start from -m_ref instead of 0),
+// row sums use plain adds, and the loop is software pipelined per 32-key half
+// tile with the instruction order written out and fenced step by step.
 #include <stdlib.h>
 
 #include <algorithm>
@@ -40,27 +57,81 @@ __device__ __forceinline__ void static_for(F&& f) {
 }
 
 constexpr int FA_KT = 64;          // keys per tile
-constexpr int FA_VLD = FA_KT + 4;  // padded V^T row (halfs)
 constexpr float FA_TAU = 8.0f;     // slack (in powers of two) before the running maximum is moved
+constexpr int FA_TRACE_TILES = 256;
 
-template <int D, int QT, int WAVES>
-__global__ __launch_bounds__(WAVES * 64) void flash_attn_kernel(const _Float16* __restrict__ Q,
+// Timeline of workgroup 0 / thread 0 when FTK_FA_TRACE is set: six stamps per key tile.
+__device__ long long fa_trace_buf[FA_TRACE_TILES * 6];
+
+typedef short v4s __attribute__((ext_vector_type(4)));
+
+// 16 bytes per lane from global memory (wave-uniform base + per-lane byte
+// offset) straight into LDS at lds_base + 16*lane (lds_base wave-uniform).
+// Issued as opaque assembly on purpose: the compiler would otherwise wait for
+// every outstanding copy before the next LDS read that it cannot prove
+// disjoint, which serialises the prefetch.  The caller waits with vmcnt(0)
+// before the barrier that publishes the tile.
+__device__ __forceinline__ void lds_dma16(const void* gbase, unsigned byte_off, void* lds_base) {
+  const unsigned lds_addr = (unsigned)reinterpret_cast<uintptr_t>((__attribute__((address_space(3))) void*)lds_base);
+  asm volatile(
+      "s_mov_b32 m0, %0\n\t"
+      "s_nop 0\n\t"
+      "global_load_lds_dwordx4 %1, %2"
+      :
+      : "s"(lds_addr), "v"(byte_off), "s"(gbase)
+      : "memory", "m0");
+}
+
+// max(x, x of lane^32) without a trip through LDS: v_permlane32_swap exchanges
+// the upper half of the first register with the lower half of the second, so
+// with both holding x, afterwards one holds the lower lanes' x in every lane
+// and the other the upper lanes'.  (Written as assembly: the compiler folds
+// the two results of its builtin into one.)
+__device__ __forceinline__ float max_with_other_half(float x) {
+  float y = x;
+  asm volatile("s_nop 1\n\tv_permlane32_swap_b32_e32 %0, %1\n\ts_nop 1" : "+v"(x), "+v"(y));
+  return fmaxf(x, y);
+}
+
+// LDS layout of a 64-key tile: rows as in memory plus padding, chosen so that
+// fragment reads are bank-conflict free with plain immediate offsets:
+//   K rows are padded by 16 bytes: a fragment read (ds_read_b128, 16 lanes =
+//     16 consecutive keys, same columns) then touches 16 different 16-byte
+//     chunks of the 256-byte bank line;
+//   V rows are padded by 64 bytes: one 32-lane pass of the transposing read
+//     covers 4 keys x 64 bytes, which land in four different 64-byte groups.
+template <int D>
+struct FaLayout {
+  static constexpr int KRS = 2 * D + 16;   // K row stride, bytes
+  static constexpr int VRS = 2 * D + 64;   // V row stride, bytes
+  static constexpr int KTB = FA_KT * KRS;  // K tile, bytes (a multiple of 1024)
+  static constexpr int VTB = FA_KT * VRS;
+  static_assert(KTB % 1024 == 0 && VTB % 1024 == 0, "tiles must be whole 1 KB copies");
+};
+
+// MINB: workgroups per CU the register budget must allow.
+template <int D, int QT, int WAVES, int MINB, bool TRACE>
+__global__ __launch_bounds__(WAVES * 64, MINB) void flash_attn_kernel(const _Float16* __restrict__ Q,
                                                          const _Float16* __restrict__ K,
                                                          const _Float16* __restrict__ V,
                                                          _Float16* __restrict__ O, int Sq, int Skv,
-                                                         float scale_log2e, int nqb) {
-  constexpr int KLD = D + 8;   // padded K row (halfs)
-  constexpr int DS = D / 16;   // k steps of S^T
-  constexpr int DT = D / 32;   // d tiles of O^T
-  constexpr int KSZ = FA_KT * KLD;
-  constexpr int VSZ = D * FA_VLD;
-  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
-  _Float16* Ks = reinterpret_cast<_Float16*>(smem);  // [2][64][KLD]
-  _Float16* Vt = Ks + 2 * KSZ;                       // [2][D][VLD]
+                                                         float scale_log2e, int nqb,
+                                                         long long* __restrict__ trace, int trace_wave) {
+  using L = FaLayout<D>;
+  constexpr int DS = D / 16;  // k steps of S^T
+  constexpr int DT = D / 32;  // d tiles of O^T
+  constexpr int RB = 2 * D;   // bytes per K or V row in global memory
+  constexpr int KRS = L::KRS, VRS = L::VRS, KTB = L::KTB, VTB = L::VTB;
+  constexpr int KCP = (KTB / 1024 + WAVES - 1) / WAVES;  // 1 KB copies per wave per K tile (upper bound)
+  constexpr int VCP = (VTB / 1024 + WAVES - 1) / WAVES;
+  extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];
+  unsigned char* const Kb = smem;            // [3][KTB]
+  unsigned char* const Vb = smem + 3 * KTB;  // [2][VTB]
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
-  const int wave = tid >> 6;
+  // wave index as a scalar, so that LDS copy destinations are provably wave-uniform
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int j = lane & 31;
   const int hh = lane >> 5;
   // One-dimensional grid of nqb query blocks x (batch*heads).  The hardware
@@ -71,7 +142,6 @@ __global__ __launch_bounds__(WAVES * 64) void flash_attn_kernel(const _Float16* 
   if ((total & 7) == 0) id = (blockIdx.x & 7) * (total >> 3) + (blockIdx.x >> 3);
   const int bh = id / nqb;
   const int qb = id - bh * nqb;
-  constexpr int NT = WAVES * 64;  // threads
   const int q_base = qb * (WAVES * 32 * QT) + wave * (32 * QT);
 
   const _Float16* Qg = Q + (size_t)bh * Sq * D;
@@ -79,7 +149,9 @@ __global__ __launch_bounds__(WAVES * 64) void flash_attn_kernel(const _Float16* 
   const _Float16* Vg = V + (size_t)bh * Skv * D;
   _Float16* Og = O + (size_t)bh * Sq * D;
 
-  // ---- Q row fragments, resident for the whole kernel
+  // ---- Q row fragments, resident for the whole kernel, pre-multiplied by
+  // scale*log2(e) (in fp32, rounded once to fp16): scores then come out of the
+  // matrix unit in exponent units and need no scaling instruction per score.
   v8h qf[QT][DS];
 #pragma unroll
   for (int qt = 0; qt < QT; ++qt) {
@@ -87,15 +159,16 @@ __global__ __launch_bounds__(WAVES * 64) void flash_attn_kernel(const _Float16* 
 #pragma unroll
     for (int s = 0; s < DS; ++s) {
       const uint4 v = *reinterpret_cast<const uint4*>(Qg + (size_t)row * D + 16 * s + 8 * hh);
-      qf[qt][s] = *reinterpret_cast<const v8h*>(&v);
+      const v8h q = *reinterpret_cast<const v8h*>(&v);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) qf[qt][s][e] = (_Float16)((float)q[e] * scale_log2e);
     }
   }
 
   v16f oacc[QT][DT];
-  float m_run[QT], l_run[QT];
+  float l_run[QT];
 #pragma unroll
   for (int qt = 0; qt < QT; ++qt) {
-    m_run[qt] = -INFINITY;
     l_run[qt] = 0.0f;
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt)
@@ -103,178 +176,329 @@ __global__ __launch_bounds__(WAVES * 64) void flash_attn_kernel(const _Float16* 
       for (int r = 0; r < 16; ++r) oacc[qt][dt][r] = 0.0f;
   }
 
-  // ---- staging assignments
-  constexpr int KN = FA_KT * (D / 8) / NT;   // 16-byte K loads per thread per tile
-  constexpr int VN = (FA_KT / 4) * (D / 4) / NT;  // 4x4 V blocks per thread per tile
-  static_assert(KN >= 1 && VN >= 1, "tile too small for this many threads");
-  v4u kreg[KN];
-  v2u vreg[VN][4];
-
-  auto load_tile = [&](int kt) __attribute__((always_inline)) {
-    const int key0 = kt * FA_KT;
-    static_for<KN>([&](auto nc) __attribute__((always_inline)) {
-      constexpr int n = decltype(nc)::value;
-      const int idx = tid + NT * n;
-      const int key = min(key0 + idx / (D / 8), Skv - 1);
-      const int c8 = idx % (D / 8);
-      kreg[n] = *reinterpret_cast<const v4u*>(Kg + (size_t)key * D + 8 * c8);
-    });
-    static_for<VN * 4>([&](auto nc) __attribute__((always_inline)) {
-      constexpr int n = decltype(nc)::value / 4;
-      constexpr int nn = decltype(nc)::value % 4;
-      const int u = tid + NT * n;
-      const int dg = u % (D / 4);
-      const int kq = u / (D / 4);
-      const int key = min(key0 + 4 * kq + nn, Skv - 1);
-      vreg[n][nn] = *reinterpret_cast<const v2u*>(Vg + (size_t)key * D + 4 * dg);
-    });
-  };
-  auto store_tile = [&](int buf) __attribute__((always_inline)) {
-    _Float16* ks = Ks + buf * KSZ;
-    _Float16* vt = Vt + buf * VSZ;
-    static_for<KN>([&](auto nc) __attribute__((always_inline)) {
-      constexpr int n = decltype(nc)::value;
-      const int idx = tid + NT * n;
-      const int key = idx / (D / 8);
-      const int c8 = idx % (D / 8);
-      *reinterpret_cast<v4u*>(ks + key * KLD + 8 * c8) = kreg[n];
-    });
-    static_for<VN>([&](auto nc) __attribute__((always_inline)) {
-      constexpr int n = decltype(nc)::value;
-      const int u = tid + NT * n;
-      const int dg = u % (D / 4);
-      const int kq = u / (D / 4);
-      const v2u r0 = vreg[n][0], r1 = vreg[n][1], r2 = vreg[n][2], r3 = vreg[n][3];
-      // 4x4 transpose of halfs: row e of the result = element e of keys 0..3
-      v2u c0, c1, c2, c3;
-      c0.x = __builtin_amdgcn_perm(r1.x, r0.x, 0x05040100u);
-      c0.y = __builtin_amdgcn_perm(r3.x, r2.x, 0x05040100u);
-      c1.x = __builtin_amdgcn_perm(r1.x, r0.x, 0x07060302u);
-      c1.y = __builtin_amdgcn_perm(r3.x, r2.x, 0x07060302u);
-      c2.x = __builtin_amdgcn_perm(r1.y, r0.y, 0x05040100u);
-      c2.y = __builtin_amdgcn_perm(r3.y, r2.y, 0x05040100u);
-      c3.x = __builtin_amdgcn_perm(r1.y, r0.y, 0x07060302u);
-      c3.y = __builtin_amdgcn_perm(r3.y, r2.y, 0x07060302u);
-      _Float16* dst = vt + (4 * dg) * FA_VLD + 4 * kq;
-      *reinterpret_cast<v2u*>(dst) = c0;
-      *reinterpret_cast<v2u*>(dst + FA_VLD) = c1;
-      *reinterpret_cast<v2u*>(dst + 2 * FA_VLD) = c2;
-      *reinterpret_cast<v2u*>(dst + 3 * FA_VLD) = c3;
-    });
-  };
-
-  const int ntiles = (Skv + FA_KT - 1) / FA_KT;
-  const float tau_raw = FA_TAU / scale_log2e;
-  load_tile(0);
-  store_tile(0);
-  __syncthreads();
-
-  auto process_tile = [&](int kt, auto ragged_c) __attribute__((always_inline)) {
-    constexpr bool ragged = decltype(ragged_c)::value;
-    const int buf = kt & 1;
-    if (kt + 1 < ntiles) load_tile(kt + 1);
-    const _Float16* ks = Ks + buf * KSZ;
-    const _Float16* vt = Vt + buf * VSZ;
-
-    // ---- S^T = K Q^T for two 32-key subtiles
-    v16f sacc[QT][2];
+  // ---- copies: copy c of a tile fills LDS bytes [1024c, 1024c + 1024) of the
+  // padded tile, lane l the 16 bytes at 1024c + 16l; slots in the padding
+  // fetch the row's first chunk (never read).  Wave w issues copies w, w+WAVES, ...
+  unsigned k_src[KCP], v_src[VCP];  // byte offset of this lane's chunk within the tile in global memory
 #pragma unroll
-    for (int qt = 0; qt < QT; ++qt)
+  for (int i = 0; i < KCP; ++i) {
+    const int x = 1024 * (wave + WAVES * i) + 16 * lane;
+    const int row = min(x / KRS, FA_KT - 1), col = x % KRS;
+    k_src[i] = row * RB + (col < RB ? col : 0);
+  }
 #pragma unroll
-      for (int k2 = 0; k2 < 2; ++k2)
-#pragma unroll
-        for (int r = 0; r < 16; ++r) sacc[qt][k2][r] = 0.0f;
-#pragma unroll
-    for (int k2 = 0; k2 < 2; ++k2) {
-      const _Float16* krow = ks + (32 * k2 + j) * KLD + 8 * hh;
-#pragma unroll
-      for (int s = 0; s < DS; ++s) {
-        const v8h kf = *reinterpret_cast<const v8h*>(krow + 16 * s);
-#pragma unroll
-        for (int qt = 0; qt < QT; ++qt)
-          sacc[qt][k2] = __builtin_amdgcn_mfma_f32_32x32x16_f16(kf, qf[qt][s], sacc[qt][k2], 0, 0, 0);
+  for (int i = 0; i < VCP; ++i) {
+    const int x = 1024 * (wave + WAVES * i) + 16 * lane;
+    const int row = min(x / VRS, FA_KT - 1), col = x % VRS;
+    v_src[i] = row * RB + (col < RB ? col : 0);
+  }
+  // copy i (of this wave's share) of K tile kt into the K buffer at dst; no-op past the wave's last copy
+  auto copy_k = [&](unsigned char* dst, int kt, auto i_c) __attribute__((always_inline)) {
+    constexpr int i = decltype(i_c)::value;
+    if constexpr (i < KCP) {
+      if (wave + WAVES * i < KTB / 1024) {
+        const int key0 = kt * FA_KT;
+        unsigned off = k_src[i];
+        if (key0 + FA_KT > Skv) {  // ragged last tile: rows past the end re-read the last key (their scores are masked)
+          const unsigned last = (unsigned)(Skv - 1 - key0), row = off / RB;
+          if (row > last) off -= (row - last) * RB;
+        }
+        lds_dma16(Kg + (size_t)key0 * D, off, dst + 1024 * (wave + WAVES * i));
       }
     }
+  };
+  auto copy_v = [&](unsigned char* dst, int kt, auto i_c) __attribute__((always_inline)) {
+    constexpr int i = decltype(i_c)::value;
+    if constexpr (i < VCP) {
+      if (wave + WAVES * i < VTB / 1024) {
+        const int key0 = kt * FA_KT;
+        unsigned off = v_src[i];
+        if (key0 + FA_KT > Skv) {
+          const unsigned last = (unsigned)(Skv - 1 - key0), row = off / RB;
+          if (row > last) off -= (row - last) * RB;
+        }
+        lds_dma16(Vg + (size_t)key0 * D, off, dst + 1024 * (wave + WAVES * i));
+      }
+    }
+  };
+  auto copy_k_all = [&](unsigned char* dst, int kt) __attribute__((always_inline)) {
+    static_for<KCP>([&](auto i_c) __attribute__((always_inline)) { copy_k(dst, kt, i_c); });
+  };
+  auto copy_v_all = [&](unsigned char* dst, int kt) __attribute__((always_inline)) {
+    static_for<VCP>([&](auto i_c) __attribute__((always_inline)) { copy_v(dst, kt, i_c); });
+  };
+  auto stamp = [&](int kt, int slot) __attribute__((always_inline)) {
+    if constexpr (TRACE) {
+      if (blockIdx.x == 0 && tid == 64 * trace_wave && kt < FA_TRACE_TILES) trace[kt * 6 + slot] = wall_clock64();
+    }
+  };
+  auto copies_landed = [&](int kt) __attribute__((always_inline)) {
+    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
+    stamp(kt, 5);
+    __syncthreads();
+  };
 
-    // ---- online softmax, one query row per lane (two lanes share a row).
-    // Scores stay in raw units; p = exp2(s*c - m_ref*c) with c = scale*log2(e)
-    // is one fused multiply-add and one exponential per score.  m_ref is a
-    // reference maximum that is only moved (and O, l rescaled) when the true
-    // row maximum has run ahead of it by more than FA_TAU in exponent units:
-    // any m_ref gives the same O = acc/l, p merely ranges up to 2^FA_TAU.
-    v8h pf[QT][2][2];
+  // ---- fragment addresses: one lane-dependent base per tile kind, everything
+  // else (half tile, contraction step, d tile) is an immediate offset.
+  // K: lane (j, hh) reads row 32*k2 + j, bytes [32s + 16hh, +16)
+  const int k_lane = j * KRS + 16 * hh;
+  // V: lane hands in (key a = (lane&15)>>2, column chunk b = lane&3) of the 16-column block
+  // dhalf = (lane>>4)&1 of d tile dt, keys 4*hh + a (+ constant) of the step
+  const int v_lane = (4 * hh + ((lane & 15) >> 2)) * VRS + 32 * ((lane >> 4) & 1) + 8 * (lane & 3);
+
+  const int ntiles = (Skv + FA_KT - 1) / FA_KT;
+  const bool has_ragged = (Skv % FA_KT) != 0;
+
+  using lds_v4s = __attribute__((address_space(3))) v4s;
+  typedef short v8s __attribute__((ext_vector_type(8)));
+  // kbase / vbase: LDS address of the half tile plus the lane's base
+  auto read_k = [&](const unsigned char* kbase, int s) __attribute__((always_inline)) {
+    return *reinterpret_cast<const v8h*>(kbase + 32 * s);
+  };
+  // A-operand of the PV product for (step s, d tile dt) of one half tile
+  auto read_v = [&](const unsigned char* vbase, int s, int dt) __attribute__((always_inline)) {
+    const unsigned char* p0 = vbase + 16 * s * VRS + 64 * dt;
+    const v4s lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4s*)(p0));
+    const v4s hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4s*)(p0 + 8 * VRS));
+    const v8s both = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+    return __builtin_bit_cast(v8h, both);
+  };
+
+  // Scores are kept relative to a per-row reference maximum m_ref, and the
+  // subtraction is free: every score chain starts its accumulator from nref =
+  // -m_ref (a 16-register vector, one query per lane) instead of zero, so the
+  // matrix unit hands back s - m_ref and p = exp2(s - m_ref) is a single
+  // exponential.  m_ref only moves (and O, l are rescaled) when a row maximum
+  // has run ahead of it by more than FA_TAU: any m_ref gives the same O =
+  // acc/l, p merely ranges up to 2^FA_TAU.  The move happens between half
+  // tiles, after everything computed with the old reference has been
+  // accumulated, and also shifts the one score vector already computed against
+  // the old reference.  A fully masked half has maximum -inf, never moves the
+  // reference and exponentiates to zeros.
+  v16f nref[QT];
+  auto move_reference = [&](const float (&mx)[QT], v16f (&sn)[QT]) __attribute__((always_inline)) {
 #pragma unroll
     for (int qt = 0; qt < QT; ++qt) {
-      if constexpr (ragged) {
-#pragma unroll
-        for (int k2 = 0; k2 < 2; ++k2)
-#pragma unroll
-          for (int r = 0; r < 16; ++r) {
-            const int key = kt * FA_KT + 32 * k2 + 8 * (r >> 2) + 4 * hh + (r & 3);
-            if (key >= Skv) sacc[qt][k2][r] = -INFINITY;
-          }
-      }
-      float mx = sacc[qt][0][0];
-#pragma unroll
-      for (int k2 = 0; k2 < 2; ++k2)
-#pragma unroll
-        for (int r = 0; r < 16; ++r) mx = fmaxf(mx, sacc[qt][k2][r]);
-      mx = fmaxf(mx, __shfl_xor(mx, 32));
-      const bool need = mx > m_run[qt] + tau_raw;
+      const bool need = mx[qt] > FA_TAU;
       if (__builtin_amdgcn_ballot_w64(need) != 0) {
-        const float m_new = need ? mx : m_run[qt];
-        const float alpha = __builtin_amdgcn_exp2f((m_run[qt] - m_new) * scale_log2e);
-        m_run[qt] = m_new;
+        const float delta = need ? -mx[qt] : 0.0f;  // new scores = old scores + delta
+        const float alpha = __builtin_amdgcn_exp2f(delta);
         l_run[qt] *= alpha;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          nref[qt][r] += delta;
+          sn[qt][r] += delta;
+        }
 #pragma unroll
         for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
           for (int r = 0; r < 16; ++r) oacc[qt][dt][r] *= alpha;
       }
-      const float mc = -m_run[qt] * scale_log2e;
-      float psum = 0.0f;
-#pragma unroll
-      for (int k2 = 0; k2 < 2; ++k2)
-#pragma unroll
-        for (int s = 0; s < 2; ++s)
-#pragma unroll
-          for (int e = 0; e < 8; e += 2) {
-            const float p0 = __builtin_amdgcn_exp2f(__builtin_fmaf(sacc[qt][k2][8 * s + e], scale_log2e, mc));
-            const float p1 = __builtin_amdgcn_exp2f(__builtin_fmaf(sacc[qt][k2][8 * s + e + 1], scale_log2e, mc));
-            const v2h pp = {(_Float16)p0, (_Float16)p1};
-            pf[qt][k2][s][e] = pp[0];
-            pf[qt][k2][s][e + 1] = pp[1];
-            // row sum over the rounded values that enter the PV product, two per instruction
-            psum = __builtin_amdgcn_fdot2(pp, v2h{(_Float16)1.0f, (_Float16)1.0f}, psum, false);
-          }
-      l_run[qt] += psum;  // this lane's half of the row sum
     }
-
-    // ---- O^T += V^T P^T
-#pragma unroll
-    for (int dt = 0; dt < DT; ++dt) {
-      const _Float16* vrow = vt + (32 * dt + j) * FA_VLD + 4 * hh;
-#pragma unroll
-      for (int k2 = 0; k2 < 2; ++k2)
-#pragma unroll
-        for (int s = 0; s < 2; ++s) {
-          const v4h v0 = *reinterpret_cast<const v4h*>(vrow + 32 * k2 + 16 * s);
-          const v4h v1 = *reinterpret_cast<const v4h*>(vrow + 32 * k2 + 16 * s + 8);
-          const v8h vf = {v0[0], v0[1], v0[2], v0[3], v1[0], v1[1], v1[2], v1[3]};
-#pragma unroll
-          for (int qt = 0; qt < QT; ++qt)
-            oacc[qt][dt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(vf, pf[qt][k2][s], oacc[qt][dt], 0, 0, 0);
-        }
-    }
-
-    if (kt + 1 < ntiles) store_tile(buf ^ 1);
-    __syncthreads();
   };
 
-  const bool has_ragged = (Skv % FA_KT) != 0;
-  const int nfull = has_ragged ? ntiles - 1 : ntiles;
-  for (int kt = 0; kt < nfull; ++kt) process_tile(kt, std::false_type{});
-  if (has_ragged) process_tile(ntiles - 1, std::true_type{});
+  // p = exp2(score e) of a half tile; pairs are packed to fp16 in the order
+  // the PV product contracts them.  The row sum adds the unrounded values with
+  // plain fp32 adds: dot-product instructions would halve the work but run on
+  // the matrix pipeline and stall the MFMAs.
+  float psum[QT], held[QT];
+  auto exp_element = [&](const v16f (&sc)[QT], v8h (&pf)[QT][2], auto e_c) __attribute__((always_inline)) {
+    constexpr int e = decltype(e_c)::value;
+#pragma unroll
+    for (int qt = 0; qt < QT; ++qt) {
+      const float p = __builtin_amdgcn_exp2f(sc[qt][e]);
+      psum[qt] += p;
+      if constexpr ((e & 1) == 0) {
+        held[qt] = p;
+      } else {
+        const v2h pp = {(_Float16)held[qt], (_Float16)p};
+        pf[qt][e / 8][(e % 8) - 1] = pp[0];
+        pf[qt][e / 8][e % 8] = pp[1];
+      }
+    }
+  };
+
+  // The loop is software pipelined per 32-key half tile in two kinds of
+  // blocks, written in the instruction order they should issue in and fenced
+  // step by step so that the order survives.  Vector instructions do not hide
+  // behind matrix instructions on this machine (each costs issue time), so the
+  // blocks are built to need few of them:
+  //   E: DS steps of { QT score MFMAs of the NEXT half | one fragment read
+  //      three steps ahead | exponentiate a few scores of THIS half }
+  //   A: 2*DT steps of { QT MFMAs of P V of THIS half | one fragment read |
+  //      first the remaining exponentials, then row maxima of the NEXT half's
+  //      scores }, then move the reference maximum if needed.
+  // NE of the 16 scores a lane holds per query are exponentiated in E, the
+  // rest in the first DT steps of A (they belong to the second contraction
+  // step of P V, which starts at step DT).  Fragment reads run three steps
+  // ahead throughout, across block boundaries: the last three steps of a block
+  // read the first three fragments of the next one (kpre / vpre).
+  constexpr int NE = 12;
+  constexpr int NS = 2 * DT;
+  v8h kpre[3], vpre[3];
+  auto block_e = [&](const unsigned char* kbase, const unsigned char* vbase, const v16f (&sc)[QT], v8h (&pf)[QT][2],
+                     v16f (&sn)[QT], auto next_c) __attribute__((always_inline)) {
+    constexpr bool has_next = decltype(next_c)::value;
+#pragma unroll
+    for (int qt = 0; qt < QT; ++qt) psum[qt] = 0.0f;
+    v8h kf[DS];
+    kf[0] = kpre[0];
+    kf[1] = kpre[1];
+    kf[2] = kpre[2];
+    __builtin_amdgcn_sched_barrier(0);
+    static_for<DS>([&](auto s_c) __attribute__((always_inline)) {
+      constexpr int s = decltype(s_c)::value;
+      if constexpr (has_next) {
+#pragma unroll
+        for (int qt = 0; qt < QT; ++qt)
+          sn[qt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(kf[s], qf[qt][s], s == 0 ? nref[qt] : sn[qt], 0, 0, 0);
+        if constexpr (s + 3 < DS) kf[s + 3] = read_k(kbase, s + 3);
+      }
+      if constexpr (s + 3 >= DS) vpre[s + 3 - DS] = read_v(vbase, (s + 3 - DS) / DT, (s + 3 - DS) % DT);
+      // scores [s*NE/DS, (s+1)*NE/DS)
+      static_for<((s + 1) * NE) / DS - (s * NE) / DS>([&](auto i_c) __attribute__((always_inline)) {
+        exp_element(sc, pf, std::integral_constant<int, (s * NE) / DS + decltype(i_c)::value>{});
+      });
+      __builtin_amdgcn_sched_barrier(0);
+    });
+  };
+  // knext: base of the K half tile whose scores the following E block computes (ignored without one)
+  auto block_a = [&](const unsigned char* vbase, const unsigned char* knext, const v16f (&sc)[QT], v8h (&pf)[QT][2],
+                     v16f (&sn)[QT], int key_next, auto next_c, auto mask_c, auto prek_c) __attribute__((always_inline)) {
+    constexpr bool has_next = decltype(next_c)::value;
+    constexpr bool mask = decltype(mask_c)::value;
+    constexpr bool prefetch_k = decltype(prek_c)::value;
+    v8h vf[NS];
+    vf[0] = vpre[0];
+    vf[1] = vpre[1];
+    vf[2] = vpre[2];
+    float mx[QT];
+    __builtin_amdgcn_sched_barrier(0);
+    static_for<NS>([&](auto i_c) __attribute__((always_inline)) {
+      constexpr int i = decltype(i_c)::value;
+      constexpr int s = i / DT, dt = i % DT;
+#pragma unroll
+      for (int qt = 0; qt < QT; ++qt)
+        oacc[qt][dt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(vf[i], pf[qt][s], oacc[qt][dt], 0, 0, 0);
+      if constexpr (i + 3 < NS) {
+        vf[i + 3] = read_v(vbase, (i + 3) / DT, (i + 3) % DT);
+      } else if constexpr (prefetch_k) {
+        kpre[i + 3 - NS] = read_k(knext, i + 3 - NS);
+      }
+      if constexpr (i < DT) {
+        // remaining scores [NE + i*(16-NE)/DT, NE + (i+1)*(16-NE)/DT)
+        constexpr int R = 16 - NE;
+        static_for<((i + 1) * R) / DT - (i * R) / DT>([&](auto j_c) __attribute__((always_inline)) {
+          exp_element(sc, pf, std::integral_constant<int, NE + (i * R) / DT + decltype(j_c)::value>{});
+        });
+        if constexpr (i == DT - 1) {
+#pragma unroll
+          for (int qt = 0; qt < QT; ++qt) l_run[qt] += psum[qt];  // this lane's half of the row sum
+        }
+      } else if constexpr (has_next) {
+        // row maxima of the next half's scores [(i-DT)*16/DT, (i-DT+1)*16/DT)
+        constexpr int e0 = ((i - DT) * 16) / DT, e1 = ((i - DT + 1) * 16) / DT;
+#pragma unroll
+        for (int qt = 0; qt < QT; ++qt) {
+          if constexpr (mask) {
+#pragma unroll
+            for (int r = e0; r < e1; ++r)
+              if (key_next + 8 * (r >> 2) + 4 * hh + (r & 3) >= Skv) sn[qt][r] = -INFINITY;
+          }
+          float m = i == DT ? sn[qt][e0] : mx[qt];
+#pragma unroll
+          for (int r = e0; r < e1; ++r) m = fmaxf(m, sn[qt][r]);
+          mx[qt] = m;
+        }
+      }
+      __builtin_amdgcn_sched_barrier(0);
+    });
+    if constexpr (has_next) {
+#pragma unroll
+      for (int qt = 0; qt < QT; ++qt) mx[qt] = max_with_other_half(mx[qt]);
+      move_reference(mx, sn);
+    }
+  };
+
+  // K buffers rotate through (current, next, free), V buffers alternate
+  int kcur = 0, knext = KTB, kfree = 2 * KTB;
+  int vcur = 0, vnext = VTB;
+
+  // ---- prologue: tiles 0 (K, V) and 1 (K) into LDS; scores of tile 0's first
+  // half from a zero start, their row maximum becomes the first reference
+  v16f sa[QT], sb[QT];
+  v8h pa[QT][2], pb[QT][2];
+  copy_k_all(Kb, 0);
+  copy_v_all(Vb, 0);
+  if (ntiles > 1) copy_k_all(Kb + KTB, 1);
+  copies_landed(FA_TRACE_TILES);
+  {
+    const unsigned char* kbase = Kb + k_lane;
+#pragma unroll
+    for (int qt = 0; qt < QT; ++qt) {
+#pragma unroll
+      for (int r = 0; r < 16; ++r) sa[qt][r] = 0.0f;
+#pragma unroll
+      for (int s = 0; s < DS; ++s)
+        sa[qt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(read_k(kbase, s), qf[qt][s], sa[qt], 0, 0, 0);
+      if (ntiles == 1 && has_ragged) {
+#pragma unroll
+        for (int r = 0; r < 16; ++r)
+          if (8 * (r >> 2) + 4 * hh + (r & 3) >= Skv) sa[qt][r] = -INFINITY;
+      }
+      float m = sa[qt][0];
+#pragma unroll
+      for (int r = 1; r < 16; ++r) m = fmaxf(m, sa[qt][r]);
+      m = max_with_other_half(m);
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        sa[qt][r] -= m;
+        nref[qt][r] = -m;
+      }
+    }
+#pragma unroll
+    for (int i = 0; i < 3; ++i) kpre[i] = read_k(kbase + 32 * KRS, i);
+  }
+
+  // One step = one 64-key tile: E and A for its first half (scores of the
+  // second half computed on the way), E and A for its second half (scores of
+  // tile kt+1's first half, whose K tile was copied one step earlier).  The
+  // copies of K(kt+2) and V(kt+1) go into buffers that every wave finished
+  // with before the barrier that ended the previous step, and are awaited at
+  // the barrier that ends this one.
+  auto step = [&](int kt, auto next_c, auto mask_c) __attribute__((always_inline)) {
+    stamp(kt, 0);
+    if (kt + 2 < ntiles) copy_k_all(Kb + kfree, kt + 2);
+    if (kt + 1 < ntiles) copy_v_all(Vb + vnext, kt + 1);
+    const unsigned char* v0 = Vb + vcur + v_lane;
+    block_e(Kb + kcur + k_lane + 32 * KRS, v0, sa, pa, sb, std::true_type{});
+    stamp(kt, 1);
+    block_a(v0, Kb + knext + k_lane, sa, pa, sb, kt * FA_KT + 32, std::true_type{}, mask_c, next_c);
+    stamp(kt, 2);
+    block_e(Kb + knext + k_lane, v0 + 32 * VRS, sb, pb, sa, next_c);
+    stamp(kt, 3);
+    block_a(v0 + 32 * VRS, Kb + knext + k_lane + 32 * KRS, sb, pb, sa, (kt + 1) * FA_KT, next_c, mask_c, next_c);
+    stamp(kt, 4);
+    copies_landed(kt);
+    int t = kcur;
+    kcur = knext;
+    knext = kfree;
+    kfree = t;
+    t = vcur;
+    vcur = vnext;
+    vnext = t;
+  };
+
+  // Only the two steps that touch the last tile pay for masking its ragged
+  // tail; they are peeled so that the main loop body is one straight line.
+  for (int kt = 0; kt + 2 < ntiles; ++kt) step(kt, std::true_type{}, std::false_type{});
+  if (has_ragged) {
+    if (ntiles > 1) step(ntiles - 2, std::true_type{}, std::true_type{});
+    step(ntiles - 1, std::false_type{}, std::true_type{});
+  } else {
+    if (ntiles > 1) step(ntiles - 2, std::true_type{}, std::false_type{});
+    step(ntiles - 1, std::false_type{}, std::false_type{});
+  }
 
   // ---- normalise and store: lane holds d = 32dt + 8g + 4*half + r of its row
 #pragma unroll
@@ -295,39 +519,73 @@ __global__ __launch_bounds__(WAVES * 64) void flash_attn_kernel(const _Float16* 
   }
 }
 
-template <int D, int QT, int WAVES>
+// FTK_FA_TRACE=1+w turns the per-tile timeline of wave w of workgroup 0 on (read once).
+static int fa_trace_wave() {
+  const char* e = getenv("FTK_FA_TRACE");
+  return e && atoi(e) > 0 ? atoi(e) - 1 : 0;
+}
+// Device address of the stamp buffer, or NULL when tracing is off.
+static long long* fa_trace_ptr() {
+  static int on = -1;
+  static long long* ptr = nullptr;
+  if (on < 0) {
+    const char* e = getenv("FTK_FA_TRACE");
+    on = (e && atoi(e) > 0) ? 1 : 0;
+    if (on && hipGetSymbolAddress((void**)&ptr, HIP_SYMBOL(fa_trace_buf)) != hipSuccess) ptr = nullptr;
+  }
+  return on ? ptr : nullptr;
+}
+
+template <int D, int QT, int WAVES, int MINB>
 static int launch_fa(const void* Q, const void* K, const void* V, void* O, int BH, int Sq, int Skv, float scale,
                      int lds_max, hipStream_t s) {
-  const size_t lds = (size_t)2 * (FA_KT * (D + 8) + D * FA_VLD) * 2;
+  const size_t lds = (size_t)3 * FaLayout<D>::KTB + (size_t)2 * FaLayout<D>::VTB;  // three K tiles, two V tiles
   if ((int)lds > lds_max) return fail(FTK_ERR_UNSUPPORTED_SHAPE, "ftk_flash_attn_f16: needs %zu bytes of LDS", lds);
-  const void* fn = (const void*)flash_attn_kernel<D, QT, WAVES>;
   static bool attr_set = false;
   if (!attr_set) {
-    FTK_HIP(hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+    FTK_HIP(hipFuncSetAttribute((const void*)flash_attn_kernel<D, QT, WAVES, MINB, false>,
+                                hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+    FTK_HIP(hipFuncSetAttribute((const void*)flash_attn_kernel<D, QT, WAVES, MINB, true>,
+                                hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
     attr_set = true;
   }
   constexpr int ROWS = WAVES * 32 * QT;
   const int nqb = (Sq + ROWS - 1) / ROWS;
   const long long total = (long long)nqb * BH;
   if (total > 0x7fffffffLL) return fail(FTK_ERR_UNSUPPORTED_SHAPE, "ftk_flash_attn_f16: grid too large");
-  hipLaunchKernelGGL((flash_attn_kernel<D, QT, WAVES>), dim3((unsigned)total), dim3(WAVES * 64), lds, s,
-                     (const _Float16*)Q, (const _Float16*)K, (const _Float16*)V, (_Float16*)O, Sq, Skv,
-                     scale * 1.4426950408889634f, nqb);
+  long long* trace = fa_trace_ptr();
+  if (trace)
+    hipLaunchKernelGGL((flash_attn_kernel<D, QT, WAVES, MINB, true>), dim3((unsigned)total), dim3(WAVES * 64), lds,
+                       s, (const _Float16*)Q, (const _Float16*)K, (const _Float16*)V, (_Float16*)O, Sq, Skv,
+                       scale * 1.4426950408889634f, nqb, trace, fa_trace_wave());
+  else
+    hipLaunchKernelGGL((flash_attn_kernel<D, QT, WAVES, MINB, false>), dim3((unsigned)total), dim3(WAVES * 64), lds,
+                       s, (const _Float16*)Q, (const _Float16*)K, (const _Float16*)V, (_Float16*)O, Sq, Skv,
+                       scale * 1.4426950408889634f, nqb, trace, fa_trace_wave());
   return check_launch("flash_attn_kernel");
 }
 
-// Tuning hook: FTK_FA_VARIANT=1|2|3 pins the tiling variant (read once).
+// Tuning hook: FTK_FA_VARIANT=1|3 pins the tiling variant (read once).
 static int fa_variant_override() {
   static int v = -1;
   if (v < 0) {
     const char* e = getenv("FTK_FA_VARIANT");
     v = e ? atoi(e) : 0;
-    if (v < 0 || v > 3) v = 0;
+    if (v != 1 && v != 3) v = 0;
   }
   return v;
 }
 
 }  // namespace ftk
+
+extern "C" int ftk_debug_read_fa_trace(long long* host_dst, int n) {
+  using namespace ftk;
+  if (!host_dst || n <= 0 || n > FA_TRACE_TILES * 6)
+    return fail(FTK_ERR_INVALID_ARGUMENT, "ftk_debug_read_fa_trace: need host_dst and 0 < n <= %d", FA_TRACE_TILES * 6);
+  FTK_HIP(hipDeviceSynchronize());
+  FTK_HIP(hipMemcpyFromSymbol(host_dst, HIP_SYMBOL(fa_trace_buf), sizeof(long long) * n));
+  return FTK_OK;
+}
 
 extern "C" int ftk_flash_attn_f16(const void* Q, const void* K, const void* V, void* O, int B, int Hd, int Sq, int Skv,
                                   int D, float scale, ftk_stream_t stream) {
@@ -342,26 +600,18 @@ extern "C" int ftk_flash_attn_f16(const void* Q, const void* K, const void* V, v
   int rc = device_props(&dp);
   if (rc) return rc;
   hipStream_t s = (hipStream_t)stream;
-  // Variant: 0 = choose by problem size, 1 = 4 waves x 32 rows, 2 = 4 waves x 64 rows, 3 = 8 waves x 32 rows.
+  // Variant: 0 = choose by problem size, 1 = 4 waves x 32 query rows, 3 = 8 waves x 32 query rows.
+  // Measured on MI355X (B8 H16 S2048): 8 waves (two per SIMD; K/V tiles shared by 256 rows) 358 us at
+  // D=128 and 203 us at D=64, against 476 / 307 us for 4 waves; for grids that do not fill the chip with
+  // 256-row blocks (B2 H8 S1024) the 128-row blocks win, 29 against 38 us.
   int variant = fa_variant_override();
-  // measured on MI355X at B8 H16 S2048 D128: 8 waves x 32 rows (two waves per SIMD, softmax of one
-  // overlapping the MFMAs of the other) beats 4 waves x 64 rows, which beats 4 waves x 32 rows
-  if (variant == 0) {
-    const bool big = (long long)((Sq + 255) / 256) * bh >= dp->cus;
-    variant = big ? (D == 128 ? 3 : 2) : 1;
-  }
+  if (variant == 0) variant = (long long)((Sq + 255) / 256) * bh >= dp->cus ? 3 : 1;
   const int lds = dp->lds_optin;
   if (D == 128) {
-    switch (variant) {
-      case 1: return launch_fa<128, 1, 4>(Q, K, V, O, (int)bh, Sq, Skv, scale, lds, s);
-      case 3: return launch_fa<128, 1, 8>(Q, K, V, O, (int)bh, Sq, Skv, scale, lds, s);
-      default: return launch_fa<128, 2, 4>(Q, K, V, O, (int)bh, Sq, Skv, scale, lds, s);
-    }
+    if (variant == 1) return launch_fa<128, 1, 4, 1>(Q, K, V, O, (int)bh, Sq, Skv, scale, lds, s);
+    return launch_fa<128, 1, 8, 1>(Q, K, V, O, (int)bh, Sq, Skv, scale, lds, s);
   }
-  switch (variant) {
-    case 1: return launch_fa<64, 1, 4>(Q, K, V, O, (int)bh, Sq, Skv, scale, lds, s);
-    case 3:  // a 64-key tile of 64-wide heads has too little to stage for 8 waves
-    default: return launch_fa<64, 2, 4>(Q, K, V, O, (int)bh, Sq, Skv, scale, lds, s);
-  }
+  if (variant == 1) return launch_fa<64, 1, 4, 1>(Q, K, V, O, (int)bh, Sq, Skv, scale, lds, s);
+  return launch_fa<64, 1, 8, 1>(Q, K, V, O, (int)bh, Sq, Skv, scale, lds, s);
 }
 

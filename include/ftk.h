@@ -171,6 +171,18 @@ int ftk_flash_attn_f16(const void* Q, const void* K, const void* V, void* O,
 int ftk_online_softmax_f32(const float* x, float* y, int rows, int cols,
                            ftk_stream_t stream);
 
+/* ---------------------------------------------------------- diagnostics -- */
+
+/*
+ * With FTK_FA_TRACE=1+w in the environment, wave w of workgroup 0 of every
+ * ftk_flash_attn_f16 launch records six 100 MHz clock stamps per key tile
+ * (tile start; after each of the four pipeline blocks: exponentials | next
+ * scores, P V | row maxima, twice; after its copies have landed).  This copies
+ * the first n stamps to HOST memory (n <= 1536); it synchronises the device.
+ * No counterpart in the reference.
+ */
+int ftk_debug_read_fa_trace(long long* host_dst, int n);
+
 #ifdef __cplusplus
 }
 #endif
