@@ -25,6 +25,8 @@
 // region so global stores are full 16-byte-per-lane row segments.  The grid is
 // one-dimensional and remapped so that the workgroups of one problem share an
 // XCD (and with it the L2 copy of B and C).
+#include <stdlib.h>
+
 #include <algorithm>
 #include <type_traits>
 
@@ -125,44 +127,45 @@ __global__ __launch_bounds__(256) void b2b_gemm_kernel(const _Float16* __restric
   };
   if (pair < row_pairs) fetch_a(pair);
 
-  // ---- stage this problem's Bs[n][k] and Cs[p][n]: loads in batches of four
+  // ---- stage this problem's Bs[n][k] and Cs[p][n].  Eight loads of each per
+  // thread are issued before the first is consumed (the accumulators are not
+  // live yet, so the registers are free): for N = K = 128 and 128 columns that
+  // is all of B and C in one round trip to memory instead of four.
   {
+    constexpr int SB = 8;
     const int nb = N * (K / 8);
-    for (int base = 0; base < nb; base += 4 * threads) {
-      v4u v[4];
+    const int n8s = N / 8;
+    const int ncq = pw * n8s;
+    for (int base = 0; base < max(nb, ncq); base += SB * threads) {
+      v4u vb[SB], vc[SB];
 #pragma unroll
-      for (int u = 0; u < 4; ++u) {
+      for (int u = 0; u < SB; ++u) {
         const int idx = base + u * threads + tid;
-        if (idx < nb) v[u] = ldg16(Bg + (size_t)idx * 8);
+        if (idx < nb) vb[u] = ldg16(Bg + (size_t)idx * 8);
       }
 #pragma unroll
-      for (int u = 0; u < 4; ++u) {
+      for (int u = 0; u < SB; ++u) {
+        const int idx = base + u * threads + tid;
+        if (idx < ncq) vc[u] = ldg16(Cg + (size_t)idx * 8);
+      }
+#pragma unroll
+      for (int u = 0; u < SB; ++u) {
         const int idx = base + u * threads + tid;
         if (idx < nb) {
           const int n = idx / (K / 8);
           const int k8 = idx - n * (K / 8);
-          *reinterpret_cast<v4u*>(Bs + n * BLD + 8 * k8) = v[u];
+          *reinterpret_cast<v4u*>(Bs + n * BLD + 8 * k8) = vb[u];
         }
       }
-    }
-    const int n8s = N / 8;
-    const int ncq = pw * n8s;
-    for (int base = 0; base < ncq; base += 4 * threads) {
-      v4u v[4];
 #pragma unroll
-      for (int u = 0; u < 4; ++u) {
-        const int idx = base + u * threads + tid;
-        if (idx < ncq) v[u] = ldg16(Cg + (size_t)idx * 8);
-      }
-#pragma unroll
-      for (int u = 0; u < 4; ++u) {
+      for (int u = 0; u < SB; ++u) {
         const int idx = base + u * threads + tid;
         if (idx < ncq) {
           const int p = idx / n8s;
           const int n8 = idx - p * n8s;
           // CLD is not a multiple of 8 halfs: two 8-byte pieces
-          *reinterpret_cast<v2u*>(Cs + p * CLD + 8 * n8) = v2u{v[u][0], v[u][1]};
-          *reinterpret_cast<v2u*>(Cs + p * CLD + 8 * n8 + 4) = v2u{v[u][2], v[u][3]};
+          *reinterpret_cast<v2u*>(Cs + p * CLD + 8 * n8) = v2u{vc[u][0], vc[u][1]};
+          *reinterpret_cast<v2u*>(Cs + p * CLD + 8 * n8 + 4) = v2u{vc[u][2], vc[u][3]};
         }
       }
     }
@@ -257,6 +260,231 @@ __global__ __launch_bounds__(256) void b2b_gemm_kernel(const _Float16* __restric
   }
 }
 
+// Eight-wave form of the same computation for the common shapes (N = 32*NT up
+// to 128, all of B and C resident): every wave takes one 64-row group at a
+// time, two waves share a SIMD, and the work is ordered so that it fits their
+// 256 registers each -- GEMM1 runs to completion first and leaves P for the 64
+// rows as fp16 B-operands in registers (64 of them at N = 128), then GEMM2 runs
+// over the D columns in groups of 64 with its own 64 accumulator registers and
+// stores each group as it finishes.  With all A loads of the workgroup issued
+// at the start and two waves per SIMD, one wave's LDS round trips, conversions
+// and D stores are covered by the other's MFMAs.  The wave-private LDS region
+// is used twice: A rows on the way in, D rows on the way out.
+template <int KS, int PT, int NT>
+__global__ __launch_bounds__(512) void b2b_gemm8_kernel(const _Float16* __restrict__ A,
+                                                        const _Float16* __restrict__ Bm,
+                                                        const _Float16* __restrict__ Cm, _Float16* __restrict__ D,
+                                                        int M, int P, int p_base, B2BGrid gr) {
+  constexpr int K = 16 * KS;
+  constexpr int N = 32 * NT;
+  constexpr int BLD = K + 8;   // padded Bs / A-staging row (halfs)
+  constexpr int CLD = N + 4;   // padded Cs row (halfs)
+  constexpr int AN = 2 * KS;   // 16-byte A loads per lane for 64 rows
+  constexpr int pw = 32 * PT;  // p columns handled here
+  constexpr int PG = (PT + 1) / 2;  // column groups of up to 64
+  constexpr int DLD = 64 + 4;  // padded D staging row (halfs)
+  constexpr int threads = 512;
+  constexpr int waves = 8;
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = tid >> 6;
+  const int j = lane & 31;
+  const int hh = lane >> 5;
+
+  int id = blockIdx.x;
+  if ((gr.total & 7) == 0) id = (blockIdx.x & 7) * (gr.total >> 3) + (blockIdx.x >> 3);
+  const int part = id % gr.per_problem;
+  const int pt_idx = (id / gr.per_problem) % gr.ptiles;
+  const int g = id / (gr.per_problem * gr.ptiles);
+  const int p0 = p_base + pt_idx * pw;
+
+  _Float16* Bs = reinterpret_cast<_Float16*>(smem);        // [N][BLD]
+  _Float16* Cs = Bs + N * BLD;                             // [pw][CLD]
+  _Float16* Wr = Cs + pw * CLD + wave * gr.wave_region;    // wave-private: [32][BLD] A rows, then [32][DLD] D rows
+
+  const _Float16* Ag = A + (size_t)g * M * K;
+  const _Float16* Bg = Bm + (size_t)g * N * K;
+  const _Float16* Cg = Cm + (size_t)g * P * N + (size_t)p0 * N;
+  _Float16* Dg = D + (size_t)g * M * P + p0;
+
+  const int row_pairs = (M + 63) / 64;
+  const int wave_stride = gr.per_problem * waves;
+  int pair = part * waves + wave;
+
+  constexpr int CPR = K / 8;  // 16-byte chunks per row
+  v4u areg[AN];
+  auto fetch_a = [&](int pr_) __attribute__((always_inline)) {
+    static_for<AN>([&](auto uc) __attribute__((always_inline)) {
+      constexpr int u = decltype(uc)::value;
+      const int chunk = u * 64 + lane;
+      const int row = min(pr_ * 64 + chunk / CPR, M - 1);
+      areg[u] = ldg16(Ag + (size_t)row * K + 8 * (chunk % CPR));
+    });
+  };
+  if (pair < row_pairs) fetch_a(pair);
+
+  // ---- stage Bs[n][k] and Cs[p][n], all loads of a thread in flight together
+  {
+    constexpr int nb = N * (K / 8), ncq = pw * (N / 8);
+    constexpr int UB = (nb + threads - 1) / threads, UC = (ncq + threads - 1) / threads;
+    v4u vb[UB], vc[UC];
+#pragma unroll
+    for (int u = 0; u < UB; ++u) {
+      const int idx = u * threads + tid;
+      if (idx < nb) vb[u] = ldg16(Bg + (size_t)idx * 8);
+    }
+#pragma unroll
+    for (int u = 0; u < UC; ++u) {
+      const int idx = u * threads + tid;
+      if (idx < ncq) vc[u] = ldg16(Cg + (size_t)idx * 8);
+    }
+#pragma unroll
+    for (int u = 0; u < UB; ++u) {
+      const int idx = u * threads + tid;
+      if (idx < nb) *reinterpret_cast<v4u*>(Bs + (idx / CPR) * BLD + 8 * (idx % CPR)) = vb[u];
+    }
+#pragma unroll
+    for (int u = 0; u < UC; ++u) {
+      const int idx = u * threads + tid;
+      if (idx < ncq) {
+        const int p = idx / (N / 8), n8 = idx % (N / 8);
+        // CLD is not a multiple of 8 halfs: two 8-byte pieces
+        *reinterpret_cast<v2u*>(Cs + p * CLD + 8 * n8) = v2u{vc[u][0], vc[u][1]};
+        *reinterpret_cast<v2u*>(Cs + p * CLD + 8 * n8 + 4) = v2u{vc[u][2], vc[u][3]};
+      }
+    }
+  }
+  __syncthreads();
+
+  for (; pair < row_pairs; pair += wave_stride) {
+    // ---- A rows: park 32 at a time in the wave's region and pull the MFMA
+    // fragments; step s contracts k in [8s, 8s+8) (lanes 0-31) and
+    // [K/2 + 8s, K/2 + 8s + 8) (lanes 32-63)
+    v8h afrag[2][KS];
+    static_for<2>([&](auto rtc) __attribute__((always_inline)) {
+      constexpr int rt = decltype(rtc)::value;
+      static_for<AN / 2>([&](auto uc) __attribute__((always_inline)) {
+        constexpr int u = decltype(uc)::value;
+        const int chunk = u * 64 + lane;
+        *reinterpret_cast<v4u*>(Wr + (chunk / CPR) * BLD + 8 * (chunk % CPR)) = areg[rt * (AN / 2) + u];
+      });
+#pragma unroll
+      for (int s = 0; s < KS; ++s) afrag[rt][s] = *reinterpret_cast<const v8h*>(Wr + j * BLD + hh * (K / 2) + 8 * s);
+    });
+
+    // ---- GEMM1 for every n tile: P^T tiles [32 n, 32 rows] of both row tiles, rounded to fp16
+    v8h pf[2][NT][2];
+    static_for<NT>([&](auto ntc) __attribute__((always_inline)) {
+      constexpr int nt = decltype(ntc)::value;
+      v16f pacc[2];
+#pragma unroll
+      for (int rt = 0; rt < 2; ++rt)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) pacc[rt][r] = 0.0f;
+      const _Float16* brow = Bs + (nt * 32 + j) * BLD + hh * (K / 2);
+#pragma unroll
+      for (int s = 0; s < KS; ++s) {
+        const v8h bfrag = *reinterpret_cast<const v8h*>(brow + 8 * s);
+        pacc[0] = __builtin_amdgcn_mfma_f32_32x32x16_f16(bfrag, afrag[0][s], pacc[0], 0, 0, 0);
+        pacc[1] = __builtin_amdgcn_mfma_f32_32x32x16_f16(bfrag, afrag[1][s], pacc[1], 0, 0, 0);
+      }
+#pragma unroll
+      for (int rt = 0; rt < 2; ++rt)
+#pragma unroll
+        for (int s = 0; s < 2; ++s)
+#pragma unroll
+          for (int e = 0; e < 8; ++e) pf[rt][nt][s][e] = (_Float16)pacc[rt][8 * s + e];
+    });
+    // ---- GEMM2 and store, 64 columns of D at a time
+    static_for<PG>([&](auto pgc) __attribute__((always_inline)) {
+      constexpr int pg = decltype(pgc)::value;
+      constexpr int PW = (PT - 2 * pg) >= 2 ? 2 : 1;  // p tiles in this group
+      v16f dacc[2][PW];
+#pragma unroll
+      for (int rt = 0; rt < 2; ++rt)
+#pragma unroll
+        for (int q = 0; q < PW; ++q)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) dacc[rt][q][r] = 0.0f;
+      static_for<NT>([&](auto ntc) __attribute__((always_inline)) {
+        constexpr int nt = decltype(ntc)::value;
+#pragma unroll
+        for (int q = 0; q < PW; ++q) {
+          const _Float16* crow = Cs + ((2 * pg + q) * 32 + j) * CLD + nt * 32 + 4 * hh;
+#pragma unroll
+          for (int s = 0; s < 2; ++s) {
+            const v4h c0 = *reinterpret_cast<const v4h*>(crow + 16 * s);
+            const v4h c1 = *reinterpret_cast<const v4h*>(crow + 16 * s + 8);
+            const v8h cfrag = {c0[0], c0[1], c0[2], c0[3], c1[0], c1[1], c1[2], c1[3]};
+            dacc[0][q] = __builtin_amdgcn_mfma_f32_32x32x16_f16(cfrag, pf[0][nt][s], dacc[0][q], 0, 0, 0);
+            dacc[1][q] = __builtin_amdgcn_mfma_f32_32x32x16_f16(cfrag, pf[1][nt][s], dacc[1][q], 0, 0, 0);
+          }
+        }
+      });
+      // D^T accumulators -> wave-private LDS [row][p] -> 16-byte row segments.
+      // A wave reads back only what it wrote itself and LDS operations of one
+      // wave complete in order, so no barrier is needed.
+#pragma unroll
+      for (int rt = 0; rt < 2; ++rt) {
+#pragma unroll
+        for (int q = 0; q < PW; ++q)
+#pragma unroll
+          for (int gq = 0; gq < 4; ++gq) {
+            const v4h o = {(_Float16)dacc[rt][q][4 * gq + 0], (_Float16)dacc[rt][q][4 * gq + 1],
+                           (_Float16)dacc[rt][q][4 * gq + 2], (_Float16)dacc[rt][q][4 * gq + 3]};
+            *reinterpret_cast<v4h*>(Wr + j * DLD + q * 32 + 8 * gq + 4 * hh) = o;
+          }
+        constexpr int segs = PW * 4;  // 16-byte segments per row
+#pragma unroll
+        for (int idx = lane; idx < 32 * segs; idx += 64) {
+          const int r = idx / segs;
+          const int sg = idx - r * segs;
+          const int grow = pair * 64 + 32 * rt + r;
+          if (grow < M) {
+            const v2u lo = *reinterpret_cast<const v2u*>(Wr + r * DLD + 8 * sg);
+            const v2u hi = *reinterpret_cast<const v2u*>(Wr + r * DLD + 8 * sg + 4);
+            *reinterpret_cast<v4u*>(Dg + (size_t)grow * P + 64 * pg + 8 * sg) = v4u{lo[0], lo[1], hi[0], hi[1]};
+          }
+        }
+      }
+    });
+    // a further row group of this wave is fetched only now: its registers are not free earlier, and
+    // the other wave on the SIMD keeps the matrix unit busy meanwhile
+    if (pair + wave_stride < row_pairs) fetch_a(pair + wave_stride);
+  }
+}
+
+template <int KS, int PT, int NT>
+static int launch_b2b8(const void* A, const void* B, const void* C, void* D, int G, int M, int P, int p_base,
+                       int ptiles, int cus, int lds_max, bool* handled, hipStream_t s) {
+  constexpr int K = 16 * KS, N = 32 * NT, pw = 32 * PT, waves = 8;
+  B2BGrid gr;
+  gr.ptiles = ptiles;
+  gr.wave_region = std::max(32 * (K + 8), 32 * (64 + 4));
+  const size_t lds = (size_t)(N * (K + 8) + pw * (N + 4) + waves * gr.wave_region) * 2;
+  *handled = (int)lds <= lds_max;
+  if (!*handled) return FTK_OK;
+  const int row_pairs = (M + 63) / 64;
+  const long long units = (long long)G * gr.ptiles;
+  long long per = (cus + units - 1) / units;
+  per = std::max(1LL, std::min(per, (long long)(row_pairs + waves - 1) / waves));
+  gr.per_problem = (int)per;
+  const long long total = units * per;
+  if (total > 0x7fffffffLL) return fail(FTK_ERR_UNSUPPORTED_SHAPE, "ftk_b2b_gemm_f16: grid too large");
+  gr.total = (int)total;
+  static bool attr_set = false;
+  if (!attr_set) {
+    FTK_HIP(hipFuncSetAttribute((const void*)b2b_gemm8_kernel<KS, PT, NT>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                (int)lds));
+    attr_set = true;
+  }
+  hipLaunchKernelGGL((b2b_gemm8_kernel<KS, PT, NT>), dim3(gr.total), dim3(waves * 64), lds, s, (const _Float16*)A,
+                     (const _Float16*)B, (const _Float16*)C, (_Float16*)D, M, P, p_base, gr);
+  return check_launch("b2b_gemm8_kernel");
+}
+
 static int b2b_wave_region(int K, int pw) { return 32 * (K + 8) + 32 * (pw + 4); }
 
 static size_t b2b_lds_bytes(int N, int K, int pw, int waves) {
@@ -306,7 +534,16 @@ static int launch_b2b(const void* A, const void* B, const void* C, void* D, int 
   const int full = P / B2B_PTILE;
   const int rem = (P % B2B_PTILE) / 32;
   int rc = FTK_OK;
-  if (full > 0) rc = launch_b2b_cols<KS, 4>(A, B, C, D, G, M, N, P, 0, full, cus, lds_max, s);
+  if (full > 0) {
+    // the eight-wave kernel covers K in {64, 128} x N in {64, 128}; FTK_B2B_WAVES=4 forces the four-wave one
+    bool handled = false;
+    static const bool allow8 = !(getenv("FTK_B2B_WAVES") && atoi(getenv("FTK_B2B_WAVES")) == 4);
+    if constexpr (KS == 4 || KS == 8) {
+      if (allow8 && N == 128) rc = launch_b2b8<KS, 4, 4>(A, B, C, D, G, M, P, 0, full, cus, lds_max, &handled, s);
+      if (allow8 && N == 64) rc = launch_b2b8<KS, 4, 2>(A, B, C, D, G, M, P, 0, full, cus, lds_max, &handled, s);
+    }
+    if (!handled) rc = launch_b2b_cols<KS, 4>(A, B, C, D, G, M, N, P, 0, full, cus, lds_max, s);
+  }
   if (rc) return rc;
   const int pb = full * B2B_PTILE;
   switch (rem) {
