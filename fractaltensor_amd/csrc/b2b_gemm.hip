@@ -261,15 +261,18 @@ __global__ __launch_bounds__(256) void b2b_gemm_kernel(const _Float16* __restric
 }
 
 // Eight-wave form of the same computation for the common shapes (N = 32*NT up
-// to 128, all of B and C resident): every wave takes one 64-row group at a
-// time, two waves share a SIMD, and the work is ordered so that it fits their
-// 256 registers each -- GEMM1 runs to completion first and leaves P for the 64
-// rows as fp16 B-operands in registers (64 of them at N = 128), then GEMM2 runs
-// over the D columns in groups of 64 with its own 64 accumulator registers and
-// stores each group as it finishes.  With all A loads of the workgroup issued
-// at the start and two waves per SIMD, one wave's LDS round trips, conversions
-// and D stores are covered by the other's MFMAs.  The wave-private LDS region
-// is used twice: A rows on the way in, D rows on the way out.
+// to 128, all of B and C resident).  Two waves share a SIMD and every wave
+// walks 32-row units, so the work is ordered to fit 256 registers and to start
+// on the first rows to arrive: GEMM1 of a unit runs to completion and leaves P
+// as fp16 B-operands in registers, then GEMM2 runs over the D columns in groups
+// of 64 with its own accumulators and stores each group as it finishes.  The
+// kernel is bound by how fast a CU's memory pipeline takes the workgroup's
+// loads (B, C and 512 rows of A are all requested up front, B and C first
+// because everything waits for them); units are small so that compute on the
+// rows that have landed overlaps the rest of the stream and little work is
+// left when the last rows arrive, and two waves per SIMD cover each other's LDS
+// round trips, conversions and D stores.  The wave-private LDS region is used
+// twice per unit: A rows on the way in, D rows on the way out.
 template <int KS, int PT, int NT>
 __global__ __launch_bounds__(512) void b2b_gemm8_kernel(const _Float16* __restrict__ A,
                                                         const _Float16* __restrict__ Bm,
@@ -279,7 +282,7 @@ __global__ __launch_bounds__(512) void b2b_gemm8_kernel(const _Float16* __restri
   constexpr int N = 32 * NT;
   constexpr int BLD = K + 8;   // padded Bs / A-staging row (halfs)
   constexpr int CLD = N + 4;   // padded Cs row (halfs)
-  constexpr int AN = 2 * KS;   // 16-byte A loads per lane for 64 rows
+  constexpr int AN = KS;       // 16-byte A loads per lane for 32 rows
   constexpr int pw = 32 * PT;  // p columns handled here
   constexpr int PG = (PT + 1) / 2;  // column groups of up to 64
   constexpr int DLD = 64 + 4;  // padded D staging row (halfs)
@@ -309,21 +312,23 @@ __global__ __launch_bounds__(512) void b2b_gemm8_kernel(const _Float16* __restri
   const _Float16* Cg = Cm + (size_t)g * P * N + (size_t)p0 * N;
   _Float16* Dg = D + (size_t)g * M * P + p0;
 
-  const int row_pairs = (M + 63) / 64;
-  const int wave_stride = gr.per_problem * waves;
-  int pair = part * waves + wave;
+  // consecutive units of a workgroup go to consecutive waves: wave w takes units w, w + 8, ... of the
+  // workgroup's contiguous row range, so the rows that are requested first belong to different waves
+  const int units = (M + 31) / 32;
+  const int per_wg = (units + gr.per_problem - 1) / gr.per_problem;
+  const int unit_end = min(units, (part + 1) * per_wg);
+  int unit = part * per_wg + wave;
 
   constexpr int CPR = K / 8;  // 16-byte chunks per row
-  v4u areg[AN];
-  auto fetch_a = [&](int pr_) __attribute__((always_inline)) {
+  v4u areg0[AN];
+  auto fetch_a = [&](int un, v4u (&ar)[AN]) __attribute__((always_inline)) {
     static_for<AN>([&](auto uc) __attribute__((always_inline)) {
       constexpr int u = decltype(uc)::value;
       const int chunk = u * 64 + lane;
-      const int row = min(pr_ * 64 + chunk / CPR, M - 1);
-      areg[u] = ldg16(Ag + (size_t)row * K + 8 * (chunk % CPR));
+      const int row = min(un * 32 + chunk / CPR, M - 1);
+      ar[u] = ldg16(Ag + (size_t)row * K + 8 * (chunk % CPR));
     });
   };
-  if (pair < row_pairs) fetch_a(pair);
 
   // ---- stage Bs[n][k] and Cs[p][n], all loads of a thread in flight together
   {
@@ -357,57 +362,56 @@ __global__ __launch_bounds__(512) void b2b_gemm8_kernel(const _Float16* __restri
     }
   }
   __syncthreads();
+  // The A rows are requested only now, and one 32-row unit per wave at a time.  Requested together
+  // with B and C they fill the CU's memory pipeline ahead of the late waves' share of B and C; and with
+  // all 512 rows requested at once every request is served late in the burst (nothing arrives early
+  // when everything is in flight), so no wave could start before the end of it.  One unit per wave
+  // (64 KB per CU) is enough in flight to keep the memory pipeline busy, and the next unit is requested
+  // as soon as the current one has been taken out of its registers.
+  if (unit < unit_end) fetch_a(unit, areg0);
 
-  for (; pair < row_pairs; pair += wave_stride) {
-    // ---- A rows: park 32 at a time in the wave's region and pull the MFMA
-    // fragments; step s contracts k in [8s, 8s+8) (lanes 0-31) and
-    // [K/2 + 8s, K/2 + 8s + 8) (lanes 32-63)
-    v8h afrag[2][KS];
-    static_for<2>([&](auto rtc) __attribute__((always_inline)) {
-      constexpr int rt = decltype(rtc)::value;
-      static_for<AN / 2>([&](auto uc) __attribute__((always_inline)) {
-        constexpr int u = decltype(uc)::value;
-        const int chunk = u * 64 + lane;
-        *reinterpret_cast<v4u*>(Wr + (chunk / CPR) * BLD + 8 * (chunk % CPR)) = areg[rt * (AN / 2) + u];
-      });
-#pragma unroll
-      for (int s = 0; s < KS; ++s) afrag[rt][s] = *reinterpret_cast<const v8h*>(Wr + j * BLD + hh * (K / 2) + 8 * s);
+  // one 32-row unit whose A chunks are in ar; refills ar with the wave's next unit
+  auto do_unit = [&](int un, v4u (&ar)[AN]) __attribute__((always_inline)) {
+    // ---- A rows: park in the wave's region and pull the MFMA fragments; step s contracts
+    // k in [8s, 8s+8) (lanes 0-31) and [K/2 + 8s, K/2 + 8s + 8) (lanes 32-63)
+    v8h afrag[KS];
+    static_for<AN>([&](auto uc) __attribute__((always_inline)) {
+      constexpr int u = decltype(uc)::value;
+      const int chunk = u * 64 + lane;
+      *reinterpret_cast<v4u*>(Wr + (chunk / CPR) * BLD + 8 * (chunk % CPR)) = ar[u];
     });
+#pragma unroll
+    for (int s = 0; s < KS; ++s) afrag[s] = *reinterpret_cast<const v8h*>(Wr + j * BLD + hh * (K / 2) + 8 * s);
+    if (un + waves < unit_end) fetch_a(un + waves, ar);
 
-    // ---- GEMM1 for every n tile: P^T tiles [32 n, 32 rows] of both row tiles, rounded to fp16
-    v8h pf[2][NT][2];
+    // ---- GEMM1 for every n tile: P^T tiles [32 n, 32 rows], rounded to fp16
+    v8h pf[NT][2];
     static_for<NT>([&](auto ntc) __attribute__((always_inline)) {
       constexpr int nt = decltype(ntc)::value;
-      v16f pacc[2];
+      v16f pacc;
 #pragma unroll
-      for (int rt = 0; rt < 2; ++rt)
-#pragma unroll
-        for (int r = 0; r < 16; ++r) pacc[rt][r] = 0.0f;
+      for (int r = 0; r < 16; ++r) pacc[r] = 0.0f;
       const _Float16* brow = Bs + (nt * 32 + j) * BLD + hh * (K / 2);
 #pragma unroll
       for (int s = 0; s < KS; ++s) {
         const v8h bfrag = *reinterpret_cast<const v8h*>(brow + 8 * s);
-        pacc[0] = __builtin_amdgcn_mfma_f32_32x32x16_f16(bfrag, afrag[0][s], pacc[0], 0, 0, 0);
-        pacc[1] = __builtin_amdgcn_mfma_f32_32x32x16_f16(bfrag, afrag[1][s], pacc[1], 0, 0, 0);
+        pacc = __builtin_amdgcn_mfma_f32_32x32x16_f16(bfrag, afrag[s], pacc, 0, 0, 0);
       }
 #pragma unroll
-      for (int rt = 0; rt < 2; ++rt)
+      for (int s = 0; s < 2; ++s)
 #pragma unroll
-        for (int s = 0; s < 2; ++s)
-#pragma unroll
-          for (int e = 0; e < 8; ++e) pf[rt][nt][s][e] = (_Float16)pacc[rt][8 * s + e];
+        for (int e = 0; e < 8; ++e) pf[nt][s][e] = (_Float16)pacc[8 * s + e];
     });
+
     // ---- GEMM2 and store, 64 columns of D at a time
     static_for<PG>([&](auto pgc) __attribute__((always_inline)) {
       constexpr int pg = decltype(pgc)::value;
       constexpr int PW = (PT - 2 * pg) >= 2 ? 2 : 1;  // p tiles in this group
-      v16f dacc[2][PW];
+      v16f dacc[PW];
 #pragma unroll
-      for (int rt = 0; rt < 2; ++rt)
+      for (int q = 0; q < PW; ++q)
 #pragma unroll
-        for (int q = 0; q < PW; ++q)
-#pragma unroll
-          for (int r = 0; r < 16; ++r) dacc[rt][q][r] = 0.0f;
+        for (int r = 0; r < 16; ++r) dacc[q][r] = 0.0f;
       static_for<NT>([&](auto ntc) __attribute__((always_inline)) {
         constexpr int nt = decltype(ntc)::value;
 #pragma unroll
@@ -418,8 +422,7 @@ __global__ __launch_bounds__(512) void b2b_gemm8_kernel(const _Float16* __restri
             const v4h c0 = *reinterpret_cast<const v4h*>(crow + 16 * s);
             const v4h c1 = *reinterpret_cast<const v4h*>(crow + 16 * s + 8);
             const v8h cfrag = {c0[0], c0[1], c0[2], c0[3], c1[0], c1[1], c1[2], c1[3]};
-            dacc[0][q] = __builtin_amdgcn_mfma_f32_32x32x16_f16(cfrag, pf[0][nt][s], dacc[0][q], 0, 0, 0);
-            dacc[1][q] = __builtin_amdgcn_mfma_f32_32x32x16_f16(cfrag, pf[1][nt][s], dacc[1][q], 0, 0, 0);
+            dacc[q] = __builtin_amdgcn_mfma_f32_32x32x16_f16(cfrag, pf[nt][s], dacc[q], 0, 0, 0);
           }
         }
       });
@@ -427,33 +430,28 @@ __global__ __launch_bounds__(512) void b2b_gemm8_kernel(const _Float16* __restri
       // A wave reads back only what it wrote itself and LDS operations of one
       // wave complete in order, so no barrier is needed.
 #pragma unroll
-      for (int rt = 0; rt < 2; ++rt) {
+      for (int q = 0; q < PW; ++q)
 #pragma unroll
-        for (int q = 0; q < PW; ++q)
+        for (int gq = 0; gq < 4; ++gq) {
+          const v4h o = {(_Float16)dacc[q][4 * gq + 0], (_Float16)dacc[q][4 * gq + 1], (_Float16)dacc[q][4 * gq + 2],
+                         (_Float16)dacc[q][4 * gq + 3]};
+          *reinterpret_cast<v4h*>(Wr + j * DLD + q * 32 + 8 * gq + 4 * hh) = o;
+        }
+      constexpr int segs = PW * 4;  // 16-byte segments per row
 #pragma unroll
-          for (int gq = 0; gq < 4; ++gq) {
-            const v4h o = {(_Float16)dacc[rt][q][4 * gq + 0], (_Float16)dacc[rt][q][4 * gq + 1],
-                           (_Float16)dacc[rt][q][4 * gq + 2], (_Float16)dacc[rt][q][4 * gq + 3]};
-            *reinterpret_cast<v4h*>(Wr + j * DLD + q * 32 + 8 * gq + 4 * hh) = o;
-          }
-        constexpr int segs = PW * 4;  // 16-byte segments per row
-#pragma unroll
-        for (int idx = lane; idx < 32 * segs; idx += 64) {
-          const int r = idx / segs;
-          const int sg = idx - r * segs;
-          const int grow = pair * 64 + 32 * rt + r;
-          if (grow < M) {
-            const v2u lo = *reinterpret_cast<const v2u*>(Wr + r * DLD + 8 * sg);
-            const v2u hi = *reinterpret_cast<const v2u*>(Wr + r * DLD + 8 * sg + 4);
-            *reinterpret_cast<v4u*>(Dg + (size_t)grow * P + 64 * pg + 8 * sg) = v4u{lo[0], lo[1], hi[0], hi[1]};
-          }
+      for (int idx = lane; idx < 32 * segs; idx += 64) {
+        const int r = idx / segs;
+        const int sg = idx - r * segs;
+        const int grow = un * 32 + r;
+        if (grow < M) {
+          const v2u lo = *reinterpret_cast<const v2u*>(Wr + r * DLD + 8 * sg);
+          const v2u hi = *reinterpret_cast<const v2u*>(Wr + r * DLD + 8 * sg + 4);
+          *reinterpret_cast<v4u*>(Dg + (size_t)grow * P + 64 * pg + 8 * sg) = v4u{lo[0], lo[1], hi[0], hi[1]};
         }
       }
     });
-    // a further row group of this wave is fetched only now: its registers are not free earlier, and
-    // the other wave on the SIMD keeps the matrix unit busy meanwhile
-    if (pair + wave_stride < row_pairs) fetch_a(pair + wave_stride);
-  }
+  };
+  for (; unit < unit_end; unit += waves) do_unit(unit, areg0);
 }
 
 template <int KS, int PT, int NT>
@@ -466,10 +464,10 @@ static int launch_b2b8(const void* A, const void* B, const void* C, void* D, int
   const size_t lds = (size_t)(N * (K + 8) + pw * (N + 4) + waves * gr.wave_region) * 2;
   *handled = (int)lds <= lds_max;
   if (!*handled) return FTK_OK;
-  const int row_pairs = (M + 63) / 64;
+  const int row_units = (M + 31) / 32;
   const long long units = (long long)G * gr.ptiles;
   long long per = (cus + units - 1) / units;
-  per = std::max(1LL, std::min(per, (long long)(row_pairs + waves - 1) / waves));
+  per = std::max(1LL, std::min(per, (long long)(row_units + waves - 1) / waves));
   gr.per_problem = (int)per;
   const long long total = units * per;
   if (total > 0x7fffffffLL) return fail(FTK_ERR_UNSUPPORTED_SHAPE, "ftk_b2b_gemm_f16: grid too large");
