@@ -181,6 +181,10 @@ def b2b_inputs(seed, G, M, N, K, P):
     (3, 256, 96, 96, 160),      # P spans two workgroup tiles, odd tile counts
     (1, 8192, 256, 64, 64),     # reference benchmark shape (fused_two_hgemms.cu:152-175)
     (1, 1024, 512, 64, 64),
+    (2, 300, 64, 64, 128),      # eight-wave kernel (N, K in {64, 128}, full 128-column tiles), ragged M
+    (2, 1000, 128, 64, 256),    # eight-wave kernel, two column tiles, units that do not divide evenly
+    (1, 4100, 128, 128, 160),   # eight-wave kernel for the first 128 columns, four-wave kernel for the last 32
+    (3, 31, 64, 128, 128),      # fewer rows than one unit
 ])
 def test_b2b_gemm(core, G, M, N, K, P):
     A, Bn, Cp = b2b_inputs(9, G, M, N, K, P)
