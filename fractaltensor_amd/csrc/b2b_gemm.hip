@@ -320,7 +320,7 @@ __global__ __launch_bounds__(512) void b2b_gemm8_kernel(const _Float16* __restri
   int unit = part * per_wg + wave;
 
   constexpr int CPR = K / 8;  // 16-byte chunks per row
-  v4u areg0[AN];
+  v4u areg0[AN], areg1[AN];
   auto fetch_a = [&](int un, v4u (&ar)[AN]) __attribute__((always_inline)) {
     static_for<AN>([&](auto uc) __attribute__((always_inline)) {
       constexpr int u = decltype(uc)::value;
@@ -345,6 +345,13 @@ __global__ __launch_bounds__(512) void b2b_gemm8_kernel(const _Float16* __restri
       const int idx = u * threads + tid;
       if (idx < ncq) vc[u] = ldg16(Cg + (size_t)idx * 8);
     }
+    // Requests are served roughly in the order the CU's memory pipeline accepted them.  The barrier
+    // puts every wave's share of B and C (which everything waits for) ahead of any A row; then one
+    // 32-row unit per wave follows, and the second unit once B and C have landed -- with all 512 rows
+    // of the workgroup requested at once nothing arrives early, and no wave could start before the end
+    // of the burst.
+    __syncthreads();
+    if (unit < unit_end) fetch_a(unit, areg0);
 #pragma unroll
     for (int u = 0; u < UB; ++u) {
       const int idx = u * threads + tid;
@@ -362,15 +369,9 @@ __global__ __launch_bounds__(512) void b2b_gemm8_kernel(const _Float16* __restri
     }
   }
   __syncthreads();
-  // The A rows are requested only now, and one 32-row unit per wave at a time.  Requested together
-  // with B and C they fill the CU's memory pipeline ahead of the late waves' share of B and C; and with
-  // all 512 rows requested at once every request is served late in the burst (nothing arrives early
-  // when everything is in flight), so no wave could start before the end of it.  One unit per wave
-  // (64 KB per CU) is enough in flight to keep the memory pipeline busy, and the next unit is requested
-  // as soon as the current one has been taken out of its registers.
-  if (unit < unit_end) fetch_a(unit, areg0);
+  if (unit + waves < unit_end) fetch_a(unit + waves, areg1);
 
-  // one 32-row unit whose A chunks are in ar; refills ar with the wave's next unit
+  // one 32-row unit whose A chunks are in ar; refills ar with the unit two further on
   auto do_unit = [&](int un, v4u (&ar)[AN]) __attribute__((always_inline)) {
     // ---- A rows: park in the wave's region and pull the MFMA fragments; step s contracts
     // k in [8s, 8s+8) (lanes 0-31) and [K/2 + 8s, K/2 + 8s + 8) (lanes 32-63)
@@ -382,7 +383,7 @@ __global__ __launch_bounds__(512) void b2b_gemm8_kernel(const _Float16* __restri
     });
 #pragma unroll
     for (int s = 0; s < KS; ++s) afrag[s] = *reinterpret_cast<const v8h*>(Wr + j * BLD + hh * (K / 2) + 8 * s);
-    if (un + waves < unit_end) fetch_a(un + waves, ar);
+    if (un + 2 * waves < unit_end) fetch_a(un + 2 * waves, ar);
 
     // ---- GEMM1 for every n tile: P^T tiles [32 n, 32 rows], rounded to fp16
     v8h pf[NT][2];
@@ -451,7 +452,10 @@ __global__ __launch_bounds__(512) void b2b_gemm8_kernel(const _Float16* __restri
       }
     });
   };
-  for (; unit < unit_end; unit += waves) do_unit(unit, areg0);
+  for (; unit < unit_end; unit += 2 * waves) {
+    do_unit(unit, areg0);
+    if (unit + waves < unit_end) do_unit(unit + waves, areg1);
+  }
 }
 
 template <int KS, int PT, int NT>
