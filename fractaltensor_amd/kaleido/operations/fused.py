@@ -22,7 +22,7 @@ import torch
 from ..fractal_tensor import FractalTensor
 from ..tensor import Tensor
 
-__all__ = ['pack_lstm_weights', 'stacked_lstm', 'dilated_lstm', 'lstm_cell', 'flash_attention', 'b2b_gemm',
+__all__ = ['pack_lstm_weights', 'pad_time_major', 'unpad_time_major', 'stacked_lstm', 'dilated_lstm', 'lstm_cell', 'flash_attention', 'b2b_gemm',
            'online_softmax']
 
 
@@ -64,26 +64,68 @@ def pack_lstm_weights(Wss: FractalTensor, Uss: FractalTensor, bss: Optional[Frac
     return WU.contiguous(), bias
 
 
+def pad_time_major(xss: FractalTensor):
+    """Time-major batch [T][B_t] of [1, H] -> (dense [T, B_0, H], batch sizes or None).
+
+    A regular batch is returned as a view.  A ragged one must be what
+    examples/utils/data_utils.py:42-66 builds for sequences sorted by length:
+    step t holds the first B_t sequences, B_t non-increasing.  It is padded with
+    zero rows; rows of a batch are independent in every LSTM layer, so the
+    padding rows compute values nobody reads and the rows that matter are exact."""
+    if not isinstance(xss, FractalTensor):
+        raise TypeError('xss should be a FractalTensor.')
+    if xss.depth != 2:
+        raise ValueError(f'xss should have depth 2, got {xss.depth}.')
+    if xss.is_regular():
+        xs = _dense_gpu(xss, 'xss', 2)
+        return xs.reshape(xs.shape[0], xs.shape[1], xs.shape[-1]), None
+    sizes = [len(step) for step in xss.indices]
+    if any(b <= 0 for b in sizes) or any(a < b for a, b in zip(sizes, sizes[1:])):
+        raise ValueError('a ragged batch must be time-major with non-increasing, positive batch sizes per step.')
+    H = xss.element_shape[-1]
+    flat = xss.data.view(-1, H)
+    if not flat.is_cuda:
+        raise RuntimeError(f'xss lives on {flat.device}; the fused kernels run on the GPU only.')
+    xs = torch.zeros((len(sizes), sizes[0], H), dtype=flat.dtype, device=flat.device)
+    off = 0
+    for t, b in enumerate(sizes):
+        xs[t, :b] = flat[off:off + b]
+        off += b
+    return xs, sizes
+
+
+def unpad_time_major(dense: torch.Tensor, sizes) -> FractalTensor:
+    """dense [T, B_0, H] -> depth-2 [T][B_t] of [1, H] keeping the first B_t rows of step t."""
+    T, B0, H = dense.shape
+    if sizes is None:
+        return FractalTensor.from_dense(dense.reshape(T, B0, 1, H), 2)
+    return FractalTensor.from_fractaltensors(
+        *[FractalTensor.from_dense(dense[t, :b].reshape(b, 1, H), 1) for t, b in enumerate(sizes)])
+
+
 def _run_stack(xss, Wss, Uss, bss, dilations, return_all_layers):
     core = _core()
-    xs = _dense_gpu(xss, 'xss', 2)   # [T, B, 1, H]
-    T, B = xs.shape[0], xs.shape[1]
-    H = xs.shape[-1]
-    xs = xs.reshape(T, B, H)
+    xs, sizes = pad_time_major(xss)
     WU, bias = pack_lstm_weights(Wss, Uss, bss)
     hsss, csss = core.stacked_lstm(xs.float(), WU.float(), None if bias is None else bias.float(), dilations=dilations)
     L = WU.shape[0]
     if return_all_layers:
-        return (FractalTensor.from_dense(hsss.view(L, T, B, 1, H), 3), FractalTensor.from_dense(csss.view(L, T, B, 1, H), 3))
-    return FractalTensor.from_dense(hsss[L - 1].reshape(T, B, 1, H), 2)
+        if sizes is None:
+            T, B, H = xs.shape
+            return (FractalTensor.from_dense(hsss.view(L, T, B, 1, H), 3),
+                    FractalTensor.from_dense(csss.view(L, T, B, 1, H), 3))
+        return (FractalTensor.from_fractaltensors(*[unpad_time_major(hsss[l], sizes) for l in range(L)]),
+                FractalTensor.from_fractaltensors(*[unpad_time_major(csss[l], sizes) for l in range(L)]))
+    return unpad_time_major(hsss[L - 1], sizes)
 
 
 def stacked_lstm(xss: FractalTensor, Wss: FractalTensor, Uss: FractalTensor, bss: Optional[FractalTensor] = None,
                  return_all_layers: bool = False):
     """Stacked LSTM over a time-major batch.
 
-    xss: depth-2 [T][B] of [1, H] (what stacked_rnn.py's `embs` is for equal-length
-    sequences).  Returns the last layer's hidden sequence as depth-2 [T][B] of
+    xss: depth-2 [T][B_t] of [1, H]: what stacked_rnn.py's `embs` is, either for
+    equal-length sequences or the ragged time-major batch of length-sorted
+    sequences (shrinking batch per step, stacked_rnn.py:49).  Returns the last layer's hidden sequence as depth-2 [T][B] of
     [1, H], which is what the reference's stacked_lstm returns; with
     return_all_layers the (h, c) of every layer as depth-3 [L][T][B]."""
     return _run_stack(xss, Wss, Uss, bss, None, return_all_layers)

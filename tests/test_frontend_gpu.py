@@ -92,10 +92,48 @@ def test_fused_b2b_gemm_equals_operator_expression():
     assert out.depth == 1 and len(out) == 2 and torch.equal(out[1].data, fused.data)
 
 
-def test_fused_paths_reject_ragged_input():
+def _ragged_batch(lengths, H, seed):
+    """Time-major batch of sequences sorted by length: step t holds the sequences longer than t."""
+    g = torch.Generator().manual_seed(seed)
+    seqs = [torch.randn((n, H), generator=g) for n in lengths]
+    steps = []
+    for t in range(max(lengths)):
+        rows = torch.stack([s[t] for s in seqs if s.shape[0] > t])
+        steps.append(FractalTensor.from_dense(rows.reshape(-1, 1, H).cuda(), 1))
+    return FractalTensor.from_fractaltensors(*steps), seqs
+
+
+def test_fused_stacked_lstm_on_ragged_time_major_batch():
+    L, H = 2, 32
+    lengths = [6, 6, 4, 3, 1]
+    Wss, Uss, bss = programs.make_lstm_params(L, H, 1 / 16, seed=7, device='cuda')
+    xss, seqs = _ragged_batch(lengths, H, seed=8)
+    assert not xss.is_regular()
+    fused = ops.fused.stacked_lstm(xss, Wss, Uss, bss)
+    assert fused.depth == 2 and [len(step) for step in fused.indices] == [5, 4, 4, 3, 2, 2]
+    WU, bias = _np_params(Wss, Uss, bss)
+    # every sequence on its own through the oracle, at its own length
+    for b, seq in enumerate(seqs):
+        ref, _ = ko.stacked_lstm(seq.numpy()[:, None, :], WU, bias)
+        for t in range(seq.shape[0]):
+            got = fused[t][b].data.cpu().numpy().reshape(H)
+            assert ko.max_rel_err(got, ref[-1][t, 0]) <= 1e-4
+    # and against the eager operator program on the same ragged FractalTensor
+    eager = programs.stacked_lstm(xss, Wss, Uss, bss)
+    assert [len(step) for step in eager.indices] == [len(step) for step in fused.indices]
+    assert ko.max_rel_err(fused.data.cpu().numpy(), eager.data.cpu().numpy()) <= 1e-4
+    hsss, csss = ops.fused.stacked_lstm(xss, Wss, Uss, bss, return_all_layers=True)
+    assert hsss.depth == 3 and len(hsss) == L and [len(step) for step in hsss[0].indices] == [5, 4, 4, 3, 2, 2]
+    assert torch.equal(hsss[L - 1].data, fused.data)
+
+
+def test_fused_paths_reject_batches_that_are_not_time_major():
     Wss, Uss, bss = programs.make_lstm_params(1, 32, 0.1, seed=1, device='cuda')
     t = torch.randn(5, 1, 32).cuda()
     row = lambda n: FractalTensor.from_dense(t[:n].contiguous(), 1)
-    ragged = FractalTensor.from_fractaltensors(row(3), row(2))
+    growing = FractalTensor.from_fractaltensors(row(2), row(3))
+    with pytest.raises(ValueError, match='non-increasing'):
+        ops.fused.stacked_lstm(growing, Wss, Uss, bss)
+    deep = FractalTensor.from_fractaltensors(growing, growing)   # depth 3, ragged
     with pytest.raises(ValueError, match='ragged'):
-        ops.fused.stacked_lstm(ragged, Wss, Uss, bss)
+        ops.fused.flash_attention(deep, deep, deep)
