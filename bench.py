@@ -91,8 +91,8 @@ def bench_b2b(torch, core, steps, warmup, cpu):
         'host_wall_ms_per_step': wall,
         'roofline': {'bound': 'hbm', 'achieved': nbytes / ms / 1e6, 'peak': PEAK_HBM_GBS, 'unit': 'GB/s',
                      'frac': nbytes / ms / 1e6 / PEAK_HBM_GBS,
-                     'traffic': MEASURED_TRAFFIC_BYTES.get('b2b_gemm_kernel'),
-                     'kernel': 'b2b_gemm_kernel<8,4>', 'algorithmic_bytes_per_launch': nbytes},
+                     'traffic': MEASURED_TRAFFIC_BYTES.get('b2b_gemm8_kernel'),
+                     'kernel': 'b2b_gemm8_kernel<8,4,4>', 'algorithmic_bytes_per_launch': nbytes},
     }
     if cpu:
         from oracle import c_oracle

@@ -500,22 +500,33 @@ __global__ __launch_bounds__(WAVES * 64, MINB) void flash_attn_kernel(const _Flo
     step(ntiles - 1, std::false_type{}, std::false_type{});
   }
 
-  // ---- normalise and store: lane holds d = 32dt + 8g + 4*half + r of its row
+  // ---- normalise and store.  A lane holds d = 32dt + 8g + 4*half + r of its row: 8-byte pieces,
+  // the other half of each 16 bytes sitting in lane^32.  The two lanes trade pieces (this one's g odd /
+  // g even piece for the partner's) so that each stores 16 contiguous bytes and every store instruction
+  // fills whole 32-byte sectors; with 8-byte stores the memory system writes twice the bytes.
 #pragma unroll
   for (int qt = 0; qt < QT; ++qt) {
     const float l = l_run[qt] + __shfl_xor(l_run[qt], 32);
     const float inv = 1.0f / l;
     const int row = q_base + 32 * qt + j;
-    if (row < Sq) {
 #pragma unroll
-      for (int dt = 0; dt < DT; ++dt)
+    for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
-        for (int g = 0; g < 4; ++g) {
-          const v4h o = {(_Float16)(oacc[qt][dt][4 * g + 0] * inv), (_Float16)(oacc[qt][dt][4 * g + 1] * inv),
-                         (_Float16)(oacc[qt][dt][4 * g + 2] * inv), (_Float16)(oacc[qt][dt][4 * g + 3] * inv)};
-          *reinterpret_cast<v4h*>(Og + (size_t)row * D + 32 * dt + 8 * g + 4 * hh) = o;
+      for (int m = 0; m < 2; ++m) {
+        v2u x, y;  // pieces g = 2m and g = 2m + 1 as packed halfs
+#pragma unroll
+        for (int w = 0; w < 2; ++w) {
+          const v2h xe = {(_Float16)(oacc[qt][dt][8 * m + 2 * w] * inv), (_Float16)(oacc[qt][dt][8 * m + 2 * w + 1] * inv)};
+          const v2h ye = {(_Float16)(oacc[qt][dt][8 * m + 4 + 2 * w] * inv),
+                          (_Float16)(oacc[qt][dt][8 * m + 4 + 2 * w + 1] * inv)};
+          x[w] = __builtin_bit_cast(unsigned, xe);
+          y[w] = __builtin_bit_cast(unsigned, ye);
+          // afterwards lanes 0-31 hold (own x, partner's x), lanes 32-63 (partner's y, own y)
+          asm volatile("s_nop 1\n\tv_permlane32_swap_b32_e32 %0, %1\n\ts_nop 1" : "+v"(x[w]), "+v"(y[w]));
         }
-    }
+        if (row < Sq)
+          *reinterpret_cast<v4u*>(Og + (size_t)row * D + 32 * dt + 16 * m + 8 * hh) = v4u{x[0], x[1], y[0], y[1]};
+      }
   }
 }
 
