@@ -385,24 +385,31 @@ __global__ __launch_bounds__(512) void b2b_gemm8_kernel(const _Float16* __restri
     for (int s = 0; s < KS; ++s) afrag[s] = *reinterpret_cast<const v8h*>(Wr + j * BLD + hh * (K / 2) + 8 * s);
     if (un + 2 * waves < unit_end) fetch_a(un + 2 * waves, ar);
 
-    // ---- GEMM1 for every n tile: P^T tiles [32 n, 32 rows], rounded to fp16
+    // ---- GEMM1 for every n tile: P^T tiles [32 n, 32 rows], rounded to fp16.  The n tiles advance
+    // together (k step outermost), so consecutive MFMAs belong to different accumulators and none waits
+    // for the one before it.
     v8h pf[NT][2];
-    static_for<NT>([&](auto ntc) __attribute__((always_inline)) {
-      constexpr int nt = decltype(ntc)::value;
-      v16f pacc;
+    {
+      v16f pacc[NT];
 #pragma unroll
-      for (int r = 0; r < 16; ++r) pacc[r] = 0.0f;
-      const _Float16* brow = Bs + (nt * 32 + j) * BLD + hh * (K / 2);
+      for (int nt = 0; nt < NT; ++nt)
 #pragma unroll
-      for (int s = 0; s < KS; ++s) {
-        const v8h bfrag = *reinterpret_cast<const v8h*>(brow + 8 * s);
-        pacc = __builtin_amdgcn_mfma_f32_32x32x16_f16(bfrag, afrag[s], pacc, 0, 0, 0);
-      }
+        for (int r = 0; r < 16; ++r) pacc[nt][r] = 0.0f;
+      const _Float16* brow = Bs + j * BLD + hh * (K / 2);
 #pragma unroll
-      for (int s = 0; s < 2; ++s)
+      for (int s = 0; s < KS; ++s)
 #pragma unroll
-        for (int e = 0; e < 8; ++e) pf[nt][s][e] = (_Float16)pacc[8 * s + e];
-    });
+        for (int nt = 0; nt < NT; ++nt) {
+          const v8h bfrag = *reinterpret_cast<const v8h*>(brow + nt * 32 * BLD + 8 * s);
+          pacc[nt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(bfrag, afrag[s], pacc[nt], 0, 0, 0);
+        }
+#pragma unroll
+      for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+        for (int s = 0; s < 2; ++s)
+#pragma unroll
+          for (int e = 0; e < 8; ++e) pf[nt][s][e] = (_Float16)pacc[nt][8 * s + e];
+    }
 
     // ---- GEMM2 and store, 64 columns of D at a time
     static_for<PG>([&](auto pgc) __attribute__((always_inline)) {
