@@ -34,14 +34,6 @@
 
 namespace ftk {
 
-template <int N, typename F>
-__device__ __forceinline__ void static_for(F&& f) {
-  if constexpr (N > 0) {
-    static_for<N - 1>(f);
-    f(std::integral_constant<int, N - 1>{});
-  }
-}
-
 constexpr int B2B_PTILE = 128;  // p columns per workgroup
 
 __device__ __forceinline__ v4u ldg16(const void* p) { return *reinterpret_cast<const v4u*>(p); }

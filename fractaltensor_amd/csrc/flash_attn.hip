@@ -45,17 +45,6 @@
 
 namespace ftk {
 
-// Compile-time loop: the body sees its index as a constant expression, so
-// register arrays indexed by it are promoted to registers even when the body
-// sits under a runtime condition.
-template <int N, typename F>
-__device__ __forceinline__ void static_for(F&& f) {
-  if constexpr (N > 0) {
-    static_for<N - 1>(f);
-    f(std::integral_constant<int, N - 1>{});
-  }
-}
-
 constexpr int FA_KT = 64;          // keys per tile
 constexpr float FA_TAU = 8.0f;     // slack (in powers of two) before the running maximum is moved
 constexpr int FA_TRACE_TILES = 256;

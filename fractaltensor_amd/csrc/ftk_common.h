@@ -6,6 +6,8 @@
 #include <stdint.h>
 #include <stdio.h>
 
+#include <type_traits>
+
 #include "../../include/ftk.h"
 
 namespace ftk {
@@ -56,6 +58,17 @@ typedef unsigned v4u __attribute__((ext_vector_type(4)));
 typedef _Float16 v2h __attribute__((ext_vector_type(2)));
 typedef _Float16 v4h __attribute__((ext_vector_type(4)));
 typedef _Float16 v8h __attribute__((ext_vector_type(8)));
+
+// Compile-time loop: the body sees its index as a constant expression
+// (std::integral_constant), so register arrays indexed by it are promoted to
+// registers even when the body sits under a runtime condition.
+template <int N, typename F>
+__device__ __forceinline__ void static_for(F&& f) {
+  if constexpr (N > 0) {
+    static_for<N - 1>(f);
+    f(std::integral_constant<int, N - 1>{});
+  }
+}
 
 // ---- device math ------------------------------------------------------------
 // exp through the hardware base-2 exponential (about 1 ulp), reciprocal through

@@ -234,25 +234,53 @@ void lstm_persistent_kernel(PersistArgs a) {
       __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
     }
   };
-  // bias, activations and state update of an item: lane-local and branch-free,
-  // so the scheduler can slot it between MFMAs of the next item
-  auto epilogue_math = [&](const v16f& acc, const float4& cp, float (&hv)[4], float (&cv)[4]) __attribute__((always_inline)) {
+  // The same with a piece of vector work after the MFMAs of every step, each step fenced so that the
+  // pieces stay where they are put: an fp32 MFMA keeps the matrix unit busy for 64 cycles, and a dozen
+  // vector instructions issued behind it cost nothing.
+  auto mfma_part_with = [&](int buf, auto q0c, auto q1c, v16f& acc0, v16f& acc1, auto&& piece) __attribute__((always_inline)) {
+    constexpr int q0 = decltype(q0c)::value;
+    constexpr int q1 = decltype(q1c)::value;
+    const float* arow = tile + buf * P_TILE + j * P_LD + 4 * hh;
+    v4f b = *reinterpret_cast<const v4f*>(arow + 8 * q0);
+    __builtin_amdgcn_sched_barrier(0);
+    static_for<q1 - q0>([&](auto ic) __attribute__((always_inline)) {
+      constexpr int qq = q0 + decltype(ic)::value;
+      v4f bn = b;
+      if constexpr (qq + 1 < q1) bn = *reinterpret_cast<const v4f*>(arow + 8 * (qq + 1));
+      acc0 = __builtin_amdgcn_mfma_f32_32x32x2f32(wr[4 * qq + 0], b[0], acc0, 0, 0, 0);
+      acc1 = __builtin_amdgcn_mfma_f32_32x32x2f32(wr[4 * qq + 1], b[1], acc1, 0, 0, 0);
+      acc0 = __builtin_amdgcn_mfma_f32_32x32x2f32(wr[4 * qq + 2], b[2], acc0, 0, 0, 0);
+      acc1 = __builtin_amdgcn_mfma_f32_32x32x2f32(wr[4 * qq + 3], b[3], acc1, 0, 0, 0);
+      piece(ic);
+      b = bn;
+      __builtin_amdgcn_sched_barrier(0);
+    });
+  };
+  // bias, activations and state update of an item: lane-local and branch-free.
+  // piece m (0..15) of the computation: gate (m & 3) of unit (m >> 2); the last
+  // gate of a unit finishes its c and h
+  float eg_i = 0.f, eg_f = 0.f, eg_o = 0.f;
+  auto epilogue_piece = [&](const v16f& acc, const float4& cp, float (&hv)[4], float (&cv)[4], auto mc) __attribute__((always_inline)) {
+    constexpr int m = decltype(mc)::value;
+    constexpr int r = m >> 2;
     const float cpv[4] = {cp.x, cp.y, cp.z, cp.w};
-#pragma unroll
-    for (int r = 0; r < 4; ++r) {
-      const float ig = sigmoid_f(acc[r] + bi[r]);
-      const float fg = sigmoid_f(acc[4 + r] + bf[r]);
-      const float og = sigmoid_f(acc[8 + r] + bo[r]);
+    if constexpr ((m & 3) == 0) eg_i = sigmoid_f(acc[r] + bi[r]);
+    if constexpr ((m & 3) == 1) eg_f = sigmoid_f(acc[4 + r] + bf[r]);
+    if constexpr ((m & 3) == 2) eg_o = sigmoid_f(acc[8 + r] + bo[r]);
+    if constexpr ((m & 3) == 3) {
       const float cand = tanh_f(acc[12 + r] + bg[r]);
-      cv[r] = fg * cpv[r] + ig * cand;
-      hv[r] = og * tanh_f(cv[r]);
+      cv[r] = eg_f * cpv[r] + eg_i * cand;
+      hv[r] = eg_o * tanh_f(cv[r]);
     }
+  };
+  auto epilogue_math = [&](const v16f& acc, const float4& cp, float (&hv)[4], float (&cv)[4]) __attribute__((always_inline)) {
+    static_for<16>([&](auto mc) __attribute__((always_inline)) { epilogue_piece(acc, cp, hv, cv, mc); });
   };
   // h leaves through write-through stores, c through the cache
   auto epilogue_store = [&](int n, const float (&hv)[4], const float (&cv)[4]) __attribute__((always_inline)) {
     const int t = item_t(n), rb = item_rb(n);
     const int rg = rb * 32 + j;
-    if (alive && rg < B) {
+    if (alive && n >= 0 && rg < B) {
       float* hdst = a.hsss + ((size_t)l * T + t) * cell + (size_t)rg * PH + u0;
       float* cdst = a.csss + ((size_t)l * T + t) * cell + (size_t)rg * PH + u0;
       *reinterpret_cast<float4*>(cdst) = make_float4(cv[0], cv[1], cv[2], cv[3]);
@@ -367,12 +395,22 @@ void lstm_persistent_kernel(PersistArgs a) {
     const float4 cp = load_cprev(n);
 #pragma unroll
     for (int r = 0; r < 16; ++r) { acc0[r] = 0.0f; acc1[r] = 0.0f; }
-    mfma_part(buf, std::integral_constant<int, 0>{}, std::integral_constant<int, PH / 8>{}, acc0, acc1);
-    // the counters are consumed before the stores go out, so that waiting for
-    // those (old) loads never waits for the stores
+    // x half of the MFMAs, with the activations and state update of item n-1 in their shadow (one
+    // gate of one unit per step) and its stores as soon as the last piece is done.  For n = 0 the
+    // pieces run on zeros and nothing is stored.
+    {
+      float hv[4], cv[4];
+      mfma_part_with(buf, std::integral_constant<int, 0>{}, std::integral_constant<int, PH / 8>{}, acc0, acc1,
+                     [&](auto ic) __attribute__((always_inline)) {
+                       constexpr int i = decltype(ic)::value;
+                       if constexpr (i < 16) epilogue_piece(acc_prev, cp_prev, hv, cv, ic);
+                       if constexpr (i == 16) epilogue_store(n - 1, hv, cv);
+                     });
+    }
+    // the counters are consumed before the flag of item n-1 goes out, so that waiting for
+    // those (old) loads never waits for newer stores
     const bool ready2 = pending && flags_ready(fl);
     if (tracing) a.trace[TS * n + 1] = wall_clock64();
-    if (n > 0) epilogue(n - 1, acc_prev, cp_prev);
     if (tracing) a.trace[TS * n + 2] = wall_clock64();
     if (publish_mid && n > 0) publish(n - 1);
     if (pending) {
