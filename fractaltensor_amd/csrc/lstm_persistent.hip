@@ -436,7 +436,13 @@ void lstm_persistent_kernel(PersistArgs a) {
     cp_prev = cp;
     if (tracing) a.trace[TS * n + 4] = wall_clock64() | ((long long)(pending ? 7 : looks) << 60);
 
-    if (!publish_mid && n > 0) publish(n - 1);
+    // Item n-1 is published at the end of this item.  Normally (tile n+1 already requested) the wait for
+    // its stores is the wait for the tile, and the count goes out after the barrier, so that nothing
+    // waits for the count's own round trip; if this wave still has to wait for the producers of tile
+    // n+1, item n-1 is published first so that its consumers do not wait along.
+    // (Dilated layers keep the early count: there it measured faster.)
+    const bool late_flag = !publish_mid && n > 0 && !pending && d == 1;
+    if (!publish_mid && n > 0 && !late_flag) publish(n - 1);
     if (tracing) a.trace[TS * n + 5] = wall_clock64();
     // last resort: wait for the producers here
     if (pending) {
@@ -454,9 +460,12 @@ void lstm_persistent_kernel(PersistArgs a) {
     // its producers by a bit more, until the first look always succeeds and
     // the tile has the whole item to arrive.
     if (first_look_failed && !publish_mid) __builtin_amdgcn_s_sleep(80);
-    __builtin_amdgcn_s_waitcnt(0);  // tile n+1 has landed in LDS
+    if (late_flag) __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+    __builtin_amdgcn_s_waitcnt(0);  // tile n+1 has landed in LDS (and the stores of item n-1 are acknowledged)
     if (tracing) a.trace[TS * n + 6] = wall_clock64();
     __syncthreads();
+    if (late_flag && lane == 0 && alive)
+      __hip_atomic_fetch_add(flag_of(l, item_t(n - 1), item_rb(n - 1)), 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     if (tracing) a.trace[TS * n + 7] = wall_clock64();
   }
   epilogue(n_items - 1, acc_prev, cp_prev);
