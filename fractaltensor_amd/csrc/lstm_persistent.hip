@@ -118,7 +118,7 @@ constexpr int TS = 8;              // trace stamps per item
 
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1)))
 void lstm_persistent_kernel(PersistArgs a) {
-  extern __shared__ __attribute__((aligned(16))) float tile[];  // [2][32][P_LD]
+  extern __shared__ __attribute__((aligned(16))) float tile[];  // [2][32][P_LD], then 256 floats of scrap
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -129,6 +129,7 @@ void lstm_persistent_kernel(PersistArgs a) {
   int q = blockIdx.x;
   if (a.xcd_remap) q = (blockIdx.x & 7) * (gridDim.x >> 3) + (blockIdx.x >> 3);
   if (q >= a.groups) return;
+  if (q == a.trace_q && tid == 0) reinterpret_cast<long long*>(a.status + 16)[0] = wall_clock64();
   const int per_layer = PC * a.pr;
   const int l = q / per_layer;
   const int within = q - l * per_layer;
@@ -164,6 +165,15 @@ void lstm_persistent_kernel(PersistArgs a) {
   }
 
   bool alive = true;
+  if (q == a.trace_q && tid == 0) {
+    long long* st = reinterpret_cast<long long*>(a.status + 16);
+    st[1] = wall_clock64();  // weights requested (st[0]: kernel entry)
+    float sink = 0.f;
+#pragma unroll
+    for (int s2 = 0; s2 < PK / 2; s2 += 32) sink += wr[s2];
+    if (sink == 12345.678f) st[3] = 0;
+    st[2] = wall_clock64();  // weights (a sample of them) have arrived
+  }
 
   auto item_t = [&](int n) { return n / my_rbs; };
   auto item_rb = [&](int n) { return prs + a.pr * (n % my_rbs); };
@@ -208,6 +218,18 @@ void lstm_persistent_kernel(PersistArgs a) {
       lds_dma16(xsrc + (size_t)rg * PH + 4 * lane, dst + r * P_LD);
       if (has_prev) lds_dma16(hsrc + (size_t)rg * PH + 4 * lane, dst + r * P_LD + PH);
     }
+    // The first layer's input rows come from memory nobody has touched; pull the rows of the item after
+    // this one towards the cache now, so that their copy into LDS one item later is served from L2 like
+    // the other layers' rows.  One 4-byte-per-lane copy touches all 64 cache lines of the wave's 8 rows;
+    // it lands in a scrap area behind the tiles (a load into registers would need them reserved until
+    // the data arrives).
+    if (l == 0 && n + 1 < n_items) {
+      const int t2 = item_t(n + 1), rb2 = item_rb(n + 1);
+      const int rg = min(rb2 * 32 + 8 * wave + (lane >> 3), B - 1);
+      __builtin_amdgcn_global_load_lds(
+          (const __attribute__((address_space(1))) void*)(a.xs + (size_t)t2 * cell + (size_t)rg * PH + 32 * (lane & 7)),
+          (__attribute__((address_space(3))) void*)(tile + 2 * P_TILE + 64 * wave), 4, 0, 0);
+    }
   };
   // steps [q0, q1) of the K loop (steps 0..31: x rows of WU, 32..63: h rows)
   // into two accumulators so that consecutive MFMAs never wait on each other's
@@ -234,28 +256,6 @@ void lstm_persistent_kernel(PersistArgs a) {
       __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
     }
   };
-  // The same with a piece of vector work after the MFMAs of every step, each step fenced so that the
-  // pieces stay where they are put: an fp32 MFMA keeps the matrix unit busy for 64 cycles, and a dozen
-  // vector instructions issued behind it cost nothing.
-  auto mfma_part_with = [&](int buf, auto q0c, auto q1c, v16f& acc0, v16f& acc1, auto&& piece) __attribute__((always_inline)) {
-    constexpr int q0 = decltype(q0c)::value;
-    constexpr int q1 = decltype(q1c)::value;
-    const float* arow = tile + buf * P_TILE + j * P_LD + 4 * hh;
-    v4f b = *reinterpret_cast<const v4f*>(arow + 8 * q0);
-    __builtin_amdgcn_sched_barrier(0);
-    static_for<q1 - q0>([&](auto ic) __attribute__((always_inline)) {
-      constexpr int qq = q0 + decltype(ic)::value;
-      v4f bn = b;
-      if constexpr (qq + 1 < q1) bn = *reinterpret_cast<const v4f*>(arow + 8 * (qq + 1));
-      acc0 = __builtin_amdgcn_mfma_f32_32x32x2f32(wr[4 * qq + 0], b[0], acc0, 0, 0, 0);
-      acc1 = __builtin_amdgcn_mfma_f32_32x32x2f32(wr[4 * qq + 1], b[1], acc1, 0, 0, 0);
-      acc0 = __builtin_amdgcn_mfma_f32_32x32x2f32(wr[4 * qq + 2], b[2], acc0, 0, 0, 0);
-      acc1 = __builtin_amdgcn_mfma_f32_32x32x2f32(wr[4 * qq + 3], b[3], acc1, 0, 0, 0);
-      piece(ic);
-      b = bn;
-      __builtin_amdgcn_sched_barrier(0);
-    });
-  };
   // bias, activations and state update of an item: lane-local and branch-free.
   // piece m (0..15) of the computation: gate (m & 3) of unit (m >> 2); the last
   // gate of a unit finishes its c and h
@@ -277,21 +277,18 @@ void lstm_persistent_kernel(PersistArgs a) {
     static_for<16>([&](auto mc) __attribute__((always_inline)) { epilogue_piece(acc, cp, hv, cv, mc); });
   };
   // h leaves through write-through stores, c through the cache
-  auto epilogue_store = [&](int n, const float (&hv)[4], const float (&cv)[4]) __attribute__((always_inline)) {
+  auto epilogue = [&](int n, const v16f& acc, const float4& cp) __attribute__((always_inline)) {
+    float hv[4], cv[4];
+    epilogue_math(acc, cp, hv, cv);
     const int t = item_t(n), rb = item_rb(n);
     const int rg = rb * 32 + j;
-    if (alive && n >= 0 && rg < B) {
+    if (alive && rg < B) {
       float* hdst = a.hsss + ((size_t)l * T + t) * cell + (size_t)rg * PH + u0;
       float* cdst = a.csss + ((size_t)l * T + t) * cell + (size_t)rg * PH + u0;
       *reinterpret_cast<float4*>(cdst) = make_float4(cv[0], cv[1], cv[2], cv[3]);
       coherent_store8(hdst, hv[0], hv[1]);
       coherent_store8(hdst + 2, hv[2], hv[3]);
     }
-  };
-  auto epilogue = [&](int n, const v16f& acc, const float4& cp) __attribute__((always_inline)) {
-    float hv[4], cv[4];
-    epilogue_math(acc, cp, hv, cv);
-    epilogue_store(n, hv, cv);
   };
   auto load_cprev = [&](int n) __attribute__((always_inline)) -> float4 {
     const int t = item_t(n), rb = item_rb(n);
@@ -315,11 +312,9 @@ void lstm_persistent_kernel(PersistArgs a) {
 
   // How far apart an item and the item that needs it are in this workgroup's
   // own sequence decides the schedule: distance 1 (one row block, dilation 1)
-  // leaves nothing to overlap; distance 2 means item n-1 must be published
-  // before the wait for item n+1 can end.
+  // leaves nothing to overlap.
   const long long own_distance = (long long)d * my_rbs;
   const bool serial = own_distance < 2;
-  const bool publish_mid = own_distance < 3;
 
   if (serial) {
     for (int n = 0; n < n_items; ++n) {
@@ -345,30 +340,29 @@ void lstm_persistent_kernel(PersistArgs a) {
   }
 
   // ---- pipelined schedule.  Per item n:
-  //   x half of the MFMAs;
-  //   activations, state update and stores of item n-1;
-  //   h half of the MFMAs;
-  //   publish item n-1 (its stores went out half an item ago, so waiting for
-  //     their acknowledgement is free; with own_distance 2 the publish moves
-  //     up to the middle of the item);
-  //   one workgroup barrier.
-  // Tile n+1 goes into the other LDS buffer as soon as its producers are seen
-  // to be done.  The counters are requested a stretch of MFMAs before each of
-  // several look-at points, so looking costs nothing; only if every look fails
-  // does the wave wait at the end of the item, and then it also backs off once
-  // so that from then on it trails its producers by enough for an early look
-  // to succeed.
+  //   the first half of the x half of the MFMAs;
+  //   publish item n-1: its h and c went out at the end of item n-1, so by now
+  //     they are acknowledged and the wait costs nothing -- and nothing newer
+  //     is outstanding yet that the wait would also catch;
+  //   request tile n+1 into the other LDS buffer if its producers are seen to
+  //     be done (their counters were requested at the end of item n-1); if
+  //     not, look again after the x half, and wait only after the h half;
+  //   the rest of the x half, the h half;
+  //   wait for tile n+1, one workgroup barrier;
+  //   activations, state update and stores of item n.  (Vector instructions do
+  //   not hide behind fp32 MFMAs on this machine, so nothing is gained by
+  //   deferring them, and the sooner the stores go out the sooner the layer
+  //   above can start: an item is visible to its consumers about 2 us after
+  //   its last MFMA.  That hand-over time, 31 times in a row, is what the
+  //   wavefront pays at the start and at the end of a 32-layer stack.)
   alive = wait_deps(0);
   if (alive) issue_tile(0, 0);
   Flags fl = (n_items > 1) ? request_flags(1) : Flags{FLAG_TARGET, FLAG_TARGET};
   __builtin_amdgcn_s_waitcnt(0);
   __syncthreads();
 
-  v16f acc_prev;
-  float4 cp_prev = make_float4(0.f, 0.f, 0.f, 0.f);
-#pragma unroll
-  for (int r = 0; r < 16; ++r) acc_prev[r] = 0.0f;
-
+  constexpr int QX = PH / 8;   // MFMA steps of the x half
+  constexpr int QE = QX / 2;   // steps before the previous item is published (its stores take about 2 us to be acknowledged)
   for (int n = 0; n < n_items; ++n) {
     const int buf = n & 1;
     if (tracing) a.trace[TS * n + 0] = wall_clock64();
@@ -390,85 +384,35 @@ void lstm_persistent_kernel(PersistArgs a) {
       }
     };
 
-    look();  // counters requested in the middle of item n-1
-    const bool first_look_failed = pending;
     const float4 cp = load_cprev(n);
 #pragma unroll
     for (int r = 0; r < 16; ++r) { acc0[r] = 0.0f; acc1[r] = 0.0f; }
-    // x half of the MFMAs, with the activations and state update of item n-1 in their shadow (one
-    // gate of one unit per step) and its stores as soon as the last piece is done.  For n = 0 the
-    // pieces run on zeros and nothing is stored.
-    {
-      float hv[4], cv[4];
-      mfma_part_with(buf, std::integral_constant<int, 0>{}, std::integral_constant<int, PH / 8>{}, acc0, acc1,
-                     [&](auto ic) __attribute__((always_inline)) {
-                       constexpr int i = decltype(ic)::value;
-                       if constexpr (i < 16) epilogue_piece(acc_prev, cp_prev, hv, cv, ic);
-                       if constexpr (i == 16) epilogue_store(n - 1, hv, cv);
-                     });
-    }
-    // the counters are consumed before the flag of item n-1 goes out, so that waiting for
-    // those (old) loads never waits for newer stores
-    const bool ready2 = pending && flags_ready(fl);
+    mfma_part(buf, std::integral_constant<int, 0>{}, std::integral_constant<int, QE>{}, acc0, acc1);
+    if (n > 0) publish(n - 1);
+    look();
     if (tracing) a.trace[TS * n + 1] = wall_clock64();
+    mfma_part(buf, std::integral_constant<int, QE>{}, std::integral_constant<int, QX>{}, acc0, acc1);
     if (tracing) a.trace[TS * n + 2] = wall_clock64();
-    if (publish_mid && n > 0) publish(n - 1);
-    if (pending) {
-      ++looks;
-      if (ready2) {
-        asm volatile("" ::: "memory");
-        issue_tile(n + 1, buf ^ 1);
-        pending = false;
-      }
-    }
-    // counters of item n+2 for the first look of the next item (in
-    // publish-in-the-middle mode: of item n+1, for the wait at the end)
-    if (publish_mid) {
-      if (pending) fl = request_flags(n + 1);
-    } else if (!pending && n + 2 < n_items) {
-      fl = request_flags(n + 2);
-    }
+    look();
     if (tracing) a.trace[TS * n + 3] = wall_clock64();
-
-    if (has_prev) mfma_part(buf, std::integral_constant<int, PH / 8>{}, std::integral_constant<int, PK / 8>{}, acc0, acc1);
-#pragma unroll
-    for (int r = 0; r < 16; ++r) acc_prev[r] = acc0[r] + acc1[r];
-    cp_prev = cp;
+    if (has_prev) mfma_part(buf, std::integral_constant<int, QX>{}, std::integral_constant<int, PK / 8>{}, acc0, acc1);
     if (tracing) a.trace[TS * n + 4] = wall_clock64() | ((long long)(pending ? 7 : looks) << 60);
-
-    // Item n-1 is published at the end of this item.  Normally (tile n+1 already requested) the wait for
-    // its stores is the wait for the tile, and the count goes out after the barrier, so that nothing
-    // waits for the count's own round trip; if this wave still has to wait for the producers of tile
-    // n+1, item n-1 is published first so that its consumers do not wait along.
-    // (Dilated layers keep the early count: there it measured faster.)
-    const bool late_flag = !publish_mid && n > 0 && !pending && d == 1;
-    if (!publish_mid && n > 0 && !late_flag) publish(n - 1);
-    if (tracing) a.trace[TS * n + 5] = wall_clock64();
     // last resort: wait for the producers here
     if (pending) {
-      if (publish_mid && flags_ready(fl)) {
-        asm volatile("" ::: "memory");
-      } else {
-        alive = wait_deps(n + 1);
-      }
+      alive = wait_deps(n + 1);
       if (alive) issue_tile(n + 1, buf ^ 1);
-      if (n + 2 < n_items) fl = request_flags(n + 2);
-    } else if (publish_mid && n + 2 < n_items) {
-      fl = request_flags(n + 2);
     }
-    // Back off a little whenever the first look failed: the wave then trails
-    // its producers by a bit more, until the first look always succeeds and
-    // the tile has the whole item to arrive.
-    if (first_look_failed && !publish_mid) __builtin_amdgcn_s_sleep(80);
-    if (late_flag) __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
-    __builtin_amdgcn_s_waitcnt(0);  // tile n+1 has landed in LDS (and the stores of item n-1 are acknowledged)
+    if (n + 2 < n_items) fl = request_flags(n + 2);
+    if (tracing) a.trace[TS * n + 5] = wall_clock64();
+    __builtin_amdgcn_s_waitcnt(0);  // tile n+1 has landed in LDS
     if (tracing) a.trace[TS * n + 6] = wall_clock64();
     __syncthreads();
-    if (late_flag && lane == 0 && alive)
-      __hip_atomic_fetch_add(flag_of(l, item_t(n - 1), item_rb(n - 1)), 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    v16f acc;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) acc[r] = acc0[r] + acc1[r];
+    epilogue(n, acc, cp);
     if (tracing) a.trace[TS * n + 7] = wall_clock64();
   }
-  epilogue(n_items - 1, acc_prev, cp_prev);
   publish(n_items - 1);
 }
 
@@ -518,7 +462,7 @@ static int run_persistent(const float* xs, const float* WU, const float* bias, c
   const DeviceProps* dp = nullptr;
   int rc = device_props(&dp);
   if (rc) return rc;
-  const size_t lds = (size_t)2 * P_TILE * sizeof(float);
+  const size_t lds = (size_t)2 * P_TILE * sizeof(float) + 1024;  // two tiles + the prefetch scrap area
   if ((int)lds > dp->lds_optin) return FTK_OK;
   const void* fn = (const void*)lstm_persistent_kernel;
   static bool attr_set = false;
