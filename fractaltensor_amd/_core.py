@@ -20,7 +20,7 @@ EXPORTS = (
     'ftk_version', 'ftk_last_error', 'ftk_device_info_query',
     'ftk_lstm_cell_f32', 'ftk_lstm_elementwise_f32',
     'ftk_stacked_lstm_workspace_bytes', 'ftk_stacked_lstm_f32', 'ftk_dilated_lstm_f32',
-    'ftk_stacked_lstm_wavefront_f32',
+    'ftk_stacked_lstm_wavefront_f32', 'ftk_lstm_set_products', 'ftk_lstm_get_products',
     'ftk_b2b_gemm_f16', 'ftk_flash_attn_f16', 'ftk_online_softmax_f32',
     'ftk_debug_read_fa_trace',
 )
@@ -188,6 +188,26 @@ def stacked_lstm(xs, WU, bias=None, dilations: Optional[Sequence[int]] = None, s
         _check(lib.ftk_dilated_lstm_f32(_ptr(xs), _ptr(WU), _ptr(bias), dil, _ptr(hsss), _ptr(csss),
                                         ci(L), ci(T), ci(B), ci(H), _ptr(workspace), ws_bytes, _stream()))
     return hsss, csss
+
+
+LSTM_PRODUCTS = {'f32': 0, 'f16x3': 1}
+
+
+def set_lstm_products(mode: str) -> None:
+    """How the persistent stacked-LSTM kernel forms the gate GEMM's products.
+
+    'f32': one fp32 MFMA per product.  'f16x3' (default): each fp32 operand as an fp16 value plus an fp16
+    remainder under a shared power-of-two scale, three fp16 MFMAs per fp32 one, fp32 accumulation; only the
+    remainder-times-remainder term (2^-22 of a product) is dropped.
+    """
+    if mode not in LSTM_PRODUCTS:
+        raise ValueError(f"mode must be one of {sorted(LSTM_PRODUCTS)}, got {mode!r}")
+    _check(lib.ftk_lstm_set_products(ctypes.c_int(LSTM_PRODUCTS[mode])))
+
+
+def get_lstm_products() -> str:
+    code = int(lib.ftk_lstm_get_products())
+    return next(k for k, v in LSTM_PRODUCTS.items() if v == code)
 
 
 def persistent_status(workspace: torch.Tensor) -> int:

@@ -55,12 +55,30 @@ constexpr int P_LD = PK + 4;       // padded activation row in LDS (floats)
 constexpr int PC = 8;              // column slices per layer (32 units each)
 constexpr int kMaxLayers = 64;
 
+// Split products.  v_mfma_f32_32x32x16_f16 moves sixteen k per 8 passes where
+// v_mfma_f32_32x32x2_f32 moves two per 16, so a product of two fp32 numbers is
+// cheaper as three fp16 products than as one fp32 product, if each number is
+// first cut in two: v * 2^e = top + rest / 2^11 with top = fp16(v * 2^e) and
+// rest = fp16((v * 2^e - top) * 2^11).  The cut is exact up to the rounding of
+// rest: 22 significant bits relative to the largest magnitude that shares the
+// scale 2^e (a weight column, an input row, or the fixed 2^14 of h in (-1, 1)),
+// where fp32 keeps 24.  top*top, top*rest and rest*top are accumulated in fp32
+// (the last two in accumulators of their own, folded in with 2^-11 at the end);
+// rest*rest, 2^-22 of the product, is dropped.
+constexpr int kSplitTop = 14;          // a scale group's largest magnitude lands in [2^14, 2^15)
+constexpr float kSplitRest = 2048.0f;  // 2^11: what the remainder is multiplied by before it is rounded
+constexpr float kSplitAct = 16384.0f;  // 2^14: the scale of h
+
 struct PersistArgs {
   const float* xs;
   const float* WU;
   const float* bias;
   float* hsss;
   float* csss;
+  // split-product mode: every activation as two fp16 planes (rounded value, scaled remainder), see below
+  const _Float16* xsp;   // [T][B][2][H] planes of the input rows
+  const float* xratio;   // [T][B] what an input row's products are multiplied by to match the hidden rows' scale
+  _Float16* hsp;         // [L][T][B][2][H] planes of every h
   int* flags;   // [L][T][NRB] completion counts
   int* status;  // [0] = error word
   int L, T, B;
@@ -75,6 +93,7 @@ struct PersistArgs {
 };
 
 typedef unsigned long long u64;
+template <int V> using IC = std::integral_constant<int, V>;
 
 __device__ __forceinline__ int flag_load(const int* flag) {
   return __hip_atomic_load(flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -105,20 +124,55 @@ __device__ __forceinline__ void coherent_store8(float* p, float a, float b) {
   __hip_atomic_store(reinterpret_cast<u64*>(p), v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
-// 16 bytes per lane from global memory straight into LDS at lds_base + 16*lane
-// (lds_base must be wave-uniform), agent scope.
-__device__ __forceinline__ void lds_dma16(const float* gsrc, float* lds_base) {
-  __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)gsrc,
-                                   (__attribute__((address_space(3))) void*)lds_base, 16, 0, /*sc1*/ 16);
+__device__ __forceinline__ void coherent_store8h(_Float16* p, v4h v) {
+  __hip_atomic_store(reinterpret_cast<u64*>(p), __builtin_bit_cast(u64, v), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
+// 16 bytes per lane from global memory (wave-uniform base + per-lane byte
+// offset + OFF) straight into LDS at lds_addr + 16*lane (wave-uniform byte
+// address in LDS).  COHERENT: agent scope; otherwise through the caches, for
+// data no other compute unit writes while it may be cached here.  Written as
+// assembly so that base, LDS address and offset stay in scalar registers and
+// the immediate field: with one wave per SIMD nothing hides the address
+// arithmetic the compiler otherwise spends on every copy.  The compiler does
+// not count these copies as outstanding loads; callers wait with vmcnt(0).
+// (The hardware adds the instruction's immediate offset to the LDS address as
+// well as to the global one, hence the subtraction.)
+template <int OFF, bool COHERENT>
+__device__ __forceinline__ void lds_dma16(const void* gbase, unsigned byte_off, unsigned lds_addr) {
+  lds_addr -= OFF;
+  if constexpr (COHERENT)
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2 offset:%3 sc1"
+                 :: "s"(lds_addr), "v"(byte_off), "s"(gbase), "n"(OFF) : "memory", "m0");
+  else
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2 offset:%3"
+                 :: "s"(lds_addr), "v"(byte_off), "s"(gbase), "n"(OFF) : "memory", "m0");
+}
+// 4 bytes per lane, through the caches: used to touch cache lines ahead of time.
+__device__ __forceinline__ void lds_dma4(const void* gbase, unsigned byte_off, unsigned lds_addr) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, %2"
+               :: "s"(lds_addr), "v"(byte_off), "s"(gbase) : "memory", "m0");
+}
+
+// Activation rows are read through the caches (false) or with agent-scope loads (true).  A row is written
+// once per launch and read only after its completion count has been seen, so a cache can hold a stale
+// copy of it only from before the launch, and those are dropped when the kernel starts.
+constexpr bool kCoherentTiles = false;
+
 constexpr int P_TILE = 32 * P_LD;  // floats per LDS buffer
+// output staging in LDS, per buffer: c and h as [32][32] fp32 with 144-byte rows, the two fp16 planes as
+// [32][32] with 80-byte rows
+constexpr int kStageRow32 = 144, kStageRow16 = 80;
+constexpr int kStageC = 0, kStageH = 32 * kStageRow32, kStageTop = 2 * 32 * kStageRow32, kStageRest = kStageTop + 32 * kStageRow16;
+constexpr int kStageBytes = kStageRest + 32 * kStageRow16;
+constexpr size_t kPersistLds = (size_t)2 * P_TILE * sizeof(float) + 1024 + 2 * kStageBytes;  // tiles, prefetch scrap, staging
 constexpr int FLAG_TARGET = PC * 4;  // one count per wave of each of the 8 column slices
 constexpr int TS = 8;              // trace stamps per item
 
+template <bool SPLIT>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1)))
 void lstm_persistent_kernel(PersistArgs a) {
-  extern __shared__ __attribute__((aligned(16))) float tile[];  // [2][32][P_LD], then 256 floats of scrap
+  extern __shared__ __attribute__((aligned(16))) float tile[];  // [2][32][P_LD], 256 floats of scrap, 2 staging buffers
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -129,6 +183,10 @@ void lstm_persistent_kernel(PersistArgs a) {
   int q = blockIdx.x;
   if (a.xcd_remap) q = (blockIdx.x & 7) * (gridDim.x >> 3) + (blockIdx.x >> 3);
   if (q >= a.groups) return;
+  // The activation rows are read through the caches.  A row is written once per launch and read only after
+  // its completion count has been seen, so a cache can hold a stale copy of it only from before the launch:
+  // drop those here.
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
   if (q == a.trace_q && tid == 0) reinterpret_cast<long long*>(a.status + 16)[0] = wall_clock64();
   const int per_layer = PC * a.pr;
   const int l = q / per_layer;
@@ -141,15 +199,44 @@ void lstm_persistent_kernel(PersistArgs a) {
   const int my_rbs = (a.nrb - prs + a.pr - 1) / a.pr;  // row blocks this workgroup walks per time step
   const int n_items = T * my_rbs;
 
-  // Resident weights: lane (i = j, half hh) of wave w holds, for MFMA step
-  // s = 4q + c, WU[l][k = 8q + 4hh + c][gate(i)*H + 32pc + 8w + i%8].
+  // Resident weights.  fp32 products: lane (i = j, half hh) of wave w holds, for
+  // MFMA step s = 4q + c, WU[l][k = 8q + 4hh + c][gate(i)*H + 32pc + 8w + i%8].
+  // Split products: for MFMA step s the lane holds rows k = 16s + 8hh .. +7 of
+  // the same column, as the fp16 pair described above.
   const int col = (j >> 3) * PH + 32 * pc + 8 * wave + (j & 7);
   const float* wl = a.WU + (size_t)l * PK * PN + col;
-  float wr[PK / 2];
+  float wr[SPLIT ? 1 : PK / 2];
+  v8h whi[SPLIT ? PK / 16 : 1], wlo[SPLIT ? PK / 16 : 1];
+  float ginv[16];  // split products: what accumulator register r is multiplied by to undo the scales
+  if constexpr (!SPLIT) {
 #pragma unroll
-  for (int s = 0; s < PK / 2; ++s) {
-    const int k = 8 * (s >> 2) + 4 * hh + (s & 3);
-    wr[s] = wl[(size_t)k * PN];
+    for (int s = 0; s < PK / 2; ++s) {
+      const int k = 8 * (s >> 2) + 4 * hh + (s & 3);
+      wr[s] = wl[(size_t)k * PN];
+    }
+  } else {
+    // the column's largest magnitude decides its power-of-two scale
+    float cmax = 0.f;
+#pragma unroll
+    for (int s = 0; s < PK / 16; ++s)
+#pragma unroll
+      for (int e = 0; e < 8; ++e) cmax = fmaxf(cmax, fabsf(wl[(size_t)(16 * s + 8 * hh + e) * PN]));
+    cmax = fmaxf(cmax, __shfl_xor(cmax, 32));
+    const int eb = min(max((int)((__float_as_uint(cmax) >> 23) & 0xff), 15), 254);
+    const float wscale = __uint_as_float((unsigned)(127 + kSplitTop + 127 - eb) << 23);  // column max -> [2^14, 2^15)
+    const float winv = __uint_as_float((unsigned)(eb - kSplitTop) << 23);
+    asm volatile("" ::: "memory");  // the second pass loads again instead of keeping 256 values alive
+#pragma unroll
+    for (int s = 0; s < PK / 16; ++s)
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const float w = wl[(size_t)(16 * s + 8 * hh + e) * PN] * wscale;
+        const _Float16 top = (_Float16)w;
+        whi[s][e] = top;
+        wlo[s][e] = (_Float16)((w - (float)top) * kSplitRest);
+      }
+#pragma unroll
+    for (int r = 0; r < 16; ++r) ginv[r] = __shfl(winv, (r & 3) + 8 * (r >> 2) + 4 * hh) * (1.0f / kSplitAct);
   }
   const int u0 = 32 * pc + 8 * wave + 4 * hh;  // first of this lane's 4 units
   float bi[4] = {0, 0, 0, 0}, bf[4] = {0, 0, 0, 0}, bo[4] = {0, 0, 0, 0}, bg[4] = {0, 0, 0, 0};
@@ -170,7 +257,7 @@ void lstm_persistent_kernel(PersistArgs a) {
     st[1] = wall_clock64();  // weights requested (st[0]: kernel entry)
     float sink = 0.f;
 #pragma unroll
-    for (int s2 = 0; s2 < PK / 2; s2 += 32) sink += wr[s2];
+    for (int s2 = 0; s2 < (SPLIT ? PK / 16 : PK / 2); s2 += (SPLIT ? 2 : 32)) sink += SPLIT ? (float)whi[SPLIT ? s2 : 0][0] : wr[SPLIT ? 0 : s2];
     if (sink == 12345.678f) st[3] = 0;
     st[2] = wall_clock64();  // weights (a sample of them) have arrived
   }
@@ -202,21 +289,46 @@ void lstm_persistent_kernel(PersistArgs a) {
   };
   auto flags_ready = [](const Flags& f) { return f.below >= FLAG_TARGET && f.own >= FLAG_TARGET; };
 
+  // Where the activation rows come from.  The two fp16 planes of a row take the
+  // 1024 bytes of its fp32 form, so the tile code is the same for both: in
+  // split mode a tile row is [x top | x rest | h top | h rest], 256 fp16 each.
+  const float* xin = SPLIT ? reinterpret_cast<const float*>(a.xsp) : a.xs;
+  const float* hin = SPLIT ? reinterpret_cast<const float*>(a.hsp) : a.hsss;
+
   // Tile n into LDS buffer buf, global -> LDS directly: wave w moves rows
-  // 8w..8w+7; one instruction carries half a row (256 floats = 64 lanes x 16
-  // bytes, consecutive lanes to consecutive LDS addresses), agent-scope so it
-  // sees what other compute units published.
+  // 8w..8w+7; one instruction carries half a tile row (1024 bytes = 64 lanes x
+  // 16, consecutive lanes to consecutive LDS addresses).
+  const int wave_u = __builtin_amdgcn_readfirstlane(wave);
+  const unsigned lane16 = 16u * lane;
+  const unsigned lane_lines = 1024u * (lane >> 3) + 128u * (lane & 7);  // one lane per cache line of 8 rows
+  const unsigned tile_lds = (unsigned)reinterpret_cast<uintptr_t>((__attribute__((address_space(3))) void*)tile);
   auto issue_tile = [&](int n, int buf) __attribute__((always_inline)) {
     const int t = item_t(n), rb = item_rb(n);
-    const float* xsrc = (l == 0) ? a.xs + (size_t)t * cell : a.hsss + ((size_t)(l - 1) * T + t) * cell;
     const bool has_prev = t >= d;
-    const float* hsrc = a.hsss + ((size_t)l * T + (has_prev ? t - d : 0)) * cell;
-    float* dst = tile + buf * P_TILE + (8 * wave) * P_LD;
+    const char* xsrc = reinterpret_cast<const char*>((l == 0) ? xin + (size_t)t * cell : hin + ((size_t)(l - 1) * T + t) * cell);
+    const char* hsrc = reinterpret_cast<const char*>(hin + ((size_t)l * T + (has_prev ? t - d : 0)) * cell);
+    const int row0 = rb * 32 + 8 * wave_u;
+    const unsigned lds0 = tile_lds + 4u * (unsigned)(buf * P_TILE + 8 * wave_u * P_LD);
+    if (row0 + 8 <= B) {
+      const char* xb = xsrc + (size_t)row0 * 1024;
+      static_for<8>([&](auto rc) __attribute__((always_inline)) {
+        constexpr int r = decltype(rc)::value;
+        lds_dma16<(r & 3) * 1024, kCoherentTiles>(xb + (r >> 2) * 4096, lane16, lds0 + 4u * r * P_LD);
+      });
+      if (has_prev) {
+        const char* hb = hsrc + (size_t)row0 * 1024;
+        static_for<8>([&](auto rc) __attribute__((always_inline)) {
+          constexpr int r = decltype(rc)::value;
+          lds_dma16<(r & 3) * 1024, kCoherentTiles>(hb + (r >> 2) * 4096, lane16, lds0 + 4u * r * P_LD + 1024u);
+        });
+      }
+    } else {  // the batch ends inside these 8 rows: rows past the end repeat the last one
 #pragma unroll
-    for (int r = 0; r < 8; ++r) {
-      const int rg = min(rb * 32 + 8 * wave + r, B - 1);
-      lds_dma16(xsrc + (size_t)rg * PH + 4 * lane, dst + r * P_LD);
-      if (has_prev) lds_dma16(hsrc + (size_t)rg * PH + 4 * lane, dst + r * P_LD + PH);
+      for (int r = 0; r < 8; ++r) {
+        const size_t rg = (size_t)min(row0 + r, B - 1);
+        lds_dma16<0, kCoherentTiles>(xsrc + rg * 1024, lane16, lds0 + 4u * r * P_LD);
+        if (has_prev) lds_dma16<0, kCoherentTiles>(hsrc + rg * 1024, lane16, lds0 + 4u * r * P_LD + 1024u);
+      }
     }
     // The first layer's input rows come from memory nobody has touched; pull the rows of the item after
     // this one towards the cache now, so that their copy into LDS one item later is served from L2 like
@@ -225,10 +337,10 @@ void lstm_persistent_kernel(PersistArgs a) {
     // the data arrives).
     if (l == 0 && n + 1 < n_items) {
       const int t2 = item_t(n + 1), rb2 = item_rb(n + 1);
-      const int rg = min(rb2 * 32 + 8 * wave + (lane >> 3), B - 1);
-      __builtin_amdgcn_global_load_lds(
-          (const __attribute__((address_space(1))) void*)(a.xs + (size_t)t2 * cell + (size_t)rg * PH + 32 * (lane & 7)),
-          (__attribute__((address_space(3))) void*)(tile + 2 * P_TILE + 64 * wave), 4, 0, 0);
+      const int row2 = rb2 * 32 + 8 * wave_u;
+      if (row2 + 8 <= B)
+        lds_dma4(reinterpret_cast<const char*>(xin + (size_t)t2 * cell) + (size_t)row2 * 1024, lane_lines,
+                 tile_lds + 4u * (unsigned)(2 * P_TILE + 64 * wave_u));
     }
   };
   // steps [q0, q1) of the K loop (steps 0..31: x rows of WU, 32..63: h rows)
@@ -256,6 +368,71 @@ void lstm_persistent_kernel(PersistArgs a) {
       __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
     }
   };
+  // the same in split mode: steps 0..15 are the x rows, 16..31 the h rows; a
+  // lane reads its 8 k of both planes and three MFMAs use them
+  auto mfma_split = [&](int buf, auto q0c, auto q1c, v16f& am, v16f& ar0, v16f& ar1) __attribute__((always_inline)) {
+    constexpr int q0 = decltype(q0c)::value;
+    constexpr int q1 = decltype(q1c)::value;
+    const _Float16* arow = reinterpret_cast<const _Float16*>(tile + buf * P_TILE + j * P_LD) + 8 * hh;
+    auto top_of = [&](int qq) { return *reinterpret_cast<const v8h*>(arow + (qq >> 4) * (2 * PH) + 16 * (qq & 15)); };
+    auto rest_of = [&](int qq) { return *reinterpret_cast<const v8h*>(arow + (qq >> 4) * (2 * PH) + PH + 16 * (qq & 15)); };
+    v8h bt = top_of(q0), br = rest_of(q0);
+#pragma unroll
+    for (int qq = q0; qq < q1; ++qq) {
+      v8h btn = bt, brn = br;
+      if (qq + 1 < q1) { btn = top_of(qq + 1); brn = rest_of(qq + 1); }
+      am = __builtin_amdgcn_mfma_f32_32x32x16_f16(whi[qq], bt, am, 0, 0, 0);
+      ar0 = __builtin_amdgcn_mfma_f32_32x32x16_f16(whi[qq], br, ar0, 0, 0, 0);
+      ar1 = __builtin_amdgcn_mfma_f32_32x32x16_f16(wlo[qq], bt, ar1, 0, 0, 0);
+      bt = btn; br = brn;
+    }
+    __builtin_amdgcn_sched_group_barrier(0x100, 4, 0);
+#pragma unroll
+    for (int g4 = q0; g4 < q1; ++g4) {
+      __builtin_amdgcn_sched_group_barrier(0x008, 3, 0);
+      __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+    }
+  };
+  // one interface for both: K steps of the x half [x0, x1) or of the h half, in
+  // units of a sixteenth of a half
+  v16f acc0, acc1, acc2;
+  auto clear_acc = [&]() __attribute__((always_inline)) {
+#pragma unroll
+    for (int r = 0; r < 16; ++r) { acc0[r] = 0.0f; acc1[r] = 0.0f; acc2[r] = 0.0f; }
+  };
+  auto mfma_range = [&](int buf, auto half_c, auto s0c, auto s1c) __attribute__((always_inline)) {
+    constexpr int hf = decltype(half_c)::value, s0 = decltype(s0c)::value, s1 = decltype(s1c)::value;
+    if constexpr (SPLIT)
+      mfma_split(buf, std::integral_constant<int, 16 * hf + s0>{}, std::integral_constant<int, 16 * hf + s1>{}, acc0, acc1, acc2);
+    else
+      mfma_part(buf, std::integral_constant<int, 32 * hf + 2 * s0>{}, std::integral_constant<int, 32 * hf + 2 * s1>{}, acc0, acc1);
+  };
+  // split mode, first layer: the x rows carry a scale of their own; before the h
+  // products join the same accumulators the x products move to h's scale (a
+  // power of two: exact)
+  auto load_ratio = [&](int n) __attribute__((always_inline)) -> float {
+    if constexpr (SPLIT) {
+      if (l == 0) return a.xratio[(size_t)item_t(n) * B + min(item_rb(n) * 32 + j, B - 1)];
+    }
+    return 1.0f;
+  };
+  auto rescale_x = [&](float ratio) __attribute__((always_inline)) {
+    if constexpr (SPLIT) {
+      if (l == 0) {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) { acc0[r] *= ratio; acc1[r] *= ratio; acc2[r] *= ratio; }
+      }
+    }
+  };
+  auto gate_sums = [&]() __attribute__((always_inline)) -> v16f {
+    v16f acc;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      if constexpr (SPLIT) acc[r] = ginv[r] * (acc0[r] + (1.0f / kSplitRest) * (acc1[r] + acc2[r]));
+      else acc[r] = acc0[r] + acc1[r];
+    }
+    return acc;
+  };
   // bias, activations and state update of an item: lane-local and branch-free.
   // piece m (0..15) of the computation: gate (m & 3) of unit (m >> 2); the last
   // gate of a unit finishes its c and h
@@ -276,19 +453,59 @@ void lstm_persistent_kernel(PersistArgs a) {
   auto epilogue_math = [&](const v16f& acc, const float4& cp, float (&hv)[4], float (&cv)[4]) __attribute__((always_inline)) {
     static_for<16>([&](auto mc) __attribute__((always_inline)) { epilogue_piece(acc, cp, hv, cv, mc); });
   };
-  // h leaves through write-through stores, c through the cache
-  auto epilogue = [&](int n, const v16f& acc, const float4& cp) __attribute__((always_inline)) {
+  // The lane that computes (row, 4 units) does not store them: 64 lanes would touch 32 rows, a sliver of a
+  // cache line in each.  The results cross a staging area in LDS instead ([32 rows][this workgroup's 32
+  // units] per output, rows padded against bank conflicts), and after a barrier wave w stores rows
+  // 8w..8w+7: 128 contiguous bytes of c and h per row, 64 of each fp16 plane.
+  unsigned char* const stage = reinterpret_cast<unsigned char*>(tile + 2 * P_TILE + 256);
+  auto epilogue_to_lds = [&](const v16f& acc, const float4& cp, int sbuf) __attribute__((always_inline)) {
     float hv[4], cv[4];
     epilogue_math(acc, cp, hv, cv);
-    const int t = item_t(n), rb = item_rb(n);
-    const int rg = rb * 32 + j;
-    if (alive && rg < B) {
-      float* hdst = a.hsss + ((size_t)l * T + t) * cell + (size_t)rg * PH + u0;
-      float* cdst = a.csss + ((size_t)l * T + t) * cell + (size_t)rg * PH + u0;
-      *reinterpret_cast<float4*>(cdst) = make_float4(cv[0], cv[1], cv[2], cv[3]);
-      coherent_store8(hdst, hv[0], hv[1]);
-      coherent_store8(hdst + 2, hv[2], hv[3]);
+    unsigned char* sb = stage + sbuf * kStageBytes;
+    const int c4 = 8 * wave + 4 * hh;
+    *reinterpret_cast<float4*>(sb + kStageC + j * kStageRow32 + 4 * c4) = make_float4(cv[0], cv[1], cv[2], cv[3]);
+    *reinterpret_cast<float4*>(sb + kStageH + j * kStageRow32 + 4 * c4) = make_float4(hv[0], hv[1], hv[2], hv[3]);
+    if constexpr (SPLIT) {
+      v4h top, rest;
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const float v = hv[r] * kSplitAct;
+        top[r] = (_Float16)v;
+        rest[r] = (_Float16)((v - (float)top[r]) * kSplitRest);
+      }
+      *reinterpret_cast<v4h*>(sb + kStageTop + j * kStageRow16 + 2 * c4) = top;
+      *reinterpret_cast<v4h*>(sb + kStageRest + j * kStageRow16 + 2 * c4) = rest;
     }
+  };
+  // What consumers on other compute units read leaves through write-through stores (fp32 products: h;
+  // split products: the two planes), the rest through the cache.
+  auto store_item = [&](int n, int sbuf) __attribute__((always_inline)) {
+    const int t = item_t(n), rb = item_rb(n);
+    const int rl = 8 * wave + (lane >> 3), cc = lane & 7;
+    const int rg = rb * 32 + rl;
+    if (alive && rg < B) {
+      const unsigned char* sb = stage + sbuf * kStageBytes;
+      const size_t at = ((size_t)l * T + t) * cell + (size_t)rg * PH + 32 * pc + 4 * cc;
+      const float4 cv = *reinterpret_cast<const float4*>(sb + kStageC + rl * kStageRow32 + 16 * cc);
+      const float4 hv = *reinterpret_cast<const float4*>(sb + kStageH + rl * kStageRow32 + 16 * cc);
+      *reinterpret_cast<float4*>(a.csss + at) = cv;
+      if constexpr (SPLIT) {
+        *reinterpret_cast<float4*>(a.hsss + at) = hv;
+        _Float16* pdst = a.hsp + (((size_t)l * T + t) * B + rg) * (2 * PH) + 32 * pc + 4 * cc;
+        coherent_store8h(pdst, *reinterpret_cast<const v4h*>(sb + kStageTop + rl * kStageRow16 + 8 * cc));
+        coherent_store8h(pdst + PH, *reinterpret_cast<const v4h*>(sb + kStageRest + rl * kStageRow16 + 8 * cc));
+      } else {
+        coherent_store8(a.hsss + at, hv.x, hv.y);
+        coherent_store8(a.hsss + at + 2, hv.z, hv.w);
+      }
+    }
+  };
+  // workgroup barrier that waits for nothing by itself: what has to be complete before it is waited for
+  // explicitly (__syncthreads would also wait for the acknowledgement of every store in flight)
+  auto barrier = [&]() __attribute__((always_inline)) {
+    asm volatile("" ::: "memory");
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
   };
   auto load_cprev = [&](int n) __attribute__((always_inline)) -> float4 {
     const int t = item_t(n), rb = item_rb(n);
@@ -308,7 +525,6 @@ void lstm_persistent_kernel(PersistArgs a) {
   };
 
   const bool tracing = (q == a.trace_q) && tid == 0;
-  v16f acc0, acc1;
 
   // How far apart an item and the item that needs it are in this workgroup's
   // own sequence decides the schedule: distance 1 (one row block, dilation 1)
@@ -324,55 +540,61 @@ void lstm_persistent_kernel(PersistArgs a) {
       const float4 cp = load_cprev(n);
       __builtin_amdgcn_s_waitcnt(0);
       __syncthreads();
-#pragma unroll
-      for (int r = 0; r < 16; ++r) { acc0[r] = 0.0f; acc1[r] = 0.0f; }
-      mfma_part(0, std::integral_constant<int, 0>{}, std::integral_constant<int, PH / 8>{}, acc0, acc1);
-      if (item_t(n) >= d) mfma_part(0, std::integral_constant<int, PH / 8>{}, std::integral_constant<int, PK / 8>{}, acc0, acc1);
-      v16f acc;
-#pragma unroll
-      for (int r = 0; r < 16; ++r) acc[r] = acc0[r] + acc1[r];
-      epilogue(n, acc, cp);
+      clear_acc();
+      mfma_range(0, IC<0>{}, IC<0>{}, IC<16>{});
+      rescale_x(load_ratio(n));
+      if (item_t(n) >= d) mfma_range(0, IC<1>{}, IC<0>{}, IC<16>{});
+      epilogue_to_lds(gate_sums(), cp, 0);
+      __syncthreads();  // results staged; the tile may be rewritten by the next item
+      store_item(n, 0);
       publish(n);
-      __syncthreads();  // the tile is rewritten by the next item
       if (tracing) a.trace[TS * n + 7] = wall_clock64();
     }
     return;
   }
 
   // ---- pipelined schedule.  Per item n:
-  //   the first half of the x half of the MFMAs;
-  //   publish item n-1: its h and c went out at the end of item n-1, so by now
-  //     they are acknowledged and the wait costs nothing -- and nothing newer
-  //     is outstanding yet that the wait would also catch;
-  //   request tile n+1 into the other LDS buffer if its producers are seen to
-  //     be done (their counters were requested at the end of item n-1); if
-  //     not, look again after the x half, and wait only after the h half;
-  //   the rest of the x half, the h half;
-  //   wait for tile n+1, one workgroup barrier;
-  //   activations, state update and stores of item n.  (Vector instructions do
-  //   not hide behind fp32 MFMAs on this machine, so nothing is gained by
-  //   deferring them, and the sooner the stores go out the sooner the layer
-  //   above can start: an item is visible to its consumers about 2 us after
-  //   its last MFMA.  That hand-over time, 31 times in a row, is what the
-  //   wavefront pays at the start and at the end of a 32-layer stack.)
+  //   the MFMAs;
+  //   if tile n+1 has not been requested yet: a look at its producers' completion counts (asked for when
+  //     the item began), and the request if they are complete.  The counts of tile n+2 are asked for;
+  //   activations and state update, results into the LDS staging area;
+  //   everything outstanding is waited for (tiles on their way, and the stores of item n-1, which left an
+  //     item ago), item n-1 is counted as complete, barrier: item n's tile buffer is free;
+  //   if tile n+2's producers were complete, the tile is requested now, a whole item ahead; the loads
+  //     item n+1 needs are issued; the stores of item n leave;
+  //   a wave that still has not been able to request its part of tile n+1 waits for the producers now --
+  //     after counting item n itself, which is what the layer above is waiting for while the wavefront
+  //     fills;
+  //   barrier: tile n+1 is complete.
+  // Loads and stores share one counter of outstanding operations and may complete out of order with
+  // respect to each other, so the result of a load is only known to have arrived when nothing at all is
+  // outstanding: a look at completion counts less than about 2 us after an item's stores have left waits
+  // for their acknowledgement.  Hence the order above: what is asked for before the barrier costs no
+  // wait of its own, requests precede the stores in the memory pipeline, and an item that finds its
+  // successor's tile already requested touches no load result until its MFMAs are done.  With split
+  // products an item's MFMAs take less than those 2 us, so the only look inside an item is the one after
+  // them; with fp32 products there is time for a look after every quarter of a half, and the previous
+  // item is counted half way through the x half.
+  constexpr int kFirstLook = SPLIT ? 7 : 0;
   alive = wait_deps(0);
   if (alive) issue_tile(0, 0);
-  Flags fl = (n_items > 1) ? request_flags(1) : Flags{FLAG_TARGET, FLAG_TARGET};
+  float4 cp = load_cprev(0);
+  float ratio = load_ratio(0);
   __builtin_amdgcn_s_waitcnt(0);
   __syncthreads();
 
-  constexpr int QX = PH / 8;   // MFMA steps of the x half
-  constexpr int QE = QX / 2;   // steps before the previous item is published (its stores take about 2 us to be acknowledged)
+  bool counted = true;                 // nothing to count before item 0
+  bool pending = alive && n_items > 1;  // tile n+1 still to be requested
+  Flags fl{0, 0};
   for (int n = 0; n < n_items; ++n) {
     const int buf = n & 1;
     if (tracing) a.trace[TS * n + 0] = wall_clock64();
     const bool has_prev = item_t(n) >= d;
-    const bool more = n + 1 < n_items;
-    bool pending = alive && more;  // tile n+1 still to be requested
-    int looks = 0;                 // looks taken before the request went out (for the trace)
+    int looks = 0;  // looks taken inside the item (for the trace)
+    if (pending) fl = request_flags(n + 1);
 
-    auto look = [&]() __attribute__((always_inline)) {
-      if (pending) {
+    auto look = [&](int point) __attribute__((always_inline)) {
+      if (pending && point >= kFirstLook) {
         ++looks;
         if (flags_ready(fl)) {
           asm volatile("" ::: "memory");
@@ -384,40 +606,93 @@ void lstm_persistent_kernel(PersistArgs a) {
       }
     };
 
-    const float4 cp = load_cprev(n);
-#pragma unroll
-    for (int r = 0; r < 16; ++r) { acc0[r] = 0.0f; acc1[r] = 0.0f; }
-    mfma_part(buf, std::integral_constant<int, 0>{}, std::integral_constant<int, QE>{}, acc0, acc1);
-    if (n > 0) publish(n - 1);
-    look();
+    clear_acc();
+    mfma_range(buf, IC<0>{}, IC<0>{}, IC<4>{});
+    look(0);
+    mfma_range(buf, IC<0>{}, IC<4>{}, IC<8>{});
+    look(1);
+    if (!SPLIT && !counted) { publish(n - 1); counted = true; }
+    mfma_range(buf, IC<0>{}, IC<8>{}, IC<12>{});
+    look(2);
+    mfma_range(buf, IC<0>{}, IC<12>{}, IC<16>{});
+    look(3);
+    rescale_x(ratio);
     if (tracing) a.trace[TS * n + 1] = wall_clock64();
-    mfma_part(buf, std::integral_constant<int, QE>{}, std::integral_constant<int, QX>{}, acc0, acc1);
+    if (has_prev) {
+      mfma_range(buf, IC<1>{}, IC<0>{}, IC<4>{});
+      look(4);
+      mfma_range(buf, IC<1>{}, IC<4>{}, IC<8>{});
+      look(5);
+      mfma_range(buf, IC<1>{}, IC<8>{}, IC<12>{});
+      look(6);
+      mfma_range(buf, IC<1>{}, IC<12>{}, IC<16>{});
+    }
     if (tracing) a.trace[TS * n + 2] = wall_clock64();
-    look();
-    if (tracing) a.trace[TS * n + 3] = wall_clock64();
-    if (has_prev) mfma_part(buf, std::integral_constant<int, QX>{}, std::integral_constant<int, PK / 8>{}, acc0, acc1);
-    if (tracing) a.trace[TS * n + 4] = wall_clock64() | ((long long)(pending ? 7 : looks) << 60);
-    // last resort: wait for the producers here
+    look(7);
+    bool pending2 = alive && n + 2 < n_items;  // tile n+2 still to be requested
+    Flags fl2{0, 0};
+    if (pending2) fl2 = request_flags(n + 2);
+    if (tracing) a.trace[TS * n + 3] = wall_clock64() | ((long long)(pending ? 7 : min(looks, 6)) << 60);
+    epilogue_to_lds(gate_sums(), cp, buf);
+    if (tracing) a.trace[TS * n + 4] = wall_clock64();
+    if (!counted) publish(n - 1);
+    else __builtin_amdgcn_s_waitcnt(0);
+    barrier();
+    if (tracing) a.trace[TS * n + 5] = wall_clock64();
+    if (pending2 && !pending && flags_ready(fl2)) {
+      issue_tile(n + 2, buf);
+      pending2 = false;
+    }
+    if (tracing) a.trace[TS * n + 6] = wall_clock64();
+    if (n + 1 < n_items) {
+      cp = load_cprev(n + 1);
+      ratio = load_ratio(n + 1);
+    }
+    store_item(n, buf);
+    counted = false;
     if (pending) {
+      publish(n);
+      counted = true;
       alive = wait_deps(n + 1);
       if (alive) issue_tile(n + 1, buf ^ 1);
+      __builtin_amdgcn_s_waitcnt(0);
     }
-    if (n + 2 < n_items) fl = request_flags(n + 2);
-    if (tracing) a.trace[TS * n + 5] = wall_clock64();
-    __builtin_amdgcn_s_waitcnt(0);  // tile n+1 has landed in LDS
-    if (tracing) a.trace[TS * n + 6] = wall_clock64();
-    __syncthreads();
-    v16f acc;
-#pragma unroll
-    for (int r = 0; r < 16; ++r) acc[r] = acc0[r] + acc1[r];
-    epilogue(n, acc, cp);
+    barrier();
     if (tracing) a.trace[TS * n + 7] = wall_clock64();
+    pending = pending2 && alive;
+    fl = fl2;
   }
-  publish(n_items - 1);
+  if (!counted) publish(n_items - 1);
 }
 
 __global__ void fill_zero_kernel(int* p, size_t n) {
   for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x) p[i] = 0;
+}
+
+// Split mode, before the persistent kernel: every input row as its two fp16
+// planes, with the row's own power-of-two scale.  One wave per row of 256.
+__global__ __launch_bounds__(256) void lstm_split_rows_kernel(const float* xs, _Float16* xsp, float* xratio, int rows) {
+  const int lane = threadIdx.x & 63;
+  const int row = blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (row >= rows) return;
+  const float4 v = *reinterpret_cast<const float4*>(xs + (size_t)row * PH + 4 * lane);
+  float m = fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w)));
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) m = fmaxf(m, __shfl_xor(m, o));
+  const int eb = min(max((int)((__float_as_uint(m) >> 23) & 0xff), 15), 254);
+  const float scale = __uint_as_float((unsigned)(127 + kSplitTop + 127 - eb) << 23);
+  const float vs[4] = {v.x * scale, v.y * scale, v.z * scale, v.w * scale};
+  v4h top, rest;
+#pragma unroll
+  for (int r = 0; r < 4; ++r) {
+    top[r] = (_Float16)vs[r];
+    rest[r] = (_Float16)((vs[r] - (float)top[r]) * kSplitRest);
+  }
+  _Float16* dst = xsp + (size_t)row * (2 * PH) + 4 * lane;
+  *reinterpret_cast<v4h*>(dst) = top;
+  *reinterpret_cast<v4h*>(dst + PH) = rest;
+  // the row's products carry 2^(141 - eb), h's carry 2^14: the ratio is 2^(eb - 127)
+  if (lane == 0) xratio[row] = __uint_as_float((unsigned)eb << 23);
 }
 
 static size_t flag_count(int L, int T, int B) {
@@ -425,10 +700,29 @@ static size_t flag_count(int L, int T, int B) {
   return (size_t)L * T * nrb;
 }
 
-// Workspace layout: [64 ints: status][flags][trace: T*nrb*8 stamps of 8 bytes].
+// Workspace layout: [64 ints: status][flags][trace: T*nrb*8 stamps of 8 bytes]
+// and, for the split-product mode, [xratio: T*B floats][xsp: T*B rows][hsp: L*T*B rows]
+// of 1024 bytes each, every part on a 256-byte boundary.
 static size_t trace_offset_bytes(int L, int T, int B) { return ((flag_count(L, T, B) + 64) * sizeof(int) + 15) / 16 * 16; }
+static size_t round256(size_t v) { return (v + 255) / 256 * 256; }
+static size_t xratio_offset_bytes(int L, int T, int B) {
+  return round256(trace_offset_bytes(L, T, B) + (size_t)T * ((B + 31) / 32) * 8 * sizeof(long long));
+}
+static size_t xsp_offset_bytes(int L, int T, int B) { return round256(xratio_offset_bytes(L, T, B) + (size_t)T * B * sizeof(float)); }
+static size_t hsp_offset_bytes(int L, int T, int B) { return xsp_offset_bytes(L, T, B) + (size_t)T * B * 2 * PH * sizeof(_Float16); }
 static size_t workspace_need(int L, int T, int B) {
-  return trace_offset_bytes(L, T, B) + (size_t)T * ((B + 31) / 32) * 8 * sizeof(long long);
+  return hsp_offset_bytes(L, T, B) + (size_t)L * T * B * 2 * PH * sizeof(_Float16);
+}
+
+// 0: fp32 products (v_mfma_f32_32x32x2_f32); 1: split products.  FTK_LSTM_PRODUCTS=f32|f16x3
+// sets the initial value, ftk_lstm_set_products() changes it.
+static int g_products = -1;
+static int products_mode() {
+  if (g_products < 0) {
+    const char* e = getenv("FTK_LSTM_PRODUCTS");
+    g_products = (e && (e[0] == 'f' && e[1] == '3')) ? 0 : 1;
+  }
+  return g_products;
 }
 
 // Profiling hook: FTK_LSTM_PLAIN_LAUNCH=1 launches without the cooperative
@@ -462,13 +756,14 @@ static int run_persistent(const float* xs, const float* WU, const float* bias, c
   const DeviceProps* dp = nullptr;
   int rc = device_props(&dp);
   if (rc) return rc;
-  const size_t lds = (size_t)2 * P_TILE * sizeof(float) + 1024;  // two tiles + the prefetch scrap area
+  const size_t lds = kPersistLds;
   if ((int)lds > dp->lds_optin) return FTK_OK;
-  const void* fn = (const void*)lstm_persistent_kernel;
-  static bool attr_set = false;
-  if (!attr_set) {
+  const bool split = products_mode() == 1;
+  const void* fn = split ? (const void*)lstm_persistent_kernel<true> : (const void*)lstm_persistent_kernel<false>;
+  static bool attr_set[2] = {false, false};
+  if (!attr_set[split]) {
     FTK_HIP(hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-    attr_set = true;
+    attr_set[split] = true;
   }
   int per_cu = 0;
   FTK_HIP(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, fn, 256, lds));
@@ -484,6 +779,12 @@ static int run_persistent(const float* xs, const float* WU, const float* bias, c
   a.xs = xs; a.WU = WU; a.bias = bias; a.hsss = hsss; a.csss = csss;
   a.status = reinterpret_cast<int*>(ws);
   a.flags = a.status + 64;
+  char* wsb = reinterpret_cast<char*>(ws);
+  float* xratio = reinterpret_cast<float*>(wsb + xratio_offset_bytes(L, T, B));
+  _Float16* xsp = reinterpret_cast<_Float16*>(wsb + xsp_offset_bytes(L, T, B));
+  a.xratio = xratio;
+  a.xsp = xsp;
+  a.hsp = reinterpret_cast<_Float16*>(wsb + hsp_offset_bytes(L, T, B));
   a.L = L; a.T = T; a.B = B;
   a.nrb = (B + 31) / 32;
   // spare compute units become row slices, but a workgroup keeps at least two
@@ -501,9 +802,17 @@ static int run_persistent(const float* xs, const float* WU, const float* bias, c
   rc = check_launch("fill_zero_kernel");
   if (rc) return rc;
 
+  if (split) {
+    const int rows = T * B;
+    hipLaunchKernelGGL(lstm_split_rows_kernel, dim3((rows + 3) / 4), dim3(256), 0, s, xs, xsp, xratio, rows);
+    rc = check_launch("lstm_split_rows_kernel");
+    if (rc) return rc;
+  }
+
   void* kargs[] = {&a};
   if (plain_launch()) {
-    hipLaunchKernelGGL(lstm_persistent_kernel, dim3(grid), dim3(256), lds, s, a);
+    if (split) hipLaunchKernelGGL(lstm_persistent_kernel<true>, dim3(grid), dim3(256), lds, s, a);
+    else hipLaunchKernelGGL(lstm_persistent_kernel<false>, dim3(grid), dim3(256), lds, s, a);
     rc = check_launch("lstm_persistent_kernel");
     if (rc) return rc;
   } else {
@@ -545,6 +854,15 @@ size_t ftk_stacked_lstm_workspace_bytes(int L, int T, int B, int H) {
   if (L <= 0 || T <= 0 || B <= 0 || H <= 0) return 0;
   return ftk::workspace_need(L, T, B);
 }
+
+int ftk_lstm_set_products(int mode) {
+  if (mode != FTK_LSTM_PRODUCTS_F32 && mode != FTK_LSTM_PRODUCTS_F16X3)
+    return ftk::fail(FTK_ERR_INVALID_ARGUMENT, "ftk_lstm_set_products: mode %d is neither FTK_LSTM_PRODUCTS_F32 nor FTK_LSTM_PRODUCTS_F16X3", mode);
+  ftk::g_products = mode;
+  return FTK_OK;
+}
+
+int ftk_lstm_get_products(void) { return ftk::products_mode(); }
 
 int ftk_stacked_lstm_f32(const float* xs, const float* WU, const float* bias, float* hsss, float* csss, int L, int T,
                          int B, int H, void* workspace, size_t workspace_bytes, ftk_stream_t stream) {

@@ -121,6 +121,23 @@ int ftk_dilated_lstm_f32(const float* xs, const float* WU, const float* bias,
                          size_t workspace_bytes, ftk_stream_t stream);
 
 /*
+ * How the persistent kernel of the two entry points above forms the products
+ * of the gate GEMM.  FTK_LSTM_PRODUCTS_F32: one v_mfma_f32_32x32x2_f32 per
+ * product.  FTK_LSTM_PRODUCTS_F16X3 (the default): every fp32 operand is cut
+ * into an fp16 value and an fp16 remainder under a power-of-two scale shared
+ * by its weight column / activation row, three fp16 MFMAs with fp32
+ * accumulation take the place of the fp32 one and only the remainder x
+ * remainder term (2^-22 of a product) is dropped; inputs, state, outputs and
+ * accumulation stay fp32.  The environment variable FTK_LSTM_PRODUCTS=f32 or
+ * =f16x3 sets the initial mode.  A tuning control of this library: the
+ * reference has one fp32 (cuBLAS) and one fp16 (CuTe) LSTM and no switch.
+ */
+#define FTK_LSTM_PRODUCTS_F32 0
+#define FTK_LSTM_PRODUCTS_F16X3 1
+int ftk_lstm_set_products(int mode);
+int ftk_lstm_get_products(void);
+
+/*
  * The same stack evaluated as one batched fused-cell launch per wavefront
  * diagonal (no persistent kernel, no workspace); any H%32==0.  This is the
  * launch structure of StackedLstmRegion3 (region3.h:50-103) and the fallback

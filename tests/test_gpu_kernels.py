@@ -114,14 +114,24 @@ def test_stacked_lstm_wavefront_launches(core, L, T, B, H, dil):
     assert_lstm_close(hsss, hr, 'hsss'); assert_lstm_close(csss, cr, 'csss')
 
 
+@pytest.fixture(params=['f16x3', 'f32'])
+def products(core, request):
+    """Both ways the persistent kernel forms the gate GEMM's products; the default is restored afterwards."""
+    before = core.get_lstm_products()
+    core.set_lstm_products(request.param)
+    yield request.param
+    core.set_lstm_products(before)
+
+
 @pytest.mark.parametrize('L,T,B,dil,bias', [
     (1, 16, 64, None, False),          # config 1: single layer scan, B 64, T 16, H 256
     (2, 4, 64, None, True),
     (3, 6, 100, None, True),           # ragged batch
+    (2, 5, 17, None, True),            # less than one 32-row block
     (4, 9, 32, [1, 2, 4, 8], True),    # dilated, one 32-row block
     (6, 12, 256, [1, 2, 4, 8, 16, 32], False),  # config 5 layer structure, short sequence
 ])
-def test_stacked_lstm_persistent(core, L, T, B, dil, bias):
+def test_stacked_lstm_persistent(core, products, L, T, B, dil, bias):
     H = 256
     xs, WU, bs = lstm_inputs(5, L, T, B, H, 1.0 / 16, bias)
     ws = torch.empty(core.stacked_lstm_workspace_bytes(L, T, B, H), dtype=torch.uint8, device='cuda')
@@ -131,7 +141,44 @@ def test_stacked_lstm_persistent(core, L, T, B, dil, bias):
     assert_lstm_close(hsss, hr, 'hsss'); assert_lstm_close(csss, cr, 'csss')
 
 
-def test_stacked_lstm_config4_full_size(core):
+def test_split_products_are_as_accurate_as_fp32_products(core):
+    """The three-fp16-products form of the gate GEMM against a float64 evaluation: its error has to stay in
+    the range of the fp32 MFMA's own (a few 1e-7 of the largest value), two orders below the 1e-4 bound,
+    also when rows of the input and columns of the weights differ in magnitude by 1e3 (each row / column
+    carries its own power-of-two scale) and when everything is small or large."""
+    H = 256
+    before = core.get_lstm_products()
+    try:
+        for (L, T, B, dil, xscale, wscale) in [(4, 12, 64, None, 1.0, 1 / 8), (3, 16, 40, [1, 2, 4], 1.0, 1 / 8),
+                                               (2, 6, 32, None, 1e-3, 1 / 8), (2, 6, 33, None, 30.0, 1 / 16)]:
+            rng = np.random.default_rng(7)
+            xs = (rng.standard_normal((T, B, H)) * xscale).astype(np.float32)
+            xs[:, ::3] *= 1e-3
+            WU = (rng.uniform(-wscale, wscale, (L, 2 * H, 4 * H))).astype(np.float32)
+            WU[:, :, ::5] *= 1e-2
+            hr, cr = ko.stacked_lstm(xs, WU, None, dilations=dil)          # float64
+            err = {}
+            for mode in ('f32', 'f16x3'):
+                core.set_lstm_products(mode)
+                ws = torch.empty(core.stacked_lstm_workspace_bytes(L, T, B, H), dtype=torch.uint8, device='cuda')
+                hsss, csss = core.stacked_lstm(dev(xs), dev(WU), dilations=dil, workspace=ws)
+                assert core.persistent_status(ws) == 0
+                err[mode] = max(ko.max_rel_err(hsss.cpu().numpy(), hr), ko.max_rel_err(csss.cpu().numpy(), cr))
+            assert err['f16x3'] <= max(2 * err['f32'], 2e-6), f'{(L, T, B, dil, xscale, wscale)}: {err}'
+            assert err['f16x3'] <= LSTM_TOL / 20, f'{(L, T, B, dil, xscale, wscale)}: {err}'
+    finally:
+        core.set_lstm_products(before)
+
+
+def test_lstm_products_switch(core):
+    assert core.get_lstm_products() in ('f32', 'f16x3')
+    with pytest.raises(ValueError):
+        core.set_lstm_products('bf16')
+    rc = core.lib.ftk_lstm_set_products(7)
+    assert rc == -1 and b'ftk_lstm_set_products' in core.lib.ftk_last_error()
+
+
+def test_stacked_lstm_config4_full_size(core, products):
     """L 32, B 256, T 64, H 256: persistent kernel vs per-stage launches on the GPU, and
     vs the oracle on a subset of batch rows (rows never interact)."""
     L, T, B, H = 32, 64, 256, 256
