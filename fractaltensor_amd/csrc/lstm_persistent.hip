@@ -154,10 +154,10 @@ __device__ __forceinline__ void lds_dma4(const void* gbase, unsigned byte_off, u
                :: "s"(lds_addr), "v"(byte_off), "s"(gbase) : "memory", "m0");
 }
 
-// Activation rows are read through the caches (false) or with agent-scope loads (true).  A row is written
-// once per launch and read only after its completion count has been seen, so a cache can hold a stale
-// copy of it only from before the launch, and those are dropped when the kernel starts.
-constexpr bool kCoherentTiles = false;
+// Activation rows are read with agent-scope loads (true) or through the caches (false).  Through the caches
+// measures the same, and is only safe while every writer of a cache line sits on the reader's side of a
+// non-coherent L2: a partly written line that such a cache fills from memory keeps the other part stale.
+constexpr bool kCoherentTiles = true;
 
 constexpr int P_TILE = 32 * P_LD;  // floats per LDS buffer
 // output staging in LDS, per buffer: c and h as [32][32] fp32 with 144-byte rows, the two fp16 planes as
@@ -183,10 +183,6 @@ void lstm_persistent_kernel(PersistArgs a) {
   int q = blockIdx.x;
   if (a.xcd_remap) q = (blockIdx.x & 7) * (gridDim.x >> 3) + (blockIdx.x >> 3);
   if (q >= a.groups) return;
-  // The activation rows are read through the caches.  A row is written once per launch and read only after
-  // its completion count has been seen, so a cache can hold a stale copy of it only from before the launch:
-  // drop those here.
-  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
   if (q == a.trace_q && tid == 0) reinterpret_cast<long long*>(a.status + 16)[0] = wall_clock64();
   const int per_layer = PC * a.pr;
   const int l = q / per_layer;
@@ -560,8 +556,9 @@ void lstm_persistent_kernel(PersistArgs a) {
   //   activations and state update, results into the LDS staging area;
   //   everything outstanding is waited for (tiles on their way, and the stores of item n-1, which left an
   //     item ago), item n-1 is counted as complete, barrier: item n's tile buffer is free;
-  //   if tile n+2's producers were complete, the tile is requested now, a whole item ahead; the loads
-  //     item n+1 needs are issued; the stores of item n leave;
+  //   the stores of item n leave (first: the sooner they are acknowledged the sooner the item counts);
+  //     the loads item n+1 needs are issued; if tile n+2's producers were complete, the tile is requested
+  //     now, a whole item ahead;
   //   a wave that still has not been able to request its part of tile n+1 waits for the producers now --
   //     after counting item n itself, which is what the layer above is waiting for while the wavefront
   //     fills;
@@ -570,8 +567,8 @@ void lstm_persistent_kernel(PersistArgs a) {
   // respect to each other, so the result of a load is only known to have arrived when nothing at all is
   // outstanding: a look at completion counts less than about 2 us after an item's stores have left waits
   // for their acknowledgement.  Hence the order above: what is asked for before the barrier costs no
-  // wait of its own, requests precede the stores in the memory pipeline, and an item that finds its
-  // successor's tile already requested touches no load result until its MFMAs are done.  With split
+  // wait of its own, and an item that finds its successor's tile already requested touches no load
+  // result until its MFMAs are done.  With split
   // products an item's MFMAs take less than those 2 us, so the only look inside an item is the one after
   // them; with fp32 products there is time for a look after every quarter of a half, and the previous
   // item is counted half way through the x half.
@@ -639,17 +636,17 @@ void lstm_persistent_kernel(PersistArgs a) {
     else __builtin_amdgcn_s_waitcnt(0);
     barrier();
     if (tracing) a.trace[TS * n + 5] = wall_clock64();
-    if (pending2 && !pending && flags_ready(fl2)) {
-      issue_tile(n + 2, buf);
-      pending2 = false;
-    }
+    store_item(n, buf);
+    counted = false;
     if (tracing) a.trace[TS * n + 6] = wall_clock64();
     if (n + 1 < n_items) {
       cp = load_cprev(n + 1);
       ratio = load_ratio(n + 1);
     }
-    store_item(n, buf);
-    counted = false;
+    if (pending2 && !pending && flags_ready(fl2)) {
+      issue_tile(n + 2, buf);
+      pending2 = false;
+    }
     if (pending) {
       publish(n);
       counted = true;
