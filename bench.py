@@ -210,9 +210,18 @@ def bench_lstm(torch, core, steps, warmup, cpu, dilated):
     cs = torch.empty_like(hs)
     ws = torch.empty(core.stacked_lstm_workspace_bytes(L, T, B, H), dtype=torch.uint8, device='cuda')
     fused = lambda: core.stacked_lstm(xs, WU, dilations=dil, out=(hs, cs), workspace=ws)
+    products = core.get_lstm_products()          # 'f16x3' unless FTK_LSTM_PRODUCTS says otherwise
     ms, wall = _events_ms(torch, fused, steps, warmup)
     status = core.persistent_status(ws)
     ref_h = hs.clone()
+    # the same launch with the other way of forming the gate GEMM's products
+    other = 'f32' if products == 'f16x3' else 'f16x3'
+    core.set_lstm_products(other)
+    ms_other, _ = _events_ms(torch, fused, max(2, steps // 2), 1)
+    other_diff = float((hs - ref_h).abs().max() / ref_h.abs().max())
+    core.set_lstm_products(products)
+    executed = 3.0 * flop if products == 'f16x3' else flop      # MFMA flops the kernel issues
+    peak = PEAK_F16_TFLOPS if products == 'f16x3' else PEAK_F32_MATRIX_TFLOPS
 
     # per-stage launches of the fused cell (no persistent kernel)
     ms_wave, _ = _events_ms(torch, lambda: core.stacked_lstm(xs, WU, dilations=dil, out=(hs, cs), schedule='wavefront'),
@@ -232,10 +241,13 @@ def bench_lstm(torch, core, steps, warmup, cpu, dilated):
 
     res = {
         'metric': 'stacked-LSTM sequences/s', 'value': B / ms * 1e3, 'unit': 'sequences/s', 'ms_per_step': ms,
-        'dtype': 'f32',
+        'dtype': 'f32 (gate products as three f16 MFMAs of split operands, f32 accumulate)' if products == 'f16x3' else 'f32',
         'config': {'workload': name, 'layers': L, 'batch': B, 'seq_len': T, 'hidden': H,
-                   'dilations': dil, 'outputs': 'h and c of every layer at every step'},
+                   'dilations': dil, 'outputs': 'h and c of every layer at every step', 'products': products},
         'tflops': flop / ms / 1e9,
+        'frac_of_f32_matrix_peak_algorithmic': flop / ms / 1e9 / PEAK_F32_MATRIX_TFLOPS,
+        'other_products': {'products': other, 'ms_per_step': ms_other, 'sequences_per_s': B / ms_other * 1e3,
+                           'max_rel_diff_vs_default': other_diff},
         'persistent_status': status,
         'per_stage_launches': {'ms_per_step': ms_wave, 'sequences_per_s': B / ms_wave * 1e3},
         'unfused_gpu_baseline': {'ms_per_step_hip_graph': ms_graph, 'ms_per_step_eager': ms_eager,
@@ -246,8 +258,10 @@ def bench_lstm(torch, core, steps, warmup, cpu, dilated):
                                          'elementwise kernel per step, layer-major; speedup_of_fused is against '
                                          'the HIP-graph replay of that sequence (no launch overhead), '
                                          'speedup_of_fused_vs_eager against its eager launches'},
-        'roofline': {'bound': 'mfma', 'achieved': flop / ms / 1e9, 'peak': PEAK_F32_MATRIX_TFLOPS, 'unit': 'TFLOP/s',
-                     'frac': flop / ms / 1e9 / PEAK_F32_MATRIX_TFLOPS,
+        # executed MFMA flops (three f16 products per algorithmic product in the default mode) against the
+        # peak of the MFMA type that executes them
+        'roofline': {'bound': 'mfma', 'achieved': executed / ms / 1e9, 'peak': peak, 'unit': 'TFLOP/s',
+                     'frac': executed / ms / 1e9 / peak,
                      'traffic': MEASURED_TRAFFIC_BYTES.get('lstm_persistent_kernel'), 'kernel': 'lstm_persistent_kernel'},
     }
     if cpu:
