@@ -193,7 +193,7 @@ def _unfused_lstm_baseline(torch, core, xs, WU, hs, cs, dil=None):
     return forward, graph
 
 
-def bench_lstm(torch, core, steps, warmup, cpu, dilated):
+def bench_lstm(torch, core, steps, warmup, cpu, dilated, baselines=True):
     if dilated:
         L, T, B, H = 6, 128, 256, 256
         dil = [1, 2, 4, 8, 16, 32]
@@ -214,30 +214,44 @@ def bench_lstm(torch, core, steps, warmup, cpu, dilated):
     ms, wall = _events_ms(torch, fused, steps, warmup)
     status = core.persistent_status(ws)
     ref_h = hs.clone()
-    # the same launch with the other way of forming the gate GEMM's products
-    other = 'f32' if products == 'f16x3' else 'f16x3'
-    core.set_lstm_products(other)
-    ms_other, _ = _events_ms(torch, fused, max(2, steps // 2), 1)
-    other_diff = float((hs - ref_h).abs().max() / ref_h.abs().max())
-    core.set_lstm_products(products)
     executed = 3.0 * flop if products == 'f16x3' else flop      # MFMA flops the kernel issues
     peak = PEAK_F16_TFLOPS if products == 'f16x3' else PEAK_F32_MATRIX_TFLOPS
-
-    # per-stage launches of the fused cell (no persistent kernel)
-    ms_wave, _ = _events_ms(torch, lambda: core.stacked_lstm(xs, WU, dilations=dil, out=(hs, cs), schedule='wavefront'),
-                            max(2, steps // 4), 1)
-    # unfused GPU baseline
-    hs_b = torch.empty_like(hs)
-    cs_b = torch.empty_like(cs)
-    eager, graph = _unfused_lstm_baseline(torch, core, xs, WU, hs_b, cs_b, dil)
-    nb = max(2, steps // 4)
-    ms_eager, _ = _events_ms(torch, eager, nb, 1)
-    ms_graph = None
-    if graph is not None:
-        hs_b.zero_()
-        ms_graph, _ = _events_ms(torch, graph.replay, nb, 2)
-    base_err = float((hs_b - ref_h).abs().max() / ref_h.abs().max())
-    ms_base = ms_graph if ms_graph is not None else ms_eager
+    extra = {}
+    if baselines:
+        # the same launch with the other way of forming the gate GEMM's products
+        other = 'f32' if products == 'f16x3' else 'f16x3'
+        core.set_lstm_products(other)
+        ms_other, _ = _events_ms(torch, fused, max(2, steps // 2), 1)
+        other_diff = float((hs - ref_h).abs().max() / ref_h.abs().max())
+        core.set_lstm_products(products)
+        # per-stage launches of the fused cell (no persistent kernel)
+        ms_wave, _ = _events_ms(torch, lambda: core.stacked_lstm(xs, WU, dilations=dil, out=(hs, cs), schedule='wavefront'),
+                                max(2, steps // 4), 1)
+        # unfused GPU baseline
+        hs_b = torch.empty_like(hs)
+        cs_b = torch.empty_like(cs)
+        eager, graph = _unfused_lstm_baseline(torch, core, xs, WU, hs_b, cs_b, dil)
+        nb = max(2, steps // 4)
+        ms_eager, _ = _events_ms(torch, eager, nb, 1)
+        ms_graph = None
+        if graph is not None:
+            hs_b.zero_()
+            ms_graph, _ = _events_ms(torch, graph.replay, nb, 2)
+        base_err = float((hs_b - ref_h).abs().max() / ref_h.abs().max())
+        ms_base = ms_graph if ms_graph is not None else ms_eager
+        extra = {
+            'other_products': {'products': other, 'ms_per_step': ms_other, 'sequences_per_s': B / ms_other * 1e3,
+                               'max_rel_diff_vs_default': other_diff},
+            'per_stage_launches': {'ms_per_step': ms_wave, 'sequences_per_s': B / ms_wave * 1e3},
+            'unfused_gpu_baseline': {'ms_per_step_hip_graph': ms_graph, 'ms_per_step_eager': ms_eager,
+                                     'sequences_per_s': B / ms_base * 1e3, 'speedup_of_fused': ms_base / ms,
+                                     'speedup_of_fused_vs_eager': ms_eager / ms,
+                                     'max_rel_diff_vs_fused': base_err,
+                                     'what': 'one x@W GEMM per layer + per-step h@U GEMM (torch/rocBLAS) + one '
+                                             'elementwise kernel per step, layer-major; speedup_of_fused is against '
+                                             'the HIP-graph replay of that sequence (no launch overhead), '
+                                             'speedup_of_fused_vs_eager against its eager launches'},
+        }
 
     res = {
         'metric': 'stacked-LSTM sequences/s', 'value': B / ms * 1e3, 'unit': 'sequences/s', 'ms_per_step': ms,
@@ -246,24 +260,15 @@ def bench_lstm(torch, core, steps, warmup, cpu, dilated):
                    'dilations': dil, 'outputs': 'h and c of every layer at every step', 'products': products},
         'tflops': flop / ms / 1e9,
         'frac_of_f32_matrix_peak_algorithmic': flop / ms / 1e9 / PEAK_F32_MATRIX_TFLOPS,
-        'other_products': {'products': other, 'ms_per_step': ms_other, 'sequences_per_s': B / ms_other * 1e3,
-                           'max_rel_diff_vs_default': other_diff},
         'persistent_status': status,
-        'per_stage_launches': {'ms_per_step': ms_wave, 'sequences_per_s': B / ms_wave * 1e3},
-        'unfused_gpu_baseline': {'ms_per_step_hip_graph': ms_graph, 'ms_per_step_eager': ms_eager,
-                                 'sequences_per_s': B / ms_base * 1e3, 'speedup_of_fused': ms_base / ms,
-                                 'speedup_of_fused_vs_eager': ms_eager / ms,
-                                 'max_rel_diff_vs_fused': base_err,
-                                 'what': 'one x@W GEMM per layer + per-step h@U GEMM (torch/rocBLAS) + one '
-                                         'elementwise kernel per step, layer-major; speedup_of_fused is against '
-                                         'the HIP-graph replay of that sequence (no launch overhead), '
-                                         'speedup_of_fused_vs_eager against its eager launches'},
         # executed MFMA flops (three f16 products per algorithmic product in the default mode) against the
         # peak of the MFMA type that executes them
         'roofline': {'bound': 'mfma', 'achieved': executed / ms / 1e9, 'peak': peak, 'unit': 'TFLOP/s',
                      'frac': executed / ms / 1e9 / peak,
-                     'traffic': MEASURED_TRAFFIC_BYTES.get('lstm_persistent_kernel'), 'kernel': 'lstm_persistent_kernel'},
+                     'traffic': MEASURED_TRAFFIC_BYTES.get('lstm_persistent_kernel' + ('_dilated' if dilated else '')),
+                     'kernel': 'lstm_persistent_kernel'},
     }
+    res.update(extra)
     if cpu:
         from oracle import c_oracle
         Ls, Ts, Bs = (8, 64, 256) if not dilated else (6, 32, 256)
@@ -289,6 +294,8 @@ def main():
     ap.add_argument('--workload', default='b2b', choices=['b2b', 'attention', 'stacked_lstm', 'dilated_lstm', 'copy'])
     ap.add_argument('--no-extras', action='store_true', help='measure only the chosen workload')
     ap.add_argument('--no-cpu', action='store_true', help='skip the CPU baseline leg')
+    ap.add_argument('--no-baselines', action='store_true',
+                    help='LSTM workloads: only the fused kernel (no unfused GPU baseline, per-stage launches, other product mode)')
     args = ap.parse_args()
     if args.gpus != 1:
         print('bench.py measures one GPU: every workload here is a single-device kernel '
@@ -306,8 +313,8 @@ def main():
     runners = {
         'b2b': lambda s, w, c: bench_b2b(torch, core, s, w, c),
         'attention': lambda s, w, c: bench_attention(torch, core, s, w, c),
-        'stacked_lstm': lambda s, w, c: bench_lstm(torch, core, max(3, s // 5), max(1, w // 5), c, False),
-        'dilated_lstm': lambda s, w, c: bench_lstm(torch, core, max(3, s // 5), max(1, w // 5), c, True),
+        'stacked_lstm': lambda s, w, c: bench_lstm(torch, core, max(3, s // 5), max(1, w // 5), c, False, not args.no_baselines),
+        'dilated_lstm': lambda s, w, c: bench_lstm(torch, core, max(3, s // 5), max(1, w // 5), c, True, not args.no_baselines),
     }
     if args.workload == 'copy':
         runners = {'copy': lambda s, w, c: bench_copy(torch, core, s, w, c)}
