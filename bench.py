@@ -239,7 +239,15 @@ def bench_lstm(torch, core, steps, warmup, cpu, dilated, baselines=True):
             ms_graph, _ = _events_ms(torch, graph.replay, nb, 2)
         base_err = float((hs_b - ref_h).abs().max() / ref_h.abs().max())
         ms_base = ms_graph if ms_graph is not None else ms_eager
+        # the same stack on a ragged batch: row lengths fall linearly from T to T/4 across the (sorted) batch
+        lens = [max(1, T - (3 * T * b) // (4 * B)) for b in range(B)]
+        active = [sum(1 for v in lens if v > t) for t in range(T)]
+        ms_ragged, _ = _events_ms(torch, lambda: core.stacked_lstm(xs, WU, dilations=dil, out=(hs, cs), workspace=ws,
+                                                                   active_rows=active), max(2, steps // 2), 1)
+        live_blocks = sum((a + 31) // 32 for a in active) / float(T * ((B + 31) // 32))
         extra = {
+            'ragged_batch': {'ms_per_step': ms_ragged, 'row_lengths': f'{lens[0]} .. {lens[-1]}, linear over the sorted batch',
+                             'live_fraction_of_row_blocks': live_blocks, 'time_vs_dense': ms_ragged / ms},
             'other_products': {'products': other, 'ms_per_step': ms_other, 'sequences_per_s': B / ms_other * 1e3,
                                'max_rel_diff_vs_default': other_diff},
             'per_stage_launches': {'ms_per_step': ms_wave, 'sequences_per_s': B / ms_wave * 1e3},

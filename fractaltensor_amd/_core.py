@@ -20,7 +20,7 @@ EXPORTS = (
     'ftk_version', 'ftk_last_error', 'ftk_device_info_query',
     'ftk_lstm_cell_f32', 'ftk_lstm_elementwise_f32',
     'ftk_stacked_lstm_workspace_bytes', 'ftk_stacked_lstm_f32', 'ftk_dilated_lstm_f32',
-    'ftk_stacked_lstm_wavefront_f32', 'ftk_lstm_set_products', 'ftk_lstm_get_products',
+    'ftk_stacked_lstm_wavefront_f32', 'ftk_stacked_lstm_ragged_f32', 'ftk_lstm_set_products', 'ftk_lstm_get_products',
     'ftk_b2b_gemm_f16', 'ftk_flash_attn_f16', 'ftk_online_softmax_f32',
     'ftk_debug_read_fa_trace',
 )
@@ -145,11 +145,14 @@ def stacked_lstm_workspace_bytes(L: int, T: int, B: int, H: int) -> int:
 
 def stacked_lstm(xs, WU, bias=None, dilations: Optional[Sequence[int]] = None, schedule: str = 'auto',
                  out: Optional[Tuple[torch.Tensor, torch.Tensor]] = None,
-                 workspace: Optional[torch.Tensor] = None) -> Tuple[torch.Tensor, torch.Tensor]:
+                 workspace: Optional[torch.Tensor] = None,
+                 active_rows: Optional[Sequence[int]] = None) -> Tuple[torch.Tensor, torch.Tensor]:
     """xs [T,B,H], WU [L,2H,4H], bias [L,4H] or None -> hsss, csss [L,T,B,H].
 
     schedule: 'auto' (persistent kernel when the shape allows, else per-stage
     launches) or 'wavefront' (always per-stage launches).
+    active_rows: for a ragged time-major batch (rows sorted by decreasing length), the number of rows still
+    running at each step; only the live (t, row) places of the outputs are defined then.
     """
     f32 = torch.float32
     _req(xs, f32, 'xs'); _req(WU, f32, 'WU')
@@ -181,7 +184,13 @@ def stacked_lstm(xs, WU, bias=None, dilations: Optional[Sequence[int]] = None, s
     if workspace is None:
         workspace = torch.empty(need, dtype=torch.uint8, device=xs.device)
     ws_bytes = ctypes.c_size_t(workspace.numel() * workspace.element_size())
-    if dil is None:
+    if active_rows is not None:
+        if len(active_rows) != T:
+            raise ValueError('active_rows must have one entry per step')
+        act = (ctypes.c_int * T)(*[int(v) for v in active_rows])
+        _check(lib.ftk_stacked_lstm_ragged_f32(_ptr(xs), _ptr(WU), _ptr(bias), dil, act, _ptr(hsss), _ptr(csss),
+                                               ci(L), ci(T), ci(B), ci(H), _ptr(workspace), ws_bytes, _stream()))
+    elif dil is None:
         _check(lib.ftk_stacked_lstm_f32(_ptr(xs), _ptr(WU), _ptr(bias), _ptr(hsss), _ptr(csss),
                                         ci(L), ci(T), ci(B), ci(H), _ptr(workspace), ws_bytes, _stream()))
     else:

@@ -54,6 +54,7 @@ constexpr int PN = 4 * PH;         // gate columns
 constexpr int P_LD = PK + 4;       // padded activation row in LDS (floats)
 constexpr int PC = 8;              // column slices per layer (32 units each)
 constexpr int kMaxLayers = 64;
+constexpr int kMaxBlocks = 64;     // 32-row blocks a ragged batch may have (B <= 2048)
 
 // Split products.  v_mfma_f32_32x32x16_f16 moves sixteen k per 8 passes where
 // v_mfma_f32_32x32x2_f32 moves two per 16, so a product of two fp32 numbers is
@@ -90,6 +91,8 @@ struct PersistArgs {
   int trace_q;            // logical workgroup whose item timeline is recorded, or -1
   long long* trace;       // [items][8] 100 MHz clock stamps of that workgroup
   int dil[kMaxLayers];
+  int ragged;                // 1: row block rb takes part in steps t < steps_of[rb] only
+  int steps_of[kMaxBlocks];
 };
 
 typedef unsigned long long u64;
@@ -260,12 +263,17 @@ void lstm_persistent_kernel(PersistArgs a) {
 
   auto item_t = [&](int n) { return n / my_rbs; };
   auto item_rb = [&](int n) { return prs + a.pr * (n % my_rbs); };
+  // Ragged batches (rows sorted by length, so a row block simply stops after its longest row): an item
+  // past its block's last step is walked through like any other, but requests, computes, stores and counts
+  // nothing; nothing that is computed depends on it.
+  auto live = [&](int n) { return !a.ragged || item_t(n) < a.steps_of[item_rb(n)]; };
   auto flag_of = [&](int ll, int t, int rb) { return a.flags + ((size_t)ll * T + t) * a.nrb + rb; };
 
   // inputs of item n complete?  Bounded spin on the two counters.
   auto wait_deps = [&](int n) __attribute__((always_inline)) -> bool {
     const int t = item_t(n), rb = item_rb(n);
     bool ok = true;
+    if (!live(n)) return true;
     if (l > 0) ok = wait_count(flag_of(l - 1, t, rb), FLAG_TARGET, a.status, a.spin_limit);
     if (ok && t >= d) ok = wait_count(flag_of(l, t - d, rb), FLAG_TARGET, a.status, a.spin_limit);
     // The data loads must stay behind the flag reads.  The hardware issues and
@@ -279,6 +287,7 @@ void lstm_persistent_kernel(PersistArgs a) {
   auto request_flags = [&](int n) __attribute__((always_inline)) -> Flags {
     Flags f{FLAG_TARGET, FLAG_TARGET};
     const int t = item_t(n), rb = item_rb(n);
+    if (!live(n)) return f;
     if (l > 0) f.below = flag_load(flag_of(l - 1, t, rb));
     if (t >= d) f.own = flag_load(flag_of(l, t - d, rb));
     return f;
@@ -300,6 +309,7 @@ void lstm_persistent_kernel(PersistArgs a) {
   const unsigned tile_lds = (unsigned)reinterpret_cast<uintptr_t>((__attribute__((address_space(3))) void*)tile);
   auto issue_tile = [&](int n, int buf) __attribute__((always_inline)) {
     const int t = item_t(n), rb = item_rb(n);
+    if (!live(n)) return;
     const bool has_prev = t >= d;
     const char* xsrc = reinterpret_cast<const char*>((l == 0) ? xin + (size_t)t * cell : hin + ((size_t)(l - 1) * T + t) * cell);
     const char* hsrc = reinterpret_cast<const char*>(hin + ((size_t)l * T + (has_prev ? t - d : 0)) * cell);
@@ -331,7 +341,7 @@ void lstm_persistent_kernel(PersistArgs a) {
     // the other layers' rows.  One 4-byte-per-lane copy touches all 64 cache lines of the wave's 8 rows;
     // it lands in a scrap area behind the tiles (a load into registers would need them reserved until
     // the data arrives).
-    if (l == 0 && n + 1 < n_items) {
+    if (l == 0 && n + 1 < n_items && live(n + 1)) {
       const int t2 = item_t(n + 1), rb2 = item_rb(n + 1);
       const int row2 = rb2 * 32 + 8 * wave_u;
       if (row2 + 8 <= B)
@@ -408,7 +418,7 @@ void lstm_persistent_kernel(PersistArgs a) {
   // power of two: exact)
   auto load_ratio = [&](int n) __attribute__((always_inline)) -> float {
     if constexpr (SPLIT) {
-      if (l == 0) return a.xratio[(size_t)item_t(n) * B + min(item_rb(n) * 32 + j, B - 1)];
+      if (l == 0 && live(n)) return a.xratio[(size_t)item_t(n) * B + min(item_rb(n) * 32 + j, B - 1)];
     }
     return 1.0f;
   };
@@ -479,7 +489,7 @@ void lstm_persistent_kernel(PersistArgs a) {
     const int t = item_t(n), rb = item_rb(n);
     const int rl = 8 * wave + (lane >> 3), cc = lane & 7;
     const int rg = rb * 32 + rl;
-    if (alive && rg < B) {
+    if (alive && rg < B && live(n)) {
       const unsigned char* sb = stage + sbuf * kStageBytes;
       const size_t at = ((size_t)l * T + t) * cell + (size_t)rg * PH + 32 * pc + 4 * cc;
       const float4 cv = *reinterpret_cast<const float4*>(sb + kStageC + rl * kStageRow32 + 16 * cc);
@@ -506,7 +516,7 @@ void lstm_persistent_kernel(PersistArgs a) {
   auto load_cprev = [&](int n) __attribute__((always_inline)) -> float4 {
     const int t = item_t(n), rb = item_rb(n);
     float4 cp = make_float4(0.f, 0.f, 0.f, 0.f);
-    if (alive && t >= d) {
+    if (alive && t >= d && live(n)) {
       const int rgc = min(rb * 32 + j, B - 1);
       cp = *reinterpret_cast<const float4*>(a.csss + ((size_t)l * T + (t - d)) * cell + (size_t)rgc * PH + u0);
     }
@@ -516,7 +526,7 @@ void lstm_persistent_kernel(PersistArgs a) {
   auto publish = [&](int n) __attribute__((always_inline)) {
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
     __builtin_amdgcn_s_waitcnt(0);
-    if (lane == 0 && alive)
+    if (lane == 0 && alive && live(n))
       __hip_atomic_fetch_add(flag_of(l, item_t(n), item_rb(n)), 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   };
 
@@ -536,11 +546,13 @@ void lstm_persistent_kernel(PersistArgs a) {
       const float4 cp = load_cprev(n);
       __builtin_amdgcn_s_waitcnt(0);
       __syncthreads();
-      clear_acc();
-      mfma_range(0, IC<0>{}, IC<0>{}, IC<16>{});
-      rescale_x(load_ratio(n));
-      if (item_t(n) >= d) mfma_range(0, IC<1>{}, IC<0>{}, IC<16>{});
-      epilogue_to_lds(gate_sums(), cp, 0);
+      if (live(n)) {
+        clear_acc();
+        mfma_range(0, IC<0>{}, IC<0>{}, IC<16>{});
+        rescale_x(load_ratio(n));
+        if (item_t(n) >= d) mfma_range(0, IC<1>{}, IC<0>{}, IC<16>{});
+        epilogue_to_lds(gate_sums(), cp, 0);
+      }
       __syncthreads();  // results staged; the tile may be rewritten by the next item
       store_item(n, 0);
       publish(n);
@@ -603,26 +615,29 @@ void lstm_persistent_kernel(PersistArgs a) {
       }
     };
 
-    clear_acc();
-    mfma_range(buf, IC<0>{}, IC<0>{}, IC<4>{});
-    look(0);
-    mfma_range(buf, IC<0>{}, IC<4>{}, IC<8>{});
-    look(1);
-    if (!SPLIT && !counted) { publish(n - 1); counted = true; }
-    mfma_range(buf, IC<0>{}, IC<8>{}, IC<12>{});
-    look(2);
-    mfma_range(buf, IC<0>{}, IC<12>{}, IC<16>{});
-    look(3);
-    rescale_x(ratio);
-    if (tracing) a.trace[TS * n + 1] = wall_clock64();
-    if (has_prev) {
-      mfma_range(buf, IC<1>{}, IC<0>{}, IC<4>{});
-      look(4);
-      mfma_range(buf, IC<1>{}, IC<4>{}, IC<8>{});
-      look(5);
-      mfma_range(buf, IC<1>{}, IC<8>{}, IC<12>{});
-      look(6);
-      mfma_range(buf, IC<1>{}, IC<12>{}, IC<16>{});
+    const bool on = live(n);
+    if (on) {
+      clear_acc();
+      mfma_range(buf, IC<0>{}, IC<0>{}, IC<4>{});
+      look(0);
+      mfma_range(buf, IC<0>{}, IC<4>{}, IC<8>{});
+      look(1);
+      if (!SPLIT && !counted) { publish(n - 1); counted = true; }
+      mfma_range(buf, IC<0>{}, IC<8>{}, IC<12>{});
+      look(2);
+      mfma_range(buf, IC<0>{}, IC<12>{}, IC<16>{});
+      look(3);
+      rescale_x(ratio);
+      if (tracing) a.trace[TS * n + 1] = wall_clock64();
+      if (has_prev) {
+        mfma_range(buf, IC<1>{}, IC<0>{}, IC<4>{});
+        look(4);
+        mfma_range(buf, IC<1>{}, IC<4>{}, IC<8>{});
+        look(5);
+        mfma_range(buf, IC<1>{}, IC<8>{}, IC<12>{});
+        look(6);
+        mfma_range(buf, IC<1>{}, IC<12>{}, IC<16>{});
+      }
     }
     if (tracing) a.trace[TS * n + 2] = wall_clock64();
     look(7);
@@ -630,7 +645,7 @@ void lstm_persistent_kernel(PersistArgs a) {
     Flags fl2{0, 0};
     if (pending2) fl2 = request_flags(n + 2);
     if (tracing) a.trace[TS * n + 3] = wall_clock64() | ((long long)(pending ? 7 : min(looks, 6)) << 60);
-    epilogue_to_lds(gate_sums(), cp, buf);
+    if (on) epilogue_to_lds(gate_sums(), cp, buf);
     if (tracing) a.trace[TS * n + 4] = wall_clock64();
     if (!counted) publish(n - 1);
     else __builtin_amdgcn_s_waitcnt(0);
@@ -746,8 +761,8 @@ static int trace_workgroup() {
   return v;
 }
 
-static int run_persistent(const float* xs, const float* WU, const float* bias, const int* dil, float* hsss,
-                          float* csss, int L, int T, int B, void* ws, size_t ws_bytes, hipStream_t s,
+static int run_persistent(const float* xs, const float* WU, const float* bias, const int* dil, const int* active,
+                          float* hsss, float* csss, int L, int T, int B, void* ws, size_t ws_bytes, hipStream_t s,
                           bool* handled) {
   *handled = false;
   const DeviceProps* dp = nullptr;
@@ -792,6 +807,17 @@ static int run_persistent(const float* xs, const float* WU, const float* bias, c
   a.trace_q = trace_workgroup();
   a.trace = reinterpret_cast<long long*>(reinterpret_cast<char*>(ws) + trace_offset_bytes(L, T, B));
   for (int l = 0; l < kMaxLayers; ++l) a.dil[l] = (l < L && dil) ? dil[l] : 1;
+  // ragged batch: how many steps each 32-row block takes part in (its first row is its longest).  Batches
+  // with more blocks than the table holds are computed in full, which gives the same live rows.
+  a.ragged = (active && a.nrb <= kMaxBlocks) ? 1 : 0;
+  for (int rb = 0; rb < kMaxBlocks; ++rb) {
+    int steps = T;
+    if (a.ragged) {
+      steps = 0;
+      while (steps < T && active[steps] > 32 * rb) ++steps;
+    }
+    a.steps_of[rb] = steps;
+  }
   const int grid = a.groups;
   a.xcd_remap = (grid % 8 == 0) ? 1 : 0;
 
@@ -831,13 +857,22 @@ static int check_stack_args(const char* who, const float* xs, const float* WU, f
 }
 
 static int run_stack(const char* who, const float* xs, const float* WU, const float* bias, const int* dil,
-                     float* hsss, float* csss, int L, int T, int B, int H, void* ws, size_t ws_bytes,
-                     hipStream_t s) {
+                     const int* active, float* hsss, float* csss, int L, int T, int B, int H, void* ws,
+                     size_t ws_bytes, hipStream_t s) {
   int rc = check_stack_args(who, xs, WU, hsss, csss, L, T, B, H, dil);
   if (rc) return rc;
+  if (active) {
+    for (int t = 0; t < T; ++t) {
+      if (active[t] < 0 || active[t] > B)
+        return fail(FTK_ERR_INVALID_ARGUMENT, "%s: active_rows[%d]=%d is outside [0, B=%d]", who, t, active[t], B);
+      if (t > 0 && active[t] > active[t - 1])
+        return fail(FTK_ERR_INVALID_ARGUMENT, "%s: active_rows must be non-increasing (rows sorted by length), but [%d]=%d > [%d]=%d",
+                    who, t, active[t], t - 1, active[t - 1]);
+    }
+  }
   if (H == PH) {
     bool handled = false;
-    rc = run_persistent(xs, WU, bias, dil, hsss, csss, L, T, B, ws, ws_bytes, s, &handled);
+    rc = run_persistent(xs, WU, bias, dil, active, hsss, csss, L, T, B, ws, ws_bytes, s, &handled);
     if (rc || handled) return rc;
   }
   return run_wavefront(xs, WU, bias, dil, hsss, csss, L, T, B, H, s);
@@ -863,7 +898,7 @@ int ftk_lstm_get_products(void) { return ftk::products_mode(); }
 
 int ftk_stacked_lstm_f32(const float* xs, const float* WU, const float* bias, float* hsss, float* csss, int L, int T,
                          int B, int H, void* workspace, size_t workspace_bytes, ftk_stream_t stream) {
-  return ftk::run_stack("ftk_stacked_lstm_f32", xs, WU, bias, nullptr, hsss, csss, L, T, B, H, workspace,
+  return ftk::run_stack("ftk_stacked_lstm_f32", xs, WU, bias, nullptr, nullptr, hsss, csss, L, T, B, H, workspace,
                         workspace_bytes, (hipStream_t)stream);
 }
 
@@ -871,8 +906,16 @@ int ftk_dilated_lstm_f32(const float* xs, const float* WU, const float* bias, co
                          float* csss, int L, int T, int B, int H, void* workspace, size_t workspace_bytes,
                          ftk_stream_t stream) {
   if (!dilations) return ftk::fail(FTK_ERR_INVALID_ARGUMENT, "ftk_dilated_lstm_f32: dilations is NULL");
-  return ftk::run_stack("ftk_dilated_lstm_f32", xs, WU, bias, dilations, hsss, csss, L, T, B, H, workspace,
+  return ftk::run_stack("ftk_dilated_lstm_f32", xs, WU, bias, dilations, nullptr, hsss, csss, L, T, B, H, workspace,
                         workspace_bytes, (hipStream_t)stream);
+}
+
+int ftk_stacked_lstm_ragged_f32(const float* xs, const float* WU, const float* bias, const int* dilations,
+                                const int* active_rows, float* hsss, float* csss, int L, int T, int B, int H,
+                                void* workspace, size_t workspace_bytes, ftk_stream_t stream) {
+  if (!active_rows) return ftk::fail(FTK_ERR_INVALID_ARGUMENT, "ftk_stacked_lstm_ragged_f32: active_rows is NULL");
+  return ftk::run_stack("ftk_stacked_lstm_ragged_f32", xs, WU, bias, dilations, active_rows, hsss, csss, L, T, B, H,
+                        workspace, workspace_bytes, (hipStream_t)stream);
 }
 
 }  // extern "C"

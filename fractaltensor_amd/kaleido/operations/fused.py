@@ -107,7 +107,9 @@ def _run_stack(xss, Wss, Uss, bss, dilations, return_all_layers):
     core = _core()
     xs, sizes = pad_time_major(xss)
     WU, bias = pack_lstm_weights(Wss, Uss, bss)
-    hsss, csss = core.stacked_lstm(xs.float(), WU.float(), None if bias is None else bias.float(), dilations=dilations)
+    # a ragged batch goes down with its per-step row counts: 32-row blocks that have ended are skipped
+    hsss, csss = core.stacked_lstm(xs.float(), WU.float(), None if bias is None else bias.float(), dilations=dilations,
+                                   active_rows=sizes)
     L = WU.shape[0]
     if return_all_layers:
         if sizes is None:

@@ -121,6 +121,25 @@ int ftk_dilated_lstm_f32(const float* xs, const float* WU, const float* bias,
                          size_t workspace_bytes, ftk_stream_t stream);
 
 /*
+ * The same for a ragged batch in the time-major layout: rows sorted by
+ * decreasing length, active_rows[t] (a HOST array of T ints, non-increasing,
+ * each in [0,B]) = how many leading rows are still running at step t.  xs is
+ * the dense [T,B,H] array with anything finite (zeros) in the dead places;
+ * hsss/csss are written for the live (t, row) pairs, what the other places
+ * hold afterwards is unspecified.  32-row blocks that have ended are skipped
+ * by the persistent kernel; the per-stage fallback computes everything.
+ * dilations: host array or NULL (all 1).  Replaces the shrinking batch of
+ * batched_cell (examples/stacked_rnn/stacked_rnn.py:45-51, hs_prev[0:xs.length])
+ * over the layout of gen_dataset_time_major (examples/utils/data_utils.py:42-66).
+ */
+int ftk_stacked_lstm_ragged_f32(const float* xs, const float* WU,
+                                const float* bias, const int* dilations,
+                                const int* active_rows, float* hsss,
+                                float* csss, int L, int T, int B, int H,
+                                void* workspace, size_t workspace_bytes,
+                                ftk_stream_t stream);
+
+/*
  * How the persistent kernel of the two entry points above forms the products
  * of the gate GEMM.  FTK_LSTM_PRODUCTS_F32: one v_mfma_f32_32x32x2_f32 per
  * product.  FTK_LSTM_PRODUCTS_F16X3 (the default): every fp32 operand is cut

@@ -170,6 +170,49 @@ def test_split_products_are_as_accurate_as_fp32_products(core):
         core.set_lstm_products(before)
 
 
+@pytest.mark.parametrize('L,T,B,dil,lengths', [
+    (3, 12, 100, None, 'linear'),              # lengths fall from T to 1 across the batch: blocks end one after another
+    (2, 9, 64, None, 'two'),                   # half the rows stop after 4 steps
+    (4, 16, 96, [1, 2, 4, 8], 'linear'),       # dilated stack
+    (2, 6, 40, None, 'full'),                  # nothing ragged about it: same as the dense entry point
+])
+def test_stacked_lstm_ragged_rows(core, products, L, T, B, dil, lengths):
+    """Rows sorted by decreasing length; every live (t, row) place equals the oracle's result for that row's own
+    sequence (rows never interact), whatever happens in the dead places."""
+    H = 256
+    xs, WU, bs = lstm_inputs(9, L, T, B, H, 1.0 / 16)
+    if lengths == 'linear':
+        lens = np.maximum(1, T - (np.arange(B) * T) // B)
+    elif lengths == 'two':
+        lens = np.where(np.arange(B) < B // 2, T, 4)
+    else:
+        lens = np.full(B, T)
+    active = [int((lens > t).sum()) for t in range(T)]
+    for b in range(B):
+        xs[lens[b]:, b] = 0.0                                    # padding
+    ws = torch.empty(core.stacked_lstm_workspace_bytes(L, T, B, H), dtype=torch.uint8, device='cuda')
+    hsss, csss = core.stacked_lstm(dev(xs), dev(WU), dev(bs), dilations=dil, workspace=ws, active_rows=active)
+    assert core.persistent_status(ws) == 0, 'a dependency wait timed out'
+    hr, cr = c_oracle.stacked_lstm(xs, WU, bs, dil)              # dense: live places do not depend on dead ones
+    live = torch.from_numpy(np.arange(T)[:, None] < lens[None, :])          # [T, B]
+    got_h = hsss.cpu()[:, live].numpy(); got_c = csss.cpu()[:, live].numpy()
+    assert_lstm_close(torch.from_numpy(got_h), hr[:, live.numpy()], 'hsss live places')
+    assert_lstm_close(torch.from_numpy(got_c), cr[:, live.numpy()], 'csss live places')
+
+
+def test_stacked_lstm_ragged_rejects_unsorted_rows(core):
+    H, L, T, B = 256, 1, 4, 32
+    xs = torch.zeros((T, B, H), device='cuda'); WU = torch.zeros((L, 2 * H, 4 * H), device='cuda')
+    with pytest.raises(core.FtkError) as e:
+        core.stacked_lstm(xs, WU, active_rows=[32, 16, 24, 8])   # grows at step 2
+    assert e.value.code == -1 and 'non-increasing' in str(e.value)
+    with pytest.raises(core.FtkError) as e:
+        core.stacked_lstm(xs, WU, active_rows=[33, 16, 8, 8])    # more rows than the batch has
+    assert e.value.code == -1
+    with pytest.raises(ValueError):
+        core.stacked_lstm(xs, WU, active_rows=[32, 16])
+
+
 def test_lstm_products_switch(core):
     assert core.get_lstm_products() in ('f32', 'f16x3')
     with pytest.raises(ValueError):
