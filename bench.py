@@ -151,6 +151,33 @@ def bench_attention(torch, core, steps, warmup, cpu):
     return res
 
 
+def bench_embedding(torch, core, steps, warmup, cpu):
+    """Embedding rows for a batch of word ids (the step that feeds the LSTM): V 5000 as in
+    examples/stacked_rnn/rnn_utils.py, E 256 to match the LSTM configurations, 1 Mi ids."""
+    V, E, n = 5000, 256, 1 << 20
+    gen = torch.Generator(device='cpu').manual_seed(1234)
+    table = torch.randn((V, E), generator=gen).cuda()
+    ids = torch.randint(0, V, (n,), generator=gen).cuda()
+    out = torch.empty((n, E), device='cuda')
+    ms, wall = _events_ms(torch, lambda: core.embedding_gather(table, ids, out=out, check=False), steps, warmup)
+    nbytes = 4.0 * n * E + 8.0 * n + 4.0 * V * E          # rows written once, ids and the table read once
+    res = {
+        'metric': 'embedding rows/s', 'value': n / ms * 1e3, 'unit': 'rows/s', 'ms_per_step': ms, 'dtype': 'f32',
+        'config': {'workload': 'embedding gather feeding the LSTM (rnn_utils.py:81-90)', 'vocab': V, 'width': E, 'ids': n},
+        'roofline': {'bound': 'hbm', 'achieved': nbytes / ms / 1e6, 'peak': PEAK_HBM_GBS, 'unit': 'GB/s',
+                     'frac': nbytes / ms / 1e6 / PEAK_HBM_GBS, 'traffic': None, 'kernel': 'embedding_gather_kernel',
+                     'algorithmic_bytes_per_launch': nbytes},
+    }
+    if cpu:
+        t, i = table.cpu(), ids.cpu()
+        t0 = time.perf_counter()
+        _ = t[i]
+        dt = time.perf_counter() - t0
+        res['cpu_baseline'] = {'value': n / dt, 'unit': 'rows/s', 'cores': torch.get_num_threads(), 'kind': 'port',
+                               'sample': f'torch index_select of the same {n} ids on the host, {dt:.2f} s'}
+    return res
+
+
 def _unfused_lstm_baseline(torch, core, xs, WU, hs, cs, dil=None):
     """Per-step GEMM (rocBLAS/hipBLASLt through torch) + one elementwise kernel, layer-major:
     the structure of benchmarks/rnn/fractaltensor/stacked_lstm (utils.h:559-625).  Returns a
@@ -299,7 +326,7 @@ def main():
     ap.add_argument('--gpus', type=int, default=1)
     ap.add_argument('--steps', type=int, default=50)
     ap.add_argument('--warmup', type=int, default=10)
-    ap.add_argument('--workload', default='b2b', choices=['b2b', 'attention', 'stacked_lstm', 'dilated_lstm', 'copy'])
+    ap.add_argument('--workload', default='b2b', choices=['b2b', 'attention', 'stacked_lstm', 'dilated_lstm', 'embedding', 'copy'])
     ap.add_argument('--no-extras', action='store_true', help='measure only the chosen workload')
     ap.add_argument('--no-cpu', action='store_true', help='skip the CPU baseline leg')
     ap.add_argument('--no-baselines', action='store_true',
@@ -323,6 +350,7 @@ def main():
         'attention': lambda s, w, c: bench_attention(torch, core, s, w, c),
         'stacked_lstm': lambda s, w, c: bench_lstm(torch, core, max(3, s // 5), max(1, w // 5), c, False, not args.no_baselines),
         'dilated_lstm': lambda s, w, c: bench_lstm(torch, core, max(3, s // 5), max(1, w // 5), c, True, not args.no_baselines),
+        'embedding': lambda s, w, c: bench_embedding(torch, core, s, w, c),
     }
     if args.workload == 'copy':
         runners = {'copy': lambda s, w, c: bench_copy(torch, core, s, w, c)}

@@ -21,7 +21,7 @@ EXPORTS = (
     'ftk_lstm_cell_f32', 'ftk_lstm_elementwise_f32',
     'ftk_stacked_lstm_workspace_bytes', 'ftk_stacked_lstm_f32', 'ftk_dilated_lstm_f32',
     'ftk_stacked_lstm_wavefront_f32', 'ftk_stacked_lstm_ragged_f32', 'ftk_lstm_set_products', 'ftk_lstm_get_products',
-    'ftk_b2b_gemm_f16', 'ftk_flash_attn_f16', 'ftk_online_softmax_f32',
+    'ftk_b2b_gemm_f16', 'ftk_flash_attn_f16', 'ftk_online_softmax_f32', 'ftk_embedding_gather_f32',
     'ftk_debug_read_fa_trace',
 )
 
@@ -271,6 +271,38 @@ def read_fa_trace(tiles: int):
     buf = (ctypes.c_longlong * (tiles * 6))()
     _check(lib.ftk_debug_read_fa_trace(buf, ctypes.c_int(tiles * 6)))
     return np.frombuffer(buf, dtype=np.int64).reshape(tiles, 6).astype(np.float64) / 100.0
+
+
+def embedding_gather(table: torch.Tensor, ids: torch.Tensor, out: Optional[torch.Tensor] = None,
+                     check: bool = True) -> torch.Tensor:
+    """table [V,E] fp32, ids int32/int64 of any shape -> [*ids.shape, E]: rows of the table.
+
+    check=True reads back the count of ids outside [0,V) (one synchronising copy of 4 bytes) and raises
+    IndexError like indexing a FractalTensor does; check=False leaves such rows zero-filled."""
+    _req(table, torch.float32, 'table')
+    if ids.dtype not in (torch.int32, torch.int64):
+        raise TypeError(f'ids must be int32 or int64, got {ids.dtype}')
+    if not ids.is_cuda or not ids.is_contiguous():
+        raise RuntimeError('ids must be a contiguous CUDA tensor')
+    if table.dim() != 2:
+        raise ValueError('table must be [V, E]')
+    V, E = table.shape
+    n = ids.numel()
+    if out is None:
+        out = torch.empty((*ids.shape, E), dtype=torch.float32, device=table.device)
+    else:
+        _req(out, torch.float32, 'out')
+        if out.numel() != n * E:
+            raise ValueError('out must hold ids.numel() * E elements')
+    if n == 0:
+        return out
+    bad = torch.zeros(1, dtype=torch.int32, device=table.device) if check else None
+    _check(lib.ftk_embedding_gather_f32(_ptr(table), _ptr(ids), ctypes.c_int(1 if ids.dtype == torch.int64 else 0),
+                                        _ptr(out), ctypes.c_longlong(n), ctypes.c_int(V), ctypes.c_int(E),
+                                        _ptr(bad), _stream()))
+    if check and int(bad.item()) != 0:
+        raise IndexError(f'{int(bad.item())} ids are outside [0, {V})')
+    return out
 
 
 def online_softmax(x) -> torch.Tensor:

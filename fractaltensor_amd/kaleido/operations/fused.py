@@ -21,9 +21,10 @@ import torch
 
 from ..fractal_tensor import FractalTensor
 from ..tensor import Tensor
+from ..types import FractalTensorStorage, TensorStorage, torch_type_to_internal_type
 
 __all__ = ['pack_lstm_weights', 'pad_time_major', 'unpad_time_major', 'stacked_lstm', 'dilated_lstm', 'lstm_cell', 'flash_attention', 'b2b_gemm',
-           'online_softmax']
+           'online_softmax', 'embedding_lookup']
 
 
 def _core():
@@ -206,3 +207,34 @@ def b2b_gemm(a, b, c):
 def online_softmax(x: Tensor) -> Tensor:
     """Row softmax of a [rows, cols] fp32 Tensor through the online (max, sum) kernel."""
     return Tensor.from_tensor(_core().online_softmax(x.data.contiguous()))
+
+
+def embedding_lookup(embedding: Tensor, words: FractalTensor) -> FractalTensor:
+    """Rows of `embedding` [V, E] for every word id of `words`: what
+    ops.map(lambda ws: ops.map(lambda word: ops.index(ops.slices(embedding, dim=0), word), ws), words)
+    builds (examples/stacked_rnn/rnn_utils.py:81-90), as one gather.  `words` is a FractalTensor of any depth
+    (regular or ragged) of single integers; the result has its structure with [1, E] elements.  An id outside
+    [0, V) raises IndexError, as indexing the sliced matrix does."""
+    if not isinstance(words, FractalTensor):
+        raise TypeError('words should be a FractalTensor.')
+    if not isinstance(embedding, Tensor):
+        raise TypeError('embedding should be a Tensor.')
+    table = embedding.data
+    if table.dim() != 2:
+        raise ValueError('embedding should be a [V, E] matrix.')
+    if words.element_size != 1:
+        raise ValueError('words should hold single integers.')
+    ids = words._T
+    if ids is None or words.indices is None:
+        raise RuntimeError('FractalTensor is not initialized.')
+    if not table.is_cuda or not ids.is_cuda:
+        raise RuntimeError('embedding_lookup runs on the GPU only; move the embedding and the words there.')
+    V, E = table.shape
+    out = _core().embedding_gather(table.contiguous().float(), ids.reshape(-1).contiguous())
+    typ = TensorStorage((1, E), torch_type_to_internal_type(out.dtype), device=out.device.type)
+    for _ in range(words.depth - 1):
+        typ = FractalTensorStorage(typ)
+    ft = FractalTensor(typ)
+    ft.indices = words.indices
+    ft._T = out.reshape(-1)
+    return ft

@@ -167,6 +167,20 @@ int ftk_stacked_lstm_wavefront_f32(const float* xs, const float* WU,
                                    float* hsss, float* csss, int L, int T,
                                    int B, int H, ftk_stream_t stream);
 
+/*
+ * Embedding lookup, the step that feeds the LSTM in the reference's RNN
+ * programs: out[i, :] = table[ids[i], :] for i < n.  table [V,E] fp32, ids [n]
+ * int32 (ids_are_64bit = 0) or int64 (1) on the device, out [n,E]; E%4==0.
+ * An id outside [0,V) zero-fills its row and adds 1 to *bad_ids (a device int
+ * the caller has zeroed, or NULL) instead of reading out of bounds; the Python
+ * side turns a non-zero count into the IndexError the reference raises.
+ * Replaces ops.map(lambda word: ops.index(ops.slices(embedding, dim=0), word), ws)
+ * (examples/stacked_rnn/rnn_utils.py:81-90; Index, access.py:36-58).
+ */
+int ftk_embedding_gather_f32(const float* table, const void* ids,
+                             int ids_are_64bit, float* out, long long n, int V,
+                             int E, int* bad_ids, ftk_stream_t stream);
+
 /* ------------------------------------------------------------ B2B GEMM -- */
 
 /*

@@ -43,6 +43,9 @@ def test_argument_errors_come_back_as_codes_not_crashes():
     assert lib.ftk_flash_attn_f16(one, one, one, one, ci(1), ci(1), ci(64), ci(64), ci(48), ctypes.c_float(1), nul) == -2
     assert lib.ftk_online_softmax_f32(nul, one, ci(1), ci(1), nul) == -1
     assert lib.ftk_stacked_lstm_wavefront_f32(one, one, nul, nul, one, one, ci(1), ci(1), ci(1), ci(48), nul) == -2
+    assert lib.ftk_embedding_gather_f32(one, one, ci(0), one, ctypes.c_longlong(4), ci(8), ci(6), nul, nul) == -2
+    assert lib.ftk_embedding_gather_f32(one, nul, ci(0), one, ctypes.c_longlong(4), ci(8), ci(8), nul, nul) == -1
+    assert lib.ftk_stacked_lstm_ragged_f32(one, one, nul, nul, nul, one, one, ci(1), ci(1), ci(1), ci(32), nul, ctypes.c_size_t(0), nul) == -1
     assert lib.ftk_stacked_lstm_workspace_bytes(32, 64, 256, 256) > 0
     assert lib.ftk_stacked_lstm_workspace_bytes(0, 64, 256, 256) == 0
 

@@ -137,3 +137,54 @@ def test_fused_paths_reject_batches_that_are_not_time_major():
     deep = FractalTensor.from_fractaltensors(growing, growing)   # depth 3, ragged
     with pytest.raises(ValueError, match='ragged'):
         ops.fused.flash_attention(deep, deep, deep)
+
+
+def _ragged_words(lengths, vocab, seed, device):
+    """Time-major batch of word ids for length-sorted sequences: step t holds one id per sequence that is
+    still running (the layout of gen_dataset_time_major, examples/utils/data_utils.py:42-66)."""
+    rng = np.random.default_rng(seed)
+    steps = []
+    for t in range(max(lengths)):
+        b = sum(1 for v in lengths if v > t)
+        ids = torch.from_numpy(rng.integers(0, vocab, size=(b, 1)).astype(np.int64)).to(device)
+        steps.append(FractalTensor.from_dense(ids, 1))
+    return FractalTensor.from_fractaltensors(*steps)
+
+
+def test_fused_embedding_lookup_equals_the_nested_map_program():
+    V, E = 50, 64
+    g = torch.Generator().manual_seed(3)
+    embedding = Tensor.from_tensor(torch.randn((V, E), generator=g).cuda())
+    words = _ragged_words([5, 4, 4, 2, 1], V, seed=4, device='cuda')
+    fused = ops.fused.embedding_lookup(embedding, words)
+    # the reference program: rnn_utils.py:85-90
+    eager = ops.map(lambda ws: ops.map(lambda word: ops.index(ops.slices(embedding, dim=0), word), ws), words)
+    assert fused.depth == eager.depth == 2 and fused.element_shape == (1, E)
+    assert [len(s) for s in fused] == [len(s) for s in eager] == [5, 4, 3, 3, 1]      # rows still running per step
+    for fs, es in zip(fused, eager):
+        for f, e in zip(fs, es):
+            assert torch.equal(f.data, e.data)       # a gather moves bits, nothing is computed
+    with pytest.raises(IndexError):
+        bad = FractalTensor.from_dense(torch.tensor([[3], [V]], device='cuda'), 1)
+        ops.fused.embedding_lookup(embedding, bad)
+    with pytest.raises(RuntimeError):
+        ops.fused.embedding_lookup(Tensor.from_tensor(embedding.data.cpu()), words)
+
+
+def test_embedding_lookup_feeds_the_fused_stacked_lstm():
+    """Words -> embedding rows -> stacked LSTM, all on the GPU, against the oracle on the same ids."""
+    V, H, L = 40, 256, 2
+    lengths = [6, 6, 5, 3, 3, 2]
+    g = torch.Generator().manual_seed(5)
+    table = torch.randn((V, H), generator=g)
+    embedding = Tensor.from_tensor(table.cuda())
+    words = _ragged_words(lengths, V, seed=6, device='cuda')
+    Wss, Uss, bss = programs.make_lstm_params(L, H, 1 / 16, seed=7, device='cuda')
+    hss = ops.fused.stacked_lstm(ops.fused.embedding_lookup(embedding, words), Wss, Uss, bss)
+    WU, bias = _np_params(Wss, Uss, bss)
+    ids = [[int(w.data.item()) for w in step] for step in words]
+    for b, n in enumerate(lengths):
+        xs = np.stack([table[ids[t][b]].numpy() for t in range(n)])[:, None, :]      # [n, 1, H]
+        ref, _ = ko.stacked_lstm(xs, WU, bias)
+        got = np.stack([hss[t][b].data.cpu().numpy().reshape(H) for t in range(n)])
+        assert ko.max_rel_err(got, ref[-1][:, 0]) <= 1e-4

@@ -399,3 +399,30 @@ def test_online_softmax(core, cols):
     np.testing.assert_allclose(y, ref, rtol=2e-5, atol=1e-7)
     np.testing.assert_allclose(y.sum(-1), 1.0, atol=1e-5)
     np.testing.assert_allclose(y, c_oracle.online_softmax(x), rtol=2e-5, atol=1e-7)
+
+
+# ------------------------------------------------------------ embedding gather
+
+@pytest.mark.parametrize('n,V,E,dtype', [(1, 7, 4, torch.int32), (1000, 5000, 64, torch.int64),   # rnn_utils.py: 5000 x 64
+                                         (777, 33, 256, torch.int32), (64 * 256, 5000, 256, torch.int64),
+                                         (1001, 90, 48, torch.int64), (5, 9, 2048, torch.int32)])   # widths off the power-of-two path
+def test_embedding_gather(core, n, V, E, dtype):
+    g = torch.Generator().manual_seed(11)
+    table = torch.randn((V, E), generator=g)
+    ids = torch.randint(0, V, (n,), generator=g).to(dtype)
+    out = core.embedding_gather(table.cuda(), ids.cuda())
+    assert torch.equal(out.cpu(), table[ids.long()])            # moved bits: exact
+
+
+def test_embedding_gather_counts_bad_ids_and_reads_nothing_out_of_bounds(core):
+    table = torch.arange(12, dtype=torch.float32).reshape(3, 4).cuda()
+    ids = torch.tensor([0, 3, -1, 2], dtype=torch.int64).cuda()
+    with pytest.raises(IndexError):
+        core.embedding_gather(table, ids)
+    out = core.embedding_gather(table, ids, check=False)
+    assert torch.equal(out.cpu(), torch.stack([table[0].cpu(), torch.zeros(4), torch.zeros(4), table[2].cpu()]))
+    with pytest.raises(core.FtkError) as e:
+        core.embedding_gather(torch.zeros((3, 6), device='cuda'), ids)     # E not a multiple of 4
+    assert e.value.code == -2
+    with pytest.raises(TypeError):
+        core.embedding_gather(table, ids.float())
