@@ -106,9 +106,11 @@ def test_lstm_elementwise(core):
     (3, 5, 40, 64, None),
     (3, 9, 33, 32, [1, 2, 4]),
     (2, 4, 64, 256, None),
+    (2, 3, 40, 512, None),             # the larger hidden sizes of the reference's sweep (stacked_lstm.cu:185-187):
+    (2, 3, 33, 1024, [1, 2]),          # weights streamed through LDS, one launch per wavefront stage
 ])
 def test_stacked_lstm_wavefront_launches(core, L, T, B, H, dil):
-    xs, WU, bs = lstm_inputs(21, L, T, B, H, 0.1)
+    xs, WU, bs = lstm_inputs(21, L, T, B, H, 0.1 if H <= 256 else 1.0 / 32)   # keeps the gate sums O(1) at any K
     hsss, csss = core.stacked_lstm(dev(xs), dev(WU), dev(bs), dilations=dil, schedule='wavefront')
     hr, cr = ko.stacked_lstm(xs, WU, bs, dilations=dil)
     assert_lstm_close(hsss, hr, 'hsss'); assert_lstm_close(csss, cr, 'csss')
@@ -239,6 +241,17 @@ def test_stacked_lstm_config4_full_size(core, products):
     # second call reuses nothing stale: same answer
     h3, _ = core.stacked_lstm(dx, dW)
     assert torch.equal(h1, h3)
+
+
+@pytest.mark.parametrize('H', [512, 1024])
+def test_stacked_lstm_larger_hidden_sizes_through_the_default_entry(core, H):
+    """H != 256 is not what the persistent kernel is specialised for: the default entry point falls back to
+    per-stage launches of the streaming cell kernel and must give the same answer."""
+    L, T, B = 2, 4, 48
+    xs, WU, bs = lstm_inputs(31, L, T, B, H, 1.0 / 32)
+    hsss, csss = core.stacked_lstm(dev(xs), dev(WU), dev(bs))
+    hr, cr = c_oracle.stacked_lstm(xs, WU, bs, None)
+    assert_lstm_close(hsss, hr, 'hsss'); assert_lstm_close(csss, cr, 'csss')
 
 
 def test_stacked_lstm_rejects_bad_arguments(core):
