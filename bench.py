@@ -165,7 +165,8 @@ def bench_embedding(torch, core, steps, warmup, cpu):
         'metric': 'embedding rows/s', 'value': n / ms * 1e3, 'unit': 'rows/s', 'ms_per_step': ms, 'dtype': 'f32',
         'config': {'workload': 'embedding gather feeding the LSTM (rnn_utils.py:81-90)', 'vocab': V, 'width': E, 'ids': n},
         'roofline': {'bound': 'hbm', 'achieved': nbytes / ms / 1e6, 'peak': PEAK_HBM_GBS, 'unit': 'GB/s',
-                     'frac': nbytes / ms / 1e6 / PEAK_HBM_GBS, 'traffic': None, 'kernel': 'embedding_gather_kernel',
+                     'frac': nbytes / ms / 1e6 / PEAK_HBM_GBS, 'traffic': MEASURED_TRAFFIC_BYTES.get('embedding_gather_pow2_kernel'),
+                     'kernel': 'embedding_gather_pow2_kernel',
                      'algorithmic_bytes_per_launch': nbytes},
     }
     if cpu:
