@@ -457,12 +457,22 @@ __global__ __launch_bounds__(WAVES * 64, MINB) void flash_attn_kernel(const _Flo
   // the barrier that ends this one.
   auto step = [&](int kt, auto next_c, auto mask_c) __attribute__((always_inline)) {
     stamp(kt, 0);
-    if (kt + 2 < ntiles) copy_k_all(Kb + kfree, kt + 2);
-    if (kt + 1 < ntiles) copy_v_all(Vb + vnext, kt + 1);
+    // A wave is held at issue while its copy instructions queue up in the memory pipeline.  With two waves
+    // per SIMD the two take turns: the first issues its copies when the step begins, the second after the
+    // first half tile, so that one of them always has MFMAs to issue.
+    const bool copy_first = WAVES < 8 || wave < WAVES / 2;
+    if (copy_first) {
+      if (kt + 2 < ntiles) copy_k_all(Kb + kfree, kt + 2);
+      if (kt + 1 < ntiles) copy_v_all(Vb + vnext, kt + 1);
+    }
     const unsigned char* v0 = Vb + vcur + v_lane;
     block_e(Kb + kcur + k_lane + 32 * KRS, v0, sa, pa, sb, std::true_type{});
     stamp(kt, 1);
     block_a(v0, Kb + knext + k_lane, sa, pa, sb, kt * FA_KT + 32, std::true_type{}, mask_c, next_c);
+    if (!copy_first) {
+      if (kt + 2 < ntiles) copy_k_all(Kb + kfree, kt + 2);
+      if (kt + 1 < ntiles) copy_v_all(Vb + vnext, kt + 1);
+    }
     stamp(kt, 2);
     block_e(Kb + knext + k_lane, v0 + 32 * VRS, sb, pb, sa, next_c);
     stamp(kt, 3);
