@@ -130,6 +130,10 @@ def products(core, request):
     (2, 4, 64, None, True),
     (3, 6, 100, None, True),           # ragged batch
     (2, 5, 17, None, True),            # less than one 32-row block
+    (1, 1, 64, None, True),            # a single step: two items, nothing to pipeline
+    (2, 1, 256, None, False),
+    (3, 2, 33, None, True),            # second row block holds one row
+    (2, 40, 1, None, True),            # one sequence
     (4, 9, 32, [1, 2, 4, 8], True),    # dilated, one 32-row block
     (6, 12, 256, [1, 2, 4, 8, 16, 32], False),  # config 5 layer structure, short sequence
 ])
