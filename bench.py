@@ -322,12 +322,69 @@ def bench_lstm(torch, core, steps, warmup, cpu, dilated, baselines=True):
     return res
 
 
+def bench_lstm_f16(torch, core, steps, warmup, cpu, baselines=True):
+    """fp16-storage stack at the second hidden size of the reference's sweep (cute_stacked_lstm/stacked_lstm.cu:186)."""
+    L, T, B, H = 32, 64, 256, 512
+    flop = 2.0 * L * T * B * (2 * H) * (4 * H)
+    gen = torch.Generator(device='cpu').manual_seed(1234)
+    xs = torch.randn((T, B, H), generator=gen).half().cuda()
+    WU = ((torch.rand((L, 2 * H, 4 * H), generator=gen) - 0.5) / 12).half().cuda()
+    hs = torch.empty((L, T, B, H), dtype=torch.float16, device='cuda')
+    cs = torch.empty_like(hs)
+    ws = torch.empty(int(core.lib.ftk_stacked_lstm_f16_workspace_bytes(L, T, B, H)), dtype=torch.uint8, device='cuda')
+    fused = lambda: core.stacked_lstm_f16(xs, WU, out=(hs, cs), workspace=ws)
+    ms, wall = _events_ms(torch, fused, steps, warmup)
+    status = core.persistent_status(ws)
+    res = {
+        'metric': 'stacked-LSTM sequences/s', 'value': B / ms * 1e3, 'unit': 'sequences/s', 'ms_per_step': ms, 'dtype': 'f16',
+        'config': {'workload': 'stacked LSTM, fp16 storage, the H = 512 row of the reference sweep', 'layers': L, 'batch': B,
+                   'seq_len': T, 'hidden': H, 'outputs': 'h and c of every layer at every step (fp16)', 'accumulate': 'f32'},
+        'tflops': flop / ms / 1e9, 'persistent_status': status,
+        'roofline': {'bound': 'mfma', 'achieved': flop / ms / 1e9, 'peak': PEAK_F16_TFLOPS, 'unit': 'TFLOP/s',
+                     'frac': flop / ms / 1e9 / PEAK_F16_TFLOPS, 'traffic': None, 'kernel': 'lstm_persistent_kernel<2>'},
+    }
+    if baselines:
+        ref_h = hs.clone()
+        W = WU[:, :H].contiguous()
+        U = WU[:, H:].contiguous()
+        hb = torch.empty_like(hs)
+
+        def unfused():   # one x@W GEMM per layer, per step h@U (hipBLASLt through torch) and the state update as torch ops
+            inp = xs
+            for l in range(L):
+                xw = torch.mm(inp.reshape(T * B, H), W[l]).reshape(T, B, 4 * H)
+                h = None
+                for t in range(T):
+                    g = xw[t] if h is None else torch.addmm(xw[t], h, U[l])
+                    i, f, o, c_ = g.chunk(4, 1)
+                    c = torch.sigmoid(i) * torch.tanh(c_) if h is None else torch.sigmoid(f) * c + torch.sigmoid(i) * torch.tanh(c_)
+                    h = torch.sigmoid(o) * torch.tanh(c)
+                    hb[l, t] = h
+                inp = hb[l]
+
+        ms_eager, _ = _events_ms(torch, unfused, 2, 1)
+        res['unfused_gpu_baseline'] = {'ms_per_step_eager': ms_eager, 'speedup_of_fused_vs_eager': ms_eager / ms,
+                                       'max_rel_diff_vs_fused': float((hb.float() - ref_h.float()).abs().max() / ref_h.float().abs().max()),
+                                       'what': 'torch fp16: one x@W GEMM per layer, per-step h@U GEMM, state update as torch ops, eager launches'}
+    if cpu:
+        from oracle import kaleido_oracle as ko
+        Ls, Ts, Bs = 4, 64, 64
+        t0 = time.perf_counter()
+        ko.stacked_lstm_f16(xs[:Ts, :Bs].cpu().numpy(), WU[:Ls].cpu().numpy())
+        dt = time.perf_counter() - t0
+        full_seconds = dt * (L * T * B) / (Ls * Ts * Bs)
+        res['cpu_baseline'] = {'value': B / full_seconds, 'unit': 'sequences/s', 'cores': 1, 'kind': 'port',
+                               'sample': f'{Ls} layer x {Ts} steps x {Bs} rows through oracle/kaleido_oracle.py (numpy float64) in '
+                                         f'{dt:.1f} s, scaled by cell-rows to the full configuration'}
+    return res
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument('--gpus', type=int, default=1)
     ap.add_argument('--steps', type=int, default=50)
     ap.add_argument('--warmup', type=int, default=10)
-    ap.add_argument('--workload', default='b2b', choices=['b2b', 'attention', 'stacked_lstm', 'dilated_lstm', 'embedding', 'copy'])
+    ap.add_argument('--workload', default='b2b', choices=['b2b', 'attention', 'stacked_lstm', 'dilated_lstm', 'lstm_f16_h512', 'embedding', 'copy'])
     ap.add_argument('--no-extras', action='store_true', help='measure only the chosen workload')
     ap.add_argument('--no-cpu', action='store_true', help='skip the CPU baseline leg')
     ap.add_argument('--no-baselines', action='store_true',
@@ -351,6 +408,7 @@ def main():
         'attention': lambda s, w, c: bench_attention(torch, core, s, w, c),
         'stacked_lstm': lambda s, w, c: bench_lstm(torch, core, max(3, s // 5), max(1, w // 5), c, False, not args.no_baselines),
         'dilated_lstm': lambda s, w, c: bench_lstm(torch, core, max(3, s // 5), max(1, w // 5), c, True, not args.no_baselines),
+        'lstm_f16_h512': lambda s, w, c: bench_lstm_f16(torch, core, max(3, s // 5), max(1, w // 5), c, not args.no_baselines),
         'embedding': lambda s, w, c: bench_embedding(torch, core, s, w, c),
     }
     if args.workload == 'copy':

@@ -21,6 +21,7 @@ EXPORTS = (
     'ftk_lstm_cell_f32', 'ftk_lstm_elementwise_f32',
     'ftk_stacked_lstm_workspace_bytes', 'ftk_stacked_lstm_f32', 'ftk_dilated_lstm_f32',
     'ftk_stacked_lstm_wavefront_f32', 'ftk_stacked_lstm_ragged_f32', 'ftk_lstm_set_products', 'ftk_lstm_get_products',
+    'ftk_stacked_lstm_f16_workspace_bytes', 'ftk_stacked_lstm_f16',
     'ftk_b2b_gemm_f16', 'ftk_flash_attn_f16', 'ftk_online_softmax_f32', 'ftk_embedding_gather_f32',
     'ftk_debug_read_fa_trace',
 )
@@ -53,8 +54,10 @@ def _load() -> ctypes.CDLL:
     lib.ftk_last_error.restype = ctypes.c_char_p
     lib.ftk_stacked_lstm_workspace_bytes.restype = ctypes.c_size_t
     lib.ftk_stacked_lstm_workspace_bytes.argtypes = [ctypes.c_int] * 4
+    lib.ftk_stacked_lstm_f16_workspace_bytes.restype = ctypes.c_size_t
+    lib.ftk_stacked_lstm_f16_workspace_bytes.argtypes = [ctypes.c_int] * 4
     for name in EXPORTS:
-        if name not in ('ftk_last_error', 'ftk_stacked_lstm_workspace_bytes'):
+        if name not in ('ftk_last_error', 'ftk_stacked_lstm_workspace_bytes', 'ftk_stacked_lstm_f16_workspace_bytes'):
             getattr(lib, name).restype = ctypes.c_int
     return lib
 
@@ -196,6 +199,42 @@ def stacked_lstm(xs, WU, bias=None, dilations: Optional[Sequence[int]] = None, s
     else:
         _check(lib.ftk_dilated_lstm_f32(_ptr(xs), _ptr(WU), _ptr(bias), dil, _ptr(hsss), _ptr(csss),
                                         ci(L), ci(T), ci(B), ci(H), _ptr(workspace), ws_bytes, _stream()))
+    return hsss, csss
+
+
+def stacked_lstm_f16(xs, WU, bias=None, dilations: Optional[Sequence[int]] = None,
+                     out: Optional[Tuple[torch.Tensor, torch.Tensor]] = None, workspace: Optional[torch.Tensor] = None,
+                     active_rows: Optional[Sequence[int]] = None) -> Tuple[torch.Tensor, torch.Tensor]:
+    """fp16 storage: xs [T,B,H], WU [L,2H,4H] fp16, bias [L,4H] fp32 or None -> hsss, csss [L,T,B,H] fp16.  H = 512."""
+    f16 = torch.float16
+    _req(xs, f16, 'xs'); _req(WU, f16, 'WU')
+    T, B, H = xs.shape
+    L = WU.shape[0]
+    if WU.shape != (L, 2 * H, 4 * H):
+        raise ValueError(f'WU must be [L, 2H, 4H] = [{L}, {2 * H}, {4 * H}], got {tuple(WU.shape)}')
+    if bias is not None and _req(bias, torch.float32, 'bias').shape != (L, 4 * H):
+        raise ValueError('bias must be [L, 4H]')
+    if out is None:
+        hsss = torch.empty((L, T, B, H), dtype=f16, device=xs.device)
+        csss = torch.empty((L, T, B, H), dtype=f16, device=xs.device)
+    else:
+        hsss, csss = out
+        _req(hsss, f16, 'hsss'); _req(csss, f16, 'csss')
+    dil = None
+    if dilations is not None:
+        if len(dilations) != L:
+            raise ValueError('dilations must have one entry per layer')
+        dil = (ctypes.c_int * L)(*[int(d) for d in dilations])
+    act = None
+    if active_rows is not None:
+        if len(active_rows) != T:
+            raise ValueError('active_rows must have one entry per step')
+        act = (ctypes.c_int * T)(*[int(v) for v in active_rows])
+    if workspace is None:
+        workspace = torch.empty(int(lib.ftk_stacked_lstm_f16_workspace_bytes(L, T, B, H)), dtype=torch.uint8, device=xs.device)
+    ci = ctypes.c_int
+    _check(lib.ftk_stacked_lstm_f16(_ptr(xs), _ptr(WU), _ptr(bias), dil, act, _ptr(hsss), _ptr(csss), ci(L), ci(T), ci(B),
+                                    ci(H), _ptr(workspace), ctypes.c_size_t(workspace.numel()), _stream()))
     return hsss, csss
 
 

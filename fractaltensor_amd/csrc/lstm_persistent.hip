@@ -169,12 +169,23 @@ constexpr int kStageRow32 = 144, kStageRow16 = 80;
 constexpr int kStageC = 0, kStageH = 32 * kStageRow32, kStageTop = 2 * 32 * kStageRow32, kStageRest = kStageTop + 32 * kStageRow16;
 constexpr int kStageBytes = kStageRest + 32 * kStageRow16;
 constexpr size_t kPersistLds = (size_t)2 * P_TILE * sizeof(float) + 1024 + 2 * kStageBytes;  // tiles, prefetch scrap, staging
-constexpr int FLAG_TARGET = PC * 4;  // one count per wave of each of the 8 column slices
+// Kernel flavours.  kProductsF32 / kProductsSplit: fp32 data, H = 256, the two ways of forming the products.
+// kHalfData: fp16 inputs, weights, h and c (what the reference's CuTe LSTM stores), one fp16 MFMA per product
+// with fp32 accumulation, H = 512: a row of 512 fp16 takes the 1024 bytes a row of 256 fp32 takes, and a
+// wave's 32 gate columns x 1024 k of fp16 weights the 256 VGPRs the other flavours' weights take, so tiles,
+// copies and schedule are shared; a layer then has 16 column slices instead of 8.
+constexpr int kProductsF32 = 0, kProductsSplit = 1, kHalfData = 2;
 constexpr int TS = 8;              // trace stamps per item
 
-template <bool SPLIT>
+template <int MODE>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1)))
 void lstm_persistent_kernel(PersistArgs a) {
+  constexpr bool SPLIT = MODE == kProductsSplit;
+  constexpr bool F16 = MODE == kHalfData;
+  constexpr int HID = F16 ? 2 * PH : PH;  // hidden size
+  constexpr int NPC = HID / 32;           // column slices per layer (32 units each)
+  constexpr int NG = 4 * HID;             // gate columns
+  constexpr int FLAG_TARGET = NPC * 4;    // one count per wave of each column slice
   extern __shared__ __attribute__((aligned(16))) float tile[];  // [2][32][P_LD], 256 floats of scrap, 2 staging buffers
 
   const int tid = threadIdx.x;
@@ -187,14 +198,14 @@ void lstm_persistent_kernel(PersistArgs a) {
   if (a.xcd_remap) q = (blockIdx.x & 7) * (gridDim.x >> 3) + (blockIdx.x >> 3);
   if (q >= a.groups) return;
   if (q == a.trace_q && tid == 0) reinterpret_cast<long long*>(a.status + 16)[0] = wall_clock64();
-  const int per_layer = PC * a.pr;
+  const int per_layer = NPC * a.pr;
   const int l = q / per_layer;
   const int within = q - l * per_layer;
-  const int pc = within % PC;
-  const int prs = within / PC;
+  const int pc = within % NPC;
+  const int prs = within / NPC;
   const int d = a.dil[l];
   const int T = a.T, B = a.B;
-  const size_t cell = (size_t)B * PH;
+  const size_t cell = (size_t)B * PH;  // floats (or pairs of fp16) per [B, H] slab of activations
   const int my_rbs = (a.nrb - prs + a.pr - 1) / a.pr;  // row blocks this workgroup walks per time step
   const int n_items = T * my_rbs;
 
@@ -202,12 +213,23 @@ void lstm_persistent_kernel(PersistArgs a) {
   // MFMA step s = 4q + c, WU[l][k = 8q + 4hh + c][gate(i)*H + 32pc + 8w + i%8].
   // Split products: for MFMA step s the lane holds rows k = 16s + 8hh .. +7 of
   // the same column, as the fp16 pair described above.
-  const int col = (j >> 3) * PH + 32 * pc + 8 * wave + (j & 7);
+  // fp16 data: rows k = 16s + 8hh .. +7 of the column for MFMA step s, 64 steps.
+  const int col = (j >> 3) * HID + 32 * pc + 8 * wave + (j & 7);
   const float* wl = a.WU + (size_t)l * PK * PN + col;
-  float wr[SPLIT ? 1 : PK / 2];
+  float wr[MODE == kProductsF32 ? PK / 2 : 1];
   v8h whi[SPLIT ? PK / 16 : 1], wlo[SPLIT ? PK / 16 : 1];
+  v8h wh[F16 ? 2 * HID / 16 : 1];
   float ginv[16];  // split products: what accumulator register r is multiplied by to undo the scales
-  if constexpr (!SPLIT) {
+  if constexpr (F16) {
+    const _Float16* wl16 = reinterpret_cast<const _Float16*>(a.WU) + (size_t)l * (2 * HID) * NG + col;
+#pragma unroll
+    for (int s = 0; s < 2 * HID / 16; ++s) {
+#pragma unroll
+      for (int e = 0; e < 8; ++e) wh[s][e] = wl16[(size_t)(16 * s + 8 * hh + e) * NG];
+      // 16-bit loads land in a register each before they are packed: keep few of them in flight
+      if (s % 4 == 3) asm volatile("" ::: "memory");
+    }
+  } else if constexpr (!SPLIT) {
 #pragma unroll
     for (int s = 0; s < PK / 2; ++s) {
       const int k = 8 * (s >> 2) + 4 * hh + (s & 3);
@@ -240,13 +262,13 @@ void lstm_persistent_kernel(PersistArgs a) {
   const int u0 = 32 * pc + 8 * wave + 4 * hh;  // first of this lane's 4 units
   float bi[4] = {0, 0, 0, 0}, bf[4] = {0, 0, 0, 0}, bo[4] = {0, 0, 0, 0}, bg[4] = {0, 0, 0, 0};
   if (a.bias) {
-    const float* bl = a.bias + (size_t)l * PN;
+    const float* bl = a.bias + (size_t)l * NG;
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
       bi[r] = bl[u0 + r];
-      bf[r] = bl[PH + u0 + r];
-      bo[r] = bl[2 * PH + u0 + r];
-      bg[r] = bl[3 * PH + u0 + r];
+      bf[r] = bl[HID + u0 + r];
+      bo[r] = bl[2 * HID + u0 + r];
+      bg[r] = bl[3 * HID + u0 + r];
     }
   }
 
@@ -256,7 +278,7 @@ void lstm_persistent_kernel(PersistArgs a) {
     st[1] = wall_clock64();  // weights requested (st[0]: kernel entry)
     float sink = 0.f;
 #pragma unroll
-    for (int s2 = 0; s2 < (SPLIT ? PK / 16 : PK / 2); s2 += (SPLIT ? 2 : 32)) sink += SPLIT ? (float)whi[SPLIT ? s2 : 0][0] : wr[SPLIT ? 0 : s2];
+    for (int s2 = 0; s2 < 32; s2 += 2) sink += F16 ? (float)wh[F16 ? s2 : 0][0] : SPLIT ? (float)whi[SPLIT ? s2 : 0][0] : wr[MODE == kProductsF32 ? 16 * s2 : 0];
     if (sink == 12345.678f) st[3] = 0;
     st[2] = wall_clock64();  // weights (a sample of them) have arrived
   }
@@ -292,13 +314,14 @@ void lstm_persistent_kernel(PersistArgs a) {
     if (t >= d) f.own = flag_load(flag_of(l, t - d, rb));
     return f;
   };
-  auto flags_ready = [](const Flags& f) { return f.below >= FLAG_TARGET && f.own >= FLAG_TARGET; };
+  auto flags_ready = [=](const Flags& f) { return f.below >= FLAG_TARGET && f.own >= FLAG_TARGET; };
 
   // Where the activation rows come from.  The two fp16 planes of a row take the
   // 1024 bytes of its fp32 form, so the tile code is the same for both: in
-  // split mode a tile row is [x top | x rest | h top | h rest], 256 fp16 each.
-  const float* xin = SPLIT ? reinterpret_cast<const float*>(a.xsp) : a.xs;
-  const float* hin = SPLIT ? reinterpret_cast<const float*>(a.hsp) : a.hsss;
+  // split mode a tile row is [x top | x rest | h top | h rest], 256 fp16 each, with
+  // fp16 data [x | h], 512 fp16 each (xsp / hsp then are the fp16 xs and hsss themselves).
+  const float* xin = (SPLIT || F16) ? reinterpret_cast<const float*>(a.xsp) : a.xs;
+  const float* hin = (SPLIT || F16) ? reinterpret_cast<const float*>(a.hsp) : a.hsss;
 
   // Tile n into LDS buffer buf, global -> LDS directly: wave w moves rows
   // 8w..8w+7; one instruction carries half a tile row (1024 bytes = 64 lanes x
@@ -399,7 +422,29 @@ void lstm_persistent_kernel(PersistArgs a) {
       __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
     }
   };
-  // one interface for both: K steps of the x half [x0, x1) or of the h half, in
+  // fp16 data: steps 0..31 are the x rows, 32..63 the h rows; one MFMA per step, two accumulation chains
+  auto mfma_half = [&](int buf, auto q0c, auto q1c, v16f& a0, v16f& a1) __attribute__((always_inline)) {
+    constexpr int q0 = decltype(q0c)::value;
+    constexpr int q1 = decltype(q1c)::value;
+    const _Float16* arow = reinterpret_cast<const _Float16*>(tile + buf * P_TILE + j * P_LD) + 8 * hh;
+    auto frag = [&](int qq) { return *reinterpret_cast<const v8h*>(arow + (qq >> 5) * HID + 16 * (qq & 31)); };
+    v8h b0 = frag(q0), b1 = frag(q0 + 1);
+#pragma unroll
+    for (int qq = q0; qq < q1; qq += 2) {
+      v8h b0n = b0, b1n = b1;
+      if (qq + 2 < q1) { b0n = frag(qq + 2); b1n = frag(qq + 3); }
+      a0 = __builtin_amdgcn_mfma_f32_32x32x16_f16(wh[F16 ? qq : 0], b0, a0, 0, 0, 0);
+      a1 = __builtin_amdgcn_mfma_f32_32x32x16_f16(wh[F16 ? qq + 1 : 0], b1, a1, 0, 0, 0);
+      b0 = b0n; b1 = b1n;
+    }
+    __builtin_amdgcn_sched_group_barrier(0x100, 4, 0);
+#pragma unroll
+    for (int g2 = q0; g2 < q1; g2 += 2) {
+      __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
+      __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+    }
+  };
+  // one interface for all: K steps of the x half [x0, x1) or of the h half, in
   // units of a sixteenth of a half
   v16f acc0, acc1, acc2;
   auto clear_acc = [&]() __attribute__((always_inline)) {
@@ -408,7 +453,9 @@ void lstm_persistent_kernel(PersistArgs a) {
   };
   auto mfma_range = [&](int buf, auto half_c, auto s0c, auto s1c) __attribute__((always_inline)) {
     constexpr int hf = decltype(half_c)::value, s0 = decltype(s0c)::value, s1 = decltype(s1c)::value;
-    if constexpr (SPLIT)
+    if constexpr (F16)
+      mfma_half(buf, std::integral_constant<int, 32 * hf + 2 * s0>{}, std::integral_constant<int, 32 * hf + 2 * s1>{}, acc0, acc1);
+    else if constexpr (SPLIT)
       mfma_split(buf, std::integral_constant<int, 16 * hf + s0>{}, std::integral_constant<int, 16 * hf + s1>{}, acc0, acc1, acc2);
     else
       mfma_part(buf, std::integral_constant<int, 32 * hf + 2 * s0>{}, std::integral_constant<int, 32 * hf + 2 * s1>{}, acc0, acc1);
@@ -469,6 +516,13 @@ void lstm_persistent_kernel(PersistArgs a) {
     epilogue_math(acc, cp, hv, cv);
     unsigned char* sb = stage + sbuf * kStageBytes;
     const int c4 = 8 * wave + 4 * hh;
+    if constexpr (F16) {  // h and c leave as fp16: the two 16-bit staging planes hold them
+      const v4h h16 = {(_Float16)hv[0], (_Float16)hv[1], (_Float16)hv[2], (_Float16)hv[3]};
+      const v4h c16 = {(_Float16)cv[0], (_Float16)cv[1], (_Float16)cv[2], (_Float16)cv[3]};
+      *reinterpret_cast<v4h*>(sb + kStageTop + j * kStageRow16 + 2 * c4) = h16;
+      *reinterpret_cast<v4h*>(sb + kStageRest + j * kStageRow16 + 2 * c4) = c16;
+      return;
+    }
     *reinterpret_cast<float4*>(sb + kStageC + j * kStageRow32 + 4 * c4) = make_float4(cv[0], cv[1], cv[2], cv[3]);
     *reinterpret_cast<float4*>(sb + kStageH + j * kStageRow32 + 4 * c4) = make_float4(hv[0], hv[1], hv[2], hv[3]);
     if constexpr (SPLIT) {
@@ -489,6 +543,16 @@ void lstm_persistent_kernel(PersistArgs a) {
     const int t = item_t(n), rb = item_rb(n);
     const int rl = 8 * wave + (lane >> 3), cc = lane & 7;
     const int rg = rb * 32 + rl;
+    if constexpr (F16) {
+      if (alive && rg < B && live(n)) {
+        const unsigned char* sb = stage + sbuf * kStageBytes;
+        const size_t at16 = (((size_t)l * T + t) * B + rg) * HID + 32 * pc + 4 * cc;
+        coherent_store8h(a.hsp + at16, *reinterpret_cast<const v4h*>(sb + kStageTop + rl * kStageRow16 + 8 * cc));
+        *reinterpret_cast<v4h*>(reinterpret_cast<_Float16*>(a.csss) + at16) =
+            *reinterpret_cast<const v4h*>(sb + kStageRest + rl * kStageRow16 + 8 * cc);
+      }
+      return;
+    }
     if (alive && rg < B && live(n)) {
       const unsigned char* sb = stage + sbuf * kStageBytes;
       const size_t at = ((size_t)l * T + t) * cell + (size_t)rg * PH + 32 * pc + 4 * cc;
@@ -518,7 +582,13 @@ void lstm_persistent_kernel(PersistArgs a) {
     float4 cp = make_float4(0.f, 0.f, 0.f, 0.f);
     if (alive && t >= d && live(n)) {
       const int rgc = min(rb * 32 + j, B - 1);
-      cp = *reinterpret_cast<const float4*>(a.csss + ((size_t)l * T + (t - d)) * cell + (size_t)rgc * PH + u0);
+      if constexpr (F16) {
+        const v4h c16 = *reinterpret_cast<const v4h*>(reinterpret_cast<const _Float16*>(a.csss) +
+                                                      (((size_t)l * T + (t - d)) * B + rgc) * HID + u0);
+        cp = make_float4((float)c16[0], (float)c16[1], (float)c16[2], (float)c16[3]);
+      } else {
+        cp = *reinterpret_cast<const float4*>(a.csss + ((size_t)l * T + (t - d)) * cell + (size_t)rgc * PH + u0);
+      }
     }
     return cp;
   };
@@ -584,7 +654,7 @@ void lstm_persistent_kernel(PersistArgs a) {
   // products an item's MFMAs take less than those 2 us, so the only look inside an item is the one after
   // them; with fp32 products there is time for a look after every quarter of a half, and the previous
   // item is counted half way through the x half.
-  constexpr int kFirstLook = SPLIT ? 7 : 0;
+  constexpr int kFirstLook = MODE == kProductsF32 ? 0 : 7;
   alive = wait_deps(0);
   if (alive) issue_tile(0, 0);
   float4 cp = load_cprev(0);
@@ -622,7 +692,7 @@ void lstm_persistent_kernel(PersistArgs a) {
       look(0);
       mfma_range(buf, IC<0>{}, IC<4>{}, IC<8>{});
       look(1);
-      if (!SPLIT && !counted) { publish(n - 1); counted = true; }
+      if (MODE == kProductsF32 && !counted) { publish(n - 1); counted = true; }
       mfma_range(buf, IC<0>{}, IC<8>{}, IC<12>{});
       look(2);
       mfma_range(buf, IC<0>{}, IC<12>{}, IC<16>{});
@@ -761,48 +831,82 @@ static int trace_workgroup() {
   return v;
 }
 
-static int run_persistent(const float* xs, const float* WU, const float* bias, const int* dil, const int* active,
-                          float* hsss, float* csss, int L, int T, int B, void* ws, size_t ws_bytes, hipStream_t s,
-                          bool* handled) {
-  *handled = false;
+template <int MODE>
+static int persistent_function(const void** fn, size_t lds) {
+  static bool attr_set = false;
+  *fn = (const void*)lstm_persistent_kernel<MODE>;
+  if (!attr_set) {
+    FTK_HIP(hipFuncSetAttribute(*fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+    attr_set = true;
+  }
+  return FTK_OK;
+}
+
+// Co-resident workgroups the device offers the persistent kernel of a flavour (0 if it cannot run at all).
+static int persistent_slots(int mode, const void** fn, int* slots) {
+  *slots = 0;
   const DeviceProps* dp = nullptr;
   int rc = device_props(&dp);
   if (rc) return rc;
   const size_t lds = kPersistLds;
   if ((int)lds > dp->lds_optin) return FTK_OK;
-  const bool split = products_mode() == 1;
-  const void* fn = split ? (const void*)lstm_persistent_kernel<true> : (const void*)lstm_persistent_kernel<false>;
-  static bool attr_set[2] = {false, false};
-  if (!attr_set[split]) {
-    FTK_HIP(hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-    attr_set[split] = true;
-  }
+  rc = mode == kHalfData ? persistent_function<kHalfData>(fn, lds)
+       : mode == kProductsSplit ? persistent_function<kProductsSplit>(fn, lds)
+                                : persistent_function<kProductsF32>(fn, lds);
+  if (rc) return rc;
   int per_cu = 0;
-  FTK_HIP(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, fn, 256, lds));
-  const int slots = per_cu * dp->cus;
-  if (L > kMaxLayers || L * PC > slots) return FTK_OK;  // cannot pin every layer on its own compute units: fall back
+  FTK_HIP(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, *fn, 256, lds));
+  *slots = per_cu * dp->cus;
+  return FTK_OK;
+}
+
+// mode kProductsF32 / kProductsSplit: fp32 xs, WU, hsss, csss, H = 256.  kHalfData: the same arrays in fp16, H = 512.
+static int run_persistent(int mode, const void* xs, const void* WU, const float* bias, const int* dil, const int* active,
+                          void* hsss, void* csss, int L, int T, int B, void* ws, size_t ws_bytes, hipStream_t s,
+                          bool* handled) {
+  *handled = false;
+  const void* fn = nullptr;
+  int slots = 0;
+  int rc = persistent_slots(mode, &fn, &slots);
+  if (rc) return rc;
+  const size_t lds = kPersistLds;
+  const bool split = mode == kProductsSplit;
+  const int npc = mode == kHalfData ? 16 : PC;  // column slices (workgroups) per layer
+  if (L > kMaxLayers || L * npc > slots) return FTK_OK;  // cannot pin every layer on its own compute units: fall back
 
   const size_t nflags = flag_count(L, T, B);
-  const size_t need = workspace_need(L, T, B);
+  const size_t need = mode == kHalfData ? xratio_offset_bytes(L, T, B) : workspace_need(L, T, B);
   if (!ws || ws_bytes < need)
     return fail(FTK_ERR_WORKSPACE, "stacked LSTM needs a %zu-byte workspace, got %zu", need, ws_bytes);
 
   PersistArgs a;
-  a.xs = xs; a.WU = WU; a.bias = bias; a.hsss = hsss; a.csss = csss;
+  a.xs = reinterpret_cast<const float*>(xs);
+  a.WU = reinterpret_cast<const float*>(WU);
+  a.bias = bias;
+  a.hsss = reinterpret_cast<float*>(hsss);
+  a.csss = reinterpret_cast<float*>(csss);
   a.status = reinterpret_cast<int*>(ws);
   a.flags = a.status + 64;
   char* wsb = reinterpret_cast<char*>(ws);
-  float* xratio = reinterpret_cast<float*>(wsb + xratio_offset_bytes(L, T, B));
-  _Float16* xsp = reinterpret_cast<_Float16*>(wsb + xsp_offset_bytes(L, T, B));
-  a.xratio = xratio;
-  a.xsp = xsp;
-  a.hsp = reinterpret_cast<_Float16*>(wsb + hsp_offset_bytes(L, T, B));
+  float* xratio = nullptr;
+  _Float16* xsp = nullptr;
+  if (mode == kHalfData) {  // the kernel reads its tiles from the fp16 arrays themselves
+    a.xratio = nullptr;
+    a.xsp = reinterpret_cast<const _Float16*>(xs);
+    a.hsp = reinterpret_cast<_Float16*>(hsss);
+  } else {
+    xratio = reinterpret_cast<float*>(wsb + xratio_offset_bytes(L, T, B));
+    xsp = reinterpret_cast<_Float16*>(wsb + xsp_offset_bytes(L, T, B));
+    a.xratio = xratio;
+    a.xsp = xsp;
+    a.hsp = reinterpret_cast<_Float16*>(wsb + hsp_offset_bytes(L, T, B));
+  }
   a.L = L; a.T = T; a.B = B;
   a.nrb = (B + 31) / 32;
   // spare compute units become row slices, but a workgroup keeps at least two
   // row blocks when it can so that the next tile never depends on the current item
-  a.pr = std::max(1, std::min(slots / (L * PC), std::max(1, a.nrb / 2)));
-  a.groups = L * PC * a.pr;
+  a.pr = std::max(1, std::min(slots / (L * npc), std::max(1, a.nrb / 2)));
+  a.groups = L * npc * a.pr;
   a.spin_limit = 1 << 22;
   a.trace_q = trace_workgroup();
   a.trace = reinterpret_cast<long long*>(reinterpret_cast<char*>(ws) + trace_offset_bytes(L, T, B));
@@ -827,15 +931,16 @@ static int run_persistent(const float* xs, const float* WU, const float* bias, c
 
   if (split) {
     const int rows = T * B;
-    hipLaunchKernelGGL(lstm_split_rows_kernel, dim3((rows + 3) / 4), dim3(256), 0, s, xs, xsp, xratio, rows);
+    hipLaunchKernelGGL(lstm_split_rows_kernel, dim3((rows + 3) / 4), dim3(256), 0, s, a.xs, xsp, xratio, rows);
     rc = check_launch("lstm_split_rows_kernel");
     if (rc) return rc;
   }
 
   void* kargs[] = {&a};
   if (plain_launch()) {
-    if (split) hipLaunchKernelGGL(lstm_persistent_kernel<true>, dim3(grid), dim3(256), lds, s, a);
-    else hipLaunchKernelGGL(lstm_persistent_kernel<false>, dim3(grid), dim3(256), lds, s, a);
+    if (mode == kHalfData) hipLaunchKernelGGL(lstm_persistent_kernel<kHalfData>, dim3(grid), dim3(256), lds, s, a);
+    else if (split) hipLaunchKernelGGL(lstm_persistent_kernel<kProductsSplit>, dim3(grid), dim3(256), lds, s, a);
+    else hipLaunchKernelGGL(lstm_persistent_kernel<kProductsF32>, dim3(grid), dim3(256), lds, s, a);
     rc = check_launch("lstm_persistent_kernel");
     if (rc) return rc;
   } else {
@@ -872,7 +977,8 @@ static int run_stack(const char* who, const float* xs, const float* WU, const fl
   }
   if (H == PH) {
     bool handled = false;
-    rc = run_persistent(xs, WU, bias, dil, active, hsss, csss, L, T, B, ws, ws_bytes, s, &handled);
+    rc = run_persistent(products_mode() == 1 ? kProductsSplit : kProductsF32, xs, WU, bias, dil, active, hsss, csss, L, T, B,
+                        ws, ws_bytes, s, &handled);
     if (rc || handled) return rc;
   }
   return run_wavefront(xs, WU, bias, dil, hsss, csss, L, T, B, H, s);
@@ -885,6 +991,55 @@ extern "C" {
 size_t ftk_stacked_lstm_workspace_bytes(int L, int T, int B, int H) {
   if (L <= 0 || T <= 0 || B <= 0 || H <= 0) return 0;
   return ftk::workspace_need(L, T, B);
+}
+
+size_t ftk_stacked_lstm_f16_workspace_bytes(int L, int T, int B, int H) {
+  if (L <= 0 || T <= 0 || B <= 0 || H <= 0) return 0;
+  return ftk::xratio_offset_bytes(L, T, B);
+}
+
+int ftk_stacked_lstm_f16(const void* xs, const void* WU, const float* bias, const int* dilations,
+                         const int* active_rows, void* hsss, void* csss, int L, int T, int B, int H, void* workspace,
+                         size_t workspace_bytes, ftk_stream_t stream) {
+  using namespace ftk;
+  const char* who = "ftk_stacked_lstm_f16";
+  if (!xs || !WU || !hsss || !csss) return fail(FTK_ERR_INVALID_ARGUMENT, "%s: xs, WU, hsss, csss must be non-NULL", who);
+  if (L <= 0 || T <= 0 || B <= 0 || H <= 0) return fail(FTK_ERR_INVALID_ARGUMENT, "%s: L, T, B, H must be positive", who);
+  if (H != 2 * PH) return fail(FTK_ERR_UNSUPPORTED_SHAPE, "%s: the fp16 stack is built for H = %d, got %d", who, 2 * PH, H);
+  if (dilations)
+    for (int l = 0; l < L; ++l)
+      if (dilations[l] <= 0) return fail(FTK_ERR_INVALID_ARGUMENT, "%s: dilations[%d]=%d must be positive", who, l, dilations[l]);
+  if (active_rows)
+    for (int t = 0; t < T; ++t) {
+      if (active_rows[t] < 0 || active_rows[t] > B)
+        return fail(FTK_ERR_INVALID_ARGUMENT, "%s: active_rows[%d]=%d is outside [0, B=%d]", who, t, active_rows[t], B);
+      if (t > 0 && active_rows[t] > active_rows[t - 1])
+        return fail(FTK_ERR_INVALID_ARGUMENT, "%s: active_rows must be non-increasing (rows sorted by length)", who);
+    }
+  const void* fn = nullptr;
+  int slots = 0;
+  int rc = persistent_slots(kHalfData, &fn, &slots);
+  if (rc) return rc;
+  const int chunk = std::min(slots / 16, kMaxLayers);  // layers whose weights fit on the chip at once
+  if (chunk < 1) return fail(FTK_ERR_DEVICE, "%s: the device cannot hold one layer's weights in registers", who);
+  // deeper stacks run as consecutive launches of `chunk` layers: a chunk reads the hidden sequence of the
+  // layer below it, complete by then, like the first chunk reads xs
+  const size_t slab = (size_t)T * B * H;  // elements of one layer's h (or c)
+  const _Float16* x16 = reinterpret_cast<const _Float16*>(xs);
+  const _Float16* w16 = reinterpret_cast<const _Float16*>(WU);
+  _Float16* h16 = reinterpret_cast<_Float16*>(hsss);
+  _Float16* c16 = reinterpret_cast<_Float16*>(csss);
+  for (int l0 = 0; l0 < L; l0 += chunk) {
+    const int lc = std::min(chunk, L - l0);
+    bool handled = false;
+    rc = run_persistent(kHalfData, l0 == 0 ? x16 : h16 + (size_t)(l0 - 1) * slab, w16 + (size_t)l0 * 2 * H * 4 * H,
+                        bias ? bias + (size_t)l0 * 4 * H : nullptr, dilations ? dilations + l0 : nullptr, active_rows,
+                        h16 + (size_t)l0 * slab, c16 + (size_t)l0 * slab, lc, T, B, workspace, workspace_bytes,
+                        (hipStream_t)stream, &handled);
+    if (rc) return rc;
+    if (!handled) return fail(FTK_ERR_DEVICE, "%s: the persistent kernel cannot run on this device", who);
+  }
+  return FTK_OK;
 }
 
 int ftk_lstm_set_products(int mode) {

@@ -164,6 +164,38 @@ def stacked_lstm(xs, WUs, biases=None, dilations=None, dtype=np.float64):
     return hsss, csss
 
 
+def stacked_lstm_f16(xs, WUs, biases=None, dilations=None):
+    """The same stack with fp16 storage: xs, WUs given in fp16, gate sums and the state update in wider
+    arithmetic (float64 here; fp16 products are exact in fp32), and every h and c rounded to fp16 when it
+    is written -- the rounded values are what the next step and the next layer read.
+
+    This is the numeric form of the reference's CuTe LSTM, whose tensors are all `half` with fp32 MFMA
+    accumulators (kaleido/core/device/kernels/lstm.h:253-348, lstm_kernels.h:25-126; element type
+    `cutlass::half_t` in benchmarks/rnn/fractaltensor/cute_stacked_lstm/stacked_lstm.cu:16-19), applied to the
+    cell of examples/stacked_rnn/stacked_rnn.py:13-36.  Returns hsss, csss [L,T,B,H] as float16.
+    """
+    xs = np.asarray(xs, dtype=np.float16)
+    L = len(WUs)
+    T, B, _ = xs.shape
+    H = np.asarray(WUs[0]).shape[1] // 4
+    hsss = np.zeros((L, T, B, H), dtype=np.float16)
+    csss = np.zeros((L, T, B, H), dtype=np.float16)
+    zero = np.zeros((B, H), dtype=np.float64)
+    inp = xs
+    for l in range(L):
+        d = 1 if dilations is None else int(dilations[l])
+        WU = np.asarray(WUs[l], dtype=np.float16).astype(np.float64)
+        b = None if biases is None else np.asarray(biases[l], dtype=np.float64)
+        for t in range(T):
+            hp = hsss[l, t - d].astype(np.float64) if t >= d else zero
+            cp = csss[l, t - d].astype(np.float64) if t >= d else zero
+            h, c = lstm_cell(inp[t].astype(np.float64), hp, cp, WU, b, dtype=np.float64)
+            hsss[l, t] = h.astype(np.float16)
+            csss[l, t] = c.astype(np.float16)
+        inp = hsss[l]
+    return hsss, csss
+
+
 def wavefront_diagonals(L, T):
     """The reference's three-region wavefront schedule as a list of stages.
 

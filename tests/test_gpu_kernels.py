@@ -219,6 +219,50 @@ def test_stacked_lstm_ragged_rejects_unsorted_rows(core):
         core.stacked_lstm(xs, WU, active_rows=[32, 16])
 
 
+# fp16 storage, H = 512: tolerance 1e-2 (north star's figure for fp16 work) against the oracle that rounds h and c
+# to fp16 wherever the kernel does
+@pytest.mark.parametrize('L,T,B,dil,bias,ragged', [
+    (1, 6, 64, None, False, False),
+    (2, 5, 40, None, True, False),             # ragged last row block
+    (3, 8, 96, [1, 2, 4], True, False),
+    (2, 9, 64, None, True, True),              # half the rows stop after 4 steps
+    (18, 3, 32, None, False, False),           # deeper than the chip holds at once: two launches
+])
+def test_stacked_lstm_f16(core, L, T, B, dil, bias, ragged):
+    H = 512
+    rng = np.random.default_rng(13)
+    xs = rng.standard_normal((T, B, H)).astype(np.float16)
+    WU = rng.uniform(-1 / 24, 1 / 24, (L, 2 * H, 4 * H)).astype(np.float16)
+    bs = rng.uniform(-0.1, 0.1, (L, 4 * H)).astype(np.float32) if bias else None
+    active = None
+    lens = np.full(B, T)
+    if ragged:
+        lens = np.where(np.arange(B) < B // 2, T, 4)
+        active = [int((lens > t).sum()) for t in range(T)]
+        for b in range(B):
+            xs[lens[b]:, b] = 0
+    hsss, csss = core.stacked_lstm_f16(dev(xs), dev(WU), None if bs is None else dev(bs), dilations=dil, active_rows=active)
+    torch.cuda.synchronize()
+    hr, cr = ko.stacked_lstm_f16(xs, WU, bs, dil)
+    live = np.arange(T)[:, None] < lens[None, :]
+    got_h = hsss.float().cpu().numpy()[:, live]; got_c = csss.float().cpu().numpy()[:, live]
+    eh = ko.max_rel_err(got_h, hr.astype(np.float32)[:, live]); ec = ko.max_rel_err(got_c, cr.astype(np.float32)[:, live])
+    assert eh <= F16_TOL and ec <= F16_TOL, (eh, ec)
+    # most values agree to the bit: the two only part where a value sat within rounding of a tie
+    same = np.mean(got_h == hr.astype(np.float32)[:, live])
+    assert same > 0.9, same
+
+
+def test_stacked_lstm_f16_rejects_other_hidden_sizes(core):
+    xs = torch.zeros((2, 32, 256), dtype=torch.float16, device='cuda')
+    WU = torch.zeros((1, 512, 1024), dtype=torch.float16, device='cuda')
+    with pytest.raises(core.FtkError) as e:
+        core.stacked_lstm_f16(xs, WU)
+    assert e.value.code == -2 and 'H = 512' in str(e.value)
+    with pytest.raises(TypeError):
+        core.stacked_lstm_f16(xs.float(), WU)
+
+
 def test_lstm_products_switch(core):
     assert core.get_lstm_products() in ('f32', 'f16x3')
     with pytest.raises(ValueError):

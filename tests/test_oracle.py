@@ -273,3 +273,42 @@ def test_c_lstm_matches_numpy_oracle():
     h, c = c_oracle.lstm_cell(x, hp, cp, WUs[0], None)
     hr, cr = ko.lstm_cell(x, hp, cp, WUs[0])
     assert ko.max_rel_err(h, hr) < 1e-6 and ko.max_rel_err(c, cr) < 1e-6
+
+
+# ------------------------------------------------------------ fp16-storage LSTM
+
+def test_f16_stack_rounds_every_state_it_writes_and_reads_the_rounded_values():
+    """Pins oracle.stacked_lstm_f16 without retyping it: one step is the (already pinned) float64 cell on the
+    fp16 inputs, rounded once; a second step must start from the ROUNDED first state; a second layer must read
+    the ROUNDED hidden sequence of the first."""
+    rng = np.random.default_rng(0)
+    B, H = 5, 32
+    xs = rng.standard_normal((2, B, H)).astype(np.float16)
+    WU = rng.uniform(-0.3, 0.3, (2, 2 * H, 4 * H)).astype(np.float16)
+    bs = rng.uniform(-0.3, 0.3, (2, 4 * H))
+    hs, cs = ko.stacked_lstm_f16(xs, WU, bs)
+    assert hs.dtype == np.float16 and cs.dtype == np.float16 and hs.shape == (2, 2, B, H)
+    z = np.zeros((B, H))
+    W0, W1 = WU[0].astype(np.float64), WU[1].astype(np.float64)
+    h00, c00 = ko.lstm_cell(xs[0].astype(np.float64), z, z, W0, bs[0])
+    assert np.array_equal(hs[0, 0], h00.astype(np.float16)) and np.array_equal(cs[0, 0], c00.astype(np.float16))
+    h01, c01 = ko.lstm_cell(xs[1].astype(np.float64), hs[0, 0].astype(np.float64), cs[0, 0].astype(np.float64), W0, bs[0])
+    assert np.array_equal(hs[0, 1], h01.astype(np.float16)) and np.array_equal(cs[0, 1], c01.astype(np.float16))
+    # ... and not from the unrounded one: that gives a different (if close) answer somewhere
+    h01u, _ = ko.lstm_cell(xs[1].astype(np.float64), h00, c00, W0, bs[0])
+    assert not np.array_equal(h01u.astype(np.float16), hs[0, 1])
+    h10, c10 = ko.lstm_cell(hs[0, 0].astype(np.float64), z, z, W1, bs[1])
+    assert np.array_equal(hs[1, 0], h10.astype(np.float16)) and np.array_equal(cs[1, 0], c10.astype(np.float16))
+
+
+def test_f16_stack_stays_within_rounding_of_the_float64_stack():
+    rng = np.random.default_rng(1)
+    L, T, B, H = 3, 10, 4, 64
+    xs = rng.standard_normal((T, B, H)).astype(np.float16)
+    WU = rng.uniform(-1 / 8, 1 / 8, (L, 2 * H, 4 * H)).astype(np.float16)
+    for dil in (None, [1, 2, 4]):
+        h16, c16 = ko.stacked_lstm_f16(xs, WU, None, dil)
+        h64, c64 = ko.stacked_lstm(xs.astype(np.float64), WU.astype(np.float64), None, dil)
+        assert ko.max_rel_err(h16.astype(np.float64), h64) < 5e-3       # a few fp16 ulps (2^-11) accumulated
+        assert ko.max_rel_err(c16.astype(np.float64), c64) < 5e-3
+        assert ko.max_rel_err(h16.astype(np.float64), h64) > 1e-5       # but it does round
