@@ -322,13 +322,13 @@ def bench_lstm(torch, core, steps, warmup, cpu, dilated, baselines=True):
     return res
 
 
-def bench_lstm_f16(torch, core, steps, warmup, cpu, baselines=True):
-    """fp16-storage stack at the second hidden size of the reference's sweep (cute_stacked_lstm/stacked_lstm.cu:186)."""
-    L, T, B, H = 32, 64, 256, 512
+def bench_lstm_f16(torch, core, steps, warmup, cpu, H, baselines=True):
+    """fp16-storage stack at the first two hidden sizes of the reference's sweep (cute_stacked_lstm/stacked_lstm.cu:185-186)."""
+    L, T, B = 32, 64, 256
     flop = 2.0 * L * T * B * (2 * H) * (4 * H)
     gen = torch.Generator(device='cpu').manual_seed(1234)
     xs = torch.randn((T, B, H), generator=gen).half().cuda()
-    WU = ((torch.rand((L, 2 * H, 4 * H), generator=gen) - 0.5) / 12).half().cuda()
+    WU = ((torch.rand((L, 2 * H, 4 * H), generator=gen) - 0.5) / (8 if H == 256 else 12)).half().cuda()
     hs = torch.empty((L, T, B, H), dtype=torch.float16, device='cuda')
     cs = torch.empty_like(hs)
     ws = torch.empty(int(core.lib.ftk_stacked_lstm_f16_workspace_bytes(L, T, B, H)), dtype=torch.uint8, device='cuda')
@@ -337,11 +337,12 @@ def bench_lstm_f16(torch, core, steps, warmup, cpu, baselines=True):
     status = core.persistent_status(ws)
     res = {
         'metric': 'stacked-LSTM sequences/s', 'value': B / ms * 1e3, 'unit': 'sequences/s', 'ms_per_step': ms, 'dtype': 'f16',
-        'config': {'workload': 'stacked LSTM, fp16 storage, the H = 512 row of the reference sweep', 'layers': L, 'batch': B,
+        'config': {'workload': f'stacked LSTM, fp16 storage, the H = {H} row of the reference sweep', 'layers': L, 'batch': B,
                    'seq_len': T, 'hidden': H, 'outputs': 'h and c of every layer at every step (fp16)', 'accumulate': 'f32'},
         'tflops': flop / ms / 1e9, 'persistent_status': status,
         'roofline': {'bound': 'mfma', 'achieved': flop / ms / 1e9, 'peak': PEAK_F16_TFLOPS, 'unit': 'TFLOP/s',
-                     'frac': flop / ms / 1e9 / PEAK_F16_TFLOPS, 'traffic': None, 'kernel': 'lstm_persistent_kernel<2>'},
+                     'frac': flop / ms / 1e9 / PEAK_F16_TFLOPS, 'traffic': None,
+                     'kernel': 'lstm_persistent_kernel<2>' if H == 512 else 'lstm_persistent_kernel<3>'},
     }
     if baselines:
         ref_h = hs.clone()
@@ -384,7 +385,7 @@ def main():
     ap.add_argument('--gpus', type=int, default=1)
     ap.add_argument('--steps', type=int, default=50)
     ap.add_argument('--warmup', type=int, default=10)
-    ap.add_argument('--workload', default='b2b', choices=['b2b', 'attention', 'stacked_lstm', 'dilated_lstm', 'lstm_f16_h512', 'embedding', 'copy'])
+    ap.add_argument('--workload', default='b2b', choices=['b2b', 'attention', 'stacked_lstm', 'dilated_lstm', 'lstm_f16_h256', 'lstm_f16_h512', 'embedding', 'copy'])
     ap.add_argument('--no-extras', action='store_true', help='measure only the chosen workload')
     ap.add_argument('--no-cpu', action='store_true', help='skip the CPU baseline leg')
     ap.add_argument('--no-baselines', action='store_true',
@@ -408,7 +409,8 @@ def main():
         'attention': lambda s, w, c: bench_attention(torch, core, s, w, c),
         'stacked_lstm': lambda s, w, c: bench_lstm(torch, core, max(3, s // 5), max(1, w // 5), c, False, not args.no_baselines),
         'dilated_lstm': lambda s, w, c: bench_lstm(torch, core, max(3, s // 5), max(1, w // 5), c, True, not args.no_baselines),
-        'lstm_f16_h512': lambda s, w, c: bench_lstm_f16(torch, core, max(3, s // 5), max(1, w // 5), c, not args.no_baselines),
+        'lstm_f16_h256': lambda s, w, c: bench_lstm_f16(torch, core, max(3, s // 5), max(1, w // 5), c, 256, not args.no_baselines),
+        'lstm_f16_h512': lambda s, w, c: bench_lstm_f16(torch, core, max(3, s // 5), max(1, w // 5), c, 512, not args.no_baselines),
         'embedding': lambda s, w, c: bench_embedding(torch, core, s, w, c),
     }
     if args.workload == 'copy':

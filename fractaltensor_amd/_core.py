@@ -205,7 +205,8 @@ def stacked_lstm(xs, WU, bias=None, dilations: Optional[Sequence[int]] = None, s
 def stacked_lstm_f16(xs, WU, bias=None, dilations: Optional[Sequence[int]] = None,
                      out: Optional[Tuple[torch.Tensor, torch.Tensor]] = None, workspace: Optional[torch.Tensor] = None,
                      active_rows: Optional[Sequence[int]] = None) -> Tuple[torch.Tensor, torch.Tensor]:
-    """fp16 storage: xs [T,B,H], WU [L,2H,4H] fp16, bias [L,4H] fp32 or None -> hsss, csss [L,T,B,H] fp16.  H = 512."""
+    """fp16 storage: xs [T,B,H], WU [L,2H,4H] fp16, bias [L,4H] fp32 or None -> hsss, csss [L,T,B,H] fp16.
+    H = 512, or H = 256 with an even batch."""
     f16 = torch.float16
     _req(xs, f16, 'xs'); _req(WU, f16, 'WU')
     T, B, H = xs.shape

@@ -174,15 +174,18 @@ constexpr size_t kPersistLds = (size_t)2 * P_TILE * sizeof(float) + 1024 + 2 * k
 // with fp32 accumulation, H = 512: a row of 512 fp16 takes the 1024 bytes a row of 256 fp32 takes, and a
 // wave's 32 gate columns x 1024 k of fp16 weights the 256 VGPRs the other flavours' weights take, so tiles,
 // copies and schedule are shared; a layer then has 16 column slices instead of 8.
-constexpr int kProductsF32 = 0, kProductsSplit = 1, kHalfData = 2;
+// kHalfData256: the same at H = 256.  A row then is 512 bytes, so a 1 KB copy carries two batch rows and a tile
+// row holds the pair: [x of row 2i | x of row 2i+1 | h of row 2i | h of row 2i+1]; B must be even.
+constexpr int kProductsF32 = 0, kProductsSplit = 1, kHalfData = 2, kHalfData256 = 3;
 constexpr int TS = 8;              // trace stamps per item
 
 template <int MODE>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1)))
 void lstm_persistent_kernel(PersistArgs a) {
   constexpr bool SPLIT = MODE == kProductsSplit;
-  constexpr bool F16 = MODE == kHalfData;
-  constexpr int HID = F16 ? 2 * PH : PH;  // hidden size
+  constexpr bool F16 = MODE == kHalfData || MODE == kHalfData256;
+  constexpr bool PAIR = MODE == kHalfData256;      // two batch rows per tile row
+  constexpr int HID = MODE == kHalfData ? 2 * PH : PH;  // hidden size
   constexpr int NPC = HID / 32;           // column slices per layer (32 units each)
   constexpr int NG = 4 * HID;             // gate columns
   constexpr int FLAG_TARGET = NPC * 4;    // one count per wave of each column slice
@@ -205,7 +208,7 @@ void lstm_persistent_kernel(PersistArgs a) {
   const int prs = within / NPC;
   const int d = a.dil[l];
   const int T = a.T, B = a.B;
-  const size_t cell = (size_t)B * PH;  // floats (or pairs of fp16) per [B, H] slab of activations
+  const size_t cell = (size_t)B * (F16 ? HID / 2 : PH);  // floats (or pairs of fp16) per [B, H] slab of activations
   const int my_rbs = (a.nrb - prs + a.pr - 1) / a.pr;  // row blocks this workgroup walks per time step
   const int n_items = T * my_rbs;
 
@@ -337,6 +340,31 @@ void lstm_persistent_kernel(PersistArgs a) {
     const char* xsrc = reinterpret_cast<const char*>((l == 0) ? xin + (size_t)t * cell : hin + ((size_t)(l - 1) * T + t) * cell);
     const char* hsrc = reinterpret_cast<const char*>(hin + ((size_t)l * T + (has_prev ? t - d : 0)) * cell);
     const int row0 = rb * 32 + 8 * wave_u;
+    if constexpr (PAIR) {  // four tile rows of two batch rows each per wave
+      const unsigned ldsp = tile_lds + 4u * (unsigned)(buf * P_TILE + 4 * wave_u * P_LD);
+      if (row0 + 8 <= B) {
+        const char* xb = xsrc + (size_t)row0 * 512;
+        const char* hb = hsrc + (size_t)row0 * 512;
+        static_for<4>([&](auto rc) __attribute__((always_inline)) {
+          constexpr int r = decltype(rc)::value;
+          lds_dma16<r * 1024, kCoherentTiles>(xb, lane16, ldsp + 4u * r * P_LD);
+        });
+        if (has_prev) {
+          static_for<4>([&](auto rc) __attribute__((always_inline)) {
+            constexpr int r = decltype(rc)::value;
+            lds_dma16<r * 1024, kCoherentTiles>(hb, lane16, ldsp + 4u * r * P_LD + 1024u);
+          });
+        }
+      } else {  // pairs past the end of the (even) batch repeat the last pair
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          const size_t rg = (size_t)max(min(row0 + 2 * r, B - 2), 0);
+          lds_dma16<0, kCoherentTiles>(xsrc + rg * 512, lane16, ldsp + 4u * r * P_LD);
+          if (has_prev) lds_dma16<0, kCoherentTiles>(hsrc + rg * 512, lane16, ldsp + 4u * r * P_LD + 1024u);
+        }
+      }
+      return;
+    }
     const unsigned lds0 = tile_lds + 4u * (unsigned)(buf * P_TILE + 8 * wave_u * P_LD);
     if (row0 + 8 <= B) {
       const char* xb = xsrc + (size_t)row0 * 1024;
@@ -364,7 +392,7 @@ void lstm_persistent_kernel(PersistArgs a) {
     // the other layers' rows.  One 4-byte-per-lane copy touches all 64 cache lines of the wave's 8 rows;
     // it lands in a scrap area behind the tiles (a load into registers would need them reserved until
     // the data arrives).
-    if (l == 0 && n + 1 < n_items && live(n + 1)) {
+    if (!PAIR && l == 0 && n + 1 < n_items && live(n + 1)) {
       const int t2 = item_t(n + 1), rb2 = item_rb(n + 1);
       const int row2 = rb2 * 32 + 8 * wave_u;
       if (row2 + 8 <= B)
@@ -422,12 +450,14 @@ void lstm_persistent_kernel(PersistArgs a) {
       __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
     }
   };
-  // fp16 data: steps 0..31 are the x rows, 32..63 the h rows; one MFMA per step, two accumulation chains
+  // fp16 data: the first HID/16 steps are the x rows, the rest the h rows; one MFMA per step, two accumulation chains
   auto mfma_half = [&](int buf, auto q0c, auto q1c, v16f& a0, v16f& a1) __attribute__((always_inline)) {
     constexpr int q0 = decltype(q0c)::value;
     constexpr int q1 = decltype(q1c)::value;
-    const _Float16* arow = reinterpret_cast<const _Float16*>(tile + buf * P_TILE + j * P_LD) + 8 * hh;
-    auto frag = [&](int qq) { return *reinterpret_cast<const v8h*>(arow + (qq >> 5) * HID + 16 * (qq & 31)); };
+    constexpr int SH = HID / 16;  // steps per half
+    const _Float16* arow = PAIR ? reinterpret_cast<const _Float16*>(tile + buf * P_TILE + (j >> 1) * P_LD) + (j & 1) * HID + 8 * hh
+                                : reinterpret_cast<const _Float16*>(tile + buf * P_TILE + j * P_LD) + 8 * hh;
+    auto frag = [&](int qq) { return *reinterpret_cast<const v8h*>(arow + (qq / SH) * 512 + 16 * (qq % SH)); };
     v8h b0 = frag(q0), b1 = frag(q0 + 1);
 #pragma unroll
     for (int qq = q0; qq < q1; qq += 2) {
@@ -454,7 +484,8 @@ void lstm_persistent_kernel(PersistArgs a) {
   auto mfma_range = [&](int buf, auto half_c, auto s0c, auto s1c) __attribute__((always_inline)) {
     constexpr int hf = decltype(half_c)::value, s0 = decltype(s0c)::value, s1 = decltype(s1c)::value;
     if constexpr (F16)
-      mfma_half(buf, std::integral_constant<int, 32 * hf + 2 * s0>{}, std::integral_constant<int, 32 * hf + 2 * s1>{}, acc0, acc1);
+      mfma_half(buf, std::integral_constant<int, (HID / 16) * hf + s0 * (HID / 256)>{},
+                std::integral_constant<int, (HID / 16) * hf + s1 * (HID / 256)>{}, acc0, acc1);
     else if constexpr (SPLIT)
       mfma_split(buf, std::integral_constant<int, 16 * hf + s0>{}, std::integral_constant<int, 16 * hf + s1>{}, acc0, acc1, acc2);
     else
@@ -851,6 +882,7 @@ static int persistent_slots(int mode, const void** fn, int* slots) {
   const size_t lds = kPersistLds;
   if ((int)lds > dp->lds_optin) return FTK_OK;
   rc = mode == kHalfData ? persistent_function<kHalfData>(fn, lds)
+       : mode == kHalfData256 ? persistent_function<kHalfData256>(fn, lds)
        : mode == kProductsSplit ? persistent_function<kProductsSplit>(fn, lds)
                                 : persistent_function<kProductsF32>(fn, lds);
   if (rc) return rc;
@@ -871,11 +903,12 @@ static int run_persistent(int mode, const void* xs, const void* WU, const float*
   if (rc) return rc;
   const size_t lds = kPersistLds;
   const bool split = mode == kProductsSplit;
+  const bool half = mode == kHalfData || mode == kHalfData256;
   const int npc = mode == kHalfData ? 16 : PC;  // column slices (workgroups) per layer
   if (L > kMaxLayers || L * npc > slots) return FTK_OK;  // cannot pin every layer on its own compute units: fall back
 
   const size_t nflags = flag_count(L, T, B);
-  const size_t need = mode == kHalfData ? xratio_offset_bytes(L, T, B) : workspace_need(L, T, B);
+  const size_t need = half ? xratio_offset_bytes(L, T, B) : workspace_need(L, T, B);
   if (!ws || ws_bytes < need)
     return fail(FTK_ERR_WORKSPACE, "stacked LSTM needs a %zu-byte workspace, got %zu", need, ws_bytes);
 
@@ -890,7 +923,7 @@ static int run_persistent(int mode, const void* xs, const void* WU, const float*
   char* wsb = reinterpret_cast<char*>(ws);
   float* xratio = nullptr;
   _Float16* xsp = nullptr;
-  if (mode == kHalfData) {  // the kernel reads its tiles from the fp16 arrays themselves
+  if (half) {  // the kernel reads its tiles from the fp16 arrays themselves
     a.xratio = nullptr;
     a.xsp = reinterpret_cast<const _Float16*>(xs);
     a.hsp = reinterpret_cast<_Float16*>(hsss);
@@ -939,6 +972,7 @@ static int run_persistent(int mode, const void* xs, const void* WU, const float*
   void* kargs[] = {&a};
   if (plain_launch()) {
     if (mode == kHalfData) hipLaunchKernelGGL(lstm_persistent_kernel<kHalfData>, dim3(grid), dim3(256), lds, s, a);
+    else if (mode == kHalfData256) hipLaunchKernelGGL(lstm_persistent_kernel<kHalfData256>, dim3(grid), dim3(256), lds, s, a);
     else if (split) hipLaunchKernelGGL(lstm_persistent_kernel<kProductsSplit>, dim3(grid), dim3(256), lds, s, a);
     else hipLaunchKernelGGL(lstm_persistent_kernel<kProductsF32>, dim3(grid), dim3(256), lds, s, a);
     rc = check_launch("lstm_persistent_kernel");
@@ -1005,7 +1039,12 @@ int ftk_stacked_lstm_f16(const void* xs, const void* WU, const float* bias, cons
   const char* who = "ftk_stacked_lstm_f16";
   if (!xs || !WU || !hsss || !csss) return fail(FTK_ERR_INVALID_ARGUMENT, "%s: xs, WU, hsss, csss must be non-NULL", who);
   if (L <= 0 || T <= 0 || B <= 0 || H <= 0) return fail(FTK_ERR_INVALID_ARGUMENT, "%s: L, T, B, H must be positive", who);
-  if (H != 2 * PH) return fail(FTK_ERR_UNSUPPORTED_SHAPE, "%s: the fp16 stack is built for H = %d, got %d", who, 2 * PH, H);
+  if (H != PH && H != 2 * PH)
+    return fail(FTK_ERR_UNSUPPORTED_SHAPE, "%s: the fp16 stack is built for H = %d and H = %d, got %d", who, PH, 2 * PH, H);
+  if (H == PH && (B & 1))
+    return fail(FTK_ERR_UNSUPPORTED_SHAPE, "%s: at H = %d two batch rows share a tile row, B = %d must be even", who, PH, B);
+  const int mode = H == PH ? kHalfData256 : kHalfData;
+  const int npc = H / 32;
   if (dilations)
     for (int l = 0; l < L; ++l)
       if (dilations[l] <= 0) return fail(FTK_ERR_INVALID_ARGUMENT, "%s: dilations[%d]=%d must be positive", who, l, dilations[l]);
@@ -1018,9 +1057,9 @@ int ftk_stacked_lstm_f16(const void* xs, const void* WU, const float* bias, cons
     }
   const void* fn = nullptr;
   int slots = 0;
-  int rc = persistent_slots(kHalfData, &fn, &slots);
+  int rc = persistent_slots(mode, &fn, &slots);
   if (rc) return rc;
-  const int chunk = std::min(slots / 16, kMaxLayers);  // layers whose weights fit on the chip at once
+  const int chunk = std::min(slots / npc, kMaxLayers);  // layers whose weights fit on the chip at once
   if (chunk < 1) return fail(FTK_ERR_DEVICE, "%s: the device cannot hold one layer's weights in registers", who);
   // deeper stacks run as consecutive launches of `chunk` layers: a chunk reads the hidden sequence of the
   // layer below it, complete by then, like the first chunk reads xs
@@ -1032,7 +1071,7 @@ int ftk_stacked_lstm_f16(const void* xs, const void* WU, const float* bias, cons
   for (int l0 = 0; l0 < L; l0 += chunk) {
     const int lc = std::min(chunk, L - l0);
     bool handled = false;
-    rc = run_persistent(kHalfData, l0 == 0 ? x16 : h16 + (size_t)(l0 - 1) * slab, w16 + (size_t)l0 * 2 * H * 4 * H,
+    rc = run_persistent(mode, l0 == 0 ? x16 : h16 + (size_t)(l0 - 1) * slab, w16 + (size_t)l0 * 2 * H * 4 * H,
                         bias ? bias + (size_t)l0 * 4 * H : nullptr, dilations ? dilations + l0 : nullptr, active_rows,
                         h16 + (size_t)l0 * slab, c16 + (size_t)l0 * slab, lc, T, B, workspace, workspace_bytes,
                         (hipStream_t)stream, &handled);

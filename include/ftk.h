@@ -143,14 +143,15 @@ int ftk_stacked_lstm_ragged_f32(const float* xs, const float* WU,
  * The stack with fp16 storage, the numeric form of the reference's CuTe LSTM:
  * xs [T,B,H], WU [L,2H,4H], hsss, csss [L,T,B,H] all fp16 (h and c are rounded
  * to fp16 when written, and read back rounded), bias [L,4H] fp32 or NULL, gate
- * sums accumulated in fp32.  H = 512, the second hidden size of the
- * reference's sweep: fp16 weights of that size take the registers the fp32
- * weights of H = 256 take, so the persistent kernel serves both; stacks deeper
- * than the chip holds at once (16 layers on 256 compute units) run as
+ * sums accumulated in fp32.  H = 512 or H = 256 (then B must be even), the
+ * first two hidden sizes of the reference's sweep: fp16 weights of H = 512
+ * take the registers the fp32 weights of H = 256 take, so the persistent
+ * kernel serves all of them; stacks deeper than the chip holds at once (16
+ * layers of H = 512, 32 of H = 256 on 256 compute units) run as
  * consecutive launches.  dilations, active_rows: host arrays or NULL, as above.
  * Replaces StackedLstmRegion1/2/3 with Element = half as instantiated by
  * benchmarks/rnn/fractaltensor/cute_stacked_lstm/stacked_lstm.cu:16-19,59-155
- * (run_bench<32, 64, 256, 512>, :186).
+ * (run_bench<32, 64, 256, 256> and <32, 64, 256, 512>, :185-186).
  */
 size_t ftk_stacked_lstm_f16_workspace_bytes(int L, int T, int B, int H);
 int ftk_stacked_lstm_f16(const void* xs, const void* WU, const float* bias,

@@ -221,18 +221,24 @@ def test_stacked_lstm_ragged_rejects_unsorted_rows(core):
 
 # fp16 storage, H = 512: tolerance 1e-2 (north star's figure for fp16 work) against the oracle that rounds h and c
 # to fp16 wherever the kernel does
-@pytest.mark.parametrize('L,T,B,dil,bias,ragged', [
-    (1, 6, 64, None, False, False),
-    (2, 5, 40, None, True, False),             # ragged last row block
-    (3, 8, 96, [1, 2, 4], True, False),
-    (2, 9, 64, None, True, True),              # half the rows stop after 4 steps
-    (18, 3, 32, None, False, False),           # deeper than the chip holds at once: two launches
+@pytest.mark.parametrize('H,L,T,B,dil,bias,ragged', [
+    (512, 1, 6, 64, None, False, False),
+    (512, 2, 5, 40, None, True, False),             # ragged last row block
+    (512, 3, 8, 96, [1, 2, 4], True, False),
+    (512, 2, 9, 64, None, True, True),              # half the rows stop after 4 steps
+    (512, 18, 3, 32, None, False, False),           # deeper than the chip holds at once: two launches
+    (256, 1, 6, 64, None, False, False),            # H = 256: two batch rows share a tile row
+    (256, 2, 5, 38, None, True, False),             # last row block holds three pairs
+    (256, 3, 8, 96, [1, 2, 4], True, False),
+    (256, 2, 9, 64, None, True, True),
+    (256, 2, 4, 2, None, True, False),              # one pair of rows
+    (256, 34, 3, 32, None, False, False),           # two launches
 ])
-def test_stacked_lstm_f16(core, L, T, B, dil, bias, ragged):
-    H = 512
+def test_stacked_lstm_f16(core, H, L, T, B, dil, bias, ragged):
     rng = np.random.default_rng(13)
     xs = rng.standard_normal((T, B, H)).astype(np.float16)
-    WU = rng.uniform(-1 / 24, 1 / 24, (L, 2 * H, 4 * H)).astype(np.float16)
+    WU = rng.uniform(-1 / 24, 1 / 24, (L, 2 * H, 4 * H)).astype(np.float16) if H == 512 else \
+        rng.uniform(-1 / 16, 1 / 16, (L, 2 * H, 4 * H)).astype(np.float16)
     bs = rng.uniform(-0.1, 0.1, (L, 4 * H)).astype(np.float32) if bias else None
     active = None
     lens = np.full(B, T)
@@ -254,11 +260,16 @@ def test_stacked_lstm_f16(core, L, T, B, dil, bias, ragged):
 
 
 def test_stacked_lstm_f16_rejects_other_hidden_sizes(core):
-    xs = torch.zeros((2, 32, 256), dtype=torch.float16, device='cuda')
-    WU = torch.zeros((1, 512, 1024), dtype=torch.float16, device='cuda')
+    xs = torch.zeros((2, 32, 128), dtype=torch.float16, device='cuda')
+    WU = torch.zeros((1, 256, 512), dtype=torch.float16, device='cuda')
     with pytest.raises(core.FtkError) as e:
         core.stacked_lstm_f16(xs, WU)
     assert e.value.code == -2 and 'H = 512' in str(e.value)
+    xs = torch.zeros((2, 33, 256), dtype=torch.float16, device='cuda')
+    WU = torch.zeros((1, 512, 1024), dtype=torch.float16, device='cuda')
+    with pytest.raises(core.FtkError) as e:
+        core.stacked_lstm_f16(xs, WU)                    # odd batch at H = 256
+    assert e.value.code == -2 and 'even' in str(e.value)
     with pytest.raises(TypeError):
         core.stacked_lstm_f16(xs.float(), WU)
 
