@@ -188,3 +188,21 @@ def test_embedding_lookup_feeds_the_fused_stacked_lstm():
         ref, _ = ko.stacked_lstm(xs, WU, bias)
         got = np.stack([hss[t][b].data.cpu().numpy().reshape(H) for t in range(n)])
         assert ko.max_rel_err(got, ref[-1][:, 0]) <= 1e-4
+
+
+def test_fused_stacked_lstm_keeps_an_fp16_program_in_fp16():
+    """FractalTensors of fp16 at a hidden size the fp16 kernel is built for stay fp16 end to end."""
+    L, T, B, H = 2, 5, 6, 256
+    g = torch.Generator().manual_seed(8)
+    Wss = FractalTensor.from_dense(((torch.rand((L, 4, H, H), generator=g) - 0.5) / 8).half().cuda(), 2)
+    Uss = FractalTensor.from_dense(((torch.rand((L, 4, H, H), generator=g) - 0.5) / 8).half().cuda(), 2)
+    bss = FractalTensor.from_dense(((torch.rand((L, 4, 1, H), generator=g) - 0.5) / 8).half().cuda(), 2)
+    xss = FractalTensor.from_dense(torch.randn((T, B, 1, H), generator=g).half().cuda(), 2)
+    hss = ops.fused.stacked_lstm(xss, Wss, Uss, bss)
+    out = hss.as_dense()
+    assert out.dtype == torch.float16 and tuple(out.shape) == (T, B, 1, H)
+    W = Wss.as_dense().cpu().numpy(); U = Uss.as_dense().cpu().numpy()
+    WU = np.stack([ko.fuse_gate_weights(W[l], U[l]) for l in range(L)])
+    bias = bss.as_dense().float().cpu().numpy().reshape(L, 4 * H)
+    ref, _ = ko.stacked_lstm_f16(xss.as_dense().cpu().numpy().reshape(T, B, H), WU, bias)
+    assert ko.max_rel_err(out.float().cpu().numpy().reshape(T, B, H), ref[-1].astype(np.float32)) <= 1e-2
