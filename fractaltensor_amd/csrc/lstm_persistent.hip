@@ -1,36 +1,40 @@
-// Persistent stacked / dilated LSTM for H = 256 on gfx950.
+// Persistent stacked / dilated LSTM on gfx950.
 //
 // One launch evaluates every (layer, time) cell.  The grid is one 256-thread
 // workgroup per compute unit; a fixed group of workgroups owns each layer for
-// the whole launch and keeps its slice of that layer's [W;U] (512 x 1024
-// fp32) in registers: a workgroup holds 128 gate columns (32 hidden units x
-// {i,f,o,c~}), each of its four waves 32 of them as 256 VGPRs per lane, the
-// MFMA "A" operands of v_mfma_f32_32x32x2_f32.  Eight such column slices make
-// a layer; with spare compute units a layer gets several row slices as well,
-// each handling its own subset of the batch's 32-row blocks.
+// the whole launch and keeps its slice of that layer's [W;U] in registers: a
+// workgroup holds 128 gate columns (32 hidden units x {i,f,o,c~}), each of its
+// four waves 32 of them as up to 256 VGPRs per lane, the MFMA "A" operands.
+// H/32 such column slices make a layer; with spare compute units a layer gets
+// several row slices as well, each handling its own subset of the batch's
+// 32-row blocks.  Four flavours share the code (see the constants below):
+// fp32 data at H = 256 with fp32 MFMAs or with every fp32 product formed as
+// three fp16 MFMAs of split operands, and fp16 data at H = 512 and H = 256.
 //
 // Work item = (t, row block).  For an item the workgroup stages the activation
-// tile [32, 512] = [x_t | h_{t-d}] in LDS, runs the K = 512 product against
-// the resident weights, applies bias, sigmoid/tanh and the state update in
-// registers (all four gates of a (row, unit) pair land in one lane, see
-// lstm_cell.hip) and writes h, c.  Batch rows never interact, so dependencies
-// are per row block: item (l, t, rb) needs h[l-1][t][rb] from the layer below
-// and h[l][t-d][rb] from all eight column slices of its own layer.  Layer l
-// therefore trails layer l-1 by an item or two: the wavefront of the
-// reference's region schedule, without launches, device syncs or scatter.
+// tile [32, x_t | h_{t-d}] in LDS, runs the product against the resident
+// weights, applies bias, sigmoid/tanh and the state update in registers (all
+// four gates of a (row, unit) pair land in one lane, see lstm_cell.hip) and
+// writes h, c.  Batch rows never interact, so dependencies are per row block:
+// item (l, t, rb) needs h[l-1][t][rb] from the layer below and h[l][t-d][rb]
+// from all column slices of its own layer.  Layer l therefore trails layer
+// l-1 by an item or two: the wavefront of the reference's region schedule,
+// without launches, device syncs or scatter.
 //
 // Hand-off between compute units (which may sit on different XCDs, whose L2
-// caches are not coherent with each other) uses no cache-wide fences: h is
-// written with agent-scope write-through stores and read with agent-scope
-// loads, every producer wave waits for its own stores to be acknowledged and
-// then increments flags[l][t][rb]; consumers poll that count with agent-scope
-// loads until it reaches 32 (8 column slices x 4 waves).  c is only ever re-read by the
-// workgroup that wrote it and goes through the cache normally.
+// caches are not coherent with each other) uses no cache-wide fences: what
+// other compute units read is written with agent-scope write-through stores
+// and read with agent-scope copies, every producer wave waits for its own
+// stores to be acknowledged and then increments flags[l][t][rb]; consumers
+// look at that count with agent-scope loads until it reaches 4 x the number of
+// column slices.  c is only ever re-read by the workgroup that wrote it and
+// goes through the cache normally.
 //
-// The activation tile is double buffered and the item loop is software
-// pipelined: the loads of tile n+1 are issued half way through item n, and the
-// activations / state update / stores of item n-1 run in the shadow of item
-// n's first MFMAs.  One workgroup barrier per item.
+// The activation tile is double buffered, global -> LDS copies are requested
+// an item ahead, results leave through an LDS staging area as full cache
+// lines, and the order of everything within an item follows from one fact
+// (comment above the loop): loads and stores share a counter, so a load result
+// is only known once nothing at all is outstanding.  Two barriers per item.
 //
 // All workgroups must be co-resident: the host launches cooperatively with at
 // most one workgroup per compute unit (each uses the whole register file of
