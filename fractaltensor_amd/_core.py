@@ -18,7 +18,7 @@ LIB_PATH = os.path.join(_HERE, 'libftkernels.so')
 # every symbol include/ftk.h declares; checked at load time
 EXPORTS = (
     'ftk_version', 'ftk_last_error', 'ftk_device_info_query',
-    'ftk_lstm_cell_f32', 'ftk_lstm_elementwise_f32',
+    'ftk_lstm_cell_f32', 'ftk_lstm_cell_f16', 'ftk_lstm_elementwise_f32',
     'ftk_stacked_lstm_workspace_bytes', 'ftk_stacked_lstm_f32', 'ftk_dilated_lstm_f32',
     'ftk_stacked_lstm_wavefront_f32', 'ftk_stacked_lstm_ragged_f32', 'ftk_lstm_set_products', 'ftk_lstm_get_products',
     'ftk_stacked_lstm_f16_workspace_bytes', 'ftk_stacked_lstm_f16',
@@ -120,6 +120,27 @@ def lstm_cell(x, h_prev, c_prev, WU, bias=None) -> Tuple[torch.Tensor, torch.Ten
     return h, c
 
 
+def lstm_cell_f16(x, h_prev, c_prev, WU, bias=None) -> Tuple[torch.Tensor, torch.Tensor]:
+    """The fused cell with fp16 storage: x [B,I], h_prev/c_prev [B,H] or None, WU [(I+H),4H] fp16, bias [4H]
+    fp32 or None; I and H multiples of 32.  Gate sums in fp32, h and c rounded to fp16 when written."""
+    f16 = torch.float16
+    _req(x, f16, 'x'); _req(WU, f16, 'WU')
+    B, I = x.shape
+    H = WU.shape[1] // 4
+    if WU.shape != (I + H, 4 * H):
+        raise ValueError(f'WU must be [(I+H), 4H] = [{I + H}, {4 * H}], got {tuple(WU.shape)}')
+    for t, n in ((h_prev, 'h_prev'), (c_prev, 'c_prev')):
+        if t is not None and _req(t, f16, n).shape != (B, H):
+            raise ValueError(f'{n} must be [{B}, {H}]')
+    if bias is not None and _req(bias, torch.float32, 'bias').numel() != 4 * H:
+        raise ValueError('bias must have 4H elements')
+    h = torch.empty((B, H), dtype=f16, device=x.device)
+    c = torch.empty((B, H), dtype=f16, device=x.device)
+    _check(lib.ftk_lstm_cell_f16(_ptr(x), _ptr(h_prev), _ptr(c_prev), _ptr(WU), _ptr(bias), _ptr(h), _ptr(c),
+                                 ctypes.c_int(B), ctypes.c_int(I), ctypes.c_int(H), _stream()))
+    return h, c
+
+
 def lstm_elementwise(gates, bias, c_prev, out: Optional[Tuple[torch.Tensor, torch.Tensor]] = None
                      ) -> Tuple[torch.Tensor, torch.Tensor]:
     """State update on pre-activation gates [B,4H] (the unfused baseline's second kernel)."""
@@ -206,7 +227,8 @@ def stacked_lstm_f16(xs, WU, bias=None, dilations: Optional[Sequence[int]] = Non
                      out: Optional[Tuple[torch.Tensor, torch.Tensor]] = None, workspace: Optional[torch.Tensor] = None,
                      active_rows: Optional[Sequence[int]] = None) -> Tuple[torch.Tensor, torch.Tensor]:
     """fp16 storage: xs [T,B,H], WU [L,2H,4H] fp16, bias [L,4H] fp32 or None -> hsss, csss [L,T,B,H] fp16.
-    H = 512, or H = 256 with an even batch."""
+    H a multiple of 32: H = 512, and H = 256 with an even batch, run in the persistent kernel, every other
+    shape as one launch of the streaming cell kernel per stage of independent cells."""
     f16 = torch.float16
     _req(xs, f16, 'xs'); _req(WU, f16, 'WU')
     T, B, H = xs.shape

@@ -16,6 +16,13 @@
 // Within a chunk the k index is permuted so that one 16-byte LDS read feeds
 // four MFMAs: step (q, c) uses k = 8q + c for lanes 0-31 and k = 8q + 4 + c
 // for lanes 32-63.
+//
+// lstm_cell_f16_kernel is the fp16-storage flavour for hidden sizes whose
+// weights no longer fit on chip: the same transposed product on
+// v_mfma_f32_32x32x16_f16, a workgroup of 4 waves owning 256 batch rows x 32
+// hidden units so that every weight is fetched once per cell, and k chunks of
+// 32 copied from global memory straight into a three-deep ring of LDS stages
+// (global_load_lds_dwordx4), two workgroups per compute unit.
 #include <algorithm>
 #include <vector>
 
@@ -206,17 +213,274 @@ __global__ __launch_bounds__(256) void lstm_elementwise_kernel(const float* __re
   }
 }
 
+// ---------------------------------------------------------------- fp16 cell
+struct CellDescH {
+  const _Float16* x;       // [B, I]
+  const _Float16* h_prev;  // [B, H] or nullptr (zero state)
+  const _Float16* c_prev;  // [B, H] or nullptr
+  const _Float16* WU;      // [(I+H), 4H]
+  const float* bias;       // [4H] or nullptr
+  _Float16* h;             // [B, H]
+  _Float16* c;             // [B, H]
+};
+
+struct CellListH {
+  int n;
+  int packed;  // WU of every cell is in the packed layout
+  CellDescH cells[kMaxCellsPerLaunch];
+};
+
+constexpr int HK = 32;                       // k chunk
+constexpr int HROWS = 256;                   // batch rows per workgroup
+constexpr int H_ACT_BYTES = HROWS * HK * 2;  // activation rows of a chunk: 64 bytes each
+constexpr int H_W_BYTES = HK * 128 * 2;      // weight rows of a chunk: 128 gate columns, 256 bytes each
+constexpr int H_STAGE = H_ACT_BYTES + H_W_BYTES;
+constexpr int H_STAGES = 3;
+constexpr size_t kCellF16Lds = (size_t)H_STAGE * H_STAGES;  // 72 KB: two workgroups per compute unit
+
+typedef short v4s __attribute__((ext_vector_type(4)));
+typedef short v8s __attribute__((ext_vector_type(8)));
+
+// 16 bytes per lane from global memory (wave-uniform base + per-lane byte offset) straight into LDS at
+// lds_addr + 16*lane (lds_addr wave-uniform).  Opaque to the compiler: the caller waits with s_waitcnt vmcnt.
+__device__ __forceinline__ void cell_dma16(const void* gbase, unsigned byte_off, unsigned lds_addr) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
+               :: "s"(lds_addr), "v"(byte_off), "s"(gbase) : "memory", "m0");
+}
+
+// LDS layout of a stage.  Both tiles are stored row-major as in memory, without padding, and their 16-byte
+// chunks are swapped around within a row so that fragment reads do not collide on banks:
+//   activation row r (64 bytes, 4 chunks): chunk c sits in slot c ^ ((r >> 2) & 3); the 16 lanes that a
+//     ds_read_b128 serves together (16 consecutive rows, one chunk index) then touch 16 different 16-byte
+//     positions of the 256-byte bank line;
+//   weight row k (256 bytes, 16 chunks; chunk 4*ug + q = gate q of the 8 units of unit group ug): chunk c sits
+//     in slot c ^ ((k & 3) << 2); the transposing read ds_read_b64_tr_b16 takes 64 bytes from each of four
+//     consecutive rows per pass, which land in four different 64-byte groups.
+// A copy instruction fills 1 KB of consecutive slots, each lane choosing the global chunk its slot holds.
+// Three stages: while chunk ch is used, chunks ch + 1 and ch + 2 are on their way; a second workgroup on the
+// compute unit fills the gaps the barriers and LDS latencies of the first leave.
+//
+// PACKED: the cell's WU points at weights laid out by lstm_pack_weights_f16_kernel, per unit block the very
+// bytes of the LDS rows above, so a workgroup streams one contiguous run of 256-byte rows; otherwise at the
+// [(I+H), 4H] matrix, from which a workgroup picks four 64-byte segments per row.
+template <bool PACKED>
+__global__ __launch_bounds__(256, 2) void lstm_cell_f16_kernel(CellListH list, int B, int I, int H) {
+  extern __shared__ __attribute__((aligned(1024))) unsigned char cell_smem[];
+  using lds_v4s = __attribute__((address_space(3))) v4s;
+
+  // Workgroups are dealt to the 8 XCDs round-robin by their linear index.  All workgroups of a cell are
+  // placed on one XCD (cell = xcd + 8 m), neighbouring unit blocks first: the cell's activation rows are then
+  // fetched into one L2 instead of eight, and the 64-byte weight segments of neighbouring unit blocks that
+  // share a cache line are served by the same L2.
+  const int nub = H / 32, nrb = (B + HROWS - 1) / HROWS;
+  const int slot = blockIdx.x >> 3;
+  const int cell = (blockIdx.x & 7) + 8 * (slot / (nub * nrb));
+  if (cell >= list.n) return;
+  const CellDescH cd = list.cells[cell];
+  const int ub = slot % nub;          // block of 32 hidden units
+  const int rb = (slot / nub) % nrb;  // block of 256 batch rows
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int wr = wave >> 1;  // rows 128*wr .. +128 of the block
+  const int wc = wave & 1;   // unit groups 2*wc, 2*wc+1 of the block's four
+  const int j = lane & 31;
+  const int hh = lane >> 5;
+  const unsigned lds0 = (unsigned)reinterpret_cast<uintptr_t>((__attribute__((address_space(3))) void*)cell_smem);
+
+  const int nch_x = I / HK;
+  const int nch = nch_x + (cd.h_prev ? H / HK : 0);
+  const bool full = rb * HROWS + HROWS <= B;
+
+  // ---- copies: per chunk a wave issues 4 activation copies (rows 64*wave + 16 i + lane/4) and 2 weight
+  // copies (k rows 8*wave + 4 i + lane/16)
+  const unsigned a_lane_chunk = (unsigned)(((lane & 3) ^ ((lane >> 4) & 3)) * 16);
+  const unsigned wl = (unsigned)lane >> 4;
+  const unsigned wchunk = ((unsigned)lane & 15) ^ (wl << 2);  // 4*ug + q
+  const unsigned w_lane_off = wl * (unsigned)(8 * H) + ((wchunk & 3) * (unsigned)H + (wchunk >> 2) * 8) * 2;
+
+  auto issue = [&](int ch, int stage) __attribute__((always_inline)) {
+    const _Float16* src;
+    int ld, k0;
+    if (ch < nch_x) {
+      src = cd.x; ld = I; k0 = ch * HK;
+    } else {
+      src = cd.h_prev; ld = H; k0 = (ch - nch_x) * HK;
+    }
+    const unsigned act_lds = lds0 + (unsigned)(stage * H_STAGE + wave * 4096);
+    if (full) {
+      const char* base = reinterpret_cast<const char*>(src + (size_t)(rb * HROWS + wave * 64) * ld + k0);
+      const unsigned off = ((unsigned)lane >> 2) * (unsigned)(2 * ld) + a_lane_chunk;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) cell_dma16(base + (size_t)i * 32 * ld, off, act_lds + 1024u * i);
+    } else {  // rows past the end of the batch repeat the last row; they are never stored
+      const char* base = reinterpret_cast<const char*>(src + k0);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int row = min(rb * HROWS + wave * 64 + 16 * i + (lane >> 2), B - 1);
+        cell_dma16(base, (unsigned)row * (unsigned)(2 * ld) + a_lane_chunk, act_lds + 1024u * i);
+      }
+    }
+    const unsigned w_lds = lds0 + (unsigned)(stage * H_STAGE + H_ACT_BYTES + wave * 2048);
+    if constexpr (PACKED) {
+      const char* wbase = reinterpret_cast<const char*>(cd.WU + ((size_t)ub * (I + H) + ch * HK + wave * 8) * 128);
+#pragma unroll
+      for (int i = 0; i < 2; ++i) cell_dma16(wbase + 1024 * i, 16u * lane, w_lds + 1024u * i);
+    } else {
+      const char* wbase = reinterpret_cast<const char*>(cd.WU + (size_t)(ch * HK + wave * 8) * 4 * H + ub * 32);
+#pragma unroll
+      for (int i = 0; i < 2; ++i) cell_dma16(wbase + (size_t)i * 32 * H, w_lane_off, w_lds + 1024u * i);
+    }
+  };
+
+  // ---- fragment addresses within a stage
+  unsigned a_off[2], w_off[2];
+#pragma unroll
+  for (int ks = 0; ks < 2; ++ks) a_off[ks] = (unsigned)((128 * wr + j) * 64 + (((2 * ks + hh) ^ ((j >> 2) & 3)) * 16));
+  {
+    const int ta = (lane & 15) >> 2, tb = lane & 3, th = (lane >> 4) & 1;
+#pragma unroll
+    for (int u2 = 0; u2 < 2; ++u2)
+      w_off[u2] = (unsigned)(H_ACT_BYTES + (8 * hh + ta) * 256 +
+                             (((4 * (2 * wc + u2) + 2 * th + (tb >> 1)) ^ (ta << 2)) * 16) + 8 * (tb & 1));
+  }
+
+  v16f acc[4][2];
+#pragma unroll
+  for (int rt = 0; rt < 4; ++rt)
+#pragma unroll
+    for (int u2 = 0; u2 < 2; ++u2)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[rt][u2][r] = 0.0f;
+
+  issue(0, 0);
+  if (nch > 1) issue(1, 1);
+  int stage = 0;
+  for (int ch = 0; ch < nch; ++ch) {
+    // 6 copies per wave and chunk, completing in order: all but the newest chunk's have landed
+    if (ch + 1 < nch)
+      __builtin_amdgcn_s_waitcnt(0x0F76);  // vmcnt(6)
+    else
+      __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
+    __syncthreads();  // chunk ch is complete, and every wave is done with the stage of chunk ch-1
+    if (ch + 2 < nch) issue(ch + 2, stage == 0 ? 2 : stage - 1);
+    const unsigned char* sb = cell_smem + stage * H_STAGE;
+#pragma unroll
+    for (int ks = 0; ks < 2; ++ks) {
+      v8h wf[2];
+#pragma unroll
+      for (int u2 = 0; u2 < 2; ++u2) {
+        const unsigned char* p0 = sb + w_off[u2] + 4096 * ks;
+        const v4s lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4s*)(p0));
+        const v4s hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4s*)(p0 + 1024));
+        const v8s both = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+        wf[u2] = __builtin_bit_cast(v8h, both);
+      }
+#pragma unroll
+      for (int rt = 0; rt < 4; ++rt) {
+        const v8h af = *reinterpret_cast<const v8h*>(sb + a_off[ks] + 2048 * rt);
+#pragma unroll
+        for (int u2 = 0; u2 < 2; ++u2)
+          acc[rt][u2] = __builtin_amdgcn_mfma_f32_32x32x16_f16(wf[u2], af, acc[rt][u2], 0, 0, 0);
+      }
+    }
+    stage = stage == 2 ? 0 : stage + 1;
+  }
+
+  // Epilogue: lane (row j, half hh) holds the four gates of units 4*hh .. 4*hh+3 of each of its unit groups.
+#pragma unroll
+  for (int rt = 0; rt < 4; ++rt) {
+    const int row_g = rb * HROWS + 128 * wr + 32 * rt + j;
+    if (row_g >= B) continue;
+#pragma unroll
+    for (int u2 = 0; u2 < 2; ++u2) {
+      const int u0 = ub * 32 + 8 * (2 * wc + u2) + 4 * hh;
+      v4h cp = {0, 0, 0, 0};
+      if (cd.c_prev) cp = *reinterpret_cast<const v4h*>(cd.c_prev + (size_t)row_g * H + u0);
+      v4f bi = {0, 0, 0, 0}, bf = bi, bo = bi, bg = bi;
+      if (cd.bias) {
+        bi = *reinterpret_cast<const v4f*>(cd.bias + u0);
+        bf = *reinterpret_cast<const v4f*>(cd.bias + H + u0);
+        bo = *reinterpret_cast<const v4f*>(cd.bias + 2 * H + u0);
+        bg = *reinterpret_cast<const v4f*>(cd.bias + 3 * H + u0);
+      }
+      v4h hv, cv;
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const float ig = sigmoid_f(acc[rt][u2][r] + bi[r]);
+        const float fg = sigmoid_f(acc[rt][u2][4 + r] + bf[r]);
+        const float og = sigmoid_f(acc[rt][u2][8 + r] + bo[r]);
+        const float cand = tanh_f(acc[rt][u2][12 + r] + bg[r]);
+        const float cn = fg * (float)cp[r] + ig * cand;
+        cv[r] = (_Float16)cn;
+        hv[r] = (_Float16)(og * tanh_f(cn));
+      }
+      *reinterpret_cast<v4h*>(cd.c + (size_t)row_g * H + u0) = cv;
+      *reinterpret_cast<v4h*>(cd.h + (size_t)row_g * H + u0) = hv;
+    }
+  }
+}
+
 static int launch_cells(const CellList& list, int B, int I, int H, hipStream_t s) {
   dim3 grid(H / 32, (B + 31) / 32, list.n);
   hipLaunchKernelGGL(lstm_cell_kernel, grid, dim3(256), 0, s, list, B, I, H);
   return check_launch("lstm_cell_kernel");
 }
 
+// WU [n_layers, K2, 4H] -> per layer and unit block ub the [K2][128] tile the cell kernel keeps in LDS: row k
+// holds 16 chunks of 8 columns, chunk 4*ug + q = gate q of units 32*ub + 8*ug .. +8, stored in slot
+// chunk ^ ((k & 3) << 2).  One thread per 16-byte chunk.
+__global__ __launch_bounds__(256) void lstm_pack_weights_f16_kernel(const _Float16* __restrict__ WU,
+                                                                    _Float16* __restrict__ packed, size_t chunks,
+                                                                    int K2, int H) {
+  const size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;
+  if (idx >= chunks) return;
+  const int per_row = H / 2;  // 4H / 8
+  const int n8 = (int)(idx % per_row);
+  const size_t lk = idx / per_row;
+  const int k = (int)(lk % K2);
+  const size_t l = lk / K2;
+  const int col = 8 * n8;
+  const int q = col / H, u = col % H;
+  const int ub = u >> 5, ug = (u & 31) >> 3;
+  const int slot = (4 * ug + q) ^ ((k & 3) << 2);
+  const v4u v = *reinterpret_cast<const v4u*>(WU + idx * 8);
+  *reinterpret_cast<v4u*>(packed + ((l * (H / 32) + ub) * K2 + k) * 128 + 8 * slot) = v;
+}
+
+int pack_weights_f16(const void* WU, void* packed, int layers, int K2, int H, hipStream_t s) {
+  const size_t chunks = (size_t)layers * K2 * (H / 2);
+  hipLaunchKernelGGL(lstm_pack_weights_f16_kernel, dim3((unsigned)((chunks + 255) / 256)), dim3(256), 0, s,
+                     (const _Float16*)WU, (_Float16*)packed, chunks, K2, H);
+  return check_launch("lstm_pack_weights_f16_kernel");
+}
+
+template <bool PACKED>
+static int launch_cells_f16(const CellListH& list, int B, int I, int H, hipStream_t s) {
+  static bool attr_set = false;  // per process; the attribute belongs to the function, on every device
+  const void* fn = (const void*)lstm_cell_f16_kernel<PACKED>;
+  if (!attr_set) {
+    FTK_HIP(hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)kCellF16Lds));
+    attr_set = true;
+  }
+  const int groups = (list.n + 7) / 8;  // cells per XCD
+  dim3 grid(8 * groups * (H / 32) * ((B + HROWS - 1) / HROWS));
+  hipLaunchKernelGGL(lstm_cell_f16_kernel<PACKED>, grid, dim3(256), kCellF16Lds, s, list, B, I, H);
+  return check_launch("lstm_cell_f16_kernel");
+}
+
+static int launch_cells(const CellListH& list, int B, int I, int H, hipStream_t s) {
+  return list.packed ? launch_cells_f16<true>(list, B, I, H, s) : launch_cells_f16<false>(list, B, I, H, s);
+}
+
 // Host side of the per-stage schedule: stage(l,t) = 1 + max(stage(l-1,t),
 // stage(l,t-d_l)); cells of equal stage are independent and go out as one
 // batched launch.  For d = 1 the stages are the diagonals l + t.
-int run_wavefront(const float* xs, const float* WU, const float* bias, const int* dil, float* hsss, float* csss,
-                  int L, int T, int B, int H, hipStream_t s) {
+static void set_packed(CellList&, bool) {}
+static void set_packed(CellListH& list, bool packed) { list.packed = packed; }
+
+template <typename Elem, typename List>
+static int run_wavefront_of(const Elem* xs, const Elem* WU, const float* bias, const int* dil, Elem* hsss, Elem* csss,
+                            int L, int T, int B, int H, hipStream_t s, bool packed = false) {
   std::vector<int> stage((size_t)L * T, 0);
   int max_stage = 0;
   for (int l = 0; l < L; ++l) {
@@ -237,12 +501,13 @@ int run_wavefront(const float* xs, const float* WU, const float* bias, const int
   for (const auto& cells : by_stage) {
     size_t pos = 0;
     while (pos < cells.size()) {
-      CellList list;
+      List list;
       list.n = 0;
+      set_packed(list, packed);
       while (pos < cells.size() && list.n < kMaxCellsPerLaunch) {
         const int l = cells[pos] / T, t = cells[pos] % T;
         const int d = dil ? dil[l] : 1;
-        CellDesc& cd = list.cells[list.n++];
+        auto& cd = list.cells[list.n++];
         cd.x = (l == 0) ? xs + (size_t)t * cell : hsss + ((size_t)(l - 1) * T + t) * cell;
         cd.h_prev = (t >= d) ? hsss + ((size_t)l * T + t - d) * cell : nullptr;
         cd.c_prev = (t >= d) ? csss + ((size_t)l * T + t - d) * cell : nullptr;
@@ -257,6 +522,23 @@ int run_wavefront(const float* xs, const float* WU, const float* bias, const int
     }
   }
   return FTK_OK;
+}
+
+int run_wavefront(const float* xs, const float* WU, const float* bias, const int* dil, float* hsss, float* csss,
+                  int L, int T, int B, int H, hipStream_t s) {
+  return run_wavefront_of<float, CellList>(xs, WU, bias, dil, hsss, csss, L, T, B, H, s);
+}
+
+// The same schedule over fp16 arrays (H a multiple of 32).  packed: a buffer of the size of WU, into which the
+// weights are first re-laid per unit block, or nullptr to read WU as it is.
+int run_wavefront_f16(const void* xs, const void* WU, const float* bias, const int* dil, void* hsss, void* csss,
+                      int L, int T, int B, int H, void* packed, hipStream_t s) {
+  if (packed) {
+    int rc = pack_weights_f16(WU, packed, L, 2 * H, H, s);
+    if (rc) return rc;
+  }
+  return run_wavefront_of<_Float16, CellListH>((const _Float16*)xs, (const _Float16*)(packed ? packed : WU), bias, dil,
+                                               (_Float16*)hsss, (_Float16*)csss, L, T, B, H, s, packed != nullptr);
 }
 
 }  // namespace ftk
@@ -275,6 +557,24 @@ int ftk_lstm_cell_f32(const float* x, const float* h_prev, const float* c_prev, 
   ftk::CellList list;
   list.n = 1;
   list.cells[0] = ftk::CellDesc{x, h_prev, c_prev, WU, bias, h, c};
+  return ftk::launch_cells(list, B, I, H, (hipStream_t)stream);
+}
+
+int ftk_lstm_cell_f16(const void* x, const void* h_prev, const void* c_prev, const void* WU, const float* bias,
+                      void* h, void* c, int B, int I, int H, ftk_stream_t stream) {
+  if (!x || !WU || !h || !c) return ftk::fail(FTK_ERR_INVALID_ARGUMENT, "ftk_lstm_cell_f16: x, WU, h, c must be non-NULL");
+  if ((h_prev == nullptr) != (c_prev == nullptr))
+    return ftk::fail(FTK_ERR_INVALID_ARGUMENT, "ftk_lstm_cell_f16: h_prev and c_prev must both be given or both be NULL");
+  if (B <= 0 || I <= 0 || H <= 0) return ftk::fail(FTK_ERR_INVALID_ARGUMENT, "ftk_lstm_cell_f16: B, I, H must be positive");
+  if (I % 32 || H % 32)
+    return ftk::fail(FTK_ERR_UNSUPPORTED_SHAPE, "ftk_lstm_cell_f16: I=%d and H=%d must be multiples of 32", I, H);
+  if ((long long)B * std::max(I, H) >= (1ll << 30))
+    return ftk::fail(FTK_ERR_UNSUPPORTED_SHAPE, "ftk_lstm_cell_f16: B=%d too large", B);
+  ftk::CellListH list;
+  list.n = 1;
+  list.packed = 0;
+  list.cells[0] = ftk::CellDescH{(const _Float16*)x, (const _Float16*)h_prev, (const _Float16*)c_prev,
+                                 (const _Float16*)WU, bias, (_Float16*)h, (_Float16*)c};
   return ftk::launch_cells(list, B, I, H, (hipStream_t)stream);
 }
 

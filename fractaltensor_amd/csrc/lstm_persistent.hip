@@ -51,6 +51,8 @@ namespace ftk {
 
 int run_wavefront(const float* xs, const float* WU, const float* bias, const int* dil, float* hsss, float* csss,
                   int L, int T, int B, int H, hipStream_t s);
+int run_wavefront_f16(const void* xs, const void* WU, const float* bias, const int* dil, void* hsss, void* csss,
+                      int L, int T, int B, int H, void* packed, hipStream_t s);
 
 constexpr int PH = 256;            // hidden size this kernel is specialised for
 constexpr int PK = 2 * PH;         // K of the gate GEMM
@@ -1033,6 +1035,8 @@ size_t ftk_stacked_lstm_workspace_bytes(int L, int T, int B, int H) {
 
 size_t ftk_stacked_lstm_f16_workspace_bytes(int L, int T, int B, int H) {
   if (L <= 0 || T <= 0 || B <= 0 || H <= 0) return 0;
+  const bool on_chip = H == 2 * ftk::PH || (H == ftk::PH && !(B & 1));
+  if (!on_chip) return (size_t)L * 2 * H * 4 * H * sizeof(_Float16);  // the re-laid weights of the streaming kernel
   return ftk::xratio_offset_bytes(L, T, B);
 }
 
@@ -1043,10 +1047,10 @@ int ftk_stacked_lstm_f16(const void* xs, const void* WU, const float* bias, cons
   const char* who = "ftk_stacked_lstm_f16";
   if (!xs || !WU || !hsss || !csss) return fail(FTK_ERR_INVALID_ARGUMENT, "%s: xs, WU, hsss, csss must be non-NULL", who);
   if (L <= 0 || T <= 0 || B <= 0 || H <= 0) return fail(FTK_ERR_INVALID_ARGUMENT, "%s: L, T, B, H must be positive", who);
-  if (H != PH && H != 2 * PH)
-    return fail(FTK_ERR_UNSUPPORTED_SHAPE, "%s: the fp16 stack is built for H = %d and H = %d, got %d", who, PH, 2 * PH, H);
-  if (H == PH && (B & 1))
-    return fail(FTK_ERR_UNSUPPORTED_SHAPE, "%s: at H = %d two batch rows share a tile row, B = %d must be even", who, PH, B);
+  if (H % 32) return fail(FTK_ERR_UNSUPPORTED_SHAPE, "%s: H=%d must be a multiple of 32", who, H);
+  if ((long long)B * H >= (1ll << 30)) return fail(FTK_ERR_UNSUPPORTED_SHAPE, "%s: B*H = %lld is too large", who, (long long)B * H);
+  // the persistent kernel holds the weights of H = 512, and of H = 256 with two batch rows per tile row (even B)
+  const bool on_chip = H == 2 * PH || (H == PH && !(B & 1));
   const int mode = H == PH ? kHalfData256 : kHalfData;
   const int npc = H / 32;
   if (dilations)
@@ -1059,6 +1063,14 @@ int ftk_stacked_lstm_f16(const void* xs, const void* WU, const float* bias, cons
       if (t > 0 && active_rows[t] > active_rows[t - 1])
         return fail(FTK_ERR_INVALID_ARGUMENT, "%s: active_rows must be non-increasing (rows sorted by length)", who);
     }
+  // every other shape streams the weights, one launch per stage of independent cells (dead rows are computed too)
+  // (the workspace takes the weights re-laid per unit block, so that a workgroup reads one contiguous run)
+  if (!on_chip) {
+    const size_t need = ftk_stacked_lstm_f16_workspace_bytes(L, T, B, H);
+    if (!workspace || workspace_bytes < need)
+      return fail(FTK_ERR_WORKSPACE, "%s: workspace of %zu bytes needed, %zu given", who, need, workspace ? workspace_bytes : (size_t)0);
+    return run_wavefront_f16(xs, WU, bias, dilations, hsss, csss, L, T, B, H, workspace, (hipStream_t)stream);
+  }
   const void* fn = nullptr;
   int slots = 0;
   int rc = persistent_slots(mode, &fn, &slots);

@@ -110,7 +110,7 @@ def _run_stack(xss, Wss, Uss, bss, dilations, return_all_layers):
     WU, bias = pack_lstm_weights(Wss, Uss, bss)
     # a ragged batch goes down with its per-step row counts: 32-row blocks that have ended are skipped
     T_, B_, H_ = xs.shape
-    if xs.dtype == torch.float16 and WU.dtype == torch.float16 and (H_ == 512 or (H_ == 256 and B_ % 2 == 0)):
+    if xs.dtype == torch.float16 and WU.dtype == torch.float16 and H_ % 32 == 0:
         # fp16 program, fp16 kernel: h and c are kept in fp16 like every other tensor of the program
         hsss, csss = core.stacked_lstm_f16(xs, WU, None if bias is None else bias.float(), dilations=dilations,
                                            active_rows=sizes)

@@ -77,6 +77,19 @@ int ftk_lstm_cell_f32(const float* x, const float* h_prev, const float* c_prev,
                       int B, int I, int H, ftk_stream_t stream);
 
 /*
+ * The same cell with fp16 storage: x, h_prev, c_prev, WU, h, c fp16, bias fp32
+ * or NULL; gate sums and the state update in fp32, h and c rounded to fp16 when
+ * written.  Needs I%32==0, H%32==0.  The weights are streamed through LDS, so
+ * any hidden size runs; a workgroup takes 256 batch rows, which at B <= 256
+ * fetches every weight once.  The element types of CuteLSTMCell as the
+ * reference instantiates it (cutlass::half_t, kaleido/core/device/kernels/lstm.h:253-348;
+ * fp32 accumulators, lstm_kernels.h:25-126).
+ */
+int ftk_lstm_cell_f16(const void* x, const void* h_prev, const void* c_prev,
+                      const void* WU, const float* bias, void* h, void* c,
+                      int B, int I, int H, ftk_stream_t stream);
+
+/*
  * The state-update half alone, for the unfused baseline: gates [B,4H] already
  * holds x@W + h@U (pre-activation, blocks i|f|o|c~); bias [4H] or NULL;
  * c_prev [B,H] or NULL.  Replaces ElementwiseLstmAct
@@ -143,15 +156,20 @@ int ftk_stacked_lstm_ragged_f32(const float* xs, const float* WU,
  * The stack with fp16 storage, the numeric form of the reference's CuTe LSTM:
  * xs [T,B,H], WU [L,2H,4H], hsss, csss [L,T,B,H] all fp16 (h and c are rounded
  * to fp16 when written, and read back rounded), bias [L,4H] fp32 or NULL, gate
- * sums accumulated in fp32.  H = 512 or H = 256 (then B must be even), the
- * first two hidden sizes of the reference's sweep: fp16 weights of H = 512
- * take the registers the fp32 weights of H = 256 take, so the persistent
- * kernel serves all of them; stacks deeper than the chip holds at once (16
- * layers of H = 512, 32 of H = 256 on 256 compute units) run as
- * consecutive launches.  dilations, active_rows: host arrays or NULL, as above.
+ * sums accumulated in fp32.  H%32==0.  H = 512 and H = 256 with even B, the
+ * first two hidden sizes of the reference's sweep, run in the persistent
+ * kernel: fp16 weights of H = 512 take the registers the fp32 weights of
+ * H = 256 take; stacks deeper than the chip holds at once (16 layers of
+ * H = 512, 32 of H = 256 on 256 compute units) run as consecutive launches.
+ * Every other shape (H = 1024, the third size of the sweep, among them) does
+ * not fit on chip: its weights are streamed, one launch of the fp16 cell
+ * kernel per stage of independent cells, which computes dead rows too; the
+ * workspace then takes a re-laid copy of WU (ftk_stacked_lstm_f16_workspace_bytes
+ * says how much for a shape).
+ * dilations, active_rows: host arrays or NULL, as above.
  * Replaces StackedLstmRegion1/2/3 with Element = half as instantiated by
  * benchmarks/rnn/fractaltensor/cute_stacked_lstm/stacked_lstm.cu:16-19,59-155
- * (run_bench<32, 64, 256, 256> and <32, 64, 256, 512>, :185-186).
+ * (run_bench<32, 64, 256, 256>, <32, 64, 256, 512>, <32, 64, 256, 1024>, :185-187).
  */
 size_t ftk_stacked_lstm_f16_workspace_bytes(int L, int T, int B, int H);
 int ftk_stacked_lstm_f16(const void* xs, const void* WU, const float* bias,

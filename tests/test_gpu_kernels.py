@@ -233,12 +233,17 @@ def test_stacked_lstm_ragged_rejects_unsorted_rows(core):
     (256, 2, 9, 64, None, True, True),
     (256, 2, 4, 2, None, True, False),              # one pair of rows
     (256, 34, 3, 32, None, False, False),           # two launches
+    (1024, 2, 4, 256, None, True, False),           # weights streamed: one launch per stage of cells
+    (1024, 3, 6, 40, [1, 2, 4], False, False),      # 40 of a workgroup's 256 rows exist
+    (128, 2, 5, 300, None, True, False),            # two row blocks, the second ragged
+    (256, 2, 5, 37, None, True, False),             # odd batch at H = 256 goes the streamed way
+    (192, 2, 7, 64, None, True, True),
+    (96, 9, 3, 20, None, False, False),             # nine cells in a stage: a second round over the XCDs
 ])
 def test_stacked_lstm_f16(core, H, L, T, B, dil, bias, ragged):
     rng = np.random.default_rng(13)
     xs = rng.standard_normal((T, B, H)).astype(np.float16)
-    WU = rng.uniform(-1 / 24, 1 / 24, (L, 2 * H, 4 * H)).astype(np.float16) if H == 512 else \
-        rng.uniform(-1 / 16, 1 / 16, (L, 2 * H, 4 * H)).astype(np.float16)
+    WU = rng.uniform(-1, 1, (L, 2 * H, 4 * H)).astype(np.float16) / np.float16(np.sqrt(H))
     bs = rng.uniform(-0.1, 0.1, (L, 4 * H)).astype(np.float32) if bias else None
     active = None
     lens = np.full(B, T)
@@ -254,24 +259,66 @@ def test_stacked_lstm_f16(core, H, L, T, B, dil, bias, ragged):
     got_h = hsss.float().cpu().numpy()[:, live]; got_c = csss.float().cpu().numpy()[:, live]
     eh = ko.max_rel_err(got_h, hr.astype(np.float32)[:, live]); ec = ko.max_rel_err(got_c, cr.astype(np.float32)[:, live])
     assert eh <= F16_TOL and ec <= F16_TOL, (eh, ec)
-    # most values agree to the bit: the two only part where a value sat within rounding of a tie
+    # most values agree to the bit: the two only part where a value sat within rounding of a tie (more often
+    # the longer the fp32 sums, and every difference is carried on through time and layers)
     same = np.mean(got_h == hr.astype(np.float32)[:, live])
-    assert same > 0.9, same
+    assert same > (0.9 if H <= 512 else 0.8), same
 
 
 def test_stacked_lstm_f16_rejects_other_hidden_sizes(core):
+    xs = torch.zeros((2, 32, 80), dtype=torch.float16, device='cuda')
+    WU = torch.zeros((1, 160, 320), dtype=torch.float16, device='cuda')
+    with pytest.raises(core.FtkError) as e:
+        core.stacked_lstm_f16(xs, WU)
+    assert e.value.code == -2 and 'multiple of 32' in str(e.value)
     xs = torch.zeros((2, 32, 128), dtype=torch.float16, device='cuda')
     WU = torch.zeros((1, 256, 512), dtype=torch.float16, device='cuda')
     with pytest.raises(core.FtkError) as e:
-        core.stacked_lstm_f16(xs, WU)
-    assert e.value.code == -2 and 'H = 512' in str(e.value)
+        core.stacked_lstm_f16(xs, WU, workspace=torch.empty(16, dtype=torch.uint8, device='cuda'))
+    assert e.value.code == -3 and 'workspace' in str(e.value)
     xs = torch.zeros((2, 33, 256), dtype=torch.float16, device='cuda')
     WU = torch.zeros((1, 512, 1024), dtype=torch.float16, device='cuda')
-    with pytest.raises(core.FtkError) as e:
-        core.stacked_lstm_f16(xs, WU)                    # odd batch at H = 256
-    assert e.value.code == -2 and 'even' in str(e.value)
     with pytest.raises(TypeError):
         core.stacked_lstm_f16(xs.float(), WU)
+
+
+@pytest.mark.parametrize('B,I,H,state,bias', [
+    (256, 1024, 1024, True, True),
+    (64, 64, 64, True, False),
+    (300, 128, 256, True, True),        # input size differs from the hidden size; second row block ragged
+    (1, 64, 128, False, True),          # zero state: only the x rows of WU are read
+    (513, 192, 64, True, False),
+    (40, 96, 32, True, True),           # one unit block, odd count of k chunks
+])
+def test_lstm_cell_f16(core, B, I, H, state, bias):
+    rng = np.random.default_rng(17)
+    x = rng.standard_normal((B, I)).astype(np.float16)
+    hp = rng.uniform(-1, 1, (B, H)).astype(np.float16) if state else None
+    cp = rng.standard_normal((B, H)).astype(np.float16) if state else None
+    WU = (rng.uniform(-1, 1, (I + H, 4 * H)) / np.sqrt(I + H) * 2).astype(np.float16)
+    b = rng.uniform(-0.2, 0.2, 4 * H).astype(np.float32) if bias else None
+    h, c = core.lstm_cell_f16(dev(x), None if hp is None else dev(hp), None if cp is None else dev(cp), dev(WU),
+                              None if b is None else dev(b))
+    torch.cuda.synchronize()
+    zero = np.zeros((B, H))
+    hr, cr = ko.lstm_cell(x.astype(np.float64), zero if hp is None else hp.astype(np.float64),
+                          zero if cp is None else cp.astype(np.float64), WU.astype(np.float64), b)
+    hr16 = hr.astype(np.float16).astype(np.float32); cr16 = cr.astype(np.float16).astype(np.float32)
+    gh = h.float().cpu().numpy(); gc = c.float().cpu().numpy()
+    eh = ko.max_rel_err(gh, hr16); ec = ko.max_rel_err(gc, cr16)
+    assert eh <= F16_TOL and ec <= F16_TOL, (eh, ec)
+    # fp32 sums of exact fp16 products, rounded once: all but values within rounding of a tie agree to the bit
+    assert np.mean(gh == hr16) > 0.98 and np.mean(gc == cr16) > 0.98
+
+
+def test_lstm_cell_f16_rejects_bad_arguments(core):
+    x = torch.zeros((4, 48), dtype=torch.float16, device='cuda')
+    WU = torch.zeros((112, 256), dtype=torch.float16, device='cuda')
+    with pytest.raises(core.FtkError) as e:
+        core.lstm_cell_f16(x, None, None, WU)
+    assert e.value.code == -2 and 'multiples of 32' in str(e.value)
+    rc = core.lib.ftk_lstm_cell_f16(None, None, None, None, None, None, None, 4, 64, 64, None)
+    assert rc == -1 and b'non-NULL' in core.lib.ftk_last_error()
 
 
 def test_lstm_products_switch(core):
