@@ -233,10 +233,11 @@ struct CellListH {
 constexpr int HK = 32;                       // k chunk
 constexpr int HROWS = 256;                   // batch rows per workgroup
 constexpr int H_ACT_BYTES = HROWS * HK * 2;  // activation rows of a chunk: 64 bytes each
-constexpr int H_W_BYTES = HK * 128 * 2;      // weight rows of a chunk: 128 gate columns, 256 bytes each
-constexpr int H_STAGE = H_ACT_BYTES + H_W_BYTES;
+// per unit-block width UB (32 or 64 hidden units = 128 or 256 gate columns): bytes of a weight row, of a stage
+constexpr int cell_row_bytes(int ub) { return ub * 4 * 2; }
+constexpr int cell_stage_bytes(int ub) { return H_ACT_BYTES + HK * cell_row_bytes(ub); }
 constexpr int H_STAGES = 3;
-constexpr size_t kCellF16Lds = (size_t)H_STAGE * H_STAGES;  // 72 KB: two workgroups per compute unit
+constexpr size_t cell_lds_bytes(int ub) { return (size_t)cell_stage_bytes(ub) * H_STAGES; }  // 72 KB / 96 KB
 
 typedef short v4s __attribute__((ext_vector_type(4)));
 typedef short v8s __attribute__((ext_vector_type(8)));
@@ -257,14 +258,24 @@ __device__ __forceinline__ void cell_dma16(const void* gbase, unsigned byte_off,
 //     in slot c ^ ((k & 3) << 2); the transposing read ds_read_b64_tr_b16 takes 64 bytes from each of four
 //     consecutive rows per pass, which land in four different 64-byte groups.
 // A copy instruction fills 1 KB of consecutive slots, each lane choosing the global chunk its slot holds.
-// Three stages: while chunk ch is used, chunks ch + 1 and ch + 2 are on their way; a second workgroup on the
-// compute unit fills the gaps the barriers and LDS latencies of the first leave.
+// Three stages: while chunk ch is used, chunks ch + 1 and ch + 2 are on their way.
+//
+// WAVES = 4: a workgroup owns 32 hidden units (two waves side by side, two on top of each other), two
+// workgroups share a compute unit.  WAVES = 8: 64 hidden units (four waves side by side; weight rows of 512
+// bytes, 32 chunks, the same slot rule), one workgroup per compute unit: every activation row then enters
+// half as many LDS tiles.  Either way a wave owns 128 rows x 2 unit groups and two waves share a SIMD, the
+// one filling the gaps that the barriers and LDS latencies of the other leave.
 //
 // PACKED: the cell's WU points at weights laid out by lstm_pack_weights_f16_kernel, per unit block the very
-// bytes of the LDS rows above, so a workgroup streams one contiguous run of 256-byte rows; otherwise at the
-// [(I+H), 4H] matrix, from which a workgroup picks four 64-byte segments per row.
-template <bool PACKED>
-__global__ __launch_bounds__(256, 2) void lstm_cell_f16_kernel(CellListH list, int B, int I, int H) {
+// bytes of the LDS rows above, so a workgroup streams one contiguous run of rows; otherwise at the
+// [(I+H), 4H] matrix, from which a workgroup picks four segments per row.
+template <bool PACKED, int WAVES>
+__global__ __launch_bounds__(WAVES * 64, 8 / WAVES) void lstm_cell_f16_kernel(CellListH list, int B, int I, int H) {
+  constexpr int UB = 8 * WAVES;             // hidden units per workgroup
+  constexpr int CW = WAVES / 2;             // waves side by side
+  constexpr int ROWB = cell_row_bytes(UB);  // bytes of a weight row in LDS
+  constexpr int H_STAGE = cell_stage_bytes(UB);
+  constexpr int ACT_COPIES = 16 / WAVES;    // activation copies per wave and chunk (1 KB = 16 rows each)
   extern __shared__ __attribute__((aligned(1024))) unsigned char cell_smem[];
   using lds_v4s = __attribute__((address_space(3))) v4s;
 
@@ -272,17 +283,17 @@ __global__ __launch_bounds__(256, 2) void lstm_cell_f16_kernel(CellListH list, i
   // placed on one XCD (cell = xcd + 8 m), neighbouring unit blocks first: the cell's activation rows are then
   // fetched into one L2 instead of eight, and the 64-byte weight segments of neighbouring unit blocks that
   // share a cache line are served by the same L2.
-  const int nub = H / 32, nrb = (B + HROWS - 1) / HROWS;
+  const int nub = H / UB, nrb = (B + HROWS - 1) / HROWS;
   const int slot = blockIdx.x >> 3;
   const int cell = (blockIdx.x & 7) + 8 * (slot / (nub * nrb));
   if (cell >= list.n) return;
   const CellDescH cd = list.cells[cell];
-  const int ub = slot % nub;          // block of 32 hidden units
+  const int ub = slot % nub;          // block of UB hidden units
   const int rb = (slot / nub) % nrb;  // block of 256 batch rows
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-  const int wr = wave >> 1;  // rows 128*wr .. +128 of the block
-  const int wc = wave & 1;   // unit groups 2*wc, 2*wc+1 of the block's four
+  const int wr = wave / CW;  // rows 128*wr .. +128 of the block
+  const int wc = wave % CW;  // unit groups 2*wc, 2*wc+1 of the block's
   const int j = lane & 31;
   const int hh = lane >> 5;
   const unsigned lds0 = (unsigned)reinterpret_cast<uintptr_t>((__attribute__((address_space(3))) void*)cell_smem);
@@ -291,12 +302,19 @@ __global__ __launch_bounds__(256, 2) void lstm_cell_f16_kernel(CellListH list, i
   const int nch = nch_x + (cd.h_prev ? H / HK : 0);
   const bool full = rb * HROWS + HROWS <= B;
 
-  // ---- copies: per chunk a wave issues 4 activation copies (rows 64*wave + 16 i + lane/4) and 2 weight
-  // copies (k rows 8*wave + 4 i + lane/16)
+  // ---- copies: per chunk a wave issues ACT_COPIES activation copies (16 rows each, row lane/4) and 2 weight
+  // copies (1 KB = 4 or 2 weight rows each)
   const unsigned a_lane_chunk = (unsigned)(((lane & 3) ^ ((lane >> 4) & 3)) * 16);
-  const unsigned wl = (unsigned)lane >> 4;
-  const unsigned wchunk = ((unsigned)lane & 15) ^ (wl << 2);  // 4*ug + q
-  const unsigned w_lane_off = wl * (unsigned)(8 * H) + ((wchunk & 3) * (unsigned)H + (wchunk >> 2) * 8) * 2;
+  constexpr int LPR = ROWB / 16;  // lanes per weight row
+  // weight copy g = 2*wave + i covers k rows g*(64/LPR) + lane/LPR; the lane's slot lane%LPR holds chunk
+  // slot ^ ((k & 3) << 2), chunk 4*ug + q = gate q of units 8*ug .. +8 of the block
+  unsigned w_lane_off[2];
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+    const unsigned krow = (unsigned)((2 * wave + i) * (64 / LPR) + lane / LPR);
+    const unsigned chunk = ((unsigned)lane % LPR) ^ ((krow & 3) << 2);
+    w_lane_off[i] = ((unsigned)(lane / LPR) * (unsigned)(4 * H) + (chunk & 3) * (unsigned)H + (chunk >> 2) * 8) * 2;
+  }
 
   auto issue = [&](int ch, int stage) __attribute__((always_inline)) {
     const _Float16* src;
@@ -306,29 +324,33 @@ __global__ __launch_bounds__(256, 2) void lstm_cell_f16_kernel(CellListH list, i
     } else {
       src = cd.h_prev; ld = H; k0 = (ch - nch_x) * HK;
     }
-    const unsigned act_lds = lds0 + (unsigned)(stage * H_STAGE + wave * 4096);
+    const int row0 = wave * 16 * ACT_COPIES;  // first of the wave's rows within the block
+    const unsigned act_lds = lds0 + (unsigned)(stage * H_STAGE + row0 * 64);
     if (full) {
-      const char* base = reinterpret_cast<const char*>(src + (size_t)(rb * HROWS + wave * 64) * ld + k0);
+      const char* base = reinterpret_cast<const char*>(src + (size_t)(rb * HROWS + row0) * ld + k0);
       const unsigned off = ((unsigned)lane >> 2) * (unsigned)(2 * ld) + a_lane_chunk;
 #pragma unroll
-      for (int i = 0; i < 4; ++i) cell_dma16(base + (size_t)i * 32 * ld, off, act_lds + 1024u * i);
+      for (int i = 0; i < ACT_COPIES; ++i) cell_dma16(base + (size_t)i * 32 * ld, off, act_lds + 1024u * i);
     } else {  // rows past the end of the batch repeat the last row; they are never stored
       const char* base = reinterpret_cast<const char*>(src + k0);
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        const int row = min(rb * HROWS + wave * 64 + 16 * i + (lane >> 2), B - 1);
+      for (int i = 0; i < ACT_COPIES; ++i) {
+        const int row = min(rb * HROWS + row0 + 16 * i + (lane >> 2), B - 1);
         cell_dma16(base, (unsigned)row * (unsigned)(2 * ld) + a_lane_chunk, act_lds + 1024u * i);
       }
     }
     const unsigned w_lds = lds0 + (unsigned)(stage * H_STAGE + H_ACT_BYTES + wave * 2048);
     if constexpr (PACKED) {
-      const char* wbase = reinterpret_cast<const char*>(cd.WU + ((size_t)ub * (I + H) + ch * HK + wave * 8) * 128);
+      const char* wbase = reinterpret_cast<const char*>(cd.WU) + ((size_t)ub * (I + H) + ch * HK) * ROWB + wave * 2048;
 #pragma unroll
       for (int i = 0; i < 2; ++i) cell_dma16(wbase + 1024 * i, 16u * lane, w_lds + 1024u * i);
     } else {
-      const char* wbase = reinterpret_cast<const char*>(cd.WU + (size_t)(ch * HK + wave * 8) * 4 * H + ub * 32);
 #pragma unroll
-      for (int i = 0; i < 2; ++i) cell_dma16(wbase + (size_t)i * 32 * H, w_lane_off, w_lds + 1024u * i);
+      for (int i = 0; i < 2; ++i) {
+        const char* wbase = reinterpret_cast<const char*>(
+            cd.WU + (size_t)(ch * HK + (2 * wave + i) * (64 / LPR)) * 4 * H + ub * UB);
+        cell_dma16(wbase, w_lane_off[i], w_lds + 1024u * i);
+      }
     }
   };
 
@@ -340,7 +362,7 @@ __global__ __launch_bounds__(256, 2) void lstm_cell_f16_kernel(CellListH list, i
     const int ta = (lane & 15) >> 2, tb = lane & 3, th = (lane >> 4) & 1;
 #pragma unroll
     for (int u2 = 0; u2 < 2; ++u2)
-      w_off[u2] = (unsigned)(H_ACT_BYTES + (8 * hh + ta) * 256 +
+      w_off[u2] = (unsigned)(H_ACT_BYTES + (8 * hh + ta) * ROWB +
                              (((4 * (2 * wc + u2) + 2 * th + (tb >> 1)) ^ (ta << 2)) * 16) + 8 * (tb & 1));
   }
 
@@ -356,9 +378,9 @@ __global__ __launch_bounds__(256, 2) void lstm_cell_f16_kernel(CellListH list, i
   if (nch > 1) issue(1, 1);
   int stage = 0;
   for (int ch = 0; ch < nch; ++ch) {
-    // 6 copies per wave and chunk, completing in order: all but the newest chunk's have landed
+    // ACT_COPIES + 2 copies per wave and chunk, completing in order: all but the newest chunk's have landed
     if (ch + 1 < nch)
-      __builtin_amdgcn_s_waitcnt(0x0F76);  // vmcnt(6)
+      __builtin_amdgcn_s_waitcnt(0x0F70 | (ACT_COPIES + 2));  // vmcnt(ACT_COPIES + 2)
     else
       __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
     __syncthreads();  // chunk ch is complete, and every wave is done with the stage of chunk ch-1
@@ -369,9 +391,9 @@ __global__ __launch_bounds__(256, 2) void lstm_cell_f16_kernel(CellListH list, i
       v8h wf[2];
 #pragma unroll
       for (int u2 = 0; u2 < 2; ++u2) {
-        const unsigned char* p0 = sb + w_off[u2] + 4096 * ks;
+        const unsigned char* p0 = sb + w_off[u2] + 16 * ROWB * ks;
         const v4s lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4s*)(p0));
-        const v4s hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4s*)(p0 + 1024));
+        const v4s hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4s*)(p0 + 4 * ROWB));
         const v8s both = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
         wf[u2] = __builtin_bit_cast(v8h, both);
       }
@@ -393,7 +415,7 @@ __global__ __launch_bounds__(256, 2) void lstm_cell_f16_kernel(CellListH list, i
     if (row_g >= B) continue;
 #pragma unroll
     for (int u2 = 0; u2 < 2; ++u2) {
-      const int u0 = ub * 32 + 8 * (2 * wc + u2) + 4 * hh;
+      const int u0 = ub * UB + 8 * (2 * wc + u2) + 4 * hh;
       v4h cp = {0, 0, 0, 0};
       if (cd.c_prev) cp = *reinterpret_cast<const v4h*>(cd.c_prev + (size_t)row_g * H + u0);
       v4f bi = {0, 0, 0, 0}, bf = bi, bo = bi, bg = bi;
@@ -426,12 +448,12 @@ static int launch_cells(const CellList& list, int B, int I, int H, hipStream_t s
   return check_launch("lstm_cell_kernel");
 }
 
-// WU [n_layers, K2, 4H] -> per layer and unit block ub the [K2][128] tile the cell kernel keeps in LDS: row k
-// holds 16 chunks of 8 columns, chunk 4*ug + q = gate q of units 32*ub + 8*ug .. +8, stored in slot
+// WU [n_layers, K2, 4H] -> per layer and block ub of UB hidden units the [K2][4*UB] tile the cell kernel keeps
+// in LDS: row k holds chunks of 8 columns, chunk 4*ug + q = gate q of units UB*ub + 8*ug .. +8, stored in slot
 // chunk ^ ((k & 3) << 2).  One thread per 16-byte chunk.
 __global__ __launch_bounds__(256) void lstm_pack_weights_f16_kernel(const _Float16* __restrict__ WU,
                                                                     _Float16* __restrict__ packed, size_t chunks,
-                                                                    int K2, int H) {
+                                                                    int K2, int H, int UB) {
   const size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;
   if (idx >= chunks) return;
   const int per_row = H / 2;  // 4H / 8
@@ -441,35 +463,41 @@ __global__ __launch_bounds__(256) void lstm_pack_weights_f16_kernel(const _Float
   const size_t l = lk / K2;
   const int col = 8 * n8;
   const int q = col / H, u = col % H;
-  const int ub = u >> 5, ug = (u & 31) >> 3;
+  const int ub = u / UB, ug = (u % UB) >> 3;
   const int slot = (4 * ug + q) ^ ((k & 3) << 2);
   const v4u v = *reinterpret_cast<const v4u*>(WU + idx * 8);
-  *reinterpret_cast<v4u*>(packed + ((l * (H / 32) + ub) * K2 + k) * 128 + 8 * slot) = v;
+  *reinterpret_cast<v4u*>(packed + ((l * (H / UB) + ub) * K2 + k) * (4 * UB) + 8 * slot) = v;
 }
+
+// Hidden units per workgroup of the streaming kernel at hidden size H.
+static int cell_unit_block(int H) { return H % 64 == 0 ? 64 : 32; }
 
 int pack_weights_f16(const void* WU, void* packed, int layers, int K2, int H, hipStream_t s) {
   const size_t chunks = (size_t)layers * K2 * (H / 2);
   hipLaunchKernelGGL(lstm_pack_weights_f16_kernel, dim3((unsigned)((chunks + 255) / 256)), dim3(256), 0, s,
-                     (const _Float16*)WU, (_Float16*)packed, chunks, K2, H);
+                     (const _Float16*)WU, (_Float16*)packed, chunks, K2, H, cell_unit_block(H));
   return check_launch("lstm_pack_weights_f16_kernel");
 }
 
-template <bool PACKED>
+template <bool PACKED, int WAVES>
 static int launch_cells_f16(const CellListH& list, int B, int I, int H, hipStream_t s) {
   static bool attr_set = false;  // per process; the attribute belongs to the function, on every device
-  const void* fn = (const void*)lstm_cell_f16_kernel<PACKED>;
+  constexpr int UB = 8 * WAVES;
+  const void* fn = (const void*)lstm_cell_f16_kernel<PACKED, WAVES>;
   if (!attr_set) {
-    FTK_HIP(hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)kCellF16Lds));
+    FTK_HIP(hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)cell_lds_bytes(UB)));
     attr_set = true;
   }
   const int groups = (list.n + 7) / 8;  // cells per XCD
-  dim3 grid(8 * groups * (H / 32) * ((B + HROWS - 1) / HROWS));
-  hipLaunchKernelGGL(lstm_cell_f16_kernel<PACKED>, grid, dim3(256), kCellF16Lds, s, list, B, I, H);
+  dim3 grid(8 * groups * (H / UB) * ((B + HROWS - 1) / HROWS));
+  hipLaunchKernelGGL((lstm_cell_f16_kernel<PACKED, WAVES>), grid, dim3(WAVES * 64), cell_lds_bytes(UB), s, list, B, I, H);
   return check_launch("lstm_cell_f16_kernel");
 }
 
 static int launch_cells(const CellListH& list, int B, int I, int H, hipStream_t s) {
-  return list.packed ? launch_cells_f16<true>(list, B, I, H, s) : launch_cells_f16<false>(list, B, I, H, s);
+  if (cell_unit_block(H) == 64)
+    return list.packed ? launch_cells_f16<true, 8>(list, B, I, H, s) : launch_cells_f16<false, 8>(list, B, I, H, s);
+  return list.packed ? launch_cells_f16<true, 4>(list, B, I, H, s) : launch_cells_f16<false, 4>(list, B, I, H, s);
 }
 
 // Host side of the per-stage schedule: stage(l,t) = 1 + max(stage(l-1,t),
