@@ -323,18 +323,20 @@ def bench_lstm(torch, core, steps, warmup, cpu, dilated, baselines=True):
 
 
 def bench_lstm_f16(torch, core, steps, warmup, cpu, H, baselines=True):
-    """fp16-storage stack at the first two hidden sizes of the reference's sweep (cute_stacked_lstm/stacked_lstm.cu:185-186)."""
+    """fp16-storage stack at the three hidden sizes of the reference's sweep (cute_stacked_lstm/stacked_lstm.cu:185-187):
+    256 and 512 in the persistent kernel, 1024 through the streaming cell kernel, one launch per stage of cells."""
     L, T, B = 32, 64, 256
     flop = 2.0 * L * T * B * (2 * H) * (4 * H)
     gen = torch.Generator(device='cpu').manual_seed(1234)
     xs = torch.randn((T, B, H), generator=gen).half().cuda()
-    WU = ((torch.rand((L, 2 * H, 4 * H), generator=gen) - 0.5) / (8 if H == 256 else 12)).half().cuda()
+    WU = ((torch.rand((L, 2 * H, 4 * H), generator=gen) - 0.5) / {256: 8, 512: 12}.get(H, 16)).half().cuda()
     hs = torch.empty((L, T, B, H), dtype=torch.float16, device='cuda')
     cs = torch.empty_like(hs)
     ws = torch.empty(int(core.lib.ftk_stacked_lstm_f16_workspace_bytes(L, T, B, H)), dtype=torch.uint8, device='cuda')
     fused = lambda: core.stacked_lstm_f16(xs, WU, out=(hs, cs), workspace=ws)
     ms, wall = _events_ms(torch, fused, steps, warmup)
-    status = core.persistent_status(ws)
+    on_chip = H in (256, 512)
+    status = core.persistent_status(ws) if on_chip else None
     res = {
         'metric': 'stacked-LSTM sequences/s', 'value': B / ms * 1e3, 'unit': 'sequences/s', 'ms_per_step': ms, 'dtype': 'f16',
         'config': {'workload': f'stacked LSTM, fp16 storage, the H = {H} row of the reference sweep', 'layers': L, 'batch': B,
@@ -344,6 +346,16 @@ def bench_lstm_f16(torch, core, steps, warmup, cpu, H, baselines=True):
                      'frac': flop / ms / 1e9 / PEAK_F16_TFLOPS, 'traffic': None,
                      'kernel': 'lstm_persistent_kernel<2>' if H == 512 else 'lstm_persistent_kernel<3>'},
     }
+    if not on_chip:
+        # every cell streams its layer's weights once (the stack's weights exceed the 256 MB of last-level cache), reads its
+        # two input rows sets and c, writes h and c: the bytes that bound this schedule from below
+        wbytes = L * T * (2 * H * 4 * H * 2.0)
+        abytes = L * T * (5 * B * H * 2.0)
+        res['roofline'] = {'bound': 'hbm', 'achieved': (wbytes + abytes) / ms / 1e6, 'peak': PEAK_HBM_GBS, 'unit': 'GB/s',
+                           'frac': (wbytes + abytes) / ms / 1e6 / PEAK_HBM_GBS, 'traffic': None,
+                           'kernel': 'lstm_cell_f16_kernel<true, 8>',
+                           'note': 'per launch: the cells of one stage; bytes = weights of every cell once + activations'}
+        res['config']['schedule'] = 'one launch of the streaming fp16 cell kernel per stage of independent cells'
     if baselines:
         ref_h = hs.clone()
         W = WU[:, :H].contiguous()
@@ -385,7 +397,7 @@ def main():
     ap.add_argument('--gpus', type=int, default=1)
     ap.add_argument('--steps', type=int, default=50)
     ap.add_argument('--warmup', type=int, default=10)
-    ap.add_argument('--workload', default='b2b', choices=['b2b', 'attention', 'stacked_lstm', 'dilated_lstm', 'lstm_f16_h256', 'lstm_f16_h512', 'embedding', 'copy'])
+    ap.add_argument('--workload', default='b2b', choices=['b2b', 'attention', 'stacked_lstm', 'dilated_lstm', 'lstm_f16_h256', 'lstm_f16_h512', 'lstm_f16_h1024', 'embedding', 'copy'])
     ap.add_argument('--no-extras', action='store_true', help='measure only the chosen workload')
     ap.add_argument('--no-cpu', action='store_true', help='skip the CPU baseline leg')
     ap.add_argument('--no-baselines', action='store_true',
@@ -411,6 +423,7 @@ def main():
         'dilated_lstm': lambda s, w, c: bench_lstm(torch, core, max(3, s // 5), max(1, w // 5), c, True, not args.no_baselines),
         'lstm_f16_h256': lambda s, w, c: bench_lstm_f16(torch, core, max(3, s // 5), max(1, w // 5), c, 256, not args.no_baselines),
         'lstm_f16_h512': lambda s, w, c: bench_lstm_f16(torch, core, max(3, s // 5), max(1, w // 5), c, 512, not args.no_baselines),
+        'lstm_f16_h1024': lambda s, w, c: bench_lstm_f16(torch, core, max(3, s // 5), max(1, w // 5), c, 1024, not args.no_baselines),
         'embedding': lambda s, w, c: bench_embedding(torch, core, s, w, c),
     }
     if args.workload == 'copy':
