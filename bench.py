@@ -343,7 +343,8 @@ def bench_lstm_f16(torch, core, steps, warmup, cpu, H, baselines=True):
                    'seq_len': T, 'hidden': H, 'outputs': 'h and c of every layer at every step (fp16)', 'accumulate': 'f32'},
         'tflops': flop / ms / 1e9, 'persistent_status': status,
         'roofline': {'bound': 'mfma', 'achieved': flop / ms / 1e9, 'peak': PEAK_F16_TFLOPS, 'unit': 'TFLOP/s',
-                     'frac': flop / ms / 1e9 / PEAK_F16_TFLOPS, 'traffic': None,
+                     'frac': flop / ms / 1e9 / PEAK_F16_TFLOPS,
+                     'traffic': MEASURED_TRAFFIC_BYTES.get('lstm_persistent_kernel<2>' if H == 512 else 'lstm_persistent_kernel<3>'),
                      'kernel': 'lstm_persistent_kernel<2>' if H == 512 else 'lstm_persistent_kernel<3>'},
     }
     if not on_chip:
@@ -352,7 +353,8 @@ def bench_lstm_f16(torch, core, steps, warmup, cpu, H, baselines=True):
         wbytes = L * T * (2 * H * 4 * H * 2.0)
         abytes = L * T * (5 * B * H * 2.0)
         res['roofline'] = {'bound': 'hbm', 'achieved': (wbytes + abytes) / ms / 1e6, 'peak': PEAK_HBM_GBS, 'unit': 'GB/s',
-                           'frac': (wbytes + abytes) / ms / 1e6 / PEAK_HBM_GBS, 'traffic': None,
+                           'frac': (wbytes + abytes) / ms / 1e6 / PEAK_HBM_GBS,
+                           'traffic': MEASURED_TRAFFIC_BYTES.get('lstm_cell_f16_kernel_per_pass'),
                            'kernel': 'lstm_cell_f16_kernel<true, 8>',
                            'note': 'per launch: the cells of one stage; bytes = weights of every cell once + activations'}
         res['config']['schedule'] = 'one launch of the streaming fp16 cell kernel per stage of independent cells'
