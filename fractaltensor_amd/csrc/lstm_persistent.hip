@@ -1026,6 +1026,25 @@ static int run_stack(const char* who, const float* xs, const float* WU, const fl
 
 }  // namespace ftk
 
+namespace ftk {
+
+// The persistent kernel holds the fp16 weights of H = 512, and of H = 256 with two batch rows per tile row (even B).
+static bool f16_fits_on_chip(int B, int H) { return H == 2 * PH || (H == PH && !(B & 1)); }
+
+// Whether the fp16 stack goes through the streaming cell kernel, one launch per stage of cells.  Always where the
+// weights do not fit on chip; at H = 512 also when the stack is deeper than the 16 layers that 256 compute units
+// hold at once: the persistent kernel then runs twice and fills its wavefront twice (5.5 ms at L = 32, T = 64,
+// B = 256), while the streamed cells find the 134 MB of weights in the last-level cache (3.75 ms).  A ragged
+// batch stays with the persistent kernel, which skips the row blocks that have ended.
+// FTK_LSTM_F16_STREAM=1 / =0 in the environment forces the one or the other where both can run.
+static bool f16_streams(int L, int B, int H, bool ragged) {
+  if (!f16_fits_on_chip(B, H)) return true;
+  if (const char* e = getenv("FTK_LSTM_F16_STREAM")) return e[0] == '1';
+  return H == 2 * PH && L > 16 && !ragged;
+}
+
+}  // namespace ftk
+
 extern "C" {
 
 size_t ftk_stacked_lstm_workspace_bytes(int L, int T, int B, int H) {
@@ -1035,9 +1054,10 @@ size_t ftk_stacked_lstm_workspace_bytes(int L, int T, int B, int H) {
 
 size_t ftk_stacked_lstm_f16_workspace_bytes(int L, int T, int B, int H) {
   if (L <= 0 || T <= 0 || B <= 0 || H <= 0) return 0;
-  const bool on_chip = H == 2 * ftk::PH || (H == ftk::PH && !(B & 1));
-  if (!on_chip) return (size_t)L * 2 * H * 4 * H * sizeof(_Float16);  // the re-laid weights of the streaming kernel
-  return ftk::xratio_offset_bytes(L, T, B);
+  const size_t packed = (size_t)L * 2 * H * 4 * H * sizeof(_Float16);  // the re-laid weights of the streaming kernel
+  if (!ftk::f16_fits_on_chip(B, H)) return packed;
+  // which of the two runs is decided per call (a ragged batch stays with the persistent kernel): room for either
+  return std::max(ftk::xratio_offset_bytes(L, T, B), ftk::f16_streams(L, B, H, false) ? packed : (size_t)0);
 }
 
 int ftk_stacked_lstm_f16(const void* xs, const void* WU, const float* bias, const int* dilations,
@@ -1050,7 +1070,7 @@ int ftk_stacked_lstm_f16(const void* xs, const void* WU, const float* bias, cons
   if (H % 32) return fail(FTK_ERR_UNSUPPORTED_SHAPE, "%s: H=%d must be a multiple of 32", who, H);
   if ((long long)B * H >= (1ll << 30)) return fail(FTK_ERR_UNSUPPORTED_SHAPE, "%s: B*H = %lld is too large", who, (long long)B * H);
   // the persistent kernel holds the weights of H = 512, and of H = 256 with two batch rows per tile row (even B)
-  const bool on_chip = H == 2 * PH || (H == PH && !(B & 1));
+  const bool on_chip = !f16_streams(L, B, H, active_rows != nullptr);
   const int mode = H == PH ? kHalfData256 : kHalfData;
   const int npc = H / 32;
   if (dilations)

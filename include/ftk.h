@@ -163,7 +163,9 @@ int ftk_stacked_lstm_ragged_f32(const float* xs, const float* WU,
  * H = 512, 32 of H = 256 on 256 compute units) run as consecutive launches.
  * Every other shape (H = 1024, the third size of the sweep, among them) does
  * not fit on chip: its weights are streamed, one launch of the fp16 cell
- * kernel per stage of independent cells, which computes dead rows too; the
+ * kernel per stage of independent cells, which computes dead rows too (and
+ * which is also the faster way for H = 512 stacks of more than 16 layers,
+ * unless active_rows is given; FTK_LSTM_F16_STREAM=1 / 0 forces either); the
  * workspace then takes a re-laid copy of WU (ftk_stacked_lstm_f16_workspace_bytes
  * says how much for a shape).
  * dilations, active_rows: host arrays or NULL, as above.

@@ -226,7 +226,8 @@ def test_stacked_lstm_ragged_rejects_unsorted_rows(core):
     (512, 2, 5, 40, None, True, False),             # ragged last row block
     (512, 3, 8, 96, [1, 2, 4], True, False),
     (512, 2, 9, 64, None, True, True),              # half the rows stop after 4 steps
-    (512, 18, 3, 32, None, False, False),           # deeper than the chip holds at once: two launches
+    (512, 18, 3, 32, None, False, False),           # deeper than the chip holds at once: streamed like H = 1024
+    (512, 18, 6, 64, None, True, True),             # ... and ragged: stays persistent, two launches
     (256, 1, 6, 64, None, False, False),            # H = 256: two batch rows share a tile row
     (256, 2, 5, 38, None, True, False),             # last row block holds three pairs
     (256, 3, 8, 96, [1, 2, 4], True, False),
