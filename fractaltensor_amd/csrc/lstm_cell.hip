@@ -21,7 +21,7 @@
 // weights no longer fit on chip: the same transposed product on
 // v_mfma_f32_32x32x16_f16, a workgroup of 4 waves owning 256 batch rows x 32
 // hidden units so that every weight is fetched once per cell, and k chunks of
-// 32 copied from global memory straight into a three-deep ring of LDS stages
+// 32 copied from global memory straight into a ring of three to five LDS stages
 // (global_load_lds_dwordx4), two workgroups per compute unit.
 #include <algorithm>
 #include <vector>
@@ -236,8 +236,16 @@ constexpr int H_ACT_BYTES = HROWS * HK * 2;  // activation rows of a chunk: 64 b
 // per unit-block width UB (32 or 64 hidden units = 128 or 256 gate columns): bytes of a weight row, of a stage
 constexpr int cell_row_bytes(int ub) { return ub * 4 * 2; }
 constexpr int cell_stage_bytes(int ub) { return H_ACT_BYTES + HK * cell_row_bytes(ub); }
-constexpr int H_STAGES = 3;
-constexpr size_t cell_lds_bytes(int ub) { return (size_t)cell_stage_bytes(ub) * H_STAGES; }  // 72 KB / 96 KB
+// s_waitcnt immediate that waits for vmcnt <= n only (n < 64: bits 3:0 and 15:14; expcnt and lgkmcnt left open)
+constexpr int vmcnt_only(int n) { return 0x0F70 | (n & 15) | ((n >> 4) << 14); }
+
+#ifndef CELL_STAGES8
+#define CELL_STAGES8 3
+#endif
+// LDS stages: chunk ch in use, the next stages - 1 chunks on their way.  What is in flight is what hides the
+// 1.5 - 2 us a copy takes under load: 32 KB per compute unit and chunk.
+constexpr int cell_stages(int ub) { return ub == 64 ? CELL_STAGES8 : 3; }
+constexpr size_t cell_lds_bytes(int ub) { return (size_t)cell_stage_bytes(ub) * cell_stages(ub); }  // 72 KB / 96 KB
 
 typedef short v4s __attribute__((ext_vector_type(4)));
 typedef short v8s __attribute__((ext_vector_type(8)));
@@ -258,7 +266,7 @@ __device__ __forceinline__ void cell_dma16(const void* gbase, unsigned byte_off,
 //     in slot c ^ ((k & 3) << 2); the transposing read ds_read_b64_tr_b16 takes 64 bytes from each of four
 //     consecutive rows per pass, which land in four different 64-byte groups.
 // A copy instruction fills 1 KB of consecutive slots, each lane choosing the global chunk its slot holds.
-// Three stages: while chunk ch is used, chunks ch + 1 and ch + 2 are on their way.
+// A ring of stages: while chunk ch is used, the next chunks are on their way (cell_stages).
 //
 // WAVES = 4: a workgroup owns 32 hidden units (two waves side by side, two on top of each other), two
 // workgroups share a compute unit.  WAVES = 8: 64 hidden units (four waves side by side; weight rows of 512
@@ -374,38 +382,52 @@ __global__ __launch_bounds__(WAVES * 64, 8 / WAVES) void lstm_cell_f16_kernel(Ce
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[rt][u2][r] = 0.0f;
 
-  issue(0, 0);
-  if (nch > 1) issue(1, 1);
+  constexpr int S = cell_stages(UB);
+  constexpr int CPC = ACT_COPIES + 2;  // copies per wave and chunk
+#pragma unroll
+  for (int c = 0; c < S - 1; ++c)
+    if (c < nch) issue(c, c);
   int stage = 0;
   for (int ch = 0; ch < nch; ++ch) {
-    // ACT_COPIES + 2 copies per wave and chunk, completing in order: all but the newest chunk's have landed
-    if (ch + 1 < nch)
-      __builtin_amdgcn_s_waitcnt(0x0F70 | (ACT_COPIES + 2));  // vmcnt(ACT_COPIES + 2)
-    else
-      __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
+    // copies complete in order: chunk ch has landed when no more are outstanding than were issued after it
+    static_assert(S >= 3 && S <= 6, "wait counts below");
+    switch (min(S - 2, nch - 1 - ch)) {
+      case 0: __builtin_amdgcn_s_waitcnt(vmcnt_only(0)); break;
+      case 1: __builtin_amdgcn_s_waitcnt(vmcnt_only(CPC)); break;
+      case 2: __builtin_amdgcn_s_waitcnt(vmcnt_only(2 * CPC)); break;
+      case 3: __builtin_amdgcn_s_waitcnt(vmcnt_only(3 * CPC)); break;
+      default: __builtin_amdgcn_s_waitcnt(vmcnt_only(4 * CPC)); break;
+    }
     __syncthreads();  // chunk ch is complete, and every wave is done with the stage of chunk ch-1
-    if (ch + 2 < nch) issue(ch + 2, stage == 0 ? 2 : stage - 1);
     const unsigned char* sb = cell_smem + stage * H_STAGE;
-#pragma unroll
-    for (int ks = 0; ks < 2; ++ks) {
-      v8h wf[2];
+    // all fragments of the chunk are requested up front, the copies of chunk ch + 2 issued while they travel
+    v8h wf[2][2], af[2][4];
+    auto read_frags = [&](int ks) __attribute__((always_inline)) {
 #pragma unroll
       for (int u2 = 0; u2 < 2; ++u2) {
         const unsigned char* p0 = sb + w_off[u2] + 16 * ROWB * ks;
         const v4s lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4s*)(p0));
         const v4s hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4s*)(p0 + 4 * ROWB));
         const v8s both = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
-        wf[u2] = __builtin_bit_cast(v8h, both);
+        wf[ks][u2] = __builtin_bit_cast(v8h, both);
       }
 #pragma unroll
-      for (int rt = 0; rt < 4; ++rt) {
-        const v8h af = *reinterpret_cast<const v8h*>(sb + a_off[ks] + 2048 * rt);
+      for (int rt = 0; rt < 4; ++rt) af[ks][rt] = *reinterpret_cast<const v8h*>(sb + a_off[ks] + 2048 * rt);
+    };
+    read_frags(0);
+    __builtin_amdgcn_sched_barrier(0);
+    if (ch + S - 1 < nch) issue(ch + S - 1, stage == 0 ? S - 1 : stage - 1);
+    __builtin_amdgcn_sched_barrier(0);
+    read_frags(1);
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int ks = 0; ks < 2; ++ks)
+#pragma unroll
+      for (int rt = 0; rt < 4; ++rt)
 #pragma unroll
         for (int u2 = 0; u2 < 2; ++u2)
-          acc[rt][u2] = __builtin_amdgcn_mfma_f32_32x32x16_f16(wf[u2], af, acc[rt][u2], 0, 0, 0);
-      }
-    }
-    stage = stage == 2 ? 0 : stage + 1;
+          acc[rt][u2] = __builtin_amdgcn_mfma_f32_32x32x16_f16(wf[ks][u2], af[ks][rt], acc[rt][u2], 0, 0, 0);
+    stage = stage == S - 1 ? 0 : stage + 1;
   }
 
   // Epilogue: lane (row j, half hh) holds the four gates of units 4*hh .. 4*hh+3 of each of its unit groups.
