@@ -215,18 +215,22 @@ __global__ __launch_bounds__(256) void lstm_elementwise_kernel(const float* __re
 
 // ---------------------------------------------------------------- fp16 cell
 struct CellDescH {
-  const _Float16* x;       // [B, I]
-  const _Float16* h_prev;  // [B, H] or nullptr (zero state)
-  const _Float16* c_prev;  // [B, H] or nullptr
-  const _Float16* WU;      // [(I+H), 4H]
+  const _Float16* x;       // [B, I]; split flavour: [B, 2I], a row = its two planes [value | remainder]
+  const _Float16* h_prev;  // [B, H] or nullptr (zero state); split flavour: [B, 2H] planes
+  const void* c_prev;      // [B, H] or nullptr; fp16, split flavour: fp32
+  const _Float16* WU;      // [(I+H), 4H], or the packed layout
   const float* bias;       // [4H] or nullptr
-  _Float16* h;             // [B, H]
-  _Float16* c;             // [B, H]
+  void* h;                 // [B, H]; fp16, split flavour: fp32
+  void* c;                 // [B, H]
+  // split flavour only
+  const float* xratio;     // [B]: scale of the x rows relative to the h rows, or nullptr (x is an h of the layer below)
+  const float* wscale;     // [4H]: what a gate sum of column n is multiplied by to undo the operand scales
+  _Float16* h_planes;      // [B, 2H]: the two planes of h for the cells that read it
 };
 
 struct CellListH {
   int n;
-  int packed;  // WU of every cell is in the packed layout
+  int packed;  // 1: WU of every cell is in the packed layout; 2: packed split weights, the split flavour
   CellDescH cells[kMaxCellsPerLaunch];
 };
 
@@ -277,8 +281,20 @@ __device__ __forceinline__ void cell_dma16(const void* gbase, unsigned byte_off,
 // PACKED: the cell's WU points at weights laid out by lstm_pack_weights_f16_kernel, per unit block the very
 // bytes of the LDS rows above, so a workgroup streams one contiguous run of rows; otherwise at the
 // [(I+H), 4H] matrix, from which a workgroup picks four segments per row.
-template <bool PACKED, int WAVES>
+//
+// SPLIT: fp32 data on fp16 MFMAs.  Every fp32 operand v of a group that shares a power-of-two scale s (an
+// activation row, a weight column) is the sum of two fp16 numbers, top = fp16(v s) and rest = fp16(v s - top),
+// to within 2^-22 |v s|, so a product is top*top + top*rest + rest*top up to a term of 2^-22 of it.  The three
+// products go into the same fp32 accumulators as three k chunks in a row -- (top, top), (top, rest), (rest,
+// top) -- of a contraction three times as long: x and h_prev arrive as rows [top | rest], the packed weights
+// hold the rows of every chunk three times in that order (lstm_pack_split_weights_kernel).  The x rows carry
+// their own scale and the h rows 2^14, so between the last x chunk and the first h chunk the sums are
+// multiplied by the ratio; the epilogue undoes the h and column scales, computes in fp32, writes h and c in
+// fp32 and the two planes of h for the cells that read it next.
+template <bool PACKED, int WAVES, bool SPLIT>
 __global__ __launch_bounds__(WAVES * 64, 8 / WAVES) void lstm_cell_f16_kernel(CellListH list, int B, int I, int H) {
+  static_assert(!SPLIT || PACKED, "the split flavour reads packed weights");
+  constexpr int REP = SPLIT ? 3 : 1;        // k chunks per chunk of the contraction
   constexpr int UB = 8 * WAVES;             // hidden units per workgroup
   constexpr int CW = WAVES / 2;             // waves side by side
   constexpr int ROWB = cell_row_bytes(UB);  // bytes of a weight row in LDS
@@ -306,8 +322,8 @@ __global__ __launch_bounds__(WAVES * 64, 8 / WAVES) void lstm_cell_f16_kernel(Ce
   const int hh = lane >> 5;
   const unsigned lds0 = (unsigned)reinterpret_cast<uintptr_t>((__attribute__((address_space(3))) void*)cell_smem);
 
-  const int nch_x = I / HK;
-  const int nch = nch_x + (cd.h_prev ? H / HK : 0);
+  const int nch_x = REP * (I / HK);
+  const int nch = nch_x + (cd.h_prev ? REP * (H / HK) : 0);
   const bool full = rb * HROWS + HROWS <= B;
 
   // ---- copies: per chunk a wave issues ACT_COPIES activation copies (16 rows each, row lane/4) and 2 weight
@@ -327,7 +343,14 @@ __global__ __launch_bounds__(WAVES * 64, 8 / WAVES) void lstm_cell_f16_kernel(Ce
   auto issue = [&](int ch, int stage) __attribute__((always_inline)) {
     const _Float16* src;
     int ld, k0;
-    if (ch < nch_x) {
+    if constexpr (SPLIT) {
+      const bool in_x = ch < nch_x;
+      const int v = in_x ? ch : ch - nch_x;
+      const int width = in_x ? I : H;
+      src = in_x ? cd.x : cd.h_prev;
+      ld = 2 * width;
+      k0 = (v / 3) * HK + (v % 3 == 2 ? width : 0);  // third pass of a chunk: the remainder plane
+    } else if (ch < nch_x) {
       src = cd.x; ld = I; k0 = ch * HK;
     } else {
       src = cd.h_prev; ld = H; k0 = (ch - nch_x) * HK;
@@ -349,7 +372,7 @@ __global__ __launch_bounds__(WAVES * 64, 8 / WAVES) void lstm_cell_f16_kernel(Ce
     }
     const unsigned w_lds = lds0 + (unsigned)(stage * H_STAGE + H_ACT_BYTES + wave * 2048);
     if constexpr (PACKED) {
-      const char* wbase = reinterpret_cast<const char*>(cd.WU) + ((size_t)ub * (I + H) + ch * HK) * ROWB + wave * 2048;
+      const char* wbase = reinterpret_cast<const char*>(cd.WU) + ((size_t)ub * REP * (I + H) + ch * HK) * ROWB + wave * 2048;
 #pragma unroll
       for (int i = 0; i < 2; ++i) cell_dma16(wbase + 1024 * i, 16u * lane, w_lds + 1024u * i);
     } else {
@@ -381,6 +404,19 @@ __global__ __launch_bounds__(WAVES * 64, 8 / WAVES) void lstm_cell_f16_kernel(Ce
     for (int u2 = 0; u2 < 2; ++u2)
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[rt][u2][r] = 0.0f;
+
+  // split flavour: the sums of the x chunks are in the x rows' scale; this brings them to the h rows'
+  auto rescale_x = [&]() __attribute__((always_inline)) {
+    if (!cd.xratio) return;
+#pragma unroll
+    for (int rt = 0; rt < 4; ++rt) {
+      const float ratio = cd.xratio[min(rb * HROWS + 128 * wr + 32 * rt + j, B - 1)];
+#pragma unroll
+      for (int u2 = 0; u2 < 2; ++u2)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[rt][u2][r] *= ratio;
+    }
+  };
 
   constexpr int S = cell_stages(UB);
   constexpr int CPC = ACT_COPIES + 2;  // copies per wave and chunk
@@ -420,6 +456,9 @@ __global__ __launch_bounds__(WAVES * 64, 8 / WAVES) void lstm_cell_f16_kernel(Ce
     __builtin_amdgcn_sched_barrier(0);
     read_frags(1);
     __builtin_amdgcn_sched_barrier(0);
+    if constexpr (SPLIT) {
+      if (ch == nch_x) rescale_x();
+    }
 #pragma unroll
     for (int ks = 0; ks < 2; ++ks)
 #pragma unroll
@@ -428,6 +467,9 @@ __global__ __launch_bounds__(WAVES * 64, 8 / WAVES) void lstm_cell_f16_kernel(Ce
         for (int u2 = 0; u2 < 2; ++u2)
           acc[rt][u2] = __builtin_amdgcn_mfma_f32_32x32x16_f16(wf[ks][u2], af[ks][rt], acc[rt][u2], 0, 0, 0);
     stage = stage == S - 1 ? 0 : stage + 1;
+  }
+  if constexpr (SPLIT) {
+    if (nch == nch_x) rescale_x();  // zero state: there was no h chunk to do it before
   }
 
   // Epilogue: lane (row j, half hh) holds the four gates of units 4*hh .. 4*hh+3 of each of its unit groups.
@@ -438,8 +480,15 @@ __global__ __launch_bounds__(WAVES * 64, 8 / WAVES) void lstm_cell_f16_kernel(Ce
 #pragma unroll
     for (int u2 = 0; u2 < 2; ++u2) {
       const int u0 = ub * UB + 8 * (2 * wc + u2) + 4 * hh;
-      v4h cp = {0, 0, 0, 0};
-      if (cd.c_prev) cp = *reinterpret_cast<const v4h*>(cd.c_prev + (size_t)row_g * H + u0);
+      v4f cp = {0, 0, 0, 0};
+      if (cd.c_prev) {
+        if constexpr (SPLIT) {
+          cp = *reinterpret_cast<const v4f*>(reinterpret_cast<const float*>(cd.c_prev) + (size_t)row_g * H + u0);
+        } else {
+          const v4h c16 = *reinterpret_cast<const v4h*>(reinterpret_cast<const _Float16*>(cd.c_prev) + (size_t)row_g * H + u0);
+          cp = v4f{(float)c16[0], (float)c16[1], (float)c16[2], (float)c16[3]};
+        }
+      }
       v4f bi = {0, 0, 0, 0}, bf = bi, bo = bi, bg = bi;
       if (cd.bias) {
         bi = *reinterpret_cast<const v4f*>(cd.bias + u0);
@@ -447,19 +496,46 @@ __global__ __launch_bounds__(WAVES * 64, 8 / WAVES) void lstm_cell_f16_kernel(Ce
         bo = *reinterpret_cast<const v4f*>(cd.bias + 2 * H + u0);
         bg = *reinterpret_cast<const v4f*>(cd.bias + 3 * H + u0);
       }
-      v4h hv, cv;
+      v4f si = {1, 1, 1, 1}, sf = si, so = si, sg = si;
+      if constexpr (SPLIT) {
+        si = *reinterpret_cast<const v4f*>(cd.wscale + u0);
+        sf = *reinterpret_cast<const v4f*>(cd.wscale + H + u0);
+        so = *reinterpret_cast<const v4f*>(cd.wscale + 2 * H + u0);
+        sg = *reinterpret_cast<const v4f*>(cd.wscale + 3 * H + u0);
+      }
+      v4f hn, cn;
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
-        const float ig = sigmoid_f(acc[rt][u2][r] + bi[r]);
-        const float fg = sigmoid_f(acc[rt][u2][4 + r] + bf[r]);
-        const float og = sigmoid_f(acc[rt][u2][8 + r] + bo[r]);
-        const float cand = tanh_f(acc[rt][u2][12 + r] + bg[r]);
-        const float cn = fg * (float)cp[r] + ig * cand;
-        cv[r] = (_Float16)cn;
-        hv[r] = (_Float16)(og * tanh_f(cn));
+        const float ig = sigmoid_f(acc[rt][u2][r] * si[r] + bi[r]);
+        const float fg = sigmoid_f(acc[rt][u2][4 + r] * sf[r] + bf[r]);
+        const float og = sigmoid_f(acc[rt][u2][8 + r] * so[r] + bo[r]);
+        const float cand = tanh_f(acc[rt][u2][12 + r] * sg[r] + bg[r]);
+        cn[r] = fg * cp[r] + ig * cand;
+        hn[r] = og * tanh_f(cn[r]);
       }
-      *reinterpret_cast<v4h*>(cd.c + (size_t)row_g * H + u0) = cv;
-      *reinterpret_cast<v4h*>(cd.h + (size_t)row_g * H + u0) = hv;
+      if constexpr (SPLIT) {
+        *reinterpret_cast<v4f*>(reinterpret_cast<float*>(cd.c) + (size_t)row_g * H + u0) = cn;
+        *reinterpret_cast<v4f*>(reinterpret_cast<float*>(cd.h) + (size_t)row_g * H + u0) = hn;
+        v4h top, rest;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          const float hs = hn[r] * 16384.0f;  // |h| < 1: 2^14 keeps the value plane below 2^14
+          top[r] = (_Float16)hs;
+          rest[r] = (_Float16)(hs - (float)top[r]);
+        }
+        _Float16* hp = cd.h_planes + (size_t)row_g * 2 * H + u0;
+        *reinterpret_cast<v4h*>(hp) = top;
+        *reinterpret_cast<v4h*>(hp + H) = rest;
+      } else {
+        v4h hv, cv;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          cv[r] = (_Float16)cn[r];
+          hv[r] = (_Float16)hn[r];
+        }
+        *reinterpret_cast<v4h*>(reinterpret_cast<_Float16*>(cd.c) + (size_t)row_g * H + u0) = cv;
+        *reinterpret_cast<v4h*>(reinterpret_cast<_Float16*>(cd.h) + (size_t)row_g * H + u0) = hv;
+      }
     }
   }
 }
@@ -501,25 +577,29 @@ int pack_weights_f16(const void* WU, void* packed, int layers, int K2, int H, hi
   return check_launch("lstm_pack_weights_f16_kernel");
 }
 
-template <bool PACKED, int WAVES>
+template <bool PACKED, int WAVES, bool SPLIT>
 static int launch_cells_f16(const CellListH& list, int B, int I, int H, hipStream_t s) {
   static bool attr_set = false;  // per process; the attribute belongs to the function, on every device
   constexpr int UB = 8 * WAVES;
-  const void* fn = (const void*)lstm_cell_f16_kernel<PACKED, WAVES>;
+  const void* fn = (const void*)lstm_cell_f16_kernel<PACKED, WAVES, SPLIT>;
   if (!attr_set) {
     FTK_HIP(hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)cell_lds_bytes(UB)));
     attr_set = true;
   }
   const int groups = (list.n + 7) / 8;  // cells per XCD
   dim3 grid(8 * groups * (H / UB) * ((B + HROWS - 1) / HROWS));
-  hipLaunchKernelGGL((lstm_cell_f16_kernel<PACKED, WAVES>), grid, dim3(WAVES * 64), cell_lds_bytes(UB), s, list, B, I, H);
+  hipLaunchKernelGGL((lstm_cell_f16_kernel<PACKED, WAVES, SPLIT>), grid, dim3(WAVES * 64), cell_lds_bytes(UB), s, list, B, I,
+                     H);
   return check_launch("lstm_cell_f16_kernel");
 }
 
 static int launch_cells(const CellListH& list, int B, int I, int H, hipStream_t s) {
+  if (list.packed == 2)  // split products
+    return cell_unit_block(H) == 64 ? launch_cells_f16<true, 8, true>(list, B, I, H, s)
+                                    : launch_cells_f16<true, 4, true>(list, B, I, H, s);
   if (cell_unit_block(H) == 64)
-    return list.packed ? launch_cells_f16<true, 8>(list, B, I, H, s) : launch_cells_f16<false, 8>(list, B, I, H, s);
-  return list.packed ? launch_cells_f16<true, 4>(list, B, I, H, s) : launch_cells_f16<false, 4>(list, B, I, H, s);
+    return list.packed ? launch_cells_f16<true, 8, false>(list, B, I, H, s) : launch_cells_f16<false, 8, false>(list, B, I, H, s);
+  return list.packed ? launch_cells_f16<true, 4, false>(list, B, I, H, s) : launch_cells_f16<false, 4, false>(list, B, I, H, s);
 }
 
 // Host side of the per-stage schedule: stage(l,t) = 1 + max(stage(l-1,t),
@@ -528,9 +608,7 @@ static int launch_cells(const CellListH& list, int B, int I, int H, hipStream_t 
 static void set_packed(CellList&, bool) {}
 static void set_packed(CellListH& list, bool packed) { list.packed = packed; }
 
-template <typename Elem, typename List>
-static int run_wavefront_of(const Elem* xs, const Elem* WU, const float* bias, const int* dil, Elem* hsss, Elem* csss,
-                            int L, int T, int B, int H, hipStream_t s, bool packed = false) {
+static std::vector<std::vector<int>> cells_by_stage(int L, int T, const int* dil) {
   std::vector<int> stage((size_t)L * T, 0);
   int max_stage = 0;
   for (int l = 0; l < L; ++l) {
@@ -546,6 +624,13 @@ static int run_wavefront_of(const Elem* xs, const Elem* WU, const float* bias, c
   std::vector<std::vector<int>> by_stage(max_stage + 1);
   for (int l = 0; l < L; ++l)
     for (int t = 0; t < T; ++t) by_stage[stage[(size_t)l * T + t]].push_back(l * T + t);
+  return by_stage;
+}
+
+template <typename Elem, typename List>
+static int run_wavefront_of(const Elem* xs, const Elem* WU, const float* bias, const int* dil, Elem* hsss, Elem* csss,
+                            int L, int T, int B, int H, hipStream_t s, bool packed = false) {
+  const std::vector<std::vector<int>> by_stage = cells_by_stage(L, T, dil);
 
   const size_t cell = (size_t)B * H;
   for (const auto& cells : by_stage) {
@@ -591,6 +676,175 @@ int run_wavefront_f16(const void* xs, const void* WU, const float* bias, const i
                                                (_Float16*)hsss, (_Float16*)csss, L, T, B, H, s, packed != nullptr);
 }
 
+// ------------------------------------------------- fp32 stack on split products
+constexpr int kSplitTopExp = 14;  // a group's largest magnitude is scaled into [2^14, 2^15)
+
+// The power of two that brings a group maximum m into [2^14, 2^15), and its biased exponent (clamped so that
+// every scale and inverse scale derived from it is a normal fp32 number).
+__device__ __forceinline__ float split_scale(float m, int* biased_exp) {
+  const int eb = min(max((int)((__float_as_uint(m) >> 23) & 0xff), 40), 230);
+  *biased_exp = eb;
+  return __uint_as_float((unsigned)(127 + kSplitTopExp + 127 - eb) << 23);
+}
+
+// Rows of xs [rows, I] -> [rows, 2I] = [value plane | remainder plane] under the row's own scale, and the factor
+// 2^(eb - 127) that turns sums of such a row's products into the h rows' 2^14 scale.  One wave per row.
+__global__ __launch_bounds__(256) void lstm_split_rows_any_kernel(const float* __restrict__ xs, _Float16* __restrict__ xp,
+                                                                  float* __restrict__ xratio, int rows, int I) {
+  const int lane = threadIdx.x & 63;
+  const int row = blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (row >= rows) return;
+  const float* src = xs + (size_t)row * I;
+  float m = 0.0f;
+  for (int k = 4 * lane; k < I; k += 256) {
+    const float4 v = *reinterpret_cast<const float4*>(src + k);
+    m = fmaxf(m, fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w))));
+  }
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) m = fmaxf(m, __shfl_xor(m, o));
+  int eb;
+  const float scale = split_scale(m, &eb);
+  _Float16* dst = xp + (size_t)row * 2 * I;
+  for (int k = 4 * lane; k < I; k += 256) {
+    const float4 v = *reinterpret_cast<const float4*>(src + k);
+    const float vs[4] = {v.x * scale, v.y * scale, v.z * scale, v.w * scale};
+    v4h top, rest;
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      top[r] = (_Float16)vs[r];
+      rest[r] = (_Float16)(vs[r] - (float)top[r]);
+    }
+    *reinterpret_cast<v4h*>(dst + k) = top;
+    *reinterpret_cast<v4h*>(dst + I + k) = rest;
+  }
+  if (lane == 0) xratio[row] = __uint_as_float((unsigned)eb << 23);
+}
+
+// Per layer and weight column: the scale its values are split under (wmul) and what undoes it together with
+// the h rows' 2^14 after the sums (wscale).  One thread per column; neighbouring threads read neighbouring columns.
+__global__ __launch_bounds__(256) void lstm_col_scale_kernel(const float* __restrict__ WU, float* __restrict__ wmul,
+                                                             float* __restrict__ wscale, int layers, int K2, int N4) {
+  const size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;
+  if (idx >= (size_t)layers * N4) return;
+  const size_t l = idx / N4;
+  const int n = (int)(idx % N4);
+  const float* col = WU + l * K2 * N4 + n;
+  float m = 0.0f;
+  for (int k = 0; k < K2; ++k) m = fmaxf(m, fabsf(col[(size_t)k * N4]));
+  int eb;
+  wmul[idx] = split_scale(m, &eb);
+  wscale[idx] = __uint_as_float((unsigned)(eb - 2 * kSplitTopExp) << 23);  // 2^-(14 + 14 + 127 - eb)
+}
+
+// WU [layers, 2H, 4H] fp32 -> the packed rows of the split flavour: per layer and block of UB hidden units a
+// [6H][4*UB] fp16 tile in the kernel's LDS chunk order (see lstm_pack_weights_f16_kernel), where chunk c of 32 k
+// rows of the x half (then of the h half) appears three times: value plane, remainder plane, value plane.
+__global__ __launch_bounds__(256) void lstm_pack_split_weights_kernel(const float* __restrict__ WU,
+                                                                      const float* __restrict__ wmul,
+                                                                      _Float16* __restrict__ packed, size_t chunks, int H,
+                                                                      int UB) {
+  const size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;
+  if (idx >= chunks) return;
+  const int per_row = H / 2;  // 4H / 8
+  const int K2 = 2 * H;
+  const int n8 = (int)(idx % per_row);
+  const size_t lk = idx / per_row;
+  const int k = (int)(lk % K2);
+  const size_t l = lk / K2;
+  const int col = 8 * n8;
+  const int q = col / H, u = col % H;
+  const int ub = u / UB, ug = (u % UB) >> 3;
+  const int part = k / H, kk = k % H;
+  const float* src = WU + idx * 8;
+  const float* mul = wmul + l * 4 * H + col;
+  v8h top, rest;
+#pragma unroll
+  for (int r = 0; r < 8; ++r) {
+    const float vs = src[r] * mul[r];
+    top[r] = (_Float16)vs;
+    rest[r] = (_Float16)(vs - (float)top[r]);
+  }
+  const int slot = (4 * ug + q) ^ ((kk & 3) << 2);
+  const size_t vrow0 = (size_t)part * 3 * H + (size_t)(kk / 32) * 96 + (kk % 32);
+  _Float16* base = packed + (l * (H / UB) + ub) * (size_t)(6 * H) * (4 * UB) + 8 * slot;
+  *reinterpret_cast<v8h*>(base + vrow0 * (4 * UB)) = top;
+  *reinterpret_cast<v8h*>(base + (vrow0 + 32) * (4 * UB)) = rest;
+  *reinterpret_cast<v8h*>(base + (vrow0 + 64) * (4 * UB)) = top;
+}
+
+static size_t round256s(size_t v) { return (v + 255) / 256 * 256; }
+
+// Workspace of the split-product stack: [wscale L*4H][wmul L*4H][xratio T*B] floats, then fp16 [xp T*B*2H]
+// [hp L*T*B*2H][packed weights L*6H*4H], every part on a 256-byte boundary.
+size_t split_stack_workspace_bytes(int L, int T, int B, int H) {
+  size_t n = 2 * round256s((size_t)L * 4 * H * sizeof(float)) + round256s((size_t)T * B * sizeof(float));
+  n += round256s((size_t)T * B * 2 * H * sizeof(_Float16)) + round256s((size_t)L * T * B * 2 * H * sizeof(_Float16));
+  n += (size_t)L * 6 * H * 4 * H * sizeof(_Float16);
+  return n;
+}
+
+// The fp32 stack through the split flavour of the streaming cell kernel (H a multiple of 32).
+int run_wavefront_split(const float* xs, const float* WU, const float* bias, const int* dil, float* hsss, float* csss,
+                        int L, int T, int B, int H, void* ws, hipStream_t s) {
+  char* p = reinterpret_cast<char*>(ws);
+  float* wscale = reinterpret_cast<float*>(p);
+  p += round256s((size_t)L * 4 * H * sizeof(float));
+  float* wmul = reinterpret_cast<float*>(p);
+  p += round256s((size_t)L * 4 * H * sizeof(float));
+  float* xratio = reinterpret_cast<float*>(p);
+  p += round256s((size_t)T * B * sizeof(float));
+  _Float16* xp = reinterpret_cast<_Float16*>(p);
+  p += round256s((size_t)T * B * 2 * H * sizeof(_Float16));
+  _Float16* hp = reinterpret_cast<_Float16*>(p);
+  p += round256s((size_t)L * T * B * 2 * H * sizeof(_Float16));
+  _Float16* wp = reinterpret_cast<_Float16*>(p);
+
+  const int UB = cell_unit_block(H);
+  const size_t cols = (size_t)L * 4 * H;
+  hipLaunchKernelGGL(lstm_col_scale_kernel, dim3((unsigned)((cols + 255) / 256)), dim3(256), 0, s, WU, wmul, wscale, L,
+                     2 * H, 4 * H);
+  int rc = check_launch("lstm_col_scale_kernel");
+  if (rc) return rc;
+  const size_t chunks = (size_t)L * 2 * H * (H / 2);
+  hipLaunchKernelGGL(lstm_pack_split_weights_kernel, dim3((unsigned)((chunks + 255) / 256)), dim3(256), 0, s, WU, wmul, wp,
+                     chunks, H, UB);
+  rc = check_launch("lstm_pack_split_weights_kernel");
+  if (rc) return rc;
+  const int rows = T * B;
+  hipLaunchKernelGGL(lstm_split_rows_any_kernel, dim3((rows + 3) / 4), dim3(256), 0, s, xs, xp, xratio, rows, H);
+  rc = check_launch("lstm_split_rows_any_kernel");
+  if (rc) return rc;
+
+  const size_t cell = (size_t)B * H;
+  for (const auto& cells : cells_by_stage(L, T, dil)) {
+    size_t pos = 0;
+    while (pos < cells.size()) {
+      CellListH list;
+      list.n = 0;
+      list.packed = 2;
+      while (pos < cells.size() && list.n < kMaxCellsPerLaunch) {
+        const int l = cells[pos] / T, t = cells[pos] % T;
+        const int d = dil ? dil[l] : 1;
+        CellDescH& cd = list.cells[list.n++];
+        cd.x = (l == 0) ? xp + (size_t)t * 2 * cell : hp + ((size_t)(l - 1) * T + t) * 2 * cell;
+        cd.h_prev = (t >= d) ? hp + ((size_t)l * T + t - d) * 2 * cell : nullptr;
+        cd.c_prev = (t >= d) ? csss + ((size_t)l * T + t - d) * cell : nullptr;
+        cd.WU = wp + (size_t)l * 6 * H * 4 * H;
+        cd.bias = bias ? bias + (size_t)l * 4 * H : nullptr;
+        cd.h = hsss + ((size_t)l * T + t) * cell;
+        cd.c = csss + ((size_t)l * T + t) * cell;
+        cd.xratio = (l == 0) ? xratio + (size_t)t * B : nullptr;
+        cd.wscale = wscale + (size_t)l * 4 * H;
+        cd.h_planes = hp + ((size_t)l * T + t) * 2 * cell;
+        ++pos;
+      }
+      rc = launch_cells(list, B, H, H, s);
+      if (rc) return rc;
+    }
+  }
+  return FTK_OK;
+}
+
 }  // namespace ftk
 
 extern "C" {
@@ -623,8 +877,8 @@ int ftk_lstm_cell_f16(const void* x, const void* h_prev, const void* c_prev, con
   ftk::CellListH list;
   list.n = 1;
   list.packed = 0;
-  list.cells[0] = ftk::CellDescH{(const _Float16*)x, (const _Float16*)h_prev, (const _Float16*)c_prev,
-                                 (const _Float16*)WU, bias, (_Float16*)h, (_Float16*)c};
+  list.cells[0] = ftk::CellDescH{(const _Float16*)x, (const _Float16*)h_prev, c_prev, (const _Float16*)WU, bias, h, c,
+                                 nullptr, nullptr, nullptr};
   return ftk::launch_cells(list, B, I, H, (hipStream_t)stream);
 }
 

@@ -53,6 +53,9 @@ int run_wavefront(const float* xs, const float* WU, const float* bias, const int
                   int L, int T, int B, int H, hipStream_t s);
 int run_wavefront_f16(const void* xs, const void* WU, const float* bias, const int* dil, void* hsss, void* csss,
                       int L, int T, int B, int H, void* packed, hipStream_t s);
+size_t split_stack_workspace_bytes(int L, int T, int B, int H);
+int run_wavefront_split(const float* xs, const float* WU, const float* bias, const int* dil, float* hsss, float* csss,
+                        int L, int T, int B, int H, void* ws, hipStream_t s);
 
 constexpr int PH = 256;            // hidden size this kernel is specialised for
 constexpr int PK = 2 * PH;         // K of the gate GEMM
@@ -1021,6 +1024,11 @@ static int run_stack(const char* who, const float* xs, const float* WU, const fl
                         ws, ws_bytes, s, &handled);
     if (rc || handled) return rc;
   }
+  // Other hidden sizes: one launch per stage of independent cells.  With split products (the default) and the
+  // workspace the size query asks for, through the fp16-MFMA streaming kernel; else on fp32 MFMAs.
+  if (H != PH && products_mode() == FTK_LSTM_PRODUCTS_F16X3 && ws && ws_bytes >= split_stack_workspace_bytes(L, T, B, H) &&
+      (long long)B * H < (1ll << 29))
+    return run_wavefront_split(xs, WU, bias, dil, hsss, csss, L, T, B, H, ws, s);
   return run_wavefront(xs, WU, bias, dil, hsss, csss, L, T, B, H, s);
 }
 
@@ -1049,6 +1057,7 @@ extern "C" {
 
 size_t ftk_stacked_lstm_workspace_bytes(int L, int T, int B, int H) {
   if (L <= 0 || T <= 0 || B <= 0 || H <= 0) return 0;
+  if (H != ftk::PH && H % 32 == 0) return ftk::split_stack_workspace_bytes(L, T, B, H);  // planes, scales, re-laid weights
   return ftk::workspace_need(L, T, B);
 }
 

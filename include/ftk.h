@@ -107,9 +107,16 @@ size_t ftk_stacked_lstm_workspace_bytes(int L, int T, int B, int H);
  * L stacked LSTM layers over T steps; layer l reads layer l-1's hidden
  * sequence; zero initial state.  xs [T,B,H], WU [L,2H,4H], bias [L,4H] or
  * NULL, outputs hsss/csss [L,T,B,H] (every layer's h and c at every step).
- * One persistent launch walks the (layer,time) wavefront with each layer's
- * weights held in registers; shapes it is not specialised for fall back to
- * one fused-cell launch per wavefront diagonal.
+ * H%32==0.  At H = 256 one persistent launch walks the (layer,time) wavefront
+ * with each layer's weights held in registers.  Other hidden sizes do not fit
+ * on chip and run as one fused-cell launch per wavefront diagonal with the
+ * weights streamed: in the default product mode (see ftk_lstm_set_products)
+ * through the fp16-MFMA kernel on operands split into two fp16 planes, for
+ * which the workspace holds the planes of xs and of every h, the column
+ * scales and a re-laid copy of the split weights (about 1.5x the bytes of WU
+ * plus those of hsss; ftk_stacked_lstm_workspace_bytes says how much); with a
+ * smaller workspace or in the fp32-product mode through the fp32-MFMA cell
+ * kernel of ftk_lstm_cell_f32, which needs none.
  * Replaces StackedLstmRegion1/2/3
  * (kaleido/core/device/kernels/lstm/stacked_lstm/region1.h:11-43,
  * region2.h:15-70, region3.h:18-140) and the Python stacked_lstm
@@ -188,7 +195,9 @@ int ftk_stacked_lstm_f16(const void* xs, const void* WU, const float* bias,
  * by its weight column / activation row, three fp16 MFMAs with fp32
  * accumulation take the place of the fp32 one and only the remainder x
  * remainder term (2^-22 of a product) is dropped; inputs, state, outputs and
- * accumulation stay fp32.  The environment variable FTK_LSTM_PRODUCTS=f32 or
+ * accumulation stay fp32.  The streamed path of the other hidden sizes forms
+ * the same three products (as three k chunks per chunk of the contraction)
+ * and keeps the remainders unscaled.  The environment variable FTK_LSTM_PRODUCTS=f32 or
  * =f16x3 sets the initial mode.  A tuning control of this library: the
  * reference has one fp32 (cuBLAS) and one fp16 (CuTe) LSTM and no switch.
  */

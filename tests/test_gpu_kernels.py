@@ -350,14 +350,51 @@ def test_stacked_lstm_config4_full_size(core, products):
     assert torch.equal(h1, h3)
 
 
-@pytest.mark.parametrize('H', [512, 1024])
-def test_stacked_lstm_larger_hidden_sizes_through_the_default_entry(core, H):
-    """H != 256 is not what the persistent kernel is specialised for: the default entry point falls back to
-    per-stage launches of the streaming cell kernel and must give the same answer."""
-    L, T, B = 2, 4, 48
-    xs, WU, bs = lstm_inputs(31, L, T, B, H, 1.0 / 32)
-    hsss, csss = core.stacked_lstm(dev(xs), dev(WU), dev(bs))
-    hr, cr = c_oracle.stacked_lstm(xs, WU, bs, None)
+@pytest.mark.parametrize('L,T,B,H,dil,bias', [
+    (2, 4, 48, 512, None, True),
+    (2, 4, 48, 1024, None, True),
+    (3, 6, 300, 96, [1, 2, 4], False),      # 32 hidden units per workgroup; two row blocks, the second ragged
+    (2, 5, 33, 64, None, True),
+    (9, 3, 20, 128, None, True),            # nine cells in a stage
+    (2, 7, 1, 320, [1, 3], True),           # one sequence
+])
+def test_stacked_lstm_other_hidden_sizes_through_the_default_entry(core, products, L, T, B, H, dil, bias):
+    """H != 256 is not what the persistent kernel holds on chip: the default entry point runs one launch per stage
+    of cells, in the split-product mode through the fp16-MFMA streaming kernel (operands as two fp16 planes, three
+    k chunks per chunk of the contraction), in the fp32-product mode through the fp32 cell kernel."""
+    xs, WU, bs = lstm_inputs(31, L, T, B, H, 1.0 / np.sqrt(4 * H), bias=bias)
+    xs[1] *= 4.0                             # rows of different magnitude: every x row has its own scale
+    xs[0, 0] *= 1e-3
+    hsss, csss = core.stacked_lstm(dev(xs), dev(WU), None if bs is None else dev(bs), dilations=dil)
+    hr, cr = c_oracle.stacked_lstm(xs, WU, bs, dil) if dil is None else ko.stacked_lstm(xs, WU, bs, dilations=dil)
+    assert_lstm_close(hsss, hr, 'hsss'); assert_lstm_close(csss, cr, 'csss')
+
+
+def test_split_products_of_the_streamed_stack_are_as_accurate_as_fp32_products(core):
+    """Against float64, the three-fp16-MFMA products of the streamed stack (H = 512) are not less accurate than
+    fp32 MFMAs: only the remainder x remainder term, 2^-22 of a product, is dropped."""
+    L, T, B, H = 3, 8, 64, 512
+    xs, WU, bs = lstm_inputs(77, L, T, B, H, 1.0 / 32)
+    hr, _ = ko.stacked_lstm(xs, WU, bs)
+    errs = {}
+    before = core.get_lstm_products()
+    try:
+        for mode in ('f16x3', 'f32'):
+            core.set_lstm_products(mode)
+            h, _ = core.stacked_lstm(dev(xs), dev(WU), dev(bs))
+            errs[mode] = ko.max_rel_err(h.cpu().numpy(), hr)
+    finally:
+        core.set_lstm_products(before)
+    assert errs['f16x3'] <= LSTM_TOL / 20 and errs['f16x3'] <= 2 * errs['f32'], errs
+
+
+def test_stacked_lstm_other_hidden_sizes_without_workspace_room(core):
+    """A workspace smaller than the split-product stack needs sends it through the fp32 cell kernel: same answer."""
+    L, T, B, H = 2, 3, 40, 128
+    xs, WU, bs = lstm_inputs(32, L, T, B, H, 0.05)
+    small = torch.empty(1024, dtype=torch.uint8, device='cuda')
+    hsss, csss = core.stacked_lstm(dev(xs), dev(WU), dev(bs), workspace=small)
+    hr, cr = ko.stacked_lstm(xs, WU, bs)
     assert_lstm_close(hsss, hr, 'hsss'); assert_lstm_close(csss, cr, 'csss')
 
 
