@@ -23,6 +23,8 @@
 // hidden units so that every weight is fetched once per cell, and k chunks of
 // 32 copied from global memory straight into a ring of three to five LDS stages
 // (global_load_lds_dwordx4), two workgroups per compute unit.
+#include <stdlib.h>
+
 #include <algorithm>
 #include <vector>
 
@@ -230,7 +232,7 @@ struct CellDescH {
 
 struct CellListH {
   int n;
-  int packed;  // 1: WU of every cell is in the packed layout; 2: packed split weights, the split flavour
+  int packed;  // 1: WU of every cell is in the packed layout; 2, 3: packed split weights (three / two planes per chunk)
   CellDescH cells[kMaxCellsPerLaunch];
 };
 
@@ -540,6 +542,195 @@ __global__ __launch_bounds__(WAVES * 64, 8 / WAVES) void lstm_cell_f16_kernel(Ce
   }
 }
 
+// ------------------------------------------------ split flavour, four tiles per chunk
+// The split products of a chunk from one copy of each plane: a stage holds the four tiles [x value][x
+// remainder][w value][w remainder] of a 32-row chunk (64 KB at 64 hidden units per workgroup), and the three
+// products (w value, x value), (w remainder, x value), (w value, x remainder) are formed from them: two thirds of
+// the copies and of the LDS fragment reads of the three-chunks-in-a-row form above.  Two stages (128 KB): the
+// next chunk is copied while this one is used, 48 MFMAs per wave.  8 waves, the wave tiling and every LDS layout
+// as in lstm_cell_f16_kernel<true, 8, true>; packed weights as [chunk][plane][32 rows][512 bytes] per unit block
+// (lstm_pack_split_weights_kernel with planes = 2).
+constexpr int S4_TILE = 16384;
+constexpr int S4_STAGE = 4 * S4_TILE;
+constexpr size_t kSplit4Lds = 2 * S4_STAGE;
+
+__global__ __launch_bounds__(512, 1) void lstm_cell_split4_kernel(CellListH list, int B, int I, int H) {
+  constexpr int UB = 64, ROWB = 512;
+  extern __shared__ __attribute__((aligned(1024))) unsigned char cell_smem[];
+  using lds_v4s = __attribute__((address_space(3))) v4s;
+
+  const int nub = H / UB, nrb = (B + HROWS - 1) / HROWS;
+  const int slot = blockIdx.x >> 3;
+  const int cell = (blockIdx.x & 7) + 8 * (slot / (nub * nrb));  // all workgroups of a cell on one XCD
+  if (cell >= list.n) return;
+  const CellDescH cd = list.cells[cell];
+  const int ub = slot % nub;
+  const int rb = (slot / nub) % nrb;
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int wr = wave >> 2;  // rows 128*wr .. +128 of the block
+  const int wc = wave & 3;   // unit groups 2*wc, 2*wc+1 of the block's eight
+  const int j = lane & 31;
+  const int hh = lane >> 5;
+  const unsigned lds0 = (unsigned)reinterpret_cast<uintptr_t>((__attribute__((address_space(3))) void*)cell_smem);
+
+  const int nch_x = I / HK;
+  const int nch = nch_x + (cd.h_prev ? H / HK : 0);
+  const bool full = rb * HROWS + HROWS <= B;
+
+  // per chunk a wave issues 2 + 2 activation copies (rows 32*wave + 16 i + lane/4 of each plane) and 2 + 2
+  // weight copies (1 KB = rows 4*wave + 2 i + lane/32 of each plane, already in LDS order)
+  const unsigned a_lane_chunk = (unsigned)(((lane & 3) ^ ((lane >> 4) & 3)) * 16);
+  auto issue = [&](int ch, int stage) __attribute__((always_inline)) {
+    const bool in_x = ch < nch_x;
+    const int width = in_x ? I : H;
+    const _Float16* src = (in_x ? cd.x : cd.h_prev) + (in_x ? ch : ch - nch_x) * HK;
+    const int ld = 2 * width;
+    const int row0 = wave * 32;
+    const unsigned st = lds0 + (unsigned)(stage * S4_STAGE);
+#pragma unroll
+    for (int pl = 0; pl < 2; ++pl) {
+      const unsigned act_lds = st + (unsigned)(pl * S4_TILE + row0 * 64);
+      if (full) {
+        const char* base = reinterpret_cast<const char*>(src + pl * width + (size_t)(rb * HROWS + row0) * ld);
+        const unsigned off = ((unsigned)lane >> 2) * (unsigned)(2 * ld) + a_lane_chunk;
+#pragma unroll
+        for (int i = 0; i < 2; ++i) cell_dma16(base + (size_t)i * 32 * ld, off, act_lds + 1024u * i);
+      } else {  // rows past the end of the batch repeat the last row; they are never stored
+        const char* base = reinterpret_cast<const char*>(src + pl * width);
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+          const int row = min(rb * HROWS + row0 + 16 * i + (lane >> 2), B - 1);
+          cell_dma16(base, (unsigned)row * (unsigned)(2 * ld) + a_lane_chunk, act_lds + 1024u * i);
+        }
+      }
+    }
+    const char* wbase = reinterpret_cast<const char*>(cd.WU) + ((size_t)ub * (I + H) + ch * HK) * 2 * ROWB + wave * 2048;
+#pragma unroll
+    for (int pl = 0; pl < 2; ++pl)
+#pragma unroll
+      for (int i = 0; i < 2; ++i)
+        cell_dma16(wbase + pl * S4_TILE + 1024 * i, 16u * lane, st + (unsigned)((2 + pl) * S4_TILE + wave * 2048 + 1024 * i));
+  };
+
+  unsigned a_off[2], w_off[2];
+#pragma unroll
+  for (int ks = 0; ks < 2; ++ks) a_off[ks] = (unsigned)((128 * wr + j) * 64 + (((2 * ks + hh) ^ ((j >> 2) & 3)) * 16));
+  {
+    const int ta = (lane & 15) >> 2, tb = lane & 3, th = (lane >> 4) & 1;
+#pragma unroll
+    for (int u2 = 0; u2 < 2; ++u2)
+      w_off[u2] = (unsigned)(2 * S4_TILE + (8 * hh + ta) * ROWB +
+                             (((4 * (2 * wc + u2) + 2 * th + (tb >> 1)) ^ (ta << 2)) * 16) + 8 * (tb & 1));
+  }
+
+  v16f acc[4][2];
+#pragma unroll
+  for (int rt = 0; rt < 4; ++rt)
+#pragma unroll
+    for (int u2 = 0; u2 < 2; ++u2)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[rt][u2][r] = 0.0f;
+
+  auto rescale_x = [&]() __attribute__((always_inline)) {
+    if (!cd.xratio) return;
+#pragma unroll
+    for (int rt = 0; rt < 4; ++rt) {
+      const float ratio = cd.xratio[min(rb * HROWS + 128 * wr + 32 * rt + j, B - 1)];
+#pragma unroll
+      for (int u2 = 0; u2 < 2; ++u2)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[rt][u2][r] *= ratio;
+    }
+  };
+
+  issue(0, 0);
+  for (int ch = 0; ch < nch; ++ch) {
+    __builtin_amdgcn_s_waitcnt(vmcnt_only(0));
+    __syncthreads();  // chunk ch is complete, and every wave is done with the stage of chunk ch-1
+    const unsigned char* sb = cell_smem + (ch & 1) * S4_STAGE;
+    if (ch + 1 < nch) issue(ch + 1, (ch + 1) & 1);
+    if (ch == nch_x) rescale_x();
+#pragma unroll
+    for (int ks = 0; ks < 2; ++ks) {
+      v8h wt[2], wre[2];
+#pragma unroll
+      for (int u2 = 0; u2 < 2; ++u2) {
+#pragma unroll
+        for (int pl = 0; pl < 2; ++pl) {
+          const unsigned char* p0 = sb + w_off[u2] + pl * S4_TILE + 16 * ROWB * ks;
+          const v4s lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4s*)(p0));
+          const v4s hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4s*)(p0 + 4 * ROWB));
+          const v8s both = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+          (pl ? wre[u2] : wt[u2]) = __builtin_bit_cast(v8h, both);
+        }
+      }
+      v8h at[4], ar[4];
+#pragma unroll
+      for (int rt = 0; rt < 4; ++rt) {
+        at[rt] = *reinterpret_cast<const v8h*>(sb + a_off[ks] + 2048 * rt);
+        ar[rt] = *reinterpret_cast<const v8h*>(sb + S4_TILE + a_off[ks] + 2048 * rt);
+      }
+      // product by product, so that the MFMAs that add into one accumulator are eight apart
+#pragma unroll
+      for (int rt = 0; rt < 4; ++rt)
+#pragma unroll
+        for (int u2 = 0; u2 < 2; ++u2) acc[rt][u2] = __builtin_amdgcn_mfma_f32_32x32x16_f16(wt[u2], at[rt], acc[rt][u2], 0, 0, 0);
+#pragma unroll
+      for (int rt = 0; rt < 4; ++rt)
+#pragma unroll
+        for (int u2 = 0; u2 < 2; ++u2) acc[rt][u2] = __builtin_amdgcn_mfma_f32_32x32x16_f16(wre[u2], at[rt], acc[rt][u2], 0, 0, 0);
+#pragma unroll
+      for (int rt = 0; rt < 4; ++rt)
+#pragma unroll
+        for (int u2 = 0; u2 < 2; ++u2) acc[rt][u2] = __builtin_amdgcn_mfma_f32_32x32x16_f16(wt[u2], ar[rt], acc[rt][u2], 0, 0, 0);
+    }
+  }
+  if (nch == nch_x) rescale_x();  // zero state: there was no h chunk to do it before
+
+#pragma unroll
+  for (int rt = 0; rt < 4; ++rt) {
+    const int row_g = rb * HROWS + 128 * wr + 32 * rt + j;
+    if (row_g >= B) continue;
+#pragma unroll
+    for (int u2 = 0; u2 < 2; ++u2) {
+      const int u0 = ub * UB + 8 * (2 * wc + u2) + 4 * hh;
+      v4f cp = {0, 0, 0, 0};
+      if (cd.c_prev) cp = *reinterpret_cast<const v4f*>(reinterpret_cast<const float*>(cd.c_prev) + (size_t)row_g * H + u0);
+      v4f bi = {0, 0, 0, 0}, bf = bi, bo = bi, bg = bi;
+      if (cd.bias) {
+        bi = *reinterpret_cast<const v4f*>(cd.bias + u0);
+        bf = *reinterpret_cast<const v4f*>(cd.bias + H + u0);
+        bo = *reinterpret_cast<const v4f*>(cd.bias + 2 * H + u0);
+        bg = *reinterpret_cast<const v4f*>(cd.bias + 3 * H + u0);
+      }
+      const v4f si = *reinterpret_cast<const v4f*>(cd.wscale + u0);
+      const v4f sf = *reinterpret_cast<const v4f*>(cd.wscale + H + u0);
+      const v4f so = *reinterpret_cast<const v4f*>(cd.wscale + 2 * H + u0);
+      const v4f sg = *reinterpret_cast<const v4f*>(cd.wscale + 3 * H + u0);
+      v4f hn, cn;
+      v4h top, rest;
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const float ig = sigmoid_f(acc[rt][u2][r] * si[r] + bi[r]);
+        const float fg = sigmoid_f(acc[rt][u2][4 + r] * sf[r] + bf[r]);
+        const float og = sigmoid_f(acc[rt][u2][8 + r] * so[r] + bo[r]);
+        const float cand = tanh_f(acc[rt][u2][12 + r] * sg[r] + bg[r]);
+        cn[r] = fg * cp[r] + ig * cand;
+        hn[r] = og * tanh_f(cn[r]);
+        const float hs = hn[r] * 16384.0f;
+        top[r] = (_Float16)hs;
+        rest[r] = (_Float16)(hs - (float)top[r]);
+      }
+      *reinterpret_cast<v4f*>(reinterpret_cast<float*>(cd.c) + (size_t)row_g * H + u0) = cn;
+      *reinterpret_cast<v4f*>(reinterpret_cast<float*>(cd.h) + (size_t)row_g * H + u0) = hn;
+      _Float16* hp = cd.h_planes + (size_t)row_g * 2 * H + u0;
+      *reinterpret_cast<v4h*>(hp) = top;
+      *reinterpret_cast<v4h*>(hp + H) = rest;
+    }
+  }
+}
+
 static int launch_cells(const CellList& list, int B, int I, int H, hipStream_t s) {
   dim3 grid(H / 32, (B + 31) / 32, list.n);
   hipLaunchKernelGGL(lstm_cell_kernel, grid, dim3(256), 0, s, list, B, I, H);
@@ -594,7 +785,19 @@ static int launch_cells_f16(const CellListH& list, int B, int I, int H, hipStrea
 }
 
 static int launch_cells(const CellListH& list, int B, int I, int H, hipStream_t s) {
-  if (list.packed == 2)  // split products
+  if (list.packed == 3) {  // split products, four tiles per chunk
+    static bool attr_set = false;
+    if (!attr_set) {
+      FTK_HIP(hipFuncSetAttribute((const void*)lstm_cell_split4_kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                  (int)kSplit4Lds));
+      attr_set = true;
+    }
+    const int groups = (list.n + 7) / 8;
+    dim3 grid(8 * groups * (H / 64) * ((B + HROWS - 1) / HROWS));
+    hipLaunchKernelGGL(lstm_cell_split4_kernel, grid, dim3(512), kSplit4Lds, s, list, B, I, H);
+    return check_launch("lstm_cell_split4_kernel");
+  }
+  if (list.packed == 2)  // split products, three chunks in a row
     return cell_unit_block(H) == 64 ? launch_cells_f16<true, 8, true>(list, B, I, H, s)
                                     : launch_cells_f16<true, 4, true>(list, B, I, H, s);
   if (cell_unit_block(H) == 64)
@@ -742,7 +945,7 @@ __global__ __launch_bounds__(256) void lstm_col_scale_kernel(const float* __rest
 __global__ __launch_bounds__(256) void lstm_pack_split_weights_kernel(const float* __restrict__ WU,
                                                                       const float* __restrict__ wmul,
                                                                       _Float16* __restrict__ packed, size_t chunks, int H,
-                                                                      int UB) {
+                                                                      int UB, int planes) {
   const size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;
   if (idx >= chunks) return;
   const int per_row = H / 2;  // 4H / 8
@@ -765,11 +968,12 @@ __global__ __launch_bounds__(256) void lstm_pack_split_weights_kernel(const floa
     rest[r] = (_Float16)(vs - (float)top[r]);
   }
   const int slot = (4 * ug + q) ^ ((kk & 3) << 2);
-  const size_t vrow0 = (size_t)part * 3 * H + (size_t)(kk / 32) * 96 + (kk % 32);
-  _Float16* base = packed + (l * (H / UB) + ub) * (size_t)(6 * H) * (4 * UB) + 8 * slot;
+  // planes = 3: value, remainder, value again (three chunks in a row); planes = 2: value, remainder
+  const size_t vrow0 = (size_t)part * planes * H + (size_t)(kk / 32) * (32 * planes) + (kk % 32);
+  _Float16* base = packed + (l * (H / UB) + ub) * (size_t)(2 * planes * H) * (4 * UB) + 8 * slot;
   *reinterpret_cast<v8h*>(base + vrow0 * (4 * UB)) = top;
   *reinterpret_cast<v8h*>(base + (vrow0 + 32) * (4 * UB)) = rest;
-  *reinterpret_cast<v8h*>(base + (vrow0 + 64) * (4 * UB)) = top;
+  if (planes == 3) *reinterpret_cast<v8h*>(base + (vrow0 + 64) * (4 * UB)) = top;
 }
 
 static size_t round256s(size_t v) { return (v + 255) / 256 * 256; }
@@ -800,6 +1004,9 @@ int run_wavefront_split(const float* xs, const float* WU, const float* bias, con
   _Float16* wp = reinterpret_cast<_Float16*>(p);
 
   const int UB = cell_unit_block(H);
+  // 64 hidden units per workgroup: every plane copied once per chunk (four tiles); else three chunks in a row
+  const bool four_tiles = UB == 64 && !getenv("FTK_LSTM_SPLIT_ROWS3");
+  const int planes = four_tiles ? 2 : 3;
   const size_t cols = (size_t)L * 4 * H;
   hipLaunchKernelGGL(lstm_col_scale_kernel, dim3((unsigned)((cols + 255) / 256)), dim3(256), 0, s, WU, wmul, wscale, L,
                      2 * H, 4 * H);
@@ -807,7 +1014,7 @@ int run_wavefront_split(const float* xs, const float* WU, const float* bias, con
   if (rc) return rc;
   const size_t chunks = (size_t)L * 2 * H * (H / 2);
   hipLaunchKernelGGL(lstm_pack_split_weights_kernel, dim3((unsigned)((chunks + 255) / 256)), dim3(256), 0, s, WU, wmul, wp,
-                     chunks, H, UB);
+                     chunks, H, UB, planes);
   rc = check_launch("lstm_pack_split_weights_kernel");
   if (rc) return rc;
   const int rows = T * B;
@@ -821,7 +1028,7 @@ int run_wavefront_split(const float* xs, const float* WU, const float* bias, con
     while (pos < cells.size()) {
       CellListH list;
       list.n = 0;
-      list.packed = 2;
+      list.packed = four_tiles ? 3 : 2;
       while (pos < cells.size() && list.n < kMaxCellsPerLaunch) {
         const int l = cells[pos] / T, t = cells[pos] % T;
         const int d = dil ? dil[l] : 1;
@@ -829,7 +1036,7 @@ int run_wavefront_split(const float* xs, const float* WU, const float* bias, con
         cd.x = (l == 0) ? xp + (size_t)t * 2 * cell : hp + ((size_t)(l - 1) * T + t) * 2 * cell;
         cd.h_prev = (t >= d) ? hp + ((size_t)l * T + t - d) * 2 * cell : nullptr;
         cd.c_prev = (t >= d) ? csss + ((size_t)l * T + t - d) * cell : nullptr;
-        cd.WU = wp + (size_t)l * 6 * H * 4 * H;
+        cd.WU = wp + (size_t)l * 2 * planes * H * 4 * H;
         cd.bias = bias ? bias + (size_t)l * 4 * H : nullptr;
         cd.h = hsss + ((size_t)l * T + t) * cell;
         cd.c = csss + ((size_t)l * T + t) * cell;

@@ -388,6 +388,20 @@ def test_split_products_of_the_streamed_stack_are_as_accurate_as_fp32_products(c
     assert errs['f16x3'] <= LSTM_TOL / 20 and errs['f16x3'] <= 2 * errs['f32'], errs
 
 
+def test_streamed_split_stack_three_chunks_in_a_row_at_64_units(core, monkeypatch):
+    """At H % 64 == 0 the split stack copies every plane once per chunk (four tiles); FTK_LSTM_SPLIT_ROWS3=1 selects
+    the form that H % 64 != 0 uses (the three products as three chunks in a row): same answer."""
+    L, T, B, H = 2, 5, 70, 128
+    xs, WU, bs = lstm_inputs(33, L, T, B, H, 0.05)
+    hr, cr = ko.stacked_lstm(xs, WU, bs)
+    h4, c4 = core.stacked_lstm(dev(xs), dev(WU), dev(bs))
+    monkeypatch.setenv('FTK_LSTM_SPLIT_ROWS3', '1')
+    h3, c3 = core.stacked_lstm(dev(xs), dev(WU), dev(bs))
+    torch.cuda.synchronize()
+    assert_lstm_close(h4, hr, 'four tiles h'); assert_lstm_close(c4, cr, 'four tiles c')
+    assert_lstm_close(h3, hr, 'three chunks h'); assert_lstm_close(c3, cr, 'three chunks c')
+
+
 def test_stacked_lstm_other_hidden_sizes_without_workspace_room(core):
     """A workspace smaller than the split-product stack needs sends it through the fp32 cell kernel: same answer."""
     L, T, B, H = 2, 3, 40, 128
