@@ -398,12 +398,59 @@ def bench_lstm_f16(torch, core, steps, warmup, cpu, H, baselines=True):
     return res
 
 
+def bench_lstm_f32_streamed(torch, core, steps, warmup, cpu, H):
+    """The fp32 stack at the larger hidden sizes of the reference's sweep: weights streamed, one launch per stage of
+    cells; split products through the fp16-MFMA streaming kernel (default) beside fp32 MFMAs."""
+    L, T, B = 32, 64, 256
+    flop = 2.0 * L * T * B * (2 * H) * (4 * H)
+    gen = torch.Generator(device='cpu').manual_seed(1234)
+    xs = torch.randn((T, B, H), generator=gen).cuda()
+    WU = ((torch.rand((L, 2 * H, 4 * H), generator=gen) - 0.5) / (H ** 0.5 / 2)).cuda()
+    hs = torch.empty((L, T, B, H), device='cuda')
+    cs = torch.empty_like(hs)
+    ws = torch.empty(int(core.stacked_lstm_workspace_bytes(L, T, B, H)), dtype=torch.uint8, device='cuda')
+    run = lambda: core.stacked_lstm(xs, WU, out=(hs, cs), workspace=ws)
+    before = core.get_lstm_products()
+    try:
+        core.set_lstm_products('f16x3')
+        ms, _ = _events_ms(torch, run, steps, warmup)
+        ref = hs.clone()
+        core.set_lstm_products('f32')
+        ms32, _ = _events_ms(torch, run, max(2, steps // 2), 1)
+        diff = float((hs - ref).abs().max() / ref.abs().max())
+    finally:
+        core.set_lstm_products(before)
+    res = {
+        'metric': 'stacked-LSTM sequences/s', 'value': B / ms * 1e3, 'unit': 'sequences/s', 'ms_per_step': ms,
+        'dtype': 'f32 (gate products as three f16 MFMAs of split operands, f32 accumulate)',
+        'config': {'workload': f'stacked LSTM, fp32, the H = {H} row of the reference sweep', 'layers': L, 'batch': B, 'seq_len': T,
+                   'hidden': H, 'outputs': 'h and c of every layer at every step',
+                   'schedule': 'one launch of the split-product streaming cell kernel per stage of independent cells'},
+        'tflops': flop / ms / 1e9, 'frac_of_f32_matrix_peak_algorithmic': flop / ms / 1e9 / PEAK_F32_MATRIX_TFLOPS,
+        'fp32_mfma_products': {'ms_per_step': ms32, 'speedup_of_split_products': ms32 / ms, 'max_rel_diff': diff},
+        'roofline': {'bound': 'mfma', 'achieved': 3 * flop / ms / 1e9, 'peak': PEAK_F16_TFLOPS, 'unit': 'TFLOP/s',
+                     'frac': 3 * flop / ms / 1e9 / PEAK_F16_TFLOPS, 'traffic': None, 'kernel': 'lstm_cell_split4_kernel',
+                     'note': 'executed f16 MFMA flops (three per algorithmic product) against the f16 MFMA peak'},
+    }
+    if cpu:
+        from oracle import c_oracle
+        Ls, Ts, Bs = 2, 16, 64
+        t0 = time.perf_counter()
+        c_oracle.stacked_lstm(xs[:Ts, :Bs].cpu().numpy(), WU[:Ls].cpu().numpy(), None, None)
+        dt = time.perf_counter() - t0
+        full_seconds = dt * (L * T * B) / (Ls * Ts * Bs)
+        res['cpu_baseline'] = {'value': B / full_seconds, 'unit': 'sequences/s', 'cores': 1, 'kind': 'port',
+                               'sample': f'{Ls} layers x {Ts} steps x {Bs} rows through oracle/oracle.c in {dt:.1f} s, '
+                                         f'scaled by cell-rows to the full configuration'}
+    return res
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument('--gpus', type=int, default=1)
     ap.add_argument('--steps', type=int, default=50)
     ap.add_argument('--warmup', type=int, default=10)
-    ap.add_argument('--workload', default='b2b', choices=['b2b', 'attention', 'stacked_lstm', 'dilated_lstm', 'lstm_f16_h256', 'lstm_f16_h512', 'lstm_f16_h1024', 'embedding', 'copy'])
+    ap.add_argument('--workload', default='b2b', choices=['b2b', 'attention', 'stacked_lstm', 'dilated_lstm', 'lstm_f16_h256', 'lstm_f16_h512', 'lstm_f16_h1024', 'lstm_f32_h512', 'lstm_f32_h1024', 'embedding', 'copy'])
     ap.add_argument('--no-extras', action='store_true', help='measure only the chosen workload')
     ap.add_argument('--no-cpu', action='store_true', help='skip the CPU baseline leg')
     ap.add_argument('--no-baselines', action='store_true',
@@ -430,6 +477,8 @@ def main():
         'lstm_f16_h256': lambda s, w, c: bench_lstm_f16(torch, core, max(3, s // 5), max(1, w // 5), c, 256, not args.no_baselines),
         'lstm_f16_h512': lambda s, w, c: bench_lstm_f16(torch, core, max(3, s // 5), max(1, w // 5), c, 512, not args.no_baselines),
         'lstm_f16_h1024': lambda s, w, c: bench_lstm_f16(torch, core, max(3, s // 5), max(1, w // 5), c, 1024, not args.no_baselines),
+        'lstm_f32_h512': lambda s, w, c: bench_lstm_f32_streamed(torch, core, max(3, s // 5), max(1, w // 5), c, 512),
+        'lstm_f32_h1024': lambda s, w, c: bench_lstm_f32_streamed(torch, core, max(3, s // 10), 1, c, 1024),
         'embedding': lambda s, w, c: bench_embedding(torch, core, s, w, c),
     }
     if args.workload == 'copy':
