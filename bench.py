@@ -348,8 +348,8 @@ def bench_lstm_f16(torch, core, steps, warmup, cpu, H, baselines=True):
                      'kernel': 'lstm_persistent_kernel<2>' if H == 512 else 'lstm_persistent_kernel<3>'},
     }
     if not on_chip and H == 512:
-        res['roofline']['kernel'] = 'lstm_cell_f16_kernel<true, 8>'
-        res['roofline']['traffic'] = None
+        res['roofline']['kernel'] = 'lstm_cell_f16_kernel<true, 8, false>'
+        res['roofline']['traffic'] = MEASURED_TRAFFIC_BYTES.get('lstm_cell_f16_kernel_h512_per_pass')
         res['config']['schedule'] = 'one launch of the streaming fp16 cell kernel per stage of independent cells'
     if not on_chip and H > 512:
         # every cell streams its layer's weights once (the stack's weights exceed the 256 MB of last-level cache), reads its
@@ -359,7 +359,7 @@ def bench_lstm_f16(torch, core, steps, warmup, cpu, H, baselines=True):
         res['roofline'] = {'bound': 'hbm', 'achieved': (wbytes + abytes) / ms / 1e6, 'peak': PEAK_HBM_GBS, 'unit': 'GB/s',
                            'frac': (wbytes + abytes) / ms / 1e6 / PEAK_HBM_GBS,
                            'traffic': MEASURED_TRAFFIC_BYTES.get('lstm_cell_f16_kernel_per_pass'),
-                           'kernel': 'lstm_cell_f16_kernel<true, 8>',
+                           'kernel': 'lstm_cell_f16_kernel<true, 8, false>',
                            'note': 'per launch: the cells of one stage; bytes = weights of every cell once + activations'}
         res['config']['schedule'] = 'one launch of the streaming fp16 cell kernel per stage of independent cells'
     if baselines:
@@ -429,7 +429,8 @@ def bench_lstm_f32_streamed(torch, core, steps, warmup, cpu, H):
         'tflops': flop / ms / 1e9, 'frac_of_f32_matrix_peak_algorithmic': flop / ms / 1e9 / PEAK_F32_MATRIX_TFLOPS,
         'fp32_mfma_products': {'ms_per_step': ms32, 'speedup_of_split_products': ms32 / ms, 'max_rel_diff': diff},
         'roofline': {'bound': 'mfma', 'achieved': 3 * flop / ms / 1e9, 'peak': PEAK_F16_TFLOPS, 'unit': 'TFLOP/s',
-                     'frac': 3 * flop / ms / 1e9 / PEAK_F16_TFLOPS, 'traffic': None, 'kernel': 'lstm_cell_split4_kernel',
+                     'frac': 3 * flop / ms / 1e9 / PEAK_F16_TFLOPS,
+                     'traffic': MEASURED_TRAFFIC_BYTES.get(f'lstm_cell_split4_kernel_h{H}_per_pass'), 'kernel': 'lstm_cell_split4_kernel',
                      'note': 'executed f16 MFMA flops (three per algorithmic product) against the f16 MFMA peak'},
     }
     if cpu:
