@@ -18,7 +18,7 @@ LIB_PATH = os.path.join(_HERE, 'libftkernels.so')
 # every symbol include/ftk.h declares; checked at load time
 EXPORTS = (
     'ftk_version', 'ftk_last_error', 'ftk_device_info_query',
-    'ftk_lstm_cell_f32', 'ftk_lstm_cell_f16', 'ftk_lstm_elementwise_f32',
+    'ftk_lstm_cell_f32', 'ftk_lstm_cell_f16', 'ftk_lstm_layer_f32', 'ftk_lstm_layer_f16', 'ftk_lstm_elementwise_f32',
     'ftk_stacked_lstm_workspace_bytes', 'ftk_stacked_lstm_f32', 'ftk_dilated_lstm_f32',
     'ftk_stacked_lstm_wavefront_f32', 'ftk_stacked_lstm_ragged_f32', 'ftk_lstm_set_products', 'ftk_lstm_get_products',
     'ftk_stacked_lstm_f16_workspace_bytes', 'ftk_stacked_lstm_f16',
@@ -118,6 +118,30 @@ def lstm_cell(x, h_prev, c_prev, WU, bias=None) -> Tuple[torch.Tensor, torch.Ten
     _check(lib.ftk_lstm_cell_f32(_ptr(x), _ptr(h_prev), _ptr(c_prev), _ptr(WU), _ptr(bias), _ptr(h), _ptr(c),
                                  ctypes.c_int(B), ctypes.c_int(I), ctypes.c_int(H), _stream()))
     return h, c
+
+
+def lstm_layer(xs, WU, bias=None, h0=None, c0=None) -> Tuple[torch.Tensor, torch.Tensor]:
+    """One layer over T steps from an initial state: xs [T,B,I], WU [(I+H),4H], bias [4H] or None, h0/c0 [B,H] or
+    None (zero state) -> hs, cs [T,B,H].  fp32 throughout, or fp16 storage (bias fp32) when xs is fp16."""
+    dt = xs.dtype
+    if dt not in (torch.float32, torch.float16):
+        raise TypeError('xs must be float32 or float16')
+    _req(xs, dt, 'xs'); _req(WU, dt, 'WU')
+    T, B, I = xs.shape
+    H = WU.shape[1] // 4
+    if WU.shape != (I + H, 4 * H):
+        raise ValueError(f'WU must be [(I+H), 4H] = [{I + H}, {4 * H}], got {tuple(WU.shape)}')
+    for t, n in ((h0, 'h0'), (c0, 'c0')):
+        if t is not None and _req(t, dt, n).shape != (B, H):
+            raise ValueError(f'{n} must be [{B}, {H}]')
+    if bias is not None and _req(bias, torch.float32, 'bias').numel() != 4 * H:
+        raise ValueError('bias must have 4H elements')
+    hs = torch.empty((T, B, H), dtype=dt, device=xs.device)
+    cs = torch.empty((T, B, H), dtype=dt, device=xs.device)
+    fn = lib.ftk_lstm_layer_f32 if dt == torch.float32 else lib.ftk_lstm_layer_f16
+    ci = ctypes.c_int
+    _check(fn(_ptr(xs), _ptr(WU), _ptr(bias), _ptr(h0), _ptr(c0), _ptr(hs), _ptr(cs), ci(T), ci(B), ci(I), ci(H), _stream()))
+    return hs, cs
 
 
 def lstm_cell_f16(x, h_prev, c_prev, WU, bias=None) -> Tuple[torch.Tensor, torch.Tensor]:

@@ -1089,6 +1089,53 @@ int ftk_lstm_cell_f16(const void* x, const void* h_prev, const void* c_prev, con
   return ftk::launch_cells(list, B, I, H, (hipStream_t)stream);
 }
 
+int ftk_lstm_layer_f32(const float* xs, const float* WU, const float* bias, const float* h0, const float* c0, float* hs,
+                       float* cs, int T, int B, int I, int H, ftk_stream_t stream) {
+  const char* who = "ftk_lstm_layer_f32";
+  if (!xs || !WU || !hs || !cs) return ftk::fail(FTK_ERR_INVALID_ARGUMENT, "%s: xs, WU, hs, cs must be non-NULL", who);
+  if ((h0 == nullptr) != (c0 == nullptr))
+    return ftk::fail(FTK_ERR_INVALID_ARGUMENT, "%s: h0 and c0 must both be given or both be NULL", who);
+  if (T <= 0 || B <= 0 || I <= 0 || H <= 0) return ftk::fail(FTK_ERR_INVALID_ARGUMENT, "%s: T, B, I, H must be positive", who);
+  if (I % 32 || H % 32) return ftk::fail(FTK_ERR_UNSUPPORTED_SHAPE, "%s: I=%d and H=%d must be multiples of 32", who, I, H);
+  if ((B + 31) / 32 > 65535) return ftk::fail(FTK_ERR_UNSUPPORTED_SHAPE, "%s: B=%d too large", who, B);
+  const size_t cell = (size_t)B * H;
+  for (int t = 0; t < T; ++t) {  // one fused-cell launch per step, stream-ordered
+    ftk::CellList list;
+    list.n = 1;
+    list.cells[0] = ftk::CellDesc{xs + (size_t)t * B * I, t ? hs + (t - 1) * cell : h0, t ? cs + (t - 1) * cell : c0,
+                                  WU,  bias, hs + t * cell, cs + t * cell};
+    int rc = ftk::launch_cells(list, B, I, H, (hipStream_t)stream);
+    if (rc) return rc;
+  }
+  return FTK_OK;
+}
+
+int ftk_lstm_layer_f16(const void* xs, const void* WU, const float* bias, const void* h0, const void* c0, void* hs,
+                       void* cs, int T, int B, int I, int H, ftk_stream_t stream) {
+  const char* who = "ftk_lstm_layer_f16";
+  if (!xs || !WU || !hs || !cs) return ftk::fail(FTK_ERR_INVALID_ARGUMENT, "%s: xs, WU, hs, cs must be non-NULL", who);
+  if ((h0 == nullptr) != (c0 == nullptr))
+    return ftk::fail(FTK_ERR_INVALID_ARGUMENT, "%s: h0 and c0 must both be given or both be NULL", who);
+  if (T <= 0 || B <= 0 || I <= 0 || H <= 0) return ftk::fail(FTK_ERR_INVALID_ARGUMENT, "%s: T, B, I, H must be positive", who);
+  if (I % 32 || H % 32) return ftk::fail(FTK_ERR_UNSUPPORTED_SHAPE, "%s: I=%d and H=%d must be multiples of 32", who, I, H);
+  if ((long long)B * std::max(I, H) >= (1ll << 30)) return ftk::fail(FTK_ERR_UNSUPPORTED_SHAPE, "%s: B=%d too large", who, B);
+  const _Float16* x16 = (const _Float16*)xs;
+  _Float16* h16 = (_Float16*)hs;
+  _Float16* c16 = (_Float16*)cs;
+  const size_t cell = (size_t)B * H;
+  for (int t = 0; t < T; ++t) {
+    ftk::CellListH list;
+    list.n = 1;
+    list.packed = 0;
+    list.cells[0] = ftk::CellDescH{x16 + (size_t)t * B * I, t ? h16 + (t - 1) * cell : (const _Float16*)h0,
+                                   t ? (const void*)(c16 + (t - 1) * cell) : c0, (const _Float16*)WU, bias, h16 + t * cell,
+                                   c16 + t * cell, nullptr, nullptr, nullptr};
+    int rc = ftk::launch_cells(list, B, I, H, (hipStream_t)stream);
+    if (rc) return rc;
+  }
+  return FTK_OK;
+}
+
 int ftk_lstm_elementwise_f32(const float* gates, const float* bias, const float* c_prev, float* h, float* c, int B,
                              int H, ftk_stream_t stream) {
   if (!gates || !h || !c) return ftk::fail(FTK_ERR_INVALID_ARGUMENT, "ftk_lstm_elementwise_f32: gates, h, c must be non-NULL");

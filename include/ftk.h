@@ -90,6 +90,23 @@ int ftk_lstm_cell_f16(const void* x, const void* h_prev, const void* c_prev,
                       int B, int I, int H, ftk_stream_t stream);
 
 /*
+ * One LSTM layer over T steps from a given initial state: step t is the cell
+ * above on xs[t] and the state of step t-1 (h0, c0 for t = 0; both NULL = zero
+ * state).  xs [T,B,I], WU [(I+H),4H], bias [4H] or NULL, h0/c0 [B,H],
+ * outputs hs/cs [T,B,H].  One fused-cell launch per step on the stream.
+ * _f32: all fp32; _f16: xs, WU, h0, c0, hs, cs fp16, bias fp32.
+ * Needs I%32==0, H%32==0.  Replaces CuteLSTMLayer::operator()(w, xs, u, c_init,
+ * h_init, csss, hsss, seq_length) (kaleido/core/device/kernels/lstm.h:479-602)
+ * and the Python lstm_layer (examples/stacked_rnn/stacked_rnn.py:54-65).
+ */
+int ftk_lstm_layer_f32(const float* xs, const float* WU, const float* bias,
+                       const float* h0, const float* c0, float* hs, float* cs,
+                       int T, int B, int I, int H, ftk_stream_t stream);
+int ftk_lstm_layer_f16(const void* xs, const void* WU, const float* bias,
+                       const void* h0, const void* c0, void* hs, void* cs,
+                       int T, int B, int I, int H, ftk_stream_t stream);
+
+/*
  * The state-update half alone, for the unfused baseline: gates [B,4H] already
  * holds x@W + h@U (pre-activation, blocks i|f|o|c~); bias [4H] or NULL;
  * c_prev [B,H] or NULL.  Replaces ElementwiseLstmAct

@@ -47,6 +47,9 @@ def test_argument_errors_come_back_as_codes_not_crashes():
     assert lib.ftk_embedding_gather_f32(one, nul, ci(0), one, ctypes.c_longlong(4), ci(8), ci(8), nul, nul) == -1
     assert lib.ftk_stacked_lstm_ragged_f32(one, one, nul, nul, nul, one, one, ci(1), ci(1), ci(1), ci(32), nul, ctypes.c_size_t(0), nul) == -1
     assert lib.ftk_lstm_cell_f16(one, nul, nul, one, nul, one, one, ci(4), ci(48), ci(64), nul) == -2
+    assert lib.ftk_lstm_layer_f32(one, one, nul, one, nul, one, one, ci(2), ci(4), ci(32), ci(32), nul) == -1
+    assert lib.ftk_lstm_layer_f16(one, one, nul, nul, nul, one, one, ci(2), ci(4), ci(32), ci(40), nul) == -2
+    assert lib.ftk_lstm_layer_f32(one, one, nul, nul, nul, one, one, ci(0), ci(4), ci(32), ci(32), nul) == -1
     assert lib.ftk_lstm_cell_f16(one, one, nul, one, nul, one, one, ci(4), ci(64), ci(64), nul) == -1
     assert lib.ftk_stacked_lstm_f16(one, one, nul, nul, nul, one, one, ci(1), ci(1), ci(4), ci(80), nul, ctypes.c_size_t(0), nul) == -2
     # a shape whose weights are streamed needs the workspace for their re-laid copy

@@ -100,6 +100,35 @@ def test_lstm_elementwise(core):
     assert_lstm_close(h, hr, 'h'); assert_lstm_close(c, cr, 'c')
 
 
+@pytest.mark.parametrize('T,B,I,H,state', [(5, 40, 64, 96, True), (3, 33, 256, 256, False), (4, 8, 32, 64, True)])
+def test_lstm_layer_from_an_initial_state(core, T, B, I, H, state):
+    rng = np.random.default_rng(3)
+    xs = rng.standard_normal((T, B, I)).astype(np.float32)
+    WU = rng.uniform(-0.1, 0.1, (I + H, 4 * H)).astype(np.float32)
+    b = rng.uniform(-0.1, 0.1, 4 * H).astype(np.float32)
+    h0 = rng.uniform(-1, 1, (B, H)).astype(np.float32) if state else None
+    c0 = rng.standard_normal((B, H)).astype(np.float32) if state else None
+    hs, cs = core.lstm_layer(dev(xs), dev(WU), dev(b), None if h0 is None else dev(h0), None if c0 is None else dev(c0))
+    hr, cr = ko.lstm_layer(xs, WU, b, h0, c0)
+    assert_lstm_close(hs, hr, 'hs'); assert_lstm_close(cs, cr, 'cs')
+    # fp16 storage: the float64 cell on explicitly rounded states
+    x16, W16 = xs.astype(np.float16), WU.astype(np.float16)
+    h16 = None if h0 is None else h0.astype(np.float16)
+    c16 = None if c0 is None else c0.astype(np.float16)
+    hs16, cs16 = core.lstm_layer(dev(x16), dev(W16), dev(b), None if h16 is None else dev(h16), None if c16 is None else dev(c16))
+    hp = np.zeros((B, H)) if h16 is None else h16.astype(np.float64)
+    cp = np.zeros((B, H)) if c16 is None else c16.astype(np.float64)
+    for t in range(T):
+        h, c = ko.lstm_cell(x16[t].astype(np.float64), hp, cp, W16.astype(np.float64), b.astype(np.float64))
+        hp, cp = h.astype(np.float16).astype(np.float64), c.astype(np.float16).astype(np.float64)
+        eh = ko.max_rel_err(hs16[t].float().cpu().numpy(), hp.astype(np.float32))
+        ec = ko.max_rel_err(cs16[t].float().cpu().numpy(), cp.astype(np.float32))
+        assert eh <= F16_TOL and ec <= F16_TOL, (t, eh, ec)
+    with pytest.raises(core.FtkError) as e:
+        core.lstm_layer(dev(xs), dev(WU), dev(b), dev(np.zeros((B, H), np.float32)), None)
+    assert e.value.code == -1 and 'h0 and c0' in str(e.value)
+
+
 # ------------------------------------------------------- stacked / dilated LSTM
 
 @pytest.mark.parametrize('L,T,B,H,dil', [
