@@ -22,7 +22,7 @@ EXPORTS = (
     'ftk_stacked_lstm_workspace_bytes', 'ftk_stacked_lstm_f32', 'ftk_dilated_lstm_f32',
     'ftk_stacked_lstm_wavefront_f32', 'ftk_stacked_lstm_ragged_f32', 'ftk_lstm_set_products', 'ftk_lstm_get_products',
     'ftk_stacked_lstm_f16_workspace_bytes', 'ftk_stacked_lstm_f16',
-    'ftk_b2b_gemm_f16', 'ftk_flash_attn_f16', 'ftk_online_softmax_f32', 'ftk_embedding_gather_f32',
+    'ftk_b2b_gemm_f16', 'ftk_b2b_gemm_rowmajor_f16', 'ftk_flash_attn_f16', 'ftk_online_softmax_f32', 'ftk_embedding_gather_f32',
     'ftk_debug_read_fa_trace',
 )
 
@@ -330,6 +330,31 @@ def b2b_gemm(A, B_nk, C_pn, out: Optional[torch.Tensor] = None) -> torch.Tensor:
     _req(D, f16, 'D')
     ci = ctypes.c_int
     _check(lib.ftk_b2b_gemm_f16(_ptr(A), _ptr(B_nk), _ptr(C_pn), _ptr(D), ci(G), ci(M), ci(N), ci(K), ci(P), _stream()))
+    return D[0] if squeeze and out is None else D
+
+
+def b2b_gemm_rowmajor_supported(N: int, K: int, P: int) -> bool:
+    """Shapes ftk_b2b_gemm_rowmajor_f16 is built for."""
+    return K in (64, 128) and N in (64, 128) and P % 128 == 0
+
+
+def b2b_gemm_rowmajor(A, B, C, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """D = (A @ B) @ C with every operand row-major: A [G,M,K], B [G,K,N], C [G,N,P], D [G,M,P]; fp16.
+    K and N in {64, 128}, P a multiple of 128."""
+    f16 = torch.float16
+    _req(A, f16, 'A'); _req(B, f16, 'B'); _req(C, f16, 'C')
+    squeeze = A.dim() == 2
+    if squeeze:
+        A, B, C = A[None], B[None], C[None]
+    G, M, K = A.shape
+    N = B.shape[2]
+    P = C.shape[2]
+    if B.shape != (G, K, N) or C.shape != (G, N, P):
+        raise ValueError(f'shape mismatch: A {tuple(A.shape)}, B {tuple(B.shape)}, C {tuple(C.shape)}')
+    D = out if out is not None else torch.empty((G, M, P), dtype=f16, device=A.device)
+    _req(D, f16, 'D')
+    ci = ctypes.c_int
+    _check(lib.ftk_b2b_gemm_rowmajor_f16(_ptr(A), _ptr(B), _ptr(C), _ptr(D), ci(G), ci(M), ci(N), ci(K), ci(P), _stream()))
     return D[0] if squeeze and out is None else D
 
 

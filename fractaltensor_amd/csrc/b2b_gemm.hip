@@ -36,6 +36,9 @@ namespace ftk {
 
 constexpr int B2B_PTILE = 128;  // p columns per workgroup
 
+typedef short v4s __attribute__((ext_vector_type(4)));
+typedef short v8s __attribute__((ext_vector_type(8)));
+
 __device__ __forceinline__ v4u ldg16(const void* p) { return *reinterpret_cast<const v4u*>(p); }
 
 struct B2BGrid {
@@ -265,7 +268,12 @@ __global__ __launch_bounds__(256) void b2b_gemm_kernel(const _Float16* __restric
 // left when the last rows arrive, and two waves per SIMD cover each other's LDS
 // round trips, conversions and D stores.  The wave-private LDS region is used
 // twice per unit: A rows on the way in, D rows on the way out.
-template <int KS, int PT, int NT>
+//
+// ROWMAJOR: B is given as [K, N] and C as [N, P], row-major, the layout of an operator program's (a @ b) @ c.
+// Both are staged as they are (rows padded by 64 bytes) and the weight-side MFMA operands, which want 8
+// consecutive k (or n) per lane, are read with ds_read_b64_tr_b16: 16 lanes hand in a 4-row x 16-column block
+// and lane i receives column i of the four rows, so nothing is transposed on the way in.
+template <int KS, int PT, int NT, bool ROWMAJOR>
 __global__ __launch_bounds__(512) void b2b_gemm8_kernel(const _Float16* __restrict__ A,
                                                         const _Float16* __restrict__ Bm,
                                                         const _Float16* __restrict__ Cm, _Float16* __restrict__ D,
@@ -274,6 +282,9 @@ __global__ __launch_bounds__(512) void b2b_gemm8_kernel(const _Float16* __restri
   constexpr int N = 32 * NT;
   constexpr int BLD = K + 8;   // padded Bs / A-staging row (halfs)
   constexpr int CLD = N + 4;   // padded Cs row (halfs)
+  constexpr int BRS = N + 32;       // ROWMAJOR: Bs[k][n] row (halfs), 64 bytes of padding
+  constexpr int CRS = 32 * PT + 32;  // ROWMAJOR: Cs[n][p] row
+  using lds_v4s = __attribute__((address_space(3))) v4s;
   constexpr int AN = KS;       // 16-byte A loads per lane for 32 rows
   constexpr int pw = 32 * PT;  // p columns handled here
   constexpr int PG = (PT + 1) / 2;  // column groups of up to 64
@@ -295,13 +306,13 @@ __global__ __launch_bounds__(512) void b2b_gemm8_kernel(const _Float16* __restri
   const int g = id / (gr.per_problem * gr.ptiles);
   const int p0 = p_base + pt_idx * pw;
 
-  _Float16* Bs = reinterpret_cast<_Float16*>(smem);        // [N][BLD]
-  _Float16* Cs = Bs + N * BLD;                             // [pw][CLD]
-  _Float16* Wr = Cs + pw * CLD + wave * gr.wave_region;    // wave-private: [32][BLD] A rows, then [32][DLD] D rows
+  _Float16* Bs = reinterpret_cast<_Float16*>(smem);        // [N][BLD], ROWMAJOR: [K][BRS]
+  _Float16* Cs = Bs + (ROWMAJOR ? K * BRS : N * BLD);      // [pw][CLD], ROWMAJOR: [N][CRS]
+  _Float16* Wr = Cs + (ROWMAJOR ? N * CRS : pw * CLD) + wave * gr.wave_region;  // wave-private: [32][BLD] A rows, then [32][DLD] D rows
 
   const _Float16* Ag = A + (size_t)g * M * K;
   const _Float16* Bg = Bm + (size_t)g * N * K;
-  const _Float16* Cg = Cm + (size_t)g * P * N + (size_t)p0 * N;
+  const _Float16* Cg = Cm + (size_t)g * P * N + (ROWMAJOR ? (size_t)p0 : (size_t)p0 * N);
   _Float16* Dg = D + (size_t)g * M * P + p0;
 
   // consecutive units of a workgroup go to consecutive waves: wave w takes units w, w + 8, ... of the
@@ -335,7 +346,10 @@ __global__ __launch_bounds__(512) void b2b_gemm8_kernel(const _Float16* __restri
 #pragma unroll
     for (int u = 0; u < UC; ++u) {
       const int idx = u * threads + tid;
-      if (idx < ncq) vc[u] = ldg16(Cg + (size_t)idx * 8);
+      if (idx < ncq) {
+        if constexpr (ROWMAJOR) vc[u] = ldg16(Cg + (size_t)(idx / (pw / 8)) * P + 8 * (idx % (pw / 8)));  // row n, 8 columns of the p tile
+        else vc[u] = ldg16(Cg + (size_t)idx * 8);
+      }
     }
     // Requests are served roughly in the order the CU's memory pipeline accepted them.  The barrier
     // puts every wave's share of B and C (which everything waits for) ahead of any A row; then one
@@ -347,16 +361,23 @@ __global__ __launch_bounds__(512) void b2b_gemm8_kernel(const _Float16* __restri
 #pragma unroll
     for (int u = 0; u < UB; ++u) {
       const int idx = u * threads + tid;
-      if (idx < nb) *reinterpret_cast<v4u*>(Bs + (idx / CPR) * BLD + 8 * (idx % CPR)) = vb[u];
+      if (idx < nb) {
+        if constexpr (ROWMAJOR) *reinterpret_cast<v4u*>(Bs + (idx / (N / 8)) * BRS + 8 * (idx % (N / 8))) = vb[u];
+        else *reinterpret_cast<v4u*>(Bs + (idx / CPR) * BLD + 8 * (idx % CPR)) = vb[u];
+      }
     }
 #pragma unroll
     for (int u = 0; u < UC; ++u) {
       const int idx = u * threads + tid;
       if (idx < ncq) {
-        const int p = idx / (N / 8), n8 = idx % (N / 8);
-        // CLD is not a multiple of 8 halfs: two 8-byte pieces
-        *reinterpret_cast<v2u*>(Cs + p * CLD + 8 * n8) = v2u{vc[u][0], vc[u][1]};
-        *reinterpret_cast<v2u*>(Cs + p * CLD + 8 * n8 + 4) = v2u{vc[u][2], vc[u][3]};
+        if constexpr (ROWMAJOR) {
+          *reinterpret_cast<v4u*>(Cs + (idx / (pw / 8)) * CRS + 8 * (idx % (pw / 8))) = vc[u];
+        } else {
+          const int p = idx / (N / 8), n8 = idx % (N / 8);
+          // CLD is not a multiple of 8 halfs: two 8-byte pieces
+          *reinterpret_cast<v2u*>(Cs + p * CLD + 8 * n8) = v2u{vc[u][0], vc[u][1]};
+          *reinterpret_cast<v2u*>(Cs + p * CLD + 8 * n8 + 4) = v2u{vc[u][2], vc[u][3]};
+        }
       }
     }
   }
@@ -388,11 +409,23 @@ __global__ __launch_bounds__(512) void b2b_gemm8_kernel(const _Float16* __restri
 #pragma unroll
         for (int r = 0; r < 16; ++r) pacc[nt][r] = 0.0f;
       const _Float16* brow = Bs + j * BLD + hh * (K / 2);
+      // ROWMAJOR: the lane's block of the transposing read: rows k = hh*K/2 + 8s + (a | a + 4), columns 4b.. of
+      // the 16-column half th of the n tile
+      const _Float16* btr = Bs + (hh * (K / 2) + ((lane & 15) >> 2)) * BRS + 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
 #pragma unroll
       for (int s = 0; s < KS; ++s)
 #pragma unroll
         for (int nt = 0; nt < NT; ++nt) {
-          const v8h bfrag = *reinterpret_cast<const v8h*>(brow + nt * 32 * BLD + 8 * s);
+          v8h bfrag;
+          if constexpr (ROWMAJOR) {
+            const _Float16* p0 = btr + 8 * s * BRS + 32 * nt;
+            const v4s lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4s*)(p0));
+            const v4s hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4s*)(p0 + 4 * BRS));
+            const v8s both = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+            bfrag = __builtin_bit_cast(v8h, both);
+          } else {
+            bfrag = *reinterpret_cast<const v8h*>(brow + nt * 32 * BLD + 8 * s);
+          }
           pacc[nt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(bfrag, afrag[s], pacc[nt], 0, 0, 0);
         }
 #pragma unroll
@@ -417,11 +450,22 @@ __global__ __launch_bounds__(512) void b2b_gemm8_kernel(const _Float16* __restri
 #pragma unroll
         for (int q = 0; q < PW; ++q) {
           const _Float16* crow = Cs + ((2 * pg + q) * 32 + j) * CLD + nt * 32 + 4 * hh;
+          // ROWMAJOR: rows n = 32 nt + 16 s + 4 hh + a (and + 8), columns of p tile 2 pg + q
+          const _Float16* ctr = Cs + (nt * 32 + 4 * hh + ((lane & 15) >> 2)) * CRS + (2 * pg + q) * 32 +
+                                16 * ((lane >> 4) & 1) + 4 * (lane & 3);
 #pragma unroll
           for (int s = 0; s < 2; ++s) {
-            const v4h c0 = *reinterpret_cast<const v4h*>(crow + 16 * s);
-            const v4h c1 = *reinterpret_cast<const v4h*>(crow + 16 * s + 8);
-            const v8h cfrag = {c0[0], c0[1], c0[2], c0[3], c1[0], c1[1], c1[2], c1[3]};
+            v8h cfrag;
+            if constexpr (ROWMAJOR) {
+              const v4s lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4s*)(ctr + 16 * s * CRS));
+              const v4s hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4s*)(ctr + (16 * s + 8) * CRS));
+              const v8s both = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+              cfrag = __builtin_bit_cast(v8h, both);
+            } else {
+              const v4h c0 = *reinterpret_cast<const v4h*>(crow + 16 * s);
+              const v4h c1 = *reinterpret_cast<const v4h*>(crow + 16 * s + 8);
+              cfrag = v8h{c0[0], c0[1], c0[2], c0[3], c1[0], c1[1], c1[2], c1[3]};
+            }
             dacc[q] = __builtin_amdgcn_mfma_f32_32x32x16_f16(cfrag, pf[nt][s], dacc[q], 0, 0, 0);
           }
         }
@@ -457,14 +501,14 @@ __global__ __launch_bounds__(512) void b2b_gemm8_kernel(const _Float16* __restri
   }
 }
 
-template <int KS, int PT, int NT>
+template <int KS, int PT, int NT, bool ROWMAJOR = false>
 static int launch_b2b8(const void* A, const void* B, const void* C, void* D, int G, int M, int P, int p_base,
                        int ptiles, int cus, int lds_max, bool* handled, hipStream_t s) {
   constexpr int K = 16 * KS, N = 32 * NT, pw = 32 * PT, waves = 8;
   B2BGrid gr;
   gr.ptiles = ptiles;
   gr.wave_region = std::max(32 * (K + 8), 32 * (64 + 4));
-  const size_t lds = (size_t)(N * (K + 8) + pw * (N + 4) + waves * gr.wave_region) * 2;
+  const size_t lds = (size_t)((ROWMAJOR ? K * (N + 32) + N * (pw + 32) : N * (K + 8) + pw * (N + 4)) + waves * gr.wave_region) * 2;
   *handled = (int)lds <= lds_max;
   if (!*handled) return FTK_OK;
   const int row_units = (M + 31) / 32;
@@ -477,11 +521,11 @@ static int launch_b2b8(const void* A, const void* B, const void* C, void* D, int
   gr.total = (int)total;
   static bool attr_set = false;
   if (!attr_set) {
-    FTK_HIP(hipFuncSetAttribute((const void*)b2b_gemm8_kernel<KS, PT, NT>, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                (int)lds));
+    FTK_HIP(hipFuncSetAttribute((const void*)b2b_gemm8_kernel<KS, PT, NT, ROWMAJOR>,
+                                hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
     attr_set = true;
   }
-  hipLaunchKernelGGL((b2b_gemm8_kernel<KS, PT, NT>), dim3(gr.total), dim3(waves * 64), lds, s, (const _Float16*)A,
+  hipLaunchKernelGGL((b2b_gemm8_kernel<KS, PT, NT, ROWMAJOR>), dim3(gr.total), dim3(waves * 64), lds, s, (const _Float16*)A,
                      (const _Float16*)B, (const _Float16*)C, (_Float16*)D, M, P, p_base, gr);
   return check_launch("b2b_gemm8_kernel");
 }
@@ -576,4 +620,29 @@ extern "C" int ftk_b2b_gemm_f16(const void* A, const void* B, const void* C, voi
     case 96: return launch_b2b<6>(A, B, C, D, G, M, N, P, dp->cus, dp->lds_optin, s);
     default: return launch_b2b<8>(A, B, C, D, G, M, N, P, dp->cus, dp->lds_optin, s);
   }
+}
+
+extern "C" int ftk_b2b_gemm_rowmajor_f16(const void* A, const void* B, const void* C, void* D, int G, int M, int N,
+                                         int K, int P, ftk_stream_t stream) {
+  using namespace ftk;
+  const char* who = "ftk_b2b_gemm_rowmajor_f16";
+  if (!A || !B || !C || !D) return fail(FTK_ERR_INVALID_ARGUMENT, "%s: A, B, C, D must be non-NULL", who);
+  if (G <= 0 || M <= 0 || N <= 0 || K <= 0 || P <= 0)
+    return fail(FTK_ERR_INVALID_ARGUMENT, "%s: G, M, N, K, P must be positive", who);
+  if ((K != 64 && K != 128) || (N != 64 && N != 128) || P % 128)
+    return fail(FTK_ERR_UNSUPPORTED_SHAPE, "%s: built for K and N in {64, 128} and P a multiple of 128, got K=%d N=%d P=%d", who,
+                K, N, P);
+  const DeviceProps* dp = nullptr;
+  int rc = device_props(&dp);
+  if (rc) return rc;
+  hipStream_t s = (hipStream_t)stream;
+  bool handled = false;
+  const int full = P / B2B_PTILE;
+  if (K == 64 && N == 64) rc = launch_b2b8<4, 4, 2, true>(A, B, C, D, G, M, P, 0, full, dp->cus, dp->lds_optin, &handled, s);
+  else if (K == 64) rc = launch_b2b8<4, 4, 4, true>(A, B, C, D, G, M, P, 0, full, dp->cus, dp->lds_optin, &handled, s);
+  else if (N == 64) rc = launch_b2b8<8, 4, 2, true>(A, B, C, D, G, M, P, 0, full, dp->cus, dp->lds_optin, &handled, s);
+  else rc = launch_b2b8<8, 4, 4, true>(A, B, C, D, G, M, P, 0, full, dp->cus, dp->lds_optin, &handled, s);
+  if (rc) return rc;
+  if (!handled) return fail(FTK_ERR_DEVICE, "%s: the device's LDS does not hold the B and C tiles", who);
+  return FTK_OK;
 }

@@ -202,9 +202,14 @@ def b2b_gemm(a, b, c):
 
     A, Bm, Cm = dense(a, 'a'), dense(b, 'b'), dense(c, 'c')
     in_dtype = A.dtype
-    # the kernel takes B and C with the contraction index contiguous
-    D = core.b2b_gemm(A.half().contiguous(), Bm.half().transpose(1, 2).contiguous(),
-                      Cm.half().transpose(1, 2).contiguous()).to(in_dtype)
+    K_, N_, P_ = A.shape[2], Bm.shape[2], Cm.shape[2]
+    if core.b2b_gemm_rowmajor_supported(N_, K_, P_):
+        # b and c as they are: the kernel transposes them between LDS and the matrix unit
+        D = core.b2b_gemm_rowmajor(A.half().contiguous(), Bm.half().contiguous(), Cm.half().contiguous()).to(in_dtype)
+    else:
+        # the general kernel takes B and C with the contraction index contiguous
+        D = core.b2b_gemm(A.half().contiguous(), Bm.half().transpose(1, 2).contiguous(),
+                          Cm.half().transpose(1, 2).contiguous()).to(in_dtype)
     if isinstance(a, Tensor):
         return Tensor.from_tensor(D[0])
     return FractalTensor.from_dense(D, 1)

@@ -264,6 +264,20 @@ int ftk_embedding_gather_f32(const float* table, const void* ids,
 int ftk_b2b_gemm_f16(const void* A, const void* B, const void* C, void* D,
                      int G, int M, int N, int K, int P, ftk_stream_t stream);
 
+/*
+ * The same product with every operand row-major, the layout an operator
+ * program's (a @ b) @ c has: A [G,M,K], B [G,K,N], C [G,N,P], D [G,M,P].
+ * B and C are staged as they are and transposed on the way from LDS to the
+ * matrix unit.  Built for the shapes of the eight-wave kernel: K and N in
+ * {64, 128}, P%128==0 (anything else: FTK_ERR_UNSUPPORTED_SHAPE; transpose B
+ * and C once and call ftk_b2b_gemm_f16).  No counterpart in the reference,
+ * whose B2BGemm takes column-major B and C only (gemm_kernel_traits.h:261-267);
+ * it is what kaleido's `(a @ b) @ c` (Tensor.__matmul__, tensor.py:110-116) maps to.
+ */
+int ftk_b2b_gemm_rowmajor_f16(const void* A, const void* B, const void* C,
+                              void* D, int G, int M, int N, int K, int P,
+                              ftk_stream_t stream);
+
 /* ------------------------------------------------------ flash attention -- */
 
 /*

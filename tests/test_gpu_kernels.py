@@ -466,6 +466,37 @@ def b2b_inputs(seed, G, M, N, K, P):
 
 
 @pytest.mark.parametrize('G,M,N,K,P', [
+    (32, 4096, 128, 128, 128),      # config 2
+    (3, 200, 64, 128, 256),         # ragged rows, two p tiles
+    (2, 64, 128, 64, 128),
+    (1, 1, 64, 64, 128),            # a single row
+])
+def test_b2b_gemm_rowmajor(core, G, M, N, K, P):
+    """Row-major B [K,N] and C [N,P]: the same answer as the column-major entry point on transposed copies (to
+    the bit: same products, same order), and the oracle on a sample of problems."""
+    A, Bn, Cp = b2b_inputs(9, G, M, N, K, P)
+    Brm = np.ascontiguousarray(Bn.transpose(0, 2, 1)); Crm = np.ascontiguousarray(Cp.transpose(0, 2, 1))
+    D = core.b2b_gemm_rowmajor(dev(A), dev(Brm), dev(Crm))
+    Dc = core.b2b_gemm(dev(A), dev(Bn), dev(Cp))
+    torch.cuda.synchronize()
+    assert torch.equal(D, Dc)
+    for g in sorted({0, G - 1}):
+        ref = ko.b2b_gemm(A[g, :256], Bn[g], Cp[g])
+        assert ko.max_rel_err(D[g, :256].float().cpu().numpy(), ref) <= F16_TOL
+
+
+def test_b2b_gemm_rowmajor_rejects_other_shapes(core):
+    A = torch.zeros((1, 64, 96), dtype=torch.float16, device='cuda')
+    B = torch.zeros((1, 96, 64), dtype=torch.float16, device='cuda')
+    C = torch.zeros((1, 64, 128), dtype=torch.float16, device='cuda')
+    with pytest.raises(core.FtkError) as e:
+        core.b2b_gemm_rowmajor(A, B, C)
+    assert e.value.code == -2 and 'K and N in {64, 128}' in str(e.value)
+    assert not core.b2b_gemm_rowmajor_supported(64, 96, 128) and core.b2b_gemm_rowmajor_supported(128, 128, 256)
+
+
+
+@pytest.mark.parametrize('G,M,N,K,P', [
     (1, 32, 32, 32, 32),
     (2, 100, 64, 32, 64),       # ragged M
     (3, 256, 96, 96, 160),      # P spans two workgroup tiles, odd tile counts
