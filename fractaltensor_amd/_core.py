@@ -22,7 +22,7 @@ EXPORTS = (
     'ftk_stacked_lstm_workspace_bytes', 'ftk_stacked_lstm_f32', 'ftk_dilated_lstm_f32',
     'ftk_stacked_lstm_wavefront_f32', 'ftk_stacked_lstm_ragged_f32', 'ftk_lstm_set_products', 'ftk_lstm_get_products',
     'ftk_stacked_lstm_f16_workspace_bytes', 'ftk_stacked_lstm_f16',
-    'ftk_b2b_gemm_f16', 'ftk_b2b_gemm_rowmajor_f16', 'ftk_flash_attn_f16', 'ftk_online_softmax_f32', 'ftk_embedding_gather_f32',
+    'ftk_b2b_gemm_f16', 'ftk_b2b_gemm_rowmajor_f16', 'ftk_gemm_f16', 'ftk_batched_gemm_f16', 'ftk_flash_attn_f16', 'ftk_online_softmax_f32', 'ftk_embedding_gather_f32',
     'ftk_debug_read_fa_trace',
 )
 
@@ -356,6 +356,29 @@ def b2b_gemm_rowmajor(A, B, C, out: Optional[torch.Tensor] = None) -> torch.Tens
     ci = ctypes.c_int
     _check(lib.ftk_b2b_gemm_rowmajor_f16(_ptr(A), _ptr(B), _ptr(C), _ptr(D), ci(G), ci(M), ci(N), ci(K), ci(P), _stream()))
     return D[0] if squeeze and out is None else D
+
+
+def gemm(A, B, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """C = A @ B, fp16 storage, fp32 accumulation, row-major: A [M,K] or [G,M,K], B [K,N] or [G,K,N].
+    N a multiple of 128, K of 32."""
+    f16 = torch.float16
+    _req(A, f16, 'A'); _req(B, f16, 'B')
+    if A.dim() != B.dim() or A.dim() not in (2, 3):
+        raise ValueError('A and B must both be matrices or both be batches of matrices')
+    batched = A.dim() == 3
+    G = A.shape[0] if batched else 1
+    M, K = A.shape[-2:]
+    N = B.shape[-1]
+    if B.shape[-2] != K or (batched and B.shape[0] != G):
+        raise ValueError(f'shape mismatch: A {tuple(A.shape)}, B {tuple(B.shape)}')
+    C = out if out is not None else torch.empty((*A.shape[:-1], N), dtype=f16, device=A.device)
+    _req(C, f16, 'C')
+    ci = ctypes.c_int
+    if batched:
+        _check(lib.ftk_batched_gemm_f16(_ptr(A), _ptr(B), _ptr(C), ci(G), ci(M), ci(N), ci(K), _stream()))
+    else:
+        _check(lib.ftk_gemm_f16(_ptr(A), _ptr(B), _ptr(C), ci(M), ci(N), ci(K), _stream()))
+    return C
 
 
 def flash_attention(Q, K, V, scale: Optional[float] = None, out: Optional[torch.Tensor] = None) -> torch.Tensor:

@@ -293,9 +293,14 @@ __device__ __forceinline__ void cell_dma16(const void* gbase, unsigned byte_off,
 // their own scale and the h rows 2^14, so between the last x chunk and the first h chunk the sums are
 // multiplied by the ratio; the epilogue undoes the h and column scales, computes in fp32, writes h and c in
 // fp32 and the two planes of h for the cells that read it next.
-template <bool PACKED, int WAVES, bool SPLIT>
+//
+// GEMM: the product alone, C = A @ Bm for row-major fp16 A [B, I] (cell.x), Bm [I, 4H] (cell.WU) and C [B, 4H]
+// (cell.h): no state, no activation; the workgroup's 4*UB columns are the four runs UB*ub .. +UB of the four
+// column quarters, stored as they come out of the accumulators.
+template <bool PACKED, int WAVES, bool SPLIT, bool GEMM = false>
 __global__ __launch_bounds__(WAVES * 64, 8 / WAVES) void lstm_cell_f16_kernel(CellListH list, int B, int I, int H) {
   static_assert(!SPLIT || PACKED, "the split flavour reads packed weights");
+  static_assert(!GEMM || (!SPLIT && !PACKED), "the plain product reads Bm as it is");
   constexpr int REP = SPLIT ? 3 : 1;        // k chunks per chunk of the contraction
   constexpr int UB = 8 * WAVES;             // hidden units per workgroup
   constexpr int CW = WAVES / 2;             // waves side by side
@@ -310,8 +315,9 @@ __global__ __launch_bounds__(WAVES * 64, 8 / WAVES) void lstm_cell_f16_kernel(Ce
   // fetched into one L2 instead of eight, and the 64-byte weight segments of neighbouring unit blocks that
   // share a cache line are served by the same L2.
   const int nub = H / UB, nrb = (B + HROWS - 1) / HROWS;
-  const int slot = blockIdx.x >> 3;
-  const int cell = (blockIdx.x & 7) + 8 * (slot / (nub * nrb));
+  // (the plain product has few, large problems: its workgroups are simply numbered problem, row block, column block)
+  const int slot = GEMM ? (int)blockIdx.x : (int)(blockIdx.x >> 3);
+  const int cell = GEMM ? slot / (nub * nrb) : (int)(blockIdx.x & 7) + 8 * (slot / (nub * nrb));
   if (cell >= list.n) return;
   const CellDescH cd = list.cells[cell];
   const int ub = slot % nub;          // block of UB hidden units
@@ -482,6 +488,16 @@ __global__ __launch_bounds__(WAVES * 64, 8 / WAVES) void lstm_cell_f16_kernel(Ce
 #pragma unroll
     for (int u2 = 0; u2 < 2; ++u2) {
       const int u0 = ub * UB + 8 * (2 * wc + u2) + 4 * hh;
+      if constexpr (GEMM) {
+        _Float16* crow = reinterpret_cast<_Float16*>(cd.h) + (size_t)row_g * 4 * H + u0;
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          const v4h o = {(_Float16)acc[rt][u2][4 * q], (_Float16)acc[rt][u2][4 * q + 1], (_Float16)acc[rt][u2][4 * q + 2],
+                         (_Float16)acc[rt][u2][4 * q + 3]};
+          *reinterpret_cast<v4h*>(crow + (size_t)q * H) = o;
+        }
+        continue;
+      }
       v4f cp = {0, 0, 0, 0};
       if (cd.c_prev) {
         if constexpr (SPLIT) {
@@ -768,19 +784,19 @@ int pack_weights_f16(const void* WU, void* packed, int layers, int K2, int H, hi
   return check_launch("lstm_pack_weights_f16_kernel");
 }
 
-template <bool PACKED, int WAVES, bool SPLIT>
+template <bool PACKED, int WAVES, bool SPLIT, bool GEMM = false>
 static int launch_cells_f16(const CellListH& list, int B, int I, int H, hipStream_t s) {
   static bool attr_set = false;  // per process; the attribute belongs to the function, on every device
   constexpr int UB = 8 * WAVES;
-  const void* fn = (const void*)lstm_cell_f16_kernel<PACKED, WAVES, SPLIT>;
+  const void* fn = (const void*)lstm_cell_f16_kernel<PACKED, WAVES, SPLIT, GEMM>;
   if (!attr_set) {
     FTK_HIP(hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)cell_lds_bytes(UB)));
     attr_set = true;
   }
   const int groups = (list.n + 7) / 8;  // cells per XCD
-  dim3 grid(8 * groups * (H / UB) * ((B + HROWS - 1) / HROWS));
-  hipLaunchKernelGGL((lstm_cell_f16_kernel<PACKED, WAVES, SPLIT>), grid, dim3(WAVES * 64), cell_lds_bytes(UB), s, list, B, I,
-                     H);
+  dim3 grid((GEMM ? list.n : 8 * groups) * (H / UB) * ((B + HROWS - 1) / HROWS));
+  hipLaunchKernelGGL((lstm_cell_f16_kernel<PACKED, WAVES, SPLIT, GEMM>), grid, dim3(WAVES * 64), cell_lds_bytes(UB), s, list,
+                     B, I, H);
   return check_launch("lstm_cell_f16_kernel");
 }
 
@@ -1161,6 +1177,41 @@ int ftk_stacked_lstm_wavefront_f32(const float* xs, const float* WU, const float
         return ftk::fail(FTK_ERR_INVALID_ARGUMENT, "ftk_stacked_lstm_wavefront_f32: dilations[%d]=%d must be positive", l,
                          dilations[l]);
   return ftk::run_wavefront(xs, WU, bias, dilations, hsss, csss, L, T, B, H, (hipStream_t)stream);
+}
+
+// G products C = A @ Bm through the streaming cell kernel's product: every problem is a "cell" with x = A,
+// no state, WU = Bm seen as four column quarters.
+static int gemm_f16(const char* who, const void* A, const void* Bm, void* C, int G, int M, int N, int K, hipStream_t s) {
+  if (!A || !Bm || !C) return ftk::fail(FTK_ERR_INVALID_ARGUMENT, "%s: A, B, C must be non-NULL", who);
+  if (G <= 0 || M <= 0 || N <= 0 || K <= 0) return ftk::fail(FTK_ERR_INVALID_ARGUMENT, "%s: G, M, N, K must be positive", who);
+  if (N % 128 || K % 32) return ftk::fail(FTK_ERR_UNSUPPORTED_SHAPE, "%s: N=%d must be a multiple of 128 and K=%d of 32", who, N, K);
+  if ((long long)M * std::max(K, N) >= (1ll << 30)) return ftk::fail(FTK_ERR_UNSUPPORTED_SHAPE, "%s: M=%d too large", who, M);
+  const int Hq = N / 4;  // a column quarter
+  const _Float16* a = (const _Float16*)A;
+  const _Float16* b = (const _Float16*)Bm;
+  _Float16* c = (_Float16*)C;
+  for (int g0 = 0; g0 < G; g0 += ftk::kMaxCellsPerLaunch) {
+    ftk::CellListH list;
+    list.n = std::min(ftk::kMaxCellsPerLaunch, G - g0);
+    list.packed = 0;
+    for (int i = 0; i < list.n; ++i) {
+      const size_t g = (size_t)(g0 + i);
+      list.cells[i] = ftk::CellDescH{a + g * M * K, nullptr, nullptr, b + g * K * N, nullptr, c + g * M * N, nullptr,
+                                     nullptr, nullptr, nullptr};
+    }
+    const int rc = Hq % 64 == 0 ? ftk::launch_cells_f16<false, 8, false, true>(list, M, K, Hq, s)
+                                : ftk::launch_cells_f16<false, 4, false, true>(list, M, K, Hq, s);
+    if (rc) return rc;
+  }
+  return FTK_OK;
+}
+
+int ftk_gemm_f16(const void* A, const void* B, void* C, int M, int N, int K, ftk_stream_t stream) {
+  return gemm_f16("ftk_gemm_f16", A, B, C, 1, M, N, K, (hipStream_t)stream);
+}
+
+int ftk_batched_gemm_f16(const void* A, const void* B, void* C, int G, int M, int N, int K, ftk_stream_t stream) {
+  return gemm_f16("ftk_batched_gemm_f16", A, B, C, G, M, N, K, (hipStream_t)stream);
 }
 
 }  // extern "C"

@@ -23,7 +23,7 @@ from ..fractal_tensor import FractalTensor
 from ..tensor import Tensor
 from ..types import FractalTensorStorage, TensorStorage, torch_type_to_internal_type
 
-__all__ = ['pack_lstm_weights', 'pad_time_major', 'unpad_time_major', 'stacked_lstm', 'dilated_lstm', 'lstm_cell', 'flash_attention', 'b2b_gemm',
+__all__ = ['pack_lstm_weights', 'pad_time_major', 'unpad_time_major', 'stacked_lstm', 'dilated_lstm', 'lstm_cell', 'flash_attention', 'b2b_gemm', 'mm',
            'online_softmax', 'embedding_lookup']
 
 
@@ -213,6 +213,19 @@ def b2b_gemm(a, b, c):
     if isinstance(a, Tensor):
         return Tensor.from_tensor(D[0])
     return FractalTensor.from_dense(D, 1)
+
+
+def mm(a: Tensor, b: Tensor) -> Tensor:
+    """a @ b for fp16 Tensors on the GPU through the library's own MFMA product (ftk_gemm_f16): a [M,K], b [K,N],
+    N a multiple of 128, K of 32.  `ops.mm` itself stays with torch (hipBLASLt), which is the faster of the two
+    for a plain product; this is the building block the fused kernels are made of, callable on its own."""
+    for x, name in ((a, 'a'), (b, 'b')):
+        if not isinstance(x, Tensor):
+            raise TypeError(f'{name} should be a Tensor.')
+        if not x.data.is_cuda:
+            raise RuntimeError(f'{name} lives on {x.data.device}; the fused kernels run on the GPU only.')
+    in_dtype = a.data.dtype
+    return Tensor.from_tensor(_core().gemm(a.data.half().contiguous(), b.data.half().contiguous()).to(in_dtype))
 
 
 def online_softmax(x: Tensor) -> Tensor:

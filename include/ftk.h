@@ -278,6 +278,24 @@ int ftk_b2b_gemm_rowmajor_f16(const void* A, const void* B, const void* C,
                               void* D, int G, int M, int N, int K, int P,
                               ftk_stream_t stream);
 
+/* ------------------------------------------------------------ plain GEMM -- */
+
+/*
+ * C = A @ B, fp16 storage, fp32 accumulation, every operand row-major:
+ * A [M,K], B [K,N], C [M,N]; the batched form takes G independent problems
+ * A [G,M,K], B [G,K,N], C [G,M,N].  Needs N%128==0, K%32==0.  The product of
+ * the streaming LSTM cell kernel without the cell (256 rows x 256 columns per
+ * workgroup, k chunks of 32 through a ring of LDS stages, B transposed between
+ * LDS and the matrix unit), offered as a building block.  Stands in for
+ * KeCuteGemm / KeBatchedCuteGemm / KeGemmPipelined
+ * (kaleido/core/device/kernels/gemm_kernels.h, cutlass_wmma.h:34-440) behind
+ * ops.mm (kaleido/frontend/operations/tensor/contraction.py:15-18).
+ */
+int ftk_gemm_f16(const void* A, const void* B, void* C, int M, int N, int K,
+                 ftk_stream_t stream);
+int ftk_batched_gemm_f16(const void* A, const void* B, void* C, int G, int M,
+                         int N, int K, ftk_stream_t stream);
+
 /* ------------------------------------------------------ flash attention -- */
 
 /*

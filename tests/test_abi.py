@@ -42,6 +42,8 @@ def test_argument_errors_come_back_as_codes_not_crashes():
     assert lib.ftk_b2b_gemm_f16(one, one, one, one, ci(0), ci(64), ci(64), ci(64), ci(64), nul) == -1
     assert lib.ftk_b2b_gemm_rowmajor_f16(one, one, one, one, ci(1), ci(64), ci(64), ci(96), ci(128), nul) == -2
     assert lib.ftk_b2b_gemm_rowmajor_f16(one, nul, one, one, ci(1), ci(64), ci(64), ci(64), ci(128), nul) == -1
+    assert lib.ftk_gemm_f16(one, one, one, ci(64), ci(96), ci(64), nul) == -2
+    assert lib.ftk_batched_gemm_f16(one, one, nul, ci(2), ci(64), ci(128), ci(64), nul) == -1
     assert lib.ftk_flash_attn_f16(one, one, one, one, ci(1), ci(1), ci(64), ci(64), ci(48), ctypes.c_float(1), nul) == -2
     assert lib.ftk_online_softmax_f32(nul, one, ci(1), ci(1), nul) == -1
     assert lib.ftk_stacked_lstm_wavefront_f32(one, one, nul, nul, one, one, ci(1), ci(1), ci(1), ci(48), nul) == -2

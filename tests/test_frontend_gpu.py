@@ -76,6 +76,16 @@ def test_fused_flash_attention_equals_eager_program():
     assert ko.max_rel_err(dense(fused), dense(eager)) <= 1e-2
 
 
+def test_fused_mm_equals_operator_mm():
+    a = Tensor.from_tensor((torch.randn(96, 64, device='cuda') / 8).half())
+    b = Tensor.from_tensor(torch.randn(64, 256, device='cuda').half())
+    got = ops.fused.mm(a, b).data.float()
+    ref = ops.mm(a, b).data.float()
+    assert float((got - ref).abs().max() / ref.abs().max()) <= 1e-2
+    with pytest.raises(RuntimeError):
+        ops.fused.mm(Tensor.from_tensor(a.data.cpu()), b)
+
+
 def test_fused_b2b_gemm_equals_operator_expression():
     M, K, N, P = 128, 64, 96, 32
     g = torch.Generator().manual_seed(8)

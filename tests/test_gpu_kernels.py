@@ -485,6 +485,38 @@ def test_b2b_gemm_rowmajor(core, G, M, N, K, P):
         assert ko.max_rel_err(D[g, :256].float().cpu().numpy(), ref) <= F16_TOL
 
 
+@pytest.mark.parametrize('G,M,N,K', [
+    (0, 512, 512, 256),         # 0: the single-problem entry point
+    (0, 300, 128, 64),          # 32 columns per quarter: four-wave workgroups; ragged rows
+    (0, 1, 256, 32),            # one row, one k chunk
+    (3, 257, 384, 96),          # batched; 96 columns per quarter
+    (45, 64, 256, 128),         # more problems than one launch takes
+])
+def test_gemm_f16(core, G, M, N, K):
+    rng = np.random.default_rng(4)
+    shape_a, shape_b = ((M, K), (K, N)) if G == 0 else ((G, M, K), (G, K, N))
+    A = (rng.standard_normal(shape_a) / np.sqrt(K)).astype(np.float16)
+    Bm = rng.standard_normal(shape_b).astype(np.float16)
+    C = core.gemm(dev(A), dev(Bm)).float().cpu().numpy()
+    ref = A.astype(np.float64) @ Bm.astype(np.float64)
+    assert ko.max_rel_err(C, ref) <= F16_TOL
+    # fp32 sums of exact products, rounded once: all but values within rounding of a tie agree with the rounded
+    # float64 product to the bit
+    assert np.mean(C == ref.astype(np.float16).astype(np.float32)) > 0.98
+
+
+def test_gemm_f16_rejects_bad_arguments(core):
+    A = torch.zeros((64, 48), dtype=torch.float16, device='cuda')
+    B = torch.zeros((48, 128), dtype=torch.float16, device='cuda')
+    with pytest.raises(core.FtkError) as e:
+        core.gemm(A, B)
+    assert e.value.code == -2 and 'multiple of 128' in str(e.value)
+    with pytest.raises(ValueError):
+        core.gemm(A, torch.zeros((32, 128), dtype=torch.float16, device='cuda'))
+    with pytest.raises(TypeError):
+        core.gemm(A.float(), B.float())
+
+
 def test_b2b_gemm_rowmajor_rejects_other_shapes(core):
     A = torch.zeros((1, 64, 96), dtype=torch.float16, device='cuda')
     B = torch.zeros((1, 96, 64), dtype=torch.float16, device='cuda')
