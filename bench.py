@@ -179,6 +179,36 @@ def bench_embedding(torch, core, steps, warmup, cpu):
     return res
 
 
+def bench_gemm(torch, core, steps, warmup, cpu):
+    """The plain fp16 product that the streaming kernels are built around, on its own: 8192^3, beside torch.mm."""
+    M = N = K = 8192
+    gen = torch.Generator(device='cpu').manual_seed(1234)
+    A = (torch.randn((M, K), generator=gen) / K ** 0.5).half().cuda()
+    B = torch.randn((K, N), generator=gen).half().cuda()
+    C = torch.empty((M, N), dtype=torch.float16, device='cuda')
+    ms, _ = _events_ms(torch, lambda: core.gemm(A, B, out=C), steps, warmup)
+    ref = C.clone()
+    ms_t, _ = _events_ms(torch, lambda: torch.mm(A, B, out=C), steps, warmup)
+    flop = 2.0 * M * N * K
+    res = {
+        'metric': 'TFLOP/s (plain GEMM)', 'value': flop / ms / 1e9, 'unit': 'TFLOP/s', 'ms_per_step': ms, 'dtype': 'f16',
+        'config': {'workload': 'plain GEMM building block (ftk_gemm_f16), row-major A, B, C', 'M': M, 'N': N, 'K': K, 'accumulate': 'f32'},
+        'roofline': {'bound': 'mfma', 'achieved': flop / ms / 1e9, 'peak': PEAK_F16_TFLOPS, 'unit': 'TFLOP/s',
+                     'frac': flop / ms / 1e9 / PEAK_F16_TFLOPS, 'traffic': None, 'kernel': 'lstm_cell_f16_kernel<false, 8, false, true>'},
+        'torch_mm': {'ms_per_step': ms_t, 'tflops': flop / ms_t / 1e9,
+                     'max_rel_diff': float((C.float() - ref.float()).abs().max() / ref.float().abs().max())},
+    }
+    if cpu:
+        n = 1024
+        a, b = A[:n, :n].float().cpu(), B[:n, :n].float().cpu()
+        t0 = time.perf_counter()
+        _ = a @ b
+        dt = time.perf_counter() - t0
+        res['cpu_baseline'] = {'value': 2.0 * n ** 3 / dt / 1e12, 'unit': 'TFLOP/s', 'cores': torch.get_num_threads(), 'kind': 'port',
+                               'sample': f'torch fp32 matmul of a {n}^3 corner on the host, {dt:.3f} s'}
+    return res
+
+
 def _unfused_lstm_baseline(torch, core, xs, WU, hs, cs, dil=None):
     """Per-step GEMM (rocBLAS/hipBLASLt through torch) + one elementwise kernel, layer-major:
     the structure of benchmarks/rnn/fractaltensor/stacked_lstm (utils.h:559-625).  Returns a
@@ -451,7 +481,7 @@ def main():
     ap.add_argument('--gpus', type=int, default=1)
     ap.add_argument('--steps', type=int, default=50)
     ap.add_argument('--warmup', type=int, default=10)
-    ap.add_argument('--workload', default='b2b', choices=['b2b', 'attention', 'stacked_lstm', 'dilated_lstm', 'lstm_f16_h256', 'lstm_f16_h512', 'lstm_f16_h1024', 'lstm_f32_h512', 'lstm_f32_h1024', 'embedding', 'copy'])
+    ap.add_argument('--workload', default='b2b', choices=['b2b', 'attention', 'stacked_lstm', 'dilated_lstm', 'lstm_f16_h256', 'lstm_f16_h512', 'lstm_f16_h1024', 'lstm_f32_h512', 'lstm_f32_h1024', 'gemm', 'embedding', 'copy'])
     ap.add_argument('--no-extras', action='store_true', help='measure only the chosen workload')
     ap.add_argument('--no-cpu', action='store_true', help='skip the CPU baseline leg')
     ap.add_argument('--no-baselines', action='store_true',
@@ -480,6 +510,7 @@ def main():
         'lstm_f16_h1024': lambda s, w, c: bench_lstm_f16(torch, core, max(3, s // 5), max(1, w // 5), c, 1024, not args.no_baselines),
         'lstm_f32_h512': lambda s, w, c: bench_lstm_f32_streamed(torch, core, max(3, s // 5), max(1, w // 5), c, 512),
         'lstm_f32_h1024': lambda s, w, c: bench_lstm_f32_streamed(torch, core, max(3, s // 10), 1, c, 1024),
+        'gemm': lambda s, w, c: bench_gemm(torch, core, max(5, s // 5), max(2, w // 5), c),
         'embedding': lambda s, w, c: bench_embedding(torch, core, s, w, c),
     }
     if args.workload == 'copy':
