@@ -14,6 +14,7 @@ steps walk a ring of input sets larger than the 256 MB memory-side cache, so
 the figure is an HBM figure; the same-buffers figure is reported next to it.
 """
 import argparse
+import ctypes
 import json
 import os
 import sys
@@ -176,6 +177,38 @@ def bench_embedding(torch, core, steps, warmup, cpu):
         dt = time.perf_counter() - t0
         res['cpu_baseline'] = {'value': n / dt, 'unit': 'rows/s', 'cores': torch.get_num_threads(), 'kind': 'port',
                                'sample': f'torch index_select of the same {n} ids on the host, {dt:.2f} s'}
+    return res
+
+
+def bench_softmax(torch, core, steps, warmup, cpu):
+    """Row softmax of [65536, 1027] fp32 (1027: the widest row of the reference's test, test_softmax.cc:77-87; rows
+    that are not 16-byte aligned), beside torch.softmax; every element read once and written once."""
+    rows, cols = 65536, 1027
+    gen = torch.Generator(device='cpu').manual_seed(1234)
+    x = (torch.randn((rows, cols), generator=gen) * 4).cuda()
+    y = torch.empty_like(x)
+    ci = ctypes.c_int
+    run = lambda: core._check(core.lib.ftk_online_softmax_f32(core._ptr(x), core._ptr(y), ci(rows), ci(cols), core._stream()))
+    ms, _ = _events_ms(torch, run, steps, warmup)
+    ms_t, _ = _events_ms(torch, lambda: torch.softmax(x, 1, out=y), steps, warmup)
+    nbytes = 2.0 * rows * cols * 4
+    res = {
+        'metric': 'softmax rows/s', 'value': rows / ms * 1e3, 'unit': 'rows/s', 'ms_per_step': ms, 'dtype': 'f32',
+        'config': {'workload': 'row softmax through (max, denominator) pairs (online_softmax_op.cu:14-36)', 'rows': rows, 'cols': cols},
+        'roofline': {'bound': 'hbm', 'achieved': nbytes / ms / 1e6, 'peak': PEAK_HBM_GBS, 'unit': 'GB/s',
+                     'frac': nbytes / ms / 1e6 / PEAK_HBM_GBS, 'traffic': None,
+                     'kernel': 'softmax_rows_in_registers_kernel<64, 32, false>', 'algorithmic_bytes_per_launch': nbytes},
+        'torch_softmax': {'ms_per_step': ms_t, 'gbs': nbytes / ms_t / 1e6},
+    }
+    if cpu:
+        from oracle import c_oracle
+        n = rows
+        xs = x[:n].cpu().numpy()
+        t0 = time.perf_counter()
+        c_oracle.online_softmax(xs)
+        dt = time.perf_counter() - t0
+        res['cpu_baseline'] = {'value': n / dt, 'unit': 'rows/s', 'cores': 1, 'kind': 'port',
+                               'sample': f'{n} rows through oracle/oracle.c in {dt:.2f} s'}
     return res
 
 
@@ -481,7 +514,7 @@ def main():
     ap.add_argument('--gpus', type=int, default=1)
     ap.add_argument('--steps', type=int, default=50)
     ap.add_argument('--warmup', type=int, default=10)
-    ap.add_argument('--workload', default='b2b', choices=['b2b', 'attention', 'stacked_lstm', 'dilated_lstm', 'lstm_f16_h256', 'lstm_f16_h512', 'lstm_f16_h1024', 'lstm_f32_h512', 'lstm_f32_h1024', 'gemm', 'embedding', 'copy'])
+    ap.add_argument('--workload', default='b2b', choices=['b2b', 'attention', 'stacked_lstm', 'dilated_lstm', 'lstm_f16_h256', 'lstm_f16_h512', 'lstm_f16_h1024', 'lstm_f32_h512', 'lstm_f32_h1024', 'gemm', 'online_softmax', 'embedding', 'copy'])
     ap.add_argument('--no-extras', action='store_true', help='measure only the chosen workload')
     ap.add_argument('--no-cpu', action='store_true', help='skip the CPU baseline leg')
     ap.add_argument('--no-baselines', action='store_true',
@@ -511,6 +544,7 @@ def main():
         'lstm_f32_h512': lambda s, w, c: bench_lstm_f32_streamed(torch, core, max(3, s // 5), max(1, w // 5), c, 512),
         'lstm_f32_h1024': lambda s, w, c: bench_lstm_f32_streamed(torch, core, max(3, s // 10), 1, c, 1024),
         'gemm': lambda s, w, c: bench_gemm(torch, core, max(5, s // 5), max(2, w // 5), c),
+        'online_softmax': lambda s, w, c: bench_softmax(torch, core, s, w, c),
         'embedding': lambda s, w, c: bench_embedding(torch, core, s, w, c),
     }
     if args.workload == 'copy':
