@@ -196,7 +196,7 @@ def bench_softmax(torch, core, steps, warmup, cpu):
         'metric': 'softmax rows/s', 'value': rows / ms * 1e3, 'unit': 'rows/s', 'ms_per_step': ms, 'dtype': 'f32',
         'config': {'workload': 'row softmax through (max, denominator) pairs (online_softmax_op.cu:14-36)', 'rows': rows, 'cols': cols},
         'roofline': {'bound': 'hbm', 'achieved': nbytes / ms / 1e6, 'peak': PEAK_HBM_GBS, 'unit': 'GB/s',
-                     'frac': nbytes / ms / 1e6 / PEAK_HBM_GBS, 'traffic': None,
+                     'frac': nbytes / ms / 1e6 / PEAK_HBM_GBS, 'traffic': MEASURED_TRAFFIC_BYTES.get('softmax_rows_in_registers_kernel'),
                      'kernel': 'softmax_rows_in_registers_kernel<64, 32, false>', 'algorithmic_bytes_per_launch': nbytes},
         'torch_softmax': {'ms_per_step': ms_t, 'gbs': nbytes / ms_t / 1e6},
     }
@@ -227,7 +227,8 @@ def bench_gemm(torch, core, steps, warmup, cpu):
         'metric': 'TFLOP/s (plain GEMM)', 'value': flop / ms / 1e9, 'unit': 'TFLOP/s', 'ms_per_step': ms, 'dtype': 'f16',
         'config': {'workload': 'plain GEMM building block (ftk_gemm_f16), row-major A, B, C', 'M': M, 'N': N, 'K': K, 'accumulate': 'f32'},
         'roofline': {'bound': 'mfma', 'achieved': flop / ms / 1e9, 'peak': PEAK_F16_TFLOPS, 'unit': 'TFLOP/s',
-                     'frac': flop / ms / 1e9 / PEAK_F16_TFLOPS, 'traffic': None, 'kernel': 'lstm_cell_f16_kernel<false, 8, false, true>'},
+                     'frac': flop / ms / 1e9 / PEAK_F16_TFLOPS, 'traffic': MEASURED_TRAFFIC_BYTES.get('gemm_8192'),
+                     'kernel': 'lstm_cell_f16_kernel<false, 8, false, true>'},
         'torch_mm': {'ms_per_step': ms_t, 'tflops': flop / ms_t / 1e9,
                      'max_rel_diff': float((C.float() - ref.float()).abs().max() / ref.float().abs().max())},
     }
