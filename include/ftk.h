@@ -272,7 +272,7 @@ int ftk_b2b_gemm_f16(const void* A, const void* B, const void* C, void* D,
  * {64, 128}, P%128==0 (anything else: FTK_ERR_UNSUPPORTED_SHAPE; transpose B
  * and C once and call ftk_b2b_gemm_f16).  No counterpart in the reference,
  * whose B2BGemm takes column-major B and C only (gemm_kernel_traits.h:261-267);
- * it is what kaleido's `(a @ b) @ c` (Tensor.__matmul__, tensor.py:110-116) maps to.
+ * it is what kaleido's `(a @ b) @ c` (Tensor.__matmul__, kaleido/frontend/tensor.py:218-220) maps to.
  */
 int ftk_b2b_gemm_rowmajor_f16(const void* A, const void* B, const void* C,
                               void* D, int G, int M, int N, int K, int P,
@@ -288,8 +288,9 @@ int ftk_b2b_gemm_rowmajor_f16(const void* A, const void* B, const void* C,
  * workgroup, k chunks of 32 through a ring of LDS stages, B transposed between
  * LDS and the matrix unit), offered as a building block.  Stands in for
  * KeCuteGemm / KeBatchedCuteGemm / KeGemmPipelined
- * (kaleido/core/device/kernels/gemm_kernels.h, cutlass_wmma.h:34-440) behind
- * ops.mm (kaleido/frontend/operations/tensor/contraction.py:15-18).
+ * (kaleido/core/device/kernels/cutlass_wmma.h:116,186,259; functors CuteGemm,
+ * GemmPipelined gemm.h:152,201 and batched_gemm.h:84) behind ops.mm (MatMul,
+ * kaleido/frontend/operations/tensor/arithmetic/contraction.py:21).
  */
 int ftk_gemm_f16(const void* A, const void* B, void* C, int M, int N, int K,
                  ftk_stream_t stream);
