@@ -93,8 +93,9 @@ struct PersistArgs {
   int* status;  // [0] = error word
   int L, T, B;
   int nrb;         // row blocks of 32*RT rows
-  int pr;          // row slices per layer
-  int groups;      // workgroups that take part (= L * PC * pr)
+  int pr_of[kMaxLayers];        // row slices of layer l (its workgroups: column slices x row slices)
+  int first_q[kMaxLayers + 1];  // first logical workgroup of layer l; [L] = all
+  int groups;      // workgroups that take part (= first_q[L])
   int xcd_remap;   // 1: grid is a multiple of 8, map workgroups so a layer shares an XCD
   int spin_limit;
   int trace_q;            // logical workgroup whose item timeline is recorded, or -1
@@ -210,15 +211,16 @@ void lstm_persistent_kernel(PersistArgs a) {
   if (a.xcd_remap) q = (blockIdx.x & 7) * (gridDim.x >> 3) + (blockIdx.x >> 3);
   if (q >= a.groups) return;
   if (q == a.trace_q && tid == 0) reinterpret_cast<long long*>(a.status + 16)[0] = wall_clock64();
-  const int per_layer = NPC * a.pr;
-  const int l = q / per_layer;
-  const int within = q - l * per_layer;
+  int l = 0;
+  while (l + 1 < a.L && q >= a.first_q[l + 1]) ++l;
+  const int pr = a.pr_of[l];
+  const int within = q - a.first_q[l];
   const int pc = within % NPC;
   const int prs = within / NPC;
   const int d = a.dil[l];
   const int T = a.T, B = a.B;
   const size_t cell = (size_t)B * (F16 ? HID / 2 : PH);  // floats (or pairs of fp16) per [B, H] slab of activations
-  const int my_rbs = (a.nrb - prs + a.pr - 1) / a.pr;  // row blocks this workgroup walks per time step
+  const int my_rbs = (a.nrb - prs + pr - 1) / pr;  // row blocks this workgroup walks per time step
   const int n_items = T * my_rbs;
 
   // Resident weights.  fp32 products: lane (i = j, half hh) of wave w holds, for
@@ -296,7 +298,7 @@ void lstm_persistent_kernel(PersistArgs a) {
   }
 
   auto item_t = [&](int n) { return n / my_rbs; };
-  auto item_rb = [&](int n) { return prs + a.pr * (n % my_rbs); };
+  auto item_rb = [&](int n) { return prs + pr * (n % my_rbs); };
   // Ragged batches (rows sorted by length, so a row block simply stops after its longest row): an item
   // past its block's last step is walked through like any other, but requests, computes, stores and counts
   // nothing; nothing that is computed depends on it.
@@ -947,8 +949,28 @@ static int run_persistent(int mode, const void* xs, const void* WU, const float*
   a.nrb = (B + 31) / 32;
   // spare compute units become row slices, but a workgroup keeps at least two
   // row blocks when it can so that the next tile never depends on the current item
-  a.pr = std::max(1, std::min(slots / (L * npc), std::max(1, a.nrb / 2)));
-  a.groups = L * npc * a.pr;
+  const int pr = std::max(1, std::min(slots / (L * npc), std::max(1, a.nrb / 2)));
+  int used = 0;
+  for (int l = 0; l < L; ++l) {
+    a.pr_of[l] = pr;
+    used += npc * pr;
+  }
+  // A layer whose own chain is shorter than four items (dilation x row blocks per workgroup) cannot have the
+  // next tile under way while it works on an item: each of its items then costs a whole hand-over.  Such a
+  // layer gets one row block per workgroup where compute units are left, so that a time step costs it one
+  // hand-over instead of one per row block it walks.
+  for (int l = 0; l < L; ++l) {
+    const int d = dil ? dil[l] : 1;
+    const int my_rbs = (a.nrb + pr - 1) / pr;
+    if (d * my_rbs < 4 && my_rbs > 1 && used - npc * pr + npc * a.nrb <= slots && !getenv("FTK_LSTM_UNIFORM_SLICES")) {
+      used += npc * (a.nrb - pr);
+      a.pr_of[l] = a.nrb;
+    }
+  }
+  a.first_q[0] = 0;
+  for (int l = 0; l < L; ++l) a.first_q[l + 1] = a.first_q[l] + npc * a.pr_of[l];
+  for (int l = L; l < kMaxLayers; ++l) { a.pr_of[l] = 1; a.first_q[l + 1] = a.first_q[L]; }
+  a.groups = a.first_q[L];
   a.spin_limit = 1 << 22;
   a.trace_q = trace_workgroup();
   a.trace = reinterpret_cast<long long*>(reinterpret_cast<char*>(ws) + trace_offset_bytes(L, T, B));
