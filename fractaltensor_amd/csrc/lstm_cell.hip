@@ -228,6 +228,7 @@ struct CellDescH {
   const float* xratio;     // [B]: scale of the x rows relative to the h rows, or nullptr (x is an h of the layer below)
   const float* wscale;     // [4H]: what a gate sum of column n is multiplied by to undo the operand scales
   _Float16* h_planes;      // [B, 2H]: the two planes of h for the cells that read it
+  int rows;                // leading batch rows this cell computes (a ragged batch at its step), 0 = all B
 };
 
 struct CellListH {
@@ -320,6 +321,7 @@ __global__ __launch_bounds__(WAVES * 64, 8 / WAVES) void lstm_cell_f16_kernel(Ce
   const int cell = GEMM ? slot / (nub * nrb) : (int)(blockIdx.x & 7) + 8 * (slot / (nub * nrb));
   if (cell >= list.n) return;
   const CellDescH cd = list.cells[cell];
+  const int Bc = cd.rows > 0 ? cd.rows : B;  // rows of this cell
   const int ub = slot % nub;          // block of UB hidden units
   const int rb = (slot / nub) % nrb;  // block of 256 batch rows
   const int lane = threadIdx.x & 63;
@@ -332,7 +334,8 @@ __global__ __launch_bounds__(WAVES * 64, 8 / WAVES) void lstm_cell_f16_kernel(Ce
 
   const int nch_x = REP * (I / HK);
   const int nch = nch_x + (cd.h_prev ? REP * (H / HK) : 0);
-  const bool full = rb * HROWS + HROWS <= B;
+  if (rb * HROWS >= Bc) return;  // a row block past the live rows of this step
+  const bool full = rb * HROWS + HROWS <= Bc;
 
   // ---- copies: per chunk a wave issues ACT_COPIES activation copies (16 rows each, row lane/4) and 2 weight
   // copies (1 KB = 4 or 2 weight rows each)
@@ -374,7 +377,7 @@ __global__ __launch_bounds__(WAVES * 64, 8 / WAVES) void lstm_cell_f16_kernel(Ce
       const char* base = reinterpret_cast<const char*>(src + k0);
 #pragma unroll
       for (int i = 0; i < ACT_COPIES; ++i) {
-        const int row = min(rb * HROWS + row0 + 16 * i + (lane >> 2), B - 1);
+        const int row = min(rb * HROWS + row0 + 16 * i + (lane >> 2), Bc - 1);
         cell_dma16(base, (unsigned)row * (unsigned)(2 * ld) + a_lane_chunk, act_lds + 1024u * i);
       }
     }
@@ -418,7 +421,7 @@ __global__ __launch_bounds__(WAVES * 64, 8 / WAVES) void lstm_cell_f16_kernel(Ce
     if (!cd.xratio) return;
 #pragma unroll
     for (int rt = 0; rt < 4; ++rt) {
-      const float ratio = cd.xratio[min(rb * HROWS + 128 * wr + 32 * rt + j, B - 1)];
+      const float ratio = cd.xratio[min(rb * HROWS + 128 * wr + 32 * rt + j, Bc - 1)];
 #pragma unroll
       for (int u2 = 0; u2 < 2; ++u2)
 #pragma unroll
@@ -484,7 +487,7 @@ __global__ __launch_bounds__(WAVES * 64, 8 / WAVES) void lstm_cell_f16_kernel(Ce
 #pragma unroll
   for (int rt = 0; rt < 4; ++rt) {
     const int row_g = rb * HROWS + 128 * wr + 32 * rt + j;
-    if (row_g >= B) continue;
+    if (row_g >= Bc) continue;
 #pragma unroll
     for (int u2 = 0; u2 < 2; ++u2) {
       const int u0 = ub * UB + 8 * (2 * wc + u2) + 4 * hh;
@@ -580,6 +583,7 @@ __global__ __launch_bounds__(512, 1) void lstm_cell_split4_kernel(CellListH list
   const int cell = (blockIdx.x & 7) + 8 * (slot / (nub * nrb));  // all workgroups of a cell on one XCD
   if (cell >= list.n) return;
   const CellDescH cd = list.cells[cell];
+  const int Bc = cd.rows > 0 ? cd.rows : B;  // rows of this cell
   const int ub = slot % nub;
   const int rb = (slot / nub) % nrb;
   const int lane = threadIdx.x & 63;
@@ -592,7 +596,8 @@ __global__ __launch_bounds__(512, 1) void lstm_cell_split4_kernel(CellListH list
 
   const int nch_x = I / HK;
   const int nch = nch_x + (cd.h_prev ? H / HK : 0);
-  const bool full = rb * HROWS + HROWS <= B;
+  if (rb * HROWS >= Bc) return;  // a row block past the live rows of this step
+  const bool full = rb * HROWS + HROWS <= Bc;
 
   // per chunk a wave issues 2 + 2 activation copies (rows 32*wave + 16 i + lane/4 of each plane) and 2 + 2
   // weight copies (1 KB = rows 4*wave + 2 i + lane/32 of each plane, already in LDS order)
@@ -616,7 +621,7 @@ __global__ __launch_bounds__(512, 1) void lstm_cell_split4_kernel(CellListH list
         const char* base = reinterpret_cast<const char*>(src + pl * width);
 #pragma unroll
         for (int i = 0; i < 2; ++i) {
-          const int row = min(rb * HROWS + row0 + 16 * i + (lane >> 2), B - 1);
+          const int row = min(rb * HROWS + row0 + 16 * i + (lane >> 2), Bc - 1);
           cell_dma16(base, (unsigned)row * (unsigned)(2 * ld) + a_lane_chunk, act_lds + 1024u * i);
         }
       }
@@ -652,7 +657,7 @@ __global__ __launch_bounds__(512, 1) void lstm_cell_split4_kernel(CellListH list
     if (!cd.xratio) return;
 #pragma unroll
     for (int rt = 0; rt < 4; ++rt) {
-      const float ratio = cd.xratio[min(rb * HROWS + 128 * wr + 32 * rt + j, B - 1)];
+      const float ratio = cd.xratio[min(rb * HROWS + 128 * wr + 32 * rt + j, Bc - 1)];
 #pragma unroll
       for (int u2 = 0; u2 < 2; ++u2)
 #pragma unroll
@@ -707,7 +712,7 @@ __global__ __launch_bounds__(512, 1) void lstm_cell_split4_kernel(CellListH list
 #pragma unroll
   for (int rt = 0; rt < 4; ++rt) {
     const int row_g = rb * HROWS + 128 * wr + 32 * rt + j;
-    if (row_g >= B) continue;
+    if (row_g >= Bc) continue;
 #pragma unroll
     for (int u2 = 0; u2 < 2; ++u2) {
       const int u0 = ub * UB + 8 * (2 * wc + u2) + 4 * hh;
@@ -846,9 +851,12 @@ static std::vector<std::vector<int>> cells_by_stage(int L, int T, const int* dil
   return by_stage;
 }
 
+static void set_rows(CellDesc&, int) {}
+static void set_rows(CellDescH& cd, int rows) { cd.rows = rows; }
+
 template <typename Elem, typename List>
 static int run_wavefront_of(const Elem* xs, const Elem* WU, const float* bias, const int* dil, Elem* hsss, Elem* csss,
-                            int L, int T, int B, int H, hipStream_t s, bool packed = false) {
+                            int L, int T, int B, int H, hipStream_t s, bool packed = false, const int* active = nullptr) {
   const std::vector<std::vector<int>> by_stage = cells_by_stage(L, T, dil);
 
   const size_t cell = (size_t)B * H;
@@ -869,8 +877,11 @@ static int run_wavefront_of(const Elem* xs, const Elem* WU, const float* bias, c
         cd.bias = bias ? bias + (size_t)l * 4 * H : nullptr;
         cd.h = hsss + ((size_t)l * T + t) * cell;
         cd.c = csss + ((size_t)l * T + t) * cell;
+        set_rows(cd, active ? active[t] : 0);
+        if (active && active[t] == 0) --list.n;  // nothing lives at this step
         ++pos;
       }
+      if (list.n == 0) continue;
       int rc = launch_cells(list, B, H, H, s);
       if (rc) return rc;
     }
@@ -885,14 +896,14 @@ int run_wavefront(const float* xs, const float* WU, const float* bias, const int
 
 // The same schedule over fp16 arrays (H a multiple of 32).  packed: a buffer of the size of WU, into which the
 // weights are first re-laid per unit block, or nullptr to read WU as it is.
-int run_wavefront_f16(const void* xs, const void* WU, const float* bias, const int* dil, void* hsss, void* csss,
-                      int L, int T, int B, int H, void* packed, hipStream_t s) {
+int run_wavefront_f16(const void* xs, const void* WU, const float* bias, const int* dil, const int* active, void* hsss,
+                      void* csss, int L, int T, int B, int H, void* packed, hipStream_t s) {
   if (packed) {
     int rc = pack_weights_f16(WU, packed, L, 2 * H, H, s);
     if (rc) return rc;
   }
   return run_wavefront_of<_Float16, CellListH>((const _Float16*)xs, (const _Float16*)(packed ? packed : WU), bias, dil,
-                                               (_Float16*)hsss, (_Float16*)csss, L, T, B, H, s, packed != nullptr);
+                                               (_Float16*)hsss, (_Float16*)csss, L, T, B, H, s, packed != nullptr, active);
 }
 
 // ------------------------------------------------- fp32 stack on split products
@@ -1004,8 +1015,8 @@ size_t split_stack_workspace_bytes(int L, int T, int B, int H) {
 }
 
 // The fp32 stack through the split flavour of the streaming cell kernel (H a multiple of 32).
-int run_wavefront_split(const float* xs, const float* WU, const float* bias, const int* dil, float* hsss, float* csss,
-                        int L, int T, int B, int H, void* ws, hipStream_t s) {
+int run_wavefront_split(const float* xs, const float* WU, const float* bias, const int* dil, const int* active, float* hsss,
+                        float* csss, int L, int T, int B, int H, void* ws, hipStream_t s) {
   char* p = reinterpret_cast<char*>(ws);
   float* wscale = reinterpret_cast<float*>(p);
   p += round256s((size_t)L * 4 * H * sizeof(float));
@@ -1059,8 +1070,11 @@ int run_wavefront_split(const float* xs, const float* WU, const float* bias, con
         cd.xratio = (l == 0) ? xratio + (size_t)t * B : nullptr;
         cd.wscale = wscale + (size_t)l * 4 * H;
         cd.h_planes = hp + ((size_t)l * T + t) * 2 * cell;
+        cd.rows = active ? active[t] : 0;
+        if (active && active[t] == 0) --list.n;  // nothing lives at this step
         ++pos;
       }
+      if (list.n == 0) continue;
       rc = launch_cells(list, B, H, H, s);
       if (rc) return rc;
     }
@@ -1101,7 +1115,7 @@ int ftk_lstm_cell_f16(const void* x, const void* h_prev, const void* c_prev, con
   list.n = 1;
   list.packed = 0;
   list.cells[0] = ftk::CellDescH{(const _Float16*)x, (const _Float16*)h_prev, c_prev, (const _Float16*)WU, bias, h, c,
-                                 nullptr, nullptr, nullptr};
+                                 nullptr, nullptr, nullptr, 0};
   return ftk::launch_cells(list, B, I, H, (hipStream_t)stream);
 }
 
@@ -1145,7 +1159,7 @@ int ftk_lstm_layer_f16(const void* xs, const void* WU, const float* bias, const 
     list.packed = 0;
     list.cells[0] = ftk::CellDescH{x16 + (size_t)t * B * I, t ? h16 + (t - 1) * cell : (const _Float16*)h0,
                                    t ? (const void*)(c16 + (t - 1) * cell) : c0, (const _Float16*)WU, bias, h16 + t * cell,
-                                   c16 + t * cell, nullptr, nullptr, nullptr};
+                                   c16 + t * cell, nullptr, nullptr, nullptr, 0};
     int rc = ftk::launch_cells(list, B, I, H, (hipStream_t)stream);
     if (rc) return rc;
   }
@@ -1197,7 +1211,7 @@ static int gemm_f16(const char* who, const void* A, const void* Bm, void* C, int
     for (int i = 0; i < list.n; ++i) {
       const size_t g = (size_t)(g0 + i);
       list.cells[i] = ftk::CellDescH{a + g * M * K, nullptr, nullptr, b + g * K * N, nullptr, c + g * M * N, nullptr,
-                                     nullptr, nullptr, nullptr};
+                                     nullptr, nullptr, nullptr, 0};
     }
     const int rc = Hq % 64 == 0 ? ftk::launch_cells_f16<false, 8, false, true>(list, M, K, Hq, s)
                                 : ftk::launch_cells_f16<false, 4, false, true>(list, M, K, Hq, s);

@@ -51,11 +51,11 @@ namespace ftk {
 
 int run_wavefront(const float* xs, const float* WU, const float* bias, const int* dil, float* hsss, float* csss,
                   int L, int T, int B, int H, hipStream_t s);
-int run_wavefront_f16(const void* xs, const void* WU, const float* bias, const int* dil, void* hsss, void* csss,
-                      int L, int T, int B, int H, void* packed, hipStream_t s);
+int run_wavefront_f16(const void* xs, const void* WU, const float* bias, const int* dil, const int* active, void* hsss,
+                      void* csss, int L, int T, int B, int H, void* packed, hipStream_t s);
 size_t split_stack_workspace_bytes(int L, int T, int B, int H);
-int run_wavefront_split(const float* xs, const float* WU, const float* bias, const int* dil, float* hsss, float* csss,
-                        int L, int T, int B, int H, void* ws, hipStream_t s);
+int run_wavefront_split(const float* xs, const float* WU, const float* bias, const int* dil, const int* active, float* hsss,
+                        float* csss, int L, int T, int B, int H, void* ws, hipStream_t s);
 
 constexpr int PH = 256;            // hidden size this kernel is specialised for
 constexpr int PK = 2 * PH;         // K of the gate GEMM
@@ -1050,7 +1050,7 @@ static int run_stack(const char* who, const float* xs, const float* WU, const fl
   // workspace the size query asks for, through the fp16-MFMA streaming kernel; else on fp32 MFMAs.
   if (H != PH && products_mode() == FTK_LSTM_PRODUCTS_F16X3 && ws && ws_bytes >= split_stack_workspace_bytes(L, T, B, H) &&
       (long long)B * H < (1ll << 29))
-    return run_wavefront_split(xs, WU, bias, dil, hsss, csss, L, T, B, H, ws, s);
+    return run_wavefront_split(xs, WU, bias, dil, active, hsss, csss, L, T, B, H, ws, s);
   return run_wavefront(xs, WU, bias, dil, hsss, csss, L, T, B, H, s);
 }
 
@@ -1120,7 +1120,7 @@ int ftk_stacked_lstm_f16(const void* xs, const void* WU, const float* bias, cons
     const size_t need = ftk_stacked_lstm_f16_workspace_bytes(L, T, B, H);
     if (!workspace || workspace_bytes < need)
       return fail(FTK_ERR_WORKSPACE, "%s: workspace of %zu bytes needed, %zu given", who, need, workspace ? workspace_bytes : (size_t)0);
-    return run_wavefront_f16(xs, WU, bias, dilations, hsss, csss, L, T, B, H, workspace, (hipStream_t)stream);
+    return run_wavefront_f16(xs, WU, bias, dilations, active_rows, hsss, csss, L, T, B, H, workspace, (hipStream_t)stream);
   }
   const void* fn = nullptr;
   int slots = 0;

@@ -164,7 +164,9 @@ int ftk_dilated_lstm_f32(const float* xs, const float* WU, const float* bias,
  * the dense [T,B,H] array with anything finite (zeros) in the dead places;
  * hsss/csss are written for the live (t, row) pairs, what the other places
  * hold afterwards is unspecified.  32-row blocks that have ended are skipped
- * by the persistent kernel; the per-stage fallback computes everything.
+ * by the persistent kernel; the streamed stacks of the other hidden sizes
+ * compute the live rows of every step only; the fp32-MFMA fallback computes
+ * everything.
  * dilations: host array or NULL (all 1).  Replaces the shrinking batch of
  * batched_cell (examples/stacked_rnn/stacked_rnn.py:45-51, hs_prev[0:xs.length])
  * over the layout of gen_dataset_time_major (examples/utils/data_utils.py:42-66).
@@ -187,9 +189,10 @@ int ftk_stacked_lstm_ragged_f32(const float* xs, const float* WU,
  * H = 512, 32 of H = 256 on 256 compute units) run as consecutive launches.
  * Every other shape (H = 1024, the third size of the sweep, among them) does
  * not fit on chip: its weights are streamed, one launch of the fp16 cell
- * kernel per stage of independent cells, which computes dead rows too (and
- * which is also the faster way for H = 512 stacks of more than 16 layers,
- * unless active_rows is given; FTK_LSTM_F16_STREAM=1 / 0 forces either); the
+ * kernel per stage of independent cells, on the rows that live at the cell's
+ * step (which is also the faster way for H = 512 stacks of more than 16
+ * layers, unless active_rows is given; FTK_LSTM_F16_STREAM=1 / 0 forces
+ * either); the
  * workspace then takes a re-laid copy of WU (ftk_stacked_lstm_f16_workspace_bytes
  * says how much for a shape).
  * dilations, active_rows: host arrays or NULL, as above.

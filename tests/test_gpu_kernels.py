@@ -235,6 +235,34 @@ def test_stacked_lstm_ragged_rows(core, products, L, T, B, dil, lengths):
     assert_lstm_close(torch.from_numpy(got_c), cr[:, live.numpy()], 'csss live places')
 
 
+@pytest.mark.parametrize('H,L,T,B,dil,lengths', [
+    (128, 3, 12, 300, None, 'linear'),         # two 256-row blocks; the second ends early, then rows of the first
+    (512, 2, 8, 64, None, 'two'),
+    (96, 3, 10, 40, [1, 2, 4], 'linear'),      # 32 hidden units per workgroup (three chunks in a row), dilated
+])
+def test_streamed_stack_ragged_rows(core, products, H, L, T, B, dil, lengths):
+    """The streamed stacks (hidden sizes other than 256) on a ragged batch: a cell computes the rows that live at
+    its step only; the poisoned dead places of xs must not reach a live place."""
+    xs, WU, bs = lstm_inputs(10, L, T, B, H, 1.0 / np.sqrt(4 * H))
+    lens = np.maximum(1, T - (np.arange(B) * T) // B) if lengths == 'linear' else np.where(np.arange(B) < B // 2, T, 3)
+    active = [int((lens > t).sum()) for t in range(T)]
+    clean = xs.copy()
+    for b in range(B):
+        clean[lens[b]:, b] = 0.0
+        xs[lens[b]:, b] = 1e30                                   # what a live place must never see
+    hsss, csss = core.stacked_lstm(dev(xs), dev(WU), dev(bs), dilations=dil, active_rows=active)
+    hr, cr = ko.stacked_lstm(clean, WU, bs, dilations=dil)
+    live = np.arange(T)[:, None] < lens[None, :]
+    assert_lstm_close(torch.from_numpy(hsss.cpu().numpy()[:, live]), hr[:, live], 'hsss live places')
+    assert_lstm_close(torch.from_numpy(csss.cpu().numpy()[:, live]), cr[:, live], 'csss live places')
+    if products == 'f16x3' and H % 64 == 0:
+        # fp16 storage through the same kernels
+        h16, c16 = core.stacked_lstm_f16(dev(clean.astype(np.float16)), dev(WU.astype(np.float16)), dev(bs), dilations=dil,
+                                         active_rows=active)
+        hr16, _ = ko.stacked_lstm_f16(clean.astype(np.float16), WU.astype(np.float16), bs, dil)
+        assert ko.max_rel_err(h16.float().cpu().numpy()[:, live], hr16.astype(np.float32)[:, live]) <= F16_TOL
+
+
 def test_stacked_lstm_ragged_rejects_unsorted_rows(core):
     H, L, T, B = 256, 1, 4, 32
     xs = torch.zeros((T, B, H), device='cuda'); WU = torch.zeros((L, 2 * H, 4 * H), device='cuda')
