@@ -1,10 +1,12 @@
 """Access operations over FractalTensors: index, zip, enumerate, product,
-last, join (kaleido/frontend/operations/fractaltensor/access.py:18-29).
+last, join and the windowed access patterns slide, window, shifted_slide,
+shifted_window (kaleido/frontend/operations/fractaltensor/access.py:18-29,
+246-531) that the reference's convolution and sparse-attention examples use.
 
-The windowed access patterns of the reference (slide, window, shifted_slide,
-shifted_window: access.py:246-531) serve its convolution and sparse-attention
-examples, which are outside the hot path built here; they raise
-NotImplementedError.
+The windowed patterns are restated from the reference's source; none of its
+tests holds an answer for them.  slide and shifted_slide (the two its examples
+call) follow the source to the letter, oddities included and named below;
+window follows its documented meaning where the source cannot mean what it does.
 """
 from __future__ import annotations
 
@@ -88,15 +90,131 @@ def join(x: FractalTensor, y: FractalTensor) -> FractalTensor:
     return out
 
 
-def _windowed(name):
-    def op(*args, **kwargs):
-        raise NotImplementedError(f'{name} belongs to the convolution / sparse-attention access patterns, '
-                                  'which this build does not cover.')
-    op.__name__ = name
-    return op
+def _window_span(window_size: int, dilation: int) -> int:
+    return (window_size - 1) * (dilation - 1) + window_size
 
 
-slide = _windowed('slide')
-window = _windowed('window')
-shifted_slide = _windowed('shifted_slide')
-shifted_window = _windowed('shifted_window')
+def _pick(x: FractalTensor, ids) -> FractalTensor:
+    items = [x[int(i)] for i in ids]
+    if not items:
+        raise IndexError('empty window')
+    return FractalTensor.from_tensors(*items) if isinstance(items[0], Tensor) else FractalTensor.from_fractaltensors(*items)
+
+
+def _copies(value, n: int) -> FractalTensor:
+    import copy
+    items = [copy.deepcopy(value) for _ in range(n)]
+    return FractalTensor.from_tensors(*items) if isinstance(value, Tensor) else FractalTensor.from_fractaltensors(*items)
+
+
+def slide(input: FractalTensor, window_size: int, stride: int, dilation: int, padding: int = None, padding_value=None):
+    """Windows of `window_size` items, `dilation` apart, every `stride` positions over the input padded on both
+    sides with `padding` copies of `padding_value`; depth grows by one (access.py:276-373).
+
+    As in the source, one more window follows the regular ones: everything from the position after the last
+    window's start to the end (access.py:346), so the result is ragged in general.
+    """
+    if window_size % 2 == 0:
+        raise ValueError('Even number of window size is not implemented yet.')
+    if not isinstance(input, FractalTensor):
+        raise TypeError(f'Expected FractalTensor, got {type(input).__name__}.')
+    if not isinstance(padding_value, (Tensor, FractalTensor)):
+        raise TypeError(f'Expected Tensor or FractalTensor, got {type(padding_value).__name__}.')
+    padded = input
+    if padding:
+        pad = _copies(padding_value, int(padding))
+        padded = join(join(pad, input), pad)
+    span = _window_span(window_size, dilation)
+    starts = list(range(0, len(padded) - span + 1, stride))
+    if not starts:
+        raise ValueError('the window does not fit the padded input')
+    slides = [_pick(padded, range(p, p + span, dilation)) for p in starts]
+    slides.append(_pick(padded, range(starts[-1] + 1, len(padded), dilation)))
+    return FractalTensor.from_fractaltensors(*slides)
+
+
+def _unzip(input):
+    """An Iterative of per-position tuples (what zip returns) as one FractalTensor per field (access.py:248-273)."""
+    if isinstance(input, FractalTensor):
+        return input
+    if not isinstance(input, Iterative):
+        raise TypeError(f'Expected FractalTensor or Iterative, got {type(input).__name__}')
+    if len(input) == 0:
+        raise ValueError('empty Iterative')
+    fields = []
+    for f in range(len(input[0])):
+        items = [input[j][f] for j in range(len(input))]
+        if isinstance(items[0], Tensor):
+            fields.append(FractalTensor.from_tensors(*items))
+        elif isinstance(items[0], FractalTensor):
+            fields.append(FractalTensor.from_fractaltensors(*items))
+        else:
+            raise TypeError('fields of the Iterative should be Tensors or FractalTensors.')
+    return fields
+
+
+def shifted_slide(input, window_size: int, dilation: int = 1):
+    """For every position the window centred on it, wrapping around at both ends; one result per field of a
+    zipped input (access.py:376-431; the call of examples/sparse_attention/sparse_attention.py:51).
+
+    The wrap is the source's: position x >= L maps to x - L, but x < 0 maps to x + L - 1 (access.py:384-390), one
+    short of the circular x + L.  A FractalTensor input is walked item by item, each item being slid (what
+    iterating the source's `xs` does), so it must be of depth 2 or more.
+    """
+    if window_size % 2 == 0:
+        raise ValueError('Even number of window size is not implemented yet.')
+    half = _window_span(window_size, dilation) // 2
+
+    def one(x: FractalTensor) -> FractalTensor:
+        if not isinstance(x, FractalTensor):
+            raise TypeError(f'Expected FractalTensor, got {type(x).__name__}.')
+        L = len(x)
+        wrap = lambda i: i + L - 1 if i < 0 else (i - L if i >= L else i)
+        return FractalTensor.from_fractaltensors(
+            *[_pick(x, [wrap(i) for i in range(pos - half, pos + half + 1, dilation)]) for pos in range(L)])
+
+    return [one(x) for x in _unzip(input)]
+
+
+def _as_index(index, length: int) -> int:
+    if isinstance(index, Tensor):
+        if index.data.numel() != 1:
+            raise ValueError('index should hold one element.')
+        index = int(index.data.reshape(-1)[0].item())
+    if index >= length:
+        raise IndexError(f'{index} exceeds length of the input.')
+    return int(index)
+
+
+def window(index, input: FractalTensor, window_size: int, dilation: int, padding_value=None) -> FractalTensor:
+    """The items in the window centred on item `index`, positions outside the input filled with copies of
+    `padding_value` (the meaning access.py:436-446 documents).
+
+    The source does not do that: it keeps only one side's padding when both are needed and starts every interior
+    window at position 0 (access.py:463-481); no caller exists in the reference.  This follows the documentation.
+    """
+    if not isinstance(input, FractalTensor):
+        raise TypeError(f'Expected FractalTensor, got {type(input).__name__}.')
+    i = _as_index(index, len(input))
+    half = _window_span(window_size, dilation) // 2
+    L = len(input)
+    picked = []
+    import copy
+    for p in range(i - half, i + half + 1, dilation):
+        if 0 <= p < L:
+            picked.append(input[p])
+        else:
+            if not isinstance(padding_value, (Tensor, FractalTensor)):
+                raise TypeError('the window leaves the input and no padding_value is given.')
+            picked.append(copy.deepcopy(padding_value))
+    return FractalTensor.from_tensors(*picked) if isinstance(picked[0], Tensor) else FractalTensor.from_fractaltensors(*picked)
+
+
+def shifted_window(index, input: FractalTensor, window_size: int, dilation: int) -> FractalTensor:
+    """The items in the window centred on item `index`, wrapping around circularly (access.py:492-528)."""
+    if not isinstance(input, FractalTensor):
+        raise TypeError(f'Expected FractalTensor, got {type(input).__name__}.')
+    i = _as_index(index, len(input))
+    half = _window_span(window_size, dilation) // 2
+    L = len(input)
+    return _pick(input, [(p + L) % L for p in range(i - half, i + half + 1, dilation)])

@@ -260,6 +260,102 @@ def test_flatten_shapes(dim):                           # test_flatten.py:39-59
         assert torch.equal(y.data[3:6], x[0][1].data)
 
 
+# ---- windowed access (operations/fractaltensor/access.py:246-531; no reference test holds an answer) ------
+
+def _vals(ft):
+    return [int(t.data.item()) for t in ft]
+
+
+def _minus_one():
+    pv = FractalTensor.from_pylist([0])[0]
+    pv.data = pv.data * 0 - 1
+    return pv
+
+
+def test_slide_windows_and_the_tail_window():
+    x = FractalTensor.from_pylist(list(range(9)))
+    s = ops.slide(x, 3, 1, 1, padding=1, padding_value=_minus_one())
+    assert s.depth == 2
+    got = [_vals(w) for w in s]
+    # padded = [-1, 0..8, -1]; nine regular windows, as torch's unfold gives them ...
+    padded = torch.tensor([-1] + list(range(9)) + [-1])
+    assert got[:9] == padded.unfold(0, 3, 1).tolist()
+    # ... and the source's one more: from the position after the last start to the end (access.py:346)
+    assert got[9] == [8, -1]
+    s = ops.slide(x, 3, 2, 2, padding=0, padding_value=_minus_one())
+    assert [_vals(w) for w in s] == [[0, 2, 4], [2, 4, 6], [4, 6, 8], [5, 7]]
+    with pytest.raises(ValueError):
+        ops.slide(x, 4, 1, 1, padding=1, padding_value=_minus_one())
+    with pytest.raises(TypeError):
+        ops.slide(x, 3, 1, 1, padding=1, padding_value=None)
+    with pytest.raises(TypeError):
+        ops.slide([1, 2, 3], 3, 1, 1, padding=1, padding_value=_minus_one())
+
+
+def test_shifted_slide_wraps_as_the_source_does():
+    ks = FractalTensor.from_pylist(list(range(6)))
+    vs = FractalTensor.from_pylist(list(range(10, 16)))
+    wk, wv = ops.shifted_slide(ops.zip(ks, vs), window_size=3)
+    # interior positions: the plain centred window; right end: circular; left end: x < 0 -> x + L - 1
+    # (access.py:384-390), i.e. position 0 sees item 4, not item 5
+    assert [_vals(w) for w in wk] == [[4, 0, 1], [0, 1, 2], [1, 2, 3], [2, 3, 4], [3, 4, 5], [4, 5, 0]]
+    assert [_vals(w) for w in wv] == [[14, 10, 11], [10, 11, 12], [11, 12, 13], [12, 13, 14], [13, 14, 15], [14, 15, 10]]
+    # window 5, dilation 2 (the call of examples/sparse_attention/sparse_attention.py:51): span 9, every other item
+    xs = FractalTensor.from_pylist(list(range(12)))
+    w, _ = ops.shifted_slide(ops.zip(xs, xs), window_size=5, dilation=2)
+    assert _vals(w[6]) == [2, 4, 6, 8, 10] and _vals(w[11]) == [7, 9, 11, 1, 3] and _vals(w[0]) == [7, 9, 0, 2, 4]
+    # a FractalTensor input is walked item by item, each item slid (what the source's loop over `xs` does)
+    nested = FractalTensor.from_pylist([[0, 1, 2, 3], [4, 5, 6, 7, 8]])
+    per_item = ops.shifted_slide(nested, window_size=3)
+    assert [_vals(win) for win in per_item[1]] == [[7, 4, 5], [4, 5, 6], [5, 6, 7], [6, 7, 8], [7, 8, 4]]
+    with pytest.raises(TypeError):
+        ops.shifted_slide(xs, window_size=3)
+    with pytest.raises(ValueError):
+        ops.shifted_slide(ops.zip(ks, vs), window_size=4)
+
+
+def test_window_and_shifted_window():
+    x = FractalTensor.from_pylist(list(range(9)))
+    pv = _minus_one()
+    assert _vals(ops.window(0, x, 3, 1, pv)) == [-1, 0, 1]
+    assert _vals(ops.window(8, x, 5, 1, pv)) == [6, 7, 8, -1, -1]
+    assert _vals(ops.window(4, x, 3, 2, pv)) == [2, 4, 6]
+    assert _vals(ops.window(1, x, 3, 2, pv)) == [-1, 1, 3]
+    for i in range(2, 7):                                   # interior: a plain slice
+        assert _vals(ops.window(i, x, 5, 1, pv)) == list(range(i - 2, i + 3))
+        assert _vals(ops.shifted_window(i, x, 5, 1)) == list(range(i - 2, i + 3))
+    assert _vals(ops.shifted_window(0, x, 3, 1)) == [8, 0, 1]
+    assert _vals(ops.shifted_window(8, x, 5, 1)) == [6, 7, 8, 0, 1]
+    idx = Tensor((1,), kaleido.int32)
+    idx.data = torch.LongTensor([7])
+    assert _vals(ops.shifted_window(idx, x, 3, 1)) == [6, 7, 8]
+    with pytest.raises(IndexError):
+        ops.window(9, x, 3, 1, pv)
+    with pytest.raises(TypeError):
+        ops.shifted_window(0, [1, 2], 3, 1)
+
+
+def test_windowed_attention_program_over_shifted_slide():
+    """The windowed part of the reference's sparse attention (examples/sparse_attention/sparse_attention.py:25-38,
+    51-53): every token attends to the window shifted_slide gives it; against a direct softmax(q K_w^T) V_w."""
+    torch.manual_seed(3)
+    S, D, W = 10, 8, 3
+    mk = lambda: FractalTensor.from_tensors(*[Tensor.from_tensor(torch.randn(1, D)) for _ in range(S)])
+    q, k, v = mk(), mk(), mk()
+    wk, wv = ops.shifted_slide(ops.zip(k, v), window_size=W)
+
+    def attn(x):
+        qt, ks, vs = x
+        return ops.softmax(qt @ ops.flatten(ks).T, dim=1) @ ops.flatten(vs)
+
+    out = ops.map(attn, ops.zip(q, wk, wv))
+    K = torch.cat([t.data for t in k]); V = torch.cat([t.data for t in v])
+    for pos in range(S):
+        ids = [(i + S - 1 if i < 0 else (i - S if i >= S else i)) for i in range(pos - 1, pos + 2)]
+        ref = torch.softmax(q[pos].data @ K[ids].T, dim=1) @ V[ids]
+        assert torch.allclose(out[pos].data, ref, atol=1e-6)
+
+
 def test_arange_slices_and_constants():                 # test_constants.py:16-34
     for args in ((11,), (5, 7), (5, 24, 3)):
         ft = ops.slices(ops.arange(*args), dim=0)
