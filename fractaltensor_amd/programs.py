@@ -1,4 +1,4 @@
-"""The three hot-path model programs written against the kaleido operator API.
+"""The hot-path model programs, and the grid RNN next to them, written against the kaleido operator API.
 
 These are the eager counterparts of the reference's example programs: every
 cell is a handful of torch calls on one sample and map / scan / fold are
@@ -12,6 +12,8 @@ baseline that bench.py times on configuration 1.
                    initialised as the README's maths requires (max -inf, sum 0, o 0;
                    the example seeds (sum, max, o) into a (max, sum, o) signature) and
                    an explicit score scale
+  grid RNN         examples/grid_rnn/grid_rnn.py:40-137 (one sample: source x target grid,
+                   two tanh cells per position sharing the state of both directions)
 """
 from __future__ import annotations
 
@@ -120,3 +122,55 @@ def _attend_query_block(q: Tensor, ks: FractalTensor, vs: FractalTensor, scale: 
 def flash_attention(qsss: FractalTensor, ksss: FractalTensor, vsss: FractalTensor, scale: float) -> FractalTensor:
     per_head = lambda qkv: ops.map(lambda q: _attend_query_block(q, qkv[1], qkv[2], scale), qkv[0])
     return ops.map(lambda sample: ops.map(per_head, ops.zip(*sample)), ops.zip(qsss, ksss, vsss))
+
+
+# ---- grid RNN -----------------------------------------------------------------
+
+def make_grid_params(depth: int, hidden: int, seed: int, scale: float = None):
+    """Per block the parameters of the two directions: (i2h [2H, H], h2h [H, H], bias [1, H]) each."""
+    gen = torch.Generator().manual_seed(seed)
+    scale = scale if scale is not None else 1.0 / (3 * hidden) ** 0.5
+    mk = lambda *shape: Tensor.from_tensor((torch.rand(shape, generator=gen) * 2 - 1) * scale)
+    cell = lambda: (mk(2 * hidden, hidden), mk(hidden, hidden), mk(1, hidden))
+    return [(cell(), cell()) for _ in range(depth)]
+
+
+def _vanilla_cell(state: Tensor, cur: Tensor, i2h: Tensor, h2h: Tensor, bias: Tensor) -> Tensor:
+    return ops.tanh(cur @ i2h + state @ h2h + bias)
+
+
+def _grid_cell(state, cur_input, block):
+    """state: the outputs (h_x, h_y) of the position before along the inner direction, of which h_y is used;
+    cur_input: (h_x of the same inner position one outer step before, (x_t, y_t) from the block below)."""
+    _, state_y = state
+    state_x, (x_t, y_t) = cur_input
+    px, py = block
+    s = ops.cat([state_x, state_y], dim=1)
+    return _vanilla_cell(x_t, s, *px), _vanilla_cell(y_t, s, *py)
+
+
+def _grid_row(state, cur_input, block, hidden: int):
+    """One outer step: a scan along the inner direction; state = the row of outputs one outer step before."""
+    state_xs, _ = state
+    zero = ops.zeros(shape=(1, hidden), device='cpu')
+    return ops.scan(lambda s, x: _grid_cell(s, x, block), ops.zip(state_xs, ops.zip(*cur_input)), initializer=(zero, zero))
+
+
+def _grid_block(inputs, block, hidden: int):
+    """One block of the stack: a scan along the outer direction over rows of (x, y) inputs."""
+    zeros = ops.repeat(ops.zeros(shape=(1, hidden), device='cpu'), len(inputs[0][0]))
+    ys1, ys2 = ops.scan(lambda s, x: _grid_row(s, x, block, hidden), inputs, initializer=(zeros, zeros))
+    return ops.zip(ys1, ys2)
+
+
+def grid_rnn(src: FractalTensor, trg: FractalTensor, params, hidden: int):
+    """Stacked grid RNN over one (source, target) pair: src [S] and trg [Tg] of [1, H] Tensors.
+    Returns (h_x, h_y), each depth-2 [Tg][S] of [1, H]: the last block's outputs at every grid position.
+    Position (i, j) of a block computes, with s = [h_x(i-1, j) | h_y(i, j-1)] (zeros outside the grid),
+      h_x(i, j) = tanh(s @ i2h_x + x_in(i, j) @ h2h_x + b_x),  h_y(i, j) = tanh(s @ i2h_y + y_in(i, j) @ h2h_y + b_y),
+    where the first block's inputs are x_in(i, j) = src[j], y_in(i, j) = trg[i] and every other block's are
+    the outputs of the block below."""
+    blocks = kaleido.Iterative.make_iterative(*params)
+    yss1, yss2 = ops.fold(lambda inputs, block: _grid_block(inputs, block, hidden), blocks,
+                          initializer=ops.zip(*ops.product(src, trg)))
+    return yss1, yss2

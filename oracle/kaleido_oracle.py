@@ -431,3 +431,39 @@ def flash_attention_blockwise(Q, K, V, scale, block_q=64, block_kv=64, dtype=np.
             prev_m, prev_l = new_m, new_l
         out[q0:q0 + block_q] = prev_o
     return out
+
+
+# ------------------------------------------------------------------ grid RNN
+
+def grid_rnn(src, trg, params, dtype=np.float64):
+    """Stacked grid RNN of examples/grid_rnn/grid_rnn.py:40-137 over one (source, target) pair.
+
+    src [S, H], trg [Tg, H]; params: per block ((i2h_x [2H,H], h2h_x [H,H], b_x [H]), (i2h_y, h2h_y, b_y)).
+    The outer scan runs over the target positions i, the inner one over the source positions j
+    (product(src, trg) puts src along the inner level, access.py:206-244; direction_x scans the outer level,
+    grid_rnn.py:99-113, direction_y the inner one, :78-95).  grid_cell (:53-74) forms s = [state_x | state_y]
+    with state_x = h_x of position (i-1, j) and state_y = h_y of position (i, j-1), zeros outside the grid,
+    and h_x = tanh(s @ i2h_x + x_t @ h2h_x + b_x), h_y = tanh(s @ i2h_y + y_t @ h2h_y + b_y)
+    (vanilla_cell is called with the input as its `state` argument and s as `cur`, :47-50, 71-73).
+    Returns h_x, h_y [Tg, S, H] of the last block.
+    """
+    src = np.asarray(src, dtype=dtype)
+    trg = np.asarray(trg, dtype=dtype)
+    S, H = src.shape
+    Tg = trg.shape[0]
+    x_in = np.broadcast_to(src[None, :, :], (Tg, S, H)).copy()
+    y_in = np.broadcast_to(trg[:, None, :], (Tg, S, H)).copy()
+    for (px, py) in params:
+        i2h_x, h2h_x, b_x = (np.asarray(p, dtype=dtype) for p in px)
+        i2h_y, h2h_y, b_y = (np.asarray(p, dtype=dtype) for p in py)
+        hx = np.zeros((Tg, S, H), dtype=dtype)
+        hy = np.zeros((Tg, S, H), dtype=dtype)
+        for i in range(Tg):
+            for j in range(S):
+                state_x = hx[i - 1, j] if i > 0 else np.zeros(H, dtype=dtype)
+                state_y = hy[i, j - 1] if j > 0 else np.zeros(H, dtype=dtype)
+                s = np.concatenate([state_x, state_y])
+                hx[i, j] = np.tanh(s @ i2h_x + x_in[i, j] @ h2h_x + b_x.reshape(-1))
+                hy[i, j] = np.tanh(s @ i2h_y + y_in[i, j] @ h2h_y + b_y.reshape(-1))
+        x_in, y_in = hx, hy
+    return x_in, y_in

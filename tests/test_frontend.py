@@ -441,6 +441,35 @@ def test_eager_flash_attention_matches_oracle():
     np.testing.assert_allclose(dense(out), ref, atol=2e-6)
 
 
+def test_eager_grid_rnn_matches_oracle():
+    """The reference's fourth model program (examples/grid_rnn/grid_rnn.py) through the frontend: nested scans
+    with tuple state over zip(product(src, trg)), folded over the blocks, against the numpy statement of the
+    recurrence; and a hand check of the first block's corner, which has no neighbours."""
+    H, S, Tg, depth = 8, 4, 3, 2
+    torch.manual_seed(11)
+    mk = lambda n: FractalTensor.from_tensors(*[Tensor.from_tensor(torch.randn(1, H)) for _ in range(n)])
+    src, trg = mk(S), mk(Tg)
+    params = programs.make_grid_params(depth, H, seed=5)
+    hx, hy = programs.grid_rnn(src, trg, params, H)
+    assert hx.depth == 2 and len(hx) == Tg and len(hx[0]) == S
+    np_params = [tuple(tuple(t.data.numpy() for t in cell) for cell in block) for block in params]
+    s_np = np.stack([t.data.numpy()[0] for t in src]); t_np = np.stack([t.data.numpy()[0] for t in trg])
+    rx, ry = ko.grid_rnn(s_np, t_np, np_params)
+    for i in range(Tg):
+        for j in range(S):
+            np.testing.assert_allclose(hx[i][j].data.numpy()[0], rx[i, j], rtol=1e-5, atol=1e-6)
+            np.testing.assert_allclose(hy[i][j].data.numpy()[0], ry[i, j], rtol=1e-5, atol=1e-6)
+    # one block, corner (0, 0): no state, so h_x = tanh(src[0] @ h2h_x + b_x), h_y = tanh(trg[0] @ h2h_y + b_y)
+    one = programs.make_grid_params(1, H, seed=6)
+    cx, cy = ko.grid_rnn(s_np, t_np, [tuple(tuple(t.data.numpy() for t in cell) for cell in one[0])])
+    (i2hx, h2hx, bx), (i2hy, h2hy, by) = one[0]
+    np.testing.assert_allclose(cx[0, 0], np.tanh(s_np[0] @ h2hx.data.numpy() + bx.data.numpy()[0]), rtol=1e-5, atol=1e-6)
+    np.testing.assert_allclose(cy[0, 0], np.tanh(t_np[0] @ h2hy.data.numpy() + by.data.numpy()[0]), rtol=1e-5, atol=1e-6)
+    # and position (1, 2) from its two neighbours
+    s12 = np.concatenate([cx[0, 2], cy[1, 1]])
+    np.testing.assert_allclose(cx[1, 2], np.tanh(s12 @ i2hx.data.numpy() + s_np[2] @ h2hx.data.numpy() + bx.data.numpy()[0]), rtol=1e-5, atol=1e-6)
+
+
 def test_fused_paths_refuse_cpu_inputs():
     Wss, Uss, bss = programs.make_lstm_params(1, 32, 0.1, seed=1)
     xss = programs.make_sequence_batch(2, 2, 32, seed=2)
