@@ -20,6 +20,8 @@ import os
 import sys
 import time
 
+import numpy as np
+
 ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
@@ -209,6 +211,81 @@ def bench_softmax(torch, core, steps, warmup, cpu):
         dt = time.perf_counter() - t0
         res['cpu_baseline'] = {'value': n / dt, 'unit': 'rows/s', 'cores': 1, 'kind': 'port',
                                'sample': f'{n} rows through oracle/oracle.c in {dt:.2f} s'}
+    return res
+
+
+def _grid_torch_planes(torch, xs, ys, W, U, b, D, L, B, H):
+    """The reference's schedule for the grid RNN on torch ops: per plane d+i+j one gather of the four operands
+    and of the plane's weights, batched products, tanh, one scatter (regions/region8.h:61-310), with the index
+    tensors built beforehand.  Level 0 of the padded array holds the first block's inputs, level d+1 block d's
+    outputs; row/column 0 of every level is the zero border."""
+    A = torch.zeros((D + 1, L + 1, L + 1, 2, B, H), device='cuda')
+    A[0, 1:, 1:, 0] = xs[:, None]
+    A[0, 1:, 1:, 1] = ys[None, :]
+    flat = A.view(-1, B, H)
+    at = lambda lvl, i, j, w: ((lvl * (L + 1) + i) * (L + 1) + j) * 2 + w
+    planes = []
+    for m in range(D + 2 * L - 2):
+        pos = [(d, i, m - d - i) for d in range(D) for i in range(L) if 0 <= m - d - i < L]
+        ix = lambda f: torch.tensor([f(d, i, j) for d, i, j in pos], device='cuda')
+        planes.append((ix(lambda d, i, j: at(d, i + 1, j + 1, 0)), ix(lambda d, i, j: at(d, i + 1, j + 1, 1)),
+                       ix(lambda d, i, j: at(d + 1, i, j + 1, 0)), ix(lambda d, i, j: at(d + 1, i + 1, j, 1)),
+                       ix(lambda d, i, j: at(d + 1, i + 1, j + 1, 0)), ix(lambda d, i, j: at(d + 1, i + 1, j + 1, 1)),
+                       ix(lambda d, i, j: d)))
+
+    def run():
+        for pxi, pyi, sxi, syi, oxi, oyi, dsel in planes:
+            s = torch.cat([flat[sxi], flat[syi]], dim=2)
+            su = torch.baddbmm(b[dsel], s, U[dsel])
+            w = W[dsel]
+            flat[oxi] = torch.tanh(torch.baddbmm(su, flat[pxi], w))
+            flat[oyi] = torch.tanh(torch.baddbmm(su, flat[pyi], w))
+    return run, A
+
+
+def bench_grid_rnn(torch, core, steps, warmup, cpu):
+    """The reference's grid benchmark shape (stacked_grid_rnn.cu:108-118, run.sh:7: batch 32, depth 32, hidden 256,
+    both lengths 10; shared parameters, a bias row per batch row), fp32, one launch per plane."""
+    D, L, B, H = 32, 10, 32, 256
+    gen = torch.Generator(device='cpu').manual_seed(1234)
+    u = lambda *shape, s=1.0: ((torch.rand(shape, generator=gen) * 2 - 1) * s).cuda()
+    sc = 2.0 / (3 * H) ** 0.5
+    xs, ys = u(L, B, H), u(L, B, H)
+    W, U, b = u(D, H, H, s=sc), u(D, 2 * H, H, s=sc), u(D, B, H, s=0.2)
+    out = torch.empty((D, L, L, 2, B, H), device='cuda')
+    ci = ctypes.c_int
+    run = lambda: core._check(core.lib.ftk_grid_rnn_f32(
+        core._ptr(xs), core._ptr(ys), core._ptr(W), core._ptr(U), core._ptr(b), core._ptr(W), core._ptr(U), core._ptr(b),
+        core._ptr(out), ci(D), ci(L), ci(L), ci(B), ci(H), ci(B), ci(0), core._stream()))
+    ms, _ = _events_ms(torch, run, steps, warmup)
+    base, A = _grid_torch_planes(torch, xs, ys, W, U, b, D, L, B, H)
+    ms_t, _ = _events_ms(torch, base, max(2, steps // 5), 1)
+    err = (A[1:, 1:, 1:] - out).abs().max().item()
+    npos = D * L * L
+    # k per position: H of input per direction; H per neighbour that exists, once (shared parameters: the state
+    # product serves both directions)
+    ksum = sum(H * (2 + (i > 0) + (j > 0)) for i in range(L) for j in range(L)) * D
+    flop = 2.0 * B * H * ksum
+    res = {
+        'metric': 'grid positions/s', 'value': npos / ms * 1e3, 'unit': 'positions/s', 'ms_per_step': ms, 'dtype': 'f32',
+        'config': {'workload': 'stacked grid RNN forward (grid_lstm/stacked_grid_rnn.cu), one launch per plane d+i+j',
+                   'depth': D, 'src_len': L, 'trg_len': L, 'batch': B, 'hidden': H, 'planes': D + 2 * L - 2},
+        'roofline': {'bound': 'mfma', 'achieved': flop / ms / 1e9, 'peak': PEAK_F32_MATRIX_TFLOPS, 'unit': 'TFLOP/s',
+                     'frac': flop / ms / 1e9 / PEAK_F32_MATRIX_TFLOPS, 'traffic': None, 'kernel': 'grid_rnn_plane_kernel',
+                     'note': 'the whole forward (50 dependent launches) against the fp32 MFMA peak; planes near the '
+                             'corners hold a handful of positions, so the chain of launches, not the matrix rate, bounds it'},
+        'torch_per_plane_gather_bmm_scatter': {'ms_per_step': ms_t, 'speedup': ms_t / ms, 'max_abs_diff': err},
+    }
+    if cpu:
+        from oracle import kaleido_oracle as ko
+        Dc = 2
+        t0 = time.perf_counter()
+        ref = ko.grid_rnn_batched(xs.cpu().numpy(), ys.cpu().numpy(), W[:Dc].cpu().numpy(), U[:Dc].cpu().numpy(), b[:Dc].cpu().numpy(),
+                                  W[:Dc].cpu().numpy(), U[:Dc].cpu().numpy(), b[:Dc].cpu().numpy(), dtype=np.float32)
+        dt = time.perf_counter() - t0
+        res['cpu_baseline'] = {'value': Dc * L * L / dt, 'unit': 'positions/s', 'cores': 1, 'kind': 'port',
+                               'sample': f'the first {Dc} blocks ({Dc * L * L} positions) through the numpy oracle in {dt:.2f} s',
+                               'max_abs_diff_vs_gpu': float(np.abs(ref - out[:Dc].cpu().numpy()).max())}
     return res
 
 
@@ -515,7 +592,7 @@ def main():
     ap.add_argument('--gpus', type=int, default=1)
     ap.add_argument('--steps', type=int, default=50)
     ap.add_argument('--warmup', type=int, default=10)
-    ap.add_argument('--workload', default='b2b', choices=['b2b', 'attention', 'stacked_lstm', 'dilated_lstm', 'lstm_f16_h256', 'lstm_f16_h512', 'lstm_f16_h1024', 'lstm_f32_h512', 'lstm_f32_h1024', 'gemm', 'online_softmax', 'embedding', 'copy'])
+    ap.add_argument('--workload', default='b2b', choices=['b2b', 'attention', 'stacked_lstm', 'dilated_lstm', 'lstm_f16_h256', 'lstm_f16_h512', 'lstm_f16_h1024', 'lstm_f32_h512', 'lstm_f32_h1024', 'gemm', 'online_softmax', 'embedding', 'grid_rnn', 'copy'])
     ap.add_argument('--no-extras', action='store_true', help='measure only the chosen workload')
     ap.add_argument('--no-cpu', action='store_true', help='skip the CPU baseline leg')
     ap.add_argument('--no-baselines', action='store_true',
@@ -547,6 +624,7 @@ def main():
         'gemm': lambda s, w, c: bench_gemm(torch, core, max(5, s // 5), max(2, w // 5), c),
         'online_softmax': lambda s, w, c: bench_softmax(torch, core, s, w, c),
         'embedding': lambda s, w, c: bench_embedding(torch, core, s, w, c),
+        'grid_rnn': lambda s, w, c: bench_grid_rnn(torch, core, max(5, s // 2), max(2, w // 2), c),
     }
     if args.workload == 'copy':
         runners = {'copy': lambda s, w, c: bench_copy(torch, core, s, w, c)}

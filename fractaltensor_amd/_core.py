@@ -23,6 +23,7 @@ EXPORTS = (
     'ftk_stacked_lstm_wavefront_f32', 'ftk_stacked_lstm_ragged_f32', 'ftk_lstm_set_products', 'ftk_lstm_get_products',
     'ftk_stacked_lstm_f16_workspace_bytes', 'ftk_stacked_lstm_f16',
     'ftk_b2b_gemm_f16', 'ftk_b2b_gemm_rowmajor_f16', 'ftk_gemm_f16', 'ftk_batched_gemm_f16', 'ftk_flash_attn_f16', 'ftk_online_softmax_f32', 'ftk_embedding_gather_f32',
+    'ftk_grid_rnn_f32',
     'ftk_debug_read_fa_trace',
 )
 
@@ -446,3 +447,39 @@ def online_softmax(x) -> torch.Tensor:
     y = torch.empty_like(x)
     _check(lib.ftk_online_softmax_f32(_ptr(x), _ptr(y), ctypes.c_int(rows), ctypes.c_int(cols), _stream()))
     return y
+
+
+def grid_rnn(xs, ys, Wx, Ux, bx, Wy, Uy, by, crossed: bool = False, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Stacked grid RNN, fp32.  W* [D, H, H], U* [D, 2H, H], biases [D, 1 or B, H] or both None.
+    crossed=False: xs [L1, B, H] feeds the first grid axis, ys [L2, B, H] the second (the layout of the
+    reference's grid benchmark); crossed=True: xs [L2, B, H] is indexed by the second axis and ys [L1, B, H] by the
+    first (the layout of its frontend program).  Returns hsss [D, L1, L2, 2, B, H]: h_x at index 0, h_y at 1."""
+    for name, t in (('xs', xs), ('ys', ys), ('Wx', Wx), ('Ux', Ux), ('Wy', Wy), ('Uy', Uy)):
+        _req(t, torch.float32, name)
+    if xs.dim() != 3 or ys.dim() != 3 or xs.shape[1:] != ys.shape[1:]:
+        raise ValueError(f'xs and ys must be [L, B, H] with equal B and H, got {tuple(xs.shape)} and {tuple(ys.shape)}')
+    _, B, H = xs.shape
+    L1, L2 = (ys.shape[0], xs.shape[0]) if crossed else (xs.shape[0], ys.shape[0])
+    D = Wx.shape[0]
+    for name, t, shape in (('Wx', Wx, (D, H, H)), ('Wy', Wy, (D, H, H)), ('Ux', Ux, (D, 2 * H, H)), ('Uy', Uy, (D, 2 * H, H))):
+        if tuple(t.shape) != shape:
+            raise ValueError(f'{name} must be {shape}, got {tuple(t.shape)}')
+    if (bx is None) != (by is None):
+        raise ValueError('give both biases or neither')
+    bias_rows = 1
+    if bx is not None:
+        _req(bx, torch.float32, 'bx')
+        _req(by, torch.float32, 'by')
+        bias_rows = bx.shape[1]
+        if tuple(bx.shape) != (D, bias_rows, H) or bx.shape != by.shape or bias_rows not in (1, B):
+            raise ValueError(f'biases must both be [D, 1 or B, H], got {tuple(bx.shape)} and {tuple(by.shape)}')
+    if out is None:
+        out = torch.empty((D, L1, L2, 2, B, H), dtype=torch.float32, device=xs.device)
+    else:
+        _req(out, torch.float32, 'out')
+        if tuple(out.shape) != (D, L1, L2, 2, B, H):
+            raise ValueError(f'out must be {(D, L1, L2, 2, B, H)}, got {tuple(out.shape)}')
+    _check(lib.ftk_grid_rnn_f32(_ptr(xs), _ptr(ys), _ptr(Wx), _ptr(Ux), _ptr(bx), _ptr(Wy), _ptr(Uy), _ptr(by), _ptr(out),
+                                ctypes.c_int(D), ctypes.c_int(L1), ctypes.c_int(L2), ctypes.c_int(B), ctypes.c_int(H),
+                                ctypes.c_int(bias_rows), ctypes.c_int(1 if crossed else 0), _stream()))
+    return out

@@ -1,0 +1,258 @@
+// Stacked grid RNN for gfx950, fp32: every position (d, i, j) of a depth x first-axis x second-axis grid holds two
+// tanh cells that share one state,
+//   s        = [ h_x(d, i-1, j) | h_y(d, i, j-1) ]                     (zeros outside the grid)
+//   h_x(d,i,j) = tanh(x_in @ Wx[d] + s @ Ux[d] + bx[d]),   h_y(d,i,j) = tanh(y_in @ Wy[d] + s @ Uy[d] + by[d])
+// with (x_in, y_in) = (h_x, h_y)(d-1, i, j) above the first block and the two input sequences in it.
+//
+// Schedule.  Position (d, i, j) needs (d-1, i, j), (d, i-1, j) and (d, i, j-1), so all positions of one
+// anti-diagonal plane m = d + i + j are independent: one launch per plane, D + L1 + L2 - 2 launches, each batched
+// over the plane's positions.  Nothing is gathered or scattered: a workgroup finds its position from its index
+// and reads the three neighbours where they lie in the output array.
+//
+// Tiling.  A workgroup owns 32 batch rows x 32 hidden units of one position, for both directions, and splits the
+// work into products of K = H, one per wave: x_in @ W, y_in @ W, state_x @ U[:H], state_y @ U[H:] when the two
+// directions share their parameters (four waves; the state products are computed once and serve both), six
+// products otherwise.  A product whose state lies outside the grid is skipped.  Each wave runs its product on
+// v_mfma_f32_32x32x2_f32 straight from global memory -- no operand is used by a second wave of the workgroup, so
+// LDS staging would only add barriers -- with the operands of the next three k chunks of 32 in registers.  Within a
+// chunk the k index is permuted so that a lane's activation values are 64 contiguous bytes: step (q, e) uses
+// k = 4q + e for lanes 0-31 and k = 16 + 4q + e for lanes 32-63.  The products are added through LDS before bias
+// and tanh.
+//
+// Placement.  Workgroups are numbered position-major, unit block fastest, and ids go round the eight XCDs: with
+// eight unit blocks (H = 256) an XCD only ever touches one 32-column slice of every block's parameters.  (Running
+// the positions of block d on XCD d % 8 instead, so that an XCD touches the parameters of four blocks only, was
+// measured and is slower: the planes' positions do not divide evenly over the blocks.)
+#include "ftk_common.h"
+
+namespace ftk {
+
+struct GridArgs {
+  const float* xs;   // [L1 or L2, B, H]
+  const float* ys;   // [L2 or L1, B, H]
+  const float* W[2];     // [D, H, H]   per direction
+  const float* U[2];     // [D, 2H, H]
+  const float* bias[2];  // [D, bias_rows, H] or nullptr
+  float* hsss;           // [D, L1, L2, 2, B, H]
+  int D, L1, L2, B, H;
+  int bias_rows;  // 1: one row for the whole batch, B: a row per batch row
+  int crossed;    // 0: x_in = xs[i], y_in = ys[j];  1: x_in = xs[j], y_in = ys[i]
+  int m;          // the plane d + i + j of this launch
+};
+
+constexpr int GKC = 32;  // k chunk
+
+// Number of positions with d + i + j = m, and the z-th of them in (d, i) order.
+__host__ __device__ inline int plane_positions(int D, int L1, int L2, int m, int z, int* d_out, int* i_out) {
+  int n = 0;
+  const int dlo = m - (L1 - 1) - (L2 - 1) > 0 ? m - (L1 - 1) - (L2 - 1) : 0;
+  const int dhi = m < D - 1 ? m : D - 1;
+  for (int d = dlo; d <= dhi; ++d) {
+    const int r = m - d;
+    const int ilo = r - (L2 - 1) > 0 ? r - (L2 - 1) : 0;
+    const int ihi = r < L1 - 1 ? r : L1 - 1;
+    const int cnt = ihi - ilo + 1;
+    if (cnt <= 0) continue;
+    if (z >= n && z < n + cnt) {
+      *d_out = d;
+      *i_out = ilo + (z - n);
+    }
+    n += cnt;
+  }
+  return n;
+}
+
+struct ChunkRegs {
+  float4 a[4];
+  float b[16];
+};
+
+// One k chunk of a product: lane (jl, hh) holds activation row jl, k = 16*hh .. 16*hh+15, and column jl of the
+// weight rows with the same k.
+__device__ __forceinline__ void load_chunk(ChunkRegs& r, const float* __restrict__ arow, const float* __restrict__ wcol,
+                                           int H, int c) {
+#pragma unroll
+  for (int q = 0; q < 4; ++q) r.a[q] = *reinterpret_cast<const float4*>(arow + c * GKC + 4 * q);
+#pragma unroll
+  for (int e = 0; e < 16; ++e) r.b[e] = wcol[(size_t)(c * GKC + e) * H];
+}
+
+__device__ __forceinline__ void mfma_chunk(v16f& acc, const ChunkRegs& r) {
+#pragma unroll
+  for (int q = 0; q < 4; ++q) {
+    acc = __builtin_amdgcn_mfma_f32_32x32x2f32(r.a[q].x, r.b[4 * q + 0], acc, 0, 0, 0);
+    acc = __builtin_amdgcn_mfma_f32_32x32x2f32(r.a[q].y, r.b[4 * q + 1], acc, 0, 0, 0);
+    acc = __builtin_amdgcn_mfma_f32_32x32x2f32(r.a[q].z, r.b[4 * q + 2], acc, 0, 0, 0);
+    acc = __builtin_amdgcn_mfma_f32_32x32x2f32(r.a[q].w, r.b[4 * q + 3], acc, 0, 0, 0);
+  }
+}
+
+// acc += act[32 rows, H] @ w[H, 32 cols] with three chunks in flight.  The scheduling fences keep the refill of a
+// register set behind the MFMAs that read it and ahead of the next set's MFMAs, so the wait the compiler puts
+// before a set's MFMAs leaves the two younger refills outstanding.  That only works where no load sits under a
+// run-time condition (at a join the compiler must assume the path with the fewest younger loads and ends up
+// waiting for all of them), hence the chunk count as a template argument for the usual hidden sizes; NCH = 0 is
+// the form for any other count.
+template <int NCH>
+__device__ __forceinline__ void product(v16f& acc, const float* __restrict__ arow, const float* __restrict__ wcol, int H) {
+  ChunkRegs r0, r1, r2;
+  auto fence = [] { __builtin_amdgcn_sched_barrier(0); };
+  if constexpr (NCH >= 3) {
+    constexpr int CE = 3 * ((NCH - 3) / 3);  // first chunk of the tail: at most five chunks from there
+    load_chunk(r0, arow, wcol, H, 0); fence();
+    load_chunk(r1, arow, wcol, H, 1); fence();
+    load_chunk(r2, arow, wcol, H, 2); fence();
+    for (int c = 0; c < CE; c += 3) {
+      mfma_chunk(acc, r0); fence();
+      load_chunk(r0, arow, wcol, H, c + 3); fence();
+      mfma_chunk(acc, r1); fence();
+      load_chunk(r1, arow, wcol, H, c + 4); fence();
+      mfma_chunk(acc, r2); fence();
+      load_chunk(r2, arow, wcol, H, c + 5); fence();
+    }
+    mfma_chunk(acc, r0); fence();
+    if constexpr (CE + 3 < NCH) { load_chunk(r0, arow, wcol, H, CE + 3); fence(); }
+    mfma_chunk(acc, r1); fence();
+    if constexpr (CE + 4 < NCH) { load_chunk(r1, arow, wcol, H, CE + 4); fence(); }
+    mfma_chunk(acc, r2); fence();
+    if constexpr (CE + 3 < NCH) { mfma_chunk(acc, r0); fence(); }
+    if constexpr (CE + 4 < NCH) { mfma_chunk(acc, r1); fence(); }
+  } else {
+    const int nch = H / GKC;
+    for (int c = 0; c < nch; c += 2) {  // two chunks per round, the second one clamped (and then not used)
+      load_chunk(r0, arow, wcol, H, c);
+      load_chunk(r1, arow, wcol, H, min(c + 1, nch - 1));
+      mfma_chunk(acc, r0);
+      if (c + 1 < nch) mfma_chunk(acc, r1);
+    }
+  }
+}
+
+// Occupancy is held at two (shared parameters) or three (six products) waves per SIMD on purpose: with more
+// workgroups in flight the weight slices they stream no longer fit the L2 together, and the whole forward is
+// slower (measured: 1.44 / 1.49 / 1.56 ms at 2 / 3 / 4 waves for H = 256, 14.0 / 18.1 / 17.2 ms for H = 1024).
+template <bool SHARED, int NCH>
+__global__ __launch_bounds__(SHARED ? 256 : 384) __attribute__((amdgpu_waves_per_eu(SHARED ? 2 : 3, SHARED ? 2 : 3)))
+void grid_rnn_plane_kernel(GridArgs a) {
+  constexpr int JOBS = SHARED ? 4 : 6;
+  __shared__ float red[JOBS][16][64];
+
+  const int H = a.H, B = a.B;
+  const int nub = H / 32, nrb = (B + 31) / 32;
+  const int per_pos = nub * nrb;
+  const int item = blockIdx.x;
+  int d = 0, i = 0;
+  plane_positions(a.D, a.L1, a.L2, a.m, item / per_pos, &d, &i);
+  const int j = a.m - d - i;
+  const int ub = item % nub;          // block of 32 hidden units
+  const int rb = (item / nub) % nrb;  // block of 32 batch rows
+
+  const int lane = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6;  // the product
+  const int jl = lane & 31;
+  const int hh = lane >> 5;
+
+  const size_t BH = (size_t)B * H;
+  auto pos = [&](int dd, int ii, int jj, int which) {
+    return a.hsss + ((((size_t)dd * a.L1 + ii) * a.L2 + jj) * 2 + which) * BH;
+  };
+  const float* x_in = d > 0 ? pos(d - 1, i, j, 0) : a.xs + (size_t)(a.crossed ? j : i) * BH;
+  const float* y_in = d > 0 ? pos(d - 1, i, j, 1) : a.ys + (size_t)(a.crossed ? i : j) * BH;
+  const float* sx = i > 0 ? pos(d, i - 1, j, 0) : nullptr;
+  const float* sy = j > 0 ? pos(d, i, j - 1, 1) : nullptr;
+
+  // this wave's product
+  const float* act;
+  const float* w;
+  if (SHARED) {
+    const float* Wd = a.W[0] + (size_t)d * H * H;
+    const float* Ud = a.U[0] + (size_t)d * 2 * H * H;
+    act = wave == 0 ? x_in : wave == 1 ? y_in : wave == 2 ? sx : sy;
+    w = wave < 2 ? Wd : wave == 2 ? Ud : Ud + (size_t)H * H;
+  } else {
+    const int dir = wave & 1;  // waves 0,1: input; 2,3: state_x; 4,5: state_y
+    const float* Ud = a.U[dir] + (size_t)d * 2 * H * H;
+    act = wave < 2 ? (dir ? y_in : x_in) : wave < 4 ? sx : sy;
+    w = wave < 2 ? a.W[dir] + (size_t)d * H * H : wave < 4 ? Ud : Ud + (size_t)H * H;
+  }
+
+  v16f acc;
+#pragma unroll
+  for (int r = 0; r < 16; ++r) acc[r] = 0.0f;
+  if (act) {
+    const int row = min(rb * 32 + jl, B - 1);
+    product<NCH>(acc, act + (size_t)row * H + 16 * hh, w + (size_t)(16 * hh) * H + ub * 32 + jl, H);
+  }
+#pragma unroll
+  for (int r = 0; r < 16; ++r) red[wave][r][lane] = acc[r];
+  __syncthreads();
+  if (wave >= 4) return;
+
+  // wave (dir, rh) finishes registers 8*rh .. 8*rh+7 of direction dir: lane (jl, hh) holds column jl of rows
+  // 8*(r/4) + 4*hh + r%4
+  const int dir = wave & 1;
+  const int rh = wave >> 1;
+  float* out = pos(d, i, j, dir);
+  const float* bias = a.bias[dir] ? a.bias[dir] + (size_t)d * a.bias_rows * H : nullptr;
+  const int col = ub * 32 + jl;
+#pragma unroll
+  for (int rr = 0; rr < 8; ++rr) {
+    const int r = 8 * rh + rr;
+    float v;
+    if (SHARED) v = red[dir][r][lane] + red[2][r][lane] + red[3][r][lane];
+    else v = red[dir][r][lane] + red[2 + dir][r][lane] + red[4 + dir][r][lane];
+    const int row = rb * 32 + 8 * (r >> 2) + 4 * hh + (r & 3);
+    if (row < B) {
+      const float bv = bias ? bias[(size_t)(a.bias_rows == 1 ? 0 : row) * H + col] : 0.0f;
+      out[(size_t)row * H + col] = tanh_f(v + bv);
+    }
+  }
+}
+
+}  // namespace ftk
+
+extern "C" int ftk_grid_rnn_f32(const float* xs, const float* ys, const float* Wx, const float* Ux, const float* bx,
+                                const float* Wy, const float* Uy, const float* by, float* hsss, int D, int L1, int L2,
+                                int B, int H, int bias_rows, int crossed, ftk_stream_t stream) {
+  using namespace ftk;
+  if (!xs || !ys || !Wx || !Ux || !Wy || !Uy || !hsss)
+    return fail(FTK_ERR_INVALID_ARGUMENT, "ftk_grid_rnn_f32: inputs, weights and the output must be non-NULL");
+  if (D <= 0 || L1 <= 0 || L2 <= 0 || B <= 0 || H <= 0)
+    return fail(FTK_ERR_INVALID_ARGUMENT, "ftk_grid_rnn_f32: D, L1, L2, B and H must be positive");
+  if (H % 32 != 0) return fail(FTK_ERR_UNSUPPORTED_SHAPE, "ftk_grid_rnn_f32: H must be a multiple of 32 (got %d)", H);
+  if (bias_rows != 1 && bias_rows != B)
+    return fail(FTK_ERR_INVALID_ARGUMENT, "ftk_grid_rnn_f32: bias_rows must be 1 or B (got %d)", bias_rows);
+  if ((bx == nullptr) != (by == nullptr))
+    return fail(FTK_ERR_INVALID_ARGUMENT, "ftk_grid_rnn_f32: give both biases or neither");
+  GridArgs a;
+  a.xs = xs; a.ys = ys;
+  a.W[0] = Wx; a.W[1] = Wy;
+  a.U[0] = Ux; a.U[1] = Uy;
+  a.bias[0] = bx; a.bias[1] = by;
+  a.hsss = hsss;
+  a.D = D; a.L1 = L1; a.L2 = L2; a.B = B; a.H = H;
+  a.bias_rows = bias_rows;
+  a.crossed = crossed ? 1 : 0;
+  const bool shared = Wx == Wy && Ux == Uy;
+  const int per_pos = (H / 32) * ((B + 31) / 32);
+  for (int m = 0; m <= D + L1 + L2 - 3; ++m) {
+    int d0 = 0, i0 = 0;
+    const long long groups = (long long)plane_positions(D, L1, L2, m, -1, &d0, &i0) * per_pos;
+    if (groups <= 0) continue;
+    if (groups > 0x7fffffffLL) return fail(FTK_ERR_UNSUPPORTED_SHAPE, "ftk_grid_rnn_f32: a plane of %lld workgroups", groups);
+    a.m = m;
+    const dim3 g((unsigned)groups);
+    hipStream_t st = (hipStream_t)stream;
+#define FTK_GRID_LAUNCH(NCH)                                                                            \
+  do {                                                                                                  \
+    if (shared) hipLaunchKernelGGL((grid_rnn_plane_kernel<true, NCH>), g, dim3(256), 0, st, a);         \
+    else hipLaunchKernelGGL((grid_rnn_plane_kernel<false, NCH>), g, dim3(384), 0, st, a);               \
+  } while (0)
+    if (H == 256) FTK_GRID_LAUNCH(8);
+    else if (H == 512) FTK_GRID_LAUNCH(16);
+    else if (H == 1024) FTK_GRID_LAUNCH(32);
+    else FTK_GRID_LAUNCH(0);
+#undef FTK_GRID_LAUNCH
+  }
+  return check_launch("grid_rnn_plane_kernel");
+}

@@ -238,6 +238,34 @@ int ftk_stacked_lstm_wavefront_f32(const float* xs, const float* WU,
                                    int B, int H, ftk_stream_t stream);
 
 /*
+ * Stacked grid RNN, fp32: D blocks over an L1 x L2 grid of positions, two tanh
+ * cells per position that share the state of both directions,
+ *   s = [h_x(d,i-1,j) | h_y(d,i,j-1)]  (zeros outside the grid),
+ *   h_x(d,i,j) = tanh(x_in @ Wx[d] + s @ Ux[d] + bx[d]),
+ *   h_y(d,i,j) = tanh(y_in @ Wy[d] + s @ Uy[d] + by[d]),
+ * where (x_in, y_in) = (h_x, h_y)(d-1,i,j) for d > 0 and, in the first block,
+ * (xs[i], ys[j]) (crossed = 0: xs [L1,B,H], ys [L2,B,H]) or (xs[j], ys[i])
+ * (crossed = 1: xs [L2,B,H], ys [L1,B,H]).  W* [D,H,H], U* [D,2H,H], biases
+ * [D,bias_rows,H] with bias_rows 1 or B, or both NULL; hsss
+ * [D,L1,L2,2,B,H] receives h_x (index 0) and h_y (index 1) of every position
+ * and is also where the kernel reads the neighbours back, so no gather or
+ * scatter buffers exist.  One launch per plane d+i+j.  H%32==0.  Passing the
+ * same pointers for both directions gives the shared-parameter model.
+ * Replaces the eight wavefront regions of
+ * benchmarks/rnn/fractaltensor/grid_lstm/regions/region1.h-region8.h (general
+ * case region8.h:61-310: gather, VanillaRNNCellBMM utils.h:671-700, scatter;
+ * crossed = 0, shared parameters, bias_rows = B, stacked_grid_rnn.cu:31-41) and
+ * is the device form of examples/grid_rnn/grid_rnn.py:40-137 (crossed = 1,
+ * parameters per direction, bias_rows = 1).  Unlike utils.h:650, a plane that
+ * holds a single position still gets its bias and tanh.
+ */
+int ftk_grid_rnn_f32(const float* xs, const float* ys, const float* Wx,
+                     const float* Ux, const float* bx, const float* Wy,
+                     const float* Uy, const float* by, float* hsss, int D,
+                     int L1, int L2, int B, int H, int bias_rows, int crossed,
+                     ftk_stream_t stream);
+
+/*
  * Embedding lookup, the step that feeds the LSTM in the reference's RNN
  * programs: out[i, :] = table[ids[i], :] for i < n.  table [V,E] fp32, ids [n]
  * int32 (ids_are_64bit = 0) or int64 (1) on the device, out [n,E]; E%4==0.

@@ -467,3 +467,38 @@ def grid_rnn(src, trg, params, dtype=np.float64):
                 hy[i, j] = np.tanh(s @ i2h_y + y_in[i, j] @ h2h_y + b_y.reshape(-1))
         x_in, y_in = hx, hy
     return x_in, y_in
+
+
+def grid_rnn_batched(xs, ys, Wx, Ux, bx, Wy, Uy, by, crossed=False, dtype=np.float64):
+    """The same recurrence over a batch, in the array layout of the reference's grid benchmark
+    (benchmarks/rnn/fractaltensor/grid_lstm/stacked_grid_rnn.cu:31-41): W* [D,H,H], U* [D,2H,H], biases
+    [D, 1 or B, H] or None, output hsss [D, L1, L2, 2, B, H] with h_x at index 0 and h_y at 1.
+    Position (d, i, j) reads x_in, y_in = hsss[d-1, i, j, 0/1], state_x = hsss[d, i-1, j, 0] and
+    state_y = hsss[d, i, j-1, 1] (the gather indices of regions/region8.h:112-140), forms
+    h = tanh(in @ W + [state_x | state_y] @ U + b) per direction (utils.h:671-700, 652-663); in the first block
+    x_in = xs[i], y_in = ys[j] (regions/region2.h:74-76, crossed=False) or xs[j], ys[i] (the frontend program,
+    where product(src, trg) puts src along the inner axis; crossed=True).
+    """
+    xs = np.asarray(xs, dtype=dtype)
+    ys = np.asarray(ys, dtype=dtype)
+    Wx, Ux, Wy, Uy = (np.asarray(t, dtype=dtype) for t in (Wx, Ux, Wy, Uy))
+    D, H = Wx.shape[0], Wx.shape[-1]
+    B = xs.shape[1]
+    L1, L2 = (ys.shape[0], xs.shape[0]) if crossed else (xs.shape[0], ys.shape[0])
+    hsss = np.zeros((D, L1, L2, 2, B, H), dtype=dtype)
+    zeros = np.zeros((B, H), dtype=dtype)
+    for d in range(D):
+        b_x = np.asarray(bx[d], dtype=dtype) if bx is not None else 0.0
+        b_y = np.asarray(by[d], dtype=dtype) if by is not None else 0.0
+        for i in range(L1):
+            for j in range(L2):
+                if d > 0:
+                    x_in, y_in = hsss[d - 1, i, j, 0], hsss[d - 1, i, j, 1]
+                else:
+                    x_in, y_in = (xs[j], ys[i]) if crossed else (xs[i], ys[j])
+                state_x = hsss[d, i - 1, j, 0] if i > 0 else zeros
+                state_y = hsss[d, i, j - 1, 1] if j > 0 else zeros
+                s = np.concatenate([state_x, state_y], axis=1)
+                hsss[d, i, j, 0] = np.tanh(x_in @ Wx[d] + s @ Ux[d] + b_x)
+                hsss[d, i, j, 1] = np.tanh(y_in @ Wy[d] + s @ Uy[d] + b_y)
+    return hsss

@@ -470,6 +470,38 @@ def test_eager_grid_rnn_matches_oracle():
     np.testing.assert_allclose(cx[1, 2], np.tanh(s12 @ i2hx.data.numpy() + s_np[2] @ h2hx.data.numpy() + bx.data.numpy()[0]), rtol=1e-5, atol=1e-6)
 
 
+def test_batched_grid_oracle_agrees_with_the_per_sample_one_and_with_a_path_product():
+    """The array-layout oracle used for the GPU kernel, pinned two ways: (1) with crossed inputs, a bias row per
+    block and one sample per batch row it is the per-sample recurrence above, sample by sample; (2) with the
+    second axis of length one and Ux's lower half unused it is a plain stacked tanh RNN along the first axis,
+    written here directly."""
+    H, S, Tg, D, B = 8, 4, 3, 2, 3
+    rng = np.random.default_rng(3)
+    params = programs.make_grid_params(D, H, seed=9)
+    npar = [tuple(tuple(t.data.numpy().astype(np.float64) for t in cell) for cell in block) for block in params]
+    Wx = np.stack([b[0][1] for b in npar]); Ux = np.stack([b[0][0] for b in npar]); bx = np.stack([b[0][2] for b in npar])
+    Wy = np.stack([b[1][1] for b in npar]); Uy = np.stack([b[1][0] for b in npar]); by = np.stack([b[1][2] for b in npar])
+    src = rng.standard_normal((S, B, H)); trg = rng.standard_normal((Tg, B, H))
+    hsss = ko.grid_rnn_batched(src, trg, Wx, Ux, bx, Wy, Uy, by, crossed=True)
+    assert hsss.shape == (D, Tg, S, 2, B, H)
+    for b in range(B):
+        rx, ry = ko.grid_rnn(src[:, b], trg[:, b], npar)
+        np.testing.assert_allclose(hsss[-1, :, :, 0, b], rx, rtol=1e-12, atol=1e-14)
+        np.testing.assert_allclose(hsss[-1, :, :, 1, b], ry, rtol=1e-12, atol=1e-14)
+    # (2) L2 = 1: state_y is always zero, so h_x(d, i) = tanh(in @ Wx + h_x(d, i-1) @ Ux[:H] + b)
+    xs = rng.standard_normal((5, B, H)); ys = rng.standard_normal((1, B, H))
+    bB = rng.standard_normal((D, B, H))                         # a bias row per batch row, as in the benchmark
+    got = ko.grid_rnn_batched(xs, ys, Wx, Ux, bB, Wy, Uy, bB, crossed=False)
+    inp = xs
+    for d in range(D):
+        h = np.zeros((B, H)); outs = []
+        for i in range(5):
+            h = np.tanh(inp[i] @ Wx[d] + h @ Ux[d][:H] + bB[d])
+            outs.append(h)
+        inp = np.stack(outs)
+        np.testing.assert_allclose(got[d, :, 0, 0], inp, rtol=1e-12, atol=1e-14)
+
+
 def test_fused_paths_refuse_cpu_inputs():
     Wss, Uss, bss = programs.make_lstm_params(1, 32, 0.1, seed=1)
     xss = programs.make_sequence_batch(2, 2, 32, seed=2)

@@ -723,3 +723,82 @@ def test_embedding_gather_counts_bad_ids_and_reads_nothing_out_of_bounds(core):
     assert e.value.code == -2
     with pytest.raises(TypeError):
         core.embedding_gather(table, ids.float())
+
+
+# ---- grid RNN ---------------------------------------------------------------------------------------------------
+
+def _grid_inputs(D, L1, L2, B, H, bias_rows, shared, crossed, seed=0):
+    g = torch.Generator().manual_seed(seed)
+    u = lambda *shape, s=1.0: (torch.rand(shape, generator=g) * 2 - 1) * s
+    sc = 1.0 / (3 * H) ** 0.5
+    xs = u(L2 if crossed else L1, B, H)
+    ys = u(L1 if crossed else L2, B, H)
+    Wx, Ux = u(D, H, H, s=sc * 2), u(D, 2 * H, H, s=sc * 2)
+    Wy, Uy = (Wx, Ux) if shared else (u(D, H, H, s=sc * 2), u(D, 2 * H, H, s=sc * 2))
+    bx = u(D, bias_rows, H, s=0.2) if bias_rows else None
+    by = (bx if shared else u(D, bias_rows, H, s=0.2)) if bias_rows else None
+    return xs, ys, Wx, Ux, bx, Wy, Uy, by
+
+
+@pytest.mark.parametrize('D,L1,L2,B,H,bias_rows,shared,crossed', [
+    (1, 1, 1, 32, 32, 1, False, False),     # a single position: no state at all
+    (2, 3, 4, 32, 64, 32, True, False),     # the benchmark's form: shared parameters, a bias row per batch row
+    (3, 4, 2, 5, 96, 1, False, True),       # the frontend program's form; a partial row block, odd chunk count
+    (2, 1, 5, 40, 32, 0, False, False),     # one axis of length one, two row blocks, no bias
+    (4, 5, 5, 32, 256, 32, True, False),    # the benchmark's hidden size
+    (2, 2, 3, 1, 128, 1, False, True),      # one sample
+    (2, 3, 3, 32, 512, 1, True, False),     # the other two hidden sizes of the benchmark's sweep (run.sh:8-9)
+    (1, 2, 2, 33, 1024, 33, False, False),
+])
+def test_grid_rnn(core, D, L1, L2, B, H, bias_rows, shared, crossed):
+    """fp32 MFMA products against the float64 recurrence: 1e-4, the tolerance of the fp32 LSTM path."""
+    args = _grid_inputs(D, L1, L2, B, H, bias_rows, shared, crossed)
+    ref = ko.grid_rnn_batched(*[None if t is None else t.numpy() for t in args], crossed=crossed)
+    dev = [None if t is None else t.cuda() for t in args]
+    out = core.grid_rnn(*dev, crossed=crossed)
+    assert out.shape == (D, L1, L2, 2, B, H)
+    np.testing.assert_allclose(out.cpu().numpy(), ref, rtol=1e-4, atol=1e-5)
+    # the output array is also where neighbours are read back: a poisoned one must give the same result
+    poisoned = torch.full_like(out, float('nan'))
+    core.grid_rnn(*dev, crossed=crossed, out=poisoned)
+    assert torch.equal(poisoned, out)
+
+
+def test_grid_rnn_benchmark_shape_properties(core):
+    """The benchmark's full shape (stacked_grid_rnn.cu:108-118, run.sh: depth 32, hidden 256, length 10, batch 32),
+    too large for the loop oracle in a test: (1) with Ux = 0 the grid decouples into independent columns, each
+    position a stack of plain tanh layers, checked against torch; (2) swapping the two directions' parameters and
+    inputs and transposing the grid swaps h_x and h_y."""
+    D, L, B, H = 32, 10, 32, 256
+    xs, ys, Wx, Ux, bx, Wy, Uy, by = [t.cuda() for t in _grid_inputs(D, L, L, B, H, B, False, False, seed=4)]
+    zero = torch.zeros_like(Ux)
+    out = core.grid_rnn(xs, ys, Wx, zero, bx, Wy, zero, by)
+    hx, hy = xs.double(), ys.double()
+    for d in range(D):
+        hx = torch.tanh(hx @ Wx[d].double() + bx[d].double())
+        hy = torch.tanh(hy @ Wy[d].double() + by[d].double())
+    np.testing.assert_allclose(out[-1, :, 3, 0].cpu().numpy(), hx.cpu().numpy(), rtol=1e-4, atol=1e-5)
+    np.testing.assert_allclose(out[-1, 6, :, 1].cpu().numpy(), hy.cpu().numpy(), rtol=1e-4, atol=1e-5)
+    # (2) mirror: U's two halves swap along with the directions
+    swap = lambda U: torch.cat([U[:, H:], U[:, :H]], dim=1).contiguous()
+    a = core.grid_rnn(xs, ys, Wx, Ux, bx, Wy, Uy, by)
+    b = core.grid_rnn(ys, xs, Wy, swap(Uy), by, Wx, swap(Ux), bx)
+    np.testing.assert_allclose(b[:, :, :, 1].cpu().numpy(), a[:, :, :, 0].transpose(1, 2).cpu().numpy(), rtol=1e-4, atol=1e-5)
+    np.testing.assert_allclose(b[:, :, :, 0].cpu().numpy(), a[:, :, :, 1].transpose(1, 2).cpu().numpy(), rtol=1e-4, atol=1e-5)
+    assert torch.isfinite(a).all() and a.abs().max() <= 1.0
+
+
+def test_grid_rnn_rejects_bad_arguments(core):
+    xs, ys, Wx, Ux, bx, Wy, Uy, by = [t.cuda() for t in _grid_inputs(1, 2, 2, 4, 48, 1, False, False)]
+    with pytest.raises(core.FtkError) as e:
+        core.grid_rnn(xs, ys, Wx, Ux, bx, Wy, Uy, by)            # H not a multiple of 32
+    assert e.value.code == -2
+    xs, ys, Wx, Ux, bx, Wy, Uy, by = [t.cuda() for t in _grid_inputs(1, 2, 2, 4, 32, 1, False, False)]
+    with pytest.raises(ValueError):
+        core.grid_rnn(xs, ys, Wx, Ux, bx, Wy, Uy, None)
+    with pytest.raises(ValueError):
+        core.grid_rnn(xs, ys[:, :2], Wx, Ux, bx, Wy, Uy, by)
+    with pytest.raises(ValueError):
+        core.grid_rnn(xs, ys, Wx, Ux[:, :32], bx, Wy, Uy, by)
+    with pytest.raises(TypeError):
+        core.grid_rnn(xs.half(), ys, Wx, Ux, bx, Wy, Uy, by)
