@@ -271,7 +271,8 @@ def bench_grid_rnn(torch, core, steps, warmup, cpu):
         'config': {'workload': 'stacked grid RNN forward (grid_lstm/stacked_grid_rnn.cu), one launch per plane d+i+j',
                    'depth': D, 'src_len': L, 'trg_len': L, 'batch': B, 'hidden': H, 'planes': D + 2 * L - 2},
         'roofline': {'bound': 'mfma', 'achieved': flop / ms / 1e9, 'peak': PEAK_F32_MATRIX_TFLOPS, 'unit': 'TFLOP/s',
-                     'frac': flop / ms / 1e9 / PEAK_F32_MATRIX_TFLOPS, 'traffic': None, 'kernel': 'grid_rnn_plane_kernel',
+                     'frac': flop / ms / 1e9 / PEAK_F32_MATRIX_TFLOPS, 'traffic': MEASURED_TRAFFIC_BYTES.get('grid_rnn_plane_kernel_per_pass'),
+                     'kernel': 'grid_rnn_plane_kernel<true, 8> (50 launches per pass)',
                      'note': 'the whole forward (50 dependent launches) against the fp32 MFMA peak; planes near the '
                              'corners hold a handful of positions, so the chain of launches, not the matrix rate, bounds it'},
         'torch_per_plane_gather_bmm_scatter': {'ms_per_step': ms_t, 'speedup': ms_t / ms, 'max_abs_diff': err},

@@ -6,6 +6,7 @@ kernel calls on FractalTensors that live on the GPU.
   dilated_lstm   the dilated_map program of examples/dilated_rnn/dilated_rnn.py:16-41
   flash_attention  the map / reduce program of examples/flash_attention/flash_attention.py:14-91
   b2b_gemm       (a @ b) @ c, the computation of benchmarks/fused_two_hgemms
+  grid_rnn       the nested-scan program of examples/grid_rnn/grid_rnn.py:40-137 over a batch of samples
 
 A regular (non-ragged) FractalTensor already is a dense row-major tensor in
 its flat buffer, so inputs are handed to the kernels as views and outputs are
@@ -24,7 +25,7 @@ from ..tensor import Tensor
 from ..types import FractalTensorStorage, TensorStorage, torch_type_to_internal_type
 
 __all__ = ['pack_lstm_weights', 'pad_time_major', 'unpad_time_major', 'stacked_lstm', 'dilated_lstm', 'lstm_cell', 'flash_attention', 'b2b_gemm', 'mm',
-           'online_softmax', 'embedding_lookup']
+           'online_softmax', 'embedding_lookup', 'grid_rnn']
 
 
 def _core():
@@ -262,3 +263,41 @@ def embedding_lookup(embedding: Tensor, words: FractalTensor) -> FractalTensor:
     ft.indices = words.indices
     ft._T = out.reshape(-1)
     return ft
+
+
+def grid_rnn(srcs: FractalTensor, trgs: FractalTensor, params):
+    """The stacked grid RNN of examples/grid_rnn/grid_rnn.py:40-137 for a batch of samples in one call per plane
+    of the (block, target, source) grid.
+
+    srcs: depth-2 [N][S] of [1, H], trgs: depth-2 [N][Tg] of [1, H] (the two sides of the reference's outer map
+    over samples, :127-137; equal lengths within the batch); params: per block ((i2h [2H, H], h2h [H, H],
+    bias [1, H]) for the x direction, the same for y), Tensors on the GPU.  Returns (h_x, h_y), each depth-3
+    [N][Tg][S] of [1, H]: the last block's outputs at every grid position, as the eager program returns them."""
+    core = _core()
+    xs = _dense_gpu(srcs, 'srcs', 2)   # [N, S, 1, H]
+    ys = _dense_gpu(trgs, 'trgs', 2)   # [N, Tg, 1, H]
+    N, S, one, H = xs.shape
+    if one != 1 or ys.shape[0] != N or tuple(ys.shape[2:]) != (1, H):
+        raise ValueError('srcs and trgs should be [N][S] and [N][Tg] of [1, H].')
+    Tg = ys.shape[1]
+
+    def stack(direction: int, which: int, shape):
+        ts = []
+        for block in params:
+            t = block[direction][which]
+            t = t.data if isinstance(t, Tensor) else t
+            if tuple(t.shape) != shape:
+                raise ValueError(f'grid parameter of shape {tuple(t.shape)}, expected {shape}.')
+            if not t.is_cuda:
+                raise RuntimeError('grid_rnn runs on the GPU only; move the parameters there.')
+            ts.append(t.float())
+        return torch.stack(ts).contiguous()
+
+    Ux, Wx, bx = stack(0, 0, (2 * H, H)), stack(0, 1, (H, H)), stack(0, 2, (1, H))
+    Uy, Wy, by = stack(1, 0, (2 * H, H)), stack(1, 1, (H, H)), stack(1, 2, (1, H))
+    xs_t = xs.reshape(N, S, H).transpose(0, 1).contiguous().float()    # [S, N, H]: the source runs along the inner axis
+    ys_t = ys.reshape(N, Tg, H).transpose(0, 1).contiguous().float()   # [Tg, N, H]
+    hsss = core.grid_rnn(xs_t, ys_t, Wx, Ux, bx, Wy, Uy, by, crossed=True)   # [D, Tg, S, 2, N, H]
+    last = hsss[-1].permute(2, 3, 0, 1, 4).contiguous()                      # [2, N, Tg, S, H]
+    return (FractalTensor.from_dense(last[0].reshape(N, Tg, S, 1, H), 3),
+            FractalTensor.from_dense(last[1].reshape(N, Tg, S, 1, H), 3))

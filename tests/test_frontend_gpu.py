@@ -216,3 +216,24 @@ def test_fused_stacked_lstm_keeps_an_fp16_program_in_fp16():
     bias = bss.as_dense().float().cpu().numpy().reshape(L, 4 * H)
     ref, _ = ko.stacked_lstm_f16(xss.as_dense().cpu().numpy().reshape(T, B, H), WU, bias)
     assert ko.max_rel_err(out.float().cpu().numpy().reshape(T, B, H), ref[-1].astype(np.float32)) <= 1e-2
+
+
+def test_fused_grid_rnn_equals_eager_program():
+    """A batch of samples through the grid kernel against the eager nested-scan program run sample by sample on
+    the CPU (fp32 both; 1e-4 as for the fp32 LSTM path)."""
+    N, S, Tg, H, depth = 3, 5, 4, 32, 3
+    torch.manual_seed(2)
+    src = torch.randn(N, S, 1, H)
+    trg = torch.randn(N, Tg, 1, H)
+    params = programs.make_grid_params(depth, H, seed=8)
+    gpu_params = [tuple(tuple(Tensor.from_tensor(t.data.cuda()) for t in cell) for cell in block) for block in params]
+    hx, hy = ops.fused.grid_rnn(FractalTensor.from_dense(src.cuda(), 2), FractalTensor.from_dense(trg.cuda(), 2), gpu_params)
+    assert hx.depth == 3 and hx.dense_shape() == (N, Tg, S) and hx.element_shape == (1, H)
+    gx = hx.as_dense().cpu().numpy().reshape(N, Tg, S, H)
+    gy = hy.as_dense().cpu().numpy().reshape(N, Tg, S, H)
+    for n in range(N):
+        ex, ey = programs.grid_rnn(FractalTensor.from_dense(src[n], 1), FractalTensor.from_dense(trg[n], 1), params, H)
+        np.testing.assert_allclose(gx[n], ex.as_dense().numpy().reshape(Tg, S, H), rtol=1e-4, atol=1e-5)
+        np.testing.assert_allclose(gy[n], ey.as_dense().numpy().reshape(Tg, S, H), rtol=1e-4, atol=1e-5)
+    with pytest.raises(RuntimeError):
+        ops.fused.grid_rnn(FractalTensor.from_dense(src, 2), FractalTensor.from_dense(trg, 2), gpu_params)
