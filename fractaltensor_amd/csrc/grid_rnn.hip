@@ -98,6 +98,7 @@ __device__ __forceinline__ void product(v16f& acc, const float* __restrict__ aro
   ChunkRegs r0, r1, r2;
   auto fence = [] { __builtin_amdgcn_sched_barrier(0); };
   if constexpr (NCH >= 3) {
+    H = NCH * GKC;  // known at compile time: the weight rows' addresses become constant offsets
     constexpr int CE = 3 * ((NCH - 3) / 3);  // first chunk of the tail: at most five chunks from there
     load_chunk(r0, arow, wcol, H, 0); fence();
     load_chunk(r1, arow, wcol, H, 1); fence();
