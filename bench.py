@@ -290,6 +290,40 @@ def bench_grid_rnn(torch, core, steps, warmup, cpu):
     return res
 
 
+def bench_windowed_attention(torch, core, steps, warmup, cpu):
+    """The reference's sparse-attention shape (examples/sparse_attention/sparse_attention.py:125-141: 16 heads of 64,
+    window 5, dilation 2, three random positions, the commented sequence length 4096) at batch 16, fp32: Q, K, V read
+    once, O written once."""
+    G, S, D, W, dl, R = 256, 4096, 64, 5, 2, 3
+    gen = torch.Generator(device='cpu').manual_seed(1234)
+    Q, K, V = ((torch.randn((G, S, D), generator=gen) * (2.0 / D ** 0.5 if i == 0 else 1.0)).cuda() for i in range(3))
+    extra = torch.randint(0, S, (G, S, R), generator=gen, dtype=torch.int32).cuda()
+    O = torch.empty_like(Q)
+    ci = ctypes.c_int
+    run = lambda: core._check(core.lib.ftk_windowed_attn_f32(core._ptr(Q), core._ptr(K), core._ptr(V), core._ptr(extra), core._ptr(O),
+                                                             ci(G), ci(S), ci(D), ci(W), ci(dl), ci(R), ctypes.c_float(1.0), core._stream()))
+    ms, _ = _events_ms(torch, run, steps, warmup)
+    nbytes = 4.0 * G * S * D * 4 + G * S * R * 4
+    res = {
+        'metric': 'tokens/s (windowed attention)', 'value': G * S / ms * 1e3, 'unit': 'tokens/s', 'ms_per_step': ms, 'dtype': 'f32',
+        'config': {'workload': 'windowed + random attention (shifted_slide + sparse_attn, sparse_attention.py:25-71)', 'batch_x_heads': G,
+                   'seq_len': S, 'head_dim': D, 'window': W, 'dilation': dl, 'random': R},
+        'roofline': {'bound': 'hbm', 'achieved': nbytes / ms / 1e6, 'peak': PEAK_HBM_GBS, 'unit': 'GB/s',
+                     'frac': nbytes / ms / 1e6 / PEAK_HBM_GBS, 'traffic': MEASURED_TRAFFIC_BYTES.get('windowed_attn_kernel'),
+                     'kernel': 'windowed_attn_kernel<16, 1>', 'algorithmic_bytes_per_launch': nbytes},
+    }
+    if cpu:
+        from oracle import kaleido_oracle as ko
+        n = 2
+        t0 = time.perf_counter()
+        ref = ko.windowed_attention(Q[:n].cpu().numpy(), K[:n].cpu().numpy(), V[:n].cpu().numpy(), W, dl, extra[:n].cpu().numpy(), dtype=np.float32)
+        dt = time.perf_counter() - t0
+        res['cpu_baseline'] = {'value': n * S / dt, 'unit': 'tokens/s', 'cores': 1, 'kind': 'port',
+                               'sample': f'{n} of {G} sequences ({n * S} tokens) through the numpy oracle in {dt:.2f} s',
+                               'max_abs_diff_vs_gpu': float(np.abs(ref - O[:n].cpu().numpy()).max())}
+    return res
+
+
 def bench_gemm(torch, core, steps, warmup, cpu):
     """The plain fp16 product that the streaming kernels are built around, on its own: 8192^3, beside torch.mm."""
     M = N = K = 8192
@@ -593,7 +627,7 @@ def main():
     ap.add_argument('--gpus', type=int, default=1)
     ap.add_argument('--steps', type=int, default=50)
     ap.add_argument('--warmup', type=int, default=10)
-    ap.add_argument('--workload', default='b2b', choices=['b2b', 'attention', 'stacked_lstm', 'dilated_lstm', 'lstm_f16_h256', 'lstm_f16_h512', 'lstm_f16_h1024', 'lstm_f32_h512', 'lstm_f32_h1024', 'gemm', 'online_softmax', 'embedding', 'grid_rnn', 'copy'])
+    ap.add_argument('--workload', default='b2b', choices=['b2b', 'attention', 'stacked_lstm', 'dilated_lstm', 'lstm_f16_h256', 'lstm_f16_h512', 'lstm_f16_h1024', 'lstm_f32_h512', 'lstm_f32_h1024', 'gemm', 'online_softmax', 'embedding', 'grid_rnn', 'windowed_attention', 'copy'])
     ap.add_argument('--no-extras', action='store_true', help='measure only the chosen workload')
     ap.add_argument('--no-cpu', action='store_true', help='skip the CPU baseline leg')
     ap.add_argument('--no-baselines', action='store_true',
@@ -626,6 +660,7 @@ def main():
         'online_softmax': lambda s, w, c: bench_softmax(torch, core, s, w, c),
         'embedding': lambda s, w, c: bench_embedding(torch, core, s, w, c),
         'grid_rnn': lambda s, w, c: bench_grid_rnn(torch, core, max(5, s // 2), max(2, w // 2), c),
+        'windowed_attention': lambda s, w, c: bench_windowed_attention(torch, core, s, w, c),
     }
     if args.workload == 'copy':
         runners = {'copy': lambda s, w, c: bench_copy(torch, core, s, w, c)}

@@ -23,7 +23,7 @@ EXPORTS = (
     'ftk_stacked_lstm_wavefront_f32', 'ftk_stacked_lstm_ragged_f32', 'ftk_lstm_set_products', 'ftk_lstm_get_products',
     'ftk_stacked_lstm_f16_workspace_bytes', 'ftk_stacked_lstm_f16',
     'ftk_b2b_gemm_f16', 'ftk_b2b_gemm_rowmajor_f16', 'ftk_gemm_f16', 'ftk_batched_gemm_f16', 'ftk_flash_attn_f16', 'ftk_online_softmax_f32', 'ftk_embedding_gather_f32',
-    'ftk_grid_rnn_f32',
+    'ftk_grid_rnn_f32', 'ftk_windowed_attn_f32',
     'ftk_debug_read_fa_trace',
 )
 
@@ -482,4 +482,35 @@ def grid_rnn(xs, ys, Wx, Ux, bx, Wy, Uy, by, crossed: bool = False, out: Optiona
     _check(lib.ftk_grid_rnn_f32(_ptr(xs), _ptr(ys), _ptr(Wx), _ptr(Ux), _ptr(bx), _ptr(Wy), _ptr(Uy), _ptr(by), _ptr(out),
                                 ctypes.c_int(D), ctypes.c_int(L1), ctypes.c_int(L2), ctypes.c_int(B), ctypes.c_int(H),
                                 ctypes.c_int(bias_rows), ctypes.c_int(1 if crossed else 0), _stream()))
+    return out
+
+
+def windowed_attention(Q, K, V, window: int, dilation: int = 1, extra_idx: Optional[torch.Tensor] = None,
+                       scale: float = 1.0, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Q, K, V [G, S, D] fp32: every token attends to the `window` positions centred on it (`dilation` apart,
+    wrapped at the ends as shifted_slide wraps them) and to extra_idx[g, t, :] (int32 [G, S, R]) if given."""
+    for name, t in (('Q', Q), ('K', K), ('V', V)):
+        _req(t, torch.float32, name)
+    if Q.dim() != 3 or K.shape != Q.shape or V.shape != Q.shape:
+        raise ValueError(f'Q, K and V must be [G, S, D] of one shape, got {tuple(Q.shape)}, {tuple(K.shape)}, {tuple(V.shape)}')
+    G, S, D = Q.shape
+    R = 0
+    if extra_idx is not None:
+        _req(extra_idx, torch.int32, 'extra_idx')
+        if extra_idx.dim() != 3 or tuple(extra_idx.shape[:2]) != (G, S):
+            raise ValueError(f'extra_idx must be [G, S, R], got {tuple(extra_idx.shape)}')
+        R = extra_idx.shape[2]
+        if R == 0:
+            extra_idx = None
+        elif int(extra_idx.min()) < 0 or int(extra_idx.max()) >= S:
+            raise IndexError(f'extra_idx holds a position outside [0, {S})')
+    if out is None:
+        out = torch.empty_like(Q)
+    else:
+        _req(out, torch.float32, 'out')
+        if out.shape != Q.shape:
+            raise ValueError(f'out must be {tuple(Q.shape)}, got {tuple(out.shape)}')
+    _check(lib.ftk_windowed_attn_f32(_ptr(Q), _ptr(K), _ptr(V), _ptr(extra_idx), _ptr(out), ctypes.c_int(G), ctypes.c_int(S),
+                                     ctypes.c_int(D), ctypes.c_int(window), ctypes.c_int(dilation), ctypes.c_int(R),
+                                     ctypes.c_float(scale), _stream()))
     return out

@@ -7,6 +7,7 @@ kernel calls on FractalTensors that live on the GPU.
   flash_attention  the map / reduce program of examples/flash_attention/flash_attention.py:14-91
   b2b_gemm       (a @ b) @ c, the computation of benchmarks/fused_two_hgemms
   grid_rnn       the nested-scan program of examples/grid_rnn/grid_rnn.py:40-137 over a batch of samples
+  windowed_attention  shifted_slide + the map of sparse_attn of examples/sparse_attention/sparse_attention.py:25-71
 
 A regular (non-ragged) FractalTensor already is a dense row-major tensor in
 its flat buffer, so inputs are handed to the kernels as views and outputs are
@@ -25,7 +26,7 @@ from ..tensor import Tensor
 from ..types import FractalTensorStorage, TensorStorage, torch_type_to_internal_type
 
 __all__ = ['pack_lstm_weights', 'pad_time_major', 'unpad_time_major', 'stacked_lstm', 'dilated_lstm', 'lstm_cell', 'flash_attention', 'b2b_gemm', 'mm',
-           'online_softmax', 'embedding_lookup', 'grid_rnn']
+           'online_softmax', 'embedding_lookup', 'grid_rnn', 'windowed_attention']
 
 
 def _core():
@@ -301,3 +302,31 @@ def grid_rnn(srcs: FractalTensor, trgs: FractalTensor, params):
     last = hsss[-1].permute(2, 3, 0, 1, 4).contiguous()                      # [2, N, Tg, S, H]
     return (FractalTensor.from_dense(last[0].reshape(N, Tg, S, 1, H), 3),
             FractalTensor.from_dense(last[1].reshape(N, Tg, S, 1, H), 3))
+
+
+def windowed_attention(query: FractalTensor, key: FractalTensor, value: FractalTensor, window_size: int,
+                       dilation: int = 1, random_attn_pos: Optional[FractalTensor] = None) -> FractalTensor:
+    """ops.shifted_slide(ops.zip(key, value), window_size, dilation) followed by the map of sparse_attn over the
+    tokens (examples/sparse_attention/sparse_attention.py:25-38, 51-53, 69-71), as one kernel.
+
+    query, key, value: regular FractalTensors of one structure, depth >= 1, of [1, D] tokens; the innermost level is
+    the sequence, the outer ones (heads, batch) are independent.  random_attn_pos: the same structure of [1, R]
+    integer tokens, or None.  The result has the structure of `query`."""
+    if not all(isinstance(t, FractalTensor) for t in (query, key, value)):
+        raise TypeError('query, key and value should be FractalTensors.')
+    depth = query.depth
+    q = _dense_gpu(query, 'query', depth)
+    k = _dense_gpu(key, 'key', depth)
+    v = _dense_gpu(value, 'value', depth)
+    if q.shape != k.shape or q.shape != v.shape or q.shape[-2] != 1:
+        raise ValueError('query, key and value should have one structure of [1, D] tokens.')
+    S, D = q.shape[-3], q.shape[-1]
+    extra = None
+    if random_attn_pos is not None:
+        r = _dense_gpu(random_attn_pos, 'random_attn_pos', depth)
+        if r.shape[:-1] != q.shape[:-1] or r.is_floating_point():
+            raise ValueError('random_attn_pos should have the structure of query and hold [1, R] integers.')
+        extra = r.reshape(-1, S, r.shape[-1]).to(torch.int32).contiguous()
+    out = _core().windowed_attention(q.reshape(-1, S, D).float().contiguous(), k.reshape(-1, S, D).float().contiguous(),
+                                     v.reshape(-1, S, D).float().contiguous(), window_size, dilation, extra, 1.0)
+    return FractalTensor.from_dense(out.reshape(q.shape), depth)

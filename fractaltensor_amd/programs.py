@@ -14,6 +14,8 @@ baseline that bench.py times on configuration 1.
                    an explicit score scale
   grid RNN         examples/grid_rnn/grid_rnn.py:40-137 (one sample: source x target grid,
                    two tanh cells per position sharing the state of both directions)
+  windowed attn    examples/sparse_attention/sparse_attention.py:25-38, 51-53, 69-71 (one head: every token
+                   attends to its shifted_slide window joined with randomly picked positions)
 """
 from __future__ import annotations
 
@@ -174,3 +176,28 @@ def grid_rnn(src: FractalTensor, trg: FractalTensor, params, hidden: int):
     yss1, yss2 = ops.fold(lambda inputs, block: _grid_block(inputs, block, hidden), blocks,
                           initializer=ops.zip(*ops.product(src, trg)))
     return yss1, yss2
+
+
+# ---- windowed (+ random) attention -----------------------------------------------------
+
+def windowed_attention(query: FractalTensor, key: FractalTensor, value: FractalTensor, window_size: int,
+                       dilation: int = 1, random_attn_pos: FractalTensor = None) -> FractalTensor:
+    """One head of the windowed part of the reference's sparse attention, for every token (the reference runs it
+    on the tokens between its global ones): query, key, value depth-1 [S] of [1, D]; random_attn_pos depth-1 [S]
+    of [1, R] integer Tensors or None.  Token t attends to the window shifted_slide gives it, joined with
+    key[ids], value[ids] of its random positions: softmax(q @ ks^T) @ vs with no score scale."""
+    windowed_key, windowed_value = ops.shifted_slide(ops.zip(key, value), window_size=window_size, dilation=dilation)
+
+    def sparse_attn(x):
+        if random_attn_pos is None:
+            query_token, w_keys, w_values = x
+            ks, vs = ops.flatten(w_keys).T, ops.flatten(w_values)
+        else:
+            query_token, w_keys, w_values, ids = x
+            ks = ops.flatten(w_keys.join(key[ids])).T
+            vs = ops.flatten(w_values.join(value[ids]))
+        return ops.softmax(query_token @ ks, dim=1) @ vs
+
+    if random_attn_pos is None:
+        return ops.map(sparse_attn, ops.zip(query, windowed_key, windowed_value))
+    return ops.map(sparse_attn, ops.zip(query, windowed_key, windowed_value, random_attn_pos))

@@ -344,6 +344,30 @@ int ftk_flash_attn_f16(const void* Q, const void* K, const void* V, void* O,
                        ftk_stream_t stream);
 
 /*
+ * Windowed attention, fp32: token t of each of the G sequences attends to the
+ * `window` (odd) positions t - half + k*dilation, k = 0..window-1,
+ * half = (window-1)*dilation/2, and to the R further positions
+ * extra_idx[g, t, 0..R-1] (int32 on the device; NULL with R = 0):
+ *   O[g,t] = softmax(scale * Q[g,t] . K[g,P]^T) . V[g,P],  P = window ++ extra.
+ * Q, K, V, O [G,S,D] row-major, 16-byte aligned; D%4==0, D <= 1024.  Window
+ * positions past an end wrap as the reference's shifted_slide wraps them:
+ * p >= S -> p - S, p < 0 -> p + S - 1 (kaleido/frontend/operations/access.py:
+ * 384-390; one short of circular at the left end, kept as it is).  An
+ * extra_idx entry outside [0,S) is clamped rather than read out of bounds;
+ * the Python side raises IndexError before the call, as indexing a
+ * FractalTensor does.
+ * Replaces, per head, ops.shifted_slide(ops.zip(key, value), window_size,
+ * dilation) followed by the map of sparse_attn over the tokens
+ * (examples/sparse_attention/sparse_attention.py:25-38, 51-53, 69-71:
+ * softmax(q @ [windowed ++ random keys]^T) @ [windowed ++ random values],
+ * scale = 1); the reference has no device kernel for it.
+ */
+int ftk_windowed_attn_f32(const float* Q, const float* K, const float* V,
+                          const int* extra_idx, float* O, int G, int S, int D,
+                          int window, int dilation, int R, float scale,
+                          ftk_stream_t stream);
+
+/*
  * Row softmax through an online (max, denominator) scan, fp32, [rows, cols].
  * Replaces OnlineNormalizedSoftmaxOp
  * (kaleido/core/operators/online_softmax_op.cu:14-36,

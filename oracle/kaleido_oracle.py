@@ -502,3 +502,34 @@ def grid_rnn_batched(xs, ys, Wx, Ux, bx, Wy, Uy, by, crossed=False, dtype=np.flo
                 hsss[d, i, j, 0] = np.tanh(x_in @ Wx[d] + s @ Ux[d] + b_x)
                 hsss[d, i, j, 1] = np.tanh(y_in @ Wy[d] + s @ Uy[d] + b_y)
     return hsss
+
+
+# ------------------------------------------------------------------ windowed attention
+
+def window_positions(t, S, window, dilation):
+    """Positions of the window centred on t as shifted_slide produces them
+    (kaleido/frontend/operations/access.py:376-431): t - half + k*dilation with half = ((window-1)*dilation+1)//2,
+    and the wrap of :384-390, x >= S -> x - S, x < 0 -> x + S - 1."""
+    half = ((window - 1) * dilation + 1) // 2
+    out = []
+    for x in range(t - half, t + half + 1, dilation):
+        out.append(x + S - 1 if x < 0 else (x - S if x >= S else x))
+    return out
+
+
+def windowed_attention(Q, K, V, window, dilation=1, extra_idx=None, scale=1.0, dtype=np.float64):
+    """softmax(scale * q_t . K[P]^T) . V[P] per token with P = window_positions(t) ++ extra_idx[g, t]: the map of
+    sparse_attn over the tokens (examples/sparse_attention/sparse_attention.py:25-38, 69-71; keys and values are the
+    windowed ones joined with the randomly picked ones, :33-34).  Q, K, V [G, S, D]."""
+    Q, K, V = (np.asarray(a, dtype=dtype) for a in (Q, K, V))
+    G, S, D = Q.shape
+    out = np.zeros_like(Q)
+    for g in range(G):
+        for t in range(S):
+            P = window_positions(t, S, window, dilation)
+            if extra_idx is not None:
+                P = P + [int(i) for i in extra_idx[g, t]]
+            s = scale * (K[g, P] @ Q[g, t])
+            e = np.exp(s - s.max())
+            out[g, t] = (e / e.sum()) @ V[g, P]
+    return out

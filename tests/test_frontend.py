@@ -356,6 +356,34 @@ def test_windowed_attention_program_over_shifted_slide():
         assert torch.allclose(out[pos].data, ref, atol=1e-6)
 
 
+def test_eager_windowed_attention_with_random_positions_matches_oracle():
+    """shifted_slide + sparse_attn over every token (examples/sparse_attention/sparse_attention.py:25-38, 51-53,
+    69-71) through the frontend, against the numpy restatement; the restatement's window positions against a
+    hand-worked case (S = 4, window 3: token 0 sees [2, 0, 1] -- the source's wrap lands one short of circular --
+    token 3 sees [2, 3, 0]) and its arithmetic against torch on explicit index lists."""
+    assert ko.window_positions(0, 4, 3, 1) == [2, 0, 1]
+    assert ko.window_positions(3, 4, 3, 1) == [2, 3, 0]
+    assert ko.window_positions(5, 12, 5, 2) == [1, 3, 5, 7, 9]
+    assert ko.window_positions(1, 12, 5, 2) == [8, 10, 1, 3, 5]        # -3 -> 8, -1 -> 10
+    torch.manual_seed(0)
+    S, D, W, dl, R = 12, 8, 5, 2, 3
+    mk = lambda: FractalTensor.from_dense(torch.randn(S, 1, D), 1)
+    q, k, v = mk(), mk(), mk()
+    ids = torch.randint(0, S, (S, 1, R))
+    dense = lambda t: t.as_dense().numpy().reshape(1, S, D)
+    out = programs.windowed_attention(q, k, v, W, dl, FractalTensor.from_dense(ids, 1))
+    ref = ko.windowed_attention(dense(q), dense(k), dense(v), W, dl, ids.numpy().reshape(1, S, R))
+    np.testing.assert_allclose(out.as_dense().numpy().reshape(S, D), ref[0], rtol=1e-5, atol=1e-6)
+    out = programs.windowed_attention(q, k, v, 3)
+    ref3 = ko.windowed_attention(dense(q), dense(k), dense(v), 3)
+    np.testing.assert_allclose(out.as_dense().numpy().reshape(S, D), ref3[0], rtol=1e-5, atol=1e-6)
+    Q, K, V = (torch.from_numpy(dense(t)[0]).double() for t in (q, k, v))
+    for t in (0, 1, 6, 11):
+        P = ko.window_positions(t, S, W, dl) + ids[t, 0].tolist()
+        direct = torch.softmax(Q[t] @ K[P].T, dim=0) @ V[P]
+        np.testing.assert_allclose(ref[0, t], direct.numpy(), rtol=1e-12)
+
+
 def test_arange_slices_and_constants():                 # test_constants.py:16-34
     for args in ((11,), (5, 7), (5, 24, 3)):
         ft = ops.slices(ops.arange(*args), dim=0)

@@ -237,3 +237,24 @@ def test_fused_grid_rnn_equals_eager_program():
         np.testing.assert_allclose(gy[n], ey.as_dense().numpy().reshape(Tg, S, H), rtol=1e-4, atol=1e-5)
     with pytest.raises(RuntimeError):
         ops.fused.grid_rnn(FractalTensor.from_dense(src, 2), FractalTensor.from_dense(trg, 2), gpu_params)
+
+
+def test_fused_windowed_attention_equals_eager_program():
+    """Two heads of a batch of two through the kernel against the eager shifted_slide + sparse_attn program run head
+    by head on the CPU, with and without random positions."""
+    Bn, Hd, S, D, W, dl, R = 2, 2, 14, 16, 5, 2, 3
+    torch.manual_seed(4)
+    q, k, v = (torch.randn(Bn, Hd, S, 1, D) for _ in range(3))
+    ids = torch.randint(0, S, (Bn, Hd, S, 1, R))
+    ft = lambda t: FractalTensor.from_dense(t.cuda(), 3)
+    for rp in (None, ids):
+        fused = ops.fused.windowed_attention(ft(q), ft(k), ft(v), W, dl, None if rp is None else ft(rp))
+        assert fused.depth == 3 and fused.dense_shape() == (Bn, Hd, S) and fused.element_shape == (1, D)
+        got = fused.as_dense().cpu().numpy()
+        for b in range(Bn):
+            for h in range(Hd):
+                one = lambda t: FractalTensor.from_dense(t[b, h], 1)
+                eager = programs.windowed_attention(one(q), one(k), one(v), W, dl, None if rp is None else one(rp))
+                np.testing.assert_allclose(got[b, h], eager.as_dense().numpy(), rtol=1e-4, atol=1e-5)
+    with pytest.raises(RuntimeError):
+        ops.fused.windowed_attention(FractalTensor.from_dense(q, 3), FractalTensor.from_dense(k, 3), FractalTensor.from_dense(v, 3), W)

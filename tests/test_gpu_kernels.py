@@ -802,3 +802,62 @@ def test_grid_rnn_rejects_bad_arguments(core):
         core.grid_rnn(xs, ys, Wx, Ux[:, :32], bx, Wy, Uy, by)
     with pytest.raises(TypeError):
         core.grid_rnn(xs.half(), ys, Wx, Ux, bx, Wy, Uy, by)
+
+
+# ---- windowed attention -----------------------------------------------------------------------------------------
+
+@pytest.mark.parametrize('G,S,D,window,dilation,R', [
+    (1, 4, 4, 3, 1, 0),          # the smallest case: both ends wrap
+    (2, 16, 64, 5, 2, 3),        # the reference's window and random count (sparse_attention.py:136-141) at its test length
+    (3, 33, 8, 1, 1, 0),         # a window of one: every token sees itself only
+    (2, 50, 256, 7, 3, 2),       # half the span (9) wraps several tokens at each end
+    (1, 20, 1024, 3, 1, 1),      # the widest row: four pieces per lane
+    (4, 64, 36, 5, 1, 0),        # a row that does not fill its lanes; tokens that do not fill the last workgroup
+    (1, 7, 512, 5, 1, 4),
+])
+def test_windowed_attention(core, G, S, D, window, dilation, R):
+    g = torch.Generator().manual_seed(5)
+    Q, K, V = (torch.randn((G, S, D), generator=g) for _ in range(3))
+    Q = Q * (2.0 / D ** 0.5)                                    # scores of a few units: a softmax that is not flat
+    extra = torch.randint(0, S, (G, S, R), generator=g, dtype=torch.int32) if R else None
+    ref = ko.windowed_attention(Q.numpy(), K.numpy(), V.numpy(), window, dilation, None if extra is None else extra.numpy())
+    out = core.windowed_attention(Q.cuda(), K.cuda(), V.cuda(), window, dilation, None if extra is None else extra.cuda())
+    np.testing.assert_allclose(out.cpu().numpy(), ref, rtol=1e-4, atol=1e-5)
+    half = core.windowed_attention(Q.cuda(), K.cuda(), V.cuda(), window, dilation, None if extra is None else extra.cuda(), scale=0.5)
+    ref_half = ko.windowed_attention(Q.numpy(), K.numpy(), V.numpy(), window, dilation, None if extra is None else extra.numpy(), scale=0.5)
+    np.testing.assert_allclose(half.cpu().numpy(), ref_half, rtol=1e-4, atol=1e-5)
+
+
+def test_windowed_attention_full_size_properties(core):
+    """The bench shape (16 x 16 heads, 4096 tokens of 64), where the loop oracle is too slow: a window of one returns
+    V bit for bit; with K = 0 every key weighs the same, so the output is the mean of the window's V rows, built here
+    with torch.roll away from the ends; constant V rows come back unchanged whatever the scores."""
+    G, S, D, W, dl = 256, 4096, 64, 5, 2
+    g = torch.Generator().manual_seed(6)
+    Q = torch.randn((G, S, D), generator=g).cuda()
+    K = torch.randn((G, S, D), generator=g).cuda()
+    V = torch.randn((G, S, D), generator=g).cuda()
+    assert torch.equal(core.windowed_attention(Q, K, V, 1), V)
+    flat = core.windowed_attention(Q, torch.zeros_like(K), V, W, dl)
+    mean = sum(torch.roll(V, -o, dims=1) for o in (-4, -2, 0, 2, 4)) / 5
+    np.testing.assert_allclose(flat[:, 4:-4].cpu().numpy(), mean[:, 4:-4].cpu().numpy(), rtol=1e-5, atol=1e-6)
+    const = torch.arange(D, dtype=torch.float32, device='cuda').expand(G, S, D).contiguous()
+    np.testing.assert_allclose(core.windowed_attention(Q, K, const, W, dl).cpu().numpy(), const.cpu().numpy(), rtol=1e-5)
+
+
+def test_windowed_attention_rejects_bad_arguments(core):
+    Q = torch.randn((2, 8, 16), device='cuda')
+    with pytest.raises(core.FtkError) as e:
+        core.windowed_attention(Q, Q, Q, 4)                      # even window: as shifted_slide
+    assert e.value.code == -2
+    with pytest.raises(core.FtkError) as e:
+        core.windowed_attention(Q, Q, Q, 5, 4)                   # half the span (8) does not fit 8 tokens
+    assert e.value.code == -2
+    with pytest.raises(core.FtkError):
+        core.windowed_attention(Q[:, :, :6].contiguous(), Q[:, :, :6].contiguous(), Q[:, :, :6].contiguous(), 3)   # D % 4
+    with pytest.raises(IndexError):
+        core.windowed_attention(Q, Q, Q, 3, 1, torch.full((2, 8, 2), 8, dtype=torch.int32, device='cuda'))
+    with pytest.raises(TypeError):
+        core.windowed_attention(Q, Q, Q, 3, 1, torch.zeros((2, 8, 2), dtype=torch.int64, device='cuda'))
+    with pytest.raises(ValueError):
+        core.windowed_attention(Q, Q[:, :4], Q, 3)
