@@ -254,10 +254,13 @@ def bench_grid_rnn(torch, core, steps, warmup, cpu):
     W, U, b = u(D, H, H, s=sc), u(D, 2 * H, H, s=sc), u(D, B, H, s=0.2)
     out = torch.empty((D, L, L, 2, B, H), device='cuda')
     ci = ctypes.c_int
+    ws = torch.empty(core.lib.ftk_grid_rnn_workspace_bytes(D, H) // 2, dtype=torch.uint8, device='cuda')   # shared parameters: one direction's worth
     run = lambda: core._check(core.lib.ftk_grid_rnn_f32(
         core._ptr(xs), core._ptr(ys), core._ptr(W), core._ptr(U), core._ptr(b), core._ptr(W), core._ptr(U), core._ptr(b),
-        core._ptr(out), ci(D), ci(L), ci(L), ci(B), ci(H), ci(B), ci(0), core._stream()))
+        core._ptr(out), ci(D), ci(L), ci(L), ci(B), ci(H), ci(B), ci(0), core._ptr(ws), ctypes.c_size_t(ws.numel()), core._stream()))
     ms, _ = _events_ms(torch, run, steps, warmup)
+    ms_plain, _ = _events_ms(torch, lambda: core.grid_rnn(xs, ys, W, U, b, W, U, b, out=out, relay_weights=False), steps, warmup)
+    run()
     base, A = _grid_torch_planes(torch, xs, ys, W, U, b, D, L, B, H)
     ms_t, _ = _events_ms(torch, base, max(2, steps // 5), 1)
     err = (A[1:, 1:, 1:] - out).abs().max().item()
@@ -272,10 +275,11 @@ def bench_grid_rnn(torch, core, steps, warmup, cpu):
                    'depth': D, 'src_len': L, 'trg_len': L, 'batch': B, 'hidden': H, 'planes': D + 2 * L - 2},
         'roofline': {'bound': 'mfma', 'achieved': flop / ms / 1e9, 'peak': PEAK_F32_MATRIX_TFLOPS, 'unit': 'TFLOP/s',
                      'frac': flop / ms / 1e9 / PEAK_F32_MATRIX_TFLOPS, 'traffic': MEASURED_TRAFFIC_BYTES.get('grid_rnn_plane_kernel_per_pass'),
-                     'kernel': 'grid_rnn_plane_kernel<true, 8> (50 launches per pass)',
+                     'kernel': 'grid_rnn_plane_kernel<true, 8, true> (50 launches per pass, after two re-lay launches)',
                      'note': 'the whole forward (50 dependent launches) against the fp32 MFMA peak; planes near the '
                              'corners hold a handful of positions, so the chain of launches, not the matrix rate, bounds it'},
         'torch_per_plane_gather_bmm_scatter': {'ms_per_step': ms_t, 'speedup': ms_t / ms, 'max_abs_diff': err},
+        'without_workspace': {'ms_per_step': ms_plain, 'note': 'parameters read where they lie, no re-laid copy'},
     }
     if cpu:
         from oracle import kaleido_oracle as ko

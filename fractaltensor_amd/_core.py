@@ -23,7 +23,7 @@ EXPORTS = (
     'ftk_stacked_lstm_wavefront_f32', 'ftk_stacked_lstm_ragged_f32', 'ftk_lstm_set_products', 'ftk_lstm_get_products',
     'ftk_stacked_lstm_f16_workspace_bytes', 'ftk_stacked_lstm_f16',
     'ftk_b2b_gemm_f16', 'ftk_b2b_gemm_rowmajor_f16', 'ftk_gemm_f16', 'ftk_batched_gemm_f16', 'ftk_flash_attn_f16', 'ftk_online_softmax_f32', 'ftk_embedding_gather_f32',
-    'ftk_grid_rnn_f32', 'ftk_windowed_attn_f32',
+    'ftk_grid_rnn_workspace_bytes', 'ftk_grid_rnn_f32', 'ftk_windowed_attn_f32',
     'ftk_debug_read_fa_trace',
 )
 
@@ -57,8 +57,10 @@ def _load() -> ctypes.CDLL:
     lib.ftk_stacked_lstm_workspace_bytes.argtypes = [ctypes.c_int] * 4
     lib.ftk_stacked_lstm_f16_workspace_bytes.restype = ctypes.c_size_t
     lib.ftk_stacked_lstm_f16_workspace_bytes.argtypes = [ctypes.c_int] * 4
+    lib.ftk_grid_rnn_workspace_bytes.restype = ctypes.c_size_t
+    lib.ftk_grid_rnn_workspace_bytes.argtypes = [ctypes.c_int] * 2
     for name in EXPORTS:
-        if name not in ('ftk_last_error', 'ftk_stacked_lstm_workspace_bytes', 'ftk_stacked_lstm_f16_workspace_bytes'):
+        if name not in ('ftk_last_error', 'ftk_stacked_lstm_workspace_bytes', 'ftk_stacked_lstm_f16_workspace_bytes', 'ftk_grid_rnn_workspace_bytes'):
             getattr(lib, name).restype = ctypes.c_int
     return lib
 
@@ -449,11 +451,14 @@ def online_softmax(x) -> torch.Tensor:
     return y
 
 
-def grid_rnn(xs, ys, Wx, Ux, bx, Wy, Uy, by, crossed: bool = False, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+def grid_rnn(xs, ys, Wx, Ux, bx, Wy, Uy, by, crossed: bool = False, out: Optional[torch.Tensor] = None,
+             workspace: Optional[torch.Tensor] = None, relay_weights: bool = True) -> torch.Tensor:
     """Stacked grid RNN, fp32.  W* [D, H, H], U* [D, 2H, H], biases [D, 1 or B, H] or both None.
     crossed=False: xs [L1, B, H] feeds the first grid axis, ys [L2, B, H] the second (the layout of the
     reference's grid benchmark); crossed=True: xs [L2, B, H] is indexed by the second axis and ys [L1, B, H] by the
-    first (the layout of its frontend program).  Returns hsss [D, L1, L2, 2, B, H]: h_x at index 0, h_y at 1."""
+    first (the layout of its frontend program).  Returns hsss [D, L1, L2, 2, B, H]: h_x at index 0, h_y at 1.
+    workspace: uint8 device tensor for the re-laid parameters (allocated here if None); relay_weights=False runs
+    the kernel that reads the parameters where they lie."""
     for name, t in (('xs', xs), ('ys', ys), ('Wx', Wx), ('Ux', Ux), ('Wy', Wy), ('Uy', Uy)):
         _req(t, torch.float32, name)
     if xs.dim() != 3 or ys.dim() != 3 or xs.shape[1:] != ys.shape[1:]:
@@ -479,9 +484,13 @@ def grid_rnn(xs, ys, Wx, Ux, bx, Wy, Uy, by, crossed: bool = False, out: Optiona
         _req(out, torch.float32, 'out')
         if tuple(out.shape) != (D, L1, L2, 2, B, H):
             raise ValueError(f'out must be {(D, L1, L2, 2, B, H)}, got {tuple(out.shape)}')
+    if relay_weights and workspace is None:
+        shared = Wx.data_ptr() == Wy.data_ptr() and Ux.data_ptr() == Uy.data_ptr()
+        workspace = torch.empty(lib.ftk_grid_rnn_workspace_bytes(D, H) // (2 if shared else 1), dtype=torch.uint8, device=xs.device)
+    ws_ptr, ws_bytes = (_ptr(workspace), workspace.numel()) if relay_weights else (None, 0)
     _check(lib.ftk_grid_rnn_f32(_ptr(xs), _ptr(ys), _ptr(Wx), _ptr(Ux), _ptr(bx), _ptr(Wy), _ptr(Uy), _ptr(by), _ptr(out),
                                 ctypes.c_int(D), ctypes.c_int(L1), ctypes.c_int(L2), ctypes.c_int(B), ctypes.c_int(H),
-                                ctypes.c_int(bias_rows), ctypes.c_int(1 if crossed else 0), _stream()))
+                                ctypes.c_int(bias_rows), ctypes.c_int(1 if crossed else 0), ws_ptr, ctypes.c_size_t(ws_bytes), _stream()))
     return out
 
 

@@ -14,15 +14,18 @@
 // directions share their parameters (four waves; the state products are computed once and serve both), six
 // products otherwise.  A product whose state lies outside the grid is skipped.  Each wave runs its product on
 // v_mfma_f32_32x32x2_f32 straight from global memory -- no operand is used by a second wave of the workgroup, so
-// LDS staging would only add barriers -- with the operands of the next three k chunks of 32 in registers.  Within a
+// LDS staging would only add barriers -- with the operands of the next two or three k chunks of 32 in registers.  Within a
 // chunk the k index is permuted so that a lane's activation values are 64 contiguous bytes: step (q, e) uses
 // k = 4q + e for lanes 0-31 and k = 16 + 4q + e for lanes 32-63.  The products are added through LDS before bias
-// and tanh.
+// and tanh.  Given a workspace, the entry point first re-lays the parameters so that the sixteen weights a lane
+// needs of a chunk are 64 contiguous bytes (four loads instead of sixteen strided ones).
 //
 // Placement.  Workgroups are numbered position-major, unit block fastest, and ids go round the eight XCDs: with
 // eight unit blocks (H = 256) an XCD only ever touches one 32-column slice of every block's parameters.  (Running
 // the positions of block d on XCD d % 8 instead, so that an XCD touches the parameters of four blocks only, was
 // measured and is slower: the planes' positions do not divide evenly over the blocks.)
+#include <algorithm>
+
 #include "ftk_common.h"
 
 namespace ftk {
@@ -38,6 +41,8 @@ struct GridArgs {
   int bias_rows;  // 1: one row for the whole batch, B: a row per batch row
   int crossed;    // 0: x_in = xs[i], y_in = ys[j];  1: x_in = xs[j], y_in = ys[i]
   int m;          // the plane d + i + j of this launch
+  const float* Wp[2];  // the same parameters re-laid per wave (pack kernel below), or nullptr
+  const float* Up[2];
 };
 
 constexpr int GKC = 32;  // k chunk
@@ -68,13 +73,43 @@ struct ChunkRegs {
 };
 
 // One k chunk of a product: lane (jl, hh) holds activation row jl, k = 16*hh .. 16*hh+15, and column jl of the
-// weight rows with the same k.
+// weight rows with the same k.  PACKED: the lane's sixteen weights are 64 contiguous bytes of the re-laid copy
+// (four loads instead of sixteen: a wave can keep 63 loads in flight, so fewer instructions per chunk mean more
+// bytes in flight), wcol then points at the lane's slot of chunk 0 and chunks are 1024 floats apart.
+template <bool PACKED>
 __device__ __forceinline__ void load_chunk(ChunkRegs& r, const float* __restrict__ arow, const float* __restrict__ wcol,
                                            int H, int c) {
 #pragma unroll
   for (int q = 0; q < 4; ++q) r.a[q] = *reinterpret_cast<const float4*>(arow + c * GKC + 4 * q);
+  if constexpr (PACKED) {
+    const float4* wp = reinterpret_cast<const float4*>(wcol + (size_t)c * 1024);
 #pragma unroll
-  for (int e = 0; e < 16; ++e) r.b[e] = wcol[(size_t)(c * GKC + e) * H];
+    for (int e4 = 0; e4 < 4; ++e4) {
+      const float4 t = wp[e4];
+      r.b[4 * e4] = t.x; r.b[4 * e4 + 1] = t.y; r.b[4 * e4 + 2] = t.z; r.b[4 * e4 + 3] = t.w;
+    }
+  } else {
+#pragma unroll
+    for (int e = 0; e < 16; ++e) r.b[e] = wcol[(size_t)(c * GKC + e) * H];
+  }
+}
+
+// Re-lays M [D][rows][H] (rows a multiple of 32) as [D][H/32 unit blocks][rows/32 chunks][64 lanes][16]: element e of
+// lane (jl, hh) of chunk c of unit block ub is M[32c + 16hh + e][32ub + jl] -- the order load_chunk reads.
+__global__ __launch_bounds__(256) void grid_pack_weights_kernel(const float* __restrict__ M, float* __restrict__ out,
+                                                                long long total4, int rows, int H) {
+  const int ctot = rows / GKC, nub = H / 32;
+  for (long long idx = (long long)blockIdx.x * 256 + threadIdx.x; idx < total4; idx += (long long)gridDim.x * 256) {
+    const int e4 = (int)(idx & 3);
+    const int lane = (int)((idx >> 2) & 63);
+    const long long rest = idx >> 8;
+    const int c = (int)(rest % ctot);
+    const int ub = (int)((rest / ctot) % nub);
+    const long long d = rest / ((long long)ctot * nub);
+    const int k = c * GKC + 16 * (lane >> 5) + 4 * e4;
+    const float* src = M + ((size_t)d * rows + k) * H + ub * 32 + (lane & 31);
+    reinterpret_cast<float4*>(out)[idx] = make_float4(src[0], src[H], src[2 * (size_t)H], src[3 * (size_t)H]);
+  }
 }
 
 __device__ __forceinline__ void mfma_chunk(v16f& acc, const ChunkRegs& r) {
@@ -87,42 +122,42 @@ __device__ __forceinline__ void mfma_chunk(v16f& acc, const ChunkRegs& r) {
   }
 }
 
-// acc += act[32 rows, H] @ w[H, 32 cols] with three chunks in flight.  The scheduling fences keep the refill of a
+// acc += act[32 rows, H] @ w[H, 32 cols] with NS chunks in flight.  The scheduling fences keep the refill of a
 // register set behind the MFMAs that read it and ahead of the next set's MFMAs, so the wait the compiler puts
-// before a set's MFMAs leaves the two younger refills outstanding.  That only works where no load sits under a
+// before a set's MFMAs leaves the younger refills outstanding.  That only works where no load sits under a
 // run-time condition (at a join the compiler must assume the path with the fewest younger loads and ends up
 // waiting for all of them), hence the chunk count as a template argument for the usual hidden sizes; NCH = 0 is
-// the form for any other count.
-template <int NCH>
+// the form for any other count.  NS is 3 with the parameters where they lie (20 loads per chunk: a wave cannot
+// have more than 63 outstanding) and 2 with the re-laid copy (8 loads per chunk; 3 to 6 sets measured slower,
+// 1.21 to 1.53 ms against 1.17 ms for H = 256, as did one).
+template <int NCH, bool PACKED, int NS>
 __device__ __forceinline__ void product(v16f& acc, const float* __restrict__ arow, const float* __restrict__ wcol, int H) {
-  ChunkRegs r0, r1, r2;
   auto fence = [] { __builtin_amdgcn_sched_barrier(0); };
-  if constexpr (NCH >= 3) {
+  if constexpr (NCH >= NS) {
     H = NCH * GKC;  // known at compile time: the weight rows' addresses become constant offsets
-    constexpr int CE = 3 * ((NCH - 3) / 3);  // first chunk of the tail: at most five chunks from there
-    load_chunk(r0, arow, wcol, H, 0); fence();
-    load_chunk(r1, arow, wcol, H, 1); fence();
-    load_chunk(r2, arow, wcol, H, 2); fence();
-    for (int c = 0; c < CE; c += 3) {
-      mfma_chunk(acc, r0); fence();
-      load_chunk(r0, arow, wcol, H, c + 3); fence();
-      mfma_chunk(acc, r1); fence();
-      load_chunk(r1, arow, wcol, H, c + 4); fence();
-      mfma_chunk(acc, r2); fence();
-      load_chunk(r2, arow, wcol, H, c + 5); fence();
+    ChunkRegs r[NS];
+    static_for<NS>([&](auto s) { load_chunk<PACKED>(r[s], arow, wcol, H, s); fence(); });
+    constexpr int MAIN = NCH / NS - 1;  // rounds all of whose refills exist
+    for (int k = 0; k < MAIN; ++k) {
+      static_for<NS>([&](auto s) {
+        mfma_chunk(acc, r[s]); fence();
+        load_chunk<PACKED>(r[s], arow, wcol, H, NS * (k + 1) + s); fence();
+      });
     }
-    mfma_chunk(acc, r0); fence();
-    if constexpr (CE + 3 < NCH) { load_chunk(r0, arow, wcol, H, CE + 3); fence(); }
-    mfma_chunk(acc, r1); fence();
-    if constexpr (CE + 4 < NCH) { load_chunk(r1, arow, wcol, H, CE + 4); fence(); }
-    mfma_chunk(acc, r2); fence();
-    if constexpr (CE + 3 < NCH) { mfma_chunk(acc, r0); fence(); }
-    if constexpr (CE + 4 < NCH) { mfma_chunk(acc, r1); fence(); }
+    constexpr int CE = NS * MAIN;  // the sets hold chunks CE .. CE+NS-1; fewer than NS more follow
+    static_for<NS>([&](auto s) {
+      mfma_chunk(acc, r[s]); fence();
+      if constexpr (CE + NS + s < NCH) { load_chunk<PACKED>(r[s], arow, wcol, H, CE + NS + s); fence(); }
+    });
+    static_for<NS>([&](auto s) {
+      if constexpr (CE + NS + s < NCH) { mfma_chunk(acc, r[s]); fence(); }
+    });
   } else {
+    ChunkRegs r0, r1;
     const int nch = H / GKC;
     for (int c = 0; c < nch; c += 2) {  // two chunks per round, the second one clamped (and then not used)
-      load_chunk(r0, arow, wcol, H, c);
-      load_chunk(r1, arow, wcol, H, min(c + 1, nch - 1));
+      load_chunk<PACKED>(r0, arow, wcol, H, c);
+      load_chunk<PACKED>(r1, arow, wcol, H, min(c + 1, nch - 1));
       mfma_chunk(acc, r0);
       if (c + 1 < nch) mfma_chunk(acc, r1);
     }
@@ -131,8 +166,9 @@ __device__ __forceinline__ void product(v16f& acc, const float* __restrict__ aro
 
 // Occupancy is held at two (shared parameters) or three (six products) waves per SIMD on purpose: with more
 // workgroups in flight the weight slices they stream no longer fit the L2 together, and the whole forward is
-// slower (measured: 1.44 / 1.49 / 1.56 ms at 2 / 3 / 4 waves for H = 256, 14.0 / 18.1 / 17.2 ms for H = 1024).
-template <bool SHARED, int NCH>
+// slower (measured: 1.44 / 1.49 / 1.56 ms at 2 / 3 / 4 waves for H = 256 with the parameters where they lie; with
+// the re-laid copy 1.17 / 1.17 / 1.21 ms, and 9.8 / 11.2 / 11.3 ms for H = 1024).
+template <bool SHARED, int NCH, bool PACKED>
 __global__ __launch_bounds__(SHARED ? 256 : 384) __attribute__((amdgpu_waves_per_eu(SHARED ? 2 : 3, SHARED ? 2 : 3)))
 void grid_rnn_plane_kernel(GridArgs a) {
   constexpr int JOBS = SHARED ? 4 : 6;
@@ -162,19 +198,21 @@ void grid_rnn_plane_kernel(GridArgs a) {
   const float* sx = i > 0 ? pos(d, i - 1, j, 0) : nullptr;
   const float* sy = j > 0 ? pos(d, i, j - 1, 1) : nullptr;
 
-  // this wave's product
-  const float* act;
-  const float* w;
-  if (SHARED) {
-    const float* Wd = a.W[0] + (size_t)d * H * H;
-    const float* Ud = a.U[0] + (size_t)d * 2 * H * H;
-    act = wave == 0 ? x_in : wave == 1 ? y_in : wave == 2 ? sx : sy;
-    w = wave < 2 ? Wd : wave == 2 ? Ud : Ud + (size_t)H * H;
+  // this wave's product: kind 0 input @ W, 1 state_x @ U[:H], 2 state_y @ U[H:]
+  const int dir = SHARED ? 0 : (wave & 1);
+  const int kind = SHARED ? (wave < 2 ? 0 : wave - 1) : (wave >> 1);
+  const bool y_side = SHARED ? wave == 1 : dir == 1;
+  const float* act = kind == 0 ? (y_side ? y_in : x_in) : kind == 1 ? sx : sy;
+  const float* w;  // where this lane's weights of chunk 0 lie
+  if (PACKED) {
+    const int cps = H / GKC;                       // chunks per product
+    const int ctot = kind == 0 ? cps : 2 * cps;    // chunks of the whole matrix: U holds both state products
+    const float* base = kind == 0 ? a.Wp[dir] + (size_t)d * H * H : a.Up[dir] + (size_t)d * 2 * H * H;
+    w = base + ((size_t)ub * ctot + (kind == 2 ? cps : 0)) * 1024 + lane * 16;
   } else {
-    const int dir = wave & 1;  // waves 0,1: input; 2,3: state_x; 4,5: state_y
     const float* Ud = a.U[dir] + (size_t)d * 2 * H * H;
-    act = wave < 2 ? (dir ? y_in : x_in) : wave < 4 ? sx : sy;
-    w = wave < 2 ? a.W[dir] + (size_t)d * H * H : wave < 4 ? Ud : Ud + (size_t)H * H;
+    const float* base = kind == 0 ? a.W[dir] + (size_t)d * H * H : kind == 1 ? Ud : Ud + (size_t)H * H;
+    w = base + (size_t)(16 * hh) * H + ub * 32 + jl;
   }
 
   v16f acc;
@@ -182,7 +220,7 @@ void grid_rnn_plane_kernel(GridArgs a) {
   for (int r = 0; r < 16; ++r) acc[r] = 0.0f;
   if (act) {
     const int row = min(rb * 32 + jl, B - 1);
-    product<NCH>(acc, act + (size_t)row * H + 16 * hh, w + (size_t)(16 * hh) * H + ub * 32 + jl, H);
+    product<NCH, PACKED, PACKED ? 2 : 3>(acc, act + (size_t)row * H + 16 * hh, w, H);
   }
 #pragma unroll
   for (int r = 0; r < 16; ++r) red[wave][r][lane] = acc[r];
@@ -191,17 +229,17 @@ void grid_rnn_plane_kernel(GridArgs a) {
 
   // wave (dir, rh) finishes registers 8*rh .. 8*rh+7 of direction dir: lane (jl, hh) holds column jl of rows
   // 8*(r/4) + 4*hh + r%4
-  const int dir = wave & 1;
+  const int od = wave & 1;
   const int rh = wave >> 1;
-  float* out = pos(d, i, j, dir);
-  const float* bias = a.bias[dir] ? a.bias[dir] + (size_t)d * a.bias_rows * H : nullptr;
+  float* out = pos(d, i, j, od);
+  const float* bias = a.bias[od] ? a.bias[od] + (size_t)d * a.bias_rows * H : nullptr;
   const int col = ub * 32 + jl;
 #pragma unroll
   for (int rr = 0; rr < 8; ++rr) {
     const int r = 8 * rh + rr;
     float v;
-    if (SHARED) v = red[dir][r][lane] + red[2][r][lane] + red[3][r][lane];
-    else v = red[dir][r][lane] + red[2 + dir][r][lane] + red[4 + dir][r][lane];
+    if (SHARED) v = red[od][r][lane] + red[2][r][lane] + red[3][r][lane];
+    else v = red[od][r][lane] + red[2 + od][r][lane] + red[4 + od][r][lane];
     const int row = rb * 32 + 8 * (r >> 2) + 4 * hh + (r & 3);
     if (row < B) {
       const float bv = bias ? bias[(size_t)(a.bias_rows == 1 ? 0 : row) * H + col] : 0.0f;
@@ -212,9 +250,15 @@ void grid_rnn_plane_kernel(GridArgs a) {
 
 }  // namespace ftk
 
+extern "C" size_t ftk_grid_rnn_workspace_bytes(int D, int H) {
+  if (D <= 0 || H <= 0) return 0;
+  return 2 * (size_t)D * 3 * H * H * sizeof(float);  // W and U of both directions, re-laid
+}
+
 extern "C" int ftk_grid_rnn_f32(const float* xs, const float* ys, const float* Wx, const float* Ux, const float* bx,
                                 const float* Wy, const float* Uy, const float* by, float* hsss, int D, int L1, int L2,
-                                int B, int H, int bias_rows, int crossed, ftk_stream_t stream) {
+                                int B, int H, int bias_rows, int crossed, void* workspace, size_t workspace_bytes,
+                                ftk_stream_t stream) {
   using namespace ftk;
   if (!xs || !ys || !Wx || !Ux || !Wy || !Uy || !hsss)
     return fail(FTK_ERR_INVALID_ARGUMENT, "ftk_grid_rnn_f32: inputs, weights and the output must be non-NULL");
@@ -235,6 +279,27 @@ extern "C" int ftk_grid_rnn_f32(const float* xs, const float* ys, const float* W
   a.bias_rows = bias_rows;
   a.crossed = crossed ? 1 : 0;
   const bool shared = Wx == Wy && Ux == Uy;
+  hipStream_t st = (hipStream_t)stream;
+  // with room for it, the parameters are re-laid first so that a lane's weights of a chunk are contiguous
+  const size_t per_dir = (size_t)D * 3 * H * H;
+  const bool packed = workspace && workspace_bytes >= (shared ? 1 : 2) * per_dir * sizeof(float) &&
+                      reinterpret_cast<uintptr_t>(workspace) % 16 == 0;
+  a.Wp[0] = a.Wp[1] = a.Up[0] = a.Up[1] = nullptr;
+  if (packed) {
+    float* ws = static_cast<float*>(workspace);
+    for (int dir = 0; dir < (shared ? 1 : 2); ++dir) {
+      float* wp = ws + dir * per_dir;
+      float* up = wp + (size_t)D * H * H;
+      const long long w4 = (long long)D * H * H / 4, u4 = 2 * w4;
+      hipLaunchKernelGGL(grid_pack_weights_kernel, dim3((unsigned)std::min<long long>((w4 + 255) / 256, 65536)), dim3(256), 0, st,
+                         dir ? Wy : Wx, wp, w4, H, H);
+      hipLaunchKernelGGL(grid_pack_weights_kernel, dim3((unsigned)std::min<long long>((u4 + 255) / 256, 65536)), dim3(256), 0, st,
+                         dir ? Uy : Ux, up, u4, 2 * H, H);
+      a.Wp[dir] = wp;
+      a.Up[dir] = up;
+    }
+    if (shared) { a.Wp[1] = a.Wp[0]; a.Up[1] = a.Up[0]; }
+  }
   const int per_pos = (H / 32) * ((B + 31) / 32);
   for (int m = 0; m <= D + L1 + L2 - 3; ++m) {
     int d0 = 0, i0 = 0;
@@ -243,17 +308,22 @@ extern "C" int ftk_grid_rnn_f32(const float* xs, const float* ys, const float* W
     if (groups > 0x7fffffffLL) return fail(FTK_ERR_UNSUPPORTED_SHAPE, "ftk_grid_rnn_f32: a plane of %lld workgroups", groups);
     a.m = m;
     const dim3 g((unsigned)groups);
-    hipStream_t st = (hipStream_t)stream;
-#define FTK_GRID_LAUNCH(NCH)                                                                            \
+#define FTK_GRID_LAUNCH_P(NCH, P)                                                                         \
   do {                                                                                                  \
-    if (shared) hipLaunchKernelGGL((grid_rnn_plane_kernel<true, NCH>), g, dim3(256), 0, st, a);         \
-    else hipLaunchKernelGGL((grid_rnn_plane_kernel<false, NCH>), g, dim3(384), 0, st, a);               \
+    if (shared) hipLaunchKernelGGL((grid_rnn_plane_kernel<true, NCH, P>), g, dim3(256), 0, st, a);      \
+    else hipLaunchKernelGGL((grid_rnn_plane_kernel<false, NCH, P>), g, dim3(384), 0, st, a);            \
+  } while (0)
+#define FTK_GRID_LAUNCH(NCH)                \
+  do {                                      \
+    if (packed) FTK_GRID_LAUNCH_P(NCH, true); \
+    else FTK_GRID_LAUNCH_P(NCH, false);     \
   } while (0)
     if (H == 256) FTK_GRID_LAUNCH(8);
     else if (H == 512) FTK_GRID_LAUNCH(16);
     else if (H == 1024) FTK_GRID_LAUNCH(32);
     else FTK_GRID_LAUNCH(0);
 #undef FTK_GRID_LAUNCH
+#undef FTK_GRID_LAUNCH_P
   }
   return check_launch("grid_rnn_plane_kernel");
 }

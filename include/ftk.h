@@ -251,6 +251,11 @@ int ftk_stacked_lstm_wavefront_f32(const float* xs, const float* WU,
  * and is also where the kernel reads the neighbours back, so no gather or
  * scatter buffers exist.  One launch per plane d+i+j.  H%32==0.  Passing the
  * same pointers for both directions gives the shared-parameter model.
+ * workspace: 16-byte aligned device memory of ftk_grid_rnn_workspace_bytes(D, H)
+ * bytes (half of it suffices with shared parameters) into which every call
+ * first re-lays the parameters in the order the kernel's lanes read them; with
+ * NULL or less room the kernel reads the parameters where they lie (about 12 %
+ * slower).
  * Replaces the eight wavefront regions of
  * benchmarks/rnn/fractaltensor/grid_lstm/regions/region1.h-region8.h (general
  * case region8.h:61-310: gather, VanillaRNNCellBMM utils.h:671-700, scatter;
@@ -259,10 +264,12 @@ int ftk_stacked_lstm_wavefront_f32(const float* xs, const float* WU,
  * parameters per direction, bias_rows = 1).  Unlike utils.h:650, a plane that
  * holds a single position still gets its bias and tanh.
  */
+size_t ftk_grid_rnn_workspace_bytes(int D, int H);
 int ftk_grid_rnn_f32(const float* xs, const float* ys, const float* Wx,
                      const float* Ux, const float* bx, const float* Wy,
                      const float* Uy, const float* by, float* hsss, int D,
                      int L1, int L2, int B, int H, int bias_rows, int crossed,
+                     void* workspace, size_t workspace_bytes,
                      ftk_stream_t stream);
 
 /*

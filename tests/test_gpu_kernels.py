@@ -758,6 +758,10 @@ def test_grid_rnn(core, D, L1, L2, B, H, bias_rows, shared, crossed):
     out = core.grid_rnn(*dev, crossed=crossed)
     assert out.shape == (D, L1, L2, 2, B, H)
     np.testing.assert_allclose(out.cpu().numpy(), ref, rtol=1e-4, atol=1e-5)
+    # the kernel that reads the parameters where they lie adds the same products in the same order
+    assert torch.equal(core.grid_rnn(*dev, crossed=crossed, relay_weights=False), out)
+    # a workspace too small for the re-laid copy selects that kernel too
+    assert torch.equal(core.grid_rnn(*dev, crossed=crossed, workspace=torch.empty(64, dtype=torch.uint8, device='cuda')), out)
     # the output array is also where neighbours are read back: a poisoned one must give the same result
     poisoned = torch.full_like(out, float('nan'))
     core.grid_rnn(*dev, crossed=crossed, out=poisoned)
