@@ -243,7 +243,7 @@ def _grid_torch_planes(torch, xs, ys, W, U, b, D, L, B, H):
     return run, A
 
 
-def bench_grid_rnn(torch, core, steps, warmup, cpu):
+def bench_grid_rnn(torch, core, steps, warmup, cpu, baselines=True):
     """The reference's grid benchmark shape (stacked_grid_rnn.cu:108-118, run.sh:7: batch 32, depth 32, hidden 256,
     both lengths 10; shared parameters, a bias row per batch row), fp32, one launch per plane."""
     D, L, B, H = 32, 10, 32, 256
@@ -259,11 +259,12 @@ def bench_grid_rnn(torch, core, steps, warmup, cpu):
         core._ptr(xs), core._ptr(ys), core._ptr(W), core._ptr(U), core._ptr(b), core._ptr(W), core._ptr(U), core._ptr(b),
         core._ptr(out), ci(D), ci(L), ci(L), ci(B), ci(H), ci(B), ci(0), core._ptr(ws), ctypes.c_size_t(ws.numel()), core._stream()))
     ms, _ = _events_ms(torch, run, steps, warmup)
-    ms_plain, _ = _events_ms(torch, lambda: core.grid_rnn(xs, ys, W, U, b, W, U, b, out=out, relay_weights=False), steps, warmup)
-    run()
-    base, A = _grid_torch_planes(torch, xs, ys, W, U, b, D, L, B, H)
-    ms_t, _ = _events_ms(torch, base, max(2, steps // 5), 1)
-    err = (A[1:, 1:, 1:] - out).abs().max().item()
+    if baselines:
+        ms_plain, _ = _events_ms(torch, lambda: core.grid_rnn(xs, ys, W, U, b, W, U, b, out=out, relay_weights=False), steps, warmup)
+        run()
+        base, A = _grid_torch_planes(torch, xs, ys, W, U, b, D, L, B, H)
+        ms_t, _ = _events_ms(torch, base, max(2, steps // 5), 1)
+        err = (A[1:, 1:, 1:] - out).abs().max().item()
     npos = D * L * L
     # k per position: H of input per direction; H per neighbour that exists, once (shared parameters: the state
     # product serves both directions)
@@ -278,9 +279,10 @@ def bench_grid_rnn(torch, core, steps, warmup, cpu):
                      'kernel': 'grid_rnn_plane_kernel<true, 8, true> (50 launches per pass, after two re-lay launches)',
                      'note': 'the whole forward (50 dependent launches) against the fp32 MFMA peak; planes near the '
                              'corners hold a handful of positions, so the chain of launches, not the matrix rate, bounds it'},
-        'torch_per_plane_gather_bmm_scatter': {'ms_per_step': ms_t, 'speedup': ms_t / ms, 'max_abs_diff': err},
-        'without_workspace': {'ms_per_step': ms_plain, 'note': 'parameters read where they lie, no re-laid copy'},
     }
+    if baselines:
+        res['torch_per_plane_gather_bmm_scatter'] = {'ms_per_step': ms_t, 'speedup': ms_t / ms, 'max_abs_diff': err}
+        res['without_workspace'] = {'ms_per_step': ms_plain, 'note': 'parameters read where they lie, no re-laid copy'}
     if cpu:
         from oracle import kaleido_oracle as ko
         Dc = 2
@@ -635,7 +637,7 @@ def main():
     ap.add_argument('--no-extras', action='store_true', help='measure only the chosen workload')
     ap.add_argument('--no-cpu', action='store_true', help='skip the CPU baseline leg')
     ap.add_argument('--no-baselines', action='store_true',
-                    help='LSTM workloads: only the fused kernel (no unfused GPU baseline, per-stage launches, other product mode)')
+                    help='LSTM and grid workloads: only the fused kernel (no unfused GPU baseline, per-stage launches, other product mode, path without workspace)')
     args = ap.parse_args()
     if args.gpus != 1:
         print('bench.py measures one GPU: every workload here is a single-device kernel '
@@ -663,7 +665,7 @@ def main():
         'gemm': lambda s, w, c: bench_gemm(torch, core, max(5, s // 5), max(2, w // 5), c),
         'online_softmax': lambda s, w, c: bench_softmax(torch, core, s, w, c),
         'embedding': lambda s, w, c: bench_embedding(torch, core, s, w, c),
-        'grid_rnn': lambda s, w, c: bench_grid_rnn(torch, core, max(5, s // 2), max(2, w // 2), c),
+        'grid_rnn': lambda s, w, c: bench_grid_rnn(torch, core, max(5, s // 2), max(2, w // 2), c, not args.no_baselines),
         'windowed_attention': lambda s, w, c: bench_windowed_attention(torch, core, s, w, c),
     }
     if args.workload == 'copy':
