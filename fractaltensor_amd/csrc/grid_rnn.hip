@@ -73,9 +73,9 @@ struct ChunkRegs {
 };
 
 // One k chunk of a product: lane (jl, hh) holds activation row jl, k = 16*hh .. 16*hh+15, and column jl of the
-// weight rows with the same k.  PACKED: the lane's sixteen weights are 64 contiguous bytes of the re-laid copy
-// (four loads instead of sixteen: a wave can keep 63 loads in flight, so fewer instructions per chunk mean more
-// bytes in flight), wcol then points at the lane's slot of chunk 0 and chunks are 1024 floats apart.
+// weight rows with the same k.  PACKED: the lane's sixteen weights are four 16-byte pieces of the re-laid copy,
+// 1 KB apart (four loads instead of sixteen, each covering 1 KB of consecutive bytes across the wave); wcol then
+// points at the lane's first piece of chunk 0 and chunks are 1024 floats apart.
 template <bool PACKED>
 __device__ __forceinline__ void load_chunk(ChunkRegs& r, const float* __restrict__ arow, const float* __restrict__ wcol,
                                            int H, int c) {
@@ -85,7 +85,7 @@ __device__ __forceinline__ void load_chunk(ChunkRegs& r, const float* __restrict
     const float4* wp = reinterpret_cast<const float4*>(wcol + (size_t)c * 1024);
 #pragma unroll
     for (int e4 = 0; e4 < 4; ++e4) {
-      const float4 t = wp[e4];
+      const float4 t = wp[64 * e4];  // one load instruction of the wave covers 1 KB of consecutive bytes
       r.b[4 * e4] = t.x; r.b[4 * e4 + 1] = t.y; r.b[4 * e4 + 2] = t.z; r.b[4 * e4 + 3] = t.w;
     }
   } else {
@@ -94,14 +94,15 @@ __device__ __forceinline__ void load_chunk(ChunkRegs& r, const float* __restrict
   }
 }
 
-// Re-lays M [D][rows][H] (rows a multiple of 32) as [D][H/32 unit blocks][rows/32 chunks][64 lanes][16]: element e of
-// lane (jl, hh) of chunk c of unit block ub is M[32c + 16hh + e][32ub + jl] -- the order load_chunk reads.
+// Re-lays M [D][rows][H] (rows a multiple of 32) as [D][H/32 unit blocks][rows/32 chunks][4][64 lanes][4]: element
+// 4*e4 + t of lane (jl, hh) of chunk c of unit block ub is M[32c + 16hh + 4*e4 + t][32ub + jl] -- the order
+// load_chunk reads, one 16-byte piece per lane and load, so that a load instruction covers 1 KB of consecutive bytes.
 __global__ __launch_bounds__(256) void grid_pack_weights_kernel(const float* __restrict__ M, float* __restrict__ out,
                                                                 long long total4, int rows, int H) {
   const int ctot = rows / GKC, nub = H / 32;
   for (long long idx = (long long)blockIdx.x * 256 + threadIdx.x; idx < total4; idx += (long long)gridDim.x * 256) {
-    const int e4 = (int)(idx & 3);
-    const int lane = (int)((idx >> 2) & 63);
+    const int lane = (int)(idx & 63);
+    const int e4 = (int)((idx >> 6) & 3);
     const long long rest = idx >> 8;
     const int c = (int)(rest % ctot);
     const int ub = (int)((rest / ctot) % nub);
@@ -208,7 +209,7 @@ void grid_rnn_plane_kernel(GridArgs a) {
     const int cps = H / GKC;                       // chunks per product
     const int ctot = kind == 0 ? cps : 2 * cps;    // chunks of the whole matrix: U holds both state products
     const float* base = kind == 0 ? a.Wp[dir] + (size_t)d * H * H : a.Up[dir] + (size_t)d * 2 * H * H;
-    w = base + ((size_t)ub * ctot + (kind == 2 ? cps : 0)) * 1024 + lane * 16;
+    w = base + ((size_t)ub * ctot + (kind == 2 ? cps : 0)) * 1024 + lane * 4;
   } else {
     const float* Ud = a.U[dir] + (size_t)d * 2 * H * H;
     const float* base = kind == 0 ? a.W[dir] + (size_t)d * H * H : kind == 1 ? Ud : Ud + (size_t)H * H;
