@@ -127,7 +127,7 @@ __device__ __forceinline__ void mfma_chunk(v16f& acc, const ChunkRegs& r) {
 // register set behind the MFMAs that read it and ahead of the next set's MFMAs, so the wait the compiler puts
 // before a set's MFMAs leaves the younger refills outstanding.  That only works where no load sits under a
 // run-time condition (at a join the compiler must assume the path with the fewest younger loads and ends up
-// waiting for all of them), hence the chunk count as a template argument for the usual hidden sizes; NCH = 0 is
+// waiting for all of them), hence the chunk count as a template argument for the usual hidden sizes (128, 256, 384, 512, 768, 1024); NCH = 0 is
 // the form for any other count.  NS is 3 with the parameters where they lie (20 loads per chunk: a wave cannot
 // have more than 63 outstanding) and 2 with the re-laid copy (8 loads per chunk; 3 to 6 sets measured slower,
 // 1.21 to 1.53 ms against 1.17 ms for H = 256, as did one).
@@ -322,6 +322,9 @@ extern "C" int ftk_grid_rnn_f32(const float* xs, const float* ys, const float* W
     if (H == 256) FTK_GRID_LAUNCH(8);
     else if (H == 512) FTK_GRID_LAUNCH(16);
     else if (H == 1024) FTK_GRID_LAUNCH(32);
+    else if (H == 128) FTK_GRID_LAUNCH(4);
+    else if (H == 384) FTK_GRID_LAUNCH(12);
+    else if (H == 768) FTK_GRID_LAUNCH(24);
     else FTK_GRID_LAUNCH(0);
 #undef FTK_GRID_LAUNCH
 #undef FTK_GRID_LAUNCH_P

@@ -749,6 +749,8 @@ def _grid_inputs(D, L1, L2, B, H, bias_rows, shared, crossed, seed=0):
     (2, 2, 3, 1, 128, 1, False, True),      # one sample
     (2, 3, 3, 32, 512, 1, True, False),     # the other two hidden sizes of the benchmark's sweep (run.sh:8-9)
     (1, 2, 2, 33, 1024, 33, False, False),
+    (2, 2, 2, 8, 384, 1, True, True),       # hidden sizes with a chunk loop of their own besides the benchmark's three
+    (1, 3, 2, 32, 768, 0, False, False),
 ])
 def test_grid_rnn(core, D, L1, L2, B, H, bias_rows, shared, crossed):
     """fp32 MFMA products against the float64 recurrence: 1e-4, the tolerance of the fp32 LSTM path."""
