@@ -24,6 +24,17 @@ the checks live in ``tests/test_oracle.py``):
 * attention / flash_attention_blockwise / md_merge / online_softmax: pinned
   by torch softmax / scaled_dot_product_attention, rows summing to one,
   block-partition invariance, uniform-key => mean(V).
+* grid_rnn / grid_rnn_batched (checks in ``tests/test_frontend.py``): pinned by
+  the corner position and one interior position worked by hand from their
+  neighbours, by the eager nested-scan program built from the frontend's own
+  operators, by equality of the two layouts sample by sample, and by the grid
+  of width one, which is a plain stacked tanh RNN written directly.
+* window_positions / windowed_attention (``tests/test_frontend.py``): pinned by
+  hand-worked windows including both wrapped ends, by torch softmax on
+  explicit index lists, and by the eager shifted_slide + sparse_attn program.
+  The reference holds no expected output for either model; the windowed
+  access operators themselves (slide, window, ...) are "parity unpinned" in
+  the sense that only their source and documentation fix them.
 """
 from __future__ import annotations
 
