@@ -61,6 +61,26 @@ def test_argument_errors_come_back_as_codes_not_crashes():
     assert lib.ftk_stacked_lstm_f16_workspace_bytes(2, 3, 4, 1024) == 2 * 2048 * 4096 * 2
     assert lib.ftk_stacked_lstm_workspace_bytes(32, 64, 256, 256) > 0
     assert lib.ftk_stacked_lstm_workspace_bytes(0, 64, 256, 256) == 0
+    # grid RNN: null operands, a hidden size that is no multiple of 32, bias rows that are neither 1 nor B, one bias only
+    cz, cf = ctypes.c_size_t, ctypes.c_float
+    grid = lambda *p, H=32, rows=1, bx=one, by=one: lib.ftk_grid_rnn_f32(*p, bx, one, one, by, one, ci(1), ci(2), ci(2), ci(4), ci(H),
+                                                                         ci(rows), ci(0), nul, cz(0), nul)
+    assert grid(nul, one, one, one) == -1
+    assert grid(one, one, one, one, H=48) == -2
+    assert grid(one, one, one, one, rows=3) == -1
+    assert grid(one, one, one, one, by=nul) == -1
+    assert lib.ftk_grid_rnn_workspace_bytes(32, 256) == 2 * 32 * 3 * 256 * 256 * 4
+    assert lib.ftk_grid_rnn_workspace_bytes(0, 256) == 0
+    # windowed attention: even window, head size off the 16-byte pieces, a span longer than the sequence, indices without a count
+    wa = lambda S=8, D=16, W=3, dl=1, R=0, idx=nul, q=one: lib.ftk_windowed_attn_f32(q, one, one, idx, one, ci(1), ci(S), ci(D), ci(W),
+                                                                                       ci(dl), ci(R), cf(1.0), nul)
+    assert wa(q=nul) == -1
+    assert wa(W=4) == -2
+    assert wa(D=6) == -2
+    assert wa(W=5, dl=4) == -2
+    assert wa(idx=one) == -1
+    assert wa(R=2) == -1
+    assert wa(q=ctypes.c_void_p(8)) == -1          # not 16-byte aligned
 
 
 def test_wrappers_refuse_cpu_tensors():
