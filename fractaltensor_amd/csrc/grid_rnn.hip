@@ -18,7 +18,8 @@
 // chunk the k index is permuted so that a lane's activation values are 64 contiguous bytes: step (q, e) uses
 // k = 4q + e for lanes 0-31 and k = 16 + 4q + e for lanes 32-63.  The products are added through LDS before bias
 // and tanh.  Given a workspace, the entry point first re-lays the parameters so that the sixteen weights a lane
-// needs of a chunk are 64 contiguous bytes (four loads instead of sixteen strided ones).
+// needs of a chunk come in four loads that each cover 1 KB of consecutive bytes, and the kernel then also loads the
+// activations as whole 128-byte row segments and turns them round through a wave-private LDS tile.
 //
 // Placement.  Workgroups are numbered position-major, unit block fastest, and ids go round the eight XCDs: with
 // eight unit blocks (H = 256) an XCD only ever touches one 32-column slice of every block's parameters.  (Running
@@ -72,16 +73,20 @@ struct ChunkRegs {
   float b[16];
 };
 
-// One k chunk of a product: lane (jl, hh) holds activation row jl, k = 16*hh .. 16*hh+15, and column jl of the
-// weight rows with the same k.  PACKED: the lane's sixteen weights are four 16-byte pieces of the re-laid copy,
-// 1 KB apart (four loads instead of sixteen, each covering 1 KB of consecutive bytes across the wave); wcol then
-// points at the lane's first piece of chunk 0 and chunks are 1024 floats apart.
+// One k chunk of a product.  Without the re-laid copy lane (jl, hh) loads what the MFMAs want of it: activation row
+// jl at k = 16*hh .. 16*hh+15 and column jl of the weight rows with the same k.  PACKED: every load instruction
+// covers whole cache lines -- what a CU runs out of here is the rate at which its L1 takes lines, not bytes.  The
+// lane's sixteen weights are four 16-byte pieces of the re-laid copy, 1 KB apart (four loads instead of sixteen,
+// each 1 KB of consecutive bytes across the wave; wcol points at the lane's first piece of chunk 0, chunks are
+// 1024 floats apart), and the activations come as row segments: load q brings rows 8q .. 8q+7 of the chunk, 128
+// consecutive bytes each (8 lines per load instead of 32), lane l holding floats 4*(l%8)..+3 of row 8q + l/8
+// (row_off); mfma_chunk turns them round.
 template <bool PACKED>
 __device__ __forceinline__ void load_chunk(ChunkRegs& r, const float* __restrict__ arow, const float* __restrict__ wcol,
-                                           int H, int c) {
-#pragma unroll
-  for (int q = 0; q < 4; ++q) r.a[q] = *reinterpret_cast<const float4*>(arow + c * GKC + 4 * q);
+                                           int H, int c, const int (&row_off)[4]) {
   if constexpr (PACKED) {
+#pragma unroll
+    for (int q = 0; q < 4; ++q) r.a[q] = *reinterpret_cast<const float4*>(arow + row_off[q] + c * GKC);
     const float4* wp = reinterpret_cast<const float4*>(wcol + (size_t)c * 1024);
 #pragma unroll
     for (int e4 = 0; e4 < 4; ++e4) {
@@ -89,6 +94,8 @@ __device__ __forceinline__ void load_chunk(ChunkRegs& r, const float* __restrict
       r.b[4 * e4] = t.x; r.b[4 * e4 + 1] = t.y; r.b[4 * e4 + 2] = t.z; r.b[4 * e4 + 3] = t.w;
     }
   } else {
+#pragma unroll
+    for (int q = 0; q < 4; ++q) r.a[q] = *reinterpret_cast<const float4*>(arow + c * GKC + 4 * q);
 #pragma unroll
     for (int e = 0; e < 16; ++e) r.b[e] = wcol[(size_t)(c * GKC + e) * H];
   }
@@ -113,13 +120,39 @@ __global__ __launch_bounds__(256) void grid_pack_weights_kernel(const float* __r
   }
 }
 
-__device__ __forceinline__ void mfma_chunk(v16f& acc, const ChunkRegs& r) {
+constexpr int kTurnLd = GKC + 4;  // padded row of a wave's 32 x 32 turn-round tile in LDS (floats)
+typedef __attribute__((address_space(3))) float lds_float;
+
+// TURN: r.a holds row segments; they go through the wave's own LDS tile and come back as the MFMAs want them (lane
+// (jl, hh): row jl, k = 16*hh + 4q..+3).  LDS operations of one wave execute in order, so the tile needs no second
+// buffer and no barrier.  The pointer carries its address space: through a generic pointer the compiler emits
+// flat loads and stores, which made this twice as slow as not turning at all.
+template <bool TURN>
+__device__ __forceinline__ void mfma_chunk(v16f& acc, const ChunkRegs& r, lds_float* turn) {
+  float4 a[4];
+  if constexpr (TURN) {
+    const int lane = threadIdx.x & 63;
+    typedef __attribute__((address_space(3))) v4f lds_v4f;
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      const v4f t = {r.a[q].x, r.a[q].y, r.a[q].z, r.a[q].w};
+      *reinterpret_cast<lds_v4f*>(turn + (8 * q + (lane >> 3)) * kTurnLd + 4 * (lane & 7)) = t;
+    }
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      const v4f t = *reinterpret_cast<lds_v4f*>(turn + (lane & 31) * kTurnLd + 16 * (lane >> 5) + 4 * q);
+      a[q] = make_float4(t[0], t[1], t[2], t[3]);
+    }
+  } else {
+#pragma unroll
+    for (int q = 0; q < 4; ++q) a[q] = r.a[q];
+  }
 #pragma unroll
   for (int q = 0; q < 4; ++q) {
-    acc = __builtin_amdgcn_mfma_f32_32x32x2f32(r.a[q].x, r.b[4 * q + 0], acc, 0, 0, 0);
-    acc = __builtin_amdgcn_mfma_f32_32x32x2f32(r.a[q].y, r.b[4 * q + 1], acc, 0, 0, 0);
-    acc = __builtin_amdgcn_mfma_f32_32x32x2f32(r.a[q].z, r.b[4 * q + 2], acc, 0, 0, 0);
-    acc = __builtin_amdgcn_mfma_f32_32x32x2f32(r.a[q].w, r.b[4 * q + 3], acc, 0, 0, 0);
+    acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a[q].x, r.b[4 * q + 0], acc, 0, 0, 0);
+    acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a[q].y, r.b[4 * q + 1], acc, 0, 0, 0);
+    acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a[q].z, r.b[4 * q + 2], acc, 0, 0, 0);
+    acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a[q].w, r.b[4 * q + 3], acc, 0, 0, 0);
   }
 }
 
@@ -132,35 +165,36 @@ __device__ __forceinline__ void mfma_chunk(v16f& acc, const ChunkRegs& r) {
 // have more than 63 outstanding) and 2 with the re-laid copy (8 loads per chunk; 3 to 6 sets measured slower,
 // 1.21 to 1.53 ms against 1.17 ms for H = 256, as did one).
 template <int NCH, bool PACKED, int NS>
-__device__ __forceinline__ void product(v16f& acc, const float* __restrict__ arow, const float* __restrict__ wcol, int H) {
+__device__ __forceinline__ void product(v16f& acc, const float* __restrict__ arow, const float* __restrict__ wcol, int H,
+                                        const int (&row_off)[4], lds_float* turn) {
   auto fence = [] { __builtin_amdgcn_sched_barrier(0); };
   if constexpr (NCH >= NS) {
     H = NCH * GKC;  // known at compile time: the weight rows' addresses become constant offsets
     ChunkRegs r[NS];
-    static_for<NS>([&](auto s) { load_chunk<PACKED>(r[s], arow, wcol, H, s); fence(); });
+    static_for<NS>([&](auto s) { load_chunk<PACKED>(r[s], arow, wcol, H, s, row_off); fence(); });
     constexpr int MAIN = NCH / NS - 1;  // rounds all of whose refills exist
     for (int k = 0; k < MAIN; ++k) {
       static_for<NS>([&](auto s) {
-        mfma_chunk(acc, r[s]); fence();
-        load_chunk<PACKED>(r[s], arow, wcol, H, NS * (k + 1) + s); fence();
+        mfma_chunk<PACKED>(acc, r[s], turn); fence();
+        load_chunk<PACKED>(r[s], arow, wcol, H, NS * (k + 1) + s, row_off); fence();
       });
     }
     constexpr int CE = NS * MAIN;  // the sets hold chunks CE .. CE+NS-1; fewer than NS more follow
     static_for<NS>([&](auto s) {
-      mfma_chunk(acc, r[s]); fence();
-      if constexpr (CE + NS + s < NCH) { load_chunk<PACKED>(r[s], arow, wcol, H, CE + NS + s); fence(); }
+      mfma_chunk<PACKED>(acc, r[s], turn); fence();
+      if constexpr (CE + NS + s < NCH) { load_chunk<PACKED>(r[s], arow, wcol, H, CE + NS + s, row_off); fence(); }
     });
     static_for<NS>([&](auto s) {
-      if constexpr (CE + NS + s < NCH) { mfma_chunk(acc, r[s]); fence(); }
+      if constexpr (CE + NS + s < NCH) { mfma_chunk<PACKED>(acc, r[s], turn); fence(); }
     });
   } else {
     ChunkRegs r0, r1;
     const int nch = H / GKC;
     for (int c = 0; c < nch; c += 2) {  // two chunks per round, the second one clamped (and then not used)
-      load_chunk<PACKED>(r0, arow, wcol, H, c);
-      load_chunk<PACKED>(r1, arow, wcol, H, min(c + 1, nch - 1));
-      mfma_chunk(acc, r0);
-      if (c + 1 < nch) mfma_chunk(acc, r1);
+      load_chunk<PACKED>(r0, arow, wcol, H, c, row_off);
+      load_chunk<PACKED>(r1, arow, wcol, H, min(c + 1, nch - 1), row_off);
+      mfma_chunk<PACKED>(acc, r0, turn);
+      if (c + 1 < nch) mfma_chunk<PACKED>(acc, r1, turn);
     }
   }
 }
@@ -174,6 +208,7 @@ __global__ __launch_bounds__(SHARED ? 256 : 384) __attribute__((amdgpu_waves_per
 void grid_rnn_plane_kernel(GridArgs a) {
   constexpr int JOBS = SHARED ? 4 : 6;
   __shared__ float red[JOBS][16][64];
+  __shared__ __attribute__((aligned(16))) float turn_tiles[PACKED ? JOBS : 1][PACKED ? 32 * kTurnLd : 4];
 
   const int H = a.H, B = a.B;
   const int nub = H / 32, nrb = (B + 31) / 32;
@@ -220,8 +255,16 @@ void grid_rnn_plane_kernel(GridArgs a) {
 #pragma unroll
   for (int r = 0; r < 16; ++r) acc[r] = 0.0f;
   if (act) {
-    const int row = min(rb * 32 + jl, B - 1);
-    product<NCH, PACKED, PACKED ? 2 : 3>(acc, act + (size_t)row * H + 16 * hh, w, H);
+    int row_off[4] = {0, 0, 0, 0};
+    lds_float* turn = (lds_float*)&turn_tiles[PACKED ? wave : 0][0];
+    if (PACKED) {
+#pragma unroll
+      for (int q = 0; q < 4; ++q) row_off[q] = min(rb * 32 + 8 * q + (lane >> 3), B - 1) * H + 4 * (lane & 7);
+      product<NCH, true, 2>(acc, act, w, H, row_off, turn);
+    } else {
+      const int row = min(rb * 32 + jl, B - 1);
+      product<NCH, false, 3>(acc, act + (size_t)row * H + 16 * hh, w, H, row_off, turn);
+    }
   }
 #pragma unroll
   for (int r = 0; r < 16; ++r) red[wave][r][lane] = acc[r];
