@@ -15,11 +15,10 @@
 // products otherwise.  A product whose state lies outside the grid is skipped.  Each wave runs its product on
 // v_mfma_f32_32x32x2_f32 straight from global memory -- no operand is used by a second wave of the workgroup, so
 // LDS staging would only add barriers -- with the operands of the next two or three k chunks of 32 in registers.  Within a
-// chunk the k index is permuted so that a lane's activation values are 64 contiguous bytes: step (q, e) uses
-// k = 4q + e for lanes 0-31 and k = 16 + 4q + e for lanes 32-63.  The products are added through LDS before bias
+// chunk the k index is permuted: step (q, e) uses k = 4q + e for lanes 0-31 and k = 16 + 4q + e for lanes 32-63.  The products are added through LDS before bias
 // and tanh.  Given a workspace, the entry point first re-lays the parameters so that the sixteen weights a lane
-// needs of a chunk come in four loads that each cover 1 KB of consecutive bytes, and the kernel then also loads the
-// activations as whole 128-byte row segments and turns them round through a wave-private LDS tile.
+// needs of a chunk come in four loads that each cover 1 KB of consecutive bytes.  The activations are loaded as whole
+// 128-byte row segments and turned round through a wave-private LDS tile.
 //
 // Placement.  Workgroups are numbered position-major, unit block fastest, and ids go round the eight XCDs: with
 // eight unit blocks (H = 256) an XCD only ever touches one 32-column slice of every block's parameters.  (Running
@@ -73,20 +72,20 @@ struct ChunkRegs {
   float b[16];
 };
 
-// One k chunk of a product.  Without the re-laid copy lane (jl, hh) loads what the MFMAs want of it: activation row
-// jl at k = 16*hh .. 16*hh+15 and column jl of the weight rows with the same k.  PACKED: every load instruction
-// covers whole cache lines -- what a CU runs out of here is the rate at which its L1 takes lines, not bytes.  The
-// lane's sixteen weights are four 16-byte pieces of the re-laid copy, 1 KB apart (four loads instead of sixteen,
-// each 1 KB of consecutive bytes across the wave; wcol points at the lane's first piece of chunk 0, chunks are
-// 1024 floats apart), and the activations come as row segments: load q brings rows 8q .. 8q+7 of the chunk, 128
-// consecutive bytes each (8 lines per load instead of 32), lane l holding floats 4*(l%8)..+3 of row 8q + l/8
-// (row_off); mfma_chunk turns them round.
+// One k chunk of a product.  Every load instruction is made to cover whole cache lines -- what a CU runs out of
+// here is the rate at which its L1 takes lines, not bytes.  The activations come as row segments: load q brings
+// rows 8q .. 8q+7 of the chunk, 128 consecutive bytes each (8 lines per load; loading what the MFMAs want of a
+// lane, 16 values of one row, touches 32), lane l holding floats 4*(l%8)..+3 of row 8q + l/8 (row_off);
+// mfma_chunk turns them round.  Weights: lane (jl, hh) needs column jl of the weight rows k = 16*hh .. 16*hh+15.
+// PACKED: they are four 16-byte pieces of the re-laid copy, 1 KB apart (four loads instead of sixteen, each 1 KB of
+// consecutive bytes across the wave; wcol points at the lane's first piece of chunk 0, chunks are 1024 floats
+// apart); otherwise sixteen loads of one value each, where they lie.
 template <bool PACKED>
 __device__ __forceinline__ void load_chunk(ChunkRegs& r, const float* __restrict__ arow, const float* __restrict__ wcol,
                                            int H, int c, const int (&row_off)[4]) {
-  if constexpr (PACKED) {
 #pragma unroll
-    for (int q = 0; q < 4; ++q) r.a[q] = *reinterpret_cast<const float4*>(arow + row_off[q] + c * GKC);
+  for (int q = 0; q < 4; ++q) r.a[q] = *reinterpret_cast<const float4*>(arow + row_off[q] + c * GKC);
+  if constexpr (PACKED) {
     const float4* wp = reinterpret_cast<const float4*>(wcol + (size_t)c * 1024);
 #pragma unroll
     for (int e4 = 0; e4 < 4; ++e4) {
@@ -94,8 +93,6 @@ __device__ __forceinline__ void load_chunk(ChunkRegs& r, const float* __restrict
       r.b[4 * e4] = t.x; r.b[4 * e4 + 1] = t.y; r.b[4 * e4 + 2] = t.z; r.b[4 * e4 + 3] = t.w;
     }
   } else {
-#pragma unroll
-    for (int q = 0; q < 4; ++q) r.a[q] = *reinterpret_cast<const float4*>(arow + c * GKC + 4 * q);
 #pragma unroll
     for (int e = 0; e < 16; ++e) r.b[e] = wcol[(size_t)(c * GKC + e) * H];
   }
@@ -123,14 +120,13 @@ __global__ __launch_bounds__(256) void grid_pack_weights_kernel(const float* __r
 constexpr int kTurnLd = GKC + 4;  // padded row of a wave's 32 x 32 turn-round tile in LDS (floats)
 typedef __attribute__((address_space(3))) float lds_float;
 
-// TURN: r.a holds row segments; they go through the wave's own LDS tile and come back as the MFMAs want them (lane
+// r.a holds row segments; they go through the wave's own LDS tile and come back as the MFMAs want them (lane
 // (jl, hh): row jl, k = 16*hh + 4q..+3).  LDS operations of one wave execute in order, so the tile needs no second
 // buffer and no barrier.  The pointer carries its address space: through a generic pointer the compiler emits
 // flat loads and stores, which made this twice as slow as not turning at all.
-template <bool TURN>
 __device__ __forceinline__ void mfma_chunk(v16f& acc, const ChunkRegs& r, lds_float* turn) {
   float4 a[4];
-  if constexpr (TURN) {
+  {
     const int lane = threadIdx.x & 63;
     typedef __attribute__((address_space(3))) v4f lds_v4f;
 #pragma unroll
@@ -143,9 +139,6 @@ __device__ __forceinline__ void mfma_chunk(v16f& acc, const ChunkRegs& r, lds_fl
       const v4f t = *reinterpret_cast<lds_v4f*>(turn + (lane & 31) * kTurnLd + 16 * (lane >> 5) + 4 * q);
       a[q] = make_float4(t[0], t[1], t[2], t[3]);
     }
-  } else {
-#pragma unroll
-    for (int q = 0; q < 4; ++q) a[q] = r.a[q];
   }
 #pragma unroll
   for (int q = 0; q < 4; ++q) {
@@ -175,17 +168,17 @@ __device__ __forceinline__ void product(v16f& acc, const float* __restrict__ aro
     constexpr int MAIN = NCH / NS - 1;  // rounds all of whose refills exist
     for (int k = 0; k < MAIN; ++k) {
       static_for<NS>([&](auto s) {
-        mfma_chunk<PACKED>(acc, r[s], turn); fence();
+        mfma_chunk(acc, r[s], turn); fence();
         load_chunk<PACKED>(r[s], arow, wcol, H, NS * (k + 1) + s, row_off); fence();
       });
     }
     constexpr int CE = NS * MAIN;  // the sets hold chunks CE .. CE+NS-1; fewer than NS more follow
     static_for<NS>([&](auto s) {
-      mfma_chunk<PACKED>(acc, r[s], turn); fence();
+      mfma_chunk(acc, r[s], turn); fence();
       if constexpr (CE + NS + s < NCH) { load_chunk<PACKED>(r[s], arow, wcol, H, CE + NS + s, row_off); fence(); }
     });
     static_for<NS>([&](auto s) {
-      if constexpr (CE + NS + s < NCH) { mfma_chunk<PACKED>(acc, r[s], turn); fence(); }
+      if constexpr (CE + NS + s < NCH) { mfma_chunk(acc, r[s], turn); fence(); }
     });
   } else {
     ChunkRegs r0, r1;
@@ -193,8 +186,8 @@ __device__ __forceinline__ void product(v16f& acc, const float* __restrict__ aro
     for (int c = 0; c < nch; c += 2) {  // two chunks per round, the second one clamped (and then not used)
       load_chunk<PACKED>(r0, arow, wcol, H, c, row_off);
       load_chunk<PACKED>(r1, arow, wcol, H, min(c + 1, nch - 1), row_off);
-      mfma_chunk<PACKED>(acc, r0, turn);
-      if (c + 1 < nch) mfma_chunk<PACKED>(acc, r1, turn);
+      mfma_chunk(acc, r0, turn);
+      if (c + 1 < nch) mfma_chunk(acc, r1, turn);
     }
   }
 }
@@ -208,7 +201,7 @@ __global__ __launch_bounds__(SHARED ? 256 : 384) __attribute__((amdgpu_waves_per
 void grid_rnn_plane_kernel(GridArgs a) {
   constexpr int JOBS = SHARED ? 4 : 6;
   __shared__ float red[JOBS][16][64];
-  __shared__ __attribute__((aligned(16))) float turn_tiles[PACKED ? JOBS : 1][PACKED ? 32 * kTurnLd : 4];
+  __shared__ __attribute__((aligned(16))) float turn_tiles[JOBS][32 * kTurnLd];
 
   const int H = a.H, B = a.B;
   const int nub = H / 32, nrb = (B + 31) / 32;
@@ -255,16 +248,12 @@ void grid_rnn_plane_kernel(GridArgs a) {
 #pragma unroll
   for (int r = 0; r < 16; ++r) acc[r] = 0.0f;
   if (act) {
-    int row_off[4] = {0, 0, 0, 0};
-    lds_float* turn = (lds_float*)&turn_tiles[PACKED ? wave : 0][0];
-    if (PACKED) {
+    // load q of a chunk: row 8q + lane/8 of the row block, floats 4*(lane%8)..+3
+    int row_off[4];
 #pragma unroll
-      for (int q = 0; q < 4; ++q) row_off[q] = min(rb * 32 + 8 * q + (lane >> 3), B - 1) * H + 4 * (lane & 7);
-      product<NCH, true, 2>(acc, act, w, H, row_off, turn);
-    } else {
-      const int row = min(rb * 32 + jl, B - 1);
-      product<NCH, false, 3>(acc, act + (size_t)row * H + 16 * hh, w, H, row_off, turn);
-    }
+    for (int q = 0; q < 4; ++q) row_off[q] = min(rb * 32 + 8 * q + (lane >> 3), B - 1) * H + 4 * (lane & 7);
+    lds_float* turn = (lds_float*)&turn_tiles[wave][0];
+    product<NCH, PACKED, PACKED ? 2 : 3>(acc, act, w, H, row_off, turn);
   }
 #pragma unroll
   for (int r = 0; r < 16; ++r) red[wave][r][lane] = acc[r];

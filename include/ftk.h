@@ -254,7 +254,7 @@ int ftk_stacked_lstm_wavefront_f32(const float* xs, const float* WU,
  * workspace: 16-byte aligned device memory of ftk_grid_rnn_workspace_bytes(D, H)
  * bytes (half of it suffices with shared parameters) into which every call
  * first re-lays the parameters in the order the kernel's lanes read them; with
- * NULL or less room the kernel reads the parameters where they lie (about 12 %
+ * NULL or less room the kernel reads the parameters where they lie (about 10 %
  * slower).
  * Replaces the eight wavefront regions of
  * benchmarks/rnn/fractaltensor/grid_lstm/regions/region1.h-region8.h (general
