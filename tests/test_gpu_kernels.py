@@ -165,6 +165,8 @@ def products(core, request):
     (2, 40, 1, None, True),            # one sequence
     (4, 9, 32, [1, 2, 4, 8], True),    # dilated, one 32-row block
     (6, 12, 256, [1, 2, 4, 8, 16, 32], False),  # config 5 layer structure, short sequence
+    (6, 72, 64, [1, 2, 4, 8, 16, 32], True),    # config 5 dilations with T > 2*32: the recurrences at d = 16 and 32 are live
+    (2, 70, 40, [32, 16], False),               # the long links first; second row block holds 8 rows
 ])
 def test_stacked_lstm_persistent(core, products, L, T, B, dil, bias):
     H = 256
@@ -209,6 +211,7 @@ def test_split_products_are_as_accurate_as_fp32_products(core):
     (3, 12, 100, None, 'linear'),              # lengths fall from T to 1 across the batch: blocks end one after another
     (2, 9, 64, None, 'two'),                   # half the rows stop after 4 steps
     (4, 16, 96, [1, 2, 4, 8], 'linear'),       # dilated stack
+    (6, 80, 96, [1, 2, 4, 8, 16, 32], 'linear'),   # config 5 dilations, rows ending all along the d = 16 / 32 links
     (2, 6, 40, None, 'full'),                  # nothing ragged about it: same as the dense entry point
 ])
 def test_stacked_lstm_ragged_rows(core, products, L, T, B, dil, lengths):
@@ -239,6 +242,7 @@ def test_stacked_lstm_ragged_rows(core, products, L, T, B, dil, lengths):
     (128, 3, 12, 300, None, 'linear'),         # two 256-row blocks; the second ends early, then rows of the first
     (512, 2, 8, 64, None, 'two'),
     (96, 3, 10, 40, [1, 2, 4], 'linear'),      # 32 hidden units per workgroup (three chunks in a row), dilated
+    (128, 3, 44, 48, [1, 16, 32], 'linear'),   # links of 16 and 32 steps with a live state behind them
 ])
 def test_streamed_stack_ragged_rows(core, products, H, L, T, B, dil, lengths):
     """The streamed stacks (hidden sizes other than 256) on a ragged batch: a cell computes the rows that live at
@@ -297,6 +301,10 @@ def test_stacked_lstm_ragged_rejects_unsorted_rows(core):
     (256, 2, 5, 37, None, True, False),             # odd batch at H = 256 goes the streamed way
     (192, 2, 7, 64, None, True, True),
     (96, 9, 3, 20, None, False, False),             # nine cells in a stage: a second round over the XCDs
+    (256, 6, 72, 64, [1, 2, 4, 8, 16, 32], True, False),    # config 5 dilations with live links of 16 and 32 steps
+    (512, 3, 70, 32, [1, 16, 32], False, False),
+    (1024, 3, 40, 32, [1, 16, 32], True, False),
+    (256, 3, 70, 64, [4, 16, 32], True, True),              # ... and rows that stop after 4 steps
 ])
 def test_stacked_lstm_f16(core, H, L, T, B, dil, bias, ragged):
     rng = np.random.default_rng(13)
@@ -320,7 +328,8 @@ def test_stacked_lstm_f16(core, H, L, T, B, dil, bias, ragged):
     # most values agree to the bit: the two only part where a value sat within rounding of a tie (more often
     # the longer the fp32 sums, and every difference is carried on through time and layers)
     same = np.mean(got_h == hr.astype(np.float32)[:, live])
-    assert same > (0.9 if H <= 512 else 0.8), same
+    # (a rounding tie that fell the other way is carried on: long, deep stacks keep fewer identical values)
+    assert same > (0.7 if L * T > 150 else 0.9 if H <= 512 else 0.8), same
 
 
 def test_stacked_lstm_f16_rejects_other_hidden_sizes(core):
@@ -407,6 +416,26 @@ def test_stacked_lstm_config4_full_size(core, products):
     assert torch.equal(h1, h3)
 
 
+def test_dilated_lstm_config5_full_size(core, products):
+    """L 6, dilations 1..32, B 256, T 128, H 256 (link lengths 2^i of dilated_lstm/region2.h:55-77,
+    examples/dilated_rnn/dilated_rnn.py:16-41): persistent kernel vs per-stage launches on the GPU, and vs the
+    float64 oracle on a subset of batch rows (rows never interact)."""
+    L, T, B, H = 6, 128, 256, 256
+    dil = [1, 2, 4, 8, 16, 32]
+    xs, WU, _ = lstm_inputs(4321, L, T, B, H, 1.0 / 16, bias=False)
+    dx, dW = dev(xs), dev(WU)
+    ws = torch.empty(core.stacked_lstm_workspace_bytes(L, T, B, H), dtype=torch.uint8, device='cuda')
+    h1, c1 = core.stacked_lstm(dx, dW, dilations=dil, workspace=ws)
+    assert core.persistent_status(ws) == 0, 'a dependency wait timed out'
+    h2, c2 = core.stacked_lstm(dx, dW, dilations=dil, schedule='wavefront')
+    torch.cuda.synchronize()
+    e12 = max(ko.max_rel_err(h1.cpu().numpy(), h2.cpu().numpy()), ko.max_rel_err(c1.cpu().numpy(), c2.cpu().numpy()))
+    assert e12 <= LSTM_TOL / 4, f'persistent vs per-stage launches: {e12:.3e}'
+    rows = [0, 31, 32, 100, 255]
+    hr, cr = ko.stacked_lstm(xs[:, rows], WU, None, dilations=dil)
+    assert_lstm_close(h1[:, :, rows], hr, 'hsss rows'); assert_lstm_close(c1[:, :, rows], cr, 'csss rows')
+
+
 @pytest.mark.parametrize('L,T,B,H,dil,bias', [
     (2, 4, 48, 512, None, True),
     (2, 4, 48, 1024, None, True),
@@ -414,6 +443,7 @@ def test_stacked_lstm_config4_full_size(core, products):
     (2, 5, 33, 64, None, True),
     (9, 3, 20, 128, None, True),            # nine cells in a stage
     (2, 7, 1, 320, [1, 3], True),           # one sequence
+    (3, 40, 33, 128, [1, 16, 32], True),    # links of 16 and 32 steps with a live state behind them
 ])
 def test_stacked_lstm_other_hidden_sizes_through_the_default_entry(core, products, L, T, B, H, dil, bias):
     """H != 256 is not what the persistent kernel holds on chip: the default entry point runs one launch per stage
