@@ -21,6 +21,7 @@ EXPORTS = (
     'ftk_lstm_cell_f32', 'ftk_lstm_cell_f16', 'ftk_lstm_layer_f32', 'ftk_lstm_layer_f16', 'ftk_lstm_elementwise_f32',
     'ftk_stacked_lstm_workspace_bytes', 'ftk_stacked_lstm_f32', 'ftk_dilated_lstm_f32',
     'ftk_stacked_lstm_wavefront_f32', 'ftk_stacked_lstm_ragged_f32', 'ftk_lstm_set_products', 'ftk_lstm_get_products',
+    'ftk_stacked_lstm_opts_f32', 'ftk_stacked_lstm_status',
     'ftk_stacked_lstm_f16_workspace_bytes', 'ftk_stacked_lstm_f16',
     'ftk_b2b_gemm_f16', 'ftk_b2b_gemm_rowmajor_f16', 'ftk_gemm_f16', 'ftk_batched_gemm_f16', 'ftk_flash_attn_f16', 'ftk_online_softmax_f32', 'ftk_embedding_gather_f32',
     'ftk_grid_rnn_workspace_bytes', 'ftk_grid_rnn_f32', 'ftk_windowed_attn_f32',
@@ -34,6 +35,11 @@ class FtkError(RuntimeError):
     def __init__(self, code: int, message: str):
         super().__init__(f'libftkernels error {code}: {message}')
         self.code = code
+
+
+class LstmOptions(ctypes.Structure):
+    """ftk_lstm_options of include/ftk.h."""
+    _fields_ = [('products', ctypes.c_int), ('spin_limit', ctypes.c_int)]
 
 
 class DeviceInfo(ctypes.Structure):
@@ -91,6 +97,29 @@ def _req(t: torch.Tensor, dtype, name: str) -> torch.Tensor:
     if not t.is_contiguous():
         raise ValueError(f'{name} must be contiguous')
     return t
+
+
+def _req_out(t: torch.Tensor, dtype, shape, name: str) -> torch.Tensor:
+    """A caller-supplied output: the kernels write the full shape, so anything smaller would be overrun."""
+    if not isinstance(t, torch.Tensor):
+        raise TypeError(f'{name} must be a torch.Tensor')
+    if tuple(t.shape) != tuple(shape):
+        raise ValueError(f'{name} must be {tuple(shape)}, got {tuple(t.shape)}')
+    return _req(t, dtype, name)
+
+
+def _req_workspace(t: torch.Tensor) -> torch.Tensor:
+    if not isinstance(t, torch.Tensor) or not t.is_cuda or not t.is_contiguous():
+        raise ValueError('workspace must be a contiguous CUDA tensor')
+    return t
+
+
+# calls of the fused entry points made through this binding, by name (what routed an operator program here)
+launch_counts: dict = {}
+
+
+def _count(name: str) -> None:
+    launch_counts[name] = launch_counts.get(name, 0) + 1
 
 
 def version() -> int:
@@ -175,16 +204,18 @@ def lstm_elementwise(gates, bias, c_prev, out: Optional[Tuple[torch.Tensor, torc
     _req(gates, f32, 'gates')
     B, H4 = gates.shape
     H = H4 // 4
-    if bias is not None:
-        _req(bias, f32, 'bias')
-    if c_prev is not None:
-        _req(c_prev, f32, 'c_prev')
+    if gates.dim() != 2 or H4 % 4:
+        raise ValueError(f'gates must be [B, 4H], got {tuple(gates.shape)}')
+    if bias is not None and _req(bias, f32, 'bias').numel() != 4 * H:
+        raise ValueError('bias must have 4H elements')
+    if c_prev is not None and tuple(_req(c_prev, f32, 'c_prev').shape) != (B, H):
+        raise ValueError(f'c_prev must be [{B}, {H}], got {tuple(c_prev.shape)}')
     if out is None:
         h = torch.empty((B, H), dtype=f32, device=gates.device)
         c = torch.empty((B, H), dtype=f32, device=gates.device)
     else:
         h, c = out
-        _req(h, f32, 'h'); _req(c, f32, 'c')
+        _req_out(h, f32, (B, H), 'h'); _req_out(c, f32, (B, H), 'c')
     _check(lib.ftk_lstm_elementwise_f32(_ptr(gates), _ptr(bias), _ptr(c_prev), _ptr(h), _ptr(c),
                                         ctypes.c_int(B), ctypes.c_int(H), _stream()))
     return h, c
@@ -197,13 +228,19 @@ def stacked_lstm_workspace_bytes(L: int, T: int, B: int, H: int) -> int:
 def stacked_lstm(xs, WU, bias=None, dilations: Optional[Sequence[int]] = None, schedule: str = 'auto',
                  out: Optional[Tuple[torch.Tensor, torch.Tensor]] = None,
                  workspace: Optional[torch.Tensor] = None,
-                 active_rows: Optional[Sequence[int]] = None) -> Tuple[torch.Tensor, torch.Tensor]:
+                 active_rows: Optional[Sequence[int]] = None, products: Optional[str] = None,
+                 spin_limit: int = 0, check: Optional[bool] = None) -> Tuple[torch.Tensor, torch.Tensor]:
     """xs [T,B,H], WU [L,2H,4H], bias [L,4H] or None -> hsss, csss [L,T,B,H].
 
     schedule: 'auto' (persistent kernel when the shape allows, else per-stage
     launches) or 'wavefront' (always per-stage launches).
     active_rows: for a ragged time-major batch (rows sorted by decreasing length), the number of rows still
     running at each step; only the live (t, row) places of the outputs are defined then.
+    products: 'f32' / 'f16x3' for this call, None for the process-wide mode (set_lstm_products).
+    spin_limit: polls a bounded wait of the persistent kernel makes before giving up (0 = the default).
+    check: wait for the stream and raise FtkError (code -6) if the persistent launch gave up a wait and left
+    the outputs incomplete.  Default: True when the workspace is allocated here (nobody else could look at its
+    status word afterwards), False when the caller passes one (check it with stacked_lstm_check(workspace)).
     """
     f32 = torch.float32
     _req(xs, f32, 'xs'); _req(WU, f32, 'WU')
@@ -218,7 +255,10 @@ def stacked_lstm(xs, WU, bias=None, dilations: Optional[Sequence[int]] = None, s
         csss = torch.empty((L, T, B, H), dtype=f32, device=xs.device)
     else:
         hsss, csss = out
-        _req(hsss, f32, 'hsss'); _req(csss, f32, 'csss')
+        _req_out(hsss, f32, (L, T, B, H), 'hsss'); _req_out(csss, f32, (L, T, B, H), 'csss')
+    if products is not None and products not in LSTM_PRODUCTS:
+        raise ValueError(f"products must be one of {sorted(LSTM_PRODUCTS)} or None, got {products!r}")
+    _count('stacked_lstm')
     dil = None
     if dilations is not None:
         if len(dilations) != L:
@@ -232,13 +272,22 @@ def stacked_lstm(xs, WU, bias=None, dilations: Optional[Sequence[int]] = None, s
     if schedule != 'auto':
         raise ValueError("schedule must be 'auto' or 'wavefront'")
     need = stacked_lstm_workspace_bytes(L, T, B, H)
+    if check is None:
+        check = workspace is None
     if workspace is None:
         workspace = torch.empty(need, dtype=torch.uint8, device=xs.device)
+    _req_workspace(workspace)
     ws_bytes = ctypes.c_size_t(workspace.numel() * workspace.element_size())
+    act = None
     if active_rows is not None:
         if len(active_rows) != T:
             raise ValueError('active_rows must have one entry per step')
         act = (ctypes.c_int * T)(*[int(v) for v in active_rows])
+    if products is not None or spin_limit:
+        opts = LstmOptions(LSTM_PRODUCTS[products] if products is not None else -1, int(spin_limit))
+        _check(lib.ftk_stacked_lstm_opts_f32(_ptr(xs), _ptr(WU), _ptr(bias), dil, act, _ptr(hsss), _ptr(csss), ci(L), ci(T),
+                                             ci(B), ci(H), ctypes.byref(opts), _ptr(workspace), ws_bytes, _stream()))
+    elif act is not None:
         _check(lib.ftk_stacked_lstm_ragged_f32(_ptr(xs), _ptr(WU), _ptr(bias), dil, act, _ptr(hsss), _ptr(csss),
                                                ci(L), ci(T), ci(B), ci(H), _ptr(workspace), ws_bytes, _stream()))
     elif dil is None:
@@ -247,12 +296,22 @@ def stacked_lstm(xs, WU, bias=None, dilations: Optional[Sequence[int]] = None, s
     else:
         _check(lib.ftk_dilated_lstm_f32(_ptr(xs), _ptr(WU), _ptr(bias), dil, _ptr(hsss), _ptr(csss),
                                         ci(L), ci(T), ci(B), ci(H), _ptr(workspace), ws_bytes, _stream()))
+    if check:
+        stacked_lstm_check(workspace)
     return hsss, csss
+
+
+def stacked_lstm_check(workspace: torch.Tensor) -> None:
+    """Waits for the current stream and raises FtkError (code -6) if the last stacked-LSTM call given this
+    workspace drained early because a bounded wait of the persistent kernel ran out."""
+    _req_workspace(workspace)
+    _check(lib.ftk_stacked_lstm_status(_ptr(workspace), _stream()))
 
 
 def stacked_lstm_f16(xs, WU, bias=None, dilations: Optional[Sequence[int]] = None,
                      out: Optional[Tuple[torch.Tensor, torch.Tensor]] = None, workspace: Optional[torch.Tensor] = None,
-                     active_rows: Optional[Sequence[int]] = None) -> Tuple[torch.Tensor, torch.Tensor]:
+                     active_rows: Optional[Sequence[int]] = None, check: Optional[bool] = None
+                     ) -> Tuple[torch.Tensor, torch.Tensor]:
     """fp16 storage: xs [T,B,H], WU [L,2H,4H] fp16, bias [L,4H] fp32 or None -> hsss, csss [L,T,B,H] fp16.
     H a multiple of 32: H = 512, and H = 256 with an even batch, run in the persistent kernel, every other
     shape as one launch of the streaming cell kernel per stage of independent cells."""
@@ -269,7 +328,8 @@ def stacked_lstm_f16(xs, WU, bias=None, dilations: Optional[Sequence[int]] = Non
         csss = torch.empty((L, T, B, H), dtype=f16, device=xs.device)
     else:
         hsss, csss = out
-        _req(hsss, f16, 'hsss'); _req(csss, f16, 'csss')
+        _req_out(hsss, f16, (L, T, B, H), 'hsss'); _req_out(csss, f16, (L, T, B, H), 'csss')
+    _count('stacked_lstm_f16')
     dil = None
     if dilations is not None:
         if len(dilations) != L:
@@ -280,11 +340,17 @@ def stacked_lstm_f16(xs, WU, bias=None, dilations: Optional[Sequence[int]] = Non
         if len(active_rows) != T:
             raise ValueError('active_rows must have one entry per step')
         act = (ctypes.c_int * T)(*[int(v) for v in active_rows])
+    if check is None:
+        check = workspace is None
     if workspace is None:
         workspace = torch.empty(int(lib.ftk_stacked_lstm_f16_workspace_bytes(L, T, B, H)), dtype=torch.uint8, device=xs.device)
+    _req_workspace(workspace)
     ci = ctypes.c_int
     _check(lib.ftk_stacked_lstm_f16(_ptr(xs), _ptr(WU), _ptr(bias), dil, act, _ptr(hsss), _ptr(csss), ci(L), ci(T), ci(B),
-                                    ci(H), _ptr(workspace), ctypes.c_size_t(workspace.numel()), _stream()))
+                                    ci(H), _ptr(workspace), ctypes.c_size_t(workspace.numel() * workspace.element_size()),
+                                    _stream()))
+    if check:
+        stacked_lstm_check(workspace)
     return hsss, csss
 
 
@@ -330,7 +396,8 @@ def b2b_gemm(A, B_nk, C_pn, out: Optional[torch.Tensor] = None) -> torch.Tensor:
     if B_nk.shape != (G, N, K) or C_pn.shape != (G, P, N):
         raise ValueError(f'shape mismatch: A {tuple(A.shape)}, B_nk {tuple(B_nk.shape)}, C_pn {tuple(C_pn.shape)}')
     D = out if out is not None else torch.empty((G, M, P), dtype=f16, device=A.device)
-    _req(D, f16, 'D')
+    _req_out(D, f16, (G, M, P), 'D')
+    _count('b2b_gemm')
     ci = ctypes.c_int
     _check(lib.ftk_b2b_gemm_f16(_ptr(A), _ptr(B_nk), _ptr(C_pn), _ptr(D), ci(G), ci(M), ci(N), ci(K), ci(P), _stream()))
     return D[0] if squeeze and out is None else D
@@ -355,7 +422,8 @@ def b2b_gemm_rowmajor(A, B, C, out: Optional[torch.Tensor] = None) -> torch.Tens
     if B.shape != (G, K, N) or C.shape != (G, N, P):
         raise ValueError(f'shape mismatch: A {tuple(A.shape)}, B {tuple(B.shape)}, C {tuple(C.shape)}')
     D = out if out is not None else torch.empty((G, M, P), dtype=f16, device=A.device)
-    _req(D, f16, 'D')
+    _req_out(D, f16, (G, M, P), 'D')
+    _count('b2b_gemm_rowmajor')
     ci = ctypes.c_int
     _check(lib.ftk_b2b_gemm_rowmajor_f16(_ptr(A), _ptr(B), _ptr(C), _ptr(D), ci(G), ci(M), ci(N), ci(K), ci(P), _stream()))
     return D[0] if squeeze and out is None else D
@@ -375,7 +443,7 @@ def gemm(A, B, out: Optional[torch.Tensor] = None) -> torch.Tensor:
     if B.shape[-2] != K or (batched and B.shape[0] != G):
         raise ValueError(f'shape mismatch: A {tuple(A.shape)}, B {tuple(B.shape)}')
     C = out if out is not None else torch.empty((*A.shape[:-1], N), dtype=f16, device=A.device)
-    _req(C, f16, 'C')
+    _req_out(C, f16, (*A.shape[:-1], N), 'C')
     ci = ctypes.c_int
     if batched:
         _check(lib.ftk_batched_gemm_f16(_ptr(A), _ptr(B), _ptr(C), ci(G), ci(M), ci(N), ci(K), _stream()))
@@ -395,7 +463,8 @@ def flash_attention(Q, K, V, scale: Optional[float] = None, out: Optional[torch.
     if scale is None:
         scale = D ** -0.5
     O = out if out is not None else torch.empty_like(Q)
-    _req(O, f16, 'O')
+    _req_out(O, f16, Q.shape, 'O')
+    _count('flash_attention')
     ci = ctypes.c_int
     _check(lib.ftk_flash_attn_f16(_ptr(Q), _ptr(K), _ptr(V), _ptr(O), ci(B), ci(Hd), ci(Sq), ci(Skv), ci(D),
                                   ctypes.c_float(scale), _stream()))

@@ -40,6 +40,10 @@ inline int check_launch(const char* what) {
       return ::ftk::fail(FTK_ERR_LAUNCH, "%s: %s", #call, hipGetErrorString(e_)); \
   } while (0)
 
+// Every workspace a stacked-LSTM entry point takes starts with this block; its first int is the status word
+// that ftk_stacked_lstm_status() reads.
+constexpr size_t kStatusBytes = 256;
+
 // Device properties, queried once per device id.
 struct DeviceProps {
   int cus = 0;

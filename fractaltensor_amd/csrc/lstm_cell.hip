@@ -1005,10 +1005,10 @@ __global__ __launch_bounds__(256) void lstm_pack_split_weights_kernel(const floa
 
 static size_t round256s(size_t v) { return (v + 255) / 256 * 256; }
 
-// Workspace of the split-product stack: [wscale L*4H][wmul L*4H][xratio T*B] floats, then fp16 [xp T*B*2H]
-// [hp L*T*B*2H][packed weights L*6H*4H], every part on a 256-byte boundary.
+// Workspace of the split-product stack: [status block][wscale L*4H][wmul L*4H][xratio T*B] floats, then fp16
+// [xp T*B*2H][hp L*T*B*2H][packed weights L*6H*4H], every part on a 256-byte boundary.
 size_t split_stack_workspace_bytes(int L, int T, int B, int H) {
-  size_t n = 2 * round256s((size_t)L * 4 * H * sizeof(float)) + round256s((size_t)T * B * sizeof(float));
+  size_t n = kStatusBytes + 2 * round256s((size_t)L * 4 * H * sizeof(float)) + round256s((size_t)T * B * sizeof(float));
   n += round256s((size_t)T * B * 2 * H * sizeof(_Float16)) + round256s((size_t)L * T * B * 2 * H * sizeof(_Float16));
   n += (size_t)L * 6 * H * 4 * H * sizeof(_Float16);
   return n;
@@ -1017,7 +1017,7 @@ size_t split_stack_workspace_bytes(int L, int T, int B, int H) {
 // The fp32 stack through the split flavour of the streaming cell kernel (H a multiple of 32).
 int run_wavefront_split(const float* xs, const float* WU, const float* bias, const int* dil, const int* active, float* hsss,
                         float* csss, int L, int T, int B, int H, void* ws, hipStream_t s) {
-  char* p = reinterpret_cast<char*>(ws);
+  char* p = reinterpret_cast<char*>(ws) + kStatusBytes;
   float* wscale = reinterpret_cast<float*>(p);
   p += round256s((size_t)L * 4 * H * sizeof(float));
   float* wmul = reinterpret_cast<float*>(p);

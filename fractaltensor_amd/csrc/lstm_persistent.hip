@@ -838,6 +838,9 @@ static size_t workspace_need(int L, int T, int B) {
   return hsp_offset_bytes(L, T, B) + (size_t)L * T * B * 2 * PH * sizeof(_Float16);
 }
 
+// Polls a bounded wait makes before it gives up (a poll is a round trip to memory, about 1 us: seconds in all).
+constexpr int kDefaultSpinLimit = 1 << 22;
+
 // 0: fp32 products (v_mfma_f32_32x32x2_f32); 1: split products.  FTK_LSTM_PRODUCTS=f32|f16x3
 // sets the initial value, ftk_lstm_set_products() changes it.
 static int g_products = -1;
@@ -906,7 +909,7 @@ static int persistent_slots(int mode, const void** fn, int* slots) {
 // mode kProductsF32 / kProductsSplit: fp32 xs, WU, hsss, csss, H = 256.  kHalfData: the same arrays in fp16, H = 512.
 static int run_persistent(int mode, const void* xs, const void* WU, const float* bias, const int* dil, const int* active,
                           void* hsss, void* csss, int L, int T, int B, void* ws, size_t ws_bytes, hipStream_t s,
-                          bool* handled) {
+                          bool* handled, int spin_limit = 0) {
   *handled = false;
   const void* fn = nullptr;
   int slots = 0;
@@ -919,7 +922,8 @@ static int run_persistent(int mode, const void* xs, const void* WU, const float*
   if (L > kMaxLayers || L * npc > slots) return FTK_OK;  // cannot pin every layer on its own compute units: fall back
 
   const size_t nflags = flag_count(L, T, B);
-  const size_t need = half ? xratio_offset_bytes(L, T, B) : workspace_need(L, T, B);
+  // only the split products read planes; the other flavours need the status block, the flags and the trace
+  const size_t need = split ? workspace_need(L, T, B) : xratio_offset_bytes(L, T, B);
   if (!ws || ws_bytes < need)
     return fail(FTK_ERR_WORKSPACE, "stacked LSTM needs a %zu-byte workspace, got %zu", need, ws_bytes);
 
@@ -938,6 +942,10 @@ static int run_persistent(int mode, const void* xs, const void* WU, const float*
     a.xratio = nullptr;
     a.xsp = reinterpret_cast<const _Float16*>(xs);
     a.hsp = reinterpret_cast<_Float16*>(hsss);
+  } else if (!split) {  // fp32 products: tiles come from xs and hsss
+    a.xratio = nullptr;
+    a.xsp = nullptr;
+    a.hsp = nullptr;
   } else {
     xratio = reinterpret_cast<float*>(wsb + xratio_offset_bytes(L, T, B));
     xsp = reinterpret_cast<_Float16*>(wsb + xsp_offset_bytes(L, T, B));
@@ -971,7 +979,7 @@ static int run_persistent(int mode, const void* xs, const void* WU, const float*
   for (int l = 0; l < L; ++l) a.first_q[l + 1] = a.first_q[l] + npc * a.pr_of[l];
   for (int l = L; l < kMaxLayers; ++l) { a.pr_of[l] = 1; a.first_q[l + 1] = a.first_q[L]; }
   a.groups = a.first_q[L];
-  a.spin_limit = 1 << 22;
+  a.spin_limit = spin_limit > 0 ? spin_limit : kDefaultSpinLimit;
   a.trace_q = trace_workgroup();
   a.trace = reinterpret_cast<long long*>(reinterpret_cast<char*>(ws) + trace_offset_bytes(L, T, B));
   for (int l = 0; l < kMaxLayers; ++l) a.dil[l] = (l < L && dil) ? dil[l] : 1;
@@ -1028,9 +1036,13 @@ static int check_stack_args(const char* who, const float* xs, const float* WU, f
 
 static int run_stack(const char* who, const float* xs, const float* WU, const float* bias, const int* dil,
                      const int* active, float* hsss, float* csss, int L, int T, int B, int H, void* ws,
-                     size_t ws_bytes, hipStream_t s) {
+                     size_t ws_bytes, hipStream_t s, int products = FTK_LSTM_PRODUCTS_DEFAULT, int spin_limit = 0) {
   int rc = check_stack_args(who, xs, WU, hsss, csss, L, T, B, H, dil);
   if (rc) return rc;
+  if (products == FTK_LSTM_PRODUCTS_DEFAULT) products = products_mode();
+  if (products != FTK_LSTM_PRODUCTS_F32 && products != FTK_LSTM_PRODUCTS_F16X3)
+    return fail(FTK_ERR_INVALID_ARGUMENT, "%s: products = %d is none of FTK_LSTM_PRODUCTS_DEFAULT, _F32, _F16X3", who, products);
+  if (spin_limit < 0) return fail(FTK_ERR_INVALID_ARGUMENT, "%s: spin_limit = %d is negative", who, spin_limit);
   if (active) {
     for (int t = 0; t < T; ++t) {
       if (active[t] < 0 || active[t] > B)
@@ -1042,13 +1054,19 @@ static int run_stack(const char* who, const float* xs, const float* WU, const fl
   }
   if (H == PH) {
     bool handled = false;
-    rc = run_persistent(products_mode() == 1 ? kProductsSplit : kProductsF32, xs, WU, bias, dil, active, hsss, csss, L, T, B,
-                        ws, ws_bytes, s, &handled);
+    rc = run_persistent(products == FTK_LSTM_PRODUCTS_F16X3 ? kProductsSplit : kProductsF32, xs, WU, bias, dil, active,
+                        hsss, csss, L, T, B, ws, ws_bytes, s, &handled, spin_limit);
     if (rc || handled) return rc;
+  }
+  // the launches below wait for nothing: their status word is zero
+  if (ws && ws_bytes >= kStatusBytes) {
+    hipLaunchKernelGGL(fill_zero_kernel, dim3(1), dim3(64), 0, s, reinterpret_cast<int*>(ws), (size_t)(kStatusBytes / sizeof(int)));
+    rc = check_launch("fill_zero_kernel");
+    if (rc) return rc;
   }
   // Other hidden sizes: one launch per stage of independent cells.  With split products (the default) and the
   // workspace the size query asks for, through the fp16-MFMA streaming kernel; else on fp32 MFMAs.
-  if (H != PH && products_mode() == FTK_LSTM_PRODUCTS_F16X3 && ws && ws_bytes >= split_stack_workspace_bytes(L, T, B, H) &&
+  if (H != PH && products == FTK_LSTM_PRODUCTS_F16X3 && ws && ws_bytes >= split_stack_workspace_bytes(L, T, B, H) &&
       (long long)B * H < (1ll << 29))
     return run_wavefront_split(xs, WU, bias, dil, active, hsss, csss, L, T, B, H, ws, s);
   return run_wavefront(xs, WU, bias, dil, hsss, csss, L, T, B, H, s);
@@ -1085,7 +1103,8 @@ size_t ftk_stacked_lstm_workspace_bytes(int L, int T, int B, int H) {
 
 size_t ftk_stacked_lstm_f16_workspace_bytes(int L, int T, int B, int H) {
   if (L <= 0 || T <= 0 || B <= 0 || H <= 0) return 0;
-  const size_t packed = (size_t)L * 2 * H * 4 * H * sizeof(_Float16);  // the re-laid weights of the streaming kernel
+  // the status block and the re-laid weights of the streaming kernel
+  const size_t packed = ftk::kStatusBytes + (size_t)L * 2 * H * 4 * H * sizeof(_Float16);
   if (!ftk::f16_fits_on_chip(B, H)) return packed;
   // which of the two runs is decided per call (a ragged batch stays with the persistent kernel): room for either
   return std::max(ftk::xratio_offset_bytes(L, T, B), ftk::f16_streams(L, B, H, false) ? packed : (size_t)0);
@@ -1120,7 +1139,12 @@ int ftk_stacked_lstm_f16(const void* xs, const void* WU, const float* bias, cons
     const size_t need = ftk_stacked_lstm_f16_workspace_bytes(L, T, B, H);
     if (!workspace || workspace_bytes < need)
       return fail(FTK_ERR_WORKSPACE, "%s: workspace of %zu bytes needed, %zu given", who, need, workspace ? workspace_bytes : (size_t)0);
-    return run_wavefront_f16(xs, WU, bias, dilations, active_rows, hsss, csss, L, T, B, H, workspace, (hipStream_t)stream);
+    hipLaunchKernelGGL(fill_zero_kernel, dim3(1), dim3(64), 0, (hipStream_t)stream, reinterpret_cast<int*>(workspace),
+                       (size_t)(kStatusBytes / sizeof(int)));  // nothing below waits: the status word is zero
+    int rcz = check_launch("fill_zero_kernel");
+    if (rcz) return rcz;
+    return run_wavefront_f16(xs, WU, bias, dilations, active_rows, hsss, csss, L, T, B, H,
+                             reinterpret_cast<char*>(workspace) + kStatusBytes, (hipStream_t)stream);
   }
   const void* fn = nullptr;
   int slots = 0;
@@ -1145,6 +1169,29 @@ int ftk_stacked_lstm_f16(const void* xs, const void* WU, const float* bias, cons
     if (rc) return rc;
     if (!handled) return fail(FTK_ERR_DEVICE, "%s: the persistent kernel cannot run on this device", who);
   }
+  return FTK_OK;
+}
+
+int ftk_stacked_lstm_opts_f32(const float* xs, const float* WU, const float* bias, const int* dilations,
+                              const int* active_rows, float* hsss, float* csss, int L, int T, int B, int H,
+                              const ftk_lstm_options* options, void* workspace, size_t workspace_bytes,
+                              ftk_stream_t stream) {
+  const int products = options ? options->products : FTK_LSTM_PRODUCTS_DEFAULT;
+  const int spin_limit = options ? options->spin_limit : 0;
+  return ftk::run_stack("ftk_stacked_lstm_opts_f32", xs, WU, bias, dilations, active_rows, hsss, csss, L, T, B, H,
+                        workspace, workspace_bytes, (hipStream_t)stream, products, spin_limit);
+}
+
+int ftk_stacked_lstm_status(const void* workspace, ftk_stream_t stream) {
+  using namespace ftk;
+  if (!workspace) return fail(FTK_ERR_INVALID_ARGUMENT, "ftk_stacked_lstm_status: workspace is NULL");
+  int word = 0;
+  FTK_HIP(hipMemcpyAsync(&word, workspace, sizeof(int), hipMemcpyDeviceToHost, (hipStream_t)stream));
+  FTK_HIP(hipStreamSynchronize((hipStream_t)stream));
+  if (word != 0)
+    return fail(FTK_ERR_TIMEOUT,
+                "stacked LSTM: a bounded wait of the persistent launch ran out of polls (status word %d); the launch drained "
+                "early and hsss / csss are incomplete", word);
   return FTK_OK;
 }
 

@@ -37,6 +37,7 @@ extern "C" {
 #define FTK_ERR_WORKSPACE (-3)        /* workspace missing or too small           */
 #define FTK_ERR_LAUNCH (-4)           /* HIP reported an error at launch          */
 #define FTK_ERR_DEVICE (-5)           /* device query failed / not a gfx950 part  */
+#define FTK_ERR_TIMEOUT (-6)          /* a persistent launch gave up waiting: see ftk_stacked_lstm_status() */
 
 typedef void* ftk_stream_t;
 
@@ -221,10 +222,51 @@ int ftk_stacked_lstm_f16(const void* xs, const void* WU, const float* bias,
  * =f16x3 sets the initial mode.  A tuning control of this library: the
  * reference has one fp32 (cuBLAS) and one fp16 (CuTe) LSTM and no switch.
  */
+#define FTK_LSTM_PRODUCTS_DEFAULT (-1)
 #define FTK_LSTM_PRODUCTS_F32 0
 #define FTK_LSTM_PRODUCTS_F16X3 1
+/* The process-wide default (initially F16X3 or what FTK_LSTM_PRODUCTS says).  One
+ * plain int shared by every thread: set it before other threads call the LSTM
+ * entry points, or choose per call through ftk_stacked_lstm_opts_f32 instead. */
 int ftk_lstm_set_products(int mode);
 int ftk_lstm_get_products(void);
+
+/*
+ * The fp32 stack with everything per call: dilations and active_rows as in
+ * the entry points above (host arrays, either may be NULL) plus
+ *   products:   FTK_LSTM_PRODUCTS_F32 / _F16X3, or _DEFAULT for the process-wide
+ *               mode.  With F16X3 non-finite inputs give NaN where fp32
+ *               arithmetic would give +-inf (the remainder plane of an infinite
+ *               value is inf - inf);
+ *   spin_limit: polls a bounded wait of the persistent kernel makes before it
+ *               gives up, 0 = the default (2^22, seconds).
+ * options == NULL means {DEFAULT, 0}.  No counterpart in the reference.
+ */
+typedef struct ftk_lstm_options {
+  int products;
+  int spin_limit;
+} ftk_lstm_options;
+int ftk_stacked_lstm_opts_f32(const float* xs, const float* WU, const float* bias,
+                              const int* dilations, const int* active_rows,
+                              float* hsss, float* csss, int L, int T, int B,
+                              int H, const ftk_lstm_options* options,
+                              void* workspace, size_t workspace_bytes,
+                              ftk_stream_t stream);
+
+/*
+ * Whether the last stacked-LSTM call that was given `workspace` ran to the end.
+ * The persistent kernel synchronises its workgroups through counters in the
+ * workspace; every wait is bounded, and a wait that runs out (workgroups not
+ * co-resident, a lost device) sets the status word -- the first int of every
+ * LSTM workspace, zeroed by every call -- and drains the launch, leaving
+ * hsss / csss partly unwritten.  The entry points have returned 0 by then:
+ * they are asynchronous.  This call WAITS for `stream`, reads the word and
+ * returns FTK_OK or FTK_ERR_TIMEOUT.  Callers must check it (here, or by
+ * reading the word themselves after synchronising) before trusting the
+ * outputs of ftk_stacked_lstm_f32 / _dilated_ / _ragged_ / _opts_ / _f16.
+ * No counterpart in the reference, whose launches do not wait for each other.
+ */
+int ftk_stacked_lstm_status(const void* workspace, ftk_stream_t stream);
 
 /*
  * The same stack evaluated as one batched fused-cell launch per wavefront
@@ -340,8 +382,8 @@ int ftk_batched_gemm_f16(const void* A, const void* B, void* C, int G, int M,
 /*
  * O = softmax(Q K^T * scale) V per (batch, head), non-causal, fp16 storage,
  * fp32 accumulation, online softmax (running max / sum) in registers.
- * Q,O [B,Hd,Sq,D]; K,V [B,Hd,Skv,D].  Needs D==128 or D==64, Sq%64==0... see
- * ftk_last_error() for the exact constraint that failed.
+ * Q,O [B,Hd,Sq,D]; K,V [B,Hd,Skv,D].  D == 128 or D == 64; any Sq, Skv >= 1 (the
+ * last, partial blocks of queries and keys are masked).
  * Replaces the map/reduce program flash_attention
  * (examples/flash_attention/flash_attention.py:14-91); the reference has no
  * device kernel for it.

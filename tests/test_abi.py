@@ -58,7 +58,15 @@ def test_argument_errors_come_back_as_codes_not_crashes():
     assert lib.ftk_stacked_lstm_f16(one, one, nul, nul, nul, one, one, ci(1), ci(1), ci(4), ci(80), nul, ctypes.c_size_t(0), nul) == -2
     # a shape whose weights are streamed needs the workspace for their re-laid copy
     assert lib.ftk_stacked_lstm_f16(one, one, nul, nul, nul, one, one, ci(2), ci(3), ci(4), ci(1024), nul, ctypes.c_size_t(0), nul) == -3
-    assert lib.ftk_stacked_lstm_f16_workspace_bytes(2, 3, 4, 1024) == 2 * 2048 * 4096 * 2
+    # the status block (256 bytes, its first int the status word) and the re-laid weights
+    assert lib.ftk_stacked_lstm_f16_workspace_bytes(2, 3, 4, 1024) == 256 + 2 * 2048 * 4096 * 2
+    # per-call options: an unknown products mode, a negative poll limit; the status query without a workspace
+    opts = core.LstmOptions(7, 0)
+    stack = lambda o: lib.ftk_stacked_lstm_opts_f32(one, one, nul, nul, nul, one, one, ci(1), ci(1), ci(1), ci(32), o, nul,
+                                                    ctypes.c_size_t(0), nul)
+    assert stack(ctypes.byref(opts)) == -1
+    assert stack(ctypes.byref(core.LstmOptions(-1, -5))) == -1
+    assert lib.ftk_stacked_lstm_status(nul, nul) == -1
     assert lib.ftk_stacked_lstm_workspace_bytes(32, 64, 256, 256) > 0
     assert lib.ftk_stacked_lstm_workspace_bytes(0, 64, 256, 256) == 0
     # grid RNN: null operands, a hidden size that is no multiple of 32, bias rows that are neither 1 nor B, one bias only
@@ -81,6 +89,22 @@ def test_argument_errors_come_back_as_codes_not_crashes():
     assert wa(idx=one) == -1
     assert wa(R=2) == -1
     assert wa(q=ctypes.c_void_p(8)) == -1          # not 16-byte aligned
+
+
+def test_wrappers_check_supplied_outputs_before_any_launch():
+    """A caller-supplied output of the wrong shape must never reach a kernel (it would be overrun), and a workspace
+    must be device memory.  The shape is looked at first, so host tensors are enough to show it."""
+    import torch
+    import fractaltensor_amd._core as core
+    f32 = torch.float32
+    with pytest.raises(ValueError, match=r'hsss must be \(2, 3, 4, 32\)'):
+        core._req_out(torch.empty((2, 3, 4, 16), dtype=f32), f32, (2, 3, 4, 32), 'hsss')
+    with pytest.raises(RuntimeError, match='no CPU path'):      # right shape: the next check is the device
+        core._req_out(torch.empty((2, 3, 4, 32), dtype=f32), f32, (2, 3, 4, 32), 'hsss')
+    with pytest.raises(ValueError, match='workspace'):
+        core._req_workspace(torch.empty(16, dtype=torch.uint8))
+    with pytest.raises(ValueError, match='workspace'):
+        core._req_workspace(None)
 
 
 def test_wrappers_refuse_cpu_tensors():

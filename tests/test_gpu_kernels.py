@@ -207,6 +207,48 @@ def test_split_products_are_as_accurate_as_fp32_products(core):
         core.set_lstm_products(before)
 
 
+def test_split_products_at_the_benchmarked_depth(core):
+    """32 layers x 64 steps (config 4's depth): the error of the split products against float64 stays within twice
+    that of the fp32 MFMAs and two orders under the 1e-4 bound after 95 dependent cells too.  Rows are independent,
+    so float64 evaluates a subset of them."""
+    L, T, B, H = 32, 64, 64, 256
+    xs, WU, bs = lstm_inputs(21, L, T, B, H, 1.0 / 16)
+    rows = [0, 31, 32, 63]
+    hr, cr = ko.stacked_lstm(xs[:, rows], WU, bs)                      # float64
+    err = {}
+    for mode in ('f32', 'f16x3'):
+        ws = torch.empty(core.stacked_lstm_workspace_bytes(L, T, B, H), dtype=torch.uint8, device='cuda')
+        hsss, csss = core.stacked_lstm(dev(xs), dev(WU), dev(bs), workspace=ws, products=mode, check=True)
+        err[mode] = max(ko.max_rel_err(hsss[:, :, rows].cpu().numpy(), hr), ko.max_rel_err(csss[:, :, rows].cpu().numpy(), cr))
+    assert err['f16x3'] <= max(2 * err['f32'], 2e-6), err
+    assert err['f16x3'] <= LSTM_TOL / 20, err
+
+
+def test_a_drained_persistent_launch_raises(core):
+    """A bounded wait that gives up must not pass for success.  One poll per wait (set from the host) makes the
+    consumers of layer 1 give up at once: the kernel sets the status word, every workgroup leaves its loop and the
+    launch ends normally; the wrapper then raises instead of returning partly written outputs.  The same call with
+    the default limit succeeds on the same workspace (every call clears the word)."""
+    L, T, B, H = 4, 8, 64, 256
+    xs, WU, bs = lstm_inputs(3, L, T, B, H, 1.0 / 16)
+    ws = torch.empty(core.stacked_lstm_workspace_bytes(L, T, B, H), dtype=torch.uint8, device='cuda')
+    with pytest.raises(core.FtkError) as info:
+        core.stacked_lstm(dev(xs), dev(WU), dev(bs), workspace=ws, spin_limit=1, check=True)
+    assert info.value.code == -6 and 'drained' in str(info.value)
+    with pytest.raises(core.FtkError):
+        core.stacked_lstm_check(ws)                                    # the word stays until the next call
+    # unchecked call with a supplied workspace: no exception, the caller asks afterwards
+    core.stacked_lstm(dev(xs), dev(WU), dev(bs), workspace=ws, spin_limit=1)
+    assert core.persistent_status(ws) == 1
+    hsss, csss = core.stacked_lstm(dev(xs), dev(WU), dev(bs), workspace=ws)
+    core.stacked_lstm_check(ws)
+    hr, cr = c_oracle.stacked_lstm(xs, WU, bs)
+    assert_lstm_close(hsss, hr, 'hsss'); assert_lstm_close(csss, cr, 'csss')
+    # a workspace the wrapper allocates itself is always checked
+    with pytest.raises(core.FtkError):
+        core.stacked_lstm(dev(xs), dev(WU), dev(bs), spin_limit=1)
+
+
 @pytest.mark.parametrize('L,T,B,dil,lengths', [
     (3, 12, 100, None, 'linear'),              # lengths fall from T to 1 across the batch: blocks end one after another
     (2, 9, 64, None, 'two'),                   # half the rows stop after 4 steps
