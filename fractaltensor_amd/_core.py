@@ -21,7 +21,7 @@ EXPORTS = (
     'ftk_lstm_cell_f32', 'ftk_lstm_cell_f16', 'ftk_lstm_layer_f32', 'ftk_lstm_layer_f16', 'ftk_lstm_elementwise_f32',
     'ftk_stacked_lstm_workspace_bytes', 'ftk_stacked_lstm_f32', 'ftk_dilated_lstm_f32',
     'ftk_stacked_lstm_wavefront_f32', 'ftk_stacked_lstm_ragged_f32', 'ftk_lstm_set_products', 'ftk_lstm_get_products',
-    'ftk_stacked_lstm_opts_f32', 'ftk_stacked_lstm_status',
+    'ftk_stacked_lstm_opts_f32', 'ftk_stacked_lstm_status', 'ftk_stacked_lstm_noalloc_f32',
     'ftk_stacked_lstm_f16_workspace_bytes', 'ftk_stacked_lstm_f16',
     'ftk_b2b_gemm_f16', 'ftk_b2b_gemm_rowmajor_f16', 'ftk_gemm_f16', 'ftk_batched_gemm_f16', 'ftk_flash_attn_f16', 'ftk_online_softmax_f32', 'ftk_embedding_gather_f32',
     'ftk_grid_rnn_workspace_bytes', 'ftk_grid_rnn_f32', 'ftk_windowed_attn_f32',
@@ -301,10 +301,36 @@ def stacked_lstm(xs, WU, bias=None, dilations: Optional[Sequence[int]] = None, s
     return hsss, csss
 
 
-def stacked_lstm_check(workspace: torch.Tensor) -> None:
+def stacked_lstm_noalloc(xs, WU, bias, out: Tuple[torch.Tensor, torch.Tensor], dilations: Optional[Sequence[int]] = None) -> None:
+    """ftk_stacked_lstm_noalloc_f32: the fp32-product persistent stack (H = 256) into caller-supplied hsss, csss
+    [L,T,B,H], with the launch's flags in the library's built-in per-device scratch.  Nothing is allocated, here or in
+    the library; the status word is read with stacked_lstm_check(None)."""
+    f32 = torch.float32
+    _req(xs, f32, 'xs'); _req(WU, f32, 'WU')
+    T, B, H = xs.shape
+    L = WU.shape[0]
+    if WU.shape != (L, 2 * H, 4 * H):
+        raise ValueError(f'WU must be [L, 2H, 4H] with H={H}, got {tuple(WU.shape)}')
+    if bias is not None and _req(bias, f32, 'bias').numel() != L * 4 * H:
+        raise ValueError('bias must be [L, 4H]')
+    hsss, csss = out
+    _req_out(hsss, f32, (L, T, B, H), 'hsss'); _req_out(csss, f32, (L, T, B, H), 'csss')
+    dil = None
+    if dilations is not None:
+        if len(dilations) != L:
+            raise ValueError('one dilation per layer')
+        dil = (ctypes.c_int * L)(*[int(d) for d in dilations])
+    ci = ctypes.c_int
+    _check(lib.ftk_stacked_lstm_noalloc_f32(_ptr(xs), _ptr(WU), _ptr(bias), dil, _ptr(hsss), _ptr(csss), ci(L), ci(T), ci(B),
+                                            ci(H), _stream()))
+
+
+def stacked_lstm_check(workspace: Optional[torch.Tensor]) -> None:
     """Waits for the current stream and raises FtkError (code -6) if the last stacked-LSTM call given this
-    workspace drained early because a bounded wait of the persistent kernel ran out."""
-    _req_workspace(workspace)
+    workspace drained early because a bounded wait of the persistent kernel ran out.  None: the built-in scratch
+    that stacked_lstm_noalloc uses on the current device."""
+    if workspace is not None:
+        _req_workspace(workspace)
     _check(lib.ftk_stacked_lstm_status(_ptr(workspace), _stream()))
 
 

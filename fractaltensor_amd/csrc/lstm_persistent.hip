@@ -43,6 +43,7 @@
 #include <stdlib.h>
 
 #include <algorithm>
+#include <mutex>
 #include <type_traits>
 
 #include "ftk_common.h"
@@ -1023,6 +1024,40 @@ static int run_persistent(int mode, const void* xs, const void* WU, const float*
   return FTK_OK;
 }
 
+// Scratch of the entry point that allocates nothing: the status block, the flags and the trace of one persistent
+// launch with fp32 products.  Every device the library runs on holds its own copy until the process ends.  In host
+// code the array's name is only a handle for hipGetSymbolAddress; device code and launches use the address that call
+// returns, kept per device.
+constexpr size_t kScratchBytes = 1u << 20;
+static __device__ __align__(256) unsigned char scratch[kScratchBytes];
+constexpr int kMaxDevices = 64;
+static void* g_scratch_ptr[kMaxDevices] = {};
+static std::mutex g_scratch_mutex;
+
+// The device address of `scratch` on the current device (looked up once per device, with that device current).
+static int scratch_of_current_device(const char* who, void** out, bool lookup) {
+  *out = nullptr;
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) {
+    (void)hipGetLastError();
+    return fail(FTK_ERR_DEVICE, "%s: hipGetDevice: %s", who, hipGetErrorString(e));
+  }
+  if (dev < 0 || dev >= kMaxDevices) return fail(FTK_ERR_DEVICE, "%s: device id %d is outside [0, %d)", who, dev, kMaxDevices);
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  if (!g_scratch_ptr[dev] && lookup) {
+    void* ptr = nullptr;
+    e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || !ptr) {
+      (void)hipGetLastError();
+      return fail(FTK_ERR_DEVICE, "%s: hipGetSymbolAddress(scratch) on device %d: %s", who, dev, hipGetErrorString(e));
+    }
+    g_scratch_ptr[dev] = ptr;
+  }
+  *out = g_scratch_ptr[dev];
+  return FTK_OK;
+}
+
 static int check_stack_args(const char* who, const float* xs, const float* WU, float* hsss, float* csss, int L, int T,
                             int B, int H, const int* dil) {
   if (!xs || !WU || !hsss || !csss) return fail(FTK_ERR_INVALID_ARGUMENT, "%s: xs, WU, hsss, csss must be non-NULL", who);
@@ -1184,7 +1219,13 @@ int ftk_stacked_lstm_opts_f32(const float* xs, const float* WU, const float* bia
 
 int ftk_stacked_lstm_status(const void* workspace, ftk_stream_t stream) {
   using namespace ftk;
-  if (!workspace) return fail(FTK_ERR_INVALID_ARGUMENT, "ftk_stacked_lstm_status: workspace is NULL");
+  if (!workspace) {  // the built-in scratch of ftk_stacked_lstm_noalloc_f32 on the current device
+    void* ptr = nullptr;
+    if (scratch_of_current_device("ftk_stacked_lstm_status", &ptr, false) != FTK_OK || !ptr)
+      return fail(FTK_ERR_INVALID_ARGUMENT,
+                  "ftk_stacked_lstm_status: workspace is NULL and ftk_stacked_lstm_noalloc_f32 has not run on the current device");
+    workspace = ptr;
+  }
   int word = 0;
   FTK_HIP(hipMemcpyAsync(&word, workspace, sizeof(int), hipMemcpyDeviceToHost, (hipStream_t)stream));
   FTK_HIP(hipStreamSynchronize((hipStream_t)stream));
@@ -1192,6 +1233,30 @@ int ftk_stacked_lstm_status(const void* workspace, ftk_stream_t stream) {
     return fail(FTK_ERR_TIMEOUT,
                 "stacked LSTM: a bounded wait of the persistent launch ran out of polls (status word %d); the launch drained "
                 "early and hsss / csss are incomplete", word);
+  return FTK_OK;
+}
+
+int ftk_stacked_lstm_noalloc_f32(const float* xs, const float* WU, const float* bias, const int* dilations, float* hsss,
+                                 float* csss, int L, int T, int B, int H, ftk_stream_t stream) {
+  using namespace ftk;
+  const char* who = "ftk_stacked_lstm_noalloc_f32";
+  int rc = check_stack_args(who, xs, WU, hsss, csss, L, T, B, H, dilations);
+  if (rc) return rc;
+  if (H != PH) return fail(FTK_ERR_UNSUPPORTED_SHAPE, "%s: H = %d; only H = %d runs without a caller workspace", who, H, PH);
+  const size_t need = xratio_offset_bytes(L, T, B);
+  if (need > kScratchBytes)
+    return fail(FTK_ERR_UNSUPPORTED_SHAPE,
+                "%s: L = %d, T = %d, B = %d needs %zu bytes of flags and trace, the built-in scratch holds %zu; use "
+                "ftk_stacked_lstm_opts_f32 with a workspace", who, L, T, B, need, kScratchBytes);
+  void* ptr = nullptr;
+  rc = scratch_of_current_device(who, &ptr, true);
+  if (rc) return rc;
+  bool handled = false;
+  rc = run_persistent(kProductsF32, xs, WU, bias, dilations, nullptr, hsss, csss, L, T, B, ptr, kScratchBytes,
+                      (hipStream_t)stream, &handled, 0);
+  if (rc) return rc;
+  if (!handled)
+    return fail(FTK_ERR_UNSUPPORTED_SHAPE, "%s: %d layers do not fit the device's compute units in one persistent launch", who, L);
   return FTK_OK;
 }
 

@@ -264,9 +264,32 @@ int ftk_stacked_lstm_opts_f32(const float* xs, const float* WU, const float* bia
  * returns FTK_OK or FTK_ERR_TIMEOUT.  Callers must check it (here, or by
  * reading the word themselves after synchronising) before trusting the
  * outputs of ftk_stacked_lstm_f32 / _dilated_ / _ragged_ / _opts_ / _f16.
+ * workspace == NULL: the built-in scratch of ftk_stacked_lstm_noalloc_f32 on
+ * the current device (FTK_ERR_INVALID_ARGUMENT if that has never run there).
  * No counterpart in the reference, whose launches do not wait for each other.
  */
 int ftk_stacked_lstm_status(const void* workspace, ftk_stream_t stream);
+
+/*
+ * ftk_stacked_lstm_opts_f32 with fp32 products for callers that cannot
+ * allocate device memory or pass a workspace: code under HIP graph capture,
+ * tight serving loops, harnesses that forbid hipMalloc.  No counterpart in
+ * the reference.  Same operands and results as ftk_stacked_lstm_opts_f32
+ * with {FTK_LSTM_PRODUCTS_F32, 0} and no active_rows; H must be 256, and the
+ * status block, flags and trace of the launch (about 4*L*T*ceil(B/32) +
+ * 64*T*ceil(B/32) + 256 bytes) must fit the library's built-in scratch of
+ * 1 MiB per device (config 4, L32 T64 B256: 98 KB), else
+ * FTK_ERR_UNSUPPORTED_SHAPE; likewise when L layers do not fit the device in
+ * one persistent launch.  The call allocates nothing, frees nothing and waits
+ * for nothing.  Every call on a device shares that device's scratch: calls
+ * that overlap on one device (two streams, two threads) race; calls on one
+ * stream are safe.  ftk_stacked_lstm_status(NULL, stream) reads the status
+ * word of the current device's scratch.
+ */
+int ftk_stacked_lstm_noalloc_f32(const float* xs, const float* WU,
+                                 const float* bias, const int* dilations,
+                                 float* hsss, float* csss, int L, int T, int B,
+                                 int H, ftk_stream_t stream);
 
 /*
  * The same stack evaluated as one batched fused-cell launch per wavefront
