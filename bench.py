@@ -1,14 +1,16 @@
 #!/usr/bin/env python3
 """Benchmark of the FractalTensor hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload b2b|attention|stacked_lstm|dilated_lstm]
-                    [--no-extras] [--no-cpu]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload b2b|config1|attention|stacked_lstm|dilated_lstm|...]
+                    [--no-extras] [--all] [--no-cpu] [--no-baselines]
 
 Prints ONE JSON line.  The headline workload is BASELINE.json configs[1], the
 fused back-to-back fp16 GEMM (32 problems of [4096,128]x[128,128]x[128,128]);
-the other single-GPU configurations (flash attention, stacked LSTM, dilated
-LSTM) are measured the same way and reported under "other_workloads" unless
---no-extras is given.  A step is one pass of the kernel over one batch of
+the other configurations (the single-layer scan with the host's eager operator
+program beside it, flash attention, stacked LSTM, dilated LSTM) are measured
+the same way and reported under "other_workloads" unless --no-extras is given,
+and summarised in "configs", the last key of the line.  --all adds the
+workloads either side of the path.  A step is one pass of the kernel over one batch of
 synthetic input that is already resident in HBM.  For the B2B GEMM the timed
 steps walk a ring of input sets larger than the 256 MB memory-side cache, so
 the figure is an HBM figure; the same-buffers figure is reported next to it.
@@ -24,6 +26,9 @@ import numpy as np
 
 ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
+
+# BASELINE.json configs[i] -> key of the compact per-configuration summary
+CONFIG_OF = {'config1': 'configs[0]', 'b2b': 'configs[1]', 'attention': 'configs[2]', 'stacked_lstm': 'configs[3]', 'dilated_lstm': 'configs[4]'}
 
 # MI355X published peaks (dense)
 PEAK_HBM_GBS = 8000.0
@@ -423,6 +428,7 @@ def bench_lstm(torch, core, steps, warmup, cpu, dilated, baselines=True):
     products = core.get_lstm_products()          # 'f16x3' unless FTK_LSTM_PRODUCTS says otherwise
     ms, wall = _events_ms(torch, fused, steps, warmup)
     status = core.persistent_status(ws)
+    assert status == 0, 'the persistent launch drained early'
     ref_h = hs.clone()
     executed = 3.0 * flop if products == 'f16x3' else flop      # MFMA flops the kernel issues
     peak = PEAK_F16_TFLOPS if products == 'f16x3' else PEAK_F32_MATRIX_TFLOPS
@@ -448,6 +454,7 @@ def bench_lstm(torch, core, steps, warmup, cpu, dilated, baselines=True):
             hs_b.zero_()
             ms_graph, _ = _events_ms(torch, graph.replay, nb, 2)
         base_err = float((hs_b - ref_h).abs().max() / ref_h.abs().max())
+        assert base_err <= 1e-4 and other_diff <= 1e-4, f'fused stack differs from its baselines: {base_err:.3e}, {other_diff:.3e}'
         ms_base = ms_graph if ms_graph is not None else ms_eager
         # the same stack on a ragged batch: row lengths fall linearly from T to T/4 across the (sorted) batch
         lens = [max(1, T - (3 * T * b) // (4 * B)) for b in range(B)]
@@ -479,10 +486,14 @@ def bench_lstm(torch, core, steps, warmup, cpu, dilated, baselines=True):
         'tflops': flop / ms / 1e9,
         'frac_of_f32_matrix_peak_algorithmic': flop / ms / 1e9 / PEAK_F32_MATRIX_TFLOPS,
         'persistent_status': status,
-        # executed MFMA flops (three f16 products per algorithmic product in the default mode) against the
-        # peak of the MFMA type that executes them
-        'roofline': {'bound': 'mfma', 'achieved': executed / ms / 1e9, 'peak': peak, 'unit': 'TFLOP/s',
-                     'frac': executed / ms / 1e9 / peak,
+        # algorithmic flops (2*B*2H*4H per cell) against the peak of the arithmetic the path is specified in, fp32
+        # matrix; the default mode forms each product from three f16 MFMAs, which is how the fraction passes 1.
+        # The MFMA flops actually issued, against the peak of the MFMA type that executes them, are given beside it.
+        'roofline': {'bound': 'mfma', 'achieved': flop / ms / 1e9, 'peak': PEAK_F32_MATRIX_TFLOPS, 'unit': 'TFLOP/s',
+                     'frac': flop / ms / 1e9 / PEAK_F32_MATRIX_TFLOPS,
+                     'executed': {'achieved': executed / ms / 1e9, 'peak': peak, 'frac': executed / ms / 1e9 / peak,
+                                  'what': 'MFMA flops issued (three f16 products per fp32 product in f16x3 mode) against '
+                                          'the peak of the MFMA type that executes them'},
                      'traffic': MEASURED_TRAFFIC_BYTES.get('lstm_persistent_kernel' + ('_dilated' if dilated else '')),
                      'kernel': 'lstm_persistent_kernel'},
     }
@@ -501,6 +512,100 @@ def bench_lstm(torch, core, steps, warmup, cpu, dilated, baselines=True):
         res['cpu_baseline'] = {'value': B / full_seconds, 'unit': 'sequences/s', 'cores': 1, 'kind': 'port',
                                'sample': f'{Ls} layers x {Ts} steps x {Bs} rows through oracle/oracle.c in {dt:.1f} s, '
                                          f'scaled by cell-rows to the full configuration'}
+    return res
+
+
+def _host_threads():
+    """Threads for the host legs: the physical cores, capped at the 16 a one-GPU box gives a job."""
+    try:
+        import psutil
+        n = psutil.cpu_count(logical=False) or os.cpu_count() or 1
+    except Exception:
+        n = os.cpu_count() or 1
+    return max(1, min(16, n))
+
+
+def bench_config1(torch, core, steps, warmup, cpu):
+    """BASELINE.json configs[0]: one LSTM layer, B 64, T 16, H 256, fp32.  The reference runs this as its eager operator
+    program on the host (examples/stacked_rnn/stacked_rnn.py:13-80); that program, written against this package's
+    operators (fractaltensor_amd/programs.py), is the cpu_eager leg: per-sample [1,H] tensors, scan over time, map
+    over batch, four gate products per cell, on torch CPU.  The batched leg is the same arithmetic as one
+    [64,512] @ [512,1024] product per step, which separates operator dispatch from host GEMM speed."""
+    from fractaltensor_amd import programs
+    from fractaltensor_amd.kaleido.operations import fused
+    L, T, B, H = 1, 16, 64, 256
+    flop = 2.0 * L * T * B * (2 * H) * (4 * H)
+    Wss, Uss, bss = programs.make_lstm_params(L, H, 0.1, 1234, bias=False)
+    xss = programs.make_sequence_batch(T, B, H, 1234)
+    xs = xss.as_dense().reshape(T, B, H).cuda()
+    W, U = Wss.as_dense(), Uss.as_dense()                      # [L, 4, H, H]
+    WU = torch.cat([W.permute(0, 2, 1, 3).reshape(L, H, 4 * H), U.permute(0, 2, 1, 3).reshape(L, H, 4 * H)], dim=1).contiguous()
+    WUd = WU.cuda()
+    hs = torch.empty((L, T, B, H), device='cuda')
+    cs = torch.empty_like(hs)
+    ws = torch.empty(core.stacked_lstm_workspace_bytes(L, T, B, H), dtype=torch.uint8, device='cuda')
+    ms, wall = _events_ms(torch, lambda: core.stacked_lstm(xs, WUd, out=(hs, cs), workspace=ws), steps, warmup)
+    core.stacked_lstm_check(ws)
+    nbytes = 4.0 * (T * B * H + L * 2 * H * 4 * H + 2 * L * T * B * H)
+    res = {
+        'metric': 'stacked-LSTM sequences/s', 'value': B / ms * 1e3, 'unit': 'sequences/s', 'ms_per_step': ms,
+        'dtype': 'f32 (gate products as three f16 MFMAs of split operands, f32 accumulate)' if core.get_lstm_products() == 'f16x3' else 'f32',
+        'config': {'workload': 'single-layer LSTM scan, BASELINE.json configs[0]', 'layers': L, 'batch': B, 'seq_len': T, 'hidden': H},
+        'tflops': flop / ms / 1e9, 'host_wall_ms_per_step': wall,
+        'roofline': {'bound': 'mfma', 'achieved': flop / ms / 1e9, 'peak': PEAK_F32_MATRIX_TFLOPS, 'unit': 'TFLOP/s',
+                     'frac': flop / ms / 1e9 / PEAK_F32_MATRIX_TFLOPS, 'traffic': None, 'kernel': 'lstm_persistent_kernel',
+                     'note': '16 dependent steps of two row blocks on 8 of 256 compute units: a latency chain, not a throughput '
+                             'shape; algorithmic flops against the fp32 matrix peak', 'algorithmic_bytes_per_launch': nbytes},
+    }
+    if cpu:
+        threads = _host_threads()
+        before = torch.get_num_threads()
+        torch.set_num_threads(threads)
+        try:
+            def timed(fn, warm, runs):
+                for _ in range(warm):
+                    out = fn()
+                t = []
+                for _ in range(runs):
+                    t0 = time.perf_counter()
+                    out = fn()
+                    t.append(time.perf_counter() - t0)
+                return out, sorted(t)[len(t) // 2], min(t)
+
+            eager_out, eager_s, eager_min = timed(lambda: programs.stacked_lstm(xss, Wss, Uss, bss), 3, 10)
+            xc, WUc = xs.cpu(), WU
+
+            def batched():
+                h = torch.zeros((B, H)); c = torch.zeros((B, H)); out = []
+                for t in range(T):
+                    g = torch.cat([xc[t], h], dim=1) @ WUc[0]
+                    i, f, o, cand = g.chunk(4, 1)
+                    c = torch.sigmoid(f) * c + torch.sigmoid(i) * torch.tanh(cand)
+                    h = torch.sigmoid(o) * torch.tanh(c)
+                    out.append(h)
+                return torch.stack(out)
+
+            batched_out, batched_s, batched_min = timed(batched, 3, 10)
+        finally:
+            torch.set_num_threads(before)
+        eager_h = eager_out.as_dense().reshape(T, B, H)
+        gpu_h = hs[L - 1].cpu()
+        diff_eager = float((eager_h - gpu_h).abs().max() / gpu_h.abs().max())
+        diff_batched = float((batched_out - gpu_h).abs().max() / gpu_h.abs().max())
+        assert diff_eager <= 1e-4 and diff_batched <= 1e-4, (diff_eager, diff_batched)
+        res['cpu_baseline'] = {
+            'value': B / eager_s, 'unit': 'sequences/s', 'cores': threads, 'kind': 'port',
+            'sample': f'the whole configuration: the eager operator program (programs.stacked_lstm: map over {B} samples of '
+                      f'[1,{H}] tensors inside a scan over {T} steps, four gate products per cell) on torch CPU, '
+                      f'torch.set_num_threads({threads}) of {os.cpu_count()} host CPUs, 3 warm-up + 10 timed runs, median '
+                      f'{eager_s * 1e3:.1f} ms (min {eager_min * 1e3:.1f} ms)',
+            'ms_per_step': eager_s * 1e3, 'max_rel_diff_vs_gpu': diff_eager,
+            'batched': {'value': B / batched_s, 'unit': 'sequences/s', 'ms_per_step': batched_s * 1e3, 'min_ms': batched_min * 1e3,
+                        'max_rel_diff_vs_gpu': diff_batched,
+                        'what': f'the same layer as one [{B},{2 * H}] @ [{2 * H},{4 * H}] torch CPU product per step + torch '
+                                f'gate arithmetic, {threads} threads, 3 warm-up + 10 timed runs, median'},
+            'gpu_speedup_vs_eager': eager_s * 1e3 / ms, 'gpu_speedup_vs_batched': batched_s * 1e3 / ms,
+        }
     return res
 
 
@@ -633,8 +738,9 @@ def main():
     ap.add_argument('--gpus', type=int, default=1)
     ap.add_argument('--steps', type=int, default=50)
     ap.add_argument('--warmup', type=int, default=10)
-    ap.add_argument('--workload', default='b2b', choices=['b2b', 'attention', 'stacked_lstm', 'dilated_lstm', 'lstm_f16_h256', 'lstm_f16_h512', 'lstm_f16_h1024', 'lstm_f32_h512', 'lstm_f32_h1024', 'gemm', 'online_softmax', 'embedding', 'grid_rnn', 'windowed_attention', 'copy'])
+    ap.add_argument('--workload', default='b2b', choices=['b2b', 'config1', 'attention', 'stacked_lstm', 'dilated_lstm', 'lstm_f16_h256', 'lstm_f16_h512', 'lstm_f16_h1024', 'lstm_f32_h512', 'lstm_f32_h1024', 'gemm', 'online_softmax', 'embedding', 'grid_rnn', 'windowed_attention', 'copy'])
     ap.add_argument('--no-extras', action='store_true', help='measure only the chosen workload')
+    ap.add_argument('--all', action='store_true', help='also the workloads either side of the path (fp16 / larger stacks, GEMM, softmax, embedding, grid RNN, windowed attention)')
     ap.add_argument('--no-cpu', action='store_true', help='skip the CPU baseline leg')
     ap.add_argument('--no-baselines', action='store_true',
                     help='LSTM and grid workloads: only the fused kernel (no unfused GPU baseline, per-stage launches, other product mode, path without workspace)')
@@ -654,6 +760,7 @@ def main():
 
     runners = {
         'b2b': lambda s, w, c: bench_b2b(torch, core, s, w, c),
+        'config1': lambda s, w, c: bench_config1(torch, core, s, w, c),
         'attention': lambda s, w, c: bench_attention(torch, core, s, w, c),
         'stacked_lstm': lambda s, w, c: bench_lstm(torch, core, max(3, s // 5), max(1, w // 5), c, False, not args.no_baselines),
         'dilated_lstm': lambda s, w, c: bench_lstm(torch, core, max(3, s // 5), max(1, w // 5), c, True, not args.no_baselines),
@@ -682,17 +789,34 @@ def main():
     line.update(res)
     info = core.device_info()
     line['device'] = {'arch': info.arch.decode(), 'compute_units': info.compute_units,
-                      'host_cpus': os.cpu_count(), 'torch': torch.__version__}
+                      'host_cpus': os.cpu_count(), 'host_threads_used': _host_threads(), 'torch': torch.__version__}
+    others = {}
     if not args.no_extras:
-        others = {}
-        for name in runners:
-            if name == args.workload:
-                continue
+        # the other BASELINE.json configurations by default; the workloads either side of the path with --all
+        extra_names = [n for n in runners if n != args.workload and (args.all or n in CONFIG_OF)]
+        for name in extra_names:
             try:
                 others[name] = runners[name](max(5, args.steps // 2), max(2, args.warmup // 2), cpu)
             except Exception as e:   # an extra must not take the headline down with it
                 others[name] = {'error': repr(e)}
         line['other_workloads'] = others
+    for r in [line] + [o for o in others.values() if 'roofline' in o]:
+        if r['roofline'].get('traffic') is not None:
+            r['roofline']['traffic_source'] = 'profiles/traffic.json (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this command, not this run)'
+    # one compact row per BASELINE.json configuration, last on the line so that a truncated record keeps it
+    rows = {}
+    for name, r in [(args.workload, line)] + list(others.items()):
+        if name not in CONFIG_OF:
+            continue
+        if 'error' in r:
+            rows[CONFIG_OF[name]] = {'workload': name, 'error': r['error']}
+            continue
+        diffs = [v for v in (r.get('cpu_baseline') or {}, r.get('unfused_gpu_baseline') or {})]
+        diff = next((d[k] for d in diffs for k in ('max_rel_diff_vs_gpu', 'max_rel_diff_vs_fused') if k in d), None)
+        rows[CONFIG_OF[name]] = {'workload': name, 'ms_per_step': round(r['ms_per_step'], 5), 'value': r.get('value'), 'unit': r.get('unit'),
+                                 'bound': r['roofline']['bound'], 'frac': round(r['roofline']['frac'], 4), 'max_rel_diff': diff,
+                                 'cpu_baseline': (r.get('cpu_baseline') or {}).get('value')}
+    line['configs'] = dict(sorted(rows.items()))
     print(json.dumps(line))
 
 
