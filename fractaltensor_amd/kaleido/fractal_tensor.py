@@ -329,6 +329,7 @@ class Iterative(Sequence):
 
     def __init__(self, *xs):
         self._items = list(xs)
+        self.sources = None   # set by zip: the sequences the items were taken from
 
     def __getitem__(self, i):
         return self._items[i]

@@ -41,7 +41,9 @@ def zip(*inputs) -> Iterative:
     for x in inputs[1:]:
         if len(x) != n:
             raise ValueError('inputs to zip should have the same length.')
-    return Iterative(*[[x[i] for x in inputs] for i in range(n)])
+    out = Iterative(*[[x[i] for x in inputs] for i in range(n)])
+    out.sources = tuple(inputs)   # what was zipped: lets a fused kernel take whole operands as the views they are
+    return out
 
 
 def enumerate(*inputs) -> Iterative:

@@ -14,8 +14,9 @@ docs/fractaltensor_operations/parallel_functions_on_fractaltensor.md:46-203):
 
 A function returning a tuple of values yields one FractalTensor per field.
 These are eager Python loops over torch payloads, on the CPU or the GPU: this
-IS the reference's execution model, and it is what the fused kernels in
-operations.fused replace for the three hot-path programs.
+IS the reference's execution model.  On GPU operands fold and map first ask
+operations.dispatch whether the call is one of the hot-path programs (a stack
+of LSTM layers, blockwise attention); if so it runs as one fused kernel.
 """
 from __future__ import annotations
 
@@ -23,6 +24,7 @@ from typing import Callable, List
 
 from ..fractal_tensor import FractalTensor, Iterative
 from ..tensor import Tensor
+from . import dispatch
 from ._base import require_iterative
 
 __all__ = ['map', 'filter', 'dilated_map', 'scan', 'fold', 'reduce']
@@ -62,6 +64,9 @@ def pack_outputs(results: List):
 
 def map(func: Callable, xs, **kwargs):
     require_iterative(xs)
+    routed = dispatch.try_map(func, xs, kwargs)      # blockwise attention on GPU operands: one kernel
+    if routed is not NotImplemented:
+        return routed
     return pack_outputs([func(x, **kwargs) for x in xs])
 
 
@@ -91,6 +96,10 @@ def scan(func: Callable, xs, initializer=None, **kwargs):
 
 
 def fold(func: Callable, xs, initializer=None, **kwargs):
+    require_iterative(xs)
+    routed = dispatch.try_fold(func, xs, initializer, kwargs)   # a stack of LSTM layers on GPU operands: one kernel
+    if routed is not NotImplemented:
+        return routed
     outs = scan(func, xs, initializer, **kwargs)
     if isinstance(outs, list):
         return [o[len(o) - 1] for o in outs]
@@ -128,6 +137,7 @@ def dilated_map(func: Callable, xs, dilation: int = 1, **kwargs):
     require_iterative(xs)
     if isinstance(dilation, Tensor):
         dilation = int(dilation.data.reshape(-1)[0].item())
+    dispatch.note_dilation(dilation)
     outs = map(lambda group: func(group, **kwargs), _dilate(xs, dilation))
     if not isinstance(outs, list):
         outs = [outs]

@@ -174,8 +174,8 @@ def flash_attention(qsss: FractalTensor, ksss: FractalTensor, vsss: FractalTenso
     [block_rows, head_dim], the layout flash_attention_utils.create_input builds.
     The result has the structure of qsss.  fp32 inputs are converted to fp16 for
     the kernel (which accumulates in fp32) and the result converted back; `scale`
-    defaults to 1/sqrt(head_dim) (the reference program applies none: pass 1.0
-    for its exact maths)."""
+    multiplies the scores and defaults to 1.0, the reference program's maths
+    (attn_func forms query @ key.T unscaled); pass head_dim ** -0.5 for the usual one."""
     core = _core()
     q = _dense_gpu(qsss, 'qsss', 3)   # [B, Hd, nb, rows, D]
     k = _dense_gpu(ksss, 'ksss', 3)
@@ -184,7 +184,7 @@ def flash_attention(qsss: FractalTensor, ksss: FractalTensor, vsss: FractalTenso
     to4 = lambda t: t.reshape(t.shape[0], t.shape[1], t.shape[2] * t.shape[3], t.shape[4])
     in_dtype = q.dtype
     O = core.flash_attention(to4(q).half().contiguous(), to4(k).half().contiguous(), to4(v).half().contiguous(),
-                             D ** -0.5 if scale is None else float(scale))
+                             1.0 if scale is None else float(scale))
     return FractalTensor.from_dense(O.to(in_dtype).view(B, Hd, nbq, rq, D), 3)
 
 

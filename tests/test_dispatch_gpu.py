@@ -1,0 +1,292 @@
+"""Operator programs, unchanged, on GPU FractalTensors: fold / map route them to one fused launch.
+
+Two sets of programs: the ones of fractaltensor_amd/programs.py, and programs written here the way the reference's
+examples are written (`import kaleido`, decorated cell functions, per-gate map over zip(ws, us, bs), fold over
+zip / enumerate of the stacked parameters: examples/stacked_rnn/stacked_rnn.py:12-79,
+examples/dilated_rnn/dilated_rnn.py:16-41, examples/flash_attention/flash_attention.py:14-91).  Every routed result
+is checked against the oracle, and against the eager loop where that is affordable."""
+import numpy as np
+import pytest
+import torch
+
+import kaleido
+from kaleido import FractalTensor, Tensor
+from kaleido import operations as ops
+
+from fractaltensor_amd import programs
+from oracle import kaleido_oracle as ko
+
+pytestmark = pytest.mark.gpu
+dispatch = ops.dispatch
+
+
+@pytest.fixture(autouse=True)
+def fresh_dispatch():
+    dispatch.reset()
+    dispatch.enabled = True
+    dispatch.allow_half_attention = False
+    yield
+    dispatch.reset()
+
+
+def _np_params(Wss, Uss, bss):
+    W = Wss.as_dense().float().cpu().numpy(); U = Uss.as_dense().float().cpu().numpy(); b = bss.as_dense().float().cpu().numpy()
+    L, _, H, _ = W.shape
+    return np.stack([ko.fuse_gate_weights(W[l], U[l]) for l in range(L)]), b.reshape(L, 4 * H)
+
+
+def _core():
+    import fractaltensor_amd._core as core
+    return core
+
+
+# ---- programs in the reference's style ---------------------------------------------------------------------------
+
+ctx = kaleido.Context()
+
+
+@kaleido.function(ctx)
+def gate_f(w, u, b, x, s):
+    return x @ w + s @ u + b
+
+
+@kaleido.function(ctx)
+def lstm_cell(h_prev, c_prev, input, ws, us, bs):
+    prev_gate = ops.map(lambda x: gate_f(*x, input, h_prev), ops.zip(ws, us, bs))
+    gate = ops.map(lambda x: ops.sigmoid(x), prev_gate[:3])
+    c = gate[1] * c_prev + gate[0] * ops.tanh(prev_gate[3])
+    h = gate[2] * ops.tanh(c)
+    return h, c
+
+
+def batched_cell(hs_prev, cs_prev, xs, ws, us, bs):
+    hs, cs = ops.map(lambda x: lstm_cell(*x, ws, us, bs), ops.zip(hs_prev[0:xs.length], cs_prev[0:xs.length], xs))
+    return hs, cs
+
+
+def lstm_layer(xss, ws, us, bs):
+    hidden = xss.element_shape[-1]
+    init = ops.repeat(ops.zeros(shape=(1, hidden), device=xss.device), xss[0].length)
+    hss, css = ops.scan(lambda state, x: batched_cell(*state, x, ws, us, bs), xss, initializer=(init, init))
+    return hss
+
+
+def stacked_lstm(embs, Wss, Uss, bss):
+    return ops.fold(lambda s, param: lstm_layer(s, *param), ops.zip(Wss, Uss, bss), initializer=embs)
+
+
+def dilated_layer(state, itr, Ws, Us, bs):
+    hidden = state.element_shape[-1]
+    zeros = ops.zeros(shape=(1, hidden), device=state.device, dtype='float')
+    h, _ = ops.dilated_map(lambda xs: ops.scan(lambda s, x: lstm_cell(*s, x, Ws, Us, bs), xs, initializer=(zeros, zeros)),
+                           state, dilation=2 ** int(itr.data.item()))
+    return h
+
+
+def dilated_model(embs, Wss, Uss, bss):
+    """Batch-major: every sample's sequence through the whole dilated stack."""
+    itrs = ops.enumerate(Wss, Uss, bss)
+    return ops.map(lambda xs: ops.fold(lambda s, x: dilated_layer(s, *x), itrs, initializer=xs), embs)
+
+
+def attn_func(prev_maxes, prev_sums, prev_out, query, key, value):
+    attn_weights = query @ key.T
+    cur_maxes = ops.max(attn_weights, dim=-1, keepdim=True)
+    exp_weights = ops.exp(attn_weights - cur_maxes)
+    exp_values = exp_weights @ value
+    cur_sums = ops.sum(exp_weights, dim=-1, keepdim=True)
+    new_maxes = ops.maximum(cur_maxes, prev_maxes)
+    renorm_prev = ops.exp(prev_maxes - new_maxes)
+    renorm_cur = ops.exp(cur_maxes - new_maxes)
+    new_sums = renorm_prev * prev_sums + renorm_cur * cur_sums
+    o = (prev_out * prev_sums * renorm_prev + renorm_cur * exp_values) / new_sums
+    return new_maxes, new_sums, o
+
+
+def per_block_func(query, ks, vs):
+    rows, dim = query.shape
+    init_sum = ops.zeros(shape=(rows, 1), device=query.device)
+    init_max = ops.full(shape=(rows, 1), fill_value=-kaleido.float32.max, device=query.device)
+    init_o = ops.zeros(shape=(rows, dim), device=query.device)
+    _, _, o = ops.reduce(lambda state, kvs: attn_func(*state, query, *kvs), ops.zip(ks, vs),
+                         initializer=(init_max, init_sum, init_o))
+    return o
+
+
+def per_head_func(qs, ks, vs):
+    return ops.map(lambda q: per_block_func(q, ks, vs), qs)
+
+
+def flash_attention(qsss, ksss, vsss):
+    return ops.map(lambda xss: ops.map(lambda xs: per_head_func(*xs), ops.zip(*xss)), ops.zip(qsss, ksss, vsss))
+
+
+# ---- stacked LSTM -------------------------------------------------------------------------------------------------
+
+def test_programs_stacked_lstm_is_routed_to_one_launch():
+    core = _core()
+    L, T, B, H = 3, 5, 33, 256
+    Wss, Uss, bss = programs.make_lstm_params(L, H, 1 / 16, seed=1, device='cuda')
+    xss = programs.make_sequence_batch(T, B, H, seed=2, device='cuda')
+    out = programs.stacked_lstm(xss, Wss, Uss, bss)                       # cold: one probe of layer 0, then the launch
+    assert dispatch.stats['stacked_lstm'] == 1 and dispatch.stats['probes'] == 1 and dispatch.stats['declined'] == 0
+    assert isinstance(out, FractalTensor) and out.depth == 2 and out.dense_shape() == (T, B) and out.element_shape == (1, H)
+    WU, bias = _np_params(Wss, Uss, bss)
+    ref, _ = ko.stacked_lstm(xss.as_dense().cpu().numpy().reshape(T, B, H), WU, bias)
+    assert ko.max_rel_err(out.as_dense().cpu().numpy().reshape(T, B, H), ref[-1]) <= 1e-4
+    before = dict(core.launch_counts)
+    out2 = programs.stacked_lstm(xss, Wss, Uss, bss)                      # warm: exactly one fused call, nothing else
+    assert core.launch_counts['stacked_lstm'] == before['stacked_lstm'] + 1
+    assert dispatch.stats['probes'] == 1 and dispatch.stats['stacked_lstm'] == 2
+    assert torch.equal(out2.as_dense(), out.as_dense())
+
+
+def test_reference_style_stacked_lstm_on_a_ragged_time_major_batch():
+    """Sequences of lengths 6, 4, 4, 2 as the time-major batch examples/utils/data_utils.py:42-66 builds; routed with
+    per-step row counts, equal to the eager loop and to the oracle run per sequence."""
+    L, H = 2, 64
+    lens = [6, 4, 4, 2]
+    Wss, Uss, bss = programs.make_lstm_params(L, H, 1 / 8, seed=3, device='cuda')
+    g = torch.Generator().manual_seed(4)
+    seqs = [torch.randn((n, H), generator=g) for n in lens]
+    steps = []
+    for t in range(max(lens)):
+        rows = [s[t] for s in seqs if len(s) > t]
+        steps.append(FractalTensor.from_dense(torch.stack(rows).reshape(len(rows), 1, H).cuda(), 1))
+    embs = FractalTensor.from_fractaltensors(*steps)
+    routed = stacked_lstm(embs, Wss, Uss, bss)
+    assert dispatch.stats['stacked_lstm'] == 1 and dispatch.stats['declined'] == 0
+    dispatch.enabled = False
+    eager = stacked_lstm(embs, Wss, Uss, bss)
+    dispatch.enabled = True
+    assert routed.indices == eager.indices
+    assert ko.max_rel_err(routed.data.cpu().numpy(), eager.data.cpu().numpy()) <= 1e-4
+    WU, bias = _np_params(Wss, Uss, bss)
+    for b, s in enumerate(seqs):
+        ref, _ = ko.stacked_lstm(s.numpy().reshape(len(s), 1, H), WU, bias)
+        got = np.stack([routed[t][b].data.cpu().numpy().reshape(H) for t in range(len(s))])
+        assert ko.max_rel_err(got, ref[-1][:, 0]) <= 1e-4
+
+
+def test_fp16_stacked_lstm_program_goes_to_the_fp16_kernel():
+    """A program whose tensors are all fp16 (its zero state included) is routed to the fp16-storage kernel."""
+    core = _core()
+    L, T, B, H = 2, 4, 8, 128
+    Wss, Uss, bss = programs.make_lstm_params(L, H, 1 / 8, seed=5, device='cuda')
+    half = lambda ft, d: FractalTensor.from_dense(ft.as_dense().half(), d)
+    xss = programs.make_sequence_batch(T, B, H, seed=6, device='cuda')
+
+    def layer_f16(seq, ws, us, bs):
+        zero = ops.repeat(ops.zeros(shape=(1, H), dtype='half', device=seq.device), seq[0].length)
+        hss, _ = ops.scan(lambda state, xs: programs.batched_cell(state[0], state[1], xs, ws, us, bs), seq, initializer=(zero, zero))
+        return hss
+
+    out = ops.fold(lambda seq, p: layer_f16(seq, *p), ops.zip(half(Wss, 2), half(Uss, 2), half(bss, 2)), initializer=half(xss, 2))
+    assert dispatch.stats['stacked_lstm'] == 1 and core.launch_counts.get('stacked_lstm_f16', 0) >= 1
+    assert out.data.dtype == torch.float16
+    WU, bias = _np_params(half(Wss, 2), half(Uss, 2), half(bss, 2))
+    ref, _ = ko.stacked_lstm(xss.as_dense().half().float().cpu().numpy().reshape(T, B, H), WU, bias)
+    assert ko.max_rel_err(out.as_dense().float().cpu().numpy().reshape(T, B, H), ref[-1]) <= 1e-2
+
+
+def test_a_fold_that_is_no_lstm_stays_eager():
+    """Same operand structure, different arithmetic (the layer's output doubled): the probe sees the difference."""
+    L, T, B, H = 2, 3, 2, 32
+    Wss, Uss, bss = programs.make_lstm_params(L, H, 1 / 8, seed=7, device='cuda')
+    xss = programs.make_sequence_batch(T, B, H, seed=8, device='cuda')
+
+    def doubled(seq, p):
+        hss = programs.lstm_layer(seq, p[0], p[1], p[2])
+        return FractalTensor.from_dense(hss.as_dense() * 2, 2)
+
+    out = ops.fold(doubled, ops.zip(Wss, Uss, bss), initializer=xss)
+    assert dispatch.stats['declined'] == 1 and dispatch.stats['stacked_lstm'] == 0
+    WU, bias = _np_params(Wss, Uss, bss)
+    x = xss.as_dense().cpu().numpy().reshape(T, B, H)
+    h0, _ = ko.stacked_lstm(x, WU[:1], bias[:1])
+    h1, _ = ko.stacked_lstm(2 * h0[-1], WU[1:], bias[1:])
+    assert ko.max_rel_err(out.as_dense().cpu().numpy().reshape(T, B, H), 2 * h1[-1]) <= 1e-4
+    ops.fold(doubled, ops.zip(Wss, Uss, bss), initializer=xss)          # the verdict is remembered: no second probe
+    assert dispatch.stats['probes'] == 1
+
+
+# ---- dilated LSTM -------------------------------------------------------------------------------------------------
+
+@pytest.mark.parametrize('L,T,B,H', [(3, 9, 2, 32), (4, 20, 5, 256)])
+def test_programs_dilated_lstm_is_routed_with_the_dilations_it_asks_for(L, T, B, H):
+    core = _core()
+    Wss, Uss, bss = programs.make_lstm_params(L, H, 1 / 16, seed=9, device='cuda')
+    xss = programs.make_sequence_batch(T, B, H, seed=10, device='cuda')
+    out = programs.dilated_lstm(xss, Wss, Uss, bss)
+    assert dispatch.stats['dilated_lstm'] == 1 and dispatch.stats['declined'] == 0
+    WU, bias = _np_params(Wss, Uss, bss)
+    ref, _ = ko.stacked_lstm(xss.as_dense().cpu().numpy().reshape(T, B, H), WU, bias, dilations=[2 ** k for k in range(L)])
+    assert ko.max_rel_err(out.as_dense().cpu().numpy().reshape(T, B, H), ref[-1]) <= 1e-4
+    before = core.launch_counts['stacked_lstm']
+    programs.dilated_lstm(xss, Wss, Uss, bss)
+    assert core.launch_counts['stacked_lstm'] == before + 1 and dispatch.stats['probes'] == 1
+
+
+def test_reference_style_dilated_model_routes_every_samples_fold():
+    """Batch-major samples of different lengths, each folded through the dilated stack on its own
+    (dilated_rnn.py:33-41): one launch per sample; a sample no longer than a layer's dilation is scanned in order
+    by that layer (the one group _dilate then makes)."""
+    L, H = 3, 32
+    lens = [9, 6, 3]
+    Wss, Uss, bss = programs.make_lstm_params(L, H, 1 / 8, seed=11, device='cuda')
+    g = torch.Generator().manual_seed(12)
+    seqs = [torch.randn((n, 1, H), generator=g) for n in lens]
+    embs = FractalTensor.from_fractaltensors(*[FractalTensor.from_dense(s.cuda(), 1) for s in seqs])
+    out = dilated_model(embs, Wss, Uss, bss)
+    assert dispatch.stats['dilated_lstm'] + dispatch.stats['stacked_lstm'] == len(lens) and dispatch.stats['declined'] == 0
+    WU, bias = _np_params(Wss, Uss, bss)
+    for b, s in enumerate(seqs):
+        n = lens[b]
+        dil = [d if n > d else 1 for d in (1, 2, 4)]
+        ref, _ = ko.stacked_lstm(s.numpy().reshape(n, 1, H), WU, bias, dilations=dil)
+        assert ko.max_rel_err(out[b].as_dense().cpu().numpy().reshape(n, H), ref[-1][:, 0]) <= 1e-4
+    dispatch.enabled = False
+    eager = dilated_model(embs, Wss, Uss, bss)
+    assert ko.max_rel_err(out.data.cpu().numpy(), eager.data.cpu().numpy()) <= 1e-4
+
+
+# ---- attention ----------------------------------------------------------------------------------------------------
+
+@pytest.mark.parametrize('D,scale', [(128, 128 ** -0.5), (64, 1.0), (64, 0.2)])
+def test_programs_flash_attention_is_routed_with_its_scale(D, scale):
+    core = _core()
+    B, Hd, S, blk = 2, 2, 256, 64
+    qsss, ksss, vsss = (programs.make_attention_input(B, Hd, S, blk, D, seed=20 + i, device='cuda', dtype=torch.float16) for i in range(3))
+    out = programs.flash_attention(qsss, ksss, vsss, scale)
+    assert dispatch.stats['flash_attention'] == 1 and dispatch.stats['declined'] == 0
+    assert out.depth == 3 and out.dense_shape() == (B, Hd, S // blk) and out.element_shape == (blk, D)
+    to4 = lambda t: t.as_dense().reshape(B, Hd, S, D).float().cpu().numpy()
+    ref = ko.attention(to4(qsss), to4(ksss), to4(vsss), scale, dtype=np.float32)
+    assert ko.max_rel_err(to4(out), ref) <= 1e-2
+    before = core.launch_counts['flash_attention']
+    programs.flash_attention(qsss, ksss, vsss, scale)
+    assert core.launch_counts['flash_attention'] == before + 1 and dispatch.stats['probes'] == 1
+    programs.flash_attention(qsss, ksss, vsss, scale * 0.5)               # another scale in the closure: probed anew
+    assert dispatch.stats['probes'] == 2
+
+
+def test_reference_style_flash_attention_without_a_scale():
+    B, Hd, S, blk, D = 1, 2, 128, 64, 64
+    qsss, ksss, vsss = (programs.make_attention_input(B, Hd, S, blk, D, seed=30 + i, device='cuda', dtype=torch.float16) for i in range(3))
+    scaled = FractalTensor.from_dense(qsss.as_dense() * 0.25, 3)           # keeps the unscaled scores in fp16's comfortable range
+    out = flash_attention(scaled, ksss, vsss)
+    assert dispatch.stats['flash_attention'] == 1
+    to4 = lambda t: t.as_dense().reshape(B, Hd, S, D).float().cpu().numpy()
+    ref = ko.attention(to4(scaled), to4(ksss), to4(vsss), 1.0, dtype=np.float32)
+    assert ko.max_rel_err(to4(out), ref) <= 1e-2
+
+
+def test_fp32_attention_program_is_not_lowered_to_fp16_unless_allowed():
+    B, Hd, S, blk, D = 1, 1, 128, 64, 64
+    qsss, ksss, vsss = (programs.make_attention_input(B, Hd, S, blk, D, seed=40 + i, device='cuda') for i in range(3))
+    eager = programs.flash_attention(qsss, ksss, vsss, D ** -0.5)
+    assert dispatch.stats['flash_attention'] == 0 and dispatch.stats['probes'] == 0
+    dispatch.allow_half_attention = True
+    routed = programs.flash_attention(qsss, ksss, vsss, D ** -0.5)
+    assert dispatch.stats['flash_attention'] == 1 and routed.data.dtype == torch.float32
+    assert ko.max_rel_err(routed.data.cpu().numpy(), eager.data.cpu().numpy()) <= 1e-2

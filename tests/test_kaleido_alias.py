@@ -1,0 +1,68 @@
+"""`import kaleido` gives the operator API under the reference's package name and module paths, and operator
+dispatch leaves host programs alone."""
+import numpy as np
+import torch
+
+from oracle import kaleido_oracle as ko
+
+
+def test_reference_import_paths_resolve_to_one_implementation():
+    import kaleido
+    from kaleido import FractalTensor, FractalTensorStorage, Iterative, StaticList, Tensor, TensorStorage   # noqa: F401
+    from kaleido import operations as ops
+    from kaleido.frontend.types import Bool, Int, Real   # noqa: F401
+    from kaleido.parser.plot import PlotProgram
+    import fractaltensor_amd.kaleido as impl
+    import fractaltensor_amd.kaleido.operations.dispatch as d
+    assert kaleido is impl and ops is impl.operations and ops.dispatch is d
+    import kaleido.operations.functional as f
+    assert f is impl.operations.functional
+    ctx = kaleido.Context()
+
+    @kaleido.function(ctx)
+    def twice(x):
+        return x + x
+
+    ctx[-1].ir_block.propagate_storage()
+    PlotProgram().plot(ctx[-1].ir_block)
+    t = Tensor.from_tensor(torch.ones((1, 4)))
+    assert float(twice(t).data.sum()) == 8.0
+    assert kaleido.float32.max == torch.finfo(torch.float32).max
+
+
+def test_host_programs_are_never_routed():
+    from kaleido import operations as ops
+    from fractaltensor_amd import programs
+    ops.dispatch.reset()
+    L, T, B, H = 2, 3, 2, 32
+    Wss, Uss, bss = programs.make_lstm_params(L, H, 1 / 8, seed=1)
+    xss = programs.make_sequence_batch(T, B, H, seed=2)
+    out = programs.stacked_lstm(xss, Wss, Uss, bss)
+    assert all(v == 0 for v in ops.dispatch.stats.values())
+    W = Wss.as_dense().numpy(); U = Uss.as_dense().numpy()
+    WU = np.stack([ko.fuse_gate_weights(W[l], U[l]) for l in range(L)])
+    ref, _ = ko.stacked_lstm(xss.as_dense().numpy().reshape(T, B, H), WU, bss.as_dense().numpy().reshape(L, 4 * H))
+    assert ko.max_rel_err(out.as_dense().numpy().reshape(T, B, H), ref[-1]) <= 1e-5
+
+
+def test_function_fingerprint_follows_code_and_closure_scalars():
+    from kaleido.operations import dispatch
+
+    def make(scale):
+        inner = lambda x: x * scale
+        return lambda y: inner(y)
+
+    assert dispatch._fingerprint(make(2.0)) == dispatch._fingerprint(make(2.0))
+    assert dispatch._fingerprint(make(2.0)) != dispatch._fingerprint(make(3.0))
+    assert dispatch._fingerprint(make(2.0)) != dispatch._fingerprint(lambda y: y)
+
+
+def test_dilations_are_noted_only_under_a_probe():
+    from kaleido.operations import dispatch
+    dispatch.note_dilation(4)                  # outside a probe: ignored
+    with dispatch._Probe() as p:
+        dispatch.note_dilation(4)
+        with dispatch._Probe() as q:           # a nested probe keeps its own list
+            dispatch.note_dilation(2)
+        assert q.dilations == [2]
+    assert p.dilations == [4] and not dispatch._probing()
