@@ -116,6 +116,69 @@ def bench_b2b(torch, core, steps, warmup, cpu):
     return res
 
 
+def _graph_us(torch, fn, calls=20, replays=10):
+    """Microseconds per call of fn with the calls replayed from a HIP graph: what is left is the device's own
+    kernel-to-kernel cost, not the host's launch path (these kernels are shorter than a ctypes call)."""
+    fn()
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        fn()
+    torch.cuda.current_stream().wait_stream(side)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        for _ in range(calls):
+            fn()
+    graph.replay()
+    torch.cuda.synchronize()
+    a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    a.record()
+    for _ in range(replays):
+        graph.replay()
+    b.record()
+    torch.cuda.synchronize()
+    return a.elapsed_time(b) / (calls * replays) * 1e3
+
+
+def bench_b2b_reference_shapes(torch, core, steps, warmup, cpu):
+    """The four shapes of the reference's own B2B benchmark, [8192 | 16384, 64] x [64, 256 | 512] x [., 64]
+    (benchmarks/fused_two_hgemms/fractaltensor/fused_two_hgemms.cu:152-175), timed as it times them: the same
+    operands again and again (2 to 4.5 MB, so they stay in the caches), here replayed from a HIP graph."""
+    gen = torch.Generator(device='cpu').manual_seed(1234)
+    shapes = {}
+    for M in (8192, 16384):
+        for N in (256, 512):
+            K = P = 64
+            A = (torch.randn((1, M, K), generator=gen) / K ** 0.5).half().cuda()
+            Bn = (torch.randn((1, N, K), generator=gen) / K ** 0.5).half().cuda()
+            Cp = (torch.randn((1, P, N), generator=gen) / N ** 0.5).half().cuda()
+            D = torch.empty((1, M, P), dtype=torch.float16, device='cuda')
+            us = _graph_us(torch, lambda: core.b2b_gemm(A, Bn, Cp, out=D))
+            Bt, Ct = Bn[0].t().contiguous(), Cp[0].t().contiguous()
+            Pm = torch.empty((M, N), dtype=torch.float16, device='cuda')
+            D2 = torch.empty((M, P), dtype=torch.float16, device='cuda')
+            us_t = _graph_us(torch, lambda: (torch.mm(A[0], Bt, out=Pm), torch.mm(Pm, Ct, out=D2)))
+            flop = 2.0 * M * N * (K + P)
+            diff = float((D[0].float() - D2.float()).abs().max() / D2.float().abs().max())
+            assert diff <= 1e-2, diff
+            shapes[f'M{M}_N{N}'] = {'us_per_call': us, 'tflops': flop / us / 1e6, 'two_torch_gemms_us': us_t,
+                                    'speedup': us_t / us, 'max_rel_diff_vs_two_gemms': diff,
+                                    'bytes': 2.0 * (M * K + N * K + P * N + M * P)}
+    top = shapes['M16384_N512']
+    flop = 2.0 * 16384 * 512 * 128
+    return {'metric': 'TFLOP/s (B2B GEMM, reference benchmark shapes)', 'value': top['tflops'], 'unit': 'TFLOP/s',
+            'ms_per_step': top['us_per_call'] / 1e3, 'dtype': 'f16',
+            'config': {'workload': 'fused back-to-back GEMM on the reference benchmark shapes, operands resident in the caches, '
+                                   'launches replayed from a HIP graph; headline figures are the largest shape (M 16384, N 512)',
+                       'K': 64, 'P': 64, 'accumulate': 'f32'},
+            'roofline': {'bound': 'mfma', 'achieved': top['tflops'], 'peak': PEAK_F16_TFLOPS, 'unit': 'TFLOP/s',
+                         'frac': top['tflops'] / PEAK_F16_TFLOPS, 'traffic': None, 'kernel': 'b2b_wide_kernel<4, 2, 2, 8>',
+                         'note': '2.1 GFLOP and 4.5 MB per launch: a launch of a few microseconds, bounded by the kernel-to-kernel '
+                                 'cost of the device and the read of B and C by every workgroup, not by the matrix rate'},
+            'shapes': shapes}
+
+
 def bench_copy(torch, core, steps, warmup, cpu):
     """Plain device copy of a known size: the calibration kernel for the FETCH_SIZE / WRITE_SIZE counters."""
     n = 64 << 20   # 64 MiB read + 64 MiB written per launch
@@ -738,7 +801,7 @@ def main():
     ap.add_argument('--gpus', type=int, default=1)
     ap.add_argument('--steps', type=int, default=50)
     ap.add_argument('--warmup', type=int, default=10)
-    ap.add_argument('--workload', default='b2b', choices=['b2b', 'config1', 'attention', 'stacked_lstm', 'dilated_lstm', 'lstm_f16_h256', 'lstm_f16_h512', 'lstm_f16_h1024', 'lstm_f32_h512', 'lstm_f32_h1024', 'gemm', 'online_softmax', 'embedding', 'grid_rnn', 'windowed_attention', 'copy'])
+    ap.add_argument('--workload', default='b2b', choices=['b2b', 'config1', 'attention', 'stacked_lstm', 'dilated_lstm', 'lstm_f16_h256', 'lstm_f16_h512', 'lstm_f16_h1024', 'lstm_f32_h512', 'lstm_f32_h1024', 'gemm', 'online_softmax', 'embedding', 'grid_rnn', 'windowed_attention', 'b2b_ref_shapes', 'copy'])
     ap.add_argument('--no-extras', action='store_true', help='measure only the chosen workload')
     ap.add_argument('--all', action='store_true', help='also the workloads either side of the path (fp16 / larger stacks, GEMM, softmax, embedding, grid RNN, windowed attention)')
     ap.add_argument('--no-cpu', action='store_true', help='skip the CPU baseline leg')
@@ -769,6 +832,7 @@ def main():
         'lstm_f16_h1024': lambda s, w, c: bench_lstm_f16(torch, core, max(3, s // 5), max(1, w // 5), c, 1024, not args.no_baselines),
         'lstm_f32_h512': lambda s, w, c: bench_lstm_f32_streamed(torch, core, max(3, s // 5), max(1, w // 5), c, 512),
         'lstm_f32_h1024': lambda s, w, c: bench_lstm_f32_streamed(torch, core, max(3, s // 10), 1, c, 1024),
+        'b2b_ref_shapes': lambda s, w, c: bench_b2b_reference_shapes(torch, core, s, w, c),
         'gemm': lambda s, w, c: bench_gemm(torch, core, max(5, s // 5), max(2, w // 5), c),
         'online_softmax': lambda s, w, c: bench_softmax(torch, core, s, w, c),
         'embedding': lambda s, w, c: bench_embedding(torch, core, s, w, c),

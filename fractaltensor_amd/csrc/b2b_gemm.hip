@@ -351,13 +351,16 @@ __global__ __launch_bounds__(512) void b2b_gemm8_kernel(const _Float16* __restri
         else vc[u] = ldg16(Cg + (size_t)idx * 8);
       }
     }
-    // Requests are served roughly in the order the CU's memory pipeline accepted them.  The barrier
-    // puts every wave's share of B and C (which everything waits for) ahead of any A row; then one
-    // 32-row unit per wave follows, and the second unit once B and C have landed -- with all 512 rows
-    // of the workgroup requested at once nothing arrives early, and no wave could start before the end
-    // of the burst.
-    __syncthreads();
-    if (unit < unit_end) fetch_a(unit, areg0);
+    // The memory system shares its bandwidth among everything that is outstanding: whatever is requested together
+    // lands together, at the end of the burst.  So the requests go out in two waves of requests: B and C (which
+    // everything waits for) and both A units of the first four waves now; the A units of the other four waves
+    // once B and C have landed.  The first four waves (one per SIMD) then compute while the rows of their SIMD
+    // partners are still on the way.  (A barrier between the B / C requests and the first A requests, which
+    // kept the order in the CU's memory pipeline strict, cost 1 us of issue time and gained nothing.)
+    if (wave < waves / 2) {
+      if (unit < unit_end) fetch_a(unit, areg0);
+      if (unit + waves < unit_end) fetch_a(unit + waves, areg1);
+    }
 #pragma unroll
     for (int u = 0; u < UB; ++u) {
       const int idx = u * threads + tid;
@@ -382,7 +385,10 @@ __global__ __launch_bounds__(512) void b2b_gemm8_kernel(const _Float16* __restri
     }
   }
   __syncthreads();
-  if (unit + waves < unit_end) fetch_a(unit + waves, areg1);
+  if (wave >= waves / 2) {
+    if (unit < unit_end) fetch_a(unit, areg0);
+    if (unit + waves < unit_end) fetch_a(unit + waves, areg1);
+  }
 
   // one 32-row unit whose A chunks are in ar; refills ar with the unit two further on
   auto do_unit = [&](int un, v4u (&ar)[AN]) __attribute__((always_inline)) {
@@ -530,6 +536,140 @@ static int launch_b2b8(const void* A, const void* B, const void* C, void* D, int
   return check_launch("b2b_gemm8_kernel");
 }
 
+// Wide-N form for the shapes of the reference's own benchmark, [M, 64] x [64, 256 | 512] x [., 64]
+// (benchmarks/fused_two_hgemms/fractaltensor/fused_two_hgemms.cu:152-175): one problem, few bytes (2 MB), so what
+// counts is the length of the dependency chain of one 32-row unit.  A workgroup takes one unit and its WAVES waves
+// split N: wave w forms the 32*NTW columns [n0, n0 + 32 NTW) of P for all 32 rows (K/16 * NTW MFMAs), rounds them to
+// fp16 and multiplies them with its rows of C (2 * NTW * PT MFMAs), which leaves a partial D tile per wave; the
+// partials are summed in fp32 through LDS and the 32 x P tile leaves as whole rows.  B and C are read once per
+// workgroup straight into MFMA operands (16-byte and 8-byte pieces from the cache hierarchy: each wave needs only its
+// own slice, nothing is staged), the A rows by every wave.  The contraction order of both products is the one of the
+// kernels above.
+template <int KS, int PT, int NTW, int WAVES>
+__global__ __launch_bounds__(WAVES * 64) void b2b_wide_kernel(const _Float16* __restrict__ A,
+                                                              const _Float16* __restrict__ Bm,
+                                                              const _Float16* __restrict__ Cm, _Float16* __restrict__ D,
+                                                              int M, int units) {
+  constexpr int K = 16 * KS;
+  constexpr int N = 32 * NTW * WAVES;
+  constexpr int P = 32 * PT;
+  constexpr int RLD = P + 4;  // padded row of a partial tile (floats)
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+  float* red = reinterpret_cast<float*>(smem);  // [WAVES][32][RLD]
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = tid >> 6;
+  const int j = lane & 31;
+  const int hh = lane >> 5;
+  const int g = blockIdx.x / units;
+  const int unit = blockIdx.x - g * units;
+  const int r0 = unit * 32;
+  const int n0 = wave * 32 * NTW;
+
+  const _Float16* Ag = A + (size_t)g * M * K;
+  const _Float16* Bg = Bm + (size_t)g * N * K;
+  const _Float16* Cg = Cm + (size_t)g * P * N;
+  _Float16* Dg = D + (size_t)g * M * P;
+
+  // every load of the wave is requested before the first is used
+  v8h afrag[KS], bfrag[NTW][KS];
+  const _Float16* arow = Ag + (size_t)min(r0 + j, M - 1) * K + hh * (K / 2);
+#pragma unroll
+  for (int s = 0; s < KS; ++s) afrag[s] = __builtin_bit_cast(v8h, ldg16(arow + 8 * s));
+#pragma unroll
+  for (int nt = 0; nt < NTW; ++nt)
+#pragma unroll
+    for (int s = 0; s < KS; ++s)
+      bfrag[nt][s] = __builtin_bit_cast(v8h, ldg16(Bg + (size_t)(n0 + 32 * nt + j) * K + hh * (K / 2) + 8 * s));
+  v4h cfrag[PT][NTW][2][2];
+#pragma unroll
+  for (int q = 0; q < PT; ++q)
+#pragma unroll
+    for (int nt = 0; nt < NTW; ++nt)
+#pragma unroll
+      for (int s = 0; s < 2; ++s) {
+        const _Float16* crow = Cg + (size_t)(32 * q + j) * N + n0 + 32 * nt + 16 * s + 4 * hh;
+        cfrag[q][nt][s][0] = *reinterpret_cast<const v4h*>(crow);
+        cfrag[q][nt][s][1] = *reinterpret_cast<const v4h*>(crow + 8);
+      }
+
+  // GEMM1: the wave's columns of P for the unit's rows, rounded to fp16
+  v8h pf[NTW][2];
+  {
+    v16f pacc[NTW];
+#pragma unroll
+    for (int nt = 0; nt < NTW; ++nt)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) pacc[nt][r] = 0.0f;
+#pragma unroll
+    for (int s = 0; s < KS; ++s)
+#pragma unroll
+      for (int nt = 0; nt < NTW; ++nt) pacc[nt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(bfrag[nt][s], afrag[s], pacc[nt], 0, 0, 0);
+#pragma unroll
+    for (int nt = 0; nt < NTW; ++nt)
+#pragma unroll
+      for (int s = 0; s < 2; ++s)
+#pragma unroll
+        for (int e = 0; e < 8; ++e) pf[nt][s][e] = (_Float16)pacc[nt][8 * s + e];
+  }
+  // GEMM2 over the wave's n: a partial D^T tile per 32 columns of D
+  v16f dacc[PT];
+#pragma unroll
+  for (int q = 0; q < PT; ++q) {
+#pragma unroll
+    for (int r = 0; r < 16; ++r) dacc[q][r] = 0.0f;
+#pragma unroll
+    for (int nt = 0; nt < NTW; ++nt)
+#pragma unroll
+      for (int s = 0; s < 2; ++s) {
+        const v4h c0 = cfrag[q][nt][s][0], c1 = cfrag[q][nt][s][1];
+        const v8h c = {c0[0], c0[1], c0[2], c0[3], c1[0], c1[1], c1[2], c1[3]};
+        dacc[q] = __builtin_amdgcn_mfma_f32_32x32x16_f16(c, pf[nt][s], dacc[q], 0, 0, 0);
+      }
+  }
+  // partial tiles -> LDS [wave][row][p] (the lane holds p = 32q + 8g + 4hh + r of row j), summed by p quadruples
+  float* mine = red + (size_t)wave * 32 * RLD + j * RLD;
+#pragma unroll
+  for (int q = 0; q < PT; ++q)
+#pragma unroll
+    for (int gq = 0; gq < 4; ++gq)
+      *reinterpret_cast<v4f*>(mine + 32 * q + 8 * gq + 4 * hh) =
+          v4f{dacc[q][4 * gq], dacc[q][4 * gq + 1], dacc[q][4 * gq + 2], dacc[q][4 * gq + 3]};
+  __syncthreads();
+  constexpr int QPR = P / 4;  // quadruples per row
+  for (int idx = tid; idx < 32 * QPR; idx += WAVES * 64) {
+    const int r = idx / QPR, c4 = idx - r * QPR;
+    v4f sum = *reinterpret_cast<const v4f*>(red + r * RLD + 4 * c4);
+#pragma unroll
+    for (int w = 1; w < WAVES; ++w) {
+      const v4f x = *reinterpret_cast<const v4f*>(red + (size_t)w * 32 * RLD + r * RLD + 4 * c4);
+      sum[0] += x[0]; sum[1] += x[1]; sum[2] += x[2]; sum[3] += x[3];
+    }
+    if (r0 + r < M) {
+      const v4h o = {(_Float16)sum[0], (_Float16)sum[1], (_Float16)sum[2], (_Float16)sum[3]};
+      *reinterpret_cast<v4h*>(Dg + (size_t)(r0 + r) * P + 4 * c4) = o;
+    }
+  }
+}
+
+template <int KS, int PT, int NTW, int WAVES>
+static int launch_b2b_wide(const void* A, const void* B, const void* C, void* D, int G, int M, int lds_max, bool* handled,
+                           hipStream_t s) {
+  const size_t lds = (size_t)WAVES * 32 * (32 * PT + 4) * sizeof(float);
+  const long long units = (M + 31) / 32;
+  *handled = (int)lds <= lds_max && units * G <= 0x7fffffffLL;
+  if (!*handled) return FTK_OK;
+  static bool attr_set = false;
+  if (!attr_set) {
+    FTK_HIP(hipFuncSetAttribute((const void*)b2b_wide_kernel<KS, PT, NTW, WAVES>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+    attr_set = true;
+  }
+  hipLaunchKernelGGL((b2b_wide_kernel<KS, PT, NTW, WAVES>), dim3((unsigned)(units * G)), dim3(WAVES * 64), lds, s,
+                     (const _Float16*)A, (const _Float16*)B, (const _Float16*)C, (_Float16*)D, M, (int)units);
+  return check_launch("b2b_wide_kernel");
+}
+
 static int b2b_wave_region(int K, int pw) { return 32 * (K + 8) + 32 * (pw + 4); }
 
 static size_t b2b_lds_bytes(int N, int K, int pw, int waves) {
@@ -614,6 +754,15 @@ extern "C" int ftk_b2b_gemm_f16(const void* A, const void* B, const void* C, voi
   int rc = device_props(&dp);
   if (rc) return rc;
   hipStream_t s = (hipStream_t)stream;
+  // wide N with few columns of D (the reference benchmark's shapes): N split over the waves of a workgroup.
+  // FTK_B2B_WIDE=0 keeps them on the general kernel.
+  static const bool allow_wide = !(getenv("FTK_B2B_WIDE") && atoi(getenv("FTK_B2B_WIDE")) == 0);
+  if (allow_wide && K == 64 && P == 64 && (N == 256 || N == 512)) {
+    bool handled = false;
+    rc = N == 256 ? launch_b2b_wide<4, 2, 1, 8>(A, B, C, D, G, M, dp->lds_optin, &handled, s)
+                  : launch_b2b_wide<4, 2, 2, 8>(A, B, C, D, G, M, dp->lds_optin, &handled, s);
+    if (rc || handled) return rc;
+  }
   switch (K) {
     case 32: return launch_b2b<2>(A, B, C, D, G, M, N, P, dp->cus, dp->lds_optin, s);
     case 64: return launch_b2b<4>(A, B, C, D, G, M, N, P, dp->cus, dp->lds_optin, s);

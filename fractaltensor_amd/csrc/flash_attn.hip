@@ -499,33 +499,36 @@ __global__ __launch_bounds__(WAVES * 64, MINB) void flash_attn_kernel(const _Flo
     step(ntiles - 1, std::false_type{}, std::false_type{});
   }
 
-  // ---- normalise and store.  A lane holds d = 32dt + 8g + 4*half + r of its row: 8-byte pieces,
-  // the other half of each 16 bytes sitting in lane^32.  The two lanes trade pieces (this one's g odd /
-  // g even piece for the partner's) so that each stores 16 contiguous bytes and every store instruction
-  // fills whole 32-byte sectors; with 8-byte stores the memory system writes twice the bytes.
+  // ---- normalise and store.  A lane holds d = 32dt + 8g + 4*half + r of its row: 8-byte pieces scattered over
+  // the row, which as stores fill no cache line (the memory system then writes more than twice the bytes of O).
+  // So the wave turns its 32 x D tile round through LDS, which nobody reads any more after the barrier that ended
+  // the last step: every lane writes its pieces into the wave's own padded tile, then 2D/16 lanes per row read 16
+  // bytes each and the wave stores whole rows, 1 KB of consecutive bytes per instruction.  LDS executes a wave's
+  // instructions in order, so the wave needs no barrier between its writes and its reads.
+  constexpr int ORS = 2 * D + 16;        // padded row: the 32 rows' 8-byte pieces spread over all banks
+  constexpr int LPR = D / 8;             // lanes per row of 16-byte chunks
+  constexpr int RPI = 64 / LPR;          // rows per store instruction
+  unsigned char* const ot = smem + wave * (32 * ORS);
 #pragma unroll
   for (int qt = 0; qt < QT; ++qt) {
     const float l = l_run[qt] + __shfl_xor(l_run[qt], 32);
     const float inv = 1.0f / l;
-    const int row = q_base + 32 * qt + j;
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
-      for (int m = 0; m < 2; ++m) {
-        v2u x, y;  // pieces g = 2m and g = 2m + 1 as packed halfs
-#pragma unroll
-        for (int w = 0; w < 2; ++w) {
-          const v2h xe = {(_Float16)(oacc[qt][dt][8 * m + 2 * w] * inv), (_Float16)(oacc[qt][dt][8 * m + 2 * w + 1] * inv)};
-          const v2h ye = {(_Float16)(oacc[qt][dt][8 * m + 4 + 2 * w] * inv),
-                          (_Float16)(oacc[qt][dt][8 * m + 4 + 2 * w + 1] * inv)};
-          x[w] = __builtin_bit_cast(unsigned, xe);
-          y[w] = __builtin_bit_cast(unsigned, ye);
-          // afterwards lanes 0-31 hold (own x, partner's x), lanes 32-63 (partner's y, own y)
-          asm volatile("s_nop 1\n\tv_permlane32_swap_b32_e32 %0, %1\n\ts_nop 1" : "+v"(x[w]), "+v"(y[w]));
-        }
-        if (row < Sq)
-          *reinterpret_cast<v4u*>(Og + (size_t)row * D + 32 * dt + 16 * m + 8 * hh) = v4u{x[0], x[1], y[0], y[1]};
+      for (int g = 0; g < 4; ++g) {
+        const v2h lo = {(_Float16)(oacc[qt][dt][4 * g] * inv), (_Float16)(oacc[qt][dt][4 * g + 1] * inv)};
+        const v2h hi = {(_Float16)(oacc[qt][dt][4 * g + 2] * inv), (_Float16)(oacc[qt][dt][4 * g + 3] * inv)};
+        *reinterpret_cast<v2u*>(ot + j * ORS + 2 * (32 * dt + 8 * g + 4 * hh)) =
+            v2u{__builtin_bit_cast(unsigned, lo), __builtin_bit_cast(unsigned, hi)};
       }
+#pragma unroll
+    for (int i = 0; i < 32 / RPI; ++i) {
+      const int r = RPI * i + lane / LPR, c = lane % LPR;
+      const v4u piece = *reinterpret_cast<const v4u*>(ot + r * ORS + 16 * c);
+      const int row = q_base + 32 * qt + r;
+      if (row < Sq) *reinterpret_cast<v4u*>(Og + (size_t)row * D + 8 * c) = piece;
+    }
   }
 }
 

@@ -632,8 +632,13 @@ def test_b2b_gemm_rowmajor_rejects_other_shapes(core):
     (1, 32, 32, 32, 32),
     (2, 100, 64, 32, 64),       # ragged M
     (3, 256, 96, 96, 160),      # P spans two workgroup tiles, odd tile counts
-    (1, 8192, 256, 64, 64),     # reference benchmark shape (fused_two_hgemms.cu:152-175)
-    (1, 1024, 512, 64, 64),
+    (1, 8192, 256, 64, 64),     # the reference benchmark's four shapes (fused_two_hgemms.cu:152-175): the wide-N kernel,
+    (1, 8192, 512, 64, 64),     # N split over the waves of a workgroup
+    (1, 16384, 256, 64, 64),
+    (1, 16384, 512, 64, 64),
+    (3, 77, 512, 64, 64),       # wide-N kernel: several problems, ragged rows
+    (2, 1, 256, 64, 64),        # wide-N kernel: a single row
+    (1, 1024, 256, 64, 128),    # wide N with 128 columns of D: the general kernel
     (2, 300, 64, 64, 128),      # eight-wave kernel (N, K in {64, 128}, full 128-column tiles), ragged M
     (2, 1000, 128, 64, 256),    # eight-wave kernel, two column tiles, units that do not divide evenly
     (1, 4100, 128, 128, 160),   # eight-wave kernel for the first 128 columns, four-wave kernel for the last 32
