@@ -537,34 +537,42 @@ static int launch_b2b8(const void* A, const void* B, const void* C, void* D, int
 }
 
 // Wide-N form for the shapes of the reference's own benchmark, [M, 64] x [64, 256 | 512] x [., 64]
-// (benchmarks/fused_two_hgemms/fractaltensor/fused_two_hgemms.cu:152-175): one problem, few bytes (2 MB), so what
-// counts is the length of the dependency chain of one 32-row unit.  A workgroup takes one unit and its WAVES waves
-// split N: wave w forms the 32*NTW columns [n0, n0 + 32 NTW) of P for all 32 rows (K/16 * NTW MFMAs), rounds them to
-// fp16 and multiplies them with its rows of C (2 * NTW * PT MFMAs), which leaves a partial D tile per wave; the
-// partials are summed in fp32 through LDS and the 32 x P tile leaves as whole rows.  B and C are read once per
-// workgroup straight into MFMA operands (16-byte and 8-byte pieces from the cache hierarchy: each wave needs only its
-// own slice, nothing is staged), the A rows by every wave.  The contraction order of both products is the one of the
-// kernels above.
+// (benchmarks/fused_two_hgemms/fractaltensor/fused_two_hgemms.cu:152-175): one problem, few bytes (2 to 4.5 MB that
+// stay in the caches), so what counts is the length of the dependency chain and how many cache lines a workgroup
+// touches.  The WAVES waves of a workgroup split N: wave w forms the 32*NTW columns [n0, n0 + 32 NTW) of P for a
+// 32-row unit (K/16 * NTW MFMAs), rounds them to fp16 and multiplies them with its rows of C (2 * NTW * PT MFMAs),
+// which leaves a partial D tile per wave; the partials are summed in fp32 through LDS and the 32 x P tile leaves as
+// whole rows.  A wave's operands of B and C do not depend on the unit: the workgroup brings B and then C through
+// LDS once (coalesced 16-byte loads, every cache line once; a wave's strided fragment loads would touch 32 lines per
+// instruction), every wave keeps its fragments in registers, and the workgroup then walks its units with the next
+// unit's A rows on the way while the current one is computed.  The contraction order of both products is the one
+// of the kernels above.
 template <int KS, int PT, int NTW, int WAVES>
 __global__ __launch_bounds__(WAVES * 64) void b2b_wide_kernel(const _Float16* __restrict__ A,
                                                               const _Float16* __restrict__ Bm,
                                                               const _Float16* __restrict__ Cm, _Float16* __restrict__ D,
-                                                              int M, int units) {
+                                                              int M, int units, int per) {
   constexpr int K = 16 * KS;
   constexpr int N = 32 * NTW * WAVES;
   constexpr int P = 32 * PT;
+  constexpr int threads = WAVES * 64;
+  constexpr int BLD = K + 8;  // padded row of B and of the A units (halfs)
+  constexpr int CLD = N + 4;  // padded row of C (halfs)
   constexpr int RLD = P + 4;  // padded row of a partial tile (floats)
+  constexpr int CPR = K / 8;  // 16-byte chunks per row of A and B
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
-  float* red = reinterpret_cast<float*>(smem);  // [WAVES][32][RLD]
+  // first B, then C pass through the whole of it; afterwards [A units x 2][partial tiles]
+  _Float16* const stage = reinterpret_cast<_Float16*>(smem);
+  _Float16* const As = reinterpret_cast<_Float16*>(smem);                  // [2][32][BLD]
+  float* const red = reinterpret_cast<float*>(smem + 2 * 32 * BLD * 2);    // [WAVES][32][RLD]
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = tid >> 6;
   const int j = lane & 31;
   const int hh = lane >> 5;
-  const int g = blockIdx.x / units;
-  const int unit = blockIdx.x - g * units;
-  const int r0 = unit * 32;
+  const int g = blockIdx.x / per;
+  const int part = blockIdx.x - g * per;
   const int n0 = wave * 32 * NTW;
 
   const _Float16* Ag = A + (size_t)g * M * K;
@@ -572,101 +580,157 @@ __global__ __launch_bounds__(WAVES * 64) void b2b_wide_kernel(const _Float16* __
   const _Float16* Cg = Cm + (size_t)g * P * N;
   _Float16* Dg = D + (size_t)g * M * P;
 
-  // every load of the wave is requested before the first is used
-  v8h afrag[KS], bfrag[NTW][KS];
-  const _Float16* arow = Ag + (size_t)min(r0 + j, M - 1) * K + hh * (K / 2);
+  // ---- B, C and the first A unit: every load requested before the first is used
+  constexpr int nb = N * CPR, nc = P * (N / 8);
+  constexpr int UB = (nb + threads - 1) / threads, UC = (nc + threads - 1) / threads;
+  constexpr bool a_all = 32 * CPR <= threads;   // one chunk of an A unit per thread
+  static_assert(a_all, "an A unit is fetched by one load per thread");
+  v4u vb[UB], vc[UC], va;
+  auto fetch_a = [&](int un) __attribute__((always_inline)) {
+    if (tid < 32 * CPR) va = ldg16(Ag + (size_t)min(un * 32 + tid / CPR, M - 1) * K + 8 * (tid % CPR));
+  };
+  auto park_a = [&](int buf) __attribute__((always_inline)) {
+    if (tid < 32 * CPR) *reinterpret_cast<v4u*>(As + buf * 32 * BLD + (tid / CPR) * BLD + 8 * (tid % CPR)) = va;
+  };
 #pragma unroll
-  for (int s = 0; s < KS; ++s) afrag[s] = __builtin_bit_cast(v8h, ldg16(arow + 8 * s));
+  for (int u = 0; u < UB; ++u) {
+    const int idx = u * threads + tid;
+    if (idx < nb) vb[u] = ldg16(Bg + (size_t)idx * 8);
+  }
+#pragma unroll
+  for (int u = 0; u < UC; ++u) {
+    const int idx = u * threads + tid;
+    if (idx < nc) vc[u] = ldg16(Cg + (size_t)idx * 8);
+  }
+  int unit = part;
+  if (unit < units) fetch_a(unit);
+
+  v8h bfrag[NTW][KS];
+  v4h cfrag[PT][NTW][2][2];
+#pragma unroll
+  for (int u = 0; u < UB; ++u) {
+    const int idx = u * threads + tid;
+    if (idx < nb) *reinterpret_cast<v4u*>(stage + (idx / CPR) * BLD + 8 * (idx % CPR)) = vb[u];
+  }
+  __syncthreads();
 #pragma unroll
   for (int nt = 0; nt < NTW; ++nt)
 #pragma unroll
     for (int s = 0; s < KS; ++s)
-      bfrag[nt][s] = __builtin_bit_cast(v8h, ldg16(Bg + (size_t)(n0 + 32 * nt + j) * K + hh * (K / 2) + 8 * s));
-  v4h cfrag[PT][NTW][2][2];
+      bfrag[nt][s] = *reinterpret_cast<const v8h*>(stage + (n0 + 32 * nt + j) * BLD + hh * (K / 2) + 8 * s);
+  __syncthreads();
+#pragma unroll
+  for (int u = 0; u < UC; ++u) {
+    const int idx = u * threads + tid;
+    if (idx < nc) {
+      const int p = idx / (N / 8), n8 = idx % (N / 8);
+      *reinterpret_cast<v2u*>(stage + p * CLD + 8 * n8) = v2u{vc[u][0], vc[u][1]};   // CLD is no multiple of 8 halfs
+      *reinterpret_cast<v2u*>(stage + p * CLD + 8 * n8 + 4) = v2u{vc[u][2], vc[u][3]};
+    }
+  }
+  __syncthreads();
 #pragma unroll
   for (int q = 0; q < PT; ++q)
 #pragma unroll
     for (int nt = 0; nt < NTW; ++nt)
 #pragma unroll
       for (int s = 0; s < 2; ++s) {
-        const _Float16* crow = Cg + (size_t)(32 * q + j) * N + n0 + 32 * nt + 16 * s + 4 * hh;
+        const _Float16* crow = stage + (32 * q + j) * CLD + n0 + 32 * nt + 16 * s + 4 * hh;
         cfrag[q][nt][s][0] = *reinterpret_cast<const v4h*>(crow);
         cfrag[q][nt][s][1] = *reinterpret_cast<const v4h*>(crow + 8);
       }
-
-  // GEMM1: the wave's columns of P for the unit's rows, rounded to fp16
-  v8h pf[NTW][2];
-  {
-    v16f pacc[NTW];
-#pragma unroll
-    for (int nt = 0; nt < NTW; ++nt)
-#pragma unroll
-      for (int r = 0; r < 16; ++r) pacc[nt][r] = 0.0f;
-#pragma unroll
-    for (int s = 0; s < KS; ++s)
-#pragma unroll
-      for (int nt = 0; nt < NTW; ++nt) pacc[nt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(bfrag[nt][s], afrag[s], pacc[nt], 0, 0, 0);
-#pragma unroll
-    for (int nt = 0; nt < NTW; ++nt)
-#pragma unroll
-      for (int s = 0; s < 2; ++s)
-#pragma unroll
-        for (int e = 0; e < 8; ++e) pf[nt][s][e] = (_Float16)pacc[nt][8 * s + e];
-  }
-  // GEMM2 over the wave's n: a partial D^T tile per 32 columns of D
-  v16f dacc[PT];
-#pragma unroll
-  for (int q = 0; q < PT; ++q) {
-#pragma unroll
-    for (int r = 0; r < 16; ++r) dacc[q][r] = 0.0f;
-#pragma unroll
-    for (int nt = 0; nt < NTW; ++nt)
-#pragma unroll
-      for (int s = 0; s < 2; ++s) {
-        const v4h c0 = cfrag[q][nt][s][0], c1 = cfrag[q][nt][s][1];
-        const v8h c = {c0[0], c0[1], c0[2], c0[3], c1[0], c1[1], c1[2], c1[3]};
-        dacc[q] = __builtin_amdgcn_mfma_f32_32x32x16_f16(c, pf[nt][s], dacc[q], 0, 0, 0);
-      }
-  }
-  // partial tiles -> LDS [wave][row][p] (the lane holds p = 32q + 8g + 4hh + r of row j), summed by p quadruples
-  float* mine = red + (size_t)wave * 32 * RLD + j * RLD;
-#pragma unroll
-  for (int q = 0; q < PT; ++q)
-#pragma unroll
-    for (int gq = 0; gq < 4; ++gq)
-      *reinterpret_cast<v4f*>(mine + 32 * q + 8 * gq + 4 * hh) =
-          v4f{dacc[q][4 * gq], dacc[q][4 * gq + 1], dacc[q][4 * gq + 2], dacc[q][4 * gq + 3]};
   __syncthreads();
-  constexpr int QPR = P / 4;  // quadruples per row
-  for (int idx = tid; idx < 32 * QPR; idx += WAVES * 64) {
-    const int r = idx / QPR, c4 = idx - r * QPR;
-    v4f sum = *reinterpret_cast<const v4f*>(red + r * RLD + 4 * c4);
+  if (unit < units) park_a(0);
+  __syncthreads();
+
+  int buf = 0;
+  for (; unit < units; unit += per) {
+    const int next = unit + per;
+    if (next < units) fetch_a(next);
+    const int r0 = unit * 32;
+    // GEMM1: the wave's columns of P for the unit's rows, rounded to fp16
+    v8h pf[NTW][2];
+    {
+      const _Float16* arow = As + buf * 32 * BLD + j * BLD + hh * (K / 2);
+      v8h afrag[KS];
 #pragma unroll
-    for (int w = 1; w < WAVES; ++w) {
-      const v4f x = *reinterpret_cast<const v4f*>(red + (size_t)w * 32 * RLD + r * RLD + 4 * c4);
-      sum[0] += x[0]; sum[1] += x[1]; sum[2] += x[2]; sum[3] += x[3];
+      for (int s = 0; s < KS; ++s) afrag[s] = *reinterpret_cast<const v8h*>(arow + 8 * s);
+      v16f pacc[NTW];
+#pragma unroll
+      for (int nt = 0; nt < NTW; ++nt)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) pacc[nt][r] = 0.0f;
+#pragma unroll
+      for (int s = 0; s < KS; ++s)
+#pragma unroll
+        for (int nt = 0; nt < NTW; ++nt) pacc[nt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(bfrag[nt][s], afrag[s], pacc[nt], 0, 0, 0);
+#pragma unroll
+      for (int nt = 0; nt < NTW; ++nt)
+#pragma unroll
+        for (int s = 0; s < 2; ++s)
+#pragma unroll
+          for (int e = 0; e < 8; ++e) pf[nt][s][e] = (_Float16)pacc[nt][8 * s + e];
     }
-    if (r0 + r < M) {
-      const v4h o = {(_Float16)sum[0], (_Float16)sum[1], (_Float16)sum[2], (_Float16)sum[3]};
-      *reinterpret_cast<v4h*>(Dg + (size_t)(r0 + r) * P + 4 * c4) = o;
+    // GEMM2 over the wave's n: a partial D^T tile per 32 columns of D, written to LDS [wave][row][p]
+    // (the lane holds p = 32q + 8g + 4hh + r of row j)
+    float* mine = red + (size_t)wave * 32 * RLD + j * RLD;
+#pragma unroll
+    for (int q = 0; q < PT; ++q) {
+      v16f dacc;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) dacc[r] = 0.0f;
+#pragma unroll
+      for (int nt = 0; nt < NTW; ++nt)
+#pragma unroll
+        for (int s = 0; s < 2; ++s) {
+          const v4h c0 = cfrag[q][nt][s][0], c1 = cfrag[q][nt][s][1];
+          const v8h c = {c0[0], c0[1], c0[2], c0[3], c1[0], c1[1], c1[2], c1[3]};
+          dacc = __builtin_amdgcn_mfma_f32_32x32x16_f16(c, pf[nt][s], dacc, 0, 0, 0);
+        }
+#pragma unroll
+      for (int gq = 0; gq < 4; ++gq)
+        *reinterpret_cast<v4f*>(mine + 32 * q + 8 * gq + 4 * hh) = v4f{dacc[4 * gq], dacc[4 * gq + 1], dacc[4 * gq + 2], dacc[4 * gq + 3]};
     }
+    __syncthreads();
+    constexpr int QPR = P / 4;  // quadruples per row
+    for (int idx = tid; idx < 32 * QPR; idx += threads) {
+      const int r = idx / QPR, c4 = idx - r * QPR;
+      v4f sum = *reinterpret_cast<const v4f*>(red + r * RLD + 4 * c4);
+#pragma unroll
+      for (int w = 1; w < WAVES; ++w) {
+        const v4f x = *reinterpret_cast<const v4f*>(red + (size_t)w * 32 * RLD + r * RLD + 4 * c4);
+        sum[0] += x[0]; sum[1] += x[1]; sum[2] += x[2]; sum[3] += x[3];
+      }
+      if (r0 + r < M) {
+        const v4h o = {(_Float16)sum[0], (_Float16)sum[1], (_Float16)sum[2], (_Float16)sum[3]};
+        *reinterpret_cast<v4h*>(Dg + (size_t)(r0 + r) * P + 4 * c4) = o;
+      }
+    }
+    if (next < units) park_a(buf ^ 1);
+    __syncthreads();
+    buf ^= 1;
   }
 }
 
 template <int KS, int PT, int NTW, int WAVES>
-static int launch_b2b_wide(const void* A, const void* B, const void* C, void* D, int G, int M, int lds_max, bool* handled,
-                           hipStream_t s) {
-  const size_t lds = (size_t)WAVES * 32 * (32 * PT + 4) * sizeof(float);
+static int launch_b2b_wide(const void* A, const void* B, const void* C, void* D, int G, int M, int cus, int lds_max,
+                           bool* handled, hipStream_t s) {
+  constexpr int K = 16 * KS, N = 32 * NTW * WAVES, P = 32 * PT;
+  const size_t loop_bytes = (size_t)2 * 32 * (K + 8) * 2 + (size_t)WAVES * 32 * (P + 4) * sizeof(float);
+  const size_t stage_bytes = std::max((size_t)N * (K + 8) * 2, (size_t)P * (N + 4) * 2);
+  const size_t lds = std::max(loop_bytes, stage_bytes);
   const long long units = (M + 31) / 32;
-  *handled = (int)lds <= lds_max && units * G <= 0x7fffffffLL;
+  // enough workgroups to fill the chip once; each walks its share of the units with B and C fragments in registers
+  const long long per = std::max(1LL, std::min(units, (long long)cus / std::max(1, G)));
+  *handled = (int)lds <= lds_max && per * G <= 0x7fffffffLL;
   if (!*handled) return FTK_OK;
   static bool attr_set = false;
   if (!attr_set) {
     FTK_HIP(hipFuncSetAttribute((const void*)b2b_wide_kernel<KS, PT, NTW, WAVES>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
     attr_set = true;
   }
-  hipLaunchKernelGGL((b2b_wide_kernel<KS, PT, NTW, WAVES>), dim3((unsigned)(units * G)), dim3(WAVES * 64), lds, s,
-                     (const _Float16*)A, (const _Float16*)B, (const _Float16*)C, (_Float16*)D, M, (int)units);
+  hipLaunchKernelGGL((b2b_wide_kernel<KS, PT, NTW, WAVES>), dim3((unsigned)(per * G)), dim3(WAVES * 64), lds, s,
+                     (const _Float16*)A, (const _Float16*)B, (const _Float16*)C, (_Float16*)D, M, (int)units, (int)per);
   return check_launch("b2b_wide_kernel");
 }
 
@@ -759,8 +823,8 @@ extern "C" int ftk_b2b_gemm_f16(const void* A, const void* B, const void* C, voi
   static const bool allow_wide = !(getenv("FTK_B2B_WIDE") && atoi(getenv("FTK_B2B_WIDE")) == 0);
   if (allow_wide && K == 64 && P == 64 && (N == 256 || N == 512)) {
     bool handled = false;
-    rc = N == 256 ? launch_b2b_wide<4, 2, 1, 8>(A, B, C, D, G, M, dp->lds_optin, &handled, s)
-                  : launch_b2b_wide<4, 2, 2, 8>(A, B, C, D, G, M, dp->lds_optin, &handled, s);
+    rc = N == 256 ? launch_b2b_wide<4, 2, 1, 8>(A, B, C, D, G, M, dp->cus, dp->lds_optin, &handled, s)
+                  : launch_b2b_wide<4, 2, 2, 8>(A, B, C, D, G, M, dp->cus, dp->lds_optin, &handled, s);
     if (rc || handled) return rc;
   }
   switch (K) {
