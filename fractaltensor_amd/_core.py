@@ -25,7 +25,6 @@ EXPORTS = (
     'ftk_stacked_lstm_f16_workspace_bytes', 'ftk_stacked_lstm_f16',
     'ftk_b2b_gemm_f16', 'ftk_b2b_gemm_rowmajor_f16', 'ftk_gemm_f16', 'ftk_batched_gemm_f16', 'ftk_flash_attn_f16', 'ftk_online_softmax_f32', 'ftk_embedding_gather_f32',
     'ftk_grid_rnn_workspace_bytes', 'ftk_grid_rnn_f32', 'ftk_windowed_attn_f32',
-    'ftk_debug_read_fa_trace',
 )
 
 
@@ -498,10 +497,15 @@ def flash_attention(Q, K, V, scale: Optional[float] = None, out: Optional[torch.
 
 
 def read_fa_trace(tiles: int):
-    """Timeline of one wave of workgroup 0 of the last flash-attention launch (needs FTK_FA_TRACE=1+wave): [tiles, 6] in us."""
+    """Timeline of one wave of workgroup 0 of the last flash-attention launch: [tiles, 6] in us.  Only a tuning
+    build of the library (make TRACE=1, run with FTK_FA_TRACE=1+wave) records it."""
     import numpy as np
+    fn = getattr(lib, 'ftk_debug_read_fa_trace', None)
+    if fn is None:
+        raise RuntimeError('this build of libftkernels.so has no attention timeline: build it with make TRACE=1')
+    fn.restype = ctypes.c_int
     buf = (ctypes.c_longlong * (tiles * 6))()
-    _check(lib.ftk_debug_read_fa_trace(buf, ctypes.c_int(tiles * 6)))
+    _check(fn(buf, ctypes.c_int(tiles * 6)))
     return np.frombuffer(buf, dtype=np.int64).reshape(tiles, 6).astype(np.float64) / 100.0
 
 

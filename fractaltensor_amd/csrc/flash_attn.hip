@@ -49,8 +49,11 @@ constexpr int FA_KT = 64;          // keys per tile
 constexpr float FA_TAU = 8.0f;     // slack (in powers of two) before the running maximum is moved
 constexpr int FA_TRACE_TILES = 256;
 
-// Timeline of workgroup 0 / thread 0 when FTK_FA_TRACE is set: six stamps per key tile.
+// Built with -DFTK_DEBUG_TRACE only (make TRACE=1): timeline of one wave of workgroup 0 when FTK_FA_TRACE is set,
+// six stamps per key tile, read back with ftk_debug_read_fa_trace.  The library as shipped has neither.
+#ifdef FTK_DEBUG_TRACE
 __device__ long long fa_trace_buf[FA_TRACE_TILES * 6];
+#endif
 
 typedef short v4s __attribute__((ext_vector_type(4)));
 
@@ -99,7 +102,10 @@ struct FaLayout {
 };
 
 // MINB: workgroups per CU the register budget must allow.
-template <int D, int QT, int WAVES, int MINB, bool TRACE>
+// RAG: Skv is no multiple of the key tile (the last tile's tail is masked); a template parameter so that the kernel
+// for whole tiles carries none of the masking code (with both in one kernel the tail steps spilled 63 registers per
+// lane to scratch, which every wave wrote once: 87 MB of extra HBM writes per launch at B8 H16 S2048).
+template <int D, int QT, int WAVES, int MINB, bool TRACE, bool RAG>
 __global__ __launch_bounds__(WAVES * 64, MINB) void flash_attn_kernel(const _Float16* __restrict__ Q,
                                                          const _Float16* __restrict__ K,
                                                          const _Float16* __restrict__ V,
@@ -236,7 +242,7 @@ __global__ __launch_bounds__(WAVES * 64, MINB) void flash_attn_kernel(const _Flo
   const int v_lane = (4 * hh + ((lane & 15) >> 2)) * VRS + 32 * ((lane >> 4) & 1) + 8 * (lane & 3);
 
   const int ntiles = (Skv + FA_KT - 1) / FA_KT;
-  const bool has_ragged = (Skv % FA_KT) != 0;
+  constexpr bool has_ragged = RAG;
 
   using lds_v4s = __attribute__((address_space(3))) v4s;
   typedef short v8s __attribute__((ext_vector_type(8)));
@@ -491,7 +497,7 @@ __global__ __launch_bounds__(WAVES * 64, MINB) void flash_attn_kernel(const _Flo
   // Only the two steps that touch the last tile pay for masking its ragged
   // tail; they are peeled so that the main loop body is one straight line.
   for (int kt = 0; kt + 2 < ntiles; ++kt) step(kt, std::true_type{}, std::false_type{});
-  if (has_ragged) {
+  if constexpr (has_ragged) {
     if (ntiles > 1) step(ntiles - 2, std::true_type{}, std::true_type{});
     step(ntiles - 1, std::false_type{}, std::true_type{});
   } else {
@@ -532,6 +538,7 @@ __global__ __launch_bounds__(WAVES * 64, MINB) void flash_attn_kernel(const _Flo
   }
 }
 
+#ifdef FTK_DEBUG_TRACE
 // FTK_FA_TRACE=1+w turns the per-tile timeline of wave w of workgroup 0 on (read once).
 static int fa_trace_wave() {
   const char* e = getenv("FTK_FA_TRACE");
@@ -548,6 +555,7 @@ static long long* fa_trace_ptr() {
   }
   return on ? ptr : nullptr;
 }
+#endif
 
 template <int D, int QT, int WAVES, int MINB>
 static int launch_fa(const void* Q, const void* K, const void* V, void* O, int BH, int Sq, int Skv, float scale,
@@ -556,25 +564,36 @@ static int launch_fa(const void* Q, const void* K, const void* V, void* O, int B
   if ((int)lds > lds_max) return fail(FTK_ERR_UNSUPPORTED_SHAPE, "ftk_flash_attn_f16: needs %zu bytes of LDS", lds);
   static bool attr_set = false;
   if (!attr_set) {
-    FTK_HIP(hipFuncSetAttribute((const void*)flash_attn_kernel<D, QT, WAVES, MINB, false>,
+    FTK_HIP(hipFuncSetAttribute((const void*)flash_attn_kernel<D, QT, WAVES, MINB, false, false>,
                                 hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-    FTK_HIP(hipFuncSetAttribute((const void*)flash_attn_kernel<D, QT, WAVES, MINB, true>,
+    FTK_HIP(hipFuncSetAttribute((const void*)flash_attn_kernel<D, QT, WAVES, MINB, false, true>,
                                 hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+#ifdef FTK_DEBUG_TRACE
+    FTK_HIP(hipFuncSetAttribute((const void*)flash_attn_kernel<D, QT, WAVES, MINB, true, true>,
+                                hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+#endif
     attr_set = true;
   }
   constexpr int ROWS = WAVES * 32 * QT;
   const int nqb = (Sq + ROWS - 1) / ROWS;
   const long long total = (long long)nqb * BH;
   if (total > 0x7fffffffLL) return fail(FTK_ERR_UNSUPPORTED_SHAPE, "ftk_flash_attn_f16: grid too large");
-  long long* trace = fa_trace_ptr();
-  if (trace)
-    hipLaunchKernelGGL((flash_attn_kernel<D, QT, WAVES, MINB, true>), dim3((unsigned)total), dim3(WAVES * 64), lds,
+#ifdef FTK_DEBUG_TRACE
+  if (long long* trace = fa_trace_ptr()) {
+    hipLaunchKernelGGL((flash_attn_kernel<D, QT, WAVES, MINB, true, true>), dim3((unsigned)total), dim3(WAVES * 64), lds,
                        s, (const _Float16*)Q, (const _Float16*)K, (const _Float16*)V, (_Float16*)O, Sq, Skv,
                        scale * 1.4426950408889634f, nqb, trace, fa_trace_wave());
+    return check_launch("flash_attn_kernel");
+  }
+#endif
+  if (Skv % FA_KT)
+    hipLaunchKernelGGL((flash_attn_kernel<D, QT, WAVES, MINB, false, true>), dim3((unsigned)total), dim3(WAVES * 64), lds,
+                       s, (const _Float16*)Q, (const _Float16*)K, (const _Float16*)V, (_Float16*)O, Sq, Skv,
+                       scale * 1.4426950408889634f, nqb, (long long*)nullptr, 0);
   else
-    hipLaunchKernelGGL((flash_attn_kernel<D, QT, WAVES, MINB, false>), dim3((unsigned)total), dim3(WAVES * 64), lds,
+    hipLaunchKernelGGL((flash_attn_kernel<D, QT, WAVES, MINB, false, false>), dim3((unsigned)total), dim3(WAVES * 64), lds,
                        s, (const _Float16*)Q, (const _Float16*)K, (const _Float16*)V, (_Float16*)O, Sq, Skv,
-                       scale * 1.4426950408889634f, nqb, trace, fa_trace_wave());
+                       scale * 1.4426950408889634f, nqb, (long long*)nullptr, 0);
   return check_launch("flash_attn_kernel");
 }
 
@@ -591,6 +610,9 @@ static int fa_variant_override() {
 
 }  // namespace ftk
 
+#ifdef FTK_DEBUG_TRACE
+// Copies the first n stamps of the last traced launch to host memory (synchronises the device).  Not part of
+// include/ftk.h: a tuning build declares it itself.
 extern "C" int ftk_debug_read_fa_trace(long long* host_dst, int n) {
   using namespace ftk;
   if (!host_dst || n <= 0 || n > FA_TRACE_TILES * 6)
@@ -599,6 +621,7 @@ extern "C" int ftk_debug_read_fa_trace(long long* host_dst, int n) {
   FTK_HIP(hipMemcpyFromSymbol(host_dst, HIP_SYMBOL(fa_trace_buf), sizeof(long long) * n));
   return FTK_OK;
 }
+#endif
 
 extern "C" int ftk_flash_attn_f16(const void* Q, const void* K, const void* V, void* O, int B, int Hd, int Sq, int Skv,
                                   int D, float scale, ftk_stream_t stream) {

@@ -448,18 +448,6 @@ int ftk_windowed_attn_f32(const float* Q, const float* K, const float* V,
 int ftk_online_softmax_f32(const float* x, float* y, int rows, int cols,
                            ftk_stream_t stream);
 
-/* ---------------------------------------------------------- diagnostics -- */
-
-/*
- * With FTK_FA_TRACE=1+w in the environment, wave w of workgroup 0 of every
- * ftk_flash_attn_f16 launch records six 100 MHz clock stamps per key tile
- * (tile start; after each of the four pipeline blocks: exponentials | next
- * scores, P V | row maxima, twice; after its copies have landed).  This copies
- * the first n stamps to HOST memory (n <= 1536); it synchronises the device.
- * No counterpart in the reference.
- */
-int ftk_debug_read_fa_trace(long long* host_dst, int n);
-
 #ifdef __cplusplus
 }
 #endif
