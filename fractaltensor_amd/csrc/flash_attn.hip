@@ -171,6 +171,7 @@ __global__ __launch_bounds__(WAVES * 64, MINB) void flash_attn_kernel(const _Flo
       for (int r = 0; r < 16; ++r) oacc[qt][dt][r] = 0.0f;
   }
 
+  constexpr bool has_ragged = RAG;
   // ---- copies: copy c of a tile fills LDS bytes [1024c, 1024c + 1024) of the
   // padded tile, lane l the 16 bytes at 1024c + 16l; slots in the padding
   // fetch the row's first chunk (never read).  Wave w issues copies w, w+WAVES, ...
@@ -194,7 +195,7 @@ __global__ __launch_bounds__(WAVES * 64, MINB) void flash_attn_kernel(const _Flo
       if (wave + WAVES * i < KTB / 1024) {
         const int key0 = kt * FA_KT;
         unsigned off = k_src[i];
-        if (key0 + FA_KT > Skv) {  // ragged last tile: rows past the end re-read the last key (their scores are masked)
+        if (has_ragged && key0 + FA_KT > Skv) {  // ragged last tile: rows past the end re-read the last key (their scores are masked)
           const unsigned last = (unsigned)(Skv - 1 - key0), row = off / RB;
           if (row > last) off -= (row - last) * RB;
         }
@@ -208,7 +209,7 @@ __global__ __launch_bounds__(WAVES * 64, MINB) void flash_attn_kernel(const _Flo
       if (wave + WAVES * i < VTB / 1024) {
         const int key0 = kt * FA_KT;
         unsigned off = v_src[i];
-        if (key0 + FA_KT > Skv) {
+        if (has_ragged && key0 + FA_KT > Skv) {
           const unsigned last = (unsigned)(Skv - 1 - key0), row = off / RB;
           if (row > last) off -= (row - last) * RB;
         }
@@ -242,7 +243,6 @@ __global__ __launch_bounds__(WAVES * 64, MINB) void flash_attn_kernel(const _Flo
   const int v_lane = (4 * hh + ((lane & 15) >> 2)) * VRS + 32 * ((lane >> 4) & 1) + 8 * (lane & 3);
 
   const int ntiles = (Skv + FA_KT - 1) / FA_KT;
-  constexpr bool has_ragged = RAG;
 
   using lds_v4s = __attribute__((address_space(3))) v4s;
   typedef short v8s __attribute__((ext_vector_type(8)));
@@ -328,18 +328,19 @@ __global__ __launch_bounds__(WAVES * 64, MINB) void flash_attn_kernel(const _Flo
   // step of P V, which starts at step DT).  Fragment reads run three steps
   // ahead throughout, across block boundaries: the last three steps of a block
   // read the first three fragments of the next one (kpre / vpre).
-  constexpr int NE = 12;
+  constexpr int NE = 12;   // 8 to 16 measure the same
   constexpr int NS = 2 * DT;
-  v8h kpre[3], vpre[3];
+  constexpr int LA = 3;   // fragments read ahead of the matrix instruction that uses them (4 to 6 measure the same)
+  static_assert(LA <= DS && LA <= NS, "the lookahead must fit in one block");
+  v8h kpre[LA], vpre[LA];
   auto block_e = [&](const unsigned char* kbase, const unsigned char* vbase, const v16f (&sc)[QT], v8h (&pf)[QT][2],
                      v16f (&sn)[QT], auto next_c) __attribute__((always_inline)) {
     constexpr bool has_next = decltype(next_c)::value;
 #pragma unroll
     for (int qt = 0; qt < QT; ++qt) psum[qt] = 0.0f;
     v8h kf[DS];
-    kf[0] = kpre[0];
-    kf[1] = kpre[1];
-    kf[2] = kpre[2];
+#pragma unroll
+    for (int i = 0; i < LA; ++i) kf[i] = kpre[i];
     __builtin_amdgcn_sched_barrier(0);
     static_for<DS>([&](auto s_c) __attribute__((always_inline)) {
       constexpr int s = decltype(s_c)::value;
@@ -347,9 +348,9 @@ __global__ __launch_bounds__(WAVES * 64, MINB) void flash_attn_kernel(const _Flo
 #pragma unroll
         for (int qt = 0; qt < QT; ++qt)
           sn[qt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(kf[s], qf[qt][s], s == 0 ? nref[qt] : sn[qt], 0, 0, 0);
-        if constexpr (s + 3 < DS) kf[s + 3] = read_k(kbase, s + 3);
+        if constexpr (s + LA < DS) kf[s + LA] = read_k(kbase, s + LA);
       }
-      if constexpr (s + 3 >= DS) vpre[s + 3 - DS] = read_v(vbase, (s + 3 - DS) / DT, (s + 3 - DS) % DT);
+      if constexpr (s + LA >= DS) vpre[s + LA - DS] = read_v(vbase, (s + LA - DS) / DT, (s + LA - DS) % DT);
       // scores [s*NE/DS, (s+1)*NE/DS)
       static_for<((s + 1) * NE) / DS - (s * NE) / DS>([&](auto i_c) __attribute__((always_inline)) {
         exp_element(sc, pf, std::integral_constant<int, (s * NE) / DS + decltype(i_c)::value>{});
@@ -364,9 +365,8 @@ __global__ __launch_bounds__(WAVES * 64, MINB) void flash_attn_kernel(const _Flo
     constexpr bool mask = decltype(mask_c)::value;
     constexpr bool prefetch_k = decltype(prek_c)::value;
     v8h vf[NS];
-    vf[0] = vpre[0];
-    vf[1] = vpre[1];
-    vf[2] = vpre[2];
+#pragma unroll
+    for (int i = 0; i < LA; ++i) vf[i] = vpre[i];
     float mx[QT];
     __builtin_amdgcn_sched_barrier(0);
     static_for<NS>([&](auto i_c) __attribute__((always_inline)) {
@@ -375,10 +375,10 @@ __global__ __launch_bounds__(WAVES * 64, MINB) void flash_attn_kernel(const _Flo
 #pragma unroll
       for (int qt = 0; qt < QT; ++qt)
         oacc[qt][dt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(vf[i], pf[qt][s], oacc[qt][dt], 0, 0, 0);
-      if constexpr (i + 3 < NS) {
-        vf[i + 3] = read_v(vbase, (i + 3) / DT, (i + 3) % DT);
+      if constexpr (i + LA < NS) {
+        vf[i + LA] = read_v(vbase, (i + LA) / DT, (i + LA) % DT);
       } else if constexpr (prefetch_k) {
-        kpre[i + 3 - NS] = read_k(knext, i + 3 - NS);
+        kpre[i + LA - NS] = read_k(knext, i + LA - NS);
       }
       if constexpr (i < DT) {
         // remaining scores [NE + i*(16-NE)/DT, NE + (i+1)*(16-NE)/DT)
@@ -452,7 +452,7 @@ __global__ __launch_bounds__(WAVES * 64, MINB) void flash_attn_kernel(const _Flo
       }
     }
 #pragma unroll
-    for (int i = 0; i < 3; ++i) kpre[i] = read_k(kbase + 32 * KRS, i);
+    for (int i = 0; i < LA; ++i) kpre[i] = read_k(kbase + 32 * KRS, i);
   }
 
   // One step = one 64-key tile: E and A for its first half (scores of the
