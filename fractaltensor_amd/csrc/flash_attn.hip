@@ -533,7 +533,9 @@ __global__ __launch_bounds__(WAVES * 64, MINB) void flash_attn_kernel(const _Flo
       const int r = RPI * i + lane / LPR, c = lane % LPR;
       const v4u piece = *reinterpret_cast<const v4u*>(ot + r * ORS + 16 * c);
       const int row = q_base + 32 * qt + r;
-      if (row < Sq) *reinterpret_cast<v4u*>(Og + (size_t)row * D + 8 * c) = piece;
+      // streaming store: O is not read again by this launch, and lines left dirty in L2 are written back only when
+      // the kernel ends, which the next launch in the stream waits for
+      if (row < Sq) __builtin_nontemporal_store(piece, reinterpret_cast<v4u*>(Og + (size_t)row * D + 8 * c));
     }
   }
 }

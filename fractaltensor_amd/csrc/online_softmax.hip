@@ -81,9 +81,10 @@ __global__ __launch_bounds__(256) void softmax_rows_in_registers_kernel(const fl
     const int c = (sub + LPR * p) * W;
     if (c < cols) {
       if constexpr (VEC) {
-        *reinterpret_cast<float4*>(yr + c) = make_float4(v[p][0] * scale, v[p][1] * scale, v[p][2] * scale, v[p][3] * scale);
+        // streaming stores: y is not read again, and lines left dirty in L2 hold up the end of the kernel
+        __builtin_nontemporal_store(v4f{v[p][0] * scale, v[p][1] * scale, v[p][2] * scale, v[p][3] * scale}, reinterpret_cast<v4f*>(yr + c));
       } else {
-        yr[c] = v[p][0] * scale;
+        __builtin_nontemporal_store(v[p][0] * scale, yr + c);
       }
     }
   }
@@ -137,10 +138,10 @@ __global__ __launch_bounds__(1024) void softmax_long_rows_kernel(const float* __
   for (int p = threadIdx.x; p < pieces; p += 1024) {
     if constexpr (VEC) {
       const float4 q = *reinterpret_cast<const float4*>(xr + 4 * p);
-      *reinterpret_cast<float4*>(yr + 4 * p) =
-          make_float4(fast_exp(q.x - m) * inv, fast_exp(q.y - m) * inv, fast_exp(q.z - m) * inv, fast_exp(q.w - m) * inv);
+      __builtin_nontemporal_store(v4f{fast_exp(q.x - m) * inv, fast_exp(q.y - m) * inv, fast_exp(q.z - m) * inv, fast_exp(q.w - m) * inv},
+                                  reinterpret_cast<v4f*>(yr + 4 * p));
     } else {
-      yr[p] = fast_exp(xr[p] - m) * inv;
+      __builtin_nontemporal_store(fast_exp(xr[p] - m) * inv, yr + p);
     }
   }
 }

@@ -138,8 +138,8 @@ __global__ __launch_bounds__(64 * WAVES) void windowed_attn_kernel(const float* 
   for (int n = 0; n < NP; ++n) {
     const int pc = sub + LPT * n;
     if (pc < D4)
-      *reinterpret_cast<float4*>(O + (size_t)tok * D + 4 * pc) =
-          make_float4(acc[n].x * inv, acc[n].y * inv, acc[n].z * inv, acc[n].w * inv);
+      __builtin_nontemporal_store(v4f{acc[n].x * inv, acc[n].y * inv, acc[n].z * inv, acc[n].w * inv},
+                                  reinterpret_cast<v4f*>(O + (size_t)tok * D + 4 * pc));   // streaming store: written once, not read again
   }
 }
 
