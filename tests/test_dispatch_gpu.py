@@ -22,11 +22,13 @@ dispatch = ops.dispatch
 
 @pytest.fixture(autouse=True)
 def fresh_dispatch():
+    before = (dispatch.enabled, dispatch.allow_half_attention)
     dispatch.reset()
     dispatch.enabled = True
     dispatch.allow_half_attention = False
     yield
     dispatch.reset()
+    dispatch.enabled, dispatch.allow_half_attention = before
 
 
 def _np_params(Wss, Uss, bss):
