@@ -25,6 +25,13 @@ eager loop it always was: that is the reference's execution model on torch's
 GPU operators, not a substitute for a missing kernel.  A routed call needs
 libftkernels.so; if it is missing the import error surfaces.
 
+`(a @ b) @ c` is routed differently, since operators are eager and nothing can
+be looked at when `a @ b` runs: on fp16 GPU tensors of shapes the back-to-back
+GEMM kernels take, `a @ b` is left pending (kaleido.Tensor.pending_product) and
+a following `@ c` runs the fused kernel on (a, b, c); any other use of the
+product forms it with torch, as before.  The arithmetic is that of the two fp16
+GEMMs (the intermediate rounded to fp16, fp32 accumulation).
+
   enabled                   False (or FTK_DISPATCH=0 in the environment) switches routing off
   allow_half_attention      route fp32 attention programs to the fp16 kernel too (off: a
                             routed program never computes in less than its own precision)
@@ -44,7 +51,7 @@ from ..tensor import Tensor
 
 enabled = os.environ.get('FTK_DISPATCH', '1') != '0'
 allow_half_attention = False
-stats = {'stacked_lstm': 0, 'dilated_lstm': 0, 'flash_attention': 0, 'probes': 0, 'declined': 0}
+stats = {'stacked_lstm': 0, 'dilated_lstm': 0, 'flash_attention': 0, 'b2b_gemm': 0, 'probes': 0, 'declined': 0}
 
 _verdicts: dict = {}
 _MAX_VERDICTS = 256
@@ -357,3 +364,36 @@ def try_map(func: Callable, xs, kwargs):
     O = core.flash_attention(to4(q).half().contiguous(), to4(k).half().contiguous(), to4(v).half().contiguous(), verdict['scale'])
     stats['flash_attention'] += 1
     return FractalTensor.from_dense(O.to(q.dtype).view(B, Hd, nq, rq, D), 3)
+
+
+# ------------------------------------------------------------------ (a @ b) @ c behind Tensor.__matmul__
+
+def _b2b_candidate(t: torch.Tensor) -> bool:
+    return t is not None and t.is_cuda and t.dtype == torch.float16 and t.dim() == 2 and t.is_contiguous()
+
+
+def try_mm(x, y):
+    """x @ y: the fused back-to-back GEMM when x is a pending a @ b, a pending product when x @ y could be the
+    first half of one, NotImplemented otherwise."""
+    if not enabled or _probing() or not isinstance(x, Tensor) or not isinstance(y, Tensor):
+        return NotImplemented
+    c = y._payload if y._pending is None else None
+    if x._pending is not None:
+        a, b = x._pending
+        if c is None or not _b2b_candidate(c) or c.shape[0] != b.shape[1] or c.shape[1] % 32:
+            return NotImplemented                       # mm goes on with torch and forms the pending product on the way
+        core = _core()
+        K, N, P = a.shape[1], b.shape[1], c.shape[1]
+        if core.b2b_gemm_rowmajor_supported(N, K, P):   # b and c as they are
+            D = core.b2b_gemm_rowmajor(a[None], b[None], c[None])[0]
+        else:                                           # the general kernels take b and c with the contraction index contiguous
+            D = core.b2b_gemm(a[None], b.t().contiguous()[None], c.t().contiguous()[None])[0]
+        stats['b2b_gemm'] += 1
+        return Tensor.from_tensor(D)
+    a = x._payload
+    b = c
+    if not (_b2b_candidate(a) and _b2b_candidate(b)) or a.shape[1] != b.shape[0]:
+        return NotImplemented
+    if a.shape[1] not in (32, 64, 96, 128) or b.shape[1] % 32 or a.shape[0] < 32:
+        return NotImplemented                           # not a first product the fused kernels take
+    return Tensor.pending_product(a, b)

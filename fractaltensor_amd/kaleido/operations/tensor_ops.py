@@ -19,6 +19,7 @@ import torch
 
 from ..tensor import Tensor
 from ..types import (float32, int32, internal_type_to_torch_type, normalize_device, str_to_internal_type)
+from . import dispatch
 from ._base import require_same_device, require_same_shape, require_tensor, wrap
 
 __all__ = [
@@ -83,6 +84,9 @@ def cross_entropy(x, y):
 # ---- contractions and broadcasts ------------------------------------------------
 
 def mm(x, y):
+    routed = dispatch.try_mm(x, y)       # (a @ b) @ c on fp16 GPU tensors: one back-to-back GEMM
+    if routed is not NotImplemented:
+        return routed
     require_tensor(x, 'x'); require_tensor(y, 'y')
     require_same_device(x, y)
     if x.ndim != 2 or y.ndim != 2 or x.shape[1] != y.shape[0]:

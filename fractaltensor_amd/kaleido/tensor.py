@@ -30,7 +30,30 @@ class Tensor:
     def __init__(self, shape: Sequence[int], dtype: Number, order: Optional[str] = None, device: Optional[str] = None,
                  strides: Optional[Sequence[int]] = None):
         self._type = TensorStorage(shape, dtype, device=device, order=order, strides=strides)
-        self._T: Optional[torch.Tensor] = None
+        self._payload: Optional[torch.Tensor] = None
+        # (a, b): this tensor is a @ b, not formed yet.  The operator dispatch leaves an fp16 product on the GPU
+        # pending so that a following `@ c` can run as one back-to-back GEMM; any other use forms it with torch.
+        self._pending = None
+
+    @property
+    def _T(self) -> Optional[torch.Tensor]:
+        if self._pending is not None:
+            a, b = self._pending
+            self._pending = None
+            self._payload = torch.matmul(a, b)
+        return self._payload
+
+    @_T.setter
+    def _T(self, v: Optional[torch.Tensor]):
+        self._pending = None
+        self._payload = v
+
+    @staticmethod
+    def pending_product(a: torch.Tensor, b: torch.Tensor) -> 'Tensor':
+        """a @ b, formed on first use."""
+        t = Tensor((a.shape[0], b.shape[1]), torch_type_to_internal_type(a.dtype), device=a.device.type)
+        t._pending = (a, b)
+        return t
 
     def __class_getitem__(cls, item):
         return _Annotation(cls, item)
@@ -38,7 +61,9 @@ class Tensor:
     # ---- meta -----------------------------------------------------------
     @property
     def shape(self) -> Tuple[int, ...]:
-        return tuple(self._T.shape) if self._T is not None else tuple(self._type.shape)
+        if self._pending is not None:
+            return (self._pending[0].shape[0], self._pending[1].shape[1])
+        return tuple(self._payload.shape) if self._payload is not None else tuple(self._type.shape)
 
     @property
     def ndim(self) -> int:
@@ -65,16 +90,18 @@ class Tensor:
 
     @property
     def dtype(self) -> Number:
-        if self._T is not None:
+        ref = self._pending[0] if self._pending is not None else self._payload
+        if ref is not None:
             try:
-                return torch_type_to_internal_type(self._T.dtype)
+                return torch_type_to_internal_type(ref.dtype)
             except NotImplementedError:
                 pass
         return self._type.dtype
 
     @property
     def device(self) -> str:
-        return normalize_device(self._T.device.type) if self._T is not None else self._type.device
+        ref = self._pending[0] if self._pending is not None else self._payload
+        return normalize_device(ref.device.type) if ref is not None else self._type.device
 
     def size(self, n: int) -> int:
         return self.shape[n]

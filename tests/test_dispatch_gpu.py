@@ -292,3 +292,48 @@ def test_fp32_attention_program_is_not_lowered_to_fp16_unless_allowed():
     routed = programs.flash_attention(qsss, ksss, vsss, D ** -0.5)
     assert dispatch.stats['flash_attention'] == 1 and routed.data.dtype == torch.float32
     assert ko.max_rel_err(routed.data.cpu().numpy(), eager.data.cpu().numpy()) <= 1e-2
+
+
+# ---- (a @ b) @ c -----------------------------------------------------------------------------------------------------
+
+@pytest.mark.parametrize('M,K,N,P', [
+    (4096, 128, 128, 128),     # one problem of BASELINE configs[1]: b and c go down row-major as they are
+    (8192, 64, 256, 64),       # a shape of the reference's own benchmark: the wide-N kernel
+    (200, 96, 64, 160),        # ragged rows, the general kernel
+])
+def test_chained_matmul_runs_as_one_back_to_back_gemm(M, K, N, P):
+    core = _core()
+    rng = np.random.default_rng(50)
+    a, b, c = ((rng.standard_normal(s) / np.sqrt(s[0])).astype(np.float16) for s in ((M, K), (K, N), (N, P)))
+    a[:] = (rng.standard_normal((M, K)) / np.sqrt(K)).astype(np.float16)
+    ta, tb, tc = (Tensor.from_tensor(torch.from_numpy(x).cuda()) for x in (a, b, c))
+    before = core.launch_counts.get('b2b_gemm', 0) + core.launch_counts.get('b2b_gemm_rowmajor', 0)
+    d = (ta @ tb) @ tc
+    assert dispatch.stats['b2b_gemm'] == 1
+    assert core.launch_counts.get('b2b_gemm', 0) + core.launch_counts.get('b2b_gemm_rowmajor', 0) == before + 1
+    assert d.shape == (M, P) and d.data.dtype == torch.float16
+    ref = ko.b2b_gemm(a, np.ascontiguousarray(b.T), np.ascontiguousarray(c.T))
+    assert ko.max_rel_err(d.data.float().cpu().numpy(), ref) <= 1e-2
+    dispatch.enabled = False
+    eager = (ta @ tb) @ tc
+    assert ko.max_rel_err(d.data.float().cpu().numpy(), eager.data.float().cpu().numpy()) <= 1e-2
+
+
+def test_a_pending_product_is_formed_by_any_other_use():
+    rng = np.random.default_rng(51)
+    a, b = (torch.from_numpy((rng.standard_normal(s) / 8).astype(np.float16)).cuda() for s in ((64, 64), (64, 96)))
+    p = Tensor.from_tensor(a) @ Tensor.from_tensor(b)
+    assert p._pending is not None and p.shape == (64, 96) and p.device == 'cuda'       # nothing has run yet
+    s = p + p                                                                           # a use: the product is formed by torch
+    assert p._pending is None and torch.equal(p.data, a @ b) and torch.equal(s.data, (a @ b) * 2)
+    # products the fused kernels do not take are never left pending: fp32 operands, a transposed view, a single row
+    q = Tensor.from_tensor(a.float()) @ Tensor.from_tensor(b.float())
+    assert q._pending is None
+    q = Tensor.from_tensor(a) @ Tensor.from_tensor(a).T
+    assert q._pending is None and torch.equal(q.data, a @ a.t())
+    q = Tensor.from_tensor(a[:1].contiguous()) @ Tensor.from_tensor(b)
+    assert q._pending is None
+    # a second factor the kernels do not take: the chain falls back to two torch products
+    c = torch.from_numpy((rng.standard_normal((96, 40)) / 8).astype(np.float16)).cuda()
+    d = (Tensor.from_tensor(a) @ Tensor.from_tensor(b)) @ Tensor.from_tensor(c)
+    assert dispatch.stats['b2b_gemm'] == 0 and torch.equal(d.data, (a @ b) @ c)
