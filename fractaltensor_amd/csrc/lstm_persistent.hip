@@ -48,6 +48,7 @@
 
 #include "ftk_common.h"
 
+
 namespace ftk {
 
 int run_wavefront(const float* xs, const float* WU, const float* bias, const int* dil, float* hsss, float* csss,
@@ -757,11 +758,16 @@ void lstm_persistent_kernel(PersistArgs a) {
     bool pending2 = alive && n + 2 < n_items;  // tile n+2 still to be requested
     Flags fl2{0, 0};
     if (pending2) fl2 = request_flags(n + 2);
+    // Split products: item n-1 is counted here, before the activations.  Its stores left an MFMA phase and a look
+    // ago (about 2 us: acknowledged by now), and the layer above gets the count 1 us earlier than after the
+    // activations; straight after the MFMAs the acknowledgements are still on their way and the wave stalls.
+    if (MODE == kProductsSplit && !counted) { publish(n - 1); counted = true; }
     if (tracing) a.trace[TS * n + 3] = wall_clock64() | ((long long)(pending ? 7 : min(looks, 6)) << 60);
     if (on) epilogue_to_lds(gate_sums(), cp, buf);
     if (tracing) a.trace[TS * n + 4] = wall_clock64();
     if (!counted) publish(n - 1);
     else __builtin_amdgcn_s_waitcnt(0);
+    look(8);   // the counts asked for after the MFMAs have arrived with everything else: one more chance before the slow path
     barrier();
     if (tracing) a.trace[TS * n + 5] = wall_clock64();
     store_item(n, buf);
