@@ -539,7 +539,7 @@ static int launch_b2b8(const void* A, const void* B, const void* C, void* D, int
   return check_launch("b2b_gemm8_kernel");
 }
 
-// Wide-N form for the shapes of the reference's own benchmark, [M, 64] x [64, 256 | 512] x [., 64]
+// Wide-N form (N = 256 or 512, K and P 64 or 128), built for the shapes of the reference's own benchmark, [M, 64] x [64, 256 | 512] x [., 64]
 // (benchmarks/fused_two_hgemms/fractaltensor/fused_two_hgemms.cu:152-175): one problem, few bytes (2 to 4.5 MB that
 // stay in the caches), so what counts is the length of the dependency chain and how many cache lines a workgroup
 // touches.  The WAVES waves of a workgroup split N: wave w forms the 32*NTW columns [n0, n0 + 32 NTW) of P for a
@@ -824,10 +824,20 @@ extern "C" int ftk_b2b_gemm_f16(const void* A, const void* B, const void* C, voi
   // wide N with few columns of D (the reference benchmark's shapes): N split over the waves of a workgroup.
   // FTK_B2B_WIDE=0 keeps them on the general kernel.
   static const bool allow_wide = !(getenv("FTK_B2B_WIDE") && atoi(getenv("FTK_B2B_WIDE")) == 0);
-  if (allow_wide && K == 64 && P == 64 && (N == 256 || N == 512)) {
+  if (allow_wide && (K == 64 || K == 128) && (P == 64 || P == 128) && (N == 256 || N == 512)) {
     bool handled = false;
-    rc = N == 256 ? launch_b2b_wide<4, 2, 1, 8>(A, B, C, D, G, M, dp->cus, dp->lds_optin, &handled, s)
-                  : launch_b2b_wide<4, 2, 2, 8>(A, B, C, D, G, M, dp->cus, dp->lds_optin, &handled, s);
+    const int cus = dp->cus, lds = dp->lds_optin;
+    const int sel = (K == 128) * 4 + (P == 128) * 2 + (N == 512);
+    switch (sel) {
+      case 0: rc = launch_b2b_wide<4, 2, 1, 8>(A, B, C, D, G, M, cus, lds, &handled, s); break;
+      case 1: rc = launch_b2b_wide<4, 2, 2, 8>(A, B, C, D, G, M, cus, lds, &handled, s); break;
+      case 2: rc = launch_b2b_wide<4, 4, 1, 8>(A, B, C, D, G, M, cus, lds, &handled, s); break;
+      case 3: rc = launch_b2b_wide<4, 4, 2, 8>(A, B, C, D, G, M, cus, lds, &handled, s); break;
+      case 4: rc = launch_b2b_wide<8, 2, 1, 8>(A, B, C, D, G, M, cus, lds, &handled, s); break;
+      case 5: rc = launch_b2b_wide<8, 2, 2, 8>(A, B, C, D, G, M, cus, lds, &handled, s); break;
+      case 6: rc = launch_b2b_wide<8, 4, 1, 8>(A, B, C, D, G, M, cus, lds, &handled, s); break;
+      default: rc = launch_b2b_wide<8, 4, 2, 8>(A, B, C, D, G, M, cus, lds, &handled, s); break;
+    }
     if (rc || handled) return rc;
   }
   switch (K) {

@@ -638,7 +638,13 @@ def test_b2b_gemm_rowmajor_rejects_other_shapes(core):
     (1, 16384, 512, 64, 64),
     (3, 77, 512, 64, 64),       # wide-N kernel: several problems, ragged rows
     (2, 1, 256, 64, 64),        # wide-N kernel: a single row
-    (1, 1024, 256, 64, 128),    # wide N with 128 columns of D: the general kernel
+    (1, 1024, 256, 64, 128),    # the wide-N kernel at every K, P in {64, 128} x N in {256, 512}
+    (2, 100, 512, 64, 128),
+    (1, 333, 256, 128, 64),
+    (1, 2048, 512, 128, 64),
+    (2, 500, 256, 128, 128),
+    (1, 4096, 512, 128, 128),   # largest operands of the family: B and C of 128 KB each pass through LDS
+    (1, 512, 384, 64, 64),      # N between the wide kernel's sizes: the general kernel
     (2, 300, 64, 64, 128),      # eight-wave kernel (N, K in {64, 128}, full 128-column tiles), ragged M
     (2, 1000, 128, 64, 256),    # eight-wave kernel, two column tiles, units that do not divide evenly
     (1, 4100, 128, 128, 160),   # eight-wave kernel for the first 128 columns, four-wave kernel for the last 32
