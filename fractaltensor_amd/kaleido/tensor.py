@@ -50,7 +50,8 @@ class Tensor:
 
     @staticmethod
     def pending_product(a: torch.Tensor, b: torch.Tensor) -> 'Tensor':
-        """a @ b, formed on first use."""
+        """a @ b, formed on first use (of .data or anything that needs the payload).  a and b are kept by reference:
+        writing into them before that use changes the product, as it would change any view."""
         t = Tensor((a.shape[0], b.shape[1]), torch_type_to_internal_type(a.dtype), device=a.device.type)
         t._pending = (a, b)
         return t

@@ -66,3 +66,21 @@ def test_dilations_are_noted_only_under_a_probe():
             dispatch.note_dilation(2)
         assert q.dilations == [2]
     assert p.dilations == [4] and not dispatch._probing()
+
+
+def test_a_pending_product_knows_its_type_and_is_formed_on_first_use():
+    from kaleido import Tensor, FractalTensor
+    a, b = torch.arange(12.).reshape(3, 4), torch.arange(8.).reshape(4, 2)
+    p = Tensor.pending_product(a, b)
+    assert p._pending is not None and p.shape == (3, 2) and p.ndim == 2 and p.device == 'cpu' and p.numel == 6
+    assert p._pending is not None                                   # the questions above did not form it
+    assert torch.equal(p.data, a @ b) and p._pending is None
+    q = Tensor.pending_product(a, b)
+    ft = FractalTensor.from_tensors(q, q)                            # any use of the payload forms it
+    assert torch.equal(ft.as_dense()[1], a @ b)
+    r = Tensor.pending_product(a, b)
+    r.data = torch.zeros(3, 2)                                       # assigning a payload drops the pending product
+    assert r._pending is None and float(r.data.sum()) == 0.0
+    # host tensors are never left pending by the operators
+    x = Tensor.from_tensor(a) @ Tensor.from_tensor(b)
+    assert x._pending is None and torch.equal(x.data, a @ b)
