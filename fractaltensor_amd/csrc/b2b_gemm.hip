@@ -286,6 +286,10 @@ __global__ __launch_bounds__(512) void b2b_gemm8_kernel(const _Float16* __restri
   constexpr int CRS = 32 * PT + 32;  // ROWMAJOR: Cs[n][p] row
   using lds_v4s = __attribute__((address_space(3))) v4s;
   constexpr int AN = KS;       // 16-byte A loads per lane for 32 rows
+#ifndef FTK_B2B_LA
+#define FTK_B2B_LA 4
+#endif
+  constexpr int LA = FTK_B2B_LA;  // LDS fragments requested ahead of the MFMA that uses them
   constexpr int pw = 32 * PT;  // p columns handled here
   constexpr int PG = (PT + 1) / 2;  // column groups of up to 64
   constexpr int DLD = 64 + 4;  // padded D staging row (halfs)
@@ -418,22 +422,30 @@ __global__ __launch_bounds__(512) void b2b_gemm8_kernel(const _Float16* __restri
       // ROWMAJOR: the lane's block of the transposing read: rows k = hh*K/2 + 8s + (a | a + 4), columns 4b.. of
       // the 16-column half th of the n tile
       const _Float16* btr = Bs + (hh * (K / 2) + ((lane & 15) >> 2)) * BRS + 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
-#pragma unroll
-      for (int s = 0; s < KS; ++s)
-#pragma unroll
-        for (int nt = 0; nt < NT; ++nt) {
-          v8h bfrag;
-          if constexpr (ROWMAJOR) {
-            const _Float16* p0 = btr + 8 * s * BRS + 32 * nt;
-            const v4s lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4s*)(p0));
-            const v4s hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4s*)(p0 + 4 * BRS));
-            const v8s both = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
-            bfrag = __builtin_bit_cast(v8h, both);
-          } else {
-            bfrag = *reinterpret_cast<const v8h*>(brow + nt * 32 * BLD + 8 * s);
-          }
-          pacc[nt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(bfrag, afrag[s], pacc[nt], 0, 0, 0);
+      // The fragment of product i + LA is requested before product i is issued: a wave that is alone on its SIMD
+      // (the first and the last unit of a workgroup's schedule) otherwise waits out the LDS latency before every MFMA.
+      constexpr int NI = KS * NT;
+      auto read_b = [&](auto ic) __attribute__((always_inline)) {
+        constexpr int i = decltype(ic)::value;
+        constexpr int s = i / NT, nt = i % NT;
+        if constexpr (ROWMAJOR) {
+          const _Float16* p0 = btr + 8 * s * BRS + 32 * nt;
+          const v4s lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4s*)(p0));
+          const v4s hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4s*)(p0 + 4 * BRS));
+          const v8s both = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+          return __builtin_bit_cast(v8h, both);
+        } else {
+          return *reinterpret_cast<const v8h*>(brow + nt * 32 * BLD + 8 * s);
         }
+      };
+      v8h bf[NI];
+      static_for<(LA < NI ? LA : NI)>([&](auto ic) __attribute__((always_inline)) { bf[decltype(ic)::value] = read_b(ic); });
+      static_for<NI>([&](auto ic) __attribute__((always_inline)) {
+        constexpr int i = decltype(ic)::value;
+        if constexpr (i + LA < NI) bf[i + LA] = read_b(std::integral_constant<int, i + LA>{});
+        pacc[i % NT] = __builtin_amdgcn_mfma_f32_32x32x16_f16(bf[i], afrag[i / NT], pacc[i % NT], 0, 0, 0);
+        __builtin_amdgcn_sched_barrier(0);
+      });
 #pragma unroll
       for (int nt = 0; nt < NT; ++nt)
 #pragma unroll
@@ -451,30 +463,33 @@ __global__ __launch_bounds__(512) void b2b_gemm8_kernel(const _Float16* __restri
       for (int q = 0; q < PW; ++q)
 #pragma unroll
         for (int r = 0; r < 16; ++r) dacc[q][r] = 0.0f;
-      static_for<NT>([&](auto ntc) __attribute__((always_inline)) {
-        constexpr int nt = decltype(ntc)::value;
-#pragma unroll
-        for (int q = 0; q < PW; ++q) {
-          const _Float16* crow = Cs + ((2 * pg + q) * 32 + j) * CLD + nt * 32 + 4 * hh;
-          // ROWMAJOR: rows n = 32 nt + 16 s + 4 hh + a (and + 8), columns of p tile 2 pg + q
+      constexpr int NI = NT * PW * 2;
+      auto read_c = [&](auto ic) __attribute__((always_inline)) {
+        constexpr int i = decltype(ic)::value;
+        constexpr int nt = i / (PW * 2), q = (i / 2) % PW, s = i % 2;
+        if constexpr (ROWMAJOR) {
+          // rows n = 32 nt + 16 s + 4 hh + a (and + 8), columns of p tile 2 pg + q
           const _Float16* ctr = Cs + (nt * 32 + 4 * hh + ((lane & 15) >> 2)) * CRS + (2 * pg + q) * 32 +
                                 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
-#pragma unroll
-          for (int s = 0; s < 2; ++s) {
-            v8h cfrag;
-            if constexpr (ROWMAJOR) {
-              const v4s lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4s*)(ctr + 16 * s * CRS));
-              const v4s hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4s*)(ctr + (16 * s + 8) * CRS));
-              const v8s both = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
-              cfrag = __builtin_bit_cast(v8h, both);
-            } else {
-              const v4h c0 = *reinterpret_cast<const v4h*>(crow + 16 * s);
-              const v4h c1 = *reinterpret_cast<const v4h*>(crow + 16 * s + 8);
-              cfrag = v8h{c0[0], c0[1], c0[2], c0[3], c1[0], c1[1], c1[2], c1[3]};
-            }
-            dacc[q] = __builtin_amdgcn_mfma_f32_32x32x16_f16(cfrag, pf[nt][s], dacc[q], 0, 0, 0);
-          }
+          const v4s lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4s*)(ctr + 16 * s * CRS));
+          const v4s hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4s*)(ctr + (16 * s + 8) * CRS));
+          const v8s both = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+          return __builtin_bit_cast(v8h, both);
+        } else {
+          const _Float16* crow = Cs + ((2 * pg + q) * 32 + j) * CLD + nt * 32 + 4 * hh;
+          const v4h c0 = *reinterpret_cast<const v4h*>(crow + 16 * s);
+          const v4h c1 = *reinterpret_cast<const v4h*>(crow + 16 * s + 8);
+          return v8h{c0[0], c0[1], c0[2], c0[3], c1[0], c1[1], c1[2], c1[3]};
         }
+      };
+      v8h cf[NI];
+      static_for<(LA < NI ? LA : NI)>([&](auto ic) __attribute__((always_inline)) { cf[decltype(ic)::value] = read_c(ic); });
+      static_for<NI>([&](auto ic) __attribute__((always_inline)) {
+        constexpr int i = decltype(ic)::value;
+        constexpr int nt = i / (PW * 2), q = (i / 2) % PW, s = i % 2;
+        if constexpr (i + LA < NI) cf[i + LA] = read_c(std::integral_constant<int, i + LA>{});
+        dacc[q] = __builtin_amdgcn_mfma_f32_32x32x16_f16(cf[i], pf[nt][s], dacc[q], 0, 0, 0);
+        __builtin_amdgcn_sched_barrier(0);
       });
       // D^T accumulators -> wave-private LDS [row][p] -> 16-byte row segments.
       // A wave reads back only what it wrote itself and LDS operations of one
