@@ -208,6 +208,11 @@ void lstm_persistent_kernel(PersistArgs a) {
   const int wave = tid >> 6;
   const int j = lane & 31;
   const int hh = lane >> 5;
+  // the batch row (within a 32-row block) whose activations this lane feeds to the MFMAs and whose results it
+  // gets back.  With two batch rows per tile row, lanes 0..15 take the first of each pair and lanes 16..31 the
+  // second: the 16 lanes of one pass of a fragment read then touch 16 different tile rows (16 bytes apart in the
+  // bank line), where lanes 2r / 2r+1 on one tile row, 512 bytes apart, hit the same banks.
+  const int jb = MODE == kHalfData256 ? 2 * (j & 15) + (j >> 4) : j;
 
   int q = blockIdx.x;
   if (a.xcd_remap) q = (blockIdx.x & 7) * (gridDim.x >> 3) + (blockIdx.x >> 3);
@@ -468,7 +473,7 @@ void lstm_persistent_kernel(PersistArgs a) {
     constexpr int q0 = decltype(q0c)::value;
     constexpr int q1 = decltype(q1c)::value;
     constexpr int SH = HID / 16;  // steps per half
-    const _Float16* arow = PAIR ? reinterpret_cast<const _Float16*>(tile + buf * P_TILE + (j >> 1) * P_LD) + (j & 1) * HID + 8 * hh
+    const _Float16* arow = PAIR ? reinterpret_cast<const _Float16*>(tile + buf * P_TILE + (jb >> 1) * P_LD) + (jb & 1) * HID + 8 * hh
                                 : reinterpret_cast<const _Float16*>(tile + buf * P_TILE + j * P_LD) + 8 * hh;
     auto frag = [&](int qq) { return *reinterpret_cast<const v8h*>(arow + (qq / SH) * 512 + 16 * (qq % SH)); };
     v8h b0 = frag(q0), b1 = frag(q0 + 1);
@@ -563,8 +568,8 @@ void lstm_persistent_kernel(PersistArgs a) {
     if constexpr (F16) {  // h and c leave as fp16: the two 16-bit staging planes hold them
       const v4h h16 = {(_Float16)hv[0], (_Float16)hv[1], (_Float16)hv[2], (_Float16)hv[3]};
       const v4h c16 = {(_Float16)cv[0], (_Float16)cv[1], (_Float16)cv[2], (_Float16)cv[3]};
-      *reinterpret_cast<v4h*>(sb + kStageTop + j * kStageRow16 + 2 * c4) = h16;
-      *reinterpret_cast<v4h*>(sb + kStageRest + j * kStageRow16 + 2 * c4) = c16;
+      *reinterpret_cast<v4h*>(sb + kStageTop + jb * kStageRow16 + 2 * c4) = h16;
+      *reinterpret_cast<v4h*>(sb + kStageRest + jb * kStageRow16 + 2 * c4) = c16;
       return;
     }
     *reinterpret_cast<float4*>(sb + kStageC + j * kStageRow32 + 4 * c4) = make_float4(cv[0], cv[1], cv[2], cv[3]);
@@ -625,7 +630,7 @@ void lstm_persistent_kernel(PersistArgs a) {
     const int t = item_t(n), rb = item_rb(n);
     float4 cp = make_float4(0.f, 0.f, 0.f, 0.f);
     if (alive && t >= d && live(n)) {
-      const int rgc = min(rb * 32 + j, B - 1);
+      const int rgc = min(rb * 32 + jb, B - 1);
       if constexpr (F16) {
         const v4h c16 = *reinterpret_cast<const v4h*>(reinterpret_cast<const _Float16*>(a.csss) +
                                                       (((size_t)l * T + (t - d)) * B + rgc) * HID + u0);
