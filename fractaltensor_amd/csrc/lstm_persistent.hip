@@ -281,18 +281,19 @@ void lstm_persistent_kernel(PersistArgs a) {
     for (int r = 0; r < 16; ++r) ginv[r] = __shfl(winv, (r & 3) + 8 * (r >> 2) + 4 * hh) * (1.0f / kSplitAct);
   }
   const int u0 = 32 * pc + 8 * wave + 4 * hh;  // first of this lane's 4 units
-  float bi[4] = {0, 0, 0, 0}, bf[4] = {0, 0, 0, 0}, bo[4] = {0, 0, 0, 0}, bg[4] = {0, 0, 0, 0};
-  if (a.bias) {
-    const float* bl = a.bias + (size_t)l * NG;
+  // The activations are exponentials of scaled sums: sigmoid(v) = 1 / (1 + 2^(-v log2 e)), tanh(v) = 1 - 2 / (1 + 2^(2 v
+  // log2 e)).  The scale of accumulator register r (gate r / 4 of unit r % 4: -log2 e for i, f, o and 2 log2 e for the
+  // candidate) is folded into what the register is multiplied by anyway (split products) and into the bias, so the
+  // argument of the exponential is one multiply-add away from the accumulators.
+  constexpr float kLog2e = 1.4426950408889634f;
+  float esc[SPLIT ? 16 : 1], ebias[16];
 #pragma unroll
-    for (int r = 0; r < 4; ++r) {
-      bi[r] = bl[u0 + r];
-      bf[r] = bl[HID + u0 + r];
-      bo[r] = bl[2 * HID + u0 + r];
-      bg[r] = bl[3 * HID + u0 + r];
-    }
+  for (int r = 0; r < 16; ++r) {
+    const float k = (r >> 2) == 3 ? 2.0f * kLog2e : -kLog2e;
+    if constexpr (SPLIT) esc[r] = ginv[r] * k;
+    ebias[r] = 0.0f;
+    if (a.bias) ebias[r] = a.bias[(size_t)l * NG + (r >> 2) * HID + u0 + (r & 3)] * k;
   }
-
   bool alive = true;
   if (q == a.trace_q && tid == 0) {
     long long* st = reinterpret_cast<long long*>(a.status + 16);
@@ -421,17 +422,22 @@ void lstm_persistent_kernel(PersistArgs a) {
   // steps [q0, q1) of the K loop (steps 0..31: x rows of WU, 32..63: h rows)
   // into two accumulators so that consecutive MFMAs never wait on each other's
   // result; the LDS read for step q+1 is issued before the MFMAs of step q
-  auto mfma_part = [&](int buf, auto q0c, auto q1c, v16f& acc0, v16f& acc1) __attribute__((always_inline)) {
+  // first_c (here and below): these are an item's first products, the accumulators start from zero -- as the
+  // matrix instruction's constant addend, which costs nothing, where clearing 48 accumulator registers costs 48
+  // vector instructions per item
+  const v16f zero16 = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+  auto mfma_part = [&](int buf, auto q0c, auto q1c, auto first_c, v16f& acc0, v16f& acc1) __attribute__((always_inline)) {
     constexpr int q0 = decltype(q0c)::value;
     constexpr int q1 = decltype(q1c)::value;
+    constexpr bool first = decltype(first_c)::value;
     const float* arow = tile + buf * P_TILE + j * P_LD + 4 * hh;
     v4f b = *reinterpret_cast<const v4f*>(arow + 8 * q0);
 #pragma unroll
     for (int qq = q0; qq < q1; ++qq) {
       v4f bn = b;
       if (qq + 1 < q1) bn = *reinterpret_cast<const v4f*>(arow + 8 * (qq + 1));
-      acc0 = __builtin_amdgcn_mfma_f32_32x32x2f32(wr[4 * qq + 0], b[0], acc0, 0, 0, 0);
-      acc1 = __builtin_amdgcn_mfma_f32_32x32x2f32(wr[4 * qq + 1], b[1], acc1, 0, 0, 0);
+      acc0 = __builtin_amdgcn_mfma_f32_32x32x2f32(wr[4 * qq + 0], b[0], first && qq == q0 ? zero16 : acc0, 0, 0, 0);
+      acc1 = __builtin_amdgcn_mfma_f32_32x32x2f32(wr[4 * qq + 1], b[1], first && qq == q0 ? zero16 : acc1, 0, 0, 0);
       acc0 = __builtin_amdgcn_mfma_f32_32x32x2f32(wr[4 * qq + 2], b[2], acc0, 0, 0, 0);
       acc1 = __builtin_amdgcn_mfma_f32_32x32x2f32(wr[4 * qq + 3], b[3], acc1, 0, 0, 0);
       b = bn;
@@ -445,9 +451,10 @@ void lstm_persistent_kernel(PersistArgs a) {
   };
   // the same in split mode: steps 0..15 are the x rows, 16..31 the h rows; a
   // lane reads its 8 k of both planes and three MFMAs use them
-  auto mfma_split = [&](int buf, auto q0c, auto q1c, v16f& am, v16f& ar0, v16f& ar1) __attribute__((always_inline)) {
+  auto mfma_split = [&](int buf, auto q0c, auto q1c, auto first_c, v16f& am, v16f& ar) __attribute__((always_inline)) {
     constexpr int q0 = decltype(q0c)::value;
     constexpr int q1 = decltype(q1c)::value;
+    constexpr bool first = decltype(first_c)::value;
     const _Float16* arow = reinterpret_cast<const _Float16*>(tile + buf * P_TILE + j * P_LD) + 8 * hh;
     auto top_of = [&](int qq) { return *reinterpret_cast<const v8h*>(arow + (qq >> 4) * (2 * PH) + 16 * (qq & 15)); };
     auto rest_of = [&](int qq) { return *reinterpret_cast<const v8h*>(arow + (qq >> 4) * (2 * PH) + PH + 16 * (qq & 15)); };
@@ -456,9 +463,10 @@ void lstm_persistent_kernel(PersistArgs a) {
     for (int qq = q0; qq < q1; ++qq) {
       v8h btn = bt, brn = br;
       if (qq + 1 < q1) { btn = top_of(qq + 1); brn = rest_of(qq + 1); }
-      am = __builtin_amdgcn_mfma_f32_32x32x16_f16(whi[qq], bt, am, 0, 0, 0);
-      ar0 = __builtin_amdgcn_mfma_f32_32x32x16_f16(whi[qq], br, ar0, 0, 0, 0);
-      ar1 = __builtin_amdgcn_mfma_f32_32x32x16_f16(wlo[qq], bt, ar1, 0, 0, 0);
+      // top x top in one accumulator; top x rest and rest x top, both 2^-11 of a product, share the other
+      am = __builtin_amdgcn_mfma_f32_32x32x16_f16(whi[qq], bt, first && qq == q0 ? zero16 : am, 0, 0, 0);
+      ar = __builtin_amdgcn_mfma_f32_32x32x16_f16(whi[qq], br, first && qq == q0 ? zero16 : ar, 0, 0, 0);
+      ar = __builtin_amdgcn_mfma_f32_32x32x16_f16(wlo[qq], bt, ar, 0, 0, 0);
       bt = btn; br = brn;
     }
     __builtin_amdgcn_sched_group_barrier(0x100, 4, 0);
@@ -469,9 +477,10 @@ void lstm_persistent_kernel(PersistArgs a) {
     }
   };
   // fp16 data: the first HID/16 steps are the x rows, the rest the h rows; one MFMA per step, two accumulation chains
-  auto mfma_half = [&](int buf, auto q0c, auto q1c, v16f& a0, v16f& a1) __attribute__((always_inline)) {
+  auto mfma_half = [&](int buf, auto q0c, auto q1c, auto first_c, v16f& a0, v16f& a1) __attribute__((always_inline)) {
     constexpr int q0 = decltype(q0c)::value;
     constexpr int q1 = decltype(q1c)::value;
+    constexpr bool first = decltype(first_c)::value;
     constexpr int SH = HID / 16;  // steps per half
     const _Float16* arow = PAIR ? reinterpret_cast<const _Float16*>(tile + buf * P_TILE + (jb >> 1) * P_LD) + (jb & 1) * HID + 8 * hh
                                 : reinterpret_cast<const _Float16*>(tile + buf * P_TILE + j * P_LD) + 8 * hh;
@@ -481,8 +490,8 @@ void lstm_persistent_kernel(PersistArgs a) {
     for (int qq = q0; qq < q1; qq += 2) {
       v8h b0n = b0, b1n = b1;
       if (qq + 2 < q1) { b0n = frag(qq + 2); b1n = frag(qq + 3); }
-      a0 = __builtin_amdgcn_mfma_f32_32x32x16_f16(wh[F16 ? qq : 0], b0, a0, 0, 0, 0);
-      a1 = __builtin_amdgcn_mfma_f32_32x32x16_f16(wh[F16 ? qq + 1 : 0], b1, a1, 0, 0, 0);
+      a0 = __builtin_amdgcn_mfma_f32_32x32x16_f16(wh[F16 ? qq : 0], b0, first && qq == q0 ? zero16 : a0, 0, 0, 0);
+      a1 = __builtin_amdgcn_mfma_f32_32x32x16_f16(wh[F16 ? qq + 1 : 0], b1, first && qq == q0 ? zero16 : a1, 0, 0, 0);
       b0 = b0n; b1 = b1n;
     }
     __builtin_amdgcn_sched_group_barrier(0x100, 4, 0);
@@ -494,20 +503,18 @@ void lstm_persistent_kernel(PersistArgs a) {
   };
   // one interface for all: K steps of the x half [x0, x1) or of the h half, in
   // units of a sixteenth of a half
-  v16f acc0, acc1, acc2;
-  auto clear_acc = [&]() __attribute__((always_inline)) {
-#pragma unroll
-    for (int r = 0; r < 16; ++r) { acc0[r] = 0.0f; acc1[r] = 0.0f; acc2[r] = 0.0f; }
-  };
+  v16f acc0, acc1;
+  // an item without an x half to start the accumulators from zero does not exist: the x half always runs
   auto mfma_range = [&](int buf, auto half_c, auto s0c, auto s1c) __attribute__((always_inline)) {
     constexpr int hf = decltype(half_c)::value, s0 = decltype(s0c)::value, s1 = decltype(s1c)::value;
+    constexpr std::integral_constant<bool, hf == 0 && s0 == 0> first{};
     if constexpr (F16)
       mfma_half(buf, std::integral_constant<int, (HID / 16) * hf + s0 * (HID / 256)>{},
-                std::integral_constant<int, (HID / 16) * hf + s1 * (HID / 256)>{}, acc0, acc1);
+                std::integral_constant<int, (HID / 16) * hf + s1 * (HID / 256)>{}, first, acc0, acc1);
     else if constexpr (SPLIT)
-      mfma_split(buf, std::integral_constant<int, 16 * hf + s0>{}, std::integral_constant<int, 16 * hf + s1>{}, acc0, acc1, acc2);
+      mfma_split(buf, std::integral_constant<int, 16 * hf + s0>{}, std::integral_constant<int, 16 * hf + s1>{}, first, acc0, acc1);
     else
-      mfma_part(buf, std::integral_constant<int, 32 * hf + 2 * s0>{}, std::integral_constant<int, 32 * hf + 2 * s1>{}, acc0, acc1);
+      mfma_part(buf, std::integral_constant<int, 32 * hf + 2 * s0>{}, std::integral_constant<int, 32 * hf + 2 * s1>{}, first, acc0, acc1);
   };
   // split mode, first layer: the x rows carry a scale of their own; before the h
   // products join the same accumulators the x products move to h's scale (a
@@ -522,34 +529,37 @@ void lstm_persistent_kernel(PersistArgs a) {
     if constexpr (SPLIT) {
       if (l == 0) {
 #pragma unroll
-        for (int r = 0; r < 16; ++r) { acc0[r] *= ratio; acc1[r] *= ratio; acc2[r] *= ratio; }
+        for (int r = 0; r < 16; ++r) { acc0[r] *= ratio; acc1[r] *= ratio; }
       }
     }
   };
+  // the arguments of the 16 exponentials of an item (see esc / ebias)
   auto gate_sums = [&]() __attribute__((always_inline)) -> v16f {
     v16f acc;
 #pragma unroll
     for (int r = 0; r < 16; ++r) {
-      if constexpr (SPLIT) acc[r] = ginv[r] * (acc0[r] + (1.0f / kSplitRest) * (acc1[r] + acc2[r]));
-      else acc[r] = acc0[r] + acc1[r];
+      if constexpr (SPLIT) acc[r] = esc[r] * (acc0[r] + (1.0f / kSplitRest) * acc1[r]) + ebias[r];
+      else acc[r] = ((r >> 2) == 3 ? 2.0f * kLog2e : -kLog2e) * (acc0[r] + acc1[r]) + ebias[r];
     }
     return acc;
   };
-  // bias, activations and state update of an item: lane-local and branch-free.
+  // activations and state update of an item: lane-local and branch-free.
   // piece m (0..15) of the computation: gate (m & 3) of unit (m >> 2); the last
-  // gate of a unit finishes its c and h
+  // gate of a unit finishes its c and h.  tanh as 1 - 2 / (1 + e^2v) is within 1.2e-7 absolute everywhere, which is
+  // what counts for a state; the relative accuracy it loses near zero is not kept here.
   float eg_i = 0.f, eg_f = 0.f, eg_o = 0.f;
   auto epilogue_piece = [&](const v16f& acc, const float4& cp, float (&hv)[4], float (&cv)[4], auto mc) __attribute__((always_inline)) {
     constexpr int m = decltype(mc)::value;
     constexpr int r = m >> 2;
     const float cpv[4] = {cp.x, cp.y, cp.z, cp.w};
-    if constexpr ((m & 3) == 0) eg_i = sigmoid_f(acc[r] + bi[r]);
-    if constexpr ((m & 3) == 1) eg_f = sigmoid_f(acc[4 + r] + bf[r]);
-    if constexpr ((m & 3) == 2) eg_o = sigmoid_f(acc[8 + r] + bo[r]);
+    auto inv1p = [](float e) { return __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(e)); };
+    if constexpr ((m & 3) == 0) eg_i = inv1p(acc[r]);
+    if constexpr ((m & 3) == 1) eg_f = inv1p(acc[4 + r]);
+    if constexpr ((m & 3) == 2) eg_o = inv1p(acc[8 + r]);
     if constexpr ((m & 3) == 3) {
-      const float cand = tanh_f(acc[12 + r] + bg[r]);
+      const float cand = 1.0f - 2.0f * inv1p(acc[12 + r]);
       cv[r] = eg_f * cpv[r] + eg_i * cand;
-      hv[r] = eg_o * tanh_f(cv[r]);
+      hv[r] = eg_o * (1.0f - 2.0f * inv1p(cv[r] * (2.0f * kLog2e)));
     }
   };
   auto epilogue_math = [&](const v16f& acc, const float4& cp, float (&hv)[4], float (&cv)[4]) __attribute__((always_inline)) {
@@ -560,9 +570,7 @@ void lstm_persistent_kernel(PersistArgs a) {
   // units] per output, rows padded against bank conflicts), and after a barrier wave w stores rows
   // 8w..8w+7: 128 contiguous bytes of c and h per row, 64 of each fp16 plane.
   unsigned char* const stage = reinterpret_cast<unsigned char*>(tile + 2 * P_TILE + 256);
-  auto epilogue_to_lds = [&](const v16f& acc, const float4& cp, int sbuf) __attribute__((always_inline)) {
-    float hv[4], cv[4];
-    epilogue_math(acc, cp, hv, cv);
+  auto stage_results = [&](const float (&hv)[4], const float (&cv)[4], int sbuf) __attribute__((always_inline)) {
     unsigned char* sb = stage + sbuf * kStageBytes;
     const int c4 = 8 * wave + 4 * hh;
     if constexpr (F16) {  // h and c leave as fp16: the two 16-bit staging planes hold them
@@ -585,6 +593,11 @@ void lstm_persistent_kernel(PersistArgs a) {
       *reinterpret_cast<v4h*>(sb + kStageTop + j * kStageRow16 + 2 * c4) = top;
       *reinterpret_cast<v4h*>(sb + kStageRest + j * kStageRow16 + 2 * c4) = rest;
     }
+  };
+  auto epilogue_to_lds = [&](const v16f& acc, const float4& cp, int sbuf) __attribute__((always_inline)) {
+    float hv[4], cv[4];
+    epilogue_math(acc, cp, hv, cv);
+    stage_results(hv, cv, sbuf);
   };
   // What consumers on other compute units read leaves through write-through stores (fp32 products: h;
   // split products: the two planes), the rest through the cache.
@@ -666,7 +679,6 @@ void lstm_persistent_kernel(PersistArgs a) {
       __builtin_amdgcn_s_waitcnt(0);
       __syncthreads();
       if (live(n)) {
-        clear_acc();
         mfma_range(0, IC<0>{}, IC<0>{}, IC<16>{});
         rescale_x(load_ratio(n));
         if (item_t(n) >= d) mfma_range(0, IC<1>{}, IC<0>{}, IC<16>{});
@@ -736,7 +748,6 @@ void lstm_persistent_kernel(PersistArgs a) {
 
     const bool on = live(n);
     if (on) {
-      clear_acc();
       mfma_range(buf, IC<0>{}, IC<0>{}, IC<4>{});
       look(0);
       mfma_range(buf, IC<0>{}, IC<4>{}, IC<8>{});
