@@ -281,15 +281,16 @@ void lstm_persistent_kernel(PersistArgs a) {
     for (int r = 0; r < 16; ++r) ginv[r] = __shfl(winv, (r & 3) + 8 * (r >> 2) + 4 * hh) * (1.0f / kSplitAct);
   }
   const int u0 = 32 * pc + 8 * wave + 4 * hh;  // first of this lane's 4 units
-  // The activations are exponentials of scaled sums: sigmoid(v) = 1 / (1 + 2^(-v log2 e)), tanh(v) = 1 - 2 / (1 + 2^(2 v
-  // log2 e)).  The scale of accumulator register r (gate r / 4 of unit r % 4: -log2 e for i, f, o and 2 log2 e for the
-  // candidate) is folded into what the register is multiplied by anyway (split products) and into the bias, so the
-  // argument of the exponential is one multiply-add away from the accumulators.
+  // sigmoid(v) = 1 / (1 + 2^(-v log2 e)): the -log2 e of the gates i, f, o (accumulator register r holds gate r / 4
+  // of unit r % 4) is folded into what the register is multiplied by anyway (split products) and into the bias, so
+  // the argument of the exponential is one multiply-add away from the accumulators.  The candidate keeps scale 1:
+  // tanh_f needs its argument as it is (it switches to a polynomial near zero, where the exponential form loses
+  // relative accuracy; with inputs of 1e-3 the states are that small and the error would reach 1e-4 of them).
   constexpr float kLog2e = 1.4426950408889634f;
   float esc[SPLIT ? 16 : 1], ebias[16];
 #pragma unroll
   for (int r = 0; r < 16; ++r) {
-    const float k = (r >> 2) == 3 ? 2.0f * kLog2e : -kLog2e;
+    const float k = (r >> 2) == 3 ? 1.0f : -kLog2e;
     if constexpr (SPLIT) esc[r] = ginv[r] * k;
     ebias[r] = 0.0f;
     if (a.bias) ebias[r] = a.bias[(size_t)l * NG + (r >> 2) * HID + u0 + (r & 3)] * k;
@@ -533,20 +534,19 @@ void lstm_persistent_kernel(PersistArgs a) {
       }
     }
   };
-  // the arguments of the 16 exponentials of an item (see esc / ebias)
+  // the arguments of an item's 12 sigmoid exponentials and its 4 candidate sums (see esc / ebias)
   auto gate_sums = [&]() __attribute__((always_inline)) -> v16f {
     v16f acc;
 #pragma unroll
     for (int r = 0; r < 16; ++r) {
       if constexpr (SPLIT) acc[r] = esc[r] * (acc0[r] + (1.0f / kSplitRest) * acc1[r]) + ebias[r];
-      else acc[r] = ((r >> 2) == 3 ? 2.0f * kLog2e : -kLog2e) * (acc0[r] + acc1[r]) + ebias[r];
+      else acc[r] = ((r >> 2) == 3 ? 1.0f : -kLog2e) * (acc0[r] + acc1[r]) + ebias[r];
     }
     return acc;
   };
   // activations and state update of an item: lane-local and branch-free.
   // piece m (0..15) of the computation: gate (m & 3) of unit (m >> 2); the last
-  // gate of a unit finishes its c and h.  tanh as 1 - 2 / (1 + e^2v) is within 1.2e-7 absolute everywhere, which is
-  // what counts for a state; the relative accuracy it loses near zero is not kept here.
+  // gate of a unit finishes its c and h
   float eg_i = 0.f, eg_f = 0.f, eg_o = 0.f;
   auto epilogue_piece = [&](const v16f& acc, const float4& cp, float (&hv)[4], float (&cv)[4], auto mc) __attribute__((always_inline)) {
     constexpr int m = decltype(mc)::value;
@@ -557,9 +557,9 @@ void lstm_persistent_kernel(PersistArgs a) {
     if constexpr ((m & 3) == 1) eg_f = inv1p(acc[4 + r]);
     if constexpr ((m & 3) == 2) eg_o = inv1p(acc[8 + r]);
     if constexpr ((m & 3) == 3) {
-      const float cand = 1.0f - 2.0f * inv1p(acc[12 + r]);
+      const float cand = tanh_f(acc[12 + r]);
       cv[r] = eg_f * cpv[r] + eg_i * cand;
-      hv[r] = eg_o * (1.0f - 2.0f * inv1p(cv[r] * (2.0f * kLog2e)));
+      hv[r] = eg_o * tanh_f(cv[r]);
     }
   };
   auto epilogue_math = [&](const v16f& acc, const float4& cp, float (&hv)[4], float (&cv)[4]) __attribute__((always_inline)) {
@@ -771,13 +771,14 @@ void lstm_persistent_kernel(PersistArgs a) {
     }
     if (tracing) a.trace[TS * n + 2] = wall_clock64();
     look(7);
+    // Split products: item n-1 is counted here, before the activations.  Its stores left an MFMA phase and a look
+    // ago (about 2 us: acknowledged by now), and the layer above gets the count 1 us earlier than after the
+    // activations.  The counts of tile n+2 are asked for after that, not before: the wait inside publish() would
+    // otherwise sit out their latency too, which the activations hide.
+    if (MODE == kProductsSplit && !counted) { publish(n - 1); counted = true; }
     bool pending2 = alive && n + 2 < n_items;  // tile n+2 still to be requested
     Flags fl2{0, 0};
     if (pending2) fl2 = request_flags(n + 2);
-    // Split products: item n-1 is counted here, before the activations.  Its stores left an MFMA phase and a look
-    // ago (about 2 us: acknowledged by now), and the layer above gets the count 1 us earlier than after the
-    // activations; straight after the MFMAs the acknowledgements are still on their way and the wave stalls.
-    if (MODE == kProductsSplit && !counted) { publish(n - 1); counted = true; }
     if (tracing) a.trace[TS * n + 3] = wall_clock64() | ((long long)(pending ? 7 : min(looks, 6)) << 60);
     if (on) epilogue_to_lds(gate_sums(), cp, buf);
     if (tracing) a.trace[TS * n + 4] = wall_clock64();
