@@ -270,8 +270,8 @@ class FractalTensor(Sequence):
         if not xs:
             raise ValueError('from_tensors needs at least one tensor')
         for x in xs:
-            if not isinstance(x, Tensor):
-                raise TypeError('from_tensors expects kaleido Tensors.')
+            if not isinstance(x, Tensor):  # a ValueError, like the reference's (frontend/fractal_tensor.py:404-405)
+                raise ValueError(f'Expected tensor, got {type(x).__name__}.')
             if tuple(x.shape) != tuple(xs[0].shape):
                 raise ValueError('tensors in a FractalTensor must share one shape.')
         ft = FractalTensor(TensorStorage(xs[0].shape, xs[0].dtype, device=xs[0].device))

@@ -42,6 +42,15 @@ def test_from_tensors_keeps_shapes():                   # :55-70
         assert tuple(t.shape) == (3, 7, 5) and torch.equal(t.data, ts[i].data)
 
 
+def test_constructors_reject_what_the_reference_rejects():   # frontend/fractal_tensor.py:398-405, 435-455
+    with pytest.raises(ValueError):
+        FractalTensor.from_tensors()                        # "input should be a non-empty list."
+    with pytest.raises(ValueError):
+        FractalTensor.from_tensors(3)                       # "Expected tensor, got int."
+    with pytest.raises(IndexError):
+        FractalTensor.from_pylist([])                       # the reference's walk deletes from an empty list
+
+
 def test_nested_from_uninitialised_children():          # :72-106
     mk = lambda: FractalTensor(TensorStorage((3, 4), kaleido.float32, device='cpu', order='row'))
     x = FractalTensor.from_fractaltensors(mk(), mk(), mk())
