@@ -821,6 +821,94 @@ static int launch_b2b(const void* A, const void* B, const void* C, void* D, int 
   }
 }
 
+
+// General form for everything the kernels above are not built for: any K % 16 == 0 (they hold a whole A row
+// as register fragments and B with all of its k in LDS, K <= 128), N up to kStreamMaxN, B and C of any size --
+// the shapes of the reference's own test, [192, 704] x [704, 448] x [448, 832] (tests/test_b2b_gemm.cu:137-149),
+// among them.  A workgroup owns 32 rows.  Its waves share out the 32-column tiles of P = A B: a tile is one
+// accumulator, the k loop runs over the whole of K with both operands read as 16-byte pieces straight from global
+// memory (every lane its own row: 32 rows x 32 bytes per product, each cache line serves four products), and the
+// tile goes to LDS rounded to fp16, [row][n].  After a barrier the waves share out the 32-column tiles of D: the
+// rows of P are the B operand out of LDS, the rows of C the A operand from global memory.  Same transposed
+// products, same rounding of P and same lane ownership as above; built for coverage, not for speed.
+constexpr int kStreamMaxN = 2048;
+
+__global__ __launch_bounds__(256) void b2b_stream_kernel(const _Float16* __restrict__ A, const _Float16* __restrict__ Bm,
+                                                         const _Float16* __restrict__ Cm, _Float16* __restrict__ D, int M,
+                                                         int N, int K, int P, int row_blocks) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+  _Float16* const Ps = reinterpret_cast<_Float16*>(smem);  // [32][N + 8]
+  const int PLD = N + 8;
+  const int lane = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6;
+  const int j = lane & 31;
+  const int hh = lane >> 5;
+  const int g = blockIdx.x / row_blocks;
+  const int rb = blockIdx.x - g * row_blocks;
+  const int row = min(rb * 32 + j, M - 1);  // rows past the end repeat the last one and are not stored
+  const _Float16* arow = A + ((size_t)g * M + row) * K + 8 * hh;
+  for (int nt = wave; nt < N / 32; nt += 4) {
+    const _Float16* brow = Bm + ((size_t)g * N + nt * 32 + j) * K + 8 * hh;
+    v16f acc;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) acc[r] = 0.0f;
+#pragma unroll 4
+    for (int k = 0; k < K; k += 16) {
+      const v8h bf = *reinterpret_cast<const v8h*>(brow + k);
+      const v8h af = *reinterpret_cast<const v8h*>(arow + k);
+      acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(bf, af, acc, 0, 0, 0);
+    }
+    // the lane holds, for row j, the columns nt * 32 + 8 q + 4 hh + r of P
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      const v4h o = {(_Float16)acc[4 * q], (_Float16)acc[4 * q + 1], (_Float16)acc[4 * q + 2], (_Float16)acc[4 * q + 3]};
+      *reinterpret_cast<v4h*>(Ps + j * PLD + nt * 32 + 8 * q + 4 * hh) = o;
+    }
+  }
+  __syncthreads();
+  const _Float16* prow = Ps + j * PLD + 8 * hh;
+  const bool stored = rb * 32 + j < M;
+  _Float16* drow = D + ((size_t)g * M + row) * P + 4 * hh;
+  for (int pt = wave; pt < P / 32; pt += 4) {
+    const _Float16* crow = Cm + ((size_t)g * P + pt * 32 + j) * N + 8 * hh;
+    v16f acc;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) acc[r] = 0.0f;
+#pragma unroll 4
+    for (int n = 0; n < N; n += 16) {
+      const v8h cf = *reinterpret_cast<const v8h*>(crow + n);
+      const v8h pf = *reinterpret_cast<const v8h*>(prow + n);
+      acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(cf, pf, acc, 0, 0, 0);
+    }
+    if (stored) {
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const v4h o = {(_Float16)acc[4 * q], (_Float16)acc[4 * q + 1], (_Float16)acc[4 * q + 2], (_Float16)acc[4 * q + 3]};
+        *reinterpret_cast<v4h*>(drow + pt * 32 + 8 * q) = o;
+      }
+    }
+  }
+}
+
+static int launch_b2b_stream(const void* A, const void* B, const void* C, void* D, int G, int M, int N, int K, int P,
+                             int lds_max, hipStream_t s) {
+  const size_t lds = (size_t)32 * (N + 8) * 2;
+  if (N > kStreamMaxN || (int)lds > lds_max)
+    return fail(FTK_ERR_UNSUPPORTED_SHAPE, "ftk_b2b_gemm_f16: N=%d: 32 rows of the intermediate product need %zu bytes of LDS (N <= %d)",
+                N, lds, kStreamMaxN);
+  const long long row_blocks = (M + 31) / 32;
+  const long long total = row_blocks * G;
+  if (total > 0x7fffffffLL) return fail(FTK_ERR_UNSUPPORTED_SHAPE, "ftk_b2b_gemm_f16: grid too large");
+  static int attr_lds = 0;
+  if ((int)lds > attr_lds) {
+    FTK_HIP(hipFuncSetAttribute((const void*)b2b_stream_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+    attr_lds = (int)lds;
+  }
+  hipLaunchKernelGGL(b2b_stream_kernel, dim3((unsigned)total), dim3(256), lds, s, (const _Float16*)A, (const _Float16*)B,
+                     (const _Float16*)C, (_Float16*)D, M, N, K, P, (int)row_blocks);
+  return check_launch("b2b_stream_kernel");
+}
+
 }  // namespace ftk
 
 extern "C" int ftk_b2b_gemm_f16(const void* A, const void* B, const void* C, void* D, int G, int M, int N, int K,
@@ -830,12 +918,17 @@ extern "C" int ftk_b2b_gemm_f16(const void* A, const void* B, const void* C, voi
   if (G <= 0 || M <= 0 || N <= 0 || K <= 0 || P <= 0)
     return fail(FTK_ERR_INVALID_ARGUMENT, "ftk_b2b_gemm_f16: G, M, N, K, P must be positive");
   if (N % 32 || P % 32) return fail(FTK_ERR_UNSUPPORTED_SHAPE, "ftk_b2b_gemm_f16: N=%d and P=%d must be multiples of 32", N, P);
-  if (K != 32 && K != 64 && K != 96 && K != 128)
-    return fail(FTK_ERR_UNSUPPORTED_SHAPE, "ftk_b2b_gemm_f16: K=%d must be one of 32, 64, 96, 128", K);
+  if (K % 16) return fail(FTK_ERR_UNSUPPORTED_SHAPE, "ftk_b2b_gemm_f16: K=%d must be a multiple of 16", K);
   const DeviceProps* dp = nullptr;
   int rc = device_props(&dp);
   if (rc) return rc;
   hipStream_t s = (hipStream_t)stream;
+  // The fused kernels keep B (all of K) and a tile of C in LDS: K of 32, 64, 96 or 128, and B and C small enough to
+  // fit beside one wave's region.  Everything else goes to the general kernel.
+  const bool fast = (K == 32 || K == 64 || K == 96 || K == 128) &&
+                    (int)b2b_lds_bytes(N, K, std::min(P, B2B_PTILE), 1) <= dp->lds_optin &&
+                    (P % B2B_PTILE == 0 || (int)b2b_lds_bytes(N, K, P % B2B_PTILE, 1) <= dp->lds_optin);
+  if (!fast) return launch_b2b_stream(A, B, C, D, G, M, N, K, P, dp->lds_optin, s);
   // wide N with few columns of D (the reference benchmark's shapes): N split over the waves of a workgroup.
   // FTK_B2B_WIDE=0 keeps them on the general kernel.
   static const bool allow_wide = !(getenv("FTK_B2B_WIDE") && atoi(getenv("FTK_B2B_WIDE")) == 0);

@@ -359,7 +359,12 @@ int ftk_embedding_gather_f32(const float* table, const void* ids,
  * A [G,M,K] row-major; B stored [G,N,K] (= K x N column-major); C stored
  * [G,P,N] (= N x P column-major); D [G,M,P] row-major -- the layouts of
  * kaleido/core/operators/tests/b2b_gemm_test_utils.h:3-9.
- * Needs K%32==0, N%32==0, P%32==0, K<=256, P<=256.
+ * Needs K%16==0, N%32==0, P%32==0, any M.  K of 32, 64, 96 or 128 with B and a
+ * 128-column tile of C small enough for LDS (N up to 256 at K=128, 512 at
+ * K=64) runs on the fused kernels that keep B and C on chip; every other
+ * shape (N <= 2048), the reference test's [192,704]x[704,448]x[448,832]
+ * (kaleido/core/operators/tests/test_b2b_gemm.cu:137-149) included, on a
+ * general kernel that streams B and C.
  * Replaces B2BGemm::operator() (kaleido/core/device/kernels/gemm.h:235-269,
  * KeBack2BackGemm cutlass_wmma.h:441-540); the reference has no batch
  * dimension, G maps to independent workgroups.

@@ -40,6 +40,7 @@ def test_argument_errors_come_back_as_codes_not_crashes():
     assert lib.ftk_lstm_cell_f32(one, one, nul, one, nul, one, one, ci(4), ci(32), ci(32), nul) == -1
     assert lib.ftk_b2b_gemm_f16(one, one, one, one, ci(1), ci(64), ci(48), ci(64), ci(64), nul) == -2
     assert lib.ftk_b2b_gemm_f16(one, one, one, one, ci(0), ci(64), ci(64), ci(64), ci(64), nul) == -1
+    assert lib.ftk_b2b_gemm_f16(one, one, one, one, ci(1), ci(64), ci(64), ci(24), ci(64), nul) == -2   # K % 16
     assert lib.ftk_b2b_gemm_rowmajor_f16(one, one, one, one, ci(1), ci(64), ci(64), ci(96), ci(128), nul) == -2
     assert lib.ftk_b2b_gemm_rowmajor_f16(one, nul, one, one, ci(1), ci(64), ci(64), ci(64), ci(128), nul) == -1
     assert lib.ftk_gemm_f16(one, one, one, ci(64), ci(96), ci(64), nul) == -2

@@ -86,8 +86,9 @@ def test_lstm_cell_closed_forms(core):
     np.testing.assert_allclose(c.cpu().numpy(), cp_np, rtol=1e-6, atol=1e-7)
 
 
-def test_lstm_elementwise(core):
-    B, H = 70, 128
+# (70, 128): ragged against the kernel's tiles; the others: core/operators/tests/test_lstm.cu:697-703
+@pytest.mark.parametrize('B,H', [(70, 128), (32, 32), (64, 64), (128, 128), (256, 256), (512, 512)])
+def test_lstm_elementwise(core, B, H):
     rng = np.random.default_rng(11)
     g = (rng.standard_normal((B, 4 * H)) * 3).astype(np.float32)
     b = rng.standard_normal(4 * H).astype(np.float32)
@@ -347,6 +348,14 @@ def test_stacked_lstm_ragged_rejects_unsorted_rows(core):
     (512, 3, 70, 32, [1, 16, 32], False, False),
     (1024, 3, 40, 32, [1, 16, 32], True, False),
     (256, 3, 70, 64, [4, 16, 32], True, True),              # ... and rows that stop after 4 steps
+    (32, 4, 4, 8, None, False, False),              # the shapes of the reference's region tests, (depth, steps, batch, hidden)
+    (32, 4, 4, 32, None, False, False),             # = (4, 4, 8, 32), (4, 4, 32, 32), (2, 16, 32, 64), (2, 32, 32, 64), (2, 50, 32, 64),
+    (64, 2, 16, 32, None, False, False),            # (16, 64, 64, 128): core/operators/tests/test_stacked_lstm_region.cu:187-270;
+    (64, 2, 32, 32, None, False, False),
+    (64, 2, 50, 32, None, False, False),            # 50 steps: the case the reference leaves commented out ("irregular seq_len")
+    (128, 16, 64, 64, None, False, False),
+    (32, 4, 4, 8, [1, 2, 4, 8], False, False),      # test_dilated_lstm_region.cu:125-148
+    (32, 4, 4, 32, [1, 2, 4, 8], False, False),
 ])
 def test_stacked_lstm_f16(core, H, L, T, B, dil, bias, ragged):
     rng = np.random.default_rng(13)
@@ -398,6 +407,13 @@ def test_stacked_lstm_f16_rejects_other_hidden_sizes(core):
     (1, 64, 128, False, True),          # zero state: only the x rows of WU are read
     (513, 192, 64, True, False),
     (40, 96, 32, True, True),           # one unit block, odd count of k chunks
+    (256, 128, 128, True, False),       # the reference's whole-cell sweep, [4 H, 256, H] for H = 128 ... 2048
+    (256, 256, 256, True, False),       # (core/operators/tests/test_lstm.cu:723-752; 1024 is the first case above)
+    (256, 512, 512, True, False),
+    (256, 2048, 2048, True, False),
+    (32, 32, 32, True, False),          # its smallest tiles, 32 columns of x and h (test_lstm.cu:705-722), at the
+    (32, 64, 32, True, False),          # smallest hidden size the kernels here take (32; the reference's is 16)
+    (256, 512, 128, True, False),       # [4 * 128, 256, 512]
 ])
 def test_lstm_cell_f16(core, B, I, H, state, bias):
     rng = np.random.default_rng(17)
@@ -645,6 +661,12 @@ def test_b2b_gemm_rowmajor_rejects_other_shapes(core):
     (2, 500, 256, 128, 128),
     (1, 4096, 512, 128, 128),   # largest operands of the family: B and C of 128 KB each pass through LDS
     (1, 512, 384, 64, 64),      # N between the wide kernel's sizes: the general kernel
+    (1, 16, 64, 64, 64),        # the shapes of the reference's own test (core/operators/tests/test_b2b_gemm.cu:110-149) ...
+    (1, 32, 64, 64, 64),
+    (1, 64, 64, 64, 64),
+    (1, 192, 448, 704, 832),    # ... whose last is past what stays on chip: the general kernel that streams B and C
+    (2, 70, 96, 48, 160),       # general kernel: K that is no multiple of 32, ragged rows, several problems
+    (1, 40, 2048, 16, 32),      # general kernel: the widest intermediate it takes, the smallest K
     (2, 300, 64, 64, 128),      # eight-wave kernel (N, K in {64, 128}, full 128-column tiles), ragged M
     (2, 1000, 128, 64, 256),    # eight-wave kernel, two column tiles, units that do not divide evenly
     (1, 4100, 128, 128, 160),   # eight-wave kernel for the first 128 columns, four-wave kernel for the last 32
