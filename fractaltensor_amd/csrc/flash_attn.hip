@@ -330,7 +330,9 @@ __global__ __launch_bounds__(WAVES * 64, MINB) void flash_attn_kernel(const _Flo
   // read the first three fragments of the next one (kpre / vpre).
   constexpr int NE = 12;   // 8 to 16 measure the same
   constexpr int NS = 2 * DT;
-  constexpr int LA = 3;   // fragments read ahead of the matrix instruction that uses them (4 to 6 measure the same)
+  // fragments read ahead of the matrix instruction that uses them (4 to 6 measure the same); a head dimension of 32
+  // has two-step blocks, so two
+  constexpr int LA = DS < 3 ? DS : 3;
   static_assert(LA <= DS && LA <= NS, "the lookahead must fit in one block");
   v8h kpre[LA], vpre[LA];
   auto block_e = [&](const unsigned char* kbase, const unsigned char* vbase, const v16f (&sc)[QT], v8h (&pf)[QT][2],
@@ -631,7 +633,7 @@ extern "C" int ftk_flash_attn_f16(const void* Q, const void* K, const void* V, v
   if (!Q || !K || !V || !O) return fail(FTK_ERR_INVALID_ARGUMENT, "ftk_flash_attn_f16: Q, K, V, O must be non-NULL");
   if (B <= 0 || Hd <= 0 || Sq <= 0 || Skv <= 0 || D <= 0)
     return fail(FTK_ERR_INVALID_ARGUMENT, "ftk_flash_attn_f16: B, Hd, Sq, Skv, D must be positive");
-  if (D != 64 && D != 128) return fail(FTK_ERR_UNSUPPORTED_SHAPE, "ftk_flash_attn_f16: D=%d must be 64 or 128", D);
+  if (D != 32 && D != 64 && D != 128) return fail(FTK_ERR_UNSUPPORTED_SHAPE, "ftk_flash_attn_f16: D=%d must be 32, 64 or 128", D);
   const long long bh = (long long)B * Hd;
   if (bh > (1LL << 24)) return fail(FTK_ERR_UNSUPPORTED_SHAPE, "ftk_flash_attn_f16: B*Hd=%lld too large", bh);
   const DeviceProps* dp = nullptr;
@@ -649,7 +651,12 @@ extern "C" int ftk_flash_attn_f16(const void* Q, const void* K, const void* V, v
     if (variant == 1) return launch_fa<128, 1, 4, 1>(Q, K, V, O, (int)bh, Sq, Skv, scale, lds, s);
     return launch_fa<128, 1, 8, 1>(Q, K, V, O, (int)bh, Sq, Skv, scale, lds, s);
   }
-  if (variant == 1) return launch_fa<64, 1, 4, 1>(Q, K, V, O, (int)bh, Sq, Skv, scale, lds, s);
-  return launch_fa<64, 1, 8, 1>(Q, K, V, O, (int)bh, Sq, Skv, scale, lds, s);
+  if (D == 64) {
+    if (variant == 1) return launch_fa<64, 1, 4, 1>(Q, K, V, O, (int)bh, Sq, Skv, scale, lds, s);
+    return launch_fa<64, 1, 8, 1>(Q, K, V, O, (int)bh, Sq, Skv, scale, lds, s);
+  }
+  // D = 32: the head dimension of the reference's example program (examples/flash_attention/flash_attention.py:96-110)
+  if (variant == 1) return launch_fa<32, 1, 4, 1>(Q, K, V, O, (int)bh, Sq, Skv, scale, lds, s);
+  return launch_fa<32, 1, 8, 1>(Q, K, V, O, (int)bh, Sq, Skv, scale, lds, s);
 }
 

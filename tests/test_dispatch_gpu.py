@@ -254,7 +254,7 @@ def test_reference_style_dilated_model_routes_every_samples_fold():
 
 # ---- attention ----------------------------------------------------------------------------------------------------
 
-@pytest.mark.parametrize('D,scale', [(128, 128 ** -0.5), (64, 1.0), (64, 0.2)])
+@pytest.mark.parametrize('D,scale', [(128, 128 ** -0.5), (64, 1.0), (64, 0.2), (32, 32 ** -0.5)])   # 32: the reference example's head dimension
 def test_programs_flash_attention_is_routed_with_its_scale(D, scale):
     core = _core()
     B, Hd, S, blk = 2, 2, 256, 64
@@ -278,6 +278,21 @@ def test_reference_style_flash_attention_without_a_scale():
     scaled = FractalTensor.from_dense(qsss.as_dense() * 0.25, 3)           # keeps the unscaled scores in fp16's comfortable range
     out = flash_attention(scaled, ksss, vsss)
     assert dispatch.stats['flash_attention'] == 1
+    to4 = lambda t: t.as_dense().reshape(B, Hd, S, D).float().cpu().numpy()
+    ref = ko.attention(to4(scaled), to4(ksss), to4(vsss), 1.0, dtype=np.float32)
+    assert ko.max_rel_err(to4(out), ref) <= 1e-2
+
+
+def test_reference_example_sizes_of_flash_attention():
+    """The example's own configuration (examples/flash_attention/flash_attention.py:96-110): batch 2, 8 heads, 1024
+    tokens in blocks of 64, head dimension 32, fp32 data, no scale.  fp32 programs go to the fp16 kernel only when
+    allowed to."""
+    B, Hd, S, blk, D = 2, 8, 1024, 64, 32
+    qsss, ksss, vsss = (programs.make_attention_input(B, Hd, S, blk, D, seed=60 + i, device='cuda') for i in range(3))
+    scaled = FractalTensor.from_dense(qsss.as_dense() * 0.25, 3)
+    dispatch.allow_half_attention = True
+    out = flash_attention(scaled, ksss, vsss)
+    assert dispatch.stats['flash_attention'] == 1 and out.data.dtype == torch.float32
     to4 = lambda t: t.as_dense().reshape(B, Hd, S, D).float().cpu().numpy()
     ref = ko.attention(to4(scaled), to4(ksss), to4(vsss), 1.0, dtype=np.float32)
     assert ko.max_rel_err(to4(out), ref) <= 1e-2

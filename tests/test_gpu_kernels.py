@@ -732,6 +732,10 @@ def fa_inputs(seed, B, Hd, Sq, Skv, D):
     (2, 3, 256, 256, 128),
     (1, 1, 300, 1000, 128),    # ragged, many tiles
     (2, 8, 1024, 1024, 64),    # the example's sizes, batch 2, 8 heads (flash_attention.py:96-110) at D 64
+    (2, 8, 1024, 1024, 32),    # ... and at the example's own head dimension of 32
+    (1, 3, 100, 77, 32),       # D 32, ragged queries and keys
+    (1, 2, 33, 1, 32),         # a single key
+    (4, 16, 512, 512, 32),     # enough query blocks for the eight-wave variant
 ])
 def test_flash_attention(core, B, Hd, Sq, Skv, D):
     Q, K, V = fa_inputs(4, B, Hd, Sq, Skv, D)
