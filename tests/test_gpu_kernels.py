@@ -168,6 +168,8 @@ def products(core, request):
     (6, 12, 256, [1, 2, 4, 8, 16, 32], False),  # config 5 layer structure, short sequence
     (6, 72, 64, [1, 2, 4, 8, 16, 32], True),    # config 5 dilations with T > 2*32: the recurrences at d = 16 and 32 are live
     (2, 70, 40, [32, 16], False),               # the long links first; second row block holds 8 rows
+    (33, 3, 32, None, True),                    # one layer more than the chip holds at eight workgroups each: per-stage launches
+    (40, 4, 40, None, False),
 ])
 def test_stacked_lstm_persistent(core, products, L, T, B, dil, bias):
     H = 256
