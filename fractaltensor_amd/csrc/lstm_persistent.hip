@@ -936,7 +936,7 @@ static int persistent_slots(int mode, const void** fn, int* slots) {
 // mode kProductsF32 / kProductsSplit: fp32 xs, WU, hsss, csss, H = 256.  kHalfData: the same arrays in fp16, H = 512.
 static int run_persistent(int mode, const void* xs, const void* WU, const float* bias, const int* dil, const int* active,
                           void* hsss, void* csss, int L, int T, int B, void* ws, size_t ws_bytes, hipStream_t s,
-                          bool* handled, int spin_limit = 0) {
+                          bool* handled, int spin_limit = 0, bool keep_status = false) {
   *handled = false;
   const void* fn = nullptr;
   int slots = 0;
@@ -1024,7 +1024,10 @@ static int run_persistent(int mode, const void* xs, const void* WU, const float*
   const int grid = a.groups;
   a.xcd_remap = (grid % 8 == 0) ? 1 : 0;
 
-  hipLaunchKernelGGL(fill_zero_kernel, dim3(64), dim3(256), 0, s, a.status, nflags + 64);
+  // flags and status block start from zero; a later launch of a stack that runs as several keeps the error word
+  // of the earlier ones (it then drains at its first long wait, and the call reports the time-out)
+  hipLaunchKernelGGL(fill_zero_kernel, dim3(64), dim3(256), 0, s, a.status + (keep_status ? 1 : 0),
+                     nflags + 64 - (keep_status ? 1 : 0));
   rc = check_launch("fill_zero_kernel");
   if (rc) return rc;
 
@@ -1114,10 +1117,26 @@ static int run_stack(const char* who, const float* xs, const float* WU, const fl
     }
   }
   if (H == PH) {
-    bool handled = false;
-    rc = run_persistent(products == FTK_LSTM_PRODUCTS_F16X3 ? kProductsSplit : kProductsF32, xs, WU, bias, dil, active,
-                        hsss, csss, L, T, B, ws, ws_bytes, s, &handled, spin_limit);
-    if (rc || handled) return rc;
+    // A stack deeper than the chip holds at eight workgroups a layer runs as consecutive persistent launches: a
+    // launch reads the hidden sequence of the layer below it, complete by then, like the first reads xs.
+    const int mode = products == FTK_LSTM_PRODUCTS_F16X3 ? kProductsSplit : kProductsF32;
+    const void* fn = nullptr;
+    int slots = 0;
+    rc = persistent_slots(mode, &fn, &slots);
+    if (rc) return rc;
+    const int chunk = std::min(slots / PC, kMaxLayers);
+    const size_t slab = (size_t)T * B * H;
+    bool handled = chunk >= 1;
+    for (int l0 = 0; handled && l0 < L; l0 += chunk) {
+      const int lc = std::min(chunk, L - l0);
+      rc = run_persistent(mode, l0 == 0 ? xs : hsss + (size_t)(l0 - 1) * slab, WU + (size_t)l0 * 2 * H * 4 * H,
+                          bias ? bias + (size_t)l0 * 4 * H : nullptr, dil ? dil + l0 : nullptr, active,
+                          hsss + (size_t)l0 * slab, csss + (size_t)l0 * slab, lc, T, B, ws, ws_bytes, s, &handled,
+                          spin_limit, l0 > 0);
+      if (rc) return rc;
+      if (!handled && l0 > 0) return fail(FTK_ERR_DEVICE, "%s: the persistent kernel ran for the first %d layers only", who, l0);
+    }
+    if (handled) return FTK_OK;
   }
   // the launches below wait for nothing: their status word is zero
   if (ws && ws_bytes >= kStatusBytes) {
@@ -1226,7 +1245,7 @@ int ftk_stacked_lstm_f16(const void* xs, const void* WU, const float* bias, cons
     rc = run_persistent(mode, l0 == 0 ? x16 : h16 + (size_t)(l0 - 1) * slab, w16 + (size_t)l0 * 2 * H * 4 * H,
                         bias ? bias + (size_t)l0 * 4 * H : nullptr, dilations ? dilations + l0 : nullptr, active_rows,
                         h16 + (size_t)l0 * slab, c16 + (size_t)l0 * slab, lc, T, B, workspace, workspace_bytes,
-                        (hipStream_t)stream, &handled);
+                        (hipStream_t)stream, &handled, 0, l0 > 0);
     if (rc) return rc;
     if (!handled) return fail(FTK_ERR_DEVICE, "%s: the persistent kernel cannot run on this device", who);
   }

@@ -250,6 +250,12 @@ def test_a_drained_persistent_launch_raises(core):
     # a workspace the wrapper allocates itself is always checked
     with pytest.raises(core.FtkError):
         core.stacked_lstm(dev(xs), dev(WU), dev(bs), spin_limit=1)
+    # a stack that runs as two persistent launches: the second keeps the first one's error word
+    L = 34
+    xs, WU, bs = lstm_inputs(4, L, 3, 32, H, 1.0 / 16)
+    with pytest.raises(core.FtkError) as info:
+        core.stacked_lstm(dev(xs), dev(WU), dev(bs), spin_limit=1)
+    assert info.value.code == -6
 
 
 @pytest.mark.parametrize('L,T,B,dil,lengths', [
