@@ -91,11 +91,12 @@ __device__ __forceinline__ float max_with_other_half(float x) {
 //     16 consecutive keys, same columns) then touches 16 different 16-byte
 //     chunks of the 256-byte bank line;
 //   V rows are padded by 64 bytes: one 32-lane pass of the transposing read
-//     covers 4 keys x 64 bytes, which land in four different 64-byte groups.
+//     covers 4 keys x 64 bytes, which land in four different 64-byte groups
+//     (by 128 bytes where 64 would make the stride a multiple of the bank line, D = 96).
 template <int D>
 struct FaLayout {
   static constexpr int KRS = 2 * D + 16;   // K row stride, bytes
-  static constexpr int VRS = 2 * D + 64;   // V row stride, bytes
+  static constexpr int VRS = (2 * D + 64) % 256 ? 2 * D + 64 : 2 * D + 128;   // V row stride, bytes
   static constexpr int KTB = FA_KT * KRS;  // K tile, bytes (a multiple of 1024)
   static constexpr int VTB = FA_KT * VRS;
   static_assert(KTB % 1024 == 0 && VTB % 1024 == 0, "tiles must be whole 1 KB copies");
@@ -514,8 +515,7 @@ __global__ __launch_bounds__(WAVES * 64, MINB) void flash_attn_kernel(const _Flo
   // bytes each and the wave stores whole rows, 1 KB of consecutive bytes per instruction.  LDS executes a wave's
   // instructions in order, so the wave needs no barrier between its writes and its reads.
   constexpr int ORS = 2 * D + 16;        // padded row: the 32 rows' 8-byte pieces spread over all banks
-  constexpr int LPR = D / 8;             // lanes per row of 16-byte chunks
-  constexpr int RPI = 64 / LPR;          // rows per store instruction
+  constexpr int LPR = D / 8;             // 16-byte chunks per row
   unsigned char* const ot = smem + wave * (32 * ORS);
 #pragma unroll
   for (int qt = 0; qt < QT; ++qt) {
@@ -531,8 +531,8 @@ __global__ __launch_bounds__(WAVES * 64, MINB) void flash_attn_kernel(const _Flo
             v2u{__builtin_bit_cast(unsigned, lo), __builtin_bit_cast(unsigned, hi)};
       }
 #pragma unroll
-    for (int i = 0; i < 32 / RPI; ++i) {
-      const int r = RPI * i + lane / LPR, c = lane % LPR;
+    for (int idx = lane; idx < 32 * LPR; idx += 64) {   // consecutive lanes: consecutive chunks of a row, then the next row
+      const int r = idx / LPR, c = idx - r * LPR;
       const v4u piece = *reinterpret_cast<const v4u*>(ot + r * ORS + 16 * c);
       const int row = q_base + 32 * qt + r;
       // streaming store: O is not read again by this launch, and lines left dirty in L2 are written back only when
@@ -633,7 +633,8 @@ extern "C" int ftk_flash_attn_f16(const void* Q, const void* K, const void* V, v
   if (!Q || !K || !V || !O) return fail(FTK_ERR_INVALID_ARGUMENT, "ftk_flash_attn_f16: Q, K, V, O must be non-NULL");
   if (B <= 0 || Hd <= 0 || Sq <= 0 || Skv <= 0 || D <= 0)
     return fail(FTK_ERR_INVALID_ARGUMENT, "ftk_flash_attn_f16: B, Hd, Sq, Skv, D must be positive");
-  if (D != 32 && D != 64 && D != 128) return fail(FTK_ERR_UNSUPPORTED_SHAPE, "ftk_flash_attn_f16: D=%d must be 32, 64 or 128", D);
+  if (D != 32 && D != 64 && D != 96 && D != 128)
+    return fail(FTK_ERR_UNSUPPORTED_SHAPE, "ftk_flash_attn_f16: D=%d must be 32, 64, 96 or 128", D);
   const long long bh = (long long)B * Hd;
   if (bh > (1LL << 24)) return fail(FTK_ERR_UNSUPPORTED_SHAPE, "ftk_flash_attn_f16: B*Hd=%lld too large", bh);
   const DeviceProps* dp = nullptr;
@@ -650,6 +651,10 @@ extern "C" int ftk_flash_attn_f16(const void* Q, const void* K, const void* V, v
   if (D == 128) {
     if (variant == 1) return launch_fa<128, 1, 4, 1>(Q, K, V, O, (int)bh, Sq, Skv, scale, lds, s);
     return launch_fa<128, 1, 8, 1>(Q, K, V, O, (int)bh, Sq, Skv, scale, lds, s);
+  }
+  if (D == 96) {
+    if (variant == 1) return launch_fa<96, 1, 4, 1>(Q, K, V, O, (int)bh, Sq, Skv, scale, lds, s);
+    return launch_fa<96, 1, 8, 1>(Q, K, V, O, (int)bh, Sq, Skv, scale, lds, s);
   }
   if (D == 64) {
     if (variant == 1) return launch_fa<64, 1, 4, 1>(Q, K, V, O, (int)bh, Sq, Skv, scale, lds, s);

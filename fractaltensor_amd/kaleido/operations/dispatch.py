@@ -286,7 +286,7 @@ def _attention_operands(xs):
     q, k, v = (t.as_dense() for t in src)
     if k.shape != v.shape or q.shape[:2] != k.shape[:2] or q.shape[-1] != k.shape[-1] or q.dtype != k.dtype or q.dtype != v.dtype:
         return None
-    if q.shape[-1] not in (32, 64, 128):
+    if q.shape[-1] not in (32, 64, 96, 128):
         return None
     return q, k, v
 

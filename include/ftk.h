@@ -410,7 +410,7 @@ int ftk_batched_gemm_f16(const void* A, const void* B, void* C, int G, int M,
 /*
  * O = softmax(Q K^T * scale) V per (batch, head), non-causal, fp16 storage,
  * fp32 accumulation, online softmax (running max / sum) in registers.
- * Q,O [B,Hd,Sq,D]; K,V [B,Hd,Skv,D].  D == 128, 64 or 32; any Sq, Skv >= 1 (the
+ * Q,O [B,Hd,Sq,D]; K,V [B,Hd,Skv,D].  D == 128, 96, 64 or 32; any Sq, Skv >= 1 (the
  * last, partial blocks of queries and keys are masked).
  * Replaces the map/reduce program flash_attention
  * (examples/flash_attention/flash_attention.py:14-91); the reference has no

@@ -747,6 +747,8 @@ def fa_inputs(seed, B, Hd, Sq, Skv, D):
     (1, 3, 100, 77, 32),       # D 32, ragged queries and keys
     (1, 2, 33, 1, 32),         # a single key
     (4, 16, 512, 512, 32),     # enough query blocks for the eight-wave variant
+    (2, 3, 200, 333, 96),      # D 96: three d tiles, V rows padded by 128 bytes
+    (4, 16, 512, 256, 96),
 ])
 def test_flash_attention(core, B, Hd, Sq, Skv, D):
     Q, K, V = fa_inputs(4, B, Hd, Sq, Skv, D)
