@@ -882,9 +882,10 @@ def main():
             continue
         diffs = [v for v in (r.get('cpu_baseline') or {}, r.get('unfused_gpu_baseline') or {})]
         diff = next((d[k] for d in diffs for k in ('max_rel_diff_vs_gpu', 'max_rel_diff_vs_fused') if k in d), None)
-        rows[CONFIG_OF[name]] = {'workload': name, 'ms_per_step': round(r['ms_per_step'], 5), 'value': r.get('value'), 'unit': r.get('unit'),
-                                 'bound': r['roofline']['bound'], 'frac': round(r['roofline']['frac'], 4), 'max_rel_diff': diff,
-                                 'cpu_baseline': (r.get('cpu_baseline') or {}).get('value')}
+        sig = lambda v: None if v is None else float(f'{v:.4g}')   # four significant digits: the summary has to stay short
+        rows[CONFIG_OF[name]] = {'workload': name, 'ms_per_step': sig(r['ms_per_step']), 'value': sig(r.get('value')), 'unit': r.get('unit'),
+                                 'bound': r['roofline']['bound'], 'frac': sig(r['roofline']['frac']), 'max_rel_diff': sig(diff),
+                                 'cpu_baseline': sig((r.get('cpu_baseline') or {}).get('value'))}
     line['configs'] = dict(sorted(rows.items()))
     print(json.dumps(line))
 
