@@ -25,9 +25,13 @@
 // caches are not coherent with each other) uses no cache-wide fences: what
 // other compute units read is written with agent-scope write-through stores
 // and read with agent-scope copies, every producer wave waits for its own
-// stores to be acknowledged and then increments flags[l][t][rb]; consumers
-// look at that count with agent-scope loads until it reaches 4 x the number of
-// column slices.  c is only ever re-read by the workgroup that wrote it and
+// stores to be acknowledged and then sets its own byte of flags[l][t][rb]
+// (byte 4 x column slice + wave, a plain write-through store); consumers read
+// the flag with one load, lane i byte i, until every producer's byte is set.
+// (A count that the producers incremented atomically was the first form: the
+// consumers' loads then queued behind up to 32 read-modify-writes of the same
+// word, and the layer right above a layer that never waits paid 0.4 us per
+// item for it.)  c is only ever re-read by the workgroup that wrote it and
 // goes through the cache normally.
 //
 // The activation tile is double buffered, global -> LDS copies are requested
@@ -91,7 +95,7 @@ struct PersistArgs {
   const _Float16* xsp;   // [T][B][2][H] planes of the input rows
   const float* xratio;   // [T][B] what an input row's products are multiplied by to match the hidden rows' scale
   _Float16* hsp;         // [L][T][B][2][H] planes of every h
-  int* flags;   // [L][T][NRB] completion counts
+  unsigned char* flags;   // [L][T][NRB][kFlagStride]: one byte per producer wave
   int* status;  // [0] = error word
   int L, T, B;
   int nrb;         // row blocks of 32*RT rows
@@ -114,11 +118,17 @@ __device__ __forceinline__ int flag_load(const int* flag) {
   return __hip_atomic_load(flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
-// Bounded wait until *flag >= target.  Every lane polls the same word, so the
-// result is wave-uniform.
-__device__ __forceinline__ bool wait_count(const int* flag, int target, int* status, int spin_limit) {
+// A flag is kFlagStride bytes, one per producer wave (up to 16 column slices x 4 waves); lane i looks at byte i.
+// Every wait is bounded: when the polls run out the status word is set and the caller drains.
+constexpr int kFlagStride = 64;
+__device__ __forceinline__ int flag_bytes_load(const unsigned char* flag, int lane, int target) {
+  if (lane >= target) return 1;
+  return __hip_atomic_load(flag + lane, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ bool all_set(int v) { return __builtin_amdgcn_ballot_w64(v != 0) == ~0ull; }
+__device__ __forceinline__ bool wait_bytes(const unsigned char* flag, int lane, int target, int* status, int spin_limit) {
   int n = 0;
-  while (flag_load(flag) < target) {
+  while (!all_set(flag_bytes_load(flag, lane, target))) {
     __builtin_amdgcn_s_sleep(1);
     if (++n >= spin_limit) {
       __hip_atomic_store(status, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -200,7 +210,7 @@ void lstm_persistent_kernel(PersistArgs a) {
   constexpr int HID = MODE == kHalfData ? 2 * PH : PH;  // hidden size
   constexpr int NPC = HID / 32;           // column slices per layer (32 units each)
   constexpr int NG = 4 * HID;             // gate columns
-  constexpr int FLAG_TARGET = NPC * 4;    // one count per wave of each column slice
+  constexpr int FLAG_TARGET = NPC * 4;    // producer waves per flag: four of each column slice
   extern __shared__ __attribute__((aligned(16))) float tile[];  // [2][32][P_LD], 256 floats of scrap, 2 staging buffers
 
   const int tid = threadIdx.x;
@@ -312,32 +322,32 @@ void lstm_persistent_kernel(PersistArgs a) {
   // past its block's last step is walked through like any other, but requests, computes, stores and counts
   // nothing; nothing that is computed depends on it.
   auto live = [&](int n) { return !a.ragged || item_t(n) < a.steps_of[item_rb(n)]; };
-  auto flag_of = [&](int ll, int t, int rb) { return a.flags + ((size_t)ll * T + t) * a.nrb + rb; };
+  auto flag_of = [&](int ll, int t, int rb) { return a.flags + (((size_t)ll * T + t) * a.nrb + rb) * kFlagStride; };
 
-  // inputs of item n complete?  Bounded spin on the two counters.
+  // inputs of item n complete?  Bounded spin on the two flags.
   auto wait_deps = [&](int n) __attribute__((always_inline)) -> bool {
     const int t = item_t(n), rb = item_rb(n);
     bool ok = true;
     if (!live(n)) return true;
-    if (l > 0) ok = wait_count(flag_of(l - 1, t, rb), FLAG_TARGET, a.status, a.spin_limit);
-    if (ok && t >= d) ok = wait_count(flag_of(l, t - d, rb), FLAG_TARGET, a.status, a.spin_limit);
+    if (l > 0) ok = wait_bytes(flag_of(l - 1, t, rb), lane, FLAG_TARGET, a.status, a.spin_limit);
+    if (ok && t >= d) ok = wait_bytes(flag_of(l, t - d, rb), lane, FLAG_TARGET, a.status, a.spin_limit);
     // The data loads must stay behind the flag reads.  The hardware issues and
     // returns loads in order, so a compiler barrier is all it takes; a fence
     // instruction here would also wait for this wave's outstanding stores.
     asm volatile("" ::: "memory");
     return ok;
   };
-  // request / test the two counters of item n without waiting
+  // request / test the two flags of item n without waiting (what a lane holds is its byte of each)
   struct Flags { int below, own; };
   auto request_flags = [&](int n) __attribute__((always_inline)) -> Flags {
-    Flags f{FLAG_TARGET, FLAG_TARGET};
+    Flags f{1, 1};
     const int t = item_t(n), rb = item_rb(n);
     if (!live(n)) return f;
-    if (l > 0) f.below = flag_load(flag_of(l - 1, t, rb));
-    if (t >= d) f.own = flag_load(flag_of(l, t - d, rb));
+    if (l > 0) f.below = flag_bytes_load(flag_of(l - 1, t, rb), lane, FLAG_TARGET);
+    if (t >= d) f.own = flag_bytes_load(flag_of(l, t - d, rb), lane, FLAG_TARGET);
     return f;
   };
-  auto flags_ready = [=](const Flags& f) { return f.below >= FLAG_TARGET && f.own >= FLAG_TARGET; };
+  auto flags_ready = [=](const Flags& f) { return all_set(f.below) && all_set(f.own); };
 
   // Where the activation rows come from.  The two fp16 planes of a row take the
   // 1024 bytes of its fp32 form, so the tile code is the same for both: in
@@ -654,12 +664,12 @@ void lstm_persistent_kernel(PersistArgs a) {
     }
     return cp;
   };
-  // every wave publishes its own part of an item: its stores acknowledged, then one count
+  // every wave publishes its own part of an item: its stores acknowledged, then its byte of the flag
   auto publish = [&](int n) __attribute__((always_inline)) {
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
     __builtin_amdgcn_s_waitcnt(0);
     if (lane == 0 && alive && live(n))
-      __hip_atomic_fetch_add(flag_of(l, item_t(n), item_rb(n)), 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      __hip_atomic_store(flag_of(l, item_t(n), item_rb(n)) + 4 * pc + wave, (unsigned char)1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   };
 
   const bool tracing = (q == a.trace_q) && tid == 0;
@@ -848,7 +858,7 @@ __global__ __launch_bounds__(256) void lstm_split_rows_kernel(const float* xs, _
 
 static size_t flag_count(int L, int T, int B) {
   const int nrb = (B + 31) / 32;
-  return (size_t)L * T * nrb;
+  return (size_t)L * T * nrb * (kFlagStride / sizeof(int));
 }
 
 // Workspace layout: [64 ints: status][flags][trace: T*nrb*8 stamps of 8 bytes]
@@ -961,7 +971,7 @@ static int run_persistent(int mode, const void* xs, const void* WU, const float*
   a.hsss = reinterpret_cast<float*>(hsss);
   a.csss = reinterpret_cast<float*>(csss);
   a.status = reinterpret_cast<int*>(ws);
-  a.flags = a.status + 64;
+  a.flags = reinterpret_cast<unsigned char*>(a.status + 64);
   char* wsb = reinterpret_cast<char*>(ws);
   float* xratio = nullptr;
   _Float16* xsp = nullptr;
@@ -1057,7 +1067,7 @@ static int run_persistent(int mode, const void* xs, const void* WU, const float*
 // launch with fp32 products.  Every device the library runs on holds its own copy until the process ends.  In host
 // code the array's name is only a handle for hipGetSymbolAddress; device code and launches use the address that call
 // returns, kept per device.
-constexpr size_t kScratchBytes = 1u << 20;
+constexpr size_t kScratchBytes = 2u << 20;
 static __device__ __align__(256) unsigned char scratch[kScratchBytes];
 constexpr int kMaxDevices = 64;
 static void* g_scratch_ptr[kMaxDevices] = {};

@@ -276,9 +276,9 @@ int ftk_stacked_lstm_status(const void* workspace, ftk_stream_t stream);
  * tight serving loops, harnesses that forbid hipMalloc.  No counterpart in
  * the reference.  Same operands and results as ftk_stacked_lstm_opts_f32
  * with {FTK_LSTM_PRODUCTS_F32, 0} and no active_rows; H must be 256, and the
- * status block, flags and trace of the launch (about 4*L*T*ceil(B/32) +
+ * status block, flags and trace of the launch (about 64*L*T*ceil(B/32) +
  * 64*T*ceil(B/32) + 256 bytes) must fit the library's built-in scratch of
- * 1 MiB per device (config 4, L32 T64 B256: 98 KB), else
+ * 2 MiB per device (config 4, L32 T64 B256: 1.03 MiB), else
  * FTK_ERR_UNSUPPORTED_SHAPE; likewise when L layers do not fit the device in
  * one persistent launch.  The call allocates nothing, frees nothing and waits
  * for nothing.  Every call on a device shares that device's scratch: calls

@@ -46,7 +46,7 @@ def test_noalloc_entry_point_rejects_what_does_not_fit():
     with pytest.raises(core.FtkError) as info:
         core.stacked_lstm_noalloc(xs, WU, bs, out)
     assert info.value.code == -2
-    # flags and trace beyond the 1 MiB scratch: L 32 x T 4096 x 8 row blocks of flags alone are 4 MiB.  Only the sizes
+    # flags and trace beyond the 2 MiB scratch: L 32 x T 4096 x 8 row blocks of flags alone are 64 MiB.  Only the sizes
     # are looked at before the refusal, so small buffers stand in for the operands.
     import ctypes
     one = ctypes.c_void_p(xs.data_ptr())
