@@ -363,10 +363,13 @@ void lstm_persistent_kernel(PersistArgs a) {
   const unsigned lane16 = 16u * lane;
   const unsigned lane_lines = 1024u * (lane >> 3) + 128u * (lane & 7);  // one lane per cache line of 8 rows
   const unsigned tile_lds = (unsigned)reinterpret_cast<uintptr_t>((__attribute__((address_space(3))) void*)tile);
-  auto issue_tile = [&](int n, int buf) __attribute__((always_inline)) {
+  // part: kWholeTile, or only its x columns / only its h columns (the serial schedule asks for them at different times)
+  constexpr int kWholeTile = 0, kTileX = 1, kTileH = 2;
+  auto issue_tile = [&](int n, int buf, int part = 0) __attribute__((always_inline)) {
     const int t = item_t(n), rb = item_rb(n);
     if (!live(n)) return;
-    const bool has_prev = t >= d;
+    const bool has_prev = t >= d && part != kTileX;
+    const bool with_x = part != kTileH;
     const char* xsrc = reinterpret_cast<const char*>((l == 0) ? xin + (size_t)t * cell : hin + ((size_t)(l - 1) * T + t) * cell);
     const char* hsrc = reinterpret_cast<const char*>(hin + ((size_t)l * T + (has_prev ? t - d : 0)) * cell);
     const int row0 = rb * 32 + 8 * wave_u;
@@ -375,10 +378,12 @@ void lstm_persistent_kernel(PersistArgs a) {
       if (row0 + 8 <= B) {
         const char* xb = xsrc + (size_t)row0 * 512;
         const char* hb = hsrc + (size_t)row0 * 512;
-        static_for<4>([&](auto rc) __attribute__((always_inline)) {
-          constexpr int r = decltype(rc)::value;
-          lds_dma16<r * 1024, kCoherentTiles>(xb, lane16, ldsp + 4u * r * P_LD);
-        });
+        if (with_x) {
+          static_for<4>([&](auto rc) __attribute__((always_inline)) {
+            constexpr int r = decltype(rc)::value;
+            lds_dma16<r * 1024, kCoherentTiles>(xb, lane16, ldsp + 4u * r * P_LD);
+          });
+        }
         if (has_prev) {
           static_for<4>([&](auto rc) __attribute__((always_inline)) {
             constexpr int r = decltype(rc)::value;
@@ -389,7 +394,7 @@ void lstm_persistent_kernel(PersistArgs a) {
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
           const size_t rg = (size_t)max(min(row0 + 2 * r, B - 2), 0);
-          lds_dma16<0, kCoherentTiles>(xsrc + rg * 512, lane16, ldsp + 4u * r * P_LD);
+          if (with_x) lds_dma16<0, kCoherentTiles>(xsrc + rg * 512, lane16, ldsp + 4u * r * P_LD);
           if (has_prev) lds_dma16<0, kCoherentTiles>(hsrc + rg * 512, lane16, ldsp + 4u * r * P_LD + 1024u);
         }
       }
@@ -398,10 +403,12 @@ void lstm_persistent_kernel(PersistArgs a) {
     const unsigned lds0 = tile_lds + 4u * (unsigned)(buf * P_TILE + 8 * wave_u * P_LD);
     if (row0 + 8 <= B) {
       const char* xb = xsrc + (size_t)row0 * 1024;
-      static_for<8>([&](auto rc) __attribute__((always_inline)) {
-        constexpr int r = decltype(rc)::value;
-        lds_dma16<(r & 3) * 1024, kCoherentTiles>(xb + (r >> 2) * 4096, lane16, lds0 + 4u * r * P_LD);
-      });
+      if (with_x) {
+        static_for<8>([&](auto rc) __attribute__((always_inline)) {
+          constexpr int r = decltype(rc)::value;
+          lds_dma16<(r & 3) * 1024, kCoherentTiles>(xb + (r >> 2) * 4096, lane16, lds0 + 4u * r * P_LD);
+        });
+      }
       if (has_prev) {
         const char* hb = hsrc + (size_t)row0 * 1024;
         static_for<8>([&](auto rc) __attribute__((always_inline)) {
@@ -413,7 +420,7 @@ void lstm_persistent_kernel(PersistArgs a) {
 #pragma unroll
       for (int r = 0; r < 8; ++r) {
         const size_t rg = (size_t)min(row0 + r, B - 1);
-        lds_dma16<0, kCoherentTiles>(xsrc + rg * 1024, lane16, lds0 + 4u * r * P_LD);
+        if (with_x) lds_dma16<0, kCoherentTiles>(xsrc + rg * 1024, lane16, lds0 + 4u * r * P_LD);
         if (has_prev) lds_dma16<0, kCoherentTiles>(hsrc + rg * 1024, lane16, lds0 + 4u * r * P_LD + 1024u);
       }
     }
@@ -422,7 +429,7 @@ void lstm_persistent_kernel(PersistArgs a) {
     // the other layers' rows.  One 4-byte-per-lane copy touches all 64 cache lines of the wave's 8 rows;
     // it lands in a scrap area behind the tiles (a load into registers would need them reserved until
     // the data arrives).
-    if (!PAIR && l == 0 && n + 1 < n_items && live(n + 1)) {
+    if (!PAIR && with_x && l == 0 && n + 1 < n_items && live(n + 1)) {
       const int t2 = item_t(n + 1), rb2 = item_rb(n + 1);
       const int row2 = rb2 * 32 + 8 * wave_u;
       if (row2 + 8 <= B)
@@ -681,21 +688,51 @@ void lstm_persistent_kernel(PersistArgs a) {
   const bool serial = own_distance < 2;
 
   if (serial) {
+    // Every item waits for the one before it, so what an item costs is the chain from one hand-over to the next:
+    // the siblings' h arrives -> its rows are copied -> h half of the products -> activations -> stores -> their
+    // acknowledgement -> this wave's byte of the flag.  Everything that does not depend on the previous item is
+    // taken off that chain: the x columns of tile n+1 are requested with the h columns of tile n (when the layer
+    // below has them already), and the x half of item n+1 is formed between the stores of item n and the wait
+    // for their acknowledgement, which takes longer than those MFMAs.
+    bool xdone = false;    // the x half of the current item is in the accumulators already
+    bool xhere = false;    // the x columns of the current item's tile are in LDS (or on their way)
     for (int n = 0; n < n_items; ++n) {
+      const int buf = n & 1;
       if (tracing) a.trace[TS * n + 0] = wall_clock64();
       if (alive) alive = wait_deps(n);
-      if (alive) issue_tile(n, 0);
+      if (alive) issue_tile(n, buf, xhere ? kTileH : kWholeTile);
+      // the x columns of the next item: its own layer's dependency is this item, but the x rows only need the layer below
+      bool xnext = false;
+      if (alive && n + 1 < n_items && live(n + 1)) {
+        bool below_ready = l == 0;
+        if (l > 0) below_ready = all_set(flag_bytes_load(flag_of(l - 1, item_t(n + 1), item_rb(n + 1)), lane, FLAG_TARGET));
+        if (below_ready) {
+          asm volatile("" ::: "memory");
+          issue_tile(n + 1, buf ^ 1, kTileX);
+          xnext = true;
+        }
+      }
       const float4 cp = load_cprev(n);
+      const float ratio_next = (xnext && SPLIT) ? load_ratio(n + 1) : 1.0f;
       __builtin_amdgcn_s_waitcnt(0);
       __syncthreads();
       if (live(n)) {
-        mfma_range(0, IC<0>{}, IC<0>{}, IC<16>{});
-        rescale_x(load_ratio(n));
-        if (item_t(n) >= d) mfma_range(0, IC<1>{}, IC<0>{}, IC<16>{});
+        if (!xdone) {
+          mfma_range(buf, IC<0>{}, IC<0>{}, IC<16>{});
+          rescale_x(load_ratio(n));
+        }
+        if (item_t(n) >= d) mfma_range(buf, IC<1>{}, IC<0>{}, IC<16>{});
         epilogue_to_lds(gate_sums(), cp, 0);
       }
-      __syncthreads();  // results staged; the tile may be rewritten by the next item
+      __syncthreads();  // results staged; the tile may be rewritten by the item after the next
       store_item(n, 0);
+      xdone = false;
+      if (xnext) {          // while the stores are acknowledged
+        mfma_range(buf ^ 1, IC<0>{}, IC<0>{}, IC<16>{});
+        rescale_x(ratio_next);
+        xdone = true;
+      }
+      xhere = xnext;
       publish(n);
       if (tracing) a.trace[TS * n + 7] = wall_clock64();
     }
