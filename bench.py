@@ -212,7 +212,7 @@ def bench_attention(torch, core, steps, warmup, cpu):
         'pct_f16_mfma_peak': 100.0 * flop / ms / 1e9 / PEAK_F16_TFLOPS,
         'roofline': {'bound': 'mfma', 'achieved': flop / ms / 1e9, 'peak': PEAK_F16_TFLOPS, 'unit': 'TFLOP/s',
                      'frac': flop / ms / 1e9 / PEAK_F16_TFLOPS,
-                     'traffic': MEASURED_TRAFFIC_BYTES.get('flash_attn_kernel'), 'kernel': 'flash_attn_kernel'},
+                     'traffic': MEASURED_TRAFFIC_BYTES.get('flash_attn_pp_kernel'), 'kernel': 'flash_attn_pp_kernel'},
     }
     if cpu:
         from oracle import c_oracle

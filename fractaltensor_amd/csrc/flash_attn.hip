@@ -36,6 +36,10 @@
 // the matrix unit itself (score accumulators start from -m_ref instead of 0),
 // row sums use plain adds, and the loop is software pipelined per 32-key half
 // tile with the instruction order written out and fenced step by step.
+//
+// flash_attn_pp_kernel (whole key tiles, D = 128 / 96) orders the same work differently: the two waves of a SIMD
+// alternate between a phase of matrix instructions only and a phase of vector instructions only, in opposite phases,
+// and the running maximum is moved only when a sum of exponentials says it must (see the comment at the kernel).
 #include <stdlib.h>
 
 #include <algorithm>
@@ -47,6 +51,7 @@ namespace ftk {
 
 constexpr int FA_KT = 64;          // keys per tile
 constexpr float FA_TAU = 8.0f;     // slack (in powers of two) before the running maximum is moved
+constexpr float FA_PMAX = 32768.0f;  // phase-alternating kernel: a lane's sum of exponentials above this moves the reference
 constexpr int FA_TRACE_TILES = 256;
 
 // Built with -DFTK_DEBUG_TRACE only (make TRACE=1): timeline of one wave of workgroup 0 when FTK_FA_TRACE is set,
@@ -561,6 +566,343 @@ static long long* fa_trace_ptr() {
 }
 #endif
 
+// The same product with the two waves of a SIMD kept in opposite phases (whole key tiles only, 8 waves x 32 query
+// rows).  A wave alternates between a phase of matrix instructions only -- M(t): O^T += V(t)^T P(t)^T, then the
+// scores of tile t+1 -- and a phase of vector instructions only -- S(t): row maximum, exponentials, row sum and
+// packing of tile t's scores -- with a workgroup barrier after every phase.  Waves 4..7 run one phase behind waves
+// 0..3 (they pass one barrier more before the loop, the others one more after it), and wave w + 4 shares its SIMD
+// with wave w: while one of the two feeds the matrix pipe the other one's vector work and copy issue run beside it,
+// instead of both waves interleaving the two kinds of work and stalling at the same places.  The raised priority of
+// the wave in M lets its next MFMA go ahead of the other wave's vector instructions.
+// Tiles: K(t+1) and V(t) are read during M(t), i.e. in two consecutive phase slots.  K has two buffers, V three:
+// waves 0..3 request V(t+1) at the start of S(t), waves 4..7 request K(t+2) at the start of their S(t), and each
+// waits for its own copies before the barrier that ends its following M phase, one slot before the first reader.
+template <int D, bool TRACE>
+__global__ __launch_bounds__(512, 1) void flash_attn_pp_kernel(const _Float16* __restrict__ Q,
+                                                                const _Float16* __restrict__ K,
+                                                                const _Float16* __restrict__ V,
+                                                                _Float16* __restrict__ O, int Sq, int Skv,
+                                                                float scale_log2e, int nqb,
+                                                                long long* __restrict__ trace, int trace_wave) {
+  using L = FaLayout<D>;
+  constexpr int DS = D / 16, DT = D / 32, RB = 2 * D;
+  constexpr int KRS = L::KRS, VRS = L::VRS, KTB = L::KTB, VTB = L::VTB;
+  constexpr int CW = 4;                                   // waves that share the copies of a tile
+  constexpr int KCP = (KTB / 1024 + CW - 1) / CW, VCP = (VTB / 1024 + CW - 1) / CW;
+  extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];
+  unsigned char* const Kb = smem;            // [2][KTB]
+  unsigned char* const Vb = smem + 2 * KTB;  // [3][VTB]
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int group = wave >> 2, cw = wave & 3;
+  const int j = lane & 31, hh = lane >> 5;
+  int id = blockIdx.x;
+  const int total = gridDim.x;
+  if ((total & 7) == 0) id = (blockIdx.x & 7) * (total >> 3) + (blockIdx.x >> 3);
+  const int bh = id / nqb;
+  const int qb = id - bh * nqb;
+  const int q_base = qb * 256 + wave * 32;
+  const _Float16* Qg = Q + (size_t)bh * Sq * D;
+  const _Float16* Kg = K + (size_t)bh * Skv * D;
+  const _Float16* Vg = V + (size_t)bh * Skv * D;
+  _Float16* Og = O + (size_t)bh * Sq * D;
+
+  v8h qf[DS];
+  {
+    const int row = min(q_base + j, Sq - 1);
+#pragma unroll
+    for (int s = 0; s < DS; ++s) {
+      const uint4 v = *reinterpret_cast<const uint4*>(Qg + (size_t)row * D + 16 * s + 8 * hh);
+      const v8h q = *reinterpret_cast<const v8h*>(&v);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) qf[s][e] = (_Float16)((float)q[e] * scale_log2e);
+    }
+  }
+  v16f oacc[DT];
+#pragma unroll
+  for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) oacc[dt][r] = 0.0f;
+  float l_run = 0.0f;
+
+  unsigned k_src[KCP], v_src[VCP];
+#pragma unroll
+  for (int i = 0; i < KCP; ++i) {
+    const int x = 1024 * (cw + CW * i) + 16 * lane;
+    const int row = min(x / KRS, FA_KT - 1), col = x % KRS;
+    k_src[i] = row * RB + (col < RB ? col : 0);
+  }
+#pragma unroll
+  for (int i = 0; i < VCP; ++i) {
+    const int x = 1024 * (cw + CW * i) + 16 * lane;
+    const int row = min(x / VRS, FA_KT - 1), col = x % VRS;
+    v_src[i] = row * RB + (col < RB ? col : 0);
+  }
+  auto copy_k_tile = [&](unsigned char* dst, int kt) __attribute__((always_inline)) {
+    static_for<KCP>([&](auto i_c) __attribute__((always_inline)) {
+      constexpr int i = decltype(i_c)::value;
+      if (cw + CW * i < KTB / 1024) lds_dma16(Kg + (size_t)kt * FA_KT * D, k_src[i], dst + 1024 * (cw + CW * i));
+    });
+  };
+  auto copy_v_tile = [&](unsigned char* dst, int kt) __attribute__((always_inline)) {
+    static_for<VCP>([&](auto i_c) __attribute__((always_inline)) {
+      constexpr int i = decltype(i_c)::value;
+      if (cw + CW * i < VTB / 1024) lds_dma16(Vg + (size_t)kt * FA_KT * D, v_src[i], dst + 1024 * (cw + CW * i));
+    });
+  };
+  // a barrier that waits for nothing of the wave's own: whoever wrote what the barrier publishes has waited before it
+  auto phase_barrier = [&]() __attribute__((always_inline)) {
+    __builtin_amdgcn_sched_barrier(0);
+    asm volatile("s_barrier" ::: "memory");
+    __builtin_amdgcn_sched_barrier(0);
+  };
+
+  const int k_lane = j * KRS + 16 * hh;
+  const int v_lane = (4 * hh + ((lane & 15) >> 2)) * VRS + 32 * ((lane >> 4) & 1) + 8 * (lane & 3);
+  const int ntiles = Skv / FA_KT;
+  using lds_v4s = __attribute__((address_space(3))) v4s;
+  typedef short v8s __attribute__((ext_vector_type(8)));
+  auto read_k = [&](const unsigned char* kbase, int s) __attribute__((always_inline)) {
+    return *reinterpret_cast<const v8h*>(kbase + 32 * s);
+  };
+  auto read_v = [&](const unsigned char* vbase, int s, int dt) __attribute__((always_inline)) {
+    const unsigned char* p0 = vbase + 16 * s * VRS + 64 * dt;
+    const v4s lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4s*)(p0));
+    const v4s hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4s*)(p0 + 8 * VRS));
+    const v8s both = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+    return __builtin_bit_cast(v8h, both);
+  };
+
+  // ---- prologue: K(0), V(0) (waves 0..3) and K(1) (waves 4..7) into LDS; scores of tile 0 from a zero start, their
+  // row maximum becomes the first reference
+  if (group == 0) {
+    copy_k_tile(Kb, 0);
+    copy_v_tile(Vb, 0);
+  } else if (ntiles > 1) {
+    copy_k_tile(Kb + KTB, 1);
+  }
+  __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
+  __syncthreads();
+  v16f sc[2], nref;   // scores of the tile's two 32-key halves, relative to the reference; minus the reference
+  v8h pf[2][2];       // their exponentials as the B operands of P V
+  {
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+#pragma unroll
+      for (int r = 0; r < 16; ++r) sc[h][r] = 0.0f;
+#pragma unroll
+      for (int s = 0; s < DS; ++s)
+        sc[h] = __builtin_amdgcn_mfma_f32_32x32x16_f16(read_k(Kb + k_lane + h * 32 * KRS, s), qf[s], sc[h], 0, 0, 0);
+    }
+    float m = sc[0][0];
+#pragma unroll
+    for (int r = 1; r < 32; ++r) m = fmaxf(m, sc[r >> 4][r & 15]);
+    m = max_with_other_half(m);
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      sc[0][r] -= m;
+      sc[1][r] -= m;
+      nref[r] = -m;
+    }
+  }
+
+  constexpr int LA = 4;          // fragments read ahead of the matrix instruction that uses them (6, 8, 12: no faster)
+  constexpr int NM = 2 * DS + 2 * 2 * DT;   // matrix instructions of an M phase: P V first, then the next tile's scores
+  constexpr int NPV = 4 * DT;
+  v8h vpre[LA];
+  int vcur = 0, vnext = VTB, vfree = 2 * VTB;   // V(t), V(t+1), and the buffer V(t+2) will go to
+  int kcur = 0, knext = KTB;                    // K(t), K(t+1)
+
+  // exponentials of the tile's scores, packed as the B operands of P V; returns this lane's share of their sum
+  auto exponentials = [&]() __attribute__((always_inline)) {
+    float psum0 = 0.0f, psum1 = 0.0f;
+#pragma unroll
+    for (int h = 0; h < 2; ++h)
+#pragma unroll
+      for (int e = 0; e < 16; e += 2) {
+        const float p0 = __builtin_amdgcn_exp2f(sc[h][e]), p1 = __builtin_amdgcn_exp2f(sc[h][e + 1]);
+        psum0 += p0;
+        psum1 += p1;
+        const v2h pp = {(_Float16)p0, (_Float16)p1};
+        pf[h][e / 8][e % 8] = pp[0];
+        pf[h][e / 8][e % 8 + 1] = pp[1];
+      }
+    return psum0 + psum1;
+  };
+  // The reference maximum is not tracked tile by tile: the scores are exponentiated against the reference as it is,
+  // and only when a lane's sum of exponentials says that one of them may not fit fp16 (or came out infinite) are the
+  // row maxima taken, the reference moved up to them, O and the row sums rescaled, and the tile exponentiated again.
+  // Any reference gives the same O = acc / l; with this one p ranges up to 2^15.  What the common path saves against a
+  // maximum per tile is sixteen v_max3, the exchange with the other half-wave and their share of the issue slots that
+  // the other wave's matrix instructions need.
+  auto phase_s = [&](int t) __attribute__((always_inline)) {
+    if (group == 0) {
+      if (t + 1 < ntiles) copy_v_tile(Vb + vnext, t + 1);
+    } else {
+      if (t + 2 < ntiles) copy_k_tile(Kb + kcur, t + 2);   // K(t) was last read in the slot before this one
+    }
+    const unsigned char* v0 = Vb + vcur + v_lane;
+#pragma unroll
+    for (int i = 0; i < LA; ++i) vpre[i] = read_v(v0, i / DT, i % DT);
+    float psum = exponentials();
+    if (__builtin_expect(__builtin_amdgcn_ballot_w64(!(psum <= FA_PMAX)) != 0, 0)) {
+      // v_max3 as assembly: fmaxf would first quieten each operand with a v_max of its own
+      float m;
+      asm("v_max3_f32 %0, %1, %2, %3" : "=v"(m) : "v"(sc[0][0]), "v"(sc[0][1]), "v"(sc[1][0]));
+      asm("v_max3_f32 %0, %0, %1, %2" : "+v"(m) : "v"(sc[1][1]), "v"(sc[0][2]));
+      asm("v_max3_f32 %0, %0, %1, %2" : "+v"(m) : "v"(sc[1][2]), "v"(sc[0][3]));
+      asm("v_max3_f32 %0, %0, %1, %2" : "+v"(m) : "v"(sc[1][3]), "v"(sc[0][4]));
+#pragma unroll
+      for (int r = 4; r < 16; r += 2) {
+        asm("v_max3_f32 %0, %0, %1, %2" : "+v"(m) : "v"(sc[1][r]), "v"(sc[1][r + 1]));
+        if (r + 2 < 16) asm("v_max3_f32 %0, %0, %1, %2" : "+v"(m) : "v"(sc[0][r + 1]), "v"(sc[0][r + 2]));
+      }
+      asm("v_max3_f32 %0, %0, %1, %2" : "+v"(m) : "v"(sc[0][15]), "v"(sc[0][15]));
+      m = max_with_other_half(m);   // both lanes of a row move by the same amount
+      const float delta = m > 0.0f ? -m : 0.0f;
+      const float alpha = __builtin_amdgcn_exp2f(delta);
+      l_run *= alpha;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        nref[r] += delta;
+        sc[0][r] += delta;
+        sc[1][r] += delta;
+      }
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) oacc[dt][r] *= alpha;
+      psum = exponentials();
+    }
+    l_run += psum;
+  };
+
+  auto phase_m = [&](auto next_c) __attribute__((always_inline)) {
+    constexpr bool has_next = decltype(next_c)::value;
+    constexpr int N = has_next ? NM : NPV;
+    const unsigned char* v0 = Vb + vcur + v_lane;
+    const unsigned char* k1 = Kb + knext + k_lane;
+    v8h fr[NM];
+#pragma unroll
+    for (int i = 0; i < LA; ++i) fr[i] = vpre[i];
+    __builtin_amdgcn_s_setprio(3);
+    __builtin_amdgcn_sched_barrier(0);
+    static_for<N>([&](auto i_c) __attribute__((always_inline)) {
+      constexpr int i = decltype(i_c)::value;
+      if constexpr (i < NPV) {          // half h of the tile, contraction step s of the half, d tile dt
+        constexpr int h = i / (2 * DT), s = (i % (2 * DT)) / DT, dt = i % DT;
+        oacc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fr[i], pf[h][s], oacc[dt], 0, 0, 0);
+      } else {                          // the two halves' score chains take turns
+        constexpr int ii = i - NPV, s = ii / 2, h = ii % 2;
+        sc[h] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fr[i], qf[s], s == 0 ? nref : sc[h], 0, 0, 0);
+      }
+      if constexpr (i + LA < N) {
+        constexpr int n = i + LA;
+        if constexpr (n < NPV) {
+          fr[n] = read_v(v0 + (n / (2 * DT)) * 32 * VRS, (n % (2 * DT)) / DT, n % DT);
+        } else {
+          fr[n] = read_k(k1 + ((n - NPV) % 2) * 32 * KRS, (n - NPV) / 2);
+        }
+      }
+      __builtin_amdgcn_sched_barrier(0);
+    });
+    __builtin_amdgcn_s_setprio(0);
+  };
+  auto rotate = [&]() __attribute__((always_inline)) {
+    int x = vcur;
+    vcur = vnext;
+    vnext = vfree;
+    vfree = x;
+    x = kcur;
+    kcur = knext;
+    knext = x;
+  };
+
+  auto stamp = [&](int kt, int slot) __attribute__((always_inline)) {
+    if constexpr (TRACE) {
+      if (blockIdx.x == 0 && tid == 64 * trace_wave && kt < FA_TRACE_TILES) trace[kt * 6 + slot] = wall_clock64();
+    }
+  };
+  if (group == 1) phase_barrier();
+  for (int t = 0; t + 1 < ntiles; ++t) {
+    stamp(t, 0);
+    phase_s(t);
+    stamp(t, 1);
+    phase_barrier();
+    stamp(t, 2);
+    phase_m(std::true_type{});
+    stamp(t, 3);
+    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): the copies this wave requested in S(t)
+    stamp(t, 4);
+    phase_barrier();
+    stamp(t, 5);
+    rotate();
+  }
+  phase_s(ntiles - 1);
+  phase_barrier();
+  phase_m(std::false_type{});
+  phase_barrier();
+  if (group == 0) phase_barrier();
+
+  // ---- normalise and store: the wave turns its 32 x D tile round through LDS (nobody reads tiles any more) and
+  // stores whole rows, 1 KB of consecutive bytes per instruction
+  constexpr int ORS = 2 * D + 16;
+  constexpr int LPR = D / 8;
+  unsigned char* const ot = smem + wave * (32 * ORS);
+  const float l = l_run + __shfl_xor(l_run, 32);
+  const float inv = 1.0f / l;
+#pragma unroll
+  for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+      const v2h lo = {(_Float16)(oacc[dt][4 * g] * inv), (_Float16)(oacc[dt][4 * g + 1] * inv)};
+      const v2h hi = {(_Float16)(oacc[dt][4 * g + 2] * inv), (_Float16)(oacc[dt][4 * g + 3] * inv)};
+      *reinterpret_cast<v2u*>(ot + j * ORS + 2 * (32 * dt + 8 * g + 4 * hh)) =
+          v2u{__builtin_bit_cast(unsigned, lo), __builtin_bit_cast(unsigned, hi)};
+    }
+#pragma unroll
+  for (int idx = lane; idx < 32 * LPR; idx += 64) {
+    const int r = idx / LPR, c = idx - r * LPR;
+    const v4u piece = *reinterpret_cast<const v4u*>(ot + r * ORS + 16 * c);
+    const int row = q_base + r;
+    if (row < Sq) __builtin_nontemporal_store(piece, reinterpret_cast<v4u*>(Og + (size_t)row * D + 8 * c));
+  }
+}
+
+template <int D>
+static int launch_fa_pp(const void* Q, const void* K, const void* V, void* O, int BH, int Sq, int Skv, float scale,
+                        int lds_max, hipStream_t s) {
+  const size_t tiles = (size_t)2 * FaLayout<D>::KTB + (size_t)3 * FaLayout<D>::VTB;
+  const size_t lds = std::max(tiles, (size_t)8 * 32 * (2 * D + 16));   // the O tiles of the eight waves go where the K / V tiles were
+  if ((int)lds > lds_max) return fail(FTK_ERR_UNSUPPORTED_SHAPE, "ftk_flash_attn_f16: needs %zu bytes of LDS", lds);
+  static bool attr_set = false;
+  if (!attr_set) {
+    FTK_HIP(hipFuncSetAttribute((const void*)flash_attn_pp_kernel<D, false>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+#ifdef FTK_DEBUG_TRACE
+    FTK_HIP(hipFuncSetAttribute((const void*)flash_attn_pp_kernel<D, true>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+#endif
+    attr_set = true;
+  }
+  const int nqb = (Sq + 255) / 256;
+  const long long total = (long long)nqb * BH;
+  if (total > 0x7fffffffLL) return fail(FTK_ERR_UNSUPPORTED_SHAPE, "ftk_flash_attn_f16: grid too large");
+#ifdef FTK_DEBUG_TRACE
+  if (long long* trace = fa_trace_ptr()) {
+    hipLaunchKernelGGL((flash_attn_pp_kernel<D, true>), dim3((unsigned)total), dim3(512), lds, s, (const _Float16*)Q,
+                       (const _Float16*)K, (const _Float16*)V, (_Float16*)O, Sq, Skv, scale * 1.4426950408889634f, nqb,
+                       trace, fa_trace_wave());
+    return check_launch("flash_attn_pp_kernel");
+  }
+#endif
+  hipLaunchKernelGGL((flash_attn_pp_kernel<D, false>), dim3((unsigned)total), dim3(512), lds, s, (const _Float16*)Q,
+                     (const _Float16*)K, (const _Float16*)V, (_Float16*)O, Sq, Skv, scale * 1.4426950408889634f, nqb,
+                     (long long*)nullptr, 0);
+  return check_launch("flash_attn_pp_kernel");
+}
+
+
 template <int D, int QT, int WAVES, int MINB>
 static int launch_fa(const void* Q, const void* K, const void* V, void* O, int BH, int Sq, int Skv, float scale,
                      int lds_max, hipStream_t s) {
@@ -648,12 +990,18 @@ extern "C" int ftk_flash_attn_f16(const void* Q, const void* K, const void* V, v
   int variant = fa_variant_override();
   if (variant == 0) variant = (long long)((Sq + 255) / 256) * bh >= dp->cus ? 3 : 1;
   const int lds = dp->lds_optin;
+  // Whole key tiles at D = 128 / 96 with enough query blocks take the kernel whose two waves per SIMD alternate between
+  // matrix and vector phases (B8 H16 S2048: 256-262 us against 291-297 at D = 128, 219 against 234 at D = 96; at D = 64
+  // the two measure the same, 183-189 us, and at D = 32, where a tile has eight matrix instructions for the same
+  // vector work, the interleaved kernel wins, 120 against 139 us).
   if (D == 128) {
     if (variant == 1) return launch_fa<128, 1, 4, 1>(Q, K, V, O, (int)bh, Sq, Skv, scale, lds, s);
+    if (Skv % FA_KT == 0) return launch_fa_pp<128>(Q, K, V, O, (int)bh, Sq, Skv, scale, lds, s);
     return launch_fa<128, 1, 8, 1>(Q, K, V, O, (int)bh, Sq, Skv, scale, lds, s);
   }
   if (D == 96) {
     if (variant == 1) return launch_fa<96, 1, 4, 1>(Q, K, V, O, (int)bh, Sq, Skv, scale, lds, s);
+    if (Skv % FA_KT == 0) return launch_fa_pp<96>(Q, K, V, O, (int)bh, Sq, Skv, scale, lds, s);
     return launch_fa<96, 1, 8, 1>(Q, K, V, O, (int)bh, Sq, Skv, scale, lds, s);
   }
   if (D == 64) {

@@ -761,6 +761,30 @@ def test_flash_attention(core, B, Hd, Sq, Skv, D):
         assert ko.max_rel_err(O.reshape(-1, Sq, D), Oc) <= F16_TOL
 
 
+@pytest.mark.parametrize('step', [3.0, 20.0, 200.0])
+def test_flash_attention_scores_that_climb_from_tile_to_tile(core, step):
+    """Keys whose scores grow by `step` (natural-log units) from one 64-key tile to the next, so the running maximum of
+    every row has to move again and again: by a little (exponentials stay in range), by more than fp16 holds, and by
+    more than fp32 exponentials hold.  Sizes are such that the eight-wave kernels for whole tiles run."""
+    B, Hd, S, D = 4, 32, 512, 128
+    rng = np.random.default_rng(21)
+    u = rng.standard_normal(D)
+    u /= np.linalg.norm(u)
+    Q = (rng.standard_normal((B, Hd, S, D)) * 0.3 + 4.0 * u).astype(np.float16)
+    ramp = step * (np.arange(S) // 64) / 4.0          # q . k grows by about `step` per tile (|q . u| is about 4)
+    K = (rng.standard_normal((B, Hd, S, D)) * 0.3 + ramp[None, None, :, None] * u).astype(np.float16)
+    V = rng.standard_normal((B, Hd, S, D)).astype(np.float16)
+    O = core.flash_attention(dev(Q), dev(K), dev(V), 1.0).cpu().numpy()
+    assert np.isfinite(O).all()
+    for (b, h) in [(0, 0), (1, 17), (3, 31)]:
+        ref = ko.attention(Q[b, h], K[b, h], V[b, h], 1.0, dtype=np.float64)
+        assert ko.max_rel_err(O[b, h], ref) <= F16_TOL
+    # and with the keys in the opposite order: the first tile sets a reference nothing later reaches
+    Kr, Vr = np.ascontiguousarray(K[:, :, ::-1]), np.ascontiguousarray(V[:, :, ::-1])
+    Or = core.flash_attention(dev(Q), dev(Kr), dev(Vr), 1.0).cpu().numpy()
+    assert ko.max_rel_err(Or[1, 17], ko.attention(Q[1, 17], Kr[1, 17], Vr[1, 17], 1.0, dtype=np.float64)) <= F16_TOL
+
+
 def test_flash_attention_uniform_keys_give_mean_of_values(core):
     B, Hd, S, D = 1, 2, 192, 128
     rng = np.random.default_rng(8)
