@@ -801,12 +801,37 @@ def bench_lstm_f32_streamed(torch, core, steps, warmup, cpu, H):
     return res
 
 
+def probe_mfma_rate():
+    """What the matrix pipes deliver under load: runs the stand-alone probe fractaltensor_amd/mfma_rate (built by
+    `make probes` / __graft_entry__.build()) as a child process and reports the fp16 MFMA rate it holds on random
+    operands, the figure the fractions of the nominal peak on the other lines have to be read against."""
+    import re
+    import subprocess
+    exe = os.path.join(os.path.dirname(os.path.abspath(__file__)), 'fractaltensor_amd', 'mfma_rate')
+    if not os.path.exists(exe):
+        raise SystemExit('bench.py --workload mfma_rate: fractaltensor_amd/mfma_rate is not built (make -C fractaltensor_amd/csrc probes)')
+    out = subprocess.run([exe], capture_output=True, text=True, timeout=120, check=True).stdout
+    alone = {}
+    for ln in out.splitlines():
+        m = re.match(r'mfma alone, (.+?)\s+([\d.]+) ns per MFMA\s+([\d.]+) clocks per MFMA\s+([\d.]+) GHz\s+->\s+(\d+) TFLOP/s', ln)
+        if m:
+            alone[m.group(1).strip()] = {'ns_per_mfma': float(m.group(2)), 'clocks_per_mfma': float(m.group(3)),
+                                         'ghz': float(m.group(4)), 'tflops': float(m.group(5))}
+    real = alone['random operands, 8 x 4 in turn']
+    return {'metric': 'fp16 MFMA rate held on random operands (register-only v_mfma_f32_32x32x16_f16, one wave per SIMD)',
+            'value': real['tflops'], 'unit': 'TFLOP/s', 'n_gpus': 1, 'steps': 3, 'warmup': 1, 'ms_per_step': 4000 * 32 * real['ns_per_mfma'] * 1e-6,
+            'higher_is_better': True, 'scaling': 'weak', 'vs_baseline': None, 'dtype': 'f16', 'data': 'synthetic',
+            'config': {'workload': 'matrix-pipe probe: 4000 x 32 MFMAs per wave, 1024 waves'},
+            'roofline': {'bound': 'mfma', 'achieved': real['tflops'], 'peak': 2500.0, 'unit': 'TFLOP/s', 'frac': real['tflops'] / 2500.0, 'traffic': None},
+            'cpu_baseline': None, 'mfma_alone': alone}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument('--gpus', type=int, default=1)
     ap.add_argument('--steps', type=int, default=50)
     ap.add_argument('--warmup', type=int, default=10)
-    ap.add_argument('--workload', default='b2b', choices=['b2b', 'config1', 'attention', 'stacked_lstm', 'dilated_lstm', 'lstm_f16_h256', 'lstm_f16_h512', 'lstm_f16_h1024', 'lstm_f32_h512', 'lstm_f32_h1024', 'gemm', 'online_softmax', 'embedding', 'grid_rnn', 'windowed_attention', 'b2b_ref_shapes', 'copy'])
+    ap.add_argument('--workload', default='b2b', choices=['b2b', 'config1', 'attention', 'stacked_lstm', 'dilated_lstm', 'lstm_f16_h256', 'lstm_f16_h512', 'lstm_f16_h1024', 'lstm_f32_h512', 'lstm_f32_h1024', 'gemm', 'online_softmax', 'embedding', 'grid_rnn', 'windowed_attention', 'b2b_ref_shapes', 'copy', 'mfma_rate'])
     ap.add_argument('--no-extras', action='store_true', help='measure only the chosen workload')
     ap.add_argument('--all', action='store_true', help='also the workloads either side of the path (fp16 / larger stacks, GEMM, softmax, embedding, grid RNN, windowed attention)')
     ap.add_argument('--no-cpu', action='store_true', help='skip the CPU baseline leg')
@@ -817,6 +842,10 @@ def main():
         print('bench.py measures one GPU: every workload here is a single-device kernel '
               '(independent problems / heads / batch rows; no collectives). Run with --gpus 1.', file=sys.stderr)
         sys.exit(2)
+
+    if args.workload == 'mfma_rate':
+        print(json.dumps(probe_mfma_rate()))
+        return
 
     import torch
     import fractaltensor_amd._core as core   # raises if libftkernels.so is missing: no fallback
