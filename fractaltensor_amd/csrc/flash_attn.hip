@@ -37,7 +37,7 @@
 // row sums use plain adds, and the loop is software pipelined per 32-key half
 // tile with the instruction order written out and fenced step by step.
 //
-// flash_attn_pp_kernel (whole key tiles, D = 128 / 96) orders the same work differently: the two waves of a SIMD
+// flash_attn_pp_kernel (D = 128 / 96, enough query blocks for 8 waves) orders the same work differently: the two waves of a SIMD
 // alternate between a phase of matrix instructions only and a phase of vector instructions only, in opposite phases,
 // and the running maximum is moved only when a sum of exponentials says it must (see the comment at the kernel).
 #include <stdlib.h>
@@ -566,8 +566,8 @@ static long long* fa_trace_ptr() {
 }
 #endif
 
-// The same product with the two waves of a SIMD kept in opposite phases (whole key tiles only, 8 waves x 32 query
-// rows).  A wave alternates between a phase of matrix instructions only -- M(t): O^T += V(t)^T P(t)^T, then the
+// The same product with the two waves of a SIMD kept in opposite phases (8 waves x 32 query rows; RAG: the key
+// length is no multiple of the tile, the tail of the last tile is masked).  A wave alternates between a phase of matrix instructions only -- M(t): O^T += V(t)^T P(t)^T, then the
 // scores of tile t+1 -- and a phase of vector instructions only -- S(t): row maximum, exponentials, row sum and
 // packing of tile t's scores -- with a workgroup barrier after every phase.  Waves 4..7 run one phase behind waves
 // 0..3 (they pass one barrier more before the loop, the others one more after it), and wave w + 4 shares its SIMD
@@ -577,7 +577,7 @@ static long long* fa_trace_ptr() {
 // Tiles: K(t+1) and V(t) are read during M(t), i.e. in two consecutive phase slots.  K has two buffers, V three:
 // waves 0..3 request V(t+1) at the start of S(t), waves 4..7 request K(t+2) at the start of their S(t), and each
 // waits for its own copies before the barrier that ends its following M phase, one slot before the first reader.
-template <int D, bool TRACE>
+template <int D, bool TRACE, bool RAG>
 __global__ __launch_bounds__(512, 1) void flash_attn_pp_kernel(const _Float16* __restrict__ Q,
                                                                 const _Float16* __restrict__ K,
                                                                 const _Float16* __restrict__ V,
@@ -640,16 +640,27 @@ __global__ __launch_bounds__(512, 1) void flash_attn_pp_kernel(const _Float16* _
     const int row = min(x / VRS, FA_KT - 1), col = x % VRS;
     v_src[i] = row * RB + (col < RB ? col : 0);
   }
+  // RAG (Skv no multiple of the tile): rows of the last tile past the end re-read the last key; their scores are masked
+  auto ragged_off = [&](unsigned off, int kt) __attribute__((always_inline)) {
+    if constexpr (RAG) {
+      const int key0 = kt * FA_KT;
+      if (key0 + FA_KT > Skv) {
+        const unsigned last = (unsigned)(Skv - 1 - key0), row = off / RB;
+        if (row > last) off -= (row - last) * RB;
+      }
+    }
+    return off;
+  };
   auto copy_k_tile = [&](unsigned char* dst, int kt) __attribute__((always_inline)) {
     static_for<KCP>([&](auto i_c) __attribute__((always_inline)) {
       constexpr int i = decltype(i_c)::value;
-      if (cw + CW * i < KTB / 1024) lds_dma16(Kg + (size_t)kt * FA_KT * D, k_src[i], dst + 1024 * (cw + CW * i));
+      if (cw + CW * i < KTB / 1024) lds_dma16(Kg + (size_t)kt * FA_KT * D, ragged_off(k_src[i], kt), dst + 1024 * (cw + CW * i));
     });
   };
   auto copy_v_tile = [&](unsigned char* dst, int kt) __attribute__((always_inline)) {
     static_for<VCP>([&](auto i_c) __attribute__((always_inline)) {
       constexpr int i = decltype(i_c)::value;
-      if (cw + CW * i < VTB / 1024) lds_dma16(Vg + (size_t)kt * FA_KT * D, v_src[i], dst + 1024 * (cw + CW * i));
+      if (cw + CW * i < VTB / 1024) lds_dma16(Vg + (size_t)kt * FA_KT * D, ragged_off(v_src[i], kt), dst + 1024 * (cw + CW * i));
     });
   };
   // a barrier that waits for nothing of the wave's own: whoever wrote what the barrier publishes has waited before it
@@ -661,7 +672,19 @@ __global__ __launch_bounds__(512, 1) void flash_attn_pp_kernel(const _Float16* _
 
   const int k_lane = j * KRS + 16 * hh;
   const int v_lane = (4 * hh + ((lane & 15) >> 2)) * VRS + 32 * ((lane >> 4) & 1) + 8 * (lane & 3);
-  const int ntiles = Skv / FA_KT;
+  const int ntiles = (Skv + FA_KT - 1) / FA_KT;
+  // scores of keys past the end of a ragged last tile: minus infinity, so they exponentiate to zero and no maximum sees them
+  auto mask_tail = [&](v16f (&sv)[2], int kt) __attribute__((always_inline)) {
+    if constexpr (RAG) {
+      if ((kt + 1) * FA_KT > Skv) {
+#pragma unroll
+        for (int h = 0; h < 2; ++h)
+#pragma unroll
+          for (int r = 0; r < 16; ++r)
+            if (kt * FA_KT + 32 * h + 8 * (r >> 2) + 4 * hh + (r & 3) >= Skv) sv[h][r] = -INFINITY;
+      }
+    }
+  };
   using lds_v4s = __attribute__((address_space(3))) v4s;
   typedef short v8s __attribute__((ext_vector_type(8)));
   auto read_k = [&](const unsigned char* kbase, int s) __attribute__((always_inline)) {
@@ -696,6 +719,7 @@ __global__ __launch_bounds__(512, 1) void flash_attn_pp_kernel(const _Float16* _
       for (int s = 0; s < DS; ++s)
         sc[h] = __builtin_amdgcn_mfma_f32_32x32x16_f16(read_k(Kb + k_lane + h * 32 * KRS, s), qf[s], sc[h], 0, 0, 0);
     }
+    mask_tail(sc, 0);
     float m = sc[0][0];
 #pragma unroll
     for (int r = 1; r < 32; ++r) m = fmaxf(m, sc[r >> 4][r & 15]);
@@ -746,6 +770,7 @@ __global__ __launch_bounds__(512, 1) void flash_attn_pp_kernel(const _Float16* _
     const unsigned char* v0 = Vb + vcur + v_lane;
 #pragma unroll
     for (int i = 0; i < LA; ++i) vpre[i] = read_v(v0, i / DT, i % DT);
+    mask_tail(sc, t);
     float psum = exponentials();
     if (__builtin_expect(__builtin_amdgcn_ballot_w64(!(psum <= FA_PMAX)) != 0, 0)) {
       // v_max3 as assembly: fmaxf would first quieten each operand with a v_max of its own
@@ -879,9 +904,10 @@ static int launch_fa_pp(const void* Q, const void* K, const void* V, void* O, in
   if ((int)lds > lds_max) return fail(FTK_ERR_UNSUPPORTED_SHAPE, "ftk_flash_attn_f16: needs %zu bytes of LDS", lds);
   static bool attr_set = false;
   if (!attr_set) {
-    FTK_HIP(hipFuncSetAttribute((const void*)flash_attn_pp_kernel<D, false>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+    FTK_HIP(hipFuncSetAttribute((const void*)flash_attn_pp_kernel<D, false, false>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+    FTK_HIP(hipFuncSetAttribute((const void*)flash_attn_pp_kernel<D, false, true>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
 #ifdef FTK_DEBUG_TRACE
-    FTK_HIP(hipFuncSetAttribute((const void*)flash_attn_pp_kernel<D, true>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+    FTK_HIP(hipFuncSetAttribute((const void*)flash_attn_pp_kernel<D, true, true>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
 #endif
     attr_set = true;
   }
@@ -890,15 +916,20 @@ static int launch_fa_pp(const void* Q, const void* K, const void* V, void* O, in
   if (total > 0x7fffffffLL) return fail(FTK_ERR_UNSUPPORTED_SHAPE, "ftk_flash_attn_f16: grid too large");
 #ifdef FTK_DEBUG_TRACE
   if (long long* trace = fa_trace_ptr()) {
-    hipLaunchKernelGGL((flash_attn_pp_kernel<D, true>), dim3((unsigned)total), dim3(512), lds, s, (const _Float16*)Q,
+    hipLaunchKernelGGL((flash_attn_pp_kernel<D, true, true>), dim3((unsigned)total), dim3(512), lds, s, (const _Float16*)Q,
                        (const _Float16*)K, (const _Float16*)V, (_Float16*)O, Sq, Skv, scale * 1.4426950408889634f, nqb,
                        trace, fa_trace_wave());
     return check_launch("flash_attn_pp_kernel");
   }
 #endif
-  hipLaunchKernelGGL((flash_attn_pp_kernel<D, false>), dim3((unsigned)total), dim3(512), lds, s, (const _Float16*)Q,
-                     (const _Float16*)K, (const _Float16*)V, (_Float16*)O, Sq, Skv, scale * 1.4426950408889634f, nqb,
-                     (long long*)nullptr, 0);
+  if (Skv % FA_KT)
+    hipLaunchKernelGGL((flash_attn_pp_kernel<D, false, true>), dim3((unsigned)total), dim3(512), lds, s, (const _Float16*)Q,
+                       (const _Float16*)K, (const _Float16*)V, (_Float16*)O, Sq, Skv, scale * 1.4426950408889634f, nqb,
+                       (long long*)nullptr, 0);
+  else
+    hipLaunchKernelGGL((flash_attn_pp_kernel<D, false, false>), dim3((unsigned)total), dim3(512), lds, s, (const _Float16*)Q,
+                       (const _Float16*)K, (const _Float16*)V, (_Float16*)O, Sq, Skv, scale * 1.4426950408889634f, nqb,
+                       (long long*)nullptr, 0);
   return check_launch("flash_attn_pp_kernel");
 }
 
@@ -990,18 +1021,19 @@ extern "C" int ftk_flash_attn_f16(const void* Q, const void* K, const void* V, v
   int variant = fa_variant_override();
   if (variant == 0) variant = (long long)((Sq + 255) / 256) * bh >= dp->cus ? 3 : 1;
   const int lds = dp->lds_optin;
-  // Whole key tiles at D = 128 / 96 with enough query blocks take the kernel whose two waves per SIMD alternate between
+  static const bool interleaved_only = getenv("FTK_FA_INTERLEAVED") != nullptr;   // tuning hook: the older kernel for every shape
+  // D = 128 / 96 with enough query blocks take the kernel whose two waves per SIMD alternate between
   // matrix and vector phases (B8 H16 S2048: 256-262 us against 291-297 at D = 128, 219 against 234 at D = 96; at D = 64
   // the two measure the same, 183-189 us, and at D = 32, where a tile has eight matrix instructions for the same
   // vector work, the interleaved kernel wins, 120 against 139 us).
   if (D == 128) {
     if (variant == 1) return launch_fa<128, 1, 4, 1>(Q, K, V, O, (int)bh, Sq, Skv, scale, lds, s);
-    if (Skv % FA_KT == 0) return launch_fa_pp<128>(Q, K, V, O, (int)bh, Sq, Skv, scale, lds, s);
+    if (!interleaved_only) return launch_fa_pp<128>(Q, K, V, O, (int)bh, Sq, Skv, scale, lds, s);
     return launch_fa<128, 1, 8, 1>(Q, K, V, O, (int)bh, Sq, Skv, scale, lds, s);
   }
   if (D == 96) {
     if (variant == 1) return launch_fa<96, 1, 4, 1>(Q, K, V, O, (int)bh, Sq, Skv, scale, lds, s);
-    if (Skv % FA_KT == 0) return launch_fa_pp<96>(Q, K, V, O, (int)bh, Sq, Skv, scale, lds, s);
+    if (!interleaved_only) return launch_fa_pp<96>(Q, K, V, O, (int)bh, Sq, Skv, scale, lds, s);
     return launch_fa<96, 1, 8, 1>(Q, K, V, O, (int)bh, Sq, Skv, scale, lds, s);
   }
   if (D == 64) {

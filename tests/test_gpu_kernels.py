@@ -749,6 +749,9 @@ def fa_inputs(seed, B, Hd, Sq, Skv, D):
     (4, 16, 512, 512, 32),     # enough query blocks for the eight-wave variant
     (2, 3, 200, 333, 96),      # D 96: three d tiles, V rows padded by 128 bytes
     (4, 16, 512, 256, 96),
+    (4, 32, 512, 500, 128),    # eight-wave kernels with a ragged last key tile
+    (4, 32, 500, 65, 96),      # ... whose last tile holds one key; ragged queries too
+    (4, 32, 512, 40, 128),     # ... a single, ragged tile
 ])
 def test_flash_attention(core, B, Hd, Sq, Skv, D):
     Q, K, V = fa_inputs(4, B, Hd, Sq, Skv, D)
