@@ -190,7 +190,8 @@ constexpr int P_TILE = 32 * P_LD;  // floats per LDS buffer
 constexpr int kStageRow32 = 144, kStageRow16 = 80;
 constexpr int kStageC = 0, kStageH = 32 * kStageRow32, kStageTop = 2 * 32 * kStageRow32, kStageRest = kStageTop + 32 * kStageRow16;
 constexpr int kStageBytes = kStageRest + 32 * kStageRow16;
-constexpr size_t kPersistLds = (size_t)2 * P_TILE * sizeof(float) + 1024 + 2 * kStageBytes;  // tiles, prefetch scrap, staging
+constexpr int kRatioOffset = 2 * P_TILE * (int)sizeof(float) + 1024 + 2 * kStageBytes;   // bytes; [2 tile buffers][64 floats]
+constexpr size_t kPersistLds = (size_t)kRatioOffset + 2 * 64 * sizeof(float);  // tiles, prefetch scrap, staging, row ratios
 // Kernel flavours.  kProductsF32 / kProductsSplit: fp32 data, H = 256, the two ways of forming the products.
 // kHalfData: fp16 inputs, weights, h and c (what the reference's CuTe LSTM stores), one fp16 MFMA per product
 // with fp32 accumulation, H = 512: a row of 512 fp16 takes the 1024 bytes a row of 256 fp32 takes, and a
@@ -401,6 +402,13 @@ void lstm_persistent_kernel(PersistArgs a) {
       return;
     }
     const unsigned lds0 = tile_lds + 4u * (unsigned)(buf * P_TILE + 8 * wave_u * P_LD);
+    // Split products, first layer: the 32 rows' ratios (see load_ratio) travel with the x columns, into LDS, instead of
+    // being loaded into a register: a register load that late in an item is waited for behind the copies of the
+    // tile after next, which nothing else waits for before the item's end.
+    if constexpr (SPLIT) {
+      if (l == 0 && with_x && wave_u == 0)
+        lds_dma4(a.xratio + (size_t)t * B, 4u * (unsigned)min(rb * 32 + (lane & 31), B - 1), tile_lds + (unsigned)kRatioOffset + 256u * (unsigned)buf);
+    }
     if (row0 + 8 <= B) {
       const char* xb = xsrc + (size_t)row0 * 1024;
       if (with_x) {
@@ -537,9 +545,10 @@ void lstm_persistent_kernel(PersistArgs a) {
   // split mode, first layer: the x rows carry a scale of their own; before the h
   // products join the same accumulators the x products move to h's scale (a
   // power of two: exact)
-  auto load_ratio = [&](int n) __attribute__((always_inline)) -> float {
+  // the ratio of this lane's row in the tile that has landed in buffer buf
+  auto load_ratio = [&](int buf) __attribute__((always_inline)) -> float {
     if constexpr (SPLIT) {
-      if (l == 0 && live(n)) return a.xratio[(size_t)item_t(n) * B + min(item_rb(n) * 32 + j, B - 1)];
+      if (l == 0) return reinterpret_cast<const float*>(reinterpret_cast<const unsigned char*>(tile) + kRatioOffset)[64 * buf + j];
     }
     return 1.0f;
   };
@@ -713,13 +722,12 @@ void lstm_persistent_kernel(PersistArgs a) {
         }
       }
       const float4 cp = load_cprev(n);
-      const float ratio_next = (xnext && SPLIT) ? load_ratio(n + 1) : 1.0f;
       __builtin_amdgcn_s_waitcnt(0);
       __syncthreads();
       if (live(n)) {
         if (!xdone) {
           mfma_range(buf, IC<0>{}, IC<0>{}, IC<16>{});
-          rescale_x(load_ratio(n));
+          rescale_x(load_ratio(buf));
         }
         if (item_t(n) >= d) mfma_range(buf, IC<1>{}, IC<0>{}, IC<16>{});
         epilogue_to_lds(gate_sums(), cp, 0);
@@ -729,7 +737,7 @@ void lstm_persistent_kernel(PersistArgs a) {
       xdone = false;
       if (xnext) {          // while the stores are acknowledged
         mfma_range(buf ^ 1, IC<0>{}, IC<0>{}, IC<16>{});
-        rescale_x(ratio_next);
+        rescale_x(load_ratio(buf ^ 1));
         xdone = true;
       }
       xhere = xnext;
@@ -766,7 +774,6 @@ void lstm_persistent_kernel(PersistArgs a) {
   alive = wait_deps(0);
   if (alive) issue_tile(0, 0);
   float4 cp = load_cprev(0);
-  float ratio = load_ratio(0);
   __builtin_amdgcn_s_waitcnt(0);
   __syncthreads();
 
@@ -777,6 +784,7 @@ void lstm_persistent_kernel(PersistArgs a) {
     const int buf = n & 1;
     if (tracing) a.trace[TS * n + 0] = wall_clock64();
     const bool has_prev = item_t(n) >= d;
+    const float ratio = load_ratio(buf);   // tile n has landed (the barrier that ended the item before)
     int looks = 0;  // looks taken inside the item (for the trace)
     if (pending) fl = request_flags(n + 1);
 
@@ -840,10 +848,7 @@ void lstm_persistent_kernel(PersistArgs a) {
     store_item(n, buf);
     counted = false;
     if (tracing) a.trace[TS * n + 6] = wall_clock64();
-    if (n + 1 < n_items) {
-      cp = load_cprev(n + 1);
-      ratio = load_ratio(n + 1);
-    }
+    if (n + 1 < n_items) cp = load_cprev(n + 1);
     if (pending2 && !pending && flags_ready(fl2)) {
       issue_tile(n + 2, buf);
       pending2 = false;
