@@ -752,6 +752,8 @@ def fa_inputs(seed, B, Hd, Sq, Skv, D):
     (4, 32, 512, 500, 128),    # eight-wave kernels with a ragged last key tile
     (4, 32, 500, 65, 96),      # ... whose last tile holds one key; ragged queries too
     (4, 32, 512, 40, 128),     # ... a single, ragged tile
+    (4, 32, 512, 64, 128),     # ... a single whole tile
+    (4, 32, 512, 256, 96),     # D 96 on the eight-wave kernel for whole tiles
 ])
 def test_flash_attention(core, B, Hd, Sq, Skv, D):
     Q, K, V = fa_inputs(4, B, Hd, Sq, Skv, D)
