@@ -37,7 +37,7 @@
 // row sums are packed fp16 adds over the rounded exponentials, and the loop is software pipelined per 32-key half
 // tile with the instruction order written out and fenced step by step.
 //
-// flash_attn_pp_kernel (D = 128 / 96, enough query blocks for 8 waves) orders the same work differently: the two waves of a SIMD
+// flash_attn_pp_kernel (enough query blocks for 8 waves) orders the same work differently: the two waves of a SIMD
 // alternate between a phase of matrix instructions only and a phase of vector instructions only, in opposite phases,
 // and the running maximum is moved only when a sum of exponentials says it must (see the comment at the kernel).
 #include <stdlib.h>
@@ -1037,10 +1037,10 @@ extern "C" int ftk_flash_attn_f16(const void* Q, const void* K, const void* V, v
   if (variant == 0) variant = (long long)((Sq + 255) / 256) * bh >= dp->cus ? 3 : 1;
   const int lds = dp->lds_optin;
   static const bool interleaved_only = getenv("FTK_FA_INTERLEAVED") != nullptr;   // tuning hook: the older kernel for every shape
-  // D = 128 / 96 with enough query blocks take the kernel whose two waves per SIMD alternate between
-  // matrix and vector phases (B8 H16 S2048: 256-262 us against 291-297 at D = 128, 219 against 234 at D = 96; at D = 64
-  // the two measure the same, 183-189 us, and at D = 32, where a tile has eight matrix instructions for the same
-  // vector work, the interleaved kernel wins, 120 against 139 us).
+  // Grids with enough query blocks for eight waves take the kernel whose two waves per SIMD alternate between matrix
+  // and vector phases (B8 H16 S2048: 248-254 us against 291-297 for the interleaved kernel at D = 128, 208 against
+  // 234 at D = 96, 165 against 180 at D = 64, 98 against 114 at D = 32); the interleaved kernel keeps the 128-row
+  // blocks of small grids.
   if (D == 128) {
     if (variant == 1) return launch_fa<128, 1, 4, 1>(Q, K, V, O, (int)bh, Sq, Skv, scale, lds, s);
     if (!interleaved_only) return launch_fa_pp<128>(Q, K, V, O, (int)bh, Sq, Skv, scale, lds, s);
@@ -1053,10 +1053,12 @@ extern "C" int ftk_flash_attn_f16(const void* Q, const void* K, const void* V, v
   }
   if (D == 64) {
     if (variant == 1) return launch_fa<64, 1, 4, 1>(Q, K, V, O, (int)bh, Sq, Skv, scale, lds, s);
+    if (!interleaved_only) return launch_fa_pp<64>(Q, K, V, O, (int)bh, Sq, Skv, scale, lds, s);
     return launch_fa<64, 1, 8, 1>(Q, K, V, O, (int)bh, Sq, Skv, scale, lds, s);
   }
   // D = 32: the head dimension of the reference's example program (examples/flash_attention/flash_attention.py:96-110)
   if (variant == 1) return launch_fa<32, 1, 4, 1>(Q, K, V, O, (int)bh, Sq, Skv, scale, lds, s);
+  if (!interleaved_only) return launch_fa_pp<32>(Q, K, V, O, (int)bh, Sq, Skv, scale, lds, s);
   return launch_fa<32, 1, 8, 1>(Q, K, V, O, (int)bh, Sq, Skv, scale, lds, s);
 }
 

@@ -754,6 +754,10 @@ def fa_inputs(seed, B, Hd, Sq, Skv, D):
     (4, 32, 512, 40, 128),     # ... a single, ragged tile
     (4, 32, 512, 64, 128),     # ... a single whole tile
     (4, 32, 512, 256, 96),     # D 96 on the eight-wave kernel for whole tiles
+    (4, 32, 512, 512, 32),     # D 32 and 64 on the eight-wave kernel, whole and ragged tiles
+    (4, 32, 512, 100, 32),
+    (4, 32, 512, 320, 64),
+    (4, 32, 500, 333, 64),
 ])
 def test_flash_attention(core, B, Hd, Sq, Skv, D):
     Q, K, V = fa_inputs(4, B, Hd, Sq, Skv, D)
