@@ -1029,12 +1029,14 @@ extern "C" int ftk_flash_attn_f16(const void* Q, const void* K, const void* V, v
   int rc = device_props(&dp);
   if (rc) return rc;
   hipStream_t s = (hipStream_t)stream;
-  // Variant: 0 = choose by problem size, 1 = 4 waves x 32 query rows, 3 = 8 waves x 32 query rows.
-  // Measured on MI355X (B8 H16 S2048): 8 waves (two per SIMD; K/V tiles shared by 256 rows) 358 us at
-  // D=128 and 203 us at D=64, against 476 / 307 us for 4 waves; for grids that do not fill the chip with
-  // 256-row blocks (B2 H8 S1024) the 128-row blocks win, 29 against 38 us.
+  // Variant: 0 = choose by problem size, 1 = 4 waves x 32 query rows (interleaved kernel), 3 = 8 waves x 32 query rows.
+  // Eight waves (two per SIMD; K / V tiles shared by 256 rows) whenever 256-row blocks fill the chip, and also on
+  // smaller grids once there are 512 keys or more: measured on MI355X at B2 H12 S2048 D64 33 against 49 us, B1 H16 S2048
+  // D128 44 against 50 us, B2 H8 S1024 D128 22.3 against 23.5 us (64 workgroups against 128), B4 H8 S1024 D32 14.6
+  // against 16.7 us; with few keys a launch is its own latency (9.5-10 us either way) and the 128-row blocks, which
+  // spread a short problem over more compute units, are kept (B1 H4 S300 D128: 10.7 against 12.2 us).
   int variant = fa_variant_override();
-  if (variant == 0) variant = (long long)((Sq + 255) / 256) * bh >= dp->cus ? 3 : 1;
+  if (variant == 0) variant = ((long long)((Sq + 255) / 256) * bh >= dp->cus || Skv >= 512) ? 3 : 1;
   const int lds = dp->lds_optin;
   static const bool interleaved_only = getenv("FTK_FA_INTERLEAVED") != nullptr;   // tuning hook: the older kernel for every shape
   // Grids with enough query blocks for eight waves take the kernel whose two waves per SIMD alternate between matrix
