@@ -1038,29 +1038,24 @@ extern "C" int ftk_flash_attn_f16(const void* Q, const void* K, const void* V, v
   int variant = fa_variant_override();
   if (variant == 0) variant = ((long long)((Sq + 255) / 256) * bh >= dp->cus || Skv >= 512) ? 3 : 1;
   const int lds = dp->lds_optin;
-  static const bool interleaved_only = getenv("FTK_FA_INTERLEAVED") != nullptr;   // tuning hook: the older kernel for every shape
   // Grids with enough query blocks for eight waves take the kernel whose two waves per SIMD alternate between matrix
   // and vector phases (B8 H16 S2048: 248-254 us against 291-297 for the interleaved kernel at D = 128, 208 against
   // 234 at D = 96, 165 against 180 at D = 64, 98 against 114 at D = 32); the interleaved kernel keeps the 128-row
   // blocks of small grids.
   if (D == 128) {
     if (variant == 1) return launch_fa<128, 1, 4, 1>(Q, K, V, O, (int)bh, Sq, Skv, scale, lds, s);
-    if (!interleaved_only) return launch_fa_pp<128>(Q, K, V, O, (int)bh, Sq, Skv, scale, lds, s);
-    return launch_fa<128, 1, 8, 1>(Q, K, V, O, (int)bh, Sq, Skv, scale, lds, s);
+    return launch_fa_pp<128>(Q, K, V, O, (int)bh, Sq, Skv, scale, lds, s);
   }
   if (D == 96) {
     if (variant == 1) return launch_fa<96, 1, 4, 1>(Q, K, V, O, (int)bh, Sq, Skv, scale, lds, s);
-    if (!interleaved_only) return launch_fa_pp<96>(Q, K, V, O, (int)bh, Sq, Skv, scale, lds, s);
-    return launch_fa<96, 1, 8, 1>(Q, K, V, O, (int)bh, Sq, Skv, scale, lds, s);
+    return launch_fa_pp<96>(Q, K, V, O, (int)bh, Sq, Skv, scale, lds, s);
   }
   if (D == 64) {
     if (variant == 1) return launch_fa<64, 1, 4, 1>(Q, K, V, O, (int)bh, Sq, Skv, scale, lds, s);
-    if (!interleaved_only) return launch_fa_pp<64>(Q, K, V, O, (int)bh, Sq, Skv, scale, lds, s);
-    return launch_fa<64, 1, 8, 1>(Q, K, V, O, (int)bh, Sq, Skv, scale, lds, s);
+    return launch_fa_pp<64>(Q, K, V, O, (int)bh, Sq, Skv, scale, lds, s);
   }
   // D = 32: the head dimension of the reference's example program (examples/flash_attention/flash_attention.py:96-110)
   if (variant == 1) return launch_fa<32, 1, 4, 1>(Q, K, V, O, (int)bh, Sq, Skv, scale, lds, s);
-  if (!interleaved_only) return launch_fa_pp<32>(Q, K, V, O, (int)bh, Sq, Skv, scale, lds, s);
-  return launch_fa<32, 1, 8, 1>(Q, K, V, O, (int)bh, Sq, Skv, scale, lds, s);
+  return launch_fa_pp<32>(Q, K, V, O, (int)bh, Sq, Skv, scale, lds, s);
 }
 
