@@ -846,6 +846,17 @@ def main():
     if args.workload == 'mfma_rate':
         print(json.dumps(probe_mfma_rate()))
         return
+    # what the matrix pipes hold on random operands, measured by the stand-alone probe before this process touches
+    # the GPU: the figure the fractions of the nominal MFMA peak below have to be read against
+    held = None
+    if not args.no_extras:
+        try:
+            pr = probe_mfma_rate()
+            held = {'tflops_random_operands': pr['value'], 'frac_of_nominal_peak': pr['roofline']['frac'],
+                    'tflops_constant_operands': pr['mfma_alone'].get('every lane the same constant', {}).get('tflops'),
+                    'how': 'fractaltensor_amd/mfma_rate: register-only v_mfma_f32_32x32x16_f16, one wave per SIMD, 2.5 ms per run'}
+        except (SystemExit, Exception) as e:   # the probe is an extra: its absence must not take the headline down
+            held = {'error': repr(e)}
 
     import torch
     import fractaltensor_amd._core as core   # raises if libftkernels.so is missing: no fallback
@@ -915,6 +926,8 @@ def main():
         rows[CONFIG_OF[name]] = {'workload': name, 'ms_per_step': sig(r['ms_per_step']), 'value': sig(r.get('value')), 'unit': r.get('unit'),
                                  'bound': r['roofline']['bound'], 'frac': sig(r['roofline']['frac']), 'max_rel_diff': sig(diff),
                                  'cpu_baseline': sig((r.get('cpu_baseline') or {}).get('value'))}
+    if held is not None:
+        line['fp16_mfma_rate_held'] = held
     line['configs'] = dict(sorted(rows.items()))
     print(json.dumps(line))
 
