@@ -758,6 +758,8 @@ def fa_inputs(seed, B, Hd, Sq, Skv, D):
     (4, 32, 512, 100, 32),
     (4, 32, 512, 320, 64),
     (4, 32, 500, 333, 64),
+    (4, 32, 300, 1, 64),       # a single key on the eight-wave kernel: every output row is that key's value row
+    (4, 32, 300, 33, 128),     # one key in the second half of the only tile
 ])
 def test_flash_attention(core, B, Hd, Sq, Skv, D):
     Q, K, V = fa_inputs(4, B, Hd, Sq, Skv, D)
