@@ -543,11 +543,12 @@ static int launch_b2b8(const void* A, const void* B, const void* C, void* D, int
   const long long total = units * per;
   if (total > 0x7fffffffLL) return fail(FTK_ERR_UNSUPPORTED_SHAPE, "ftk_b2b_gemm_f16: grid too large");
   gr.total = (int)total;
-  static bool attr_set = false;
-  if (!attr_set) {
+  static DeviceOnce attr_once;
+  unsigned attr_bit;
+  if (attr_once.pending(&attr_bit)) {
     FTK_HIP(hipFuncSetAttribute((const void*)b2b_gemm8_kernel<KS, PT, NT, ROWMAJOR>,
                                 hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-    attr_set = true;
+    attr_once.done(attr_bit);
   }
   hipLaunchKernelGGL((b2b_gemm8_kernel<KS, PT, NT, ROWMAJOR>), dim3(gr.total), dim3(waves * 64), lds, s, (const _Float16*)A,
                      (const _Float16*)B, (const _Float16*)C, (_Float16*)D, M, P, p_base, gr);
@@ -742,10 +743,11 @@ static int launch_b2b_wide(const void* A, const void* B, const void* C, void* D,
   const long long per = std::max(1LL, std::min(units, (long long)cus / std::max(1, G)));
   *handled = (int)lds <= lds_max && per * G <= 0x7fffffffLL;
   if (!*handled) return FTK_OK;
-  static bool attr_set = false;
-  if (!attr_set) {
+  static DeviceOnce attr_once;
+  unsigned attr_bit;
+  if (attr_once.pending(&attr_bit)) {
     FTK_HIP(hipFuncSetAttribute((const void*)b2b_wide_kernel<KS, PT, NTW, WAVES>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-    attr_set = true;
+    attr_once.done(attr_bit);
   }
   hipLaunchKernelGGL((b2b_wide_kernel<KS, PT, NTW, WAVES>), dim3((unsigned)(per * G)), dim3(WAVES * 64), lds, s,
                      (const _Float16*)A, (const _Float16*)B, (const _Float16*)C, (_Float16*)D, M, (int)units, (int)per);

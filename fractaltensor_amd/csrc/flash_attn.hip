@@ -917,14 +917,15 @@ static int launch_fa_pp(const void* Q, const void* K, const void* V, void* O, in
   const size_t tiles = (size_t)2 * FaLayout<D>::KTB + (size_t)3 * FaLayout<D>::VTB;
   const size_t lds = std::max(tiles, (size_t)8 * 32 * (2 * D + 16));   // the O tiles of the eight waves go where the K / V tiles were
   if ((int)lds > lds_max) return fail(FTK_ERR_UNSUPPORTED_SHAPE, "ftk_flash_attn_f16: needs %zu bytes of LDS", lds);
-  static bool attr_set = false;
-  if (!attr_set) {
+  static DeviceOnce attr_once;
+  unsigned attr_bit;
+  if (attr_once.pending(&attr_bit)) {
     FTK_HIP(hipFuncSetAttribute((const void*)flash_attn_pp_kernel<D, false, false>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
     FTK_HIP(hipFuncSetAttribute((const void*)flash_attn_pp_kernel<D, false, true>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
 #ifdef FTK_DEBUG_TRACE
     FTK_HIP(hipFuncSetAttribute((const void*)flash_attn_pp_kernel<D, true, true>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
 #endif
-    attr_set = true;
+    attr_once.done(attr_bit);
   }
   const int nqb = (Sq + 255) / 256;
   const long long total = (long long)nqb * BH;
@@ -954,8 +955,9 @@ static int launch_fa(const void* Q, const void* K, const void* V, void* O, int B
                      int lds_max, hipStream_t s) {
   const size_t lds = (size_t)3 * FaLayout<D>::KTB + (size_t)2 * FaLayout<D>::VTB;  // three K tiles, two V tiles
   if ((int)lds > lds_max) return fail(FTK_ERR_UNSUPPORTED_SHAPE, "ftk_flash_attn_f16: needs %zu bytes of LDS", lds);
-  static bool attr_set = false;
-  if (!attr_set) {
+  static DeviceOnce attr_once;
+  unsigned attr_bit;
+  if (attr_once.pending(&attr_bit)) {
     FTK_HIP(hipFuncSetAttribute((const void*)flash_attn_kernel<D, QT, WAVES, MINB, false, false>,
                                 hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
     FTK_HIP(hipFuncSetAttribute((const void*)flash_attn_kernel<D, QT, WAVES, MINB, false, true>,
@@ -964,7 +966,7 @@ static int launch_fa(const void* Q, const void* K, const void* V, void* O, int B
     FTK_HIP(hipFuncSetAttribute((const void*)flash_attn_kernel<D, QT, WAVES, MINB, true, true>,
                                 hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
 #endif
-    attr_set = true;
+    attr_once.done(attr_bit);
   }
   constexpr int ROWS = WAVES * 32 * QT;
   const int nqb = (Sq + ROWS - 1) / ROWS;

@@ -6,6 +6,7 @@
 #include <stdint.h>
 #include <stdio.h>
 
+#include <atomic>
 #include <type_traits>
 
 #include "../../include/ftk.h"
@@ -39,6 +40,27 @@ inline int check_launch(const char* what) {
     if (e_ != hipSuccess)                                                    \
       return ::ftk::fail(FTK_ERR_LAUNCH, "%s: %s", #call, hipGetErrorString(e_)); \
   } while (0)
+
+// Set-up that a call site owes every device once (a function attribute is kept with the device's copy of the code
+// object, so a process that drives two devices has to set it on both).  The set-up is idempotent: two threads that
+// both find the device unprepared both do it.
+class DeviceOnce {
+ public:
+  // true while the current device has not been prepared by this call site; *bit then goes to done()
+  bool pending(unsigned* bit) const {
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev > 31) {
+      *bit = 0;
+      return true;
+    }
+    *bit = 1u << dev;
+    return !(seen_.load(std::memory_order_acquire) & *bit);
+  }
+  void done(unsigned bit) { seen_.fetch_or(bit, std::memory_order_release); }
+
+ private:
+  std::atomic<unsigned> seen_{0};
+};
 
 // Every workspace a stacked-LSTM entry point takes starts with this block; its first int is the status word
 // that ftk_stacked_lstm_status() reads.

@@ -791,12 +791,13 @@ int pack_weights_f16(const void* WU, void* packed, int layers, int K2, int H, hi
 
 template <bool PACKED, int WAVES, bool SPLIT, bool GEMM = false>
 static int launch_cells_f16(const CellListH& list, int B, int I, int H, hipStream_t s) {
-  static bool attr_set = false;  // per process; the attribute belongs to the function, on every device
+  static DeviceOnce attr_once;
   constexpr int UB = 8 * WAVES;
   const void* fn = (const void*)lstm_cell_f16_kernel<PACKED, WAVES, SPLIT, GEMM>;
-  if (!attr_set) {
+  unsigned attr_bit;
+  if (attr_once.pending(&attr_bit)) {
     FTK_HIP(hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)cell_lds_bytes(UB)));
-    attr_set = true;
+    attr_once.done(attr_bit);
   }
   const int groups = (list.n + 7) / 8;  // cells per XCD
   dim3 grid((GEMM ? list.n : 8 * groups) * (H / UB) * ((B + HROWS - 1) / HROWS));
@@ -807,11 +808,12 @@ static int launch_cells_f16(const CellListH& list, int B, int I, int H, hipStrea
 
 static int launch_cells(const CellListH& list, int B, int I, int H, hipStream_t s) {
   if (list.packed == 3) {  // split products, four tiles per chunk
-    static bool attr_set = false;
-    if (!attr_set) {
+    static DeviceOnce attr_once;
+    unsigned attr_bit;
+    if (attr_once.pending(&attr_bit)) {
       FTK_HIP(hipFuncSetAttribute((const void*)lstm_cell_split4_kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
                                   (int)kSplit4Lds));
-      attr_set = true;
+      attr_once.done(attr_bit);
     }
     const int groups = (list.n + 7) / 8;
     dim3 grid(8 * groups * (H / 64) * ((B + HROWS - 1) / HROWS));

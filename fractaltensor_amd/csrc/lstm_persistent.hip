@@ -957,11 +957,12 @@ static int trace_workgroup() {
 
 template <int MODE>
 static int persistent_function(const void** fn, size_t lds) {
-  static bool attr_set = false;
+  static DeviceOnce attr_once;
   *fn = (const void*)lstm_persistent_kernel<MODE>;
-  if (!attr_set) {
+  unsigned attr_bit;
+  if (attr_once.pending(&attr_bit)) {
     FTK_HIP(hipFuncSetAttribute(*fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-    attr_set = true;
+    attr_once.done(attr_bit);
   }
   return FTK_OK;
 }
