@@ -483,6 +483,14 @@ def test_stacked_lstm_config4_full_size(core, products):
     # second call reuses nothing stale: same answer
     h3, _ = core.stacked_lstm(dx, dW)
     assert torch.equal(h1, h3)
+    # batch rows never interact: the rows in another order give the same numbers bit for bit, whichever row block,
+    # lane and item of the schedule they land in
+    perm = torch.randperm(B, generator=torch.Generator().manual_seed(3)).cuda()
+    hp, cp = core.stacked_lstm(dx[:, perm].contiguous(), dW)
+    assert torch.equal(hp, h1[:, :, perm]) and torch.equal(cp, c1[:, :, perm])
+    # a step depends on earlier steps only: the first half of the sequence alone gives the first half of the outputs
+    hh, ch = core.stacked_lstm(dx[:T // 2].contiguous(), dW)
+    assert torch.equal(hh, h1[:, :T // 2]) and torch.equal(ch, c1[:, :T // 2])
 
 
 def test_dilated_lstm_config5_full_size(core, products):
@@ -503,6 +511,12 @@ def test_dilated_lstm_config5_full_size(core, products):
     rows = [0, 31, 32, 100, 255]
     hr, cr = ko.stacked_lstm(xs[:, rows], WU, None, dilations=dil)
     assert_lstm_close(h1[:, :, rows], hr, 'hsss rows'); assert_lstm_close(c1[:, :, rows], cr, 'csss rows')
+    # rows never interact and a step depends on earlier steps only: bit for bit
+    perm = torch.randperm(B, generator=torch.Generator().manual_seed(3)).cuda()
+    hp, cp = core.stacked_lstm(dx[:, perm].contiguous(), dW, dilations=dil)
+    assert torch.equal(hp, h1[:, :, perm]) and torch.equal(cp, c1[:, :, perm])
+    hh, ch = core.stacked_lstm(dx[:80].contiguous(), dW, dilations=dil)
+    assert torch.equal(hh, h1[:, :80]) and torch.equal(ch, c1[:, :80])
 
 
 @pytest.mark.parametrize('L,T,B,H,dil,bias', [
@@ -717,6 +731,17 @@ def test_b2b_config2_full_size(core):
     assert worst <= F16_TOL
     Dc = c_oracle.b2b_gemm(A[5:6, :256], Bn[5:6], Cp[5:6], round_intermediate=True)
     assert ko.max_rel_err(D[5, :256], Dc[0]) <= 2e-3
+    # every row of D depends on its own row of A only: the rows of A in another order give the rows of D in that
+    # order, bit for bit, whichever wave and workgroup they land in
+    perm = np.random.default_rng(5).permutation(M)
+    Dp = core.b2b_gemm(dev(np.ascontiguousarray(A[:, perm])), dev(Bn), dev(Cp)).cpu().numpy()
+    assert np.array_equal(Dp, D[:, perm])
+    # D is linear in C, and doubling is exact in fp16 and in the fp32 sums: bit-identical after scaling back wherever
+    # D is a normal fp16 number (subnormal results were rounded on the coarser grid of 2^-24)
+    D2 = core.b2b_gemm(dev(A), dev(Bn), dev((Cp * np.float16(2)).astype(np.float16))).cpu().numpy()
+    normal = np.abs(D.astype(np.float32)) > 2.0 ** -14
+    assert np.array_equal(D2[normal], (D * np.float16(2))[normal])
+    assert np.max(np.abs(D2.astype(np.float32) - 2 * D.astype(np.float32))) <= 2.0 ** -23
 
 
 def test_b2b_rejects_bad_shapes(core):
@@ -827,6 +852,17 @@ def test_flash_attention_config3_full_size(core):
     ones = torch.ones_like(V).cuda()
     O1 = core.flash_attention(Q.cuda(), K.cuda(), ones, scale)
     assert (O1.float() - 1).abs().max().item() <= 2e-3
+    # the order of the keys does not matter: K and V permuted alike give the same O up to the rounding of P and of the
+    # sums, which now meet the keys in another order and in other tiles
+    perm = torch.randperm(S, generator=g).cuda()
+    Op = core.flash_attention(Q.cuda(), K.cuda()[:, :, perm].contiguous(), V.cuda()[:, :, perm].contiguous(), scale)
+    assert (Op.float() - O.float()).abs().max().item() / ref_all.abs().max().item() <= 5e-3
+    # O is linear in V, and a power of two is exact in fp16 and in every fp32 sum: the outputs agree bit for bit after
+    # scaling back, except where O itself is a subnormal fp16 number and was rounded on a coarser grid (2^-24)
+    O4 = core.flash_attention(Q.cuda(), K.cuda(), (V * 4).cuda(), scale)
+    assert (O4.float() - 4 * O.float()).abs().max().item() <= 2.0 ** -22
+    normal = O.float().abs() > 2.0 ** -14      # 2^-14 itself may have been rounded up to from the coarser grid
+    assert torch.equal(O4[normal], (O * 4)[normal])
 
 
 def test_flash_attention_rejects_bad_shapes(core):
