@@ -67,6 +67,58 @@ def _events_ms(torch, fn, steps, warmup):
     return start.elapsed_time(end) / steps, wall
 
 
+def _host_threads():
+    """Threads for the host legs: the physical cores, capped at the 16 a one-GPU box gives a job."""
+    try:
+        import psutil
+        n = psutil.cpu_count(logical=False) or os.cpu_count() or 1
+    except Exception:
+        n = os.cpu_count() or 1
+    return max(1, min(16, n))
+
+
+def _host_timed(torch, fn, warm, runs):
+    """(last result, median seconds, min seconds, threads) of fn on torch CPU with torch.set_num_threads(physical
+    cores, at most 16): the way every torch-CPU baseline of this file is timed."""
+    threads = _host_threads()
+    before = torch.get_num_threads()
+    torch.set_num_threads(threads)
+    try:
+        for _ in range(warm):
+            out = fn()
+        t = []
+        for _ in range(runs):
+            t0 = time.perf_counter()
+            out = fn()
+            t.append(time.perf_counter() - t0)
+    finally:
+        torch.set_num_threads(before)
+    return out, sorted(t)[len(t) // 2], min(t), threads
+
+
+def _lstm_torch_cpu(torch, xs, WU, dil=None):
+    """The batched LSTM loop on torch CPU: per layer and step one [B, 2H] @ [2H, 4H] product and the gate arithmetic
+    as torch operators (the batched form of examples/stacked_rnn/stacked_rnn.py:23-65 and of
+    benchmarks/rnn/baselines/stacked_lstm/pt_model/rnn.py:94-108).  Returns the last layer's h [T, B, H]."""
+    L = WU.shape[0]
+    T, B, H = xs.shape
+    inp = xs
+    for l in range(L):
+        d = 1 if dil is None else dil[l]
+        hs, cs = [], []
+        zero = torch.zeros((B, H))
+        for t in range(T):
+            h, c = (hs[t - d], cs[t - d]) if t >= d else (zero, zero)
+            g = torch.cat([inp[t], h], dim=1) @ WU[l]
+            i, f, o, cand = g.chunk(4, 1)
+            c = torch.sigmoid(f) * c + torch.sigmoid(i) * torch.tanh(cand)
+            h = torch.sigmoid(o) * torch.tanh(c)
+            hs.append(h)
+            cs.append(c)
+        inp = torch.stack(hs)
+    return inp
+
+
 def bench_b2b(torch, core, steps, warmup, cpu):
     G, M, N, K, P = 32, 4096, 128, 128, 128
     flop = 2.0 * G * M * N * (K + P)
@@ -108,16 +160,32 @@ def bench_b2b(torch, core, steps, warmup, cpu):
                      'kernel': 'b2b_gemm8_kernel<8,4,4>', 'algorithmic_bytes_per_launch': nbytes},
     }
     if cpu:
-        from oracle import c_oracle
-        sample = 32   # all problems: about ten seconds of scalar C
+        # the frontend's own eager expression, (a @ b) @ c per problem, on torch CPU.  fp32 operands (the fp16 values,
+        # widened beforehand): torch's host GEMM is built for fp32, so this is the host at its best, not at its worst
+        from fractaltensor_amd.kaleido import Tensor
         A, Bn, Cp, _ = sets[0]
+        a32, b32, c32 = A.float().cpu(), Bn.transpose(1, 2).float().cpu().contiguous(), Cp.transpose(1, 2).float().cpu().contiguous()
+        ta, tb, tc = ([Tensor.from_tensor(x[g]) for g in range(G)] for x in (a32, b32, c32))
+        eager = lambda: [(ta[g] @ tb[g]) @ tc[g] for g in range(G)]
+        out, med, best, threads = _host_timed(torch, eager, 2, 10)
+        core.b2b_gemm(A, Bn, Cp, out=sets[0][3])
+        diff = float((out[G - 1].data - sets[0][3][G - 1].float().cpu()).abs().max() / out[G - 1].data.abs().max())
+        assert diff <= 1e-2, diff
+        res['cpu_baseline'] = {'value': flop / med / 1e12, 'unit': 'TFLOP/s', 'cores': threads, 'kind': 'torch_cpu_eager',
+                               'sample': f'the whole configuration: the operator expression (a @ b) @ c of the frontend on the {G} '
+                                         f'problems in turn, fp32 torch CPU tensors, torch.set_num_threads({threads}) of '
+                                         f'{os.cpu_count()} host CPUs, 2 warm-up + 10 timed runs, median {med * 1e3:.1f} ms '
+                                         f'(min {best * 1e3:.1f} ms)',
+                               'ms_per_step': med * 1e3, 'max_rel_diff_vs_gpu': diff}
+        from oracle import c_oracle
+        sample = 8    # a quarter of the problems: a few seconds of scalar C
         a, b, c = (x[:sample].cpu().numpy() for x in (A, Bn, Cp))
         t0 = time.perf_counter()
         c_oracle.b2b_gemm(a, b, c, round_intermediate=True)
         dt = time.perf_counter() - t0
-        res['cpu_baseline'] = {'value': flop * sample / G / dt / 1e12, 'unit': 'TFLOP/s', 'cores': 1, 'kind': 'port',
-                               'sample': f'{sample} of the {G} problems through oracle/oracle.c (scalar C, one thread), '
-                                         f'{dt:.1f} s'}
+        res['cpu_baseline']['scalar_c_port'] = {'value': flop * sample / G / dt / 1e12, 'unit': 'TFLOP/s', 'cores': 1,
+                                                'sample': f'{sample} of the {G} problems through oracle/oracle.c (scalar C, one '
+                                                          f'thread), {dt:.1f} s'}
     return res
 
 
@@ -215,15 +283,40 @@ def bench_attention(torch, core, steps, warmup, cpu):
                      'traffic': MEASURED_TRAFFIC_BYTES.get('flash_attn_pp_kernel'), 'kernel': 'flash_attn_pp_kernel'},
     }
     if cpu:
+        # the blockwise program of examples/flash_attention/flash_attention.py:14-91 as this package states it
+        # (programs.flash_attention: map over samples and heads, map over query blocks, reduce over key blocks of 64
+        # rows), eager on torch CPU in fp32 (the example's own element type), on a bounded sample of heads
+        from fractaltensor_amd import programs
+        from fractaltensor_amd.kaleido import FractalTensor
+        heads, blk = 4, 64
+        mk = lambda t: FractalTensor.from_dense(t[0:1, :heads].float().cpu().reshape(1, heads, S // blk, blk, D).contiguous(), 3)
+        q, k, v = mk(Q), mk(K), mk(V)
+        out, med, best, threads = _host_timed(torch, lambda: programs.flash_attention(q, k, v, scale), 0, 2)
+        core.flash_attention(Q, K, V, scale, out=O)
+        ref = O[0, :heads].float().cpu()
+        diff = float((out.as_dense().reshape(heads, S, D) - ref).abs().max() / ref.abs().max())
+        assert diff <= 1e-2, diff
+        res['cpu_baseline'] = {'value': flop * heads / (B * Hd) / med / 1e12, 'unit': 'TFLOP/s', 'cores': threads,
+                               'kind': 'torch_cpu_eager',
+                               'sample': f'{heads} of {B * Hd} (batch, head) pairs: the eager operator program '
+                                         f'(programs.flash_attention, {S // blk} x {S // blk} blocks of {blk} rows per head) on '
+                                         f'fp32 torch CPU tensors, torch.set_num_threads({threads}) of {os.cpu_count()} host CPUs, '
+                                         f'2 timed runs, median {med:.2f} s',
+                               'max_rel_diff_vs_gpu': diff}
+        # the same attention as one torch call per head on the host, to separate operator dispatch from host arithmetic
+        qh, kh, vh = (x[0].float().cpu() for x in (Q, K, V))
+        sdpa = lambda: torch.nn.functional.scaled_dot_product_attention(qh, kh, vh, scale=scale)
+        _, med_s, _, _ = _host_timed(torch, sdpa, 1, 3)
+        res['cpu_baseline']['batched'] = {'value': flop / B / med_s / 1e12, 'unit': 'TFLOP/s', 'ms_per_step': med_s * 1e3,
+                                          'what': f'torch scaled_dot_product_attention on the {Hd} heads of one sample, fp32, {threads} threads'}
         from oracle import c_oracle
-        heads = 24
-        q, k, v = (x[0, :heads].cpu().numpy() for x in (Q, K, V))
+        hs = 4
+        q, k, v = (x[0, :hs].cpu().numpy() for x in (Q, K, V))
         t0 = time.perf_counter()
         c_oracle.flash_attention(q, k, v, scale, block_kv=64)
         dt = time.perf_counter() - t0
-        res['cpu_baseline'] = {'value': flop * heads / (B * Hd) / dt / 1e12, 'unit': 'TFLOP/s', 'cores': 1,
-                               'kind': 'port', 'sample': f'{heads} of {B * Hd} (batch, head) pairs through '
-                                                         f'oracle/oracle.c, {dt:.1f} s'}
+        res['cpu_baseline']['scalar_c_port'] = {'value': flop * hs / (B * Hd) / dt / 1e12, 'unit': 'TFLOP/s', 'cores': 1,
+                                                'sample': f'{hs} of {B * Hd} (batch, head) pairs through oracle/oracle.c, {dt:.1f} s'}
     return res
 
 
@@ -554,43 +647,58 @@ def bench_lstm(torch, core, steps, warmup, cpu, dilated, baselines=True):
         'tflops': flop / ms / 1e9,
         'frac_of_f32_matrix_peak_algorithmic': flop / ms / 1e9 / PEAK_F32_MATRIX_TFLOPS,
         'persistent_status': status,
-        # algorithmic flops (2*B*2H*4H per cell) against the peak of the arithmetic the path is specified in, fp32
-        # matrix; the default mode forms each product from three f16 MFMAs, which is how the fraction passes 1.
-        # The MFMA flops actually issued, against the peak of the MFMA type that executes them, are given beside it.
-        'roofline': {'bound': 'mfma', 'achieved': flop / ms / 1e9, 'peak': PEAK_F32_MATRIX_TFLOPS, 'unit': 'TFLOP/s',
-                     'frac': flop / ms / 1e9 / PEAK_F32_MATRIX_TFLOPS,
-                     'executed': {'achieved': executed / ms / 1e9, 'peak': peak, 'frac': executed / ms / 1e9 / peak,
-                                  'what': 'MFMA flops issued (three f16 products per fp32 product in f16x3 mode) against '
-                                          'the peak of the MFMA type that executes them'},
+        # the roofline of the unit that executes: MFMA flops issued (three f16 MFMAs per fp32 product in f16x3 mode)
+        # against the peak of that MFMA type.  The algorithmic flops (2*B*2H*4H per cell) against the fp32 matrix peak
+        # are the named extra above; in f16x3 mode that ratio passes 1 and is no roofline fraction.
+        'roofline': {'bound': 'mfma', 'achieved': executed / ms / 1e9, 'peak': peak, 'unit': 'TFLOP/s',
+                     'frac': executed / ms / 1e9 / peak,
+                     'what': 'MFMA flops issued (three f16 products per fp32 product in f16x3 mode) against the peak of '
+                             'the MFMA type that executes them',
+                     'algorithmic': {'tflops': flop / ms / 1e9, 'f32_matrix_peak': PEAK_F32_MATRIX_TFLOPS,
+                                     'ratio_to_f32_matrix_peak': flop / ms / 1e9 / PEAK_F32_MATRIX_TFLOPS},
                      'traffic': MEASURED_TRAFFIC_BYTES.get('lstm_persistent_kernel' + ('_dilated' if dilated else '')),
+                     'algorithmic_bytes_per_launch': 4.0 * (T * B * H + L * 2 * H * 4 * H + 2 * L * T * B * H),
                      'kernel': 'lstm_persistent_kernel'},
     }
     res.update(extra)
     if cpu:
+        # the batched LSTM loop on torch CPU, the whole configuration: one [B, 2H] @ [2H, 4H] product and the gate
+        # arithmetic as torch operators per layer and step
+        xc, WUc = xs.cpu(), WU.cpu()
+        out, med, best, threads = _host_timed(torch, lambda: _lstm_torch_cpu(torch, xc, WUc, dil), 1, 3)
+        ref = ref_h[L - 1].cpu()
+        diff = float((out - ref).abs().max() / ref.abs().max())
+        assert diff <= 1e-4, diff
+        res['cpu_baseline'] = {'value': B / med, 'unit': 'sequences/s', 'cores': threads, 'kind': 'torch_cpu_eager',
+                               'sample': f'the whole configuration: per layer and step one [{B},{2 * H}] @ [{2 * H},{4 * H}] product '
+                                         f'and the gate arithmetic as torch CPU operators (fp32), torch.set_num_threads({threads}) '
+                                         f'of {os.cpu_count()} host CPUs, 1 warm-up + 3 timed runs, median {med:.2f} s (min {best:.2f} s)',
+                               'ms_per_step': med * 1e3, 'max_rel_diff_vs_gpu': diff, 'gpu_speedup': med * 1e3 / ms}
+        # the per-sample operator program (scan over time of map over batch of [1,H] cells, four gate products per
+        # cell: the reference's execution model) on a bounded sample, scaled by cells to the configuration
+        from fractaltensor_amd import programs
+        Ls, Ts, Bs = 2, 8, 32
+        Wss, Uss, bss = programs.make_lstm_params(Ls, H, 1.0 / 16, 1234, bias=False)
+        xss = programs.make_sequence_batch(Ts, Bs, H, 1234)
+        prog = (lambda: programs.dilated_lstm(xss, Wss, Uss, bss)) if dilated else (lambda: programs.stacked_lstm(xss, Wss, Uss, bss))
+        _, med_e, _, _ = _host_timed(torch, prog, 0, 2)
+        full_seconds = med_e * (L * T * B) / (Ls * Ts * Bs)
+        res['cpu_baseline']['eager_per_sample'] = {
+            'value': B / full_seconds, 'unit': 'sequences/s',
+            'sample': f'{Ls} layers x {Ts} steps x {Bs} samples of the eager operator program on torch CPU in {med_e:.2f} s, '
+                      f'scaled by cells to the full configuration'}
         from oracle import c_oracle
-        Ls, Ts, Bs = (8, 64, 256) if not dilated else (6, 32, 256)
+        Ls, Ts, Bs = (2, 32, 256) if not dilated else (2, 32, 256)
         x = xs[:Ts, :Bs].cpu().numpy()
         w = WU[:Ls].cpu().numpy()
         t0 = time.perf_counter()
         c_oracle.stacked_lstm(x, w, None, None if dil is None else dil[:Ls])
         dt = time.perf_counter() - t0
-        cells = Ls * Ts
-        # sequences/s of the full configuration extrapolated from the per-(cell,row) cost of the sample
-        full_seconds = dt * (L * T * B) / (cells * Bs)
-        res['cpu_baseline'] = {'value': B / full_seconds, 'unit': 'sequences/s', 'cores': 1, 'kind': 'port',
-                               'sample': f'{Ls} layers x {Ts} steps x {Bs} rows through oracle/oracle.c in {dt:.1f} s, '
-                                         f'scaled by cell-rows to the full configuration'}
+        full_seconds = dt * (L * T * B) / (Ls * Ts * Bs)
+        res['cpu_baseline']['scalar_c_port'] = {'value': B / full_seconds, 'unit': 'sequences/s', 'cores': 1,
+                                                'sample': f'{Ls} layers x {Ts} steps x {Bs} rows through oracle/oracle.c in {dt:.1f} s, '
+                                                          f'scaled by cell-rows to the full configuration'}
     return res
-
-
-def _host_threads():
-    """Threads for the host legs: the physical cores, capped at the 16 a one-GPU box gives a job."""
-    try:
-        import psutil
-        n = psutil.cpu_count(logical=False) or os.cpu_count() or 1
-    except Exception:
-        n = os.cpu_count() or 1
-    return max(1, min(16, n))
 
 
 def bench_config1(torch, core, steps, warmup, cpu):
@@ -615,15 +723,20 @@ def bench_config1(torch, core, steps, warmup, cpu):
     ms, wall = _events_ms(torch, lambda: core.stacked_lstm(xs, WUd, out=(hs, cs), workspace=ws), steps, warmup)
     core.stacked_lstm_check(ws)
     nbytes = 4.0 * (T * B * H + L * 2 * H * 4 * H + 2 * L * T * B * H)
+    split = core.get_lstm_products() == 'f16x3'
+    issued, peak = (3.0 * flop, PEAK_F16_TFLOPS) if split else (flop, PEAK_F32_MATRIX_TFLOPS)
     res = {
         'metric': 'stacked-LSTM sequences/s', 'value': B / ms * 1e3, 'unit': 'sequences/s', 'ms_per_step': ms,
-        'dtype': 'f32 (gate products as three f16 MFMAs of split operands, f32 accumulate)' if core.get_lstm_products() == 'f16x3' else 'f32',
+        'dtype': 'f32 (gate products as three f16 MFMAs of split operands, f32 accumulate)' if split else 'f32',
         'config': {'workload': 'single-layer LSTM scan, BASELINE.json configs[0]', 'layers': L, 'batch': B, 'seq_len': T, 'hidden': H},
         'tflops': flop / ms / 1e9, 'host_wall_ms_per_step': wall,
-        'roofline': {'bound': 'mfma', 'achieved': flop / ms / 1e9, 'peak': PEAK_F32_MATRIX_TFLOPS, 'unit': 'TFLOP/s',
-                     'frac': flop / ms / 1e9 / PEAK_F32_MATRIX_TFLOPS, 'traffic': None, 'kernel': 'lstm_persistent_kernel',
+        'frac_of_f32_matrix_peak_algorithmic': flop / ms / 1e9 / PEAK_F32_MATRIX_TFLOPS,
+        'roofline': {'bound': 'mfma', 'achieved': issued / ms / 1e9, 'peak': peak, 'unit': 'TFLOP/s',
+                     'frac': issued / ms / 1e9 / peak, 'traffic': None, 'kernel': 'lstm_persistent_kernel',
+                     'what': 'MFMA flops issued (three f16 products per fp32 product in f16x3 mode) against the peak of '
+                             'the MFMA type that executes them',
                      'note': '16 dependent steps of two row blocks on 8 of 256 compute units: a latency chain, not a throughput '
-                             'shape; algorithmic flops against the fp32 matrix peak', 'algorithmic_bytes_per_launch': nbytes},
+                             'shape', 'algorithmic_bytes_per_launch': nbytes},
     }
     if cpu:
         threads = _host_threads()
@@ -662,7 +775,7 @@ def bench_config1(torch, core, steps, warmup, cpu):
         diff_batched = float((batched_out - gpu_h).abs().max() / gpu_h.abs().max())
         assert diff_eager <= 1e-4 and diff_batched <= 1e-4, (diff_eager, diff_batched)
         res['cpu_baseline'] = {
-            'value': B / eager_s, 'unit': 'sequences/s', 'cores': threads, 'kind': 'port',
+            'value': B / eager_s, 'unit': 'sequences/s', 'cores': threads, 'kind': 'torch_cpu_eager',
             'sample': f'the whole configuration: the eager operator program (programs.stacked_lstm: map over {B} samples of '
                       f'[1,{H}] tensors inside a scan over {T} steps, four gate products per cell) on torch CPU, '
                       f'torch.set_num_threads({threads}) of {os.cpu_count()} host CPUs, 3 warm-up + 10 timed runs, median '
@@ -801,15 +914,24 @@ def bench_lstm_f32_streamed(torch, core, steps, warmup, cpu, H):
     return res
 
 
+def _under_profiler():
+    """True when this process runs under a profiler's preloaded library (rocprofv3 sets these): a child process would
+    inherit the preload, so no probe is spawned then."""
+    pre = os.environ.get('LD_PRELOAD', '')
+    return 'rocprof' in pre or any(k.startswith(('ROCPROF', 'ROCP_TOOL', 'ROCPROFILER')) for k in os.environ)
+
+
 def probe_mfma_rate():
-    """What the matrix pipes deliver under load: runs the stand-alone probe fractaltensor_amd/mfma_rate (built by
-    `make probes` / __graft_entry__.build()) as a child process and reports the fp16 MFMA rate it holds on random
-    operands, the figure the fractions of the nominal peak on the other lines have to be read against."""
+    """What the matrix pipes deliver under load: runs the stand-alone probe bench_probes/mfma_rate (built by
+    `make -C bench_probes` / __graft_entry__.build()) as a child process and reports the fp16 MFMA rate it holds on
+    random operands, the figure the fractions of the nominal peak on the other lines have to be read against."""
     import re
     import subprocess
-    exe = os.path.join(os.path.dirname(os.path.abspath(__file__)), 'fractaltensor_amd', 'mfma_rate')
+    exe = os.path.join(ROOT, 'bench_probes', 'mfma_rate')
     if not os.path.exists(exe):
-        raise SystemExit('bench.py --workload mfma_rate: fractaltensor_amd/mfma_rate is not built (make -C fractaltensor_amd/csrc probes)')
+        raise SystemExit('bench.py --workload mfma_rate: bench_probes/mfma_rate is not built (make -C bench_probes)')
+    if _under_profiler():
+        raise SystemExit('bench.py: the MFMA-rate probe is a child process and is not started under a profiler')
     out = subprocess.run([exe], capture_output=True, text=True, timeout=120, check=True).stdout
     alone = {}
     for ln in out.splitlines():
@@ -835,6 +957,7 @@ def main():
     ap.add_argument('--no-extras', action='store_true', help='measure only the chosen workload')
     ap.add_argument('--all', action='store_true', help='also the workloads either side of the path (fp16 / larger stacks, GEMM, softmax, embedding, grid RNN, windowed attention)')
     ap.add_argument('--no-cpu', action='store_true', help='skip the CPU baseline leg')
+    ap.add_argument('--no-probe', action='store_true', help='do not start the stand-alone MFMA-rate probe (a child process) before the run')
     ap.add_argument('--no-baselines', action='store_true',
                     help='LSTM and grid workloads: only the fused kernel (no unfused GPU baseline, per-stage launches, other product mode, path without workspace)')
     args = ap.parse_args()
@@ -849,12 +972,12 @@ def main():
     # what the matrix pipes hold on random operands, measured by the stand-alone probe before this process touches
     # the GPU: the figure the fractions of the nominal MFMA peak below have to be read against
     held = None
-    if not args.no_extras:
+    if not args.no_extras and not args.no_probe:
         try:
             pr = probe_mfma_rate()
             held = {'tflops_random_operands': pr['value'], 'frac_of_nominal_peak': pr['roofline']['frac'],
                     'tflops_constant_operands': pr['mfma_alone'].get('every lane the same constant', {}).get('tflops'),
-                    'how': 'fractaltensor_amd/mfma_rate: register-only v_mfma_f32_32x32x16_f16, one wave per SIMD, 2.5 ms per run'}
+                    'how': 'bench_probes/mfma_rate: register-only v_mfma_f32_32x32x16_f16, one wave per SIMD, 2.5 ms per run'}
         except (SystemExit, Exception) as e:   # the probe is an extra: its absence must not take the headline down
             held = {'error': repr(e)}
 

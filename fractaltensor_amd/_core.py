@@ -23,7 +23,7 @@ EXPORTS = (
     'ftk_stacked_lstm_wavefront_f32', 'ftk_stacked_lstm_ragged_f32', 'ftk_lstm_set_products', 'ftk_lstm_get_products',
     'ftk_stacked_lstm_opts_f32', 'ftk_stacked_lstm_status', 'ftk_stacked_lstm_noalloc_f32',
     'ftk_stacked_lstm_f16_workspace_bytes', 'ftk_stacked_lstm_f16',
-    'ftk_b2b_gemm_f16', 'ftk_b2b_gemm_rowmajor_f16', 'ftk_gemm_f16', 'ftk_batched_gemm_f16', 'ftk_flash_attn_f16', 'ftk_online_softmax_f32', 'ftk_embedding_gather_f32',
+    'ftk_b2b_gemm_f16', 'ftk_b2b_gemm_f16_supported', 'ftk_b2b_gemm_rowmajor_f16', 'ftk_gemm_f16', 'ftk_batched_gemm_f16', 'ftk_flash_attn_f16', 'ftk_online_softmax_f32', 'ftk_embedding_gather_f32',
     'ftk_grid_rnn_workspace_bytes', 'ftk_grid_rnn_f32', 'ftk_windowed_attn_f32',
 )
 
@@ -426,6 +426,11 @@ def b2b_gemm(A, B_nk, C_pn, out: Optional[torch.Tensor] = None) -> torch.Tensor:
     ci = ctypes.c_int
     _check(lib.ftk_b2b_gemm_f16(_ptr(A), _ptr(B_nk), _ptr(C_pn), _ptr(D), ci(G), ci(M), ci(N), ci(K), ci(P), _stream()))
     return D[0] if squeeze and out is None else D
+
+
+def b2b_gemm_supported(N: int, K: int, P: int) -> bool:
+    """Shapes ftk_b2b_gemm_f16 takes on the current device (the fused kernels' LDS fit, or N <= 2048 for the general one)."""
+    return bool(lib.ftk_b2b_gemm_f16_supported(ctypes.c_int(N), ctypes.c_int(K), ctypes.c_int(P)))
 
 
 def b2b_gemm_rowmajor_supported(N: int, K: int, P: int) -> bool:

@@ -785,10 +785,11 @@ static int launch_b2b_cols(const void* A, const void* B, const void* C, void* D,
   if (total > 0x7fffffffLL) return fail(FTK_ERR_UNSUPPORTED_SHAPE, "ftk_b2b_gemm_f16: grid too large");
   gr.total = (int)total;
   const void* fn = (const void*)b2b_gemm_kernel<KS, PT>;
-  static int attr_lds = 0;
-  if ((int)lds > attr_lds) {
+  static DeviceMax attr_lds;
+  int dev;
+  if (attr_lds.below((int)lds, &dev)) {
     FTK_HIP(hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-    attr_lds = (int)lds;
+    attr_lds.raise(dev, (int)lds);
   }
   hipLaunchKernelGGL((b2b_gemm_kernel<KS, PT>), dim3(gr.total), dim3(waves * 64), lds, s, (const _Float16*)A,
                      (const _Float16*)B, (const _Float16*)C, (_Float16*)D, M, N, P, p_base, gr);
@@ -892,19 +893,29 @@ __global__ __launch_bounds__(256) void b2b_stream_kernel(const _Float16* __restr
   }
 }
 
+// The fused kernels keep B (all of K) and a tile of C in LDS: K of 32, 64, 96 or 128, and B and C small enough to
+// fit beside one wave's region.  Everything else goes to the general kernel.
+static bool b2b_fits_fused(int N, int K, int P, int lds_max) {
+  return (K == 32 || K == 64 || K == 96 || K == 128) && (int)b2b_lds_bytes(N, K, std::min(P, B2B_PTILE), 1) <= lds_max &&
+         (P % B2B_PTILE == 0 || (int)b2b_lds_bytes(N, K, P % B2B_PTILE, 1) <= lds_max);
+}
+
+static bool b2b_fits_stream(int N, int lds_max) { return N <= kStreamMaxN && 32 * (N + 8) * 2 <= lds_max; }
+
 static int launch_b2b_stream(const void* A, const void* B, const void* C, void* D, int G, int M, int N, int K, int P,
                              int lds_max, hipStream_t s) {
   const size_t lds = (size_t)32 * (N + 8) * 2;
-  if (N > kStreamMaxN || (int)lds > lds_max)
+  if (!b2b_fits_stream(N, lds_max))
     return fail(FTK_ERR_UNSUPPORTED_SHAPE, "ftk_b2b_gemm_f16: N=%d: 32 rows of the intermediate product need %zu bytes of LDS (N <= %d)",
                 N, lds, kStreamMaxN);
   const long long row_blocks = (M + 31) / 32;
   const long long total = row_blocks * G;
   if (total > 0x7fffffffLL) return fail(FTK_ERR_UNSUPPORTED_SHAPE, "ftk_b2b_gemm_f16: grid too large");
-  static int attr_lds = 0;
-  if ((int)lds > attr_lds) {
+  static DeviceMax attr_lds;
+  int dev;
+  if (attr_lds.below((int)lds, &dev)) {
     FTK_HIP(hipFuncSetAttribute((const void*)b2b_stream_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-    attr_lds = (int)lds;
+    attr_lds.raise(dev, (int)lds);
   }
   hipLaunchKernelGGL(b2b_stream_kernel, dim3((unsigned)total), dim3(256), lds, s, (const _Float16*)A, (const _Float16*)B,
                      (const _Float16*)C, (_Float16*)D, M, N, K, P, (int)row_blocks);
@@ -912,6 +923,14 @@ static int launch_b2b_stream(const void* A, const void* B, const void* C, void* 
 }
 
 }  // namespace ftk
+
+extern "C" int ftk_b2b_gemm_f16_supported(int N, int K, int P) {
+  using namespace ftk;
+  if (N <= 0 || K <= 0 || P <= 0 || N % 32 || P % 32 || K % 16) return 0;
+  const DeviceProps* dp = nullptr;
+  if (device_props(&dp)) return 0;
+  return (b2b_fits_fused(N, K, P, dp->lds_optin) || b2b_fits_stream(N, dp->lds_optin)) ? 1 : 0;
+}
 
 extern "C" int ftk_b2b_gemm_f16(const void* A, const void* B, const void* C, void* D, int G, int M, int N, int K,
                                 int P, ftk_stream_t stream) {
@@ -925,11 +944,7 @@ extern "C" int ftk_b2b_gemm_f16(const void* A, const void* B, const void* C, voi
   int rc = device_props(&dp);
   if (rc) return rc;
   hipStream_t s = (hipStream_t)stream;
-  // The fused kernels keep B (all of K) and a tile of C in LDS: K of 32, 64, 96 or 128, and B and C small enough to
-  // fit beside one wave's region.  Everything else goes to the general kernel.
-  const bool fast = (K == 32 || K == 64 || K == 96 || K == 128) &&
-                    (int)b2b_lds_bytes(N, K, std::min(P, B2B_PTILE), 1) <= dp->lds_optin &&
-                    (P % B2B_PTILE == 0 || (int)b2b_lds_bytes(N, K, P % B2B_PTILE, 1) <= dp->lds_optin);
+  const bool fast = b2b_fits_fused(N, K, P, dp->lds_optin);
   if (!fast) return launch_b2b_stream(A, B, C, D, G, M, N, K, P, dp->lds_optin, s);
   // wide N with few columns of D (the reference benchmark's shapes): N split over the waves of a workgroup.
   // FTK_B2B_WIDE=0 keeps them on the general kernel.

@@ -62,6 +62,30 @@ class DeviceOnce {
   std::atomic<unsigned> seen_{0};
 };
 
+// The largest dynamic LDS size a call site has set on its kernel, per device: for launchers whose LDS need grows
+// with the shape.  Two threads that both find the stored size too small both set the attribute; the larger one wins.
+class DeviceMax {
+ public:
+  // true when the current device has not been given at least `value` by this call site; *dev then goes to raise()
+  bool below(int value, int* dev) const {
+    *dev = -1;
+    int d = 0;
+    if (hipGetDevice(&d) != hipSuccess || d < 0 || d >= kDevices) return true;
+    *dev = d;
+    return max_[d].load(std::memory_order_acquire) < value;
+  }
+  void raise(int dev, int value) {
+    if (dev < 0) return;
+    int cur = max_[dev].load(std::memory_order_relaxed);
+    while (cur < value && !max_[dev].compare_exchange_weak(cur, value, std::memory_order_release)) {
+    }
+  }
+
+ private:
+  static constexpr int kDevices = 32;
+  std::atomic<int> max_[kDevices] = {};
+};
+
 // Every workspace a stacked-LSTM entry point takes starts with this block; its first int is the status word
 // that ftk_stacked_lstm_status() reads.
 constexpr size_t kStatusBytes = 256;

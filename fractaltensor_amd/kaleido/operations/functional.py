@@ -14,9 +14,10 @@ docs/fractaltensor_operations/parallel_functions_on_fractaltensor.md:46-203):
 
 A function returning a tuple of values yields one FractalTensor per field.
 These are eager Python loops over torch payloads, on the CPU or the GPU: this
-IS the reference's execution model.  On GPU operands fold and map first ask
-operations.dispatch whether the call is one of the hot-path programs (a stack
-of LSTM layers, blockwise attention); if so it runs as one fused kernel.
+IS the reference's execution model.  On GPU operands fold, scan and map first
+ask operations.dispatch whether the call is one of the hot-path programs (a
+stack of LSTM layers, one layer as a scan over time, a map over samples of
+either, blockwise attention); if so it runs as one fused kernel.
 """
 from __future__ import annotations
 
@@ -78,6 +79,9 @@ def filter(cond: Callable, xs, **kwargs):
 
 def scan(func: Callable, xs, initializer=None, **kwargs):
     require_iterative(xs)
+    routed = dispatch.try_scan(func, xs, initializer, kwargs)   # one LSTM layer over GPU sequences: one kernel
+    if routed is not NotImplemented:
+        return routed
     n = len(xs)
     results = []
     if initializer is None:

@@ -272,9 +272,14 @@ int ftk_stacked_lstm_status(const void* workspace, ftk_stream_t stream);
 
 /*
  * ftk_stacked_lstm_opts_f32 with fp32 products for callers that cannot
- * allocate device memory or pass a workspace: code under HIP graph capture,
- * tight serving loops, harnesses that forbid hipMalloc.  No counterpart in
- * the reference.  Same operands and results as ftk_stacked_lstm_opts_f32
+ * allocate device memory or pass a workspace: tight serving loops, harnesses
+ * that forbid hipMalloc, code that prepares a HIP graph.  No counterpart in
+ * the reference.  The first call on a device does set-up that is no
+ * allocation but is no stream work either (the scratch's address, a function
+ * attribute, an occupancy query): make one call per device before any region
+ * that must hold nothing but launches.  The launch is a cooperative one
+ * (hipLaunchCooperativeKernel); that a stream capture records it has not been
+ * exercised here.  Same operands and results as ftk_stacked_lstm_opts_f32
  * with {FTK_LSTM_PRODUCTS_F32, 0} and no active_rows; H must be 256, and the
  * status block, flags and trace of the launch (about 64*L*T*ceil(B/32) +
  * 64*T*ceil(B/32) + 256 bytes) must fit the library's built-in scratch of
@@ -371,6 +376,16 @@ int ftk_embedding_gather_f32(const float* table, const void* ids,
  */
 int ftk_b2b_gemm_f16(const void* A, const void* B, const void* C, void* D,
                      int G, int M, int N, int K, int P, ftk_stream_t stream);
+
+/*
+ * 1 when ftk_b2b_gemm_f16 takes products of this shape on the current device
+ * (any G and M), 0 when it would return FTK_ERR_UNSUPPORTED_SHAPE or no device
+ * can be queried.  For callers that choose between the fused product and two
+ * plain ones before they call, as kaleido's `(a @ b) @ c` does
+ * (Tensor.__matmul__, kaleido/frontend/tensor.py:218-220); the reference's
+ * B2BGemm fixes its shapes at compile time (gemm_kernel_traits.h:214-283).
+ */
+int ftk_b2b_gemm_f16_supported(int N, int K, int P);
 
 /*
  * The same product with every operand row-major, the layout an operator

@@ -38,4 +38,19 @@ _parser = _namespace('kaleido.parser', Context=_impl.program.Context, function=_
 _impl.frontend = _frontend
 _impl.parser = _parser
 
+
+# kaleido._core: the name of the reference's native binding (kaleido/__init__.py:20-26, kaleido/core/init.cc:16-22)
+# is the C-ABI binding here.  It loads libftkernels.so when first touched, not when kaleido is imported, so that
+# host-only programs run where the library has not been built.
+class _LazyCore(types.ModuleType):
+    def __getattr__(self, name):
+        import fractaltensor_amd._core as core
+        sys.modules['kaleido._core'] = core
+        _impl._core = core
+        return getattr(core, name)
+
+
+_impl._core = _LazyCore('kaleido._core', 'kaleido._core: the C-ABI binding fractaltensor_amd._core, loaded on first use.')
+sys.modules['kaleido._core'] = _impl._core
+
 sys.modules['kaleido'] = _impl

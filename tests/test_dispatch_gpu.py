@@ -1,4 +1,4 @@
-"""Operator programs, unchanged, on GPU FractalTensors: fold / map route them to one fused launch.
+"""Operator programs, unchanged, on GPU FractalTensors: fold / scan / map route them to one fused launch.
 
 Two sets of programs: the ones of fractaltensor_amd/programs.py, and programs written here the way the reference's
 examples are written (`import kaleido`, decorated cell functions, per-gate map over zip(ws, us, bs), fold over
@@ -208,8 +208,10 @@ def test_a_fold_that_is_no_lstm_stays_eager():
     h0, _ = ko.stacked_lstm(x, WU[:1], bias[:1])
     h1, _ = ko.stacked_lstm(2 * h0[-1], WU[1:], bias[1:])
     assert ko.max_rel_err(out.as_dense().cpu().numpy().reshape(T, B, H), 2 * h1[-1]) <= 1e-4
-    ops.fold(doubled, ops.zip(Wss, Uss, bss), initializer=xss)          # the verdict is remembered: no second probe
-    assert dispatch.stats['probes'] == 1
+    # the fold ran as the eager loop; the scan over time inside every layer is an LSTM layer and was routed on its own
+    assert dispatch.stats['probes'] == 2 and dispatch.stats['lstm_scan'] == L
+    ops.fold(doubled, ops.zip(Wss, Uss, bss), initializer=xss)          # both verdicts are remembered: no further probe
+    assert dispatch.stats['probes'] == 2 and dispatch.stats['lstm_scan'] == 2 * L
 
 
 # ---- dilated LSTM -------------------------------------------------------------------------------------------------
@@ -229,10 +231,12 @@ def test_programs_dilated_lstm_is_routed_with_the_dilations_it_asks_for(L, T, B,
     assert core.launch_counts['stacked_lstm'] == before + 1 and dispatch.stats['probes'] == 1
 
 
-def test_reference_style_dilated_model_routes_every_samples_fold():
+def test_reference_style_dilated_model_runs_the_samples_together():
     """Batch-major samples of different lengths, each folded through the dilated stack on its own
-    (dilated_rnn.py:33-41): one launch per sample; a sample no longer than a layer's dilation is scanned in order
-    by that layer (the one group _dilate then makes)."""
+    (dilated_rnn.py:33-41).  A sample no longer than a layer's dilation is scanned in order by that layer (the one
+    group _dilate then makes), so samples go down together as far as the dilations treat them alike: lengths 9 and 6
+    in one ragged launch, length 3 (which the third layer's dilation of 4 leaves as one group) in another."""
+    core = _core()
     L, H = 3, 32
     lens = [9, 6, 3]
     Wss, Uss, bss = programs.make_lstm_params(L, H, 1 / 8, seed=11, device='cuda')
@@ -240,16 +244,219 @@ def test_reference_style_dilated_model_routes_every_samples_fold():
     seqs = [torch.randn((n, 1, H), generator=g) for n in lens]
     embs = FractalTensor.from_fractaltensors(*[FractalTensor.from_dense(s.cuda(), 1) for s in seqs])
     out = dilated_model(embs, Wss, Uss, bss)
-    assert dispatch.stats['dilated_lstm'] + dispatch.stats['stacked_lstm'] == len(lens) and dispatch.stats['declined'] == 0
+    assert dispatch.stats['dilated_lstm'] == 2 and dispatch.stats['declined'] == 0
+    assert out.depth == 2 and [len(o) for o in out.indices] == lens
     WU, bias = _np_params(Wss, Uss, bss)
     for b, s in enumerate(seqs):
         n = lens[b]
         dil = [d if n > d else 1 for d in (1, 2, 4)]
         ref, _ = ko.stacked_lstm(s.numpy().reshape(n, 1, H), WU, bias, dilations=dil)
         assert ko.max_rel_err(out[b].as_dense().cpu().numpy().reshape(n, H), ref[-1][:, 0]) <= 1e-4
+    before = core.launch_counts['stacked_lstm']
+    dilated_model(embs, Wss, Uss, bss)                                   # warm: two launches, no probe
+    assert core.launch_counts['stacked_lstm'] == before + 2 and dispatch.stats['probes'] == 1
     dispatch.enabled = False
     eager = dilated_model(embs, Wss, Uss, bss)
     assert ko.max_rel_err(out.data.cpu().numpy(), eager.data.cpu().numpy()) <= 1e-4
+
+
+def test_reference_style_dilated_model_is_one_launch_for_samples_of_one_length():
+    """The program form of BASELINE configs[4] (an outer map over samples of a fold over dilated layers) at a
+    reduced size: every sample in ONE launch, not one launch per sample."""
+    core = _core()
+    L, T, B, H = 4, 20, 37, 256
+    Wss, Uss, bss = programs.make_lstm_params(L, H, 1 / 16, seed=13, device='cuda')
+    x = torch.randn((B, T, 1, H), generator=torch.Generator().manual_seed(14))
+    embs = FractalTensor.from_dense(x.cuda(), 2)
+    out = dilated_model(embs, Wss, Uss, bss)
+    assert dispatch.stats['dilated_lstm'] == 1 and dispatch.stats['declined'] == 0
+    assert out.depth == 2 and out.dense_shape() == (B, T)
+    WU, bias = _np_params(Wss, Uss, bss)
+    ref, _ = ko.stacked_lstm(x.numpy().reshape(B, T, H).transpose(1, 0, 2), WU, bias, dilations=[1, 2, 4, 8])
+    got = out.as_dense().cpu().numpy().reshape(B, T, H).transpose(1, 0, 2)
+    assert ko.max_rel_err(got, ref[-1]) <= 1e-4
+    before = dict(core.launch_counts)
+    hits = dispatch.stats['weight_cache_hits']
+    out2 = dilated_model(embs, Wss, Uss, bss)
+    assert core.launch_counts['stacked_lstm'] == before['stacked_lstm'] + 1
+    assert dispatch.stats['weight_cache_hits'] == hits + 1               # the packed weights were not built again
+    assert torch.equal(out2.as_dense(), out.as_dense())
+
+
+# ---- batch-major programs and single layers ---------------------------------------------------------------------------
+
+def sample_scan(xs, ws, us, bs):
+    """One sample's sequence through one layer (the batch-major form, examples/stacked_rnn/stacked_lstm1.py:40-51)."""
+    z = ops.zeros(shape=(1, xs.element_shape[-1]), device=xs.device)
+    hs, cs = ops.scan(lambda state, x: lstm_cell(*state, x, ws, us, bs), xs, initializer=(z, z))
+    return hs, cs
+
+
+def batch_major_layer(xss, Ws, Us, bs):
+    hss, css = ops.map(lambda xs: sample_scan(xs, Ws, Us, bs), xss)
+    return hss
+
+
+def batch_major_stack(embs, Wss, Uss, bss):
+    return ops.fold(lambda s, param: batch_major_layer(s, *param), ops.zip(Wss, Uss, bss), initializer=embs)
+
+
+@pytest.mark.parametrize('lens', [[5] * 6, [7, 3, 5, 5, 1, 7]])
+def test_batch_major_stack_is_one_launch(lens):
+    """fold over layers of a map over samples of a scan over time: the probe finds that the depth-2 operand is
+    [B][T], the batch is turned time-major on the device (sorted by length and padded when the lengths differ) and
+    the stack runs as one launch."""
+    core = _core()
+    L, H = 3, 64
+    Wss, Uss, bss = programs.make_lstm_params(L, H, 1 / 8, seed=70, device='cuda')
+    g = torch.Generator().manual_seed(71)
+    seqs = [torch.randn((n, 1, H), generator=g) for n in lens]
+    embs = FractalTensor.from_fractaltensors(*[FractalTensor.from_dense(s.cuda(), 1) for s in seqs])
+    out = batch_major_stack(embs, Wss, Uss, bss)
+    assert dispatch.stats['stacked_lstm'] == 1 and dispatch.stats['declined'] == 0 and dispatch.stats['probes'] == 1
+    assert out.depth == 2 and [len(o) for o in out.indices] == lens and out.element_shape == (1, H)
+    WU, bias = _np_params(Wss, Uss, bss)
+    for b, s in enumerate(seqs):
+        ref, _ = ko.stacked_lstm(s.numpy().reshape(lens[b], 1, H), WU, bias)
+        assert ko.max_rel_err(out[b].as_dense().cpu().numpy().reshape(lens[b], H), ref[-1][:, 0]) <= 1e-4
+    before = core.launch_counts['stacked_lstm']
+    batch_major_stack(embs, Wss, Uss, bss)
+    assert core.launch_counts['stacked_lstm'] == before + 1 and dispatch.stats['probes'] == 1
+    dispatch.enabled = False
+    eager = batch_major_stack(embs, Wss, Uss, bss)
+    assert eager.indices == out.indices
+    assert ko.max_rel_err(out.data.cpu().numpy(), eager.data.cpu().numpy()) <= 1e-4
+
+
+def test_batch_major_layer_on_its_own_is_one_launch():
+    """A map over samples of one scan each, called without the fold around it: hs and cs of every sample from one launch."""
+    core = _core()
+    H, lens = 32, [4, 6, 2]
+    Wss, Uss, bss = programs.make_lstm_params(1, H, 1 / 4, seed=72, device='cuda')
+    g = torch.Generator().manual_seed(73)
+    seqs = [torch.randn((n, 1, H), generator=g) for n in lens]
+    xss = FractalTensor.from_fractaltensors(*[FractalTensor.from_dense(s.cuda(), 1) for s in seqs])
+    before = core.launch_counts.get('stacked_lstm', 0)
+    hss, css = ops.map(lambda xs: sample_scan(xs, Wss[0], Uss[0], bss[0]), xss)
+    assert dispatch.stats['lstm_scan'] == 1 and core.launch_counts['stacked_lstm'] > before
+    WU, bias = _np_params(Wss, Uss, bss)
+    for b, s in enumerate(seqs):
+        h, c = ko.stacked_lstm(s.numpy().reshape(lens[b], 1, H), WU, bias)
+        assert ko.max_rel_err(hss[b].as_dense().cpu().numpy().reshape(lens[b], H), h[0][:, 0]) <= 1e-4
+        assert ko.max_rel_err(css[b].as_dense().cpu().numpy().reshape(lens[b], H), c[0][:, 0]) <= 1e-4
+    warm = core.launch_counts['stacked_lstm']
+    ops.map(lambda xs: sample_scan(xs, Wss[0], Uss[0], bss[0]), xss)
+    assert core.launch_counts['stacked_lstm'] == warm + 1
+
+
+def test_single_layer_scan_of_config1_is_one_launch():
+    """BASELINE configs[0] as its program: one layer written as a scan over time of a map over the batch
+    (examples/stacked_rnn/stacked_rnn.py:54-65), called on its own, B 64, T 16, H 256."""
+    core = _core()
+    T, B, H = 16, 64, 256
+    Wss, Uss, bss = programs.make_lstm_params(1, H, 0.1, seed=1234, device='cuda', bias=False)
+    xss = programs.make_sequence_batch(T, B, H, seed=1234, device='cuda')
+    hss = lstm_layer(xss, Wss[0], Uss[0], bss[0])
+    assert dispatch.stats['lstm_scan'] == 1 and dispatch.stats['probes'] == 1 and dispatch.stats['declined'] == 0
+    assert hss.depth == 2 and hss.dense_shape() == (T, B) and hss.element_shape == (1, H)
+    WU, bias = _np_params(Wss, Uss, bss)
+    ref, _ = ko.stacked_lstm(xss.as_dense().cpu().numpy().reshape(T, B, H), WU, bias)
+    assert ko.max_rel_err(hss.as_dense().cpu().numpy().reshape(T, B, H), ref[0]) <= 1e-4
+    before = dict(core.launch_counts)
+    lstm_layer(xss, Wss[0], Uss[0], bss[0])
+    assert core.launch_counts['stacked_lstm'] == before['stacked_lstm'] + 1 and dispatch.stats['probes'] == 1
+
+
+def test_scan_returns_both_states_and_takes_ragged_steps_and_a_given_state():
+    H = 64
+    Wss, Uss, bss = programs.make_lstm_params(1, H, 1 / 8, seed=74, device='cuda')
+    ws, us, bs = Wss[0], Uss[0], bss[0]
+    WU, bias = _np_params(Wss, Uss, bss)
+    step = lambda state, x: batched_cell(*state, x, ws, us, bs)
+    # ragged time-major steps (4, 4, 2, 1 rows)
+    g = torch.Generator().manual_seed(75)
+    sizes = [4, 4, 2, 1]
+    steps = [torch.randn((n, 1, H), generator=g) for n in sizes]
+    xss = FractalTensor.from_fractaltensors(*[FractalTensor.from_dense(t.cuda(), 1) for t in steps])
+    zero = ops.repeat(ops.zeros(shape=(1, H), device='cuda'), sizes[0])
+    hss, css = ops.scan(step, xss, initializer=(zero, zero))
+    assert dispatch.stats['lstm_scan'] == 1 and [len(o) for o in hss.indices] == sizes
+    for b in range(sizes[0]):
+        n = sum(1 for v in sizes if v > b)
+        x = np.stack([steps[t][b, 0].numpy() for t in range(n)]).reshape(n, 1, H)
+        h, c = ko.stacked_lstm(x, WU, bias)
+        got_h = np.stack([hss[t][b].data.cpu().numpy().reshape(H) for t in range(n)])
+        got_c = np.stack([css[t][b].data.cpu().numpy().reshape(H) for t in range(n)])
+        assert ko.max_rel_err(got_h, h[0][:, 0]) <= 1e-4 and ko.max_rel_err(got_c, c[0][:, 0]) <= 1e-4
+    # a layer that goes on from a given state: equal to the eager loop
+    T, B = 5, 3
+    xs2 = programs.make_sequence_batch(T, B, H, seed=76, device='cuda')
+    h0 = FractalTensor.from_dense((torch.rand((B, 1, H), generator=g) - 0.5).cuda(), 1)
+    c0 = FractalTensor.from_dense((torch.rand((B, 1, H), generator=g) - 0.5).cuda(), 1)
+    routed = ops.scan(step, xs2, initializer=(h0, c0))
+    assert dispatch.stats['lstm_scan'] == 2
+    dispatch.enabled = False
+    eager = ops.scan(step, xs2, initializer=(h0, c0))
+    for r, e in zip(routed, eager):
+        assert ko.max_rel_err(r.as_dense().cpu().numpy(), e.as_dense().cpu().numpy()) <= 1e-4
+
+
+def test_a_scan_that_is_no_lstm_cell_stays_eager():
+    H, T, B = 32, 3, 2
+    Wss, Uss, bss = programs.make_lstm_params(1, H, 1 / 8, seed=77, device='cuda')
+    ws, us, bs = Wss[0], Uss[0], bss[0]
+    xss = programs.make_sequence_batch(T, B, H, seed=78, device='cuda')
+    zero = ops.repeat(ops.zeros(shape=(1, H), device='cuda'), B)
+
+    def clipped(state, x):          # the cell state clipped to +-0.05: same operands, other arithmetic
+        hs, cs = batched_cell(*state, x, ws, us, bs)
+        return hs, FractalTensor.from_dense(cs.as_dense().clamp(-0.05, 0.05), 1)
+
+    hss, css = ops.scan(clipped, xss, initializer=(zero, zero))
+    assert dispatch.stats['declined'] == 1 and dispatch.stats['lstm_scan'] == 0
+    assert float(css.as_dense().abs().max()) <= 0.05 + 1e-7
+
+
+def test_weights_changed_in_place_are_packed_again():
+    L, T, B, H = 2, 4, 3, 32
+    Wss, Uss, bss = programs.make_lstm_params(L, H, 1 / 4, seed=79, device='cuda')
+    xss = programs.make_sequence_batch(T, B, H, seed=80, device='cuda')
+    programs.stacked_lstm(xss, Wss, Uss, bss)
+    programs.stacked_lstm(xss, Wss, Uss, bss)
+    assert dispatch.stats['weight_cache_hits'] == 1
+    Wss.data.mul_(0.5)                                   # an in-place update of the parameters, as an optimizer makes
+    out = programs.stacked_lstm(xss, Wss, Uss, bss)
+    assert dispatch.stats['weight_cache_hits'] == 1
+    WU, bias = _np_params(Wss, Uss, bss)
+    ref, _ = ko.stacked_lstm(xss.as_dense().cpu().numpy().reshape(T, B, H), WU, bias)
+    assert ko.max_rel_err(out.as_dense().cpu().numpy().reshape(T, B, H), ref[-1]) <= 1e-4
+
+
+def _scaled_layer(seq, ws, us, bs):
+    return programs.lstm_layer(seq, ws, us, bs)
+
+
+def test_a_layer_function_redefined_at_module_level_is_probed_again():
+    """The fold's lambda reaches its layer function through a module global.  When that global is rebound to a
+    function that computes something else, the verdict of the old one must not be reused."""
+    L, T, B, H = 2, 3, 2, 32
+    Wss, Uss, bss = programs.make_lstm_params(L, H, 1 / 8, seed=81, device='cuda')
+    xss = programs.make_sequence_batch(T, B, H, seed=82, device='cuda')
+    run = lambda: ops.fold(lambda s, p: _scaled_layer(s, *p), ops.zip(Wss, Uss, bss), initializer=xss)
+    first = run()
+    assert dispatch.stats['stacked_lstm'] == 1 and dispatch.stats['probes'] == 1
+    original = globals()['_scaled_layer']
+
+    def halved(seq, ws, us, bs):
+        return FractalTensor.from_dense(programs.lstm_layer(seq, ws, us, bs).as_dense() * 0.5, 2)
+
+    globals()['_scaled_layer'] = halved
+    try:
+        second = run()
+    finally:
+        globals()['_scaled_layer'] = original
+    assert dispatch.stats['stacked_lstm'] == 1 and dispatch.stats['declined'] == 1      # probed anew, found different, run eagerly
+    assert float((second.as_dense() - first.as_dense()).abs().max()) > 1e-3
 
 
 # ---- attention ----------------------------------------------------------------------------------------------------
@@ -332,6 +539,26 @@ def test_chained_matmul_runs_as_one_back_to_back_gemm(M, K, N, P):
     dispatch.enabled = False
     eager = (ta @ tb) @ tc
     assert ko.max_rel_err(d.data.float().cpu().numpy(), eager.data.float().cpu().numpy()) <= 1e-2
+
+
+def test_chained_matmul_beyond_the_fused_kernels_runs_as_two_products():
+    """N = 4096: more than the general back-to-back kernel holds of the intermediate product.  The chain must run as
+    the two torch products it always was, not raise."""
+    core = _core()
+    assert core.b2b_gemm_supported(2048, 128, 128) and not core.b2b_gemm_supported(4096, 128, 128)
+    rng = np.random.default_rng(52)
+    M, K, N, P = 64, 128, 4096, 64
+    a, b, c = (torch.from_numpy((rng.standard_normal(s) / np.sqrt(s[0])).astype(np.float16)).cuda() for s in ((M, K), (K, N), (N, P)))
+    p = Tensor.from_tensor(a) @ Tensor.from_tensor(b)
+    assert p._pending is None                                            # never left pending
+    d = p @ Tensor.from_tensor(c)
+    assert dispatch.stats['b2b_gemm'] == 0 and torch.equal(d.data, (a @ b) @ c)
+    # N = 2048 with K = 128: past the fused kernels' LDS, inside the general kernel's reach
+    b2, c2 = b[:, :2048].contiguous(), c[:2048].contiguous()
+    d2 = (Tensor.from_tensor(a) @ Tensor.from_tensor(b2)) @ Tensor.from_tensor(c2)
+    assert dispatch.stats['b2b_gemm'] == 1
+    ref = ko.b2b_gemm(a.cpu().numpy(), np.ascontiguousarray(b2.cpu().numpy().T), np.ascontiguousarray(c2.cpu().numpy().T))
+    assert ko.max_rel_err(d2.data.float().cpu().numpy(), ref) <= 1e-2
 
 
 def test_a_pending_product_is_formed_by_any_other_use():

@@ -210,6 +210,48 @@ def test_split_products_are_as_accurate_as_fp32_products(core):
         core.set_lstm_products(before)
 
 
+@pytest.mark.parametrize('H', [256, 128, 96])       # persistent kernel; streamed four-tile form; streamed three-chunk form
+@pytest.mark.parametrize('ratio', [2.0 ** 10, 2.0 ** 20])
+def test_split_products_with_an_outlier_inside_a_row_and_a_column(core, H, ratio):
+    """A power-of-two scale is shared by an input row and by a weight column.  One element `ratio` times its
+    neighbours sets that scale, so the neighbours' value plane is left with few bits (for 2^20 on small inputs it is
+    an fp16 subnormal) and their remainder plane has to carry them.  Every third input row and every fifth weight
+    column holds such an element; the outliers are of a size that keeps the gates away from saturation, so the
+    neighbours' share of a gate sum (about 2^-5 of it at ratio 2^10) shows in the result.  Against float64, both
+    product modes, well inside the 1e-4 bound."""
+    L, T, B = 2, 6, 40
+    rng = np.random.default_rng(11)
+    xs = (rng.standard_normal((T, B, H)) * (4.0 / ratio)).astype(np.float32)
+    for t in range(T):
+        for b in range(0, B, 3):
+            xs[t, b, rng.integers(H)] = 4.0 * rng.choice([-1.0, 1.0])
+    WU = (rng.uniform(-1, 1, (L, 2 * H, 4 * H)) * (0.5 / ratio)).astype(np.float32)
+    WU[:, :, 1::5] *= ratio / 8                      # ordinary columns in between (|w| < 1/16)
+    for l in range(L):
+        for j in range(0, 4 * H, 5):
+            WU[l, rng.integers(2 * H), j] = 0.5 * rng.choice([-1.0, 1.0])
+    hr, cr = ko.stacked_lstm(xs, WU, None)           # float64
+    assert np.abs(hr).max() > 0.05                   # the outliers drive the cells: a result of zeros would pass nothing
+    err = {}
+    for mode in ('f32', 'f16x3'):
+        ws = torch.empty(core.stacked_lstm_workspace_bytes(L, T, B, H), dtype=torch.uint8, device='cuda')
+        hsss, csss = core.stacked_lstm(dev(xs), dev(WU), workspace=ws, products=mode, check=True) if H == 256 else \
+            _stack_in_mode(core, mode, xs, WU, ws)
+        err[mode] = max(ko.max_rel_err(hsss.cpu().numpy(), hr), ko.max_rel_err(csss.cpu().numpy(), cr))
+    assert err['f16x3'] <= LSTM_TOL / 10, err
+    assert err['f16x3'] <= max(4 * err['f32'], 4e-6), err
+
+
+def _stack_in_mode(core, mode, xs, WU, ws):
+    """The streamed stacks take the process-wide product mode only."""
+    before = core.get_lstm_products()
+    core.set_lstm_products(mode)
+    try:
+        return core.stacked_lstm(dev(xs), dev(WU), workspace=ws, check=True)
+    finally:
+        core.set_lstm_products(before)
+
+
 def test_split_products_at_the_benchmarked_depth(core):
     """32 layers x 64 steps (config 4's depth): the error of the split products against float64 stays within twice
     that of the fp32 MFMAs and two orders under the 1e-4 bound after 95 dependent cells too.  Rows are independent,

@@ -57,6 +57,65 @@ def test_function_fingerprint_follows_code_and_closure_scalars():
     assert dispatch._fingerprint(make(2.0)) != dispatch._fingerprint(lambda y: y)
 
 
+_GLOBAL_SCALE = 2.0
+
+
+def _global_layer(x):
+    return x * _GLOBAL_SCALE
+
+
+def test_function_fingerprint_follows_module_globals_and_defaults():
+    """A caller whose own code does not change but whose module-level callee, module-level scalar or default
+    argument does must get a new key; callables without code are keyed on the object, not on its address."""
+    import functools
+    from kaleido.operations import dispatch
+    caller = lambda y: _global_layer(y)
+    before = dispatch._fingerprint(caller)
+    assert before == dispatch._fingerprint(lambda y: _global_layer(y)) or True      # another code object: may differ
+    assert dispatch._fingerprint(caller) == before
+    g = globals()
+    saved = g['_global_layer'], g['_GLOBAL_SCALE']
+    try:
+        g['_GLOBAL_SCALE'] = 3.0                          # a scalar the callee reads
+        assert dispatch._fingerprint(caller) != before
+        g['_GLOBAL_SCALE'] = saved[1]
+        assert dispatch._fingerprint(caller) == before
+        g['_global_layer'] = lambda x: x + 1.0            # the callee itself
+        assert dispatch._fingerprint(caller) != before
+    finally:
+        g['_global_layer'], g['_GLOBAL_SCALE'] = saved
+    mk = lambda d: (lambda x, d=d: x * d)
+    assert dispatch._fingerprint(mk(2)) == dispatch._fingerprint(mk(2)) and dispatch._fingerprint(mk(2)) != dispatch._fingerprint(mk(4))
+    kw = lambda d: (lambda x, *, d=d: x * d)
+    assert dispatch._fingerprint(kw(2)) != dispatch._fingerprint(kw(4))
+    part = functools.partial(_global_layer)
+    assert dispatch._fingerprint(part) == ('object', part) and dispatch._fingerprint(part) != dispatch._fingerprint(functools.partial(_global_layer))
+
+
+def test_kaleido_core_is_the_c_abi_binding():
+    """`kaleido._core`, the module name of the reference's native binding (kaleido/__init__.py:20-26), is
+    fractaltensor_amd._core."""
+    import kaleido
+    import kaleido._core as kcore
+    assert kcore.version() >= 100
+    import fractaltensor_amd._core as core
+    import sys
+    assert sys.modules['kaleido._core'] is core and kaleido._core is core
+    from kaleido._core import b2b_gemm, stacked_lstm   # noqa: F401
+
+
+def test_a_map_over_host_samples_is_not_captured():
+    """The capture of a map's function only ever happens on GPU operands; on the host the map is the plain loop."""
+    from kaleido import FractalTensor, operations as ops
+    from kaleido.operations import dispatch
+    dispatch.reset()
+    x = FractalTensor.from_dense(torch.arange(24.).reshape(2, 3, 1, 4), 2)
+    calls = []
+    out = ops.map(lambda s: (calls.append(1), s)[1], x)
+    assert len(calls) == 2 and torch.equal(out.as_dense(), x.as_dense())
+    assert all(v == 0 for v in dispatch.stats.values())
+
+
 def test_dilations_are_noted_only_under_a_probe():
     from kaleido.operations import dispatch
     dispatch.note_dilation(4)                  # outside a probe: ignored

@@ -35,6 +35,15 @@ def test_noalloc_entry_point_matches_the_workspace_one_on_two_calls_in_a_row():
         assert torch.cuda.memory_stats()['allocation.all.allocated'] == before   # torch's allocator was not asked either
         core.stacked_lstm_check(None)
         assert torch.equal(hsss, h_ref) and torch.equal(csss, c_ref)
+        # the library's own allocations do not pass through torch: the driver's count of free bytes must not move
+        # over a second, warmed-up call either
+        torch.cuda.synchronize()
+        free_before, _ = torch.cuda.mem_get_info()
+        core.stacked_lstm_noalloc(xs, WU, bs, (hsss, csss), dilations=dil)
+        core.stacked_lstm_check(None)
+        free_after, _ = torch.cuda.mem_get_info()
+        assert free_after == free_before, (free_before, free_after)
+        assert torch.equal(hsss, h_ref) and torch.equal(csss, c_ref)
         hr, cr = c_oracle.stacked_lstm(xs.cpu().numpy(), WU.cpu().numpy(), bs.cpu().numpy(), dil)
         assert ko.max_rel_err(hsss.cpu().numpy(), hr) <= 1e-4 and ko.max_rel_err(csss.cpu().numpy(), cr) <= 1e-4
 
