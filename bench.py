@@ -99,10 +99,11 @@ def _host_timed(torch, fn, warm, runs):
 def _lstm_torch_cpu(torch, xs, WU, dil=None):
     """The batched LSTM loop on torch CPU: per layer and step one [B, 2H] @ [2H, 4H] product and the gate arithmetic
     as torch operators (the batched form of examples/stacked_rnn/stacked_rnn.py:23-65 and of
-    benchmarks/rnn/baselines/stacked_lstm/pt_model/rnn.py:94-108).  Returns the last layer's h [T, B, H]."""
+    benchmarks/rnn/baselines/stacked_lstm/pt_model/rnn.py:94-108).  Returns every layer's h, a list of [T, B, H]."""
     L = WU.shape[0]
     T, B, H = xs.shape
     inp = xs
+    layers = []
     for l in range(L):
         d = 1 if dil is None else dil[l]
         hs, cs = [], []
@@ -116,7 +117,8 @@ def _lstm_torch_cpu(torch, xs, WU, dil=None):
             hs.append(h)
             cs.append(c)
         inp = torch.stack(hs)
-    return inp
+        layers.append(inp)
+    return layers
 
 
 def bench_b2b(torch, core, steps, warmup, cpu):
@@ -590,6 +592,7 @@ def bench_lstm(torch, core, steps, warmup, cpu, dilated, baselines=True):
     ms, wall = _events_ms(torch, fused, steps, warmup)
     status = core.persistent_status(ws)
     assert status == 0, 'the persistent launch drained early'
+    small_states = core.stacked_lstm_small_states(ws)
     ref_h = hs.clone()
     executed = 3.0 * flop if products == 'f16x3' else flop      # MFMA flops the kernel issues
     peak = PEAK_F16_TFLOPS if products == 'f16x3' else PEAK_F32_MATRIX_TFLOPS
@@ -666,14 +669,24 @@ def bench_lstm(torch, core, steps, warmup, cpu, dilated, baselines=True):
         # arithmetic as torch operators per layer and step
         xc, WUc = xs.cpu(), WU.cpu()
         out, med, best, threads = _host_timed(torch, lambda: _lstm_torch_cpu(torch, xc, WUc, dil), 1, 3)
-        ref = ref_h[L - 1].cpu()
-        diff = float((out - ref).abs().max() / ref.abs().max())
+        # the tolerance of the path: largest difference over the whole output (every layer's h) relative to its largest
+        # value.  Beside it, per layer relative to that layer's own largest value: layers that fade towards zero
+        # (config 4's upper ones: no bias, small weights) fall below what the fixed scale of the split products'
+        # fp16 planes resolves, which the status block's small-states word reports (ftk_stacked_lstm_small_states)
+        top = max(float(o.abs().max()) for o in out)
+        per_layer = [(float((ref_h[l].cpu() - out[l]).abs().max()), float(out[l].abs().max())) for l in range(L)]
+        diff = max(e for e, _ in per_layer) / top
         assert diff <= 1e-4, diff
+        worst = max(range(L), key=lambda l: per_layer[l][0] / max(per_layer[l][1], 1e-300))
+        layer_rel = {'worst_layer': worst, 'rel_to_that_layers_max': per_layer[worst][0] / max(per_layer[worst][1], 1e-300),
+                     'that_layers_max_abs_h': per_layer[worst][1], 'top_layers_max_abs_h': per_layer[L - 1][1],
+                     'small_states_word': small_states}
         res['cpu_baseline'] = {'value': B / med, 'unit': 'sequences/s', 'cores': threads, 'kind': 'torch_cpu_eager',
                                'sample': f'the whole configuration: per layer and step one [{B},{2 * H}] @ [{2 * H},{4 * H}] product '
                                          f'and the gate arithmetic as torch CPU operators (fp32), torch.set_num_threads({threads}) '
                                          f'of {os.cpu_count()} host CPUs, 1 warm-up + 3 timed runs, median {med:.2f} s (min {best:.2f} s)',
-                               'ms_per_step': med * 1e3, 'max_rel_diff_vs_gpu': diff, 'gpu_speedup': med * 1e3 / ms}
+                               'ms_per_step': med * 1e3, 'max_rel_diff_vs_gpu': diff, 'per_layer_diff_vs_gpu': layer_rel,
+                               'gpu_speedup': med * 1e3 / ms}
         # the per-sample operator program (scan over time of map over batch of [1,H] cells, four gate products per
         # cell: the reference's execution model) on a bounded sample, scaled by cells to the configuration
         from fractaltensor_amd import programs

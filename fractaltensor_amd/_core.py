@@ -21,7 +21,7 @@ EXPORTS = (
     'ftk_lstm_cell_f32', 'ftk_lstm_cell_f16', 'ftk_lstm_layer_f32', 'ftk_lstm_layer_f16', 'ftk_lstm_elementwise_f32',
     'ftk_stacked_lstm_workspace_bytes', 'ftk_stacked_lstm_f32', 'ftk_dilated_lstm_f32',
     'ftk_stacked_lstm_wavefront_f32', 'ftk_stacked_lstm_ragged_f32', 'ftk_lstm_set_products', 'ftk_lstm_get_products',
-    'ftk_stacked_lstm_opts_f32', 'ftk_stacked_lstm_status', 'ftk_stacked_lstm_noalloc_f32',
+    'ftk_stacked_lstm_opts_f32', 'ftk_stacked_lstm_status', 'ftk_stacked_lstm_small_states', 'ftk_stacked_lstm_noalloc_f32',
     'ftk_stacked_lstm_f16_workspace_bytes', 'ftk_stacked_lstm_f16',
     'ftk_b2b_gemm_f16', 'ftk_b2b_gemm_f16_supported', 'ftk_b2b_gemm_rowmajor_f16', 'ftk_gemm_f16', 'ftk_batched_gemm_f16', 'ftk_flash_attn_f16', 'ftk_online_softmax_f32', 'ftk_embedding_gather_f32',
     'ftk_grid_rnn_workspace_bytes', 'ftk_grid_rnn_f32', 'ftk_windowed_attn_f32',
@@ -228,7 +228,8 @@ def stacked_lstm(xs, WU, bias=None, dilations: Optional[Sequence[int]] = None, s
                  out: Optional[Tuple[torch.Tensor, torch.Tensor]] = None,
                  workspace: Optional[torch.Tensor] = None,
                  active_rows: Optional[Sequence[int]] = None, products: Optional[str] = None,
-                 spin_limit: int = 0, check: Optional[bool] = None) -> Tuple[torch.Tensor, torch.Tensor]:
+                 spin_limit: int = 0, check: Optional[bool] = None, exact_small_states: bool = False
+                 ) -> Tuple[torch.Tensor, torch.Tensor]:
     """xs [T,B,H], WU [L,2H,4H], bias [L,4H] or None -> hsss, csss [L,T,B,H].
 
     schedule: 'auto' (persistent kernel when the shape allows, else per-stage
@@ -240,6 +241,9 @@ def stacked_lstm(xs, WU, bias=None, dilations: Optional[Sequence[int]] = None, s
     check: wait for the stream and raise FtkError (code -6) if the persistent launch gave up a wait and left
     the outputs incomplete.  Default: True when the workspace is allocated here (nobody else could look at its
     status word afterwards), False when the caller passes one (check it with stacked_lstm_check(workspace)).
+    exact_small_states: after a call on split products, wait for the stream and, if hidden states too small for
+    the fixed scale of their fp16 planes were written (stacked_lstm_small_states), compute the stack again on fp32
+    products, so that layers that fade towards zero are accurate relative to their own size as well.
     """
     f32 = torch.float32
     _req(xs, f32, 'xs'); _req(WU, f32, 'WU')
@@ -297,6 +301,10 @@ def stacked_lstm(xs, WU, bias=None, dilations: Optional[Sequence[int]] = None, s
                                         ci(L), ci(T), ci(B), ci(H), _ptr(workspace), ws_bytes, _stream()))
     if check:
         stacked_lstm_check(workspace)
+    if exact_small_states and products != 'f32' and stacked_lstm_small_states(workspace):
+        _count('stacked_lstm_repeated_on_f32_products')
+        return stacked_lstm(xs, WU, bias, dilations=dilations, out=(hsss, csss), workspace=workspace, active_rows=active_rows,
+                            products='f32', spin_limit=spin_limit, check=check)
     return hsss, csss
 
 
@@ -331,6 +339,19 @@ def stacked_lstm_check(workspace: Optional[torch.Tensor]) -> None:
     if workspace is not None:
         _req_workspace(workspace)
     _check(lib.ftk_stacked_lstm_status(_ptr(workspace), _stream()))
+
+
+def stacked_lstm_small_states(workspace: torch.Tensor) -> bool:
+    """Waits for the current stream; True if the last fp32 stacked-LSTM call given this workspace ran on split
+    products and wrote hidden states too small for the fixed scale of their fp16 planes (non-zero |h| below 2^-37
+    at H = 256, 2^-26 at other hidden sizes): such values reach the cells that read them with fewer than 13 bits.
+    The whole output is still accurate relative to its largest value; layers that faded that far are not accurate
+    relative to themselves.  stacked_lstm(..., exact_small_states=True) repeats such a call on fp32 products."""
+    _req_workspace(workspace)
+    rc = lib.ftk_stacked_lstm_small_states(_ptr(workspace), _stream())
+    if rc < 0:
+        _check(rc)
+    return rc == 1
 
 
 def stacked_lstm_f16(xs, WU, bias=None, dilations: Optional[Sequence[int]] = None,

@@ -84,6 +84,9 @@ constexpr int kMaxBlocks = 64;     // 32-row blocks a ragged batch may have (B <
 constexpr int kSplitTop = 14;          // a scale group's largest magnitude lands in [2^14, 2^15)
 constexpr float kSplitRest = 2048.0f;  // 2^11: what the remainder is multiplied by before it is rounded
 constexpr float kSplitAct = 16384.0f;  // 2^14: the scale of h
+// h * 2^14 below 2^-23 (|h| < 2^-37, 7e-12): the remainder plane is an fp16 subnormal there and value plus remainder
+// keep fewer than 13 bits
+constexpr unsigned kSmallStateBits = (127u - 23u) << 23;
 
 struct PersistArgs {
   const float* xs;
@@ -191,7 +194,8 @@ constexpr int kStageRow32 = 144, kStageRow16 = 80;
 constexpr int kStageC = 0, kStageH = 32 * kStageRow32, kStageTop = 2 * 32 * kStageRow32, kStageRest = kStageTop + 32 * kStageRow16;
 constexpr int kStageBytes = kStageRest + 32 * kStageRow16;
 constexpr int kRatioOffset = 2 * P_TILE * (int)sizeof(float) + 1024 + 2 * kStageBytes;   // bytes; [2 tile buffers][64 floats]
-constexpr size_t kPersistLds = (size_t)kRatioOffset + 2 * 64 * sizeof(float);  // tiles, prefetch scrap, staging, row ratios
+constexpr int kVoteOffset = kRatioOffset + 2 * 64 * (int)sizeof(float);   // bytes; one int per wave (serial schedule)
+constexpr size_t kPersistLds = (size_t)kVoteOffset + 64;  // tiles, prefetch scrap, staging, row ratios, votes
 // Kernel flavours.  kProductsF32 / kProductsSplit: fp32 data, H = 256, the two ways of forming the products.
 // kHalfData: fp16 inputs, weights, h and c (what the reference's CuTe LSTM stores), one fp16 MFMA per product
 // with fp32 accumulation, H = 512: a row of 512 fp16 takes the 1024 bytes a row of 256 fp32 takes, and a
@@ -596,6 +600,7 @@ void lstm_persistent_kernel(PersistArgs a) {
   // units] per output, rows padded against bank conflicts), and after a barrier wave w stores rows
   // 8w..8w+7: 128 contiguous bytes of c and h per row, 64 of each fp16 plane.
   unsigned char* const stage = reinterpret_cast<unsigned char*>(tile + 2 * P_TILE + 256);
+  bool small_reported = false;   // this wave has set the status block's small-states word
   auto stage_results = [&](const float (&hv)[4], const float (&cv)[4], int sbuf) __attribute__((always_inline)) {
     unsigned char* sb = stage + sbuf * kStageBytes;
     const int c4 = 8 * wave + 4 * hh;
@@ -610,14 +615,25 @@ void lstm_persistent_kernel(PersistArgs a) {
     *reinterpret_cast<float4*>(sb + kStageH + j * kStageRow32 + 4 * c4) = make_float4(hv[0], hv[1], hv[2], hv[3]);
     if constexpr (SPLIT) {
       v4h top, rest;
+      unsigned smallest = 0xffffffffu;  // bit pattern of the smallest non-zero |h * 2^14|, less one (zero wraps to the top)
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
         const float v = hv[r] * kSplitAct;
         top[r] = (_Float16)v;
         rest[r] = (_Float16)((v - (float)top[r]) * kSplitRest);
+        smallest = min(smallest, (__float_as_uint(v) & 0x7fffffffu) - 1u);
       }
       *reinterpret_cast<v4h*>(sb + kStageTop + j * kStageRow16 + 2 * c4) = top;
       *reinterpret_cast<v4h*>(sb + kStageRest + j * kStageRow16 + 2 * c4) = rest;
+      // the planes have a fixed scale: below kSmallState the two of them hold fewer than 13 bits of a value, and the
+      // cells that read it see it less accurately than 1e-4 of ITS size (the fp32 h and c in hsss / csss are exact
+      // either way).  The status block's second word tells the caller that this happened.
+      // (once per wave: a store per item to one word from every compute unit of a faded layer queues up behind
+      // itself, and the wait for an item's stores then waits for it)
+      if (!small_reported && __builtin_amdgcn_ballot_w64(smallest < kSmallStateBits - 1u) != 0) {
+        small_reported = true;
+        if (lane == 0) __hip_atomic_store(a.status + 1, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      }
     }
   };
   auto epilogue_to_lds = [&](const v16f& acc, const float4& cp, int sbuf) __attribute__((always_inline)) {
@@ -703,8 +719,13 @@ void lstm_persistent_kernel(PersistArgs a) {
     // taken off that chain: the x columns of tile n+1 are requested with the h columns of tile n (when the layer
     // below has them already), and the x half of item n+1 is formed between the stores of item n and the wait
     // for their acknowledgement, which takes longer than those MFMAs.
+    // Whether the layer below is ready is something every wave sees for itself, at its own moment: a wave that
+    // finds it ready requests its rows of the next tile's x columns early, and must not multiply with them before
+    // the other waves' rows are there as well.  So the waves vote through LDS, and the early x half happens only
+    // when all four requested their rows before this item's first barrier.
+    int* const votes = reinterpret_cast<int*>(reinterpret_cast<unsigned char*>(tile) + kVoteOffset);
     bool xdone = false;    // the x half of the current item is in the accumulators already
-    bool xhere = false;    // the x columns of the current item's tile are in LDS (or on their way)
+    bool xhere = false;    // the x columns of this wave's rows of the current item's tile are in LDS (or on their way)
     for (int n = 0; n < n_items; ++n) {
       const int buf = n & 1;
       if (tracing) a.trace[TS * n + 0] = wall_clock64();
@@ -722,8 +743,11 @@ void lstm_persistent_kernel(PersistArgs a) {
         }
       }
       const float4 cp = load_cprev(n);
+      if (lane == 0) votes[wave] = xnext ? 1 : 0;
       __builtin_amdgcn_s_waitcnt(0);
       __syncthreads();
+      const int4 vote = *reinterpret_cast<const int4*>(votes);
+      const bool xall = (vote.x & vote.y & vote.z & vote.w) != 0;   // the whole of tile n+1's x columns has landed
       if (live(n)) {
         if (!xdone) {
           mfma_range(buf, IC<0>{}, IC<0>{}, IC<16>{});
@@ -735,7 +759,7 @@ void lstm_persistent_kernel(PersistArgs a) {
       __syncthreads();  // results staged; the tile may be rewritten by the item after the next
       store_item(n, 0);
       xdone = false;
-      if (xnext) {          // while the stores are acknowledged
+      if (xall) {           // while the stores are acknowledged
         mfma_range(buf ^ 1, IC<0>{}, IC<0>{}, IC<16>{});
         rescale_x(load_ratio(buf ^ 1));
         xdone = true;
@@ -842,7 +866,13 @@ void lstm_persistent_kernel(PersistArgs a) {
     // the counts asked for after the MFMAs have arrived with everything else: one more chance before the slow path
     // (not with fp16 data: an item is short there, and the extra request of counts behind a failed look costs more
     // than the look gains: 1.96 -> 2.36 ms at H = 256)
-    if constexpr (!F16) look(8);
+    // A tile requested here leaves AFTER the wait above, and nothing later in the item waits for it (the copies are
+    // opaque to the compiler, and a wave only ever waits for its own): the wave waits for them on the spot.
+    if constexpr (!F16) {
+      const bool was_pending = pending;
+      look(8);
+      if (was_pending && !pending) __builtin_amdgcn_s_waitcnt(0);   // only the copies are outstanding here: no store has left yet
+    }
     barrier();
     if (tracing) a.trace[TS * n + 5] = wall_clock64();
     store_item(n, buf);
@@ -860,7 +890,7 @@ void lstm_persistent_kernel(PersistArgs a) {
       if (alive) issue_tile(n + 1, buf ^ 1);
       __builtin_amdgcn_s_waitcnt(0);
     }
-    barrier();
+    barrier();   // tile n+1 is complete: every wave that requested a part of it has waited for that part
     if (tracing) a.trace[TS * n + 7] = wall_clock64();
     pending = pending2 && alive;
     fl = fl2;
@@ -1079,8 +1109,9 @@ static int run_persistent(int mode, const void* xs, const void* WU, const float*
 
   // flags and status block start from zero; a later launch of a stack that runs as several keeps the error word
   // of the earlier ones (it then drains at its first long wait, and the call reports the time-out)
-  hipLaunchKernelGGL(fill_zero_kernel, dim3(64), dim3(256), 0, s, a.status + (keep_status ? 1 : 0),
-                     nflags + 64 - (keep_status ? 1 : 0));
+  // (and its word for small states, see ftk_stacked_lstm_small_states)
+  hipLaunchKernelGGL(fill_zero_kernel, dim3(64), dim3(256), 0, s, a.status + (keep_status ? 2 : 0),
+                     nflags + 64 - (keep_status ? 2 : 0));
   rc = check_launch("fill_zero_kernel");
   if (rc) return rc;
 
@@ -1332,6 +1363,15 @@ int ftk_stacked_lstm_status(const void* workspace, ftk_stream_t stream) {
                 "stacked LSTM: a bounded wait of the persistent launch ran out of polls (status word %d); the launch drained "
                 "early and hsss / csss are incomplete", word);
   return FTK_OK;
+}
+
+int ftk_stacked_lstm_small_states(const void* workspace, ftk_stream_t stream) {
+  using namespace ftk;
+  if (!workspace) return fail(FTK_ERR_INVALID_ARGUMENT, "ftk_stacked_lstm_small_states: workspace is NULL");
+  int word = 0;
+  FTK_HIP(hipMemcpyAsync(&word, reinterpret_cast<const int*>(workspace) + 1, sizeof(int), hipMemcpyDeviceToHost, (hipStream_t)stream));
+  FTK_HIP(hipStreamSynchronize((hipStream_t)stream));
+  return word != 0 ? 1 : 0;
 }
 
 int ftk_stacked_lstm_noalloc_f32(const float* xs, const float* WU, const float* bias, const int* dilations, float* hsss,

@@ -52,7 +52,7 @@ from ..tensor import Tensor
 enabled = os.environ.get('FTK_DISPATCH', '1') != '0'
 allow_half_attention = False
 stats = {'stacked_lstm': 0, 'dilated_lstm': 0, 'lstm_scan': 0, 'flash_attention': 0, 'b2b_gemm': 0, 'probes': 0, 'declined': 0,
-         'weight_cache_hits': 0}
+         'weight_cache_hits': 0, 'repeated_on_f32_products': 0}
 
 _verdicts: dict = {}
 _MAX_VERDICTS = 256
@@ -67,7 +67,7 @@ _local = threading.local()
 def reset() -> None:
     """Forget every verdict and zero the counters."""
     _verdicts.clear()
-    _weights.clear()
+    clear_weight_cache()
     for k in stats:
         stats[k] = 0
 
@@ -221,10 +221,12 @@ def _pack_layer(ws, us, bs):
 # torch (a kernel given the raw pointer) are not seen: clear_weight_cache() after such a write.
 _weights: dict = {}
 _MAX_WEIGHTS = 4
+_fading_stacks: set = set()        # packed weights whose last launch on split products met states too small for them
 
 
 def clear_weight_cache() -> None:
     _weights.clear()
+    _fading_stacks.clear()
 
 
 def _packed_stack(layers):
@@ -257,7 +259,18 @@ def _run_lstm(xs: torch.Tensor, WU: torch.Tensor, bias: torch.Tensor, dilations,
     if xs.dtype == torch.float16:
         hsss, csss = core.stacked_lstm_f16(xs.contiguous(), WU.contiguous(), bias.float().contiguous(), dilations=dil, active_rows=active)
     else:
-        hsss, csss = core.stacked_lstm(xs.contiguous(), WU.contiguous(), bias.contiguous(), dilations=dil, active_rows=active)
+        # A program's every layer is accurate relative to its own size: a stack whose hidden states fall below what
+        # the split products' planes resolve is computed again on fp32 products, and goes there directly next time.
+        key = (WU.data_ptr(), WU._version)
+        counter = 'stacked_lstm_repeated_on_f32_products'
+        before = core.launch_counts.get(counter, 0)
+        hsss, csss = core.stacked_lstm(xs.contiguous(), WU.contiguous(), bias.contiguous(), dilations=dil, active_rows=active,
+                                       products='f32' if key in _fading_stacks else None, exact_small_states=True)
+        if core.launch_counts.get(counter, 0) != before:
+            if len(_fading_stacks) >= 64:
+                _fading_stacks.clear()
+            _fading_stacks.add(key)
+            stats['repeated_on_f32_products'] += 1
     return (hsss[-1], csss[-1]) if both else hsss[-1]
 
 

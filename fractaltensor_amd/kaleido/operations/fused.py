@@ -118,7 +118,7 @@ def _run_stack(xss, Wss, Uss, bss, dilations, return_all_layers):
                                            active_rows=sizes)
     else:
         hsss, csss = core.stacked_lstm(xs.float(), WU.float(), None if bias is None else bias.float(), dilations=dilations,
-                                       active_rows=sizes)
+                                       active_rows=sizes, exact_small_states=True)
     L = WU.shape[0]
     if return_all_layers:
         if sizes is None:

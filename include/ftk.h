@@ -271,6 +271,23 @@ int ftk_stacked_lstm_opts_f32(const float* xs, const float* WU, const float* bia
 int ftk_stacked_lstm_status(const void* workspace, ftk_stream_t stream);
 
 /*
+ * Waits for `stream`; 1 if the last fp32 stacked-LSTM call given this
+ * workspace ran on split products (FTK_LSTM_PRODUCTS_F16X3) and met hidden
+ * states too small for them, 0 if not, negative on error.  Split products
+ * hand h from cell to cell as two fp16 planes under a fixed scale (|h| < 1):
+ * the results are accurate to a few 1e-7 of the LARGEST |h|, but a non-zero
+ * |h| below 2^-37 (H = 256; 2^-26 at other hidden sizes) reaches the cells
+ * that read it with fewer than 13 bits, and below about 2^-49 (2^-38) as zero.
+ * A stack whose upper layers fade towards zero (small weights, no bias: the
+ * benchmark configuration) is then exact relative to the whole output and
+ * inexact relative to those layers; a caller that needs every layer accurate
+ * to its own size repeats the call with FTK_LSTM_PRODUCTS_F32 when this
+ * returns 1.  No counterpart in the reference (its CuTe stack is fp16
+ * throughout, benchmarks/rnn/fractaltensor/cute_stacked_lstm/stacked_lstm.cu:16-19).
+ */
+int ftk_stacked_lstm_small_states(const void* workspace, ftk_stream_t stream);
+
+/*
  * ftk_stacked_lstm_opts_f32 with fp32 products for callers that cannot
  * allocate device memory or pass a workspace: tight serving loops, harnesses
  * that forbid hipMalloc, code that prepares a HIP graph.  No counterpart in

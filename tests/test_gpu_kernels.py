@@ -269,6 +269,106 @@ def test_split_products_at_the_benchmarked_depth(core):
     assert err['f16x3'] <= LSTM_TOL / 20, err
 
 
+@pytest.mark.parametrize('H,L', [(256, 32), (128, 24)])          # persistent kernel; streamed split-product cells
+def test_fading_layers_are_reported_and_recomputed_on_fp32_products(core, H, L):
+    """Without a bias and with weights of +-1/16 every layer hands on a fraction of what it receives: thirty layers
+    up the hidden states are 1e-17.  The fp32 outputs are exact to a few 1e-7 of the largest |h| in either product
+    mode, but the split products hand h from cell to cell as fp16 planes under a fixed scale, so the layers that
+    have faded below it are inexact relative to their own size (the top ones come out as zeros).  The library says
+    so (ftk_stacked_lstm_small_states) and exact_small_states=True computes such a stack again on fp32 products:
+    then every layer is within 1e-4 of the float64 result relative to that layer's own largest value."""
+    T, B = 6, 32
+    xs, WU, _ = lstm_inputs(31, L, T, B, H, 1.0 / 16, bias=False)
+    rows = [0, 17, 31]
+    hr, cr = ko.stacked_lstm(xs[:, rows], WU, None)                     # float64
+    assert np.abs(hr[-1]).max() < 1e-12 and np.abs(hr[-1]).max() > 0
+    layer_err = lambda got, ref: max(float(np.abs(got[l] - ref[l]).max() / np.abs(ref[l]).max()) for l in range(L))
+    ws = torch.empty(core.stacked_lstm_workspace_bytes(L, T, B, H), dtype=torch.uint8, device='cuda')
+
+    def run(**kw):
+        before = core.get_lstm_products()
+        if 'products' in kw and H != 256:                                # the streamed stacks take the process-wide mode
+            core.set_lstm_products(kw.pop('products'))
+        try:
+            return core.stacked_lstm(dev(xs), dev(WU), workspace=ws, check=True, **kw)
+        finally:
+            core.set_lstm_products(before)
+
+    h, c = run(products='f16x3')
+    assert core.stacked_lstm_small_states(ws)
+    assert ko.max_rel_err(h[:, :, rows].cpu().numpy(), hr) <= LSTM_TOL / 20     # relative to the largest |h| of the stack
+    assert layer_err(h[:, :, rows].cpu().numpy(), hr) > LSTM_TOL                 # but not relative to every layer
+    h, c = run(products='f32')
+    assert not core.stacked_lstm_small_states(ws)
+    assert layer_err(h[:, :, rows].cpu().numpy(), hr) <= LSTM_TOL and layer_err(c[:, :, rows].cpu().numpy(), cr) <= LSTM_TOL
+    n = core.launch_counts.get('stacked_lstm_repeated_on_f32_products', 0)
+    h, c = run(exact_small_states=True)                                          # default mode, repeated on fp32 products
+    if core.get_lstm_products() == 'f16x3':
+        assert core.launch_counts['stacked_lstm_repeated_on_f32_products'] == n + 1
+    assert layer_err(h[:, :, rows].cpu().numpy(), hr) <= LSTM_TOL and layer_err(c[:, :, rows].cpu().numpy(), cr) <= LSTM_TOL
+    # a stack whose states keep their size is not repeated
+    xs2, WU2, b2 = lstm_inputs(32, 3, T, B, H, 1.0 / 8)
+    ws2 = torch.empty(core.stacked_lstm_workspace_bytes(3, T, B, H), dtype=torch.uint8, device='cuda')
+    core.stacked_lstm(dev(xs2), dev(WU2), dev(b2), workspace=ws2, check=True, exact_small_states=True)
+    assert not core.stacked_lstm_small_states(ws2)
+    assert core.launch_counts.get('stacked_lstm_repeated_on_f32_products', 0) == n + (1 if core.get_lstm_products() == 'f16x3' else 0)
+
+
+def test_hand_over_between_compute_units_gives_the_same_bits_every_launch(core):
+    """The persistent kernel hands rows of h from one compute unit to another through write-through stores, a
+    wait for their acknowledgement and a flag byte (the schedule it stands in for: region3.h:50-103).  A hand-over
+    that could be observed out of order, or a wave that multiplied with rows of a tile another wave had not copied
+    yet, would show as a result that differs from launch to launch (the second happened: the serial schedule's early
+    x half was a per-wave decision, and one launch in three of the 16-layer case below differed).  About 300 launches
+    over seven shapes -- config 4's depth, the dilated stack, a ragged batch, a stack that runs as two launches,
+    shallow stacks on the serial schedule -- every one bit-equal to the first of its shape (which is checked against
+    the oracle on a subset of rows), the status word clear every time; the test stops at the first difference."""
+    H = 256
+    lens = [24 - (b * 18) // 96 for b in range(96)]                       # 24 .. 6, sorted
+    cases = [
+        (32, 64, 256, None, None, 60),                                    # config 4
+        (6, 128, 256, [1, 2, 4, 8, 16, 32], None, 60),                    # config 5
+        (8, 24, 96, None, lens, 40),                                      # ragged rows
+        (34, 8, 64, None, None, 40),                                      # 34 layers: two persistent launches
+        # few layers on a chip with compute units to spare: every layer gets one row block per workgroup and runs the
+        # serial schedule, in which a wave that finds the layer below ready asks for its rows of the next tile early
+        (16, 24, 96, None, None, 40),
+        (8, 24, 32, None, None, 40),
+        (3, 16, 40, [1, 2, 4], None, 40),
+    ]
+    for ci, (L, T, B, dil, lengths, launches) in enumerate(cases):
+        print(f'soak case {ci}: L{L} T{T} B{B} dil {dil} ragged {lengths is not None}', flush=True)
+        xs, WU, bs = lstm_inputs(90 + ci, L, T, B, H, 1.0 / 16)
+        active = None if lengths is None else [sum(1 for v in lengths if v > t) for t in range(T)]
+        x_d, w_d, b_d = dev(xs), dev(WU), dev(bs)
+        ws = torch.empty(core.stacked_lstm_workspace_bytes(L, T, B, H), dtype=torch.uint8, device='cuda')
+        out = (torch.empty((L, T, B, H), device='cuda'), torch.empty((L, T, B, H), device='cuda'))
+        first = None
+        for i in range(launches):
+            out[0].fill_(float('nan')); out[1].fill_(float('nan'))
+            core.stacked_lstm(x_d, w_d, b_d, dilations=dil, out=out, workspace=ws, active_rows=active)
+            assert core.persistent_status(ws) == 0, f'case {ci}, launch {i}: a wait gave up'
+            if first is None:
+                first = (out[0].clone(), out[1].clone())
+                rows = [0, B // 2, B - 1]
+                hr, cr = ko.stacked_lstm(xs[:, rows], WU, bs, dilations=dil)
+                got_h, got_c = first[0][:, :, rows].cpu().numpy(), first[1][:, :, rows].cpu().numpy()
+                if lengths is not None:                                   # only the live places of a ragged batch are defined
+                    for k, r in enumerate(rows):
+                        got_h[:, lengths[r]:, k] = hr[:, lengths[r]:, k]
+                        got_c[:, lengths[r]:, k] = cr[:, lengths[r]:, k]
+                assert ko.max_rel_err(got_h, hr) <= LSTM_TOL and ko.max_rel_err(got_c, cr) <= LSTM_TOL
+                continue
+            if lengths is None:
+                same = torch.equal(out[0], first[0]) and torch.equal(out[1], first[1])
+            else:                                                         # dead places keep the NaN fill
+                same = bool(((out[0] == first[0]) | (out[0].isnan() & first[0].isnan())).all()) and \
+                    bool(((out[1] == first[1]) | (out[1].isnan() & first[1].isnan())).all())
+            assert same, f'case {ci}, launch {i} differs from launch 0'
+        del first, out, ws, x_d, w_d, b_d
+        torch.cuda.empty_cache()
+
+
 def test_a_drained_persistent_launch_raises(core):
     """A bounded wait that gives up must not pass for success.  One poll per wait (set from the host) makes the
     consumers of layer 1 give up at once: the kernel sets the status word, every workgroup leaves its loop and the
