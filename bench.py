@@ -322,6 +322,42 @@ def bench_attention(torch, core, steps, warmup, cpu):
     return res
 
 
+def bench_attention_f32(torch, core, steps, warmup, cpu):
+    """BASELINE configs[2]'s shape with fp32 Q, K, V, O (the element type of the reference's own attention program):
+    every product as three fp16 MFMAs of split operands.  The timed step is the whole entry point: the largest
+    |K|, |V| per head, the split of Q, K and V into planes, the attention kernel."""
+    B, Hd, S, D = 8, 16, 2048, 128
+    flop = 4.0 * B * Hd * S * S * D
+    gen = torch.Generator(device='cpu').manual_seed(1234)
+    Q, K, V = (torch.randn((B, Hd, S, D), generator=gen).cuda() for _ in range(3))
+    O = torch.empty_like(Q)
+    ws = torch.empty(int(core.lib.ftk_flash_attn_f32_workspace_bytes(B, Hd, S, S, D)), dtype=torch.uint8, device='cuda')
+    scale = D ** -0.5
+    ms, _ = _events_ms(torch, lambda: core.flash_attention_f32(Q, K, V, scale, out=O, workspace=ws), steps, warmup)
+    ms_t, _ = _events_ms(torch, lambda: torch.nn.functional.scaled_dot_product_attention(Q, K, V, scale=scale), max(2, steps // 4), 1)
+    ref = torch.nn.functional.scaled_dot_product_attention(Q[:1].double(), K[:1].double(), V[:1].double(), scale=scale)
+    res = {
+        'metric': 'TFLOP/s (attention, fp32 data)', 'value': flop / ms / 1e9, 'unit': 'TFLOP/s', 'ms_per_step': ms,
+        'dtype': 'f32 (products as three f16 MFMAs of split operands, f32 accumulate)',
+        'config': {'workload': 'flash attention, non-causal, fp32 Q/K/V/O at the shape of BASELINE.json configs[2]', 'batch': B,
+                   'heads': Hd, 'seq': S, 'head_dim': D},
+        'roofline': {'bound': 'mfma', 'achieved': 3 * flop / ms / 1e9, 'peak': PEAK_F16_TFLOPS, 'unit': 'TFLOP/s',
+                     'frac': 3 * flop / ms / 1e9 / PEAK_F16_TFLOPS, 'traffic': None, 'kernel': 'flash_attn_f32_kernel<128>',
+                     'what': 'MFMA flops issued (three f16 products per fp32 product) against the f16 MFMA peak; the step also '
+                             'holds the three launches that split the operands',
+                     'algorithmic': {'tflops': flop / ms / 1e9, 'ratio_to_f32_matrix_peak': flop / ms / 1e9 / PEAK_F32_MATRIX_TFLOPS}},
+        'torch_sdpa_f32': {'ms_per_step': ms_t, 'speedup': ms_t / ms},
+        'max_rel_diff_vs_float64_first_batch': float((O[:1].double() - ref).abs().max() / ref.abs().max()),
+    }
+    if cpu:
+        qh, kh, vh = (x[0].cpu() for x in (Q, K, V))
+        _, med, _, threads = _host_timed(torch, lambda: torch.nn.functional.scaled_dot_product_attention(qh, kh, vh, scale=scale), 1, 3)
+        res['cpu_baseline'] = {'value': flop / B / med / 1e12, 'unit': 'TFLOP/s', 'cores': threads, 'kind': 'torch_cpu_eager',
+                               'sample': f'the {Hd} heads of one sample through torch scaled_dot_product_attention, fp32, {threads} threads, '
+                                         f'median of 3: {med * 1e3:.0f} ms'}
+    return res
+
+
 def bench_embedding(torch, core, steps, warmup, cpu):
     """Embedding rows for a batch of word ids (the step that feeds the LSTM): V 5000 as in
     examples/stacked_rnn/rnn_utils.py, E 256 to match the LSTM configurations, 1 Mi ids."""
@@ -966,7 +1002,7 @@ def main():
     ap.add_argument('--gpus', type=int, default=1)
     ap.add_argument('--steps', type=int, default=50)
     ap.add_argument('--warmup', type=int, default=10)
-    ap.add_argument('--workload', default='b2b', choices=['b2b', 'config1', 'attention', 'stacked_lstm', 'dilated_lstm', 'lstm_f16_h256', 'lstm_f16_h512', 'lstm_f16_h1024', 'lstm_f32_h512', 'lstm_f32_h1024', 'gemm', 'online_softmax', 'embedding', 'grid_rnn', 'windowed_attention', 'b2b_ref_shapes', 'copy', 'mfma_rate'])
+    ap.add_argument('--workload', default='b2b', choices=['b2b', 'config1', 'attention', 'stacked_lstm', 'dilated_lstm', 'lstm_f16_h256', 'lstm_f16_h512', 'lstm_f16_h1024', 'lstm_f32_h512', 'lstm_f32_h1024', 'attention_f32', 'gemm', 'online_softmax', 'embedding', 'grid_rnn', 'windowed_attention', 'b2b_ref_shapes', 'copy', 'mfma_rate'])
     ap.add_argument('--no-extras', action='store_true', help='measure only the chosen workload')
     ap.add_argument('--all', action='store_true', help='also the workloads either side of the path (fp16 / larger stacks, GEMM, softmax, embedding, grid RNN, windowed attention)')
     ap.add_argument('--no-cpu', action='store_true', help='skip the CPU baseline leg')
@@ -1014,6 +1050,7 @@ def main():
         'lstm_f32_h512': lambda s, w, c: bench_lstm_f32_streamed(torch, core, max(3, s // 5), max(1, w // 5), c, 512),
         'lstm_f32_h1024': lambda s, w, c: bench_lstm_f32_streamed(torch, core, max(3, s // 10), 1, c, 1024),
         'b2b_ref_shapes': lambda s, w, c: bench_b2b_reference_shapes(torch, core, s, w, c),
+        'attention_f32': lambda s, w, c: bench_attention_f32(torch, core, max(5, s // 2), max(2, w // 2), c),
         'gemm': lambda s, w, c: bench_gemm(torch, core, max(5, s // 5), max(2, w // 5), c),
         'online_softmax': lambda s, w, c: bench_softmax(torch, core, s, w, c),
         'embedding': lambda s, w, c: bench_embedding(torch, core, s, w, c),

@@ -23,7 +23,7 @@ EXPORTS = (
     'ftk_stacked_lstm_wavefront_f32', 'ftk_stacked_lstm_ragged_f32', 'ftk_lstm_set_products', 'ftk_lstm_get_products',
     'ftk_stacked_lstm_opts_f32', 'ftk_stacked_lstm_status', 'ftk_stacked_lstm_small_states', 'ftk_stacked_lstm_noalloc_f32',
     'ftk_stacked_lstm_f16_workspace_bytes', 'ftk_stacked_lstm_f16',
-    'ftk_b2b_gemm_f16', 'ftk_b2b_gemm_f16_supported', 'ftk_b2b_gemm_rowmajor_f16', 'ftk_gemm_f16', 'ftk_batched_gemm_f16', 'ftk_flash_attn_f16', 'ftk_online_softmax_f32', 'ftk_embedding_gather_f32',
+    'ftk_b2b_gemm_f16', 'ftk_b2b_gemm_f16_supported', 'ftk_b2b_gemm_rowmajor_f16', 'ftk_gemm_f16', 'ftk_batched_gemm_f16', 'ftk_flash_attn_f16', 'ftk_flash_attn_f32_workspace_bytes', 'ftk_flash_attn_f32', 'ftk_online_softmax_f32', 'ftk_embedding_gather_f32',
     'ftk_grid_rnn_workspace_bytes', 'ftk_grid_rnn_f32', 'ftk_windowed_attn_f32',
 )
 
@@ -64,8 +64,11 @@ def _load() -> ctypes.CDLL:
     lib.ftk_stacked_lstm_f16_workspace_bytes.argtypes = [ctypes.c_int] * 4
     lib.ftk_grid_rnn_workspace_bytes.restype = ctypes.c_size_t
     lib.ftk_grid_rnn_workspace_bytes.argtypes = [ctypes.c_int] * 2
+    lib.ftk_flash_attn_f32_workspace_bytes.restype = ctypes.c_size_t
+    lib.ftk_flash_attn_f32_workspace_bytes.argtypes = [ctypes.c_int] * 5
     for name in EXPORTS:
-        if name not in ('ftk_last_error', 'ftk_stacked_lstm_workspace_bytes', 'ftk_stacked_lstm_f16_workspace_bytes', 'ftk_grid_rnn_workspace_bytes'):
+        if name not in ('ftk_last_error', 'ftk_stacked_lstm_workspace_bytes', 'ftk_stacked_lstm_f16_workspace_bytes', 'ftk_grid_rnn_workspace_bytes',
+                        'ftk_flash_attn_f32_workspace_bytes'):
             getattr(lib, name).restype = ctypes.c_int
     return lib
 
@@ -519,6 +522,31 @@ def flash_attention(Q, K, V, scale: Optional[float] = None, out: Optional[torch.
     ci = ctypes.c_int
     _check(lib.ftk_flash_attn_f16(_ptr(Q), _ptr(K), _ptr(V), _ptr(O), ci(B), ci(Hd), ci(Sq), ci(Skv), ci(D),
                                   ctypes.c_float(scale), _stream()))
+    return O
+
+
+def flash_attention_f32(Q, K, V, scale: Optional[float] = None, out: Optional[torch.Tensor] = None,
+                        workspace: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Non-causal attention with fp32 Q [B,Hd,Sq,D], K, V [B,Hd,Skv,D] -> O [B,Hd,Sq,D] fp32; D of 32, 64, 96 or 128.
+    Every product as three fp16 MFMAs of split operands, fp32 accumulation and softmax state."""
+    f32 = torch.float32
+    _req(Q, f32, 'Q'); _req(K, f32, 'K'); _req(V, f32, 'V')
+    if Q.dim() != 4 or K.dim() != 4 or K.shape != V.shape or Q.shape[:2] != K.shape[:2] or Q.shape[3] != K.shape[3]:
+        raise ValueError(f'Q [B,Hd,Sq,D] and K, V [B,Hd,Skv,D] expected, got {tuple(Q.shape)}, {tuple(K.shape)}, {tuple(V.shape)}')
+    B, Hd, Sq, D = Q.shape
+    Skv = K.shape[2]
+    if scale is None:
+        scale = D ** -0.5
+    O = out if out is not None else torch.empty_like(Q)
+    _req_out(O, f32, (B, Hd, Sq, D), 'O')
+    need = int(lib.ftk_flash_attn_f32_workspace_bytes(B, Hd, Sq, Skv, D))
+    if workspace is None:
+        workspace = torch.empty(need, dtype=torch.uint8, device=Q.device)
+    _req_workspace(workspace)
+    _count('flash_attention_f32')
+    ci = ctypes.c_int
+    _check(lib.ftk_flash_attn_f32(_ptr(Q), _ptr(K), _ptr(V), _ptr(O), ci(B), ci(Hd), ci(Sq), ci(Skv), ci(D), ctypes.c_float(scale),
+                                  _ptr(workspace), ctypes.c_size_t(workspace.numel() * workspace.element_size()), _stream()))
     return O
 
 

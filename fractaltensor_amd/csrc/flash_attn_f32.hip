@@ -1,0 +1,396 @@
+// Non-causal flash attention with fp32 Q, K, V and O on the fp16 matrix pipe of gfx950: every product of two
+// fp32 numbers is formed as three fp16 products of split operands, accumulated in fp32.
+//
+// The reference's attention program computes in fp32 (examples/flash_attention/flash_attention.py:14-91 with
+// kaleido.float32 blocks, flash_attention_utils.py:20-24).  fp32 MFMAs move two k per 16 passes where fp16
+// MFMAs move sixteen per 8, so, as in the stacked LSTM, an fp32 product is cheaper as three fp16 ones:
+//   v * 2^e = top + rest / 2^11,  top = fp16(v * 2^e),  rest = fp16((v * 2^e - top) * 2^11),
+// top * top in one accumulator, top * rest and rest * top in a second one that is folded in with 2^-11;
+// rest * rest, 2^-22 of a product, is dropped.  What shares a power-of-two scale 2^e (its largest magnitude
+// lands in [2^14, 2^15)): a row of Q, all of K of one (batch, head), all of V of one (batch, head), and the
+// fixed 2^14 for the softmax weights p in [0, 1].  An element keeps 22 significant bits of its own as long as it
+// is within 2^-28 of its group's largest; smaller ones lose bits, of products that are that much smaller too.
+//
+// Three launches: the largest |K| and |V| per (batch, head); the split of Q (times scale * log2 e), K and V into
+// planes [row][top D | rest D] in the workspace; the attention kernel.  A plane row is an fp16 row of 2 D
+// elements, so tiles, copies and fragment reads are those of the fp16 kernel at twice the head dimension
+// (fa_common.h), and the contractions are its transposed ones: S^T = K Q^T, O^T += V^T P^T, a lane owns one query
+// row, the running maximum and sum are lane-local.  The maximum is tracked per 32-key half tile, exactly (fp32
+// results leave no room for the fp16 kernel's lazily moved reference).
+#include <algorithm>
+#include <type_traits>
+
+#include "fa_common.h"
+
+namespace ftk {
+
+constexpr int kF32Top = 14;             // a scale group's largest magnitude lands in [2^14, 2^15)
+constexpr float kF32Rest = 2048.0f;     // 2^11
+constexpr float kF32P = 16384.0f;       // 2^14: the scale of the softmax weights
+
+// the power of two that brings a largest magnitude with these float bits into [2^14, 2^15), and its inverse
+__device__ __forceinline__ void split_scale(unsigned max_bits, float* scale, float* inv) {
+  const int eb = min(max((int)((max_bits >> 23) & 0xff), 15), 254 - kF32Top);
+  *scale = __uint_as_float((unsigned)(127 + kF32Top + 127 - eb) << 23);
+  *inv = __uint_as_float((unsigned)(eb - kF32Top) << 23);
+}
+
+__global__ void attn_f32_clear_kernel(unsigned* p, int n) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) p[i] = 0;
+}
+
+// largest |x| of every (batch, head) of K and V, as float bits (which order like the magnitudes): grid
+// (chunks, BH, 2), per_bh a multiple of 4
+__global__ __launch_bounds__(256) void attn_f32_absmax_kernel(const float* K, const float* V, unsigned* bits, size_t per_bh, int BH) {
+  const float* x = (blockIdx.z ? V : K) + (size_t)blockIdx.y * per_bh;
+  unsigned m = 0;
+  for (size_t i = ((size_t)blockIdx.x * 256 + threadIdx.x) * 4; i < per_bh; i += (size_t)gridDim.x * 1024) {
+    const float4 v = *reinterpret_cast<const float4*>(x + i);
+    m = max(max(m, __float_as_uint(fabsf(v.x))), max(__float_as_uint(fabsf(v.y)), max(__float_as_uint(fabsf(v.z)), __float_as_uint(fabsf(v.w)))));
+  }
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) m = max(m, (unsigned)__shfl_xor((int)m, o));
+  if ((threadIdx.x & 63) == 0 && m) atomicMax(bits + blockIdx.z * BH + blockIdx.y, m);
+}
+
+// One wave per row of D floats: planes [top D | rest D] of the row times `mul`, under the row's own scale
+// (row_inv != nullptr: Q; the inverse scale goes to row_inv[row]) or under the (batch, head)'s (K, V).
+template <int D>
+__global__ __launch_bounds__(256) void attn_f32_split_kernel(const float* X, _Float16* planes, float* row_inv, const unsigned* group_bits,
+                                                            int rows_per_bh, long long rows, float mul) {
+  constexpr int PER = D / 32;   // floats per lane: 1, 2, 3 or 4; lanes 32..63 idle for D = 32 only when PER * 64 > D
+  const int lane = threadIdx.x & 63;
+  const long long row = (long long)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (row >= rows) return;
+  constexpr int LANES = D / PER > 64 ? 64 : D / PER;   // 32 lanes x PER floats cover a row
+  float v[PER];
+  unsigned m = 0;
+  if (lane < LANES) {
+#pragma unroll
+    for (int e = 0; e < PER; ++e) {
+      v[e] = X[row * D + lane * PER + e] * mul;
+      m = max(m, __float_as_uint(fabsf(v[e])));
+    }
+  }
+  float scale, inv;
+  if (row_inv) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) m = max(m, (unsigned)__shfl_xor((int)m, o));
+    split_scale(m, &scale, &inv);
+    if (lane == 0) row_inv[row] = inv;
+  } else {
+    split_scale(group_bits[row / rows_per_bh], &scale, &inv);
+  }
+  if (lane < LANES) {
+    _Float16* dst = planes + row * (2 * D) + lane * PER;
+#pragma unroll
+    for (int e = 0; e < PER; ++e) {
+      const float s = v[e] * scale;
+      const _Float16 top = (_Float16)s;
+      dst[e] = top;
+      dst[D + e] = (_Float16)((s - (float)top) * kF32Rest);
+    }
+  }
+}
+
+// 4 waves x 32 query rows per workgroup, one workgroup per compute unit (the accumulators of O, both planes of Q
+// and the scores take more than 256 registers at D = 128).  K and V tiles of 64 keys, both double buffered; the
+// tile after the current one is requested when the current one's products begin and waited for at the barrier
+// that ends them.
+template <int D>
+__global__ __launch_bounds__(256, 1) void flash_attn_f32_kernel(const _Float16* __restrict__ Qp, const _Float16* __restrict__ Kp,
+                                                                const _Float16* __restrict__ Vp, const float* __restrict__ q_inv,
+                                                                const unsigned* __restrict__ kv_bits, float* __restrict__ O,
+                                                                int Sq, int Skv, int nqb, int BH) {
+  using L = FaLayout<2 * D>;          // a plane row is an fp16 row of 2 D elements
+  constexpr int DS = D / 16;          // k steps of S^T
+  constexpr int DT = D / 32;          // d tiles of O^T
+  constexpr int RB = 4 * D;           // bytes per plane row in global memory
+  constexpr int KRS = L::KRS, VRS = L::VRS, KTB = L::KTB, VTB = L::VTB;
+  constexpr int WAVES = 4;
+  constexpr int KCP = (KTB / 1024 + WAVES - 1) / WAVES, VCP = (VTB / 1024 + WAVES - 1) / WAVES;
+  extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];
+  unsigned char* const Kb = smem;            // [2][KTB]
+  unsigned char* const Vb = smem + 2 * KTB;  // [2][VTB]
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int j = lane & 31;
+  const int hh = lane >> 5;
+  int id = blockIdx.x;
+  const int total = gridDim.x;
+  if ((total & 7) == 0) id = (blockIdx.x & 7) * (total >> 3) + (blockIdx.x >> 3);   // a head's query blocks share an XCD
+  const int bh = id / nqb;
+  const int qb = id - bh * nqb;
+  const int q_base = qb * (WAVES * 32) + wave * 32;
+
+  const _Float16* Qg = Qp + (size_t)bh * Sq * (2 * D);
+  const _Float16* Kg = Kp + (size_t)bh * Skv * (2 * D);
+  const _Float16* Vg = Vp + (size_t)bh * Skv * (2 * D);
+  float* Og = O + (size_t)bh * Sq * D;
+
+  // the lane's query row: both planes of its fragments, and what a score is multiplied by to undo the scales
+  const int qrow = min(q_base + j, Sq - 1);
+  v8h qt[DS], qr[DS];
+#pragma unroll
+  for (int s = 0; s < DS; ++s) {
+    qt[s] = *reinterpret_cast<const v8h*>(Qg + (size_t)qrow * (2 * D) + 16 * s + 8 * hh);
+    qr[s] = *reinterpret_cast<const v8h*>(Qg + (size_t)qrow * (2 * D) + D + 16 * s + 8 * hh);
+  }
+  float k_scale, k_inv, v_scale, v_inv;
+  split_scale(kv_bits[bh], &k_scale, &k_inv);
+  split_scale(kv_bits[BH + bh], &v_scale, &v_inv);
+  const float s_mul = q_inv[(size_t)bh * Sq + qrow] * k_inv;
+
+  v16f om[DT], oc[DT];
+#pragma unroll
+  for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) { om[dt][r] = 0.0f; oc[dt][r] = 0.0f; }
+  float m_run = -INFINITY, l_run = 0.0f;
+
+  // copies: as in the fp16 kernel, copy c of a tile fills LDS bytes [1024 c, 1024 c + 1024) of the padded tile
+  unsigned k_src[KCP], v_src[VCP];
+#pragma unroll
+  for (int i = 0; i < KCP; ++i) {
+    const int x = 1024 * (wave + WAVES * i) + 16 * lane;
+    const int row = min(x / KRS, FA_KT - 1), col = x % KRS;
+    k_src[i] = row * RB + (col < RB ? col : 0);
+  }
+#pragma unroll
+  for (int i = 0; i < VCP; ++i) {
+    const int x = 1024 * (wave + WAVES * i) + 16 * lane;
+    const int row = min(x / VRS, FA_KT - 1), col = x % VRS;
+    v_src[i] = row * RB + (col < RB ? col : 0);
+  }
+  auto copy_tile = [&](int kt, int buf) __attribute__((always_inline)) {
+    const int key0 = kt * FA_KT;
+    const bool tail = key0 + FA_KT > Skv;   // rows past the end re-read the last key; their scores are masked
+    static_for<KCP>([&](auto i_c) __attribute__((always_inline)) {
+      constexpr int i = decltype(i_c)::value;
+      if (wave + WAVES * i < KTB / 1024) {
+        unsigned off = k_src[i];
+        if (tail) {
+          const unsigned last = (unsigned)(Skv - 1 - key0), row = off / RB;
+          if (row > last) off -= (row - last) * RB;
+        }
+        lds_dma16(Kg + (size_t)key0 * (2 * D), off, Kb + buf * KTB + 1024 * (wave + WAVES * i));
+      }
+    });
+    static_for<VCP>([&](auto i_c) __attribute__((always_inline)) {
+      constexpr int i = decltype(i_c)::value;
+      if (wave + WAVES * i < VTB / 1024) {
+        unsigned off = v_src[i];
+        if (tail) {
+          const unsigned last = (unsigned)(Skv - 1 - key0), row = off / RB;
+          if (row > last) off -= (row - last) * RB;
+        }
+        lds_dma16(Vg + (size_t)key0 * (2 * D), off, Vb + buf * VTB + 1024 * (wave + WAVES * i));
+      }
+    });
+  };
+
+  const int k_lane = j * KRS + 16 * hh;
+  const int v_lane = (4 * hh + ((lane & 15) >> 2)) * VRS + 32 * ((lane >> 4) & 1) + 8 * (lane & 3);
+  using lds_v4s = __attribute__((address_space(3))) v4s;
+  typedef short v8s __attribute__((ext_vector_type(8)));
+  // A-operand of the P V product: step s (16 keys) and d tile dt of one half tile; plane 0 = values, 1 = remainders
+  auto read_v = [&](const unsigned char* vbase, int s, int dt, int plane) __attribute__((always_inline)) {
+    const unsigned char* p0 = vbase + 16 * s * VRS + 64 * dt + plane * (2 * D);
+    const v4s lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4s*)(p0));
+    const v4s hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4s*)(p0 + 8 * VRS));
+    const v8s both = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+    return __builtin_bit_cast(v8h, both);
+  };
+
+  const int ntiles = (Skv + FA_KT - 1) / FA_KT;
+  copy_tile(0, 0);
+  __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
+  __syncthreads();
+
+  for (int kt = 0; kt < ntiles; ++kt) {
+    const int buf = kt & 1;
+    if (kt + 1 < ntiles) copy_tile(kt + 1, buf ^ 1);   // its buffers were last read before the barrier that ended tile kt - 1
+#pragma unroll
+    for (int half = 0; half < 2; ++half) {
+      const int key0 = kt * FA_KT + 32 * half;
+      if (key0 >= Skv) break;
+      const unsigned char* kbase = Kb + buf * KTB + k_lane + 32 * half * KRS;
+      const unsigned char* vbase = Vb + buf * VTB + v_lane + 32 * half * VRS;
+      // scores of 32 keys: value x value, and the two mixed products at 2^-11
+      v16f am, ar;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) { am[r] = 0.0f; ar[r] = 0.0f; }
+#pragma unroll
+      for (int s = 0; s < DS; ++s) {
+        const v8h kt_ = *reinterpret_cast<const v8h*>(kbase + 32 * s);
+        const v8h kr_ = *reinterpret_cast<const v8h*>(kbase + 2 * D + 32 * s);
+        am = __builtin_amdgcn_mfma_f32_32x32x16_f16(kt_, qt[s], am, 0, 0, 0);
+        ar = __builtin_amdgcn_mfma_f32_32x32x16_f16(kt_, qr[s], ar, 0, 0, 0);
+        ar = __builtin_amdgcn_mfma_f32_32x32x16_f16(kr_, qt[s], ar, 0, 0, 0);
+      }
+      float sc[16];
+      float mx = -INFINITY;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        sc[r] = (am[r] + (1.0f / kF32Rest) * ar[r]) * s_mul;
+        if (key0 + 8 * (r >> 2) + 4 * hh + (r & 3) >= Skv) sc[r] = -INFINITY;
+        mx = fmaxf(mx, sc[r]);
+      }
+      mx = max_with_other_half(mx);
+      const float m_new = fmaxf(m_run, mx);   // finite: the half holds at least one key
+      const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);   // 0 the first time (m_run = -inf)
+      m_run = m_new;
+      float lsum = 0.0f;
+      v8h pt[2], pr[2];
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const float p = __builtin_amdgcn_exp2f(sc[r] - m_new);
+        lsum += p;
+        const float ps = p * kF32P;
+        const _Float16 top = (_Float16)ps;
+        pt[r >> 3][r & 7] = top;
+        pr[r >> 3][r & 7] = (_Float16)((ps - (float)top) * kF32Rest);
+      }
+      l_run = l_run * alpha + lsum;
+      if (__builtin_amdgcn_ballot_w64(alpha != 1.0f) != 0) {
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) { om[dt][r] *= alpha; oc[dt][r] *= alpha; }
+      }
+#pragma unroll
+      for (int s = 0; s < 2; ++s)
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt) {
+          const v8h vt_ = read_v(vbase, s, dt, 0);
+          const v8h vr_ = read_v(vbase, s, dt, 1);
+          om[dt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(vt_, pt[s], om[dt], 0, 0, 0);
+          oc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(vt_, pr[s], oc[dt], 0, 0, 0);
+          oc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(vr_, pt[s], oc[dt], 0, 0, 0);
+        }
+    }
+    __builtin_amdgcn_s_waitcnt(0x0F70);  // this wave's copies of tile kt + 1 have landed
+    __syncthreads();
+  }
+
+  // ---- normalise and store: the wave turns its 32 x D tile round through the LDS nobody reads any more (the
+  // barrier above ended the last tile), so that whole rows leave as consecutive bytes
+  constexpr int ORS = 4 * D + 16;
+  constexpr int LPR = D / 4;   // 16-byte chunks per row
+  unsigned char* const ot = smem + wave * (32 * ORS);
+  const float l = l_run + __shfl_xor(l_run, 32);
+  const float fin = v_inv * (1.0f / kF32P) / l;
+#pragma unroll
+  for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+      float4 o;
+      o.x = (om[dt][4 * g + 0] + (1.0f / kF32Rest) * oc[dt][4 * g + 0]) * fin;
+      o.y = (om[dt][4 * g + 1] + (1.0f / kF32Rest) * oc[dt][4 * g + 1]) * fin;
+      o.z = (om[dt][4 * g + 2] + (1.0f / kF32Rest) * oc[dt][4 * g + 2]) * fin;
+      o.w = (om[dt][4 * g + 3] + (1.0f / kF32Rest) * oc[dt][4 * g + 3]) * fin;
+      *reinterpret_cast<float4*>(ot + j * ORS + 4 * (32 * dt + 8 * g + 4 * hh)) = o;
+    }
+#pragma unroll
+  for (int idx = lane; idx < 32 * LPR; idx += 64) {
+    const int r = idx / LPR, c = idx - r * LPR;
+    const v4u piece = *reinterpret_cast<const v4u*>(ot + r * ORS + 16 * c);
+    const int row = q_base + r;
+    if (row < Sq) __builtin_nontemporal_store(piece, reinterpret_cast<v4u*>(Og + (size_t)row * D + 4 * c));
+  }
+}
+
+static size_t round256f(size_t v) { return (v + 255) / 256 * 256; }
+
+struct F32Layout {
+  size_t bits, qinv, qp, kp, vp, total;
+};
+static F32Layout f32_layout(long long bh, int Sq, int Skv, int D) {
+  F32Layout w;
+  w.bits = 0;
+  w.qinv = round256f((size_t)2 * bh * sizeof(unsigned));
+  w.qp = w.qinv + round256f((size_t)bh * Sq * sizeof(float));
+  w.kp = w.qp + round256f((size_t)bh * Sq * 2 * D * sizeof(_Float16));
+  w.vp = w.kp + round256f((size_t)bh * Skv * 2 * D * sizeof(_Float16));
+  w.total = w.vp + round256f((size_t)bh * Skv * 2 * D * sizeof(_Float16));
+  return w;
+}
+
+template <int D>
+static int launch_fa_f32(const float* Q, const float* K, const float* V, float* O, int BH, int Sq, int Skv, float scale, char* ws,
+                         const F32Layout& w, int lds_max, hipStream_t s) {
+  using L = FaLayout<2 * D>;
+  const size_t lds = std::max((size_t)2 * (L::KTB + L::VTB), (size_t)4 * 32 * (4 * D + 16));
+  if ((int)lds > lds_max) return fail(FTK_ERR_DEVICE, "ftk_flash_attn_f32: D=%d needs %zu bytes of LDS, the device offers %d", D, lds, lds_max);
+  unsigned* bits = reinterpret_cast<unsigned*>(ws + w.bits);
+  float* qinv = reinterpret_cast<float*>(ws + w.qinv);
+  _Float16* qp = reinterpret_cast<_Float16*>(ws + w.qp);
+  _Float16* kp = reinterpret_cast<_Float16*>(ws + w.kp);
+  _Float16* vp = reinterpret_cast<_Float16*>(ws + w.vp);
+  hipLaunchKernelGGL(attn_f32_clear_kernel, dim3((2 * BH + 255) / 256), dim3(256), 0, s, bits, 2 * BH);
+  int rc = check_launch("attn_f32_clear_kernel");
+  if (rc) return rc;
+  const size_t per_bh = (size_t)Skv * D;
+  const int chunks = (int)std::min<size_t>(64, (per_bh + 4095) / 4096);
+  hipLaunchKernelGGL(attn_f32_absmax_kernel, dim3(chunks, BH, 2), dim3(256), 0, s, K, V, bits, per_bh, BH);
+  rc = check_launch("attn_f32_absmax_kernel");
+  if (rc) return rc;
+  const long long qrows = (long long)BH * Sq, krows = (long long)BH * Skv;
+  hipLaunchKernelGGL(attn_f32_split_kernel<D>, dim3((unsigned)((qrows + 3) / 4)), dim3(256), 0, s, Q, qp, qinv, (const unsigned*)nullptr, Sq,
+                     qrows, scale * 1.4426950408889634f);
+  hipLaunchKernelGGL(attn_f32_split_kernel<D>, dim3((unsigned)((krows + 3) / 4)), dim3(256), 0, s, K, kp, (float*)nullptr, (const unsigned*)bits,
+                     Skv, krows, 1.0f);
+  hipLaunchKernelGGL(attn_f32_split_kernel<D>, dim3((unsigned)((krows + 3) / 4)), dim3(256), 0, s, V, vp, (float*)nullptr,
+                     (const unsigned*)(bits + BH), Skv, krows, 1.0f);
+  rc = check_launch("attn_f32_split_kernel");
+  if (rc) return rc;
+  const int nqb = (Sq + 127) / 128;
+  const long long blocks = (long long)nqb * BH;
+  if (blocks > 0x7fffffffLL) return fail(FTK_ERR_UNSUPPORTED_SHAPE, "ftk_flash_attn_f32: grid too large");
+  static DeviceOnce attr_once;
+  unsigned attr_bit;
+  if (attr_once.pending(&attr_bit)) {
+    FTK_HIP(hipFuncSetAttribute((const void*)flash_attn_f32_kernel<D>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+    attr_once.done(attr_bit);
+  }
+  hipLaunchKernelGGL(flash_attn_f32_kernel<D>, dim3((unsigned)blocks), dim3(256), lds, s, qp, kp, vp, qinv, bits, O, Sq, Skv, nqb, BH);
+  return check_launch("flash_attn_f32_kernel");
+}
+
+}  // namespace ftk
+
+extern "C" size_t ftk_flash_attn_f32_workspace_bytes(int B, int Hd, int Sq, int Skv, int D) {
+  if (B <= 0 || Hd <= 0 || Sq <= 0 || Skv <= 0 || D <= 0) return 0;
+  return ftk::f32_layout((long long)B * Hd, Sq, Skv, D).total;
+}
+
+extern "C" int ftk_flash_attn_f32(const float* Q, const float* K, const float* V, float* O, int B, int Hd, int Sq, int Skv, int D,
+                                  float scale, void* workspace, size_t workspace_bytes, ftk_stream_t stream) {
+  using namespace ftk;
+  const char* who = "ftk_flash_attn_f32";
+  if (!Q || !K || !V || !O) return fail(FTK_ERR_INVALID_ARGUMENT, "%s: Q, K, V, O must be non-NULL", who);
+  if (B <= 0 || Hd <= 0 || Sq <= 0 || Skv <= 0 || D <= 0) return fail(FTK_ERR_INVALID_ARGUMENT, "%s: B, Hd, Sq, Skv, D must be positive", who);
+  if (D != 32 && D != 64 && D != 96 && D != 128) return fail(FTK_ERR_UNSUPPORTED_SHAPE, "%s: D=%d must be 32, 64, 96 or 128", who, D);
+  if (!(scale > 0.0f) || !(scale < INFINITY)) return fail(FTK_ERR_INVALID_ARGUMENT, "%s: scale must be positive and finite", who);
+  const long long bh = (long long)B * Hd;
+  if (bh > (1LL << 16)) return fail(FTK_ERR_UNSUPPORTED_SHAPE, "%s: B*Hd=%lld too large", who, bh);
+  if ((long long)Skv * D >= (1LL << 31) || (long long)Sq * D >= (1LL << 31)) return fail(FTK_ERR_UNSUPPORTED_SHAPE, "%s: a head is too large", who);
+  const F32Layout w = f32_layout(bh, Sq, Skv, D);
+  if (!workspace || workspace_bytes < w.total)
+    return fail(FTK_ERR_WORKSPACE, "%s: workspace of %zu bytes needed, %zu given", who, w.total, workspace ? workspace_bytes : (size_t)0);
+  if (reinterpret_cast<uintptr_t>(workspace) % 256) return fail(FTK_ERR_INVALID_ARGUMENT, "%s: workspace must be 256-byte aligned", who);
+  const DeviceProps* dp = nullptr;
+  int rc = device_props(&dp);
+  if (rc) return rc;
+  hipStream_t s = (hipStream_t)stream;
+  char* ws = reinterpret_cast<char*>(workspace);
+  switch (D) {
+    case 32: return launch_fa_f32<32>(Q, K, V, O, (int)bh, Sq, Skv, scale, ws, w, dp->lds_optin, s);
+    case 64: return launch_fa_f32<64>(Q, K, V, O, (int)bh, Sq, Skv, scale, ws, w, dp->lds_optin, s);
+    case 96: return launch_fa_f32<96>(Q, K, V, O, (int)bh, Sq, Skv, scale, ws, w, dp->lds_optin, s);
+    default: return launch_fa_f32<128>(Q, K, V, O, (int)bh, Sq, Skv, scale, ws, w, dp->lds_optin, s);
+  }
+}

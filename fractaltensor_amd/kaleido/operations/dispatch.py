@@ -33,8 +33,8 @@ product forms it with torch, as before.  The arithmetic is that of the two fp16
 GEMMs (the intermediate rounded to fp16, fp32 accumulation).
 
   enabled                   False (or FTK_DISPATCH=0 in the environment) switches routing off
-  allow_half_attention      route fp32 attention programs to the fp16 kernel too (off: a
-                            routed program never computes in less than its own precision)
+  allow_half_attention      route fp32 attention programs to the fp16 kernel instead of the fp32
+                            one (off: a routed program never computes in less than its own precision)
   stats                     counts of routed calls, probes and declined probes
 """
 from __future__ import annotations
@@ -779,12 +779,13 @@ def _attention_operands(xs):
     return q, k, v
 
 
-def _probe_attention(func: Callable, rq: int, rk: int, D: int, gen) -> Optional[float]:
-    """The score scale of the program, if func is blockwise softmax(scale * q k^T) v; None otherwise."""
+def _probe_attention(func: Callable, rq: int, rk: int, D: int, gen, dtype=torch.float16) -> Optional[float]:
+    """The score scale of the program, if func is blockwise softmax(scale * q k^T) v; None otherwise.  The probe runs
+    in the program's own element type against the kernel of that type (1e-2 for fp16, 1e-4 for fp32)."""
     core = _core()
     nk = 2
     n = nk * rk
-    mk = lambda t: FractalTensor.from_dense(t.cuda(), 2)
+    mk = lambda t: FractalTensor.from_dense(t.to(device='cuda', dtype=dtype), 2)
 
     def run(q, k, v):      # one sample's item: [heads = 1][blocks] of [rows, D] each
         with _Probe():
@@ -817,6 +818,9 @@ def _probe_attention(func: Callable, rq: int, rk: int, D: int, gen) -> Optional[
     out = run(q, k, v)
     if out is None:
         return None
+    if dtype == torch.float32:
+        ref = core.flash_attention_f32(q.cuda().reshape(1, 1, rq, D), k.cuda().reshape(1, 1, n, D), v.cuda().reshape(1, 1, n, D), s)
+        return s if _rel_err(out, ref.reshape(rq, D)) <= 1e-4 else None
     ref = core.flash_attention(q.half().cuda().reshape(1, 1, rq, D), k.half().cuda().reshape(1, 1, n, D),
                                v.half().cuda().reshape(1, 1, n, D), s).reshape(rq, D)
     return s if _rel_err(out, ref) <= 1e-2 else None
@@ -834,15 +838,15 @@ def try_map(func: Callable, xs, kwargs):
     if ops is None:
         return NotImplemented
     q, k, v = ops
-    if q.dtype != torch.float16 and not (q.dtype == torch.float32 and allow_half_attention):
+    if q.dtype not in (torch.float16, torch.float32):
         return NotImplemented
     B, Hd, nq, rq, D = q.shape
     nk, rk = k.shape[2], k.shape[3]
-    key = ('map', _fingerprint(func), rq, rk, D)
+    key = ('map', _fingerprint(func), rq, rk, D, q.dtype)
     if key not in _verdicts:
         stats['probes'] += 1
         try:
-            scale = _probe_attention(func, rq, rk, D, torch.Generator().manual_seed(20240301))
+            scale = _probe_attention(func, rq, rk, D, torch.Generator().manual_seed(20240301), q.dtype)
         except Exception:
             scale = None
         if scale is None:
@@ -853,7 +857,10 @@ def try_map(func: Callable, xs, kwargs):
         return NotImplemented
     core = _core()
     to4 = lambda t: t.reshape(B, Hd, t.shape[2] * t.shape[3], D)
-    O = core.flash_attention(to4(q).half().contiguous(), to4(k).half().contiguous(), to4(v).half().contiguous(), verdict['scale'])
+    if q.dtype == torch.float32 and not allow_half_attention:       # a program computes in its own precision
+        O = core.flash_attention_f32(to4(q).contiguous(), to4(k).contiguous(), to4(v).contiguous(), verdict['scale'])
+    else:
+        O = core.flash_attention(to4(q).half().contiguous(), to4(k).half().contiguous(), to4(v).half().contiguous(), verdict['scale'])
     stats['flash_attention'] += 1
     return FractalTensor.from_dense(O.to(q.dtype).view(B, Hd, nq, rq, D), 3)
 

@@ -453,6 +453,26 @@ int ftk_flash_attn_f16(const void* Q, const void* K, const void* V, void* O,
                        ftk_stream_t stream);
 
 /*
+ * The same attention with fp32 Q, K, V and O, [B,Hd,S,D] row-major, D of 32,
+ * 64, 96 or 128: the element type of the reference's program
+ * (examples/flash_attention/flash_attention.py:14-91 on kaleido.float32
+ * blocks, flash_attention_utils.py:20-24; batch 2 x 8 heads x 1024 x 32 at
+ * :96-110).  Products run on the fp16 matrix pipe as three fp16 products of
+ * split operands with fp32 accumulation (a row of Q, all of K and all of V of
+ * a (batch, head) each share a power-of-two scale), the softmax state is fp32:
+ * results agree with a float64 evaluation to a few 1e-6 of the largest |O|.
+ * Non-finite inputs give NaN.  The workspace (ftk_flash_attn_f32_workspace_bytes,
+ * about the size of Q, K and V together, 256-byte aligned) holds the split
+ * operands; three small launches precede the attention kernel.  The reference
+ * has no device kernel for this program.
+ */
+size_t ftk_flash_attn_f32_workspace_bytes(int B, int Hd, int Sq, int Skv, int D);
+int ftk_flash_attn_f32(const float* Q, const float* K, const float* V, float* O,
+                       int B, int Hd, int Sq, int Skv, int D, float scale,
+                       void* workspace, size_t workspace_bytes,
+                       ftk_stream_t stream);
+
+/*
  * Windowed attention, fp32: token t of each of the G sequences attends to the
  * `window` (odd) positions t - half + k*dilation, k = 0..window-1,
  * half = (window-1)*dilation/2, and to the R further positions

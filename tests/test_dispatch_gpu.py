@@ -492,28 +492,39 @@ def test_reference_style_flash_attention_without_a_scale():
 
 def test_reference_example_sizes_of_flash_attention():
     """The example's own configuration (examples/flash_attention/flash_attention.py:96-110): batch 2, 8 heads, 1024
-    tokens in blocks of 64, head dimension 32, fp32 data, no scale.  fp32 programs go to the fp16 kernel only when
-    allowed to."""
+    tokens in blocks of 64, head dimension 32, fp32 data, no scale.  Routed by default, to the fp32 kernel: the
+    result is within 1e-4 of float64."""
+    core = _core()
     B, Hd, S, blk, D = 2, 8, 1024, 64, 32
     qsss, ksss, vsss = (programs.make_attention_input(B, Hd, S, blk, D, seed=60 + i, device='cuda') for i in range(3))
     scaled = FractalTensor.from_dense(qsss.as_dense() * 0.25, 3)
-    dispatch.allow_half_attention = True
+    before = core.launch_counts.get('flash_attention_f32', 0)
     out = flash_attention(scaled, ksss, vsss)
     assert dispatch.stats['flash_attention'] == 1 and out.data.dtype == torch.float32
-    to4 = lambda t: t.as_dense().reshape(B, Hd, S, D).float().cpu().numpy()
-    ref = ko.attention(to4(scaled), to4(ksss), to4(vsss), 1.0, dtype=np.float32)
-    assert ko.max_rel_err(to4(out), ref) <= 1e-2
+    assert core.launch_counts['flash_attention_f32'] == before + 2      # the probe's reference and the program
+    to4 = lambda t: t.as_dense().reshape(B, Hd, S, D).double().cpu().numpy()
+    ref = ko.attention(to4(scaled), to4(ksss), to4(vsss), 1.0)
+    assert ko.max_rel_err(to4(out), ref) <= 1e-4
+    flash_attention(scaled, ksss, vsss)                                  # warm: one launch, no probe
+    assert core.launch_counts['flash_attention_f32'] == before + 3 and dispatch.stats['probes'] == 1
 
 
-def test_fp32_attention_program_is_not_lowered_to_fp16_unless_allowed():
+def test_fp32_attention_program_goes_to_the_fp32_kernel_unless_half_is_allowed():
+    core = _core()
     B, Hd, S, blk, D = 1, 1, 128, 64, 64
     qsss, ksss, vsss = (programs.make_attention_input(B, Hd, S, blk, D, seed=40 + i, device='cuda') for i in range(3))
+    dispatch.enabled = False
     eager = programs.flash_attention(qsss, ksss, vsss, D ** -0.5)
-    assert dispatch.stats['flash_attention'] == 0 and dispatch.stats['probes'] == 0
-    dispatch.allow_half_attention = True
+    dispatch.enabled = True
     routed = programs.flash_attention(qsss, ksss, vsss, D ** -0.5)
     assert dispatch.stats['flash_attention'] == 1 and routed.data.dtype == torch.float32
-    assert ko.max_rel_err(routed.data.cpu().numpy(), eager.data.cpu().numpy()) <= 1e-2
+    assert core.launch_counts.get('flash_attention_f32', 0) >= 1
+    assert ko.max_rel_err(routed.data.cpu().numpy(), eager.data.cpu().numpy()) <= 1e-4
+    dispatch.allow_half_attention = True
+    half_before = core.launch_counts.get('flash_attention', 0)
+    lowered = programs.flash_attention(qsss, ksss, vsss, D ** -0.5)
+    assert core.launch_counts.get('flash_attention', 0) == half_before + 1 and lowered.data.dtype == torch.float32
+    assert ko.max_rel_err(lowered.data.cpu().numpy(), eager.data.cpu().numpy()) <= 1e-2
 
 
 # ---- (a @ b) @ c -----------------------------------------------------------------------------------------------------

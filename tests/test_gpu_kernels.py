@@ -1007,6 +1007,94 @@ def test_flash_attention_config3_full_size(core):
     assert torch.equal(O4[normal], (O * 4)[normal])
 
 
+F32_ATTN_TOL = 1e-4      # the fp32 path's bound; the split products are expected two orders inside it
+
+
+@pytest.mark.parametrize('B,Hd,Sq,Skv,D,scale', [
+    (2, 8, 1024, 1024, 32, 1.0),         # the reference example's own sizes and (absent) scale, flash_attention.py:96-110
+    (1, 2, 256, 256, 128, None),
+    (1, 3, 100, 77, 64, None),           # ragged queries and keys, one key tile and a part
+    (2, 1, 33, 200, 96, 0.2),
+    (1, 1, 1, 1, 32, None),              # a single query and key
+    (1, 2, 130, 64, 128, None),          # a second query block of two rows
+    (1, 1, 64, 1000, 64, 0.05),
+])
+def test_flash_attention_f32(core, B, Hd, Sq, Skv, D, scale):
+    rng = np.random.default_rng(17)
+    Q = rng.standard_normal((B, Hd, Sq, D)).astype(np.float32)
+    K = rng.standard_normal((B, Hd, Skv, D)).astype(np.float32)
+    V = rng.standard_normal((B, Hd, Skv, D)).astype(np.float32)
+    if scale == 1.0:
+        Q *= 0.25                                                        # unscaled scores: keep them in a softmax's working range
+    sc = D ** -0.5 if scale is None else scale
+    O = core.flash_attention_f32(dev(Q), dev(K), dev(V), sc).cpu().numpy()
+    ref = ko.attention(Q, K, V, sc)                                      # float64
+    err = ko.max_rel_err(O, ref)
+    assert err <= F32_ATTN_TOL / 10, err
+    # and no worse than fp32 arithmetic itself by more than a small factor
+    err32 = ko.max_rel_err(ko.attention(Q, K, V, sc, dtype=np.float32), ref)
+    assert err <= max(8 * err32, 2e-6), (err, err32)
+
+
+def test_flash_attention_f32_closed_forms_and_scales(core):
+    """Uniform keys give the mean of the values; a (batch, head) whose K and V are 2^20 times another's gets its own
+    scale; rows of Q of very different sizes get theirs; scores that climb by 30 per key tile move the maximum every
+    half tile; one huge element in K must not cost the small ones their accuracy relative to the result."""
+    rng = np.random.default_rng(18)
+    B, Hd, S, D = 1, 2, 256, 64
+    Q = rng.standard_normal((B, Hd, S, D)).astype(np.float32)
+    V = rng.standard_normal((B, Hd, S, D)).astype(np.float32)
+    K = np.tile(rng.standard_normal((B, Hd, 1, D)).astype(np.float32), (1, 1, S, 1))
+    O = core.flash_attention_f32(dev(Q), dev(K), dev(V), 0.125).cpu().numpy()
+    assert np.abs(O - V.astype(np.float64).mean(axis=2, keepdims=True)).max() <= 5e-6
+    K = rng.standard_normal((B, Hd, S, D)).astype(np.float32)
+    K[0, 1] *= 2.0 ** 10; V[0, 1] *= 2.0 ** 20; Q[0, 1] *= 2.0 ** -10
+    Q[0, 0, ::3] *= 1e-3
+    O = core.flash_attention_f32(dev(Q), dev(K), dev(V), 0.125).cpu().numpy()
+    ref = ko.attention(Q, K, V, 0.125)
+    for h in range(Hd):
+        assert ko.max_rel_err(O[0, h], ref[0, h]) <= F32_ATTN_TOL / 10
+    K = rng.standard_normal((B, Hd, S, D)).astype(np.float32)
+    K += (np.arange(S) // 64)[None, None, :, None].astype(np.float32) * 30.0 * np.sign(Q.mean(axis=2, keepdims=True))
+    O = core.flash_attention_f32(dev(Q), dev(K), dev(V), 0.125).cpu().numpy()
+    assert ko.max_rel_err(O, ko.attention(Q, K, V, 0.125)) <= F32_ATTN_TOL / 10
+    K = rng.standard_normal((B, Hd, S, D)).astype(np.float32) * 1e-3
+    K[0, 0, 5, 7] = 50.0
+    O = core.flash_attention_f32(dev(Q), dev(K), dev(V), 0.125).cpu().numpy()
+    assert ko.max_rel_err(O, ko.attention(Q, K, V, 0.125)) <= F32_ATTN_TOL / 10
+
+
+def test_flash_attention_f32_config3_shape_properties(core):
+    """BASELINE configs[2]'s shape in fp32: a slice of heads against float64, the whole against fp16-rounded inputs
+    through the fp16 kernel (the two must agree to the fp16 kernel's tolerance), and 4 V gives 4 O bit for bit."""
+    B, Hd, S, D = 8, 16, 2048, 128
+    g = torch.Generator().manual_seed(1234)
+    Q, K, V = (torch.randn((B, Hd, S, D), generator=g).cuda() for _ in range(3))
+    sc = D ** -0.5
+    O = core.flash_attention_f32(Q, K, V, sc)
+    ref = ko.attention(Q[3, 5:7].cpu().numpy(), K[3, 5:7].cpu().numpy(), V[3, 5:7].cpu().numpy(), sc)
+    assert ko.max_rel_err(O[3, 5:7].cpu().numpy(), ref) <= F32_ATTN_TOL / 10
+    O16 = core.flash_attention(Q.half(), K.half(), V.half(), sc)
+    assert float((O16.float() - O).abs().max() / O.abs().max()) <= F16_TOL
+    O4 = core.flash_attention_f32(Q, K, V * 4, sc)
+    assert torch.equal(O4, O * 4)
+
+
+def test_flash_attention_f32_rejects_bad_arguments(core):
+    Q = torch.zeros((1, 1, 64, 48), device='cuda')
+    with pytest.raises(core.FtkError) as e:
+        core.flash_attention_f32(Q, Q, Q)
+    assert e.value.code == -2
+    Q = torch.zeros((1, 1, 64, 64), device='cuda')
+    with pytest.raises(core.FtkError) as e:
+        core.flash_attention_f32(Q, Q, Q, workspace=torch.empty(256, dtype=torch.uint8, device='cuda'))
+    assert e.value.code == -3 and 'workspace' in str(e.value)
+    with pytest.raises(TypeError):
+        core.flash_attention_f32(Q.half(), Q.half(), Q.half())
+    with pytest.raises(ValueError):
+        core.flash_attention_f32(Q, Q[:, :, :32], Q)
+
+
 def test_flash_attention_rejects_bad_shapes(core):
     z = lambda *s: torch.zeros(s, dtype=torch.float16, device='cuda')
     with pytest.raises(core.FtkError) as e:
