@@ -322,6 +322,33 @@ def bench_attention(torch, core, steps, warmup, cpu):
     return res
 
 
+def bench_attention_few_queries(torch, core, steps, warmup, cpu):
+    """Few queries against many keys (a step of decoding with a block of 128 queries): 8 heads x 128 queries x 32768
+    keys, D 128, fp16.  Eight workgroups without a split over the keys; with it the grid fills the chip."""
+    B, Hd, Sq, Skv, D = 1, 8, 128, 32768, 128
+    flop = 4.0 * B * Hd * Sq * Skv * D
+    gen = torch.Generator(device='cpu').manual_seed(1234)
+    Q = torch.randn((B, Hd, Sq, D), generator=gen).half().cuda()
+    K, V = (torch.randn((B, Hd, Skv, D), generator=gen).half().cuda() for _ in range(2))
+    O = torch.empty_like(Q)
+    scale = D ** -0.5
+    ws = torch.empty(int(core.lib.ftk_flash_attn_f16_workspace_bytes(B, Hd, Sq, Skv, D)), dtype=torch.uint8, device='cuda')
+    ms, _ = _events_ms(torch, lambda: core.flash_attention(Q, K, V, scale, out=O, workspace=ws), steps, warmup)
+    ref = O.clone()
+    ms_one, _ = _events_ms(torch, lambda: core.flash_attention(Q, K, V, scale, out=O, split_keys=False), max(3, steps // 4), 1)
+    diff = float((O.float() - ref.float()).abs().max() / ref.float().abs().max())
+    ms_t, _ = _events_ms(torch, lambda: torch.nn.functional.scaled_dot_product_attention(Q, K, V, scale=scale), max(3, steps // 4), 1)
+    nbytes = 2.0 * (2 * B * Hd * Skv * D + 2 * B * Hd * Sq * D)
+    return {'metric': 'TFLOP/s (attention, few queries)', 'value': flop / ms / 1e9, 'unit': 'TFLOP/s', 'ms_per_step': ms, 'dtype': 'f16',
+            'config': {'workload': 'flash attention split over the keys', 'batch': B, 'heads': Hd, 'queries': Sq, 'keys': Skv, 'head_dim': D},
+            'roofline': {'bound': 'hbm', 'achieved': nbytes / ms / 1e6, 'peak': PEAK_HBM_GBS, 'unit': 'GB/s', 'frac': nbytes / ms / 1e6 / PEAK_HBM_GBS,
+                         'traffic': None, 'kernel': 'flash_attn_kernel<128,1,4,1,false,true,true> + attn_merge_kernel<128>',
+                         'algorithmic_bytes_per_launch': nbytes, 'note': '128 MB of K and V read once for 137 GFLOP: AI 1024 FLOP/B, but a launch of '
+                         'tens of microseconds; K and V of this size stay in the 256 MB memory-side cache between steps'},
+            'single_launch': {'ms_per_step': ms_one, 'speedup_of_split': ms_one / ms, 'max_rel_diff': diff},
+            'torch_sdpa': {'ms_per_step': ms_t, 'speedup': ms_t / ms}}
+
+
 def bench_attention_f32(torch, core, steps, warmup, cpu):
     """BASELINE configs[2]'s shape with fp32 Q, K, V, O (the element type of the reference's own attention program):
     every product as three fp16 MFMAs of split operands.  The timed step is the whole entry point: the largest
@@ -1002,7 +1029,7 @@ def main():
     ap.add_argument('--gpus', type=int, default=1)
     ap.add_argument('--steps', type=int, default=50)
     ap.add_argument('--warmup', type=int, default=10)
-    ap.add_argument('--workload', default='b2b', choices=['b2b', 'config1', 'attention', 'stacked_lstm', 'dilated_lstm', 'lstm_f16_h256', 'lstm_f16_h512', 'lstm_f16_h1024', 'lstm_f32_h512', 'lstm_f32_h1024', 'attention_f32', 'gemm', 'online_softmax', 'embedding', 'grid_rnn', 'windowed_attention', 'b2b_ref_shapes', 'copy', 'mfma_rate'])
+    ap.add_argument('--workload', default='b2b', choices=['b2b', 'config1', 'attention', 'stacked_lstm', 'dilated_lstm', 'lstm_f16_h256', 'lstm_f16_h512', 'lstm_f16_h1024', 'lstm_f32_h512', 'lstm_f32_h1024', 'attention_f32', 'attention_few_queries', 'gemm', 'online_softmax', 'embedding', 'grid_rnn', 'windowed_attention', 'b2b_ref_shapes', 'copy', 'mfma_rate'])
     ap.add_argument('--no-extras', action='store_true', help='measure only the chosen workload')
     ap.add_argument('--all', action='store_true', help='also the workloads either side of the path (fp16 / larger stacks, GEMM, softmax, embedding, grid RNN, windowed attention)')
     ap.add_argument('--no-cpu', action='store_true', help='skip the CPU baseline leg')
@@ -1051,6 +1078,7 @@ def main():
         'lstm_f32_h1024': lambda s, w, c: bench_lstm_f32_streamed(torch, core, max(3, s // 10), 1, c, 1024),
         'b2b_ref_shapes': lambda s, w, c: bench_b2b_reference_shapes(torch, core, s, w, c),
         'attention_f32': lambda s, w, c: bench_attention_f32(torch, core, max(5, s // 2), max(2, w // 2), c),
+        'attention_few_queries': lambda s, w, c: bench_attention_few_queries(torch, core, s, w, c),
         'gemm': lambda s, w, c: bench_gemm(torch, core, max(5, s // 5), max(2, w // 5), c),
         'online_softmax': lambda s, w, c: bench_softmax(torch, core, s, w, c),
         'embedding': lambda s, w, c: bench_embedding(torch, core, s, w, c),

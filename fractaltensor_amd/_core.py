@@ -23,7 +23,7 @@ EXPORTS = (
     'ftk_stacked_lstm_wavefront_f32', 'ftk_stacked_lstm_ragged_f32', 'ftk_lstm_set_products', 'ftk_lstm_get_products',
     'ftk_stacked_lstm_opts_f32', 'ftk_stacked_lstm_status', 'ftk_stacked_lstm_small_states', 'ftk_stacked_lstm_noalloc_f32',
     'ftk_stacked_lstm_f16_workspace_bytes', 'ftk_stacked_lstm_f16',
-    'ftk_b2b_gemm_f16', 'ftk_b2b_gemm_f16_supported', 'ftk_b2b_gemm_rowmajor_f16', 'ftk_gemm_f16', 'ftk_batched_gemm_f16', 'ftk_flash_attn_f16', 'ftk_flash_attn_f32_workspace_bytes', 'ftk_flash_attn_f32', 'ftk_online_softmax_f32', 'ftk_embedding_gather_f32',
+    'ftk_b2b_gemm_f16', 'ftk_b2b_gemm_f16_supported', 'ftk_b2b_gemm_rowmajor_f16', 'ftk_gemm_f16', 'ftk_batched_gemm_f16', 'ftk_flash_attn_f16', 'ftk_flash_attn_f16_workspace_bytes', 'ftk_flash_attn_ws_f16', 'ftk_flash_attn_f32_workspace_bytes', 'ftk_flash_attn_f32', 'ftk_online_softmax_f32', 'ftk_embedding_gather_f32',
     'ftk_grid_rnn_workspace_bytes', 'ftk_grid_rnn_f32', 'ftk_windowed_attn_f32',
 )
 
@@ -66,9 +66,11 @@ def _load() -> ctypes.CDLL:
     lib.ftk_grid_rnn_workspace_bytes.argtypes = [ctypes.c_int] * 2
     lib.ftk_flash_attn_f32_workspace_bytes.restype = ctypes.c_size_t
     lib.ftk_flash_attn_f32_workspace_bytes.argtypes = [ctypes.c_int] * 5
+    lib.ftk_flash_attn_f16_workspace_bytes.restype = ctypes.c_size_t
+    lib.ftk_flash_attn_f16_workspace_bytes.argtypes = [ctypes.c_int] * 5
     for name in EXPORTS:
         if name not in ('ftk_last_error', 'ftk_stacked_lstm_workspace_bytes', 'ftk_stacked_lstm_f16_workspace_bytes', 'ftk_grid_rnn_workspace_bytes',
-                        'ftk_flash_attn_f32_workspace_bytes'):
+                        'ftk_flash_attn_f32_workspace_bytes', 'ftk_flash_attn_f16_workspace_bytes'):
             getattr(lib, name).restype = ctypes.c_int
     return lib
 
@@ -506,8 +508,12 @@ def gemm(A, B, out: Optional[torch.Tensor] = None) -> torch.Tensor:
     return C
 
 
-def flash_attention(Q, K, V, scale: Optional[float] = None, out: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """O = softmax(Q K^T scale) V.  Q [B,Hd,Sq,D], K/V [B,Hd,Skv,D], fp16, non-causal."""
+def flash_attention(Q, K, V, scale: Optional[float] = None, out: Optional[torch.Tensor] = None,
+                    workspace: Optional[torch.Tensor] = None, split_keys: bool = True) -> torch.Tensor:
+    """O = softmax(Q K^T scale) V.  Q [B,Hd,Sq,D], K/V [B,Hd,Skv,D], fp16, non-causal.
+    A grid that does not fill the chip (few queries, heads and samples) with many keys is split over the keys and
+    merged (ftk_flash_attn_ws_f16); the workspace for that is allocated here unless one is given, split_keys=False
+    keeps the single launch."""
     f16 = torch.float16
     _req(Q, f16, 'Q'); _req(K, f16, 'K'); _req(V, f16, 'V')
     B, Hd, Sq, D = Q.shape
@@ -520,6 +526,15 @@ def flash_attention(Q, K, V, scale: Optional[float] = None, out: Optional[torch.
     _req_out(O, f16, Q.shape, 'O')
     _count('flash_attention')
     ci = ctypes.c_int
+    need = int(lib.ftk_flash_attn_f16_workspace_bytes(B, Hd, Sq, Skv, D)) if split_keys else 0
+    if need:
+        if workspace is None:
+            workspace = torch.empty(need, dtype=torch.uint8, device=Q.device)
+        _req_workspace(workspace)
+        _count('flash_attention_split_keys')
+        _check(lib.ftk_flash_attn_ws_f16(_ptr(Q), _ptr(K), _ptr(V), _ptr(O), ci(B), ci(Hd), ci(Sq), ci(Skv), ci(D), ctypes.c_float(scale),
+                                         _ptr(workspace), ctypes.c_size_t(workspace.numel() * workspace.element_size()), _stream()))
+        return O
     _check(lib.ftk_flash_attn_f16(_ptr(Q), _ptr(K), _ptr(V), _ptr(O), ci(B), ci(Hd), ci(Sq), ci(Skv), ci(D),
                                   ctypes.c_float(scale), _stream()))
     return O

@@ -64,13 +64,19 @@ __device__ long long fa_trace_buf[FA_TRACE_TILES * 6];
 // RAG: Skv is no multiple of the key tile (the last tile's tail is masked); a template parameter so that the kernel
 // for whole tiles carries none of the masking code (with both in one kernel the tail steps spilled 63 registers per
 // lane to scratch, which every wave wrote once: 87 MB of extra HBM writes per launch at B8 H16 S2048).
-template <int D, int QT, int WAVES, int MINB, bool TRACE, bool RAG>
+// PART: the workgroup takes one contiguous range of the keys (part_keys of them, a multiple of the tile) and leaves
+// its unnormalised accumulators, reference maximum and sum of exponentials in part_o / part_ml for attn_merge_kernel:
+// small grids with many keys are split over the keys so that they fill the chip.
+template <int D, int QT, int WAVES, int MINB, bool TRACE, bool RAG, bool PART = false>
 __global__ __launch_bounds__(WAVES * 64, MINB) void flash_attn_kernel(const _Float16* __restrict__ Q,
                                                          const _Float16* __restrict__ K,
                                                          const _Float16* __restrict__ V,
-                                                         _Float16* __restrict__ O, int Sq, int Skv,
+                                                         _Float16* __restrict__ O, int Sq, int Skv_all,
                                                          float scale_log2e, int nqb,
-                                                         long long* __restrict__ trace, int trace_wave) {
+                                                         long long* __restrict__ trace, int trace_wave,
+                                                         int nparts = 1, int part_keys = 0,
+                                                         float* __restrict__ part_o = nullptr,
+                                                         float* __restrict__ part_ml = nullptr) {
   using L = FaLayout<D>;
   constexpr int DS = D / 16;  // k steps of S^T
   constexpr int DT = D / 32;  // d tiles of O^T
@@ -94,13 +100,20 @@ __global__ __launch_bounds__(WAVES * 64, MINB) void flash_attn_kernel(const _Flo
   int id = blockIdx.x;
   const int total = gridDim.x;
   if ((total & 7) == 0) id = (blockIdx.x & 7) * (total >> 3) + (blockIdx.x >> 3);
+  int part = 0;
+  if constexpr (PART) {
+    part = id % nparts;
+    id /= nparts;
+  }
   const int bh = id / nqb;
   const int qb = id - bh * nqb;
   const int q_base = qb * (WAVES * 32 * QT) + wave * (32 * QT);
+  const int key_first = PART ? part * part_keys : 0;
+  const int Skv = PART ? min(part_keys, Skv_all - key_first) : Skv_all;   // the keys this workgroup sees
 
   const _Float16* Qg = Q + (size_t)bh * Sq * D;
-  const _Float16* Kg = K + (size_t)bh * Skv * D;
-  const _Float16* Vg = V + (size_t)bh * Skv * D;
+  const _Float16* Kg = K + ((size_t)bh * Skv_all + key_first) * D;
+  const _Float16* Vg = V + ((size_t)bh * Skv_all + key_first) * D;
   _Float16* Og = O + (size_t)bh * Sq * D;
 
   // ---- Q row fragments, resident for the whole kernel, pre-multiplied by
@@ -480,6 +493,30 @@ __global__ __launch_bounds__(WAVES * 64, MINB) void flash_attn_kernel(const _Flo
   // the last step: every lane writes its pieces into the wave's own padded tile, then 2D/16 lanes per row read 16
   // bytes each and the wave stores whole rows, 1 KB of consecutive bytes per instruction.  LDS executes a wave's
   // instructions in order, so the wave needs no barrier between its writes and its reads.
+  if constexpr (PART) {
+    // a part's result: O^T unnormalised, relative to the part's reference maximum m (in exponent units), and the sum
+    // of exponentials l relative to the same m: what the merge rule of an online softmax takes
+    // (kaleido/core/device/kernels/online_softmax.h:27-30)
+#pragma unroll
+    for (int qt = 0; qt < QT; ++qt) {
+      const float l = l_run[qt] + __shfl_xor(l_run[qt], 32);
+      const int row = q_base + 32 * qt + j;
+      if (row < Sq) {
+        const size_t at = ((size_t)bh * nparts + part) * Sq + row;
+        if (hh == 0) {
+          part_ml[2 * at] = -nref[qt][0];
+          part_ml[2 * at + 1] = l;
+        }
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+          for (int g = 0; g < 4; ++g)
+            *reinterpret_cast<float4*>(part_o + at * D + 32 * dt + 8 * g + 4 * hh) =
+                make_float4(oacc[qt][dt][4 * g], oacc[qt][dt][4 * g + 1], oacc[qt][dt][4 * g + 2], oacc[qt][dt][4 * g + 3]);
+      }
+    }
+    return;
+  }
   constexpr int ORS = 2 * D + 16;        // padded row: the 32 rows' 8-byte pieces spread over all banks
   constexpr int LPR = D / 8;             // 16-byte chunks per row
   unsigned char* const ot = smem + wave * (32 * ORS);
@@ -944,6 +981,80 @@ static int launch_fa(const void* Q, const void* K, const void* V, void* O, int B
   return check_launch("flash_attn_kernel");
 }
 
+// The parts of a row merged by the rule of an online softmax: m = max m_p, l = sum l_p 2^(m_p - m),
+// O = sum O_p 2^(m_p - m) / l.  One thread per (row, four columns).
+template <int D>
+__global__ __launch_bounds__(256) void attn_merge_kernel(const float* __restrict__ part_o, const float* __restrict__ part_ml,
+                                                        _Float16* __restrict__ O, int nparts, int Sq, long long rows) {
+  constexpr int CPR = D / 4;
+  const long long idx = (long long)blockIdx.x * 256 + threadIdx.x;
+  if (idx >= rows * CPR) return;
+  const long long row = idx / CPR;
+  const int c = (int)(idx - row * CPR);
+  const long long bh = row / Sq;
+  const int r = (int)(row - bh * Sq);
+  float m = -INFINITY;
+  for (int p = 0; p < nparts; ++p) m = fmaxf(m, part_ml[2 * ((bh * nparts + p) * Sq + r)]);
+  float l = 0.0f;
+  float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
+  for (int p = 0; p < nparts; ++p) {
+    const long long at = (bh * nparts + p) * Sq + r;
+    const float w = __builtin_amdgcn_exp2f(part_ml[2 * at] - m);
+    l += w * part_ml[2 * at + 1];
+    const float4 o = *reinterpret_cast<const float4*>(part_o + at * D + 4 * c);
+    acc.x += w * o.x; acc.y += w * o.y; acc.z += w * o.z; acc.w += w * o.w;
+  }
+  const float inv = 1.0f / l;
+  const v4h out = {(_Float16)(acc.x * inv), (_Float16)(acc.y * inv), (_Float16)(acc.z * inv), (_Float16)(acc.w * inv)};
+  *reinterpret_cast<v4h*>(O + row * D + 4 * c) = out;
+}
+
+// How many parts the keys are cut into (1: no split).  A grid of 128-row query blocks that fills less than half the
+// chip, with enough keys that every part keeps at least four tiles.
+static int fa_split_parts(long long bh, int Sq, int Skv, int cus, int* part_keys) {
+  *part_keys = Skv;
+  const long long blocks = (long long)((Sq + 127) / 128) * bh;
+  if (blocks * 2 > cus || Skv < 2048) return 1;
+  long long want = std::min<long long>(std::min<long long>(cus / blocks, 64), Skv / (4 * FA_KT));
+  if (want < 2) return 1;
+  const int keys = (int)(((Skv + want - 1) / want + FA_KT - 1) / FA_KT * FA_KT);
+  *part_keys = keys;
+  return (Skv + keys - 1) / keys;
+}
+
+static size_t fa_split_bytes(long long bh, int Sq, int D, int nparts) {
+  return (size_t)nparts * bh * Sq * (D + 2) * sizeof(float);
+}
+
+template <int D>
+static int launch_fa_split(const void* Q, const void* K, const void* V, void* O, int BH, int Sq, int Skv, float scale, int nparts,
+                           int part_keys, float* ws, int lds_max, hipStream_t s) {
+  constexpr int WAVES = 4;
+  const size_t lds = (size_t)3 * FaLayout<D>::KTB + (size_t)2 * FaLayout<D>::VTB;
+  if ((int)lds > lds_max) return fail(FTK_ERR_UNSUPPORTED_SHAPE, "ftk_flash_attn_ws_f16: needs %zu bytes of LDS", lds);
+  static DeviceOnce attr_once;
+  unsigned attr_bit;
+  if (attr_once.pending(&attr_bit)) {
+    FTK_HIP(hipFuncSetAttribute((const void*)flash_attn_kernel<D, 1, WAVES, 1, false, true, true>,
+                                hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+    attr_once.done(attr_bit);
+  }
+  const int nqb = (Sq + WAVES * 32 - 1) / (WAVES * 32);
+  const long long total = (long long)nqb * BH * nparts;
+  if (total > 0x7fffffffLL) return fail(FTK_ERR_UNSUPPORTED_SHAPE, "ftk_flash_attn_ws_f16: grid too large");
+  float* part_o = ws;
+  float* part_ml = ws + (size_t)nparts * BH * Sq * D;
+  hipLaunchKernelGGL((flash_attn_kernel<D, 1, WAVES, 1, false, true, true>), dim3((unsigned)total), dim3(WAVES * 64), lds, s,
+                     (const _Float16*)Q, (const _Float16*)K, (const _Float16*)V, (_Float16*)O, Sq, Skv, scale * 1.4426950408889634f, nqb,
+                     (long long*)nullptr, 0, nparts, part_keys, part_o, part_ml);
+  int rc = check_launch("flash_attn_kernel (key parts)");
+  if (rc) return rc;
+  const long long rows = (long long)BH * Sq;
+  const long long threads = rows * (D / 4);
+  hipLaunchKernelGGL(attn_merge_kernel<D>, dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, s, part_o, part_ml, (_Float16*)O, nparts, Sq, rows);
+  return check_launch("attn_merge_kernel");
+}
+
 // Tuning hook: FTK_FA_VARIANT=1|3 pins the tiling variant (read once).
 static int fa_variant_override() {
   static int v = -1;
@@ -969,6 +1080,41 @@ extern "C" int ftk_debug_read_fa_trace(long long* host_dst, int n) {
   return FTK_OK;
 }
 #endif
+
+extern "C" size_t ftk_flash_attn_f16_workspace_bytes(int B, int Hd, int Sq, int Skv, int D) {
+  using namespace ftk;
+  if (B <= 0 || Hd <= 0 || Sq <= 0 || Skv <= 0 || D <= 0) return 0;
+  const DeviceProps* dp = nullptr;
+  const int cus = device_props(&dp) == FTK_OK ? dp->cus : 256;   // without a device: the part this library is written for
+  int keys = 0;
+  const int nparts = fa_split_parts((long long)B * Hd, Sq, Skv, cus, &keys);
+  return nparts > 1 ? fa_split_bytes((long long)B * Hd, Sq, D, nparts) : 0;
+}
+
+extern "C" int ftk_flash_attn_ws_f16(const void* Q, const void* K, const void* V, void* O, int B, int Hd, int Sq, int Skv, int D,
+                                     float scale, void* workspace, size_t workspace_bytes, ftk_stream_t stream) {
+  using namespace ftk;
+  if (Q && K && V && O && B > 0 && Hd > 0 && Sq > 0 && Skv > 0 && (D == 32 || D == 64 || D == 96 || D == 128) && workspace &&
+      (long long)B * Hd <= (1LL << 24)) {
+    const DeviceProps* dp = nullptr;
+    int rc = device_props(&dp);
+    if (rc) return rc;
+    int keys = 0;
+    const long long bh = (long long)B * Hd;
+    const int nparts = fa_split_parts(bh, Sq, Skv, dp->cus, &keys);
+    if (nparts > 1 && workspace_bytes >= fa_split_bytes(bh, Sq, D, nparts) && reinterpret_cast<uintptr_t>(workspace) % 16 == 0) {
+      hipStream_t s = (hipStream_t)stream;
+      float* ws = reinterpret_cast<float*>(workspace);
+      switch (D) {
+        case 32: return launch_fa_split<32>(Q, K, V, O, (int)bh, Sq, Skv, scale, nparts, keys, ws, dp->lds_optin, s);
+        case 64: return launch_fa_split<64>(Q, K, V, O, (int)bh, Sq, Skv, scale, nparts, keys, ws, dp->lds_optin, s);
+        case 96: return launch_fa_split<96>(Q, K, V, O, (int)bh, Sq, Skv, scale, nparts, keys, ws, dp->lds_optin, s);
+        default: return launch_fa_split<128>(Q, K, V, O, (int)bh, Sq, Skv, scale, nparts, keys, ws, dp->lds_optin, s);
+      }
+    }
+  }
+  return ftk_flash_attn_f16(Q, K, V, O, B, Hd, Sq, Skv, D, scale, stream);   // argument checks and the unsplit kernels
+}
 
 extern "C" int ftk_flash_attn_f16(const void* Q, const void* K, const void* V, void* O, int B, int Hd, int Sq, int Skv,
                                   int D, float scale, ftk_stream_t stream) {

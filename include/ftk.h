@@ -453,6 +453,24 @@ int ftk_flash_attn_f16(const void* Q, const void* K, const void* V, void* O,
                        ftk_stream_t stream);
 
 /*
+ * The same call with a workspace, for grids that do not fill the chip: when
+ * batch x heads x (query blocks of 128 rows) covers less than half of the
+ * compute units and there are at least 2048 keys, the keys are cut into up to
+ * 64 contiguous parts, every part runs as a workgroup of its own and leaves
+ * (reference maximum, sum of exponentials, unnormalised O) in the workspace,
+ * and a second launch merges the parts by the rule of an online softmax
+ * (kaleido/core/device/kernels/online_softmax.h:27-30).
+ * ftk_flash_attn_f16_workspace_bytes is 0 for shapes that are not split;
+ * without a sufficient workspace the call is ftk_flash_attn_f16.  The
+ * reference has no device kernel for this program.
+ */
+size_t ftk_flash_attn_f16_workspace_bytes(int B, int Hd, int Sq, int Skv, int D);
+int ftk_flash_attn_ws_f16(const void* Q, const void* K, const void* V, void* O,
+                          int B, int Hd, int Sq, int Skv, int D, float scale,
+                          void* workspace, size_t workspace_bytes,
+                          ftk_stream_t stream);
+
+/*
  * The same attention with fp32 Q, K, V and O, [B,Hd,S,D] row-major, D of 32,
  * 64, 96 or 128: the element type of the reference's program
  * (examples/flash_attention/flash_attention.py:14-91 on kaleido.float32

@@ -1007,6 +1007,32 @@ def test_flash_attention_config3_full_size(core):
     assert torch.equal(O4[normal], (O * 4)[normal])
 
 
+@pytest.mark.parametrize('B,Hd,Sq,Skv,D', [
+    (1, 2, 100, 4096, 128),        # two heads of 100 queries: two workgroups without the split
+    (1, 1, 1, 8192, 64),           # one query against 8192 keys
+    (2, 2, 130, 5000, 96),         # ragged keys (the last part ends inside a tile), two query blocks
+    (1, 4, 64, 2048, 32),          # the fewest keys that are split
+    (1, 8, 128, 32768, 128),
+])
+def test_flash_attention_split_over_the_keys(core, B, Hd, Sq, Skv, D):
+    """A grid that fills less than half the chip is cut over the keys; the parts' (maximum, sum, unnormalised O) are
+    merged by the rule of an online softmax (online_softmax.h:27-30).  Against float64, and against the single launch."""
+    rng = np.random.default_rng(23)
+    Q, K, V = (rng.standard_normal((B, Hd, s, D)).astype(np.float16) for s in (Sq, Skv, Skv))
+    K[..., : Skv // 3, :] *= 0.5                                         # parts with different maxima
+    sc = D ** -0.5
+    before = core.launch_counts.get('flash_attention_split_keys', 0)
+    O = core.flash_attention(dev(Q), dev(K), dev(V), sc)
+    assert core.launch_counts.get('flash_attention_split_keys', 0) == before + 1
+    assert int(core.lib.ftk_flash_attn_f16_workspace_bytes(B, Hd, Sq, Skv, D)) > 0
+    ref = ko.attention(Q[:, :2, :64], K[:, :2], V[:, :2], sc, dtype=np.float32)
+    assert ko.max_rel_err(O[:, :2, :64].float().cpu().numpy(), ref) <= F16_TOL
+    single = core.flash_attention(dev(Q), dev(K), dev(V), sc, split_keys=False)
+    assert float((O.float() - single.float()).abs().max() / single.float().abs().max()) <= 2e-3
+    # a grid that fills the chip is not split
+    assert int(core.lib.ftk_flash_attn_f16_workspace_bytes(8, 16, 2048, 2048, 128)) == 0
+
+
 F32_ATTN_TOL = 1e-4      # the fp32 path's bound; the split products are expected two orders inside it
 
 
