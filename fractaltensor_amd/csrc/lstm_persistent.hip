@@ -84,6 +84,7 @@ constexpr int kMaxBlocks = 64;     // 32-row blocks a ragged batch may have (B <
 constexpr int kSplitTop = 14;          // a scale group's largest magnitude lands in [2^14, 2^15)
 constexpr float kSplitRest = 2048.0f;  // 2^11: what the remainder is multiplied by before it is rounded
 constexpr float kSplitAct = 16384.0f;  // 2^14: the scale of h
+constexpr int kSplitCommon = 12;       // input rows whose largest magnitude is below 2^(16 - 12) take the scale 2^12
 // h * 2^14 below 2^-23 (|h| < 2^-37, 7e-12): the remainder plane is an fp16 subnormal there and value plus remainder
 // keep fewer than 13 bits
 constexpr unsigned kSmallStateBits = (127u - 23u) << 23;
@@ -110,6 +111,7 @@ struct PersistArgs {
   int trace_q;            // logical workgroup whose item timeline is recorded, or -1
   long long* trace;       // [items][8] 100 MHz clock stamps of that workgroup
   int dil[kMaxLayers];
+  int paired;                // 1: workgroups of pipelined layers take two row blocks per item (split products)
   int ragged;                // 1: row block rb takes part in steps t < steps_of[rb] only
   int steps_of[kMaxBlocks];
 };
@@ -124,9 +126,10 @@ __device__ __forceinline__ int flag_load(const int* flag) {
 // A flag is kFlagStride bytes, one per producer wave (up to 16 column slices x 4 waves); lane i looks at byte i.
 // Every wait is bounded: when the polls run out the status word is set and the caller drains.
 constexpr int kFlagStride = 64;
+// (Lanes past the last producer look at the last producer's byte: with a branch around the load the compiler waits for
+// the byte where the branches join, and a look that is meant to be on its way while the wave works costs a round trip.)
 __device__ __forceinline__ int flag_bytes_load(const unsigned char* flag, int lane, int target) {
-  if (lane >= target) return 1;
-  return __hip_atomic_load(flag + lane, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  return __hip_atomic_load(flag + min(lane, target - 1), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 __device__ __forceinline__ bool all_set(int v) { return __builtin_amdgcn_ballot_w64(v != 0) == ~0ull; }
 __device__ __forceinline__ bool wait_bytes(const unsigned char* flag, int lane, int target, int* status, int spin_limit) {
@@ -195,7 +198,9 @@ constexpr int kStageC = 0, kStageH = 32 * kStageRow32, kStageTop = 2 * 32 * kSta
 constexpr int kStageBytes = kStageRest + 32 * kStageRow16;
 constexpr int kRatioOffset = 2 * P_TILE * (int)sizeof(float) + 1024 + 2 * kStageBytes;   // bytes; [2 tile buffers][64 floats]
 constexpr int kVoteOffset = kRatioOffset + 2 * 64 * (int)sizeof(float);   // bytes; one int per wave (serial schedule)
-constexpr size_t kPersistLds = (size_t)kVoteOffset + 64;  // tiles, prefetch scrap, staging, row ratios, votes
+constexpr int kGateTableOffset = kVoteOffset + 64;   // bytes; [4 waves][2 lane halves][16 x (factor, bias)] (paired schedule)
+constexpr size_t kPersistLds = (size_t)kGateTableOffset + 8 * 32 * sizeof(float);  // tiles, prefetch scrap, staging, row ratios, votes, gate table
+static_assert(kPersistLds <= 160 * 1024, "the workgroup's LDS");
 // Kernel flavours.  kProductsF32 / kProductsSplit: fp32 data, H = 256, the two ways of forming the products.
 // kHalfData: fp16 inputs, weights, h and c (what the reference's CuTe LSTM stores), one fp16 MFMA per product
 // with fp32 accumulation, H = 512: a row of 512 fp16 takes the 1024 bytes a row of 256 fp32 takes, and a
@@ -252,6 +257,14 @@ void lstm_persistent_kernel(PersistArgs a) {
   // fp16 data: rows k = 16s + 8hh .. +7 of the column for MFMA step s, 64 steps.
   const int col = (j >> 3) * HID + 32 * pc + 8 * wave + (j & 7);
   const float* wl = a.WU + (size_t)l * PK * PN + col;
+  // Split products, first layer: input rows are split on a scale of their own, and their products move to h's scale
+  // by a per-row factor before the h products join them -- unless every row of this launch's input took the common
+  // scale 2^kSplitCommon (lstm_split_rows_kernel says so in the status block's third word).  Then the factor is the
+  // same power of two for all rows, the input half of this layer's weights takes it, exactly, and nothing is
+  // rescaled per item.
+  const bool x_has_common_scale = SPLIT && l == 0 && flag_load(a.status + 2) == 0;
+  const float xfold = x_has_common_scale ? kSplitAct / (float)(1 << kSplitCommon) : 1.0f;
+  const bool x_rescaled = SPLIT && l == 0 && !x_has_common_scale;
   float wr[MODE == kProductsF32 ? PK / 2 : 1];
   v8h whi[SPLIT ? PK / 16 : 1], wlo[SPLIT ? PK / 16 : 1];
   v8h wh[F16 ? 2 * HID / 16 : 1];
@@ -272,12 +285,13 @@ void lstm_persistent_kernel(PersistArgs a) {
       wr[s] = wl[(size_t)k * PN];
     }
   } else {
-    // the column's largest magnitude decides its power-of-two scale
+    // the column's largest magnitude decides its power-of-two scale.  (First layer, every input row on the common
+    // scale: the input rows of WU take the factor between that scale and h's, see x_has_common_scale.)
     float cmax = 0.f;
 #pragma unroll
     for (int s = 0; s < PK / 16; ++s)
 #pragma unroll
-      for (int e = 0; e < 8; ++e) cmax = fmaxf(cmax, fabsf(wl[(size_t)(16 * s + 8 * hh + e) * PN]));
+      for (int e = 0; e < 8; ++e) cmax = fmaxf(cmax, fabsf(wl[(size_t)(16 * s + 8 * hh + e) * PN]) * (s < PK / 32 ? xfold : 1.0f));
     cmax = fmaxf(cmax, __shfl_xor(cmax, 32));
     const int eb = min(max((int)((__float_as_uint(cmax) >> 23) & 0xff), 15), 254);
     const float wscale = __uint_as_float((unsigned)(127 + kSplitTop + 127 - eb) << 23);  // column max -> [2^14, 2^15)
@@ -287,7 +301,7 @@ void lstm_persistent_kernel(PersistArgs a) {
     for (int s = 0; s < PK / 16; ++s)
 #pragma unroll
       for (int e = 0; e < 8; ++e) {
-        const float w = wl[(size_t)(16 * s + 8 * hh + e) * PN] * wscale;
+        const float w = wl[(size_t)(16 * s + 8 * hh + e) * PN] * (s < PK / 32 ? xfold * wscale : wscale);
         const _Float16 top = (_Float16)w;
         whi[s][e] = top;
         wlo[s][e] = (_Float16)((w - (float)top) * kSplitRest);
@@ -410,7 +424,7 @@ void lstm_persistent_kernel(PersistArgs a) {
     // being loaded into a register: a register load that late in an item is waited for behind the copies of the
     // tile after next, which nothing else waits for before the item's end.
     if constexpr (SPLIT) {
-      if (l == 0 && with_x && wave_u == 0)
+      if (x_rescaled && with_x && wave_u == 0)
         lds_dma4(a.xratio + (size_t)t * B, 4u * (unsigned)min(rb * 32 + (lane & 31), B - 1), tile_lds + (unsigned)kRatioOffset + 256u * (unsigned)buf);
     }
     if (row0 + 8 <= B) {
@@ -552,13 +566,13 @@ void lstm_persistent_kernel(PersistArgs a) {
   // the ratio of this lane's row in the tile that has landed in buffer buf
   auto load_ratio = [&](int buf) __attribute__((always_inline)) -> float {
     if constexpr (SPLIT) {
-      if (l == 0) return reinterpret_cast<const float*>(reinterpret_cast<const unsigned char*>(tile) + kRatioOffset)[64 * buf + j];
+      if (x_rescaled) return reinterpret_cast<const float*>(reinterpret_cast<const unsigned char*>(tile) + kRatioOffset)[64 * buf + j];
     }
     return 1.0f;
   };
   auto rescale_x = [&](float ratio) __attribute__((always_inline)) {
     if constexpr (SPLIT) {
-      if (l == 0) {
+      if (x_rescaled) {
 #pragma unroll
         for (int r = 0; r < 16; ++r) { acc0[r] *= ratio; acc1[r] *= ratio; }
       }
@@ -643,12 +657,11 @@ void lstm_persistent_kernel(PersistArgs a) {
   };
   // What consumers on other compute units read leaves through write-through stores (fp32 products: h;
   // split products: the two planes), the rest through the cache.
-  auto store_item = [&](int n, int sbuf) __attribute__((always_inline)) {
-    const int t = item_t(n), rb = item_rb(n);
+  auto store_block = [&](int t, int rb, bool is_live, int sbuf) __attribute__((always_inline)) {
     const int rl = 8 * wave + (lane >> 3), cc = lane & 7;
     const int rg = rb * 32 + rl;
     if constexpr (F16) {
-      if (alive && rg < B && live(n)) {
+      if (alive && rg < B && is_live) {
         const unsigned char* sb = stage + sbuf * kStageBytes;
         const size_t at16 = (((size_t)l * T + t) * B + rg) * HID + 32 * pc + 4 * cc;
         coherent_store8h(a.hsp + at16, *reinterpret_cast<const v4h*>(sb + kStageTop + rl * kStageRow16 + 8 * cc));
@@ -657,7 +670,7 @@ void lstm_persistent_kernel(PersistArgs a) {
       }
       return;
     }
-    if (alive && rg < B && live(n)) {
+    if (alive && rg < B && is_live) {
       const unsigned char* sb = stage + sbuf * kStageBytes;
       const size_t at = ((size_t)l * T + t) * cell + (size_t)rg * PH + 32 * pc + 4 * cc;
       const float4 cv = *reinterpret_cast<const float4*>(sb + kStageC + rl * kStageRow32 + 16 * cc);
@@ -674,6 +687,7 @@ void lstm_persistent_kernel(PersistArgs a) {
       }
     }
   };
+  auto store_item = [&](int n, int sbuf) __attribute__((always_inline)) { store_block(item_t(n), item_rb(n), live(n), sbuf); };
   // workgroup barrier that waits for nothing by itself: what has to be complete before it is waited for
   // explicitly (__syncthreads would also wait for the acknowledgement of every store in flight)
   auto barrier = [&]() __attribute__((always_inline)) {
@@ -681,10 +695,9 @@ void lstm_persistent_kernel(PersistArgs a) {
     __builtin_amdgcn_s_barrier();
     asm volatile("" ::: "memory");
   };
-  auto load_cprev = [&](int n) __attribute__((always_inline)) -> float4 {
-    const int t = item_t(n), rb = item_rb(n);
+  auto load_cprev_of = [&](int t, int rb, bool is_live) __attribute__((always_inline)) -> float4 {
     float4 cp = make_float4(0.f, 0.f, 0.f, 0.f);
-    if (alive && t >= d && live(n)) {
+    if (alive && t >= d && is_live) {
       const int rgc = min(rb * 32 + jb, B - 1);
       if constexpr (F16) {
         const v4h c16 = *reinterpret_cast<const v4h*>(reinterpret_cast<const _Float16*>(a.csss) +
@@ -696,6 +709,7 @@ void lstm_persistent_kernel(PersistArgs a) {
     }
     return cp;
   };
+  auto load_cprev = [&](int n) __attribute__((always_inline)) -> float4 { return load_cprev_of(item_t(n), item_rb(n), live(n)); };
   // every wave publishes its own part of an item: its stores acknowledged, then its byte of the flag
   auto publish = [&](int n) __attribute__((always_inline)) {
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
@@ -769,6 +783,313 @@ void lstm_persistent_kernel(PersistArgs a) {
       if (tracing) a.trace[TS * n + 7] = wall_clock64();
     }
     return;
+  }
+
+  // ---- paired schedule (split products): an item is TWO row blocks (a, b) of one time step, 64 batch rows.
+  // What an item costs beyond its MFMAs -- the looks at the producers' flags, the waits for the stores'
+  // acknowledgement, the barriers -- is paid once per hand-over whatever the number of rows, and with two blocks in
+  // flight the activations of one block run on the vector pipeline while the matrix pipeline forms the other block's
+  // products.  LDS has no room for two 64-row tiles; the tile is kept as two half buffers instead, XA = the 64 rows'
+  // x columns and HB = their h columns (1 KB per row each), and the copies into one half are dealt out, one per
+  // contraction step, over the MFMAs that read the other half, where a copy instruction meets a memory pipeline that
+  // is not busy and does not hold the wave at issue.  Per item p, with X / H the halves of the products and E the
+  // activations (which also split h into its planes and leave everything in a staging area):
+  //   Xa(p) with Eb(p-1) -> staging 1    | the own layer's flags for item p are on their way
+  //   Xb(p)                              | this wave's rows of item p's h columns -> HB
+  //   wait for everything outstanding (the stores of block a of item p-1 among it: that block is published)
+  //   barrier 1: HB and staging 1 complete, XA free
+  //   stores of block b of item p-1 from staging 1
+  //   Ha(p)                              | rows of item p+1's x columns -> XA, if the layer below was seen ready
+  //   Hb(p) with Ea(p) -> staging 0      | the same, second block
+  //   (a wave that could not request its x rows waits for the layer below and requests them now)
+  //   wait for everything outstanding (block b of item p-1 is published)
+  //   barrier 2: XA and staging 0 complete, HB free
+  //   stores of block a of item p from staging 0
+  // A wave only ever waits for the copies it issued itself, and fragment reads of a half follow a barrier that every
+  // wave reached after such a wait.  Flags stay per 32-row block, so layers on the other schedules hand over to this
+  // one and back.  The h columns of item p need this layer's item p - (own distance >= 2), whose second block was
+  // published before barrier 2 of item p-1.
+  if constexpr (SPLIT) {
+    const int ppt = (my_rbs + 1) / 2;            // pair items per time step
+    if (a.paired && my_rbs >= 2 && (long long)d * ppt >= 2) {
+      constexpr int HLD = 1040;                  // bytes per row of a half buffer: 16 more than the row's two planes
+      const int n_pairs = T * ppt;
+      unsigned char* const xa = reinterpret_cast<unsigned char*>(tile);
+      unsigned char* const hb = xa + 64 * HLD;
+      const unsigned xa_lds = tile_lds, hb_lds = tile_lds + 64u * HLD;
+      // The per-register factors and biases of the gate sums move to a table in LDS, one set per wave and lane half,
+      // in the order the activations take them: with four accumulators per lane the registers are needed elsewhere.
+      float2* const gtab = reinterpret_cast<float2*>(reinterpret_cast<unsigned char*>(tile) + kGateTableOffset) + 16 * (2 * wave + hh);
+      if (j == 0) {
+#pragma unroll
+        for (int m = 0; m < 16; ++m) gtab[m] = make_float2(esc[4 * (m & 3) + (m >> 2)], ebias[4 * (m & 3) + (m >> 2)]);
+      }
+      // an item: time step t, row blocks rb0 and rb1 = rb0 + pr; on0 / on1: the block exists and is live at t.  Rows
+      // are sorted by length, so a live second block has a live first one.
+      struct Pair { int t, i, rb0, rb1; bool on0, on1; };
+      auto pair_at = [&](int t, int i) __attribute__((always_inline)) -> Pair {
+        Pair x;
+        x.t = t; x.i = i;
+        x.rb0 = prs + pr * (2 * i);
+        x.rb1 = x.rb0 + pr;
+        x.on0 = !a.ragged || t < a.steps_of[x.rb0];
+        x.on1 = 2 * i + 1 < my_rbs && (!a.ragged || t < a.steps_of[min(x.rb1, kMaxBlocks - 1)]);
+        return x;
+      };
+      auto pair_after = [&](const Pair& x) __attribute__((always_inline)) -> Pair {
+        return x.i + 1 < ppt ? pair_at(x.t, x.i + 1) : pair_at(x.t + 1, 0);
+      };
+      auto x_rows = [&](int t) { return reinterpret_cast<const char*>((l == 0) ? xin + (size_t)t * cell : hin + ((size_t)(l - 1) * T + t) * cell); };
+      auto h_rows = [&](int t) { return reinterpret_cast<const char*>(hin + ((size_t)l * T + (t - d)) * cell); };
+      // A wave's 8 rows of a row block: where the first of them lies in global memory (the rows are 1 KB apart) and
+      // where it goes in LDS.  The batch is a multiple of 8 rows here, so the 8 rows are all inside it or all beyond
+      // its end; those beyond are copied from the batch's last 8 rows instead (nobody stores what comes of them).
+      struct Rows { bool on; const char* g; unsigned lds; };
+      auto rows_of = [&](const char* src, int rb, unsigned half_lds, int sub, bool on) __attribute__((always_inline)) -> Rows {
+        return Rows{on, src + (size_t)min(rb * 32 + 8 * wave_u, B - 8) * 1024, half_lds + (unsigned)((32 * sub + 8 * wave_u) * HLD)};
+      };
+      auto copy_row = [&](const Rows& x, auto r_c) __attribute__((always_inline)) {
+        constexpr int r = decltype(r_c)::value;
+        lds_dma16<(r & 3) * 1024, kCoherentTiles>(x.g + (r >> 2) * 4096, lane16, x.lds + (unsigned)(r * HLD));
+      };
+      auto copy_block = [&](const char* src, int rb, unsigned half_lds, int sub) __attribute__((always_inline)) {
+        const Rows x = rows_of(src, rb, half_lds, sub, true);
+        static_for<8>([&](auto r_c) __attribute__((always_inline)) { copy_row(x, r_c); });
+      };
+      auto copy_ratios = [&](const Pair& x) __attribute__((always_inline)) {   // first layer: the rows' scale ratios travel with their x columns
+        if (!x_rescaled || wave_u != 0) return;
+        if (x.on0) lds_dma4(a.xratio + (size_t)x.t * B, 4u * (unsigned)min(x.rb0 * 32 + (lane & 31), B - 1), tile_lds + (unsigned)kRatioOffset);
+        if (x.on1) lds_dma4(a.xratio + (size_t)x.t * B, 4u * (unsigned)min(x.rb1 * 32 + (lane & 31), B - 1), tile_lds + (unsigned)kRatioOffset + 256u);
+      };
+      // One look at an item's two flags of layer ll, step t: lanes 0..31 take the bytes of block a's 32 producer
+      // waves, lanes 32..63 those of block b (of block a again when there is no block b).  The load is unconditional
+      // and its address always valid, so that nothing makes the compiler wait for it where it is issued: the wave
+      // asks, works, and reads the answer later.  Callers ignore the answer where there is no such dependency.
+      static_assert(FLAG_TARGET == 32, "one half of the wave per row block");
+      auto look = [&](int ll, int t, const Pair& x) __attribute__((always_inline)) -> int {
+        const unsigned char* f = flag_of(max(ll, 0), max(t, 0), x.rb0) + (lane & 31);
+        if (lane >= 32 && x.on1) f += (x.rb1 - x.rb0) * kFlagStride;
+        return __hip_atomic_load(f, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      };
+      auto wait_pair = [&](const Pair& x, int ll, int t) __attribute__((always_inline)) -> bool {
+        bool ok = true;
+        if (x.on0) ok = wait_bytes(flag_of(ll, t, x.rb0), lane, FLAG_TARGET, a.status, a.spin_limit);
+        if (ok && x.on1) ok = wait_bytes(flag_of(ll, t, x.rb1), lane, FLAG_TARGET, a.status, a.spin_limit);
+        asm volatile("" ::: "memory");   // the copies stay behind the flag reads
+        return ok;
+      };
+      auto wait_below = [&](const Pair& x) __attribute__((always_inline)) -> bool { return l == 0 || wait_pair(x, l - 1, x.t); };
+      auto wait_own = [&](const Pair& x) __attribute__((always_inline)) -> bool { return x.t < d || wait_pair(x, l, x.t - d); };
+      // a wave publishes its part of one row block of an item; its stores have been waited for
+      auto publish_block = [&](int t, int rb, bool on) __attribute__((always_inline)) {
+        if (lane == 0 && alive && on)
+          __hip_atomic_store(flag_of(l, t, rb) + 4 * pc + wave, (unsigned char)1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      };
+      auto wait_all = [&]() __attribute__((always_inline)) {
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+        __builtin_amdgcn_s_waitcnt(0);
+      };
+      // piece m (0..15) of a block's activations, straight from the two accumulators: gate m & 3 of unit m >> 2
+      auto pair_piece = [&](const v16f& em, const v16f& er, const float4& cp, float (&hv)[4], float (&cv)[4], const float2 sb, auto mc) __attribute__((always_inline)) {
+        constexpr int m = decltype(mc)::value;
+        constexpr int r = m >> 2, g = m & 3, reg = 4 * g + r;
+        const float cpv[4] = {cp.x, cp.y, cp.z, cp.w};
+        auto inv1p = [](float e) { return __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(e)); };
+        const float v = sb.x * (em[reg] + (1.0f / kSplitRest) * er[reg]) + sb.y;
+        if constexpr (g == 0) eg_i = inv1p(v);
+        if constexpr (g == 1) eg_f = inv1p(v);
+        if constexpr (g == 2) eg_o = inv1p(v);
+        if constexpr (g == 3) {
+          const float cand = tanh_f(v);
+          cv[r] = eg_f * cpv[r] + eg_i * cand;
+          hv[r] = eg_o * tanh_f(cv[r]);
+        }
+      };
+      auto activations_alone = [&](const v16f& em, const v16f& er, const float4& cp, int sbuf) __attribute__((always_inline)) {
+        float hv[4], cv[4];
+        static_for<16>([&](auto mc) __attribute__((always_inline)) { pair_piece(em, er, cp, hv, cv, gtab[decltype(mc)::value], mc); });
+        stage_results(hv, cv, sbuf);
+      };
+      // Copies dealt out over a phase's 16 steps.  NW = 16: one per step, rows 0..7 of group lo, then of group hi;
+      // NW = 8: group lo only, every other step.
+      struct Weave { Rows lo, hi; };
+      // One half (HF 0: x columns, 1: h columns) of one row block's products: rows 32 SUB.. of half buffer hbuf, into
+      // am / ar.  EPI: the activations of ANOTHER block, from em / er, cp, are dealt out over the steps as well and
+      // end in staging buffer esbuf.  A step's fragments are requested a step ahead.
+      auto block_products = [&](const unsigned char* hbuf, auto sub_c, auto hf_c, v16f& am, v16f& ar, auto nw_c, const Weave& w,
+                                auto epi_c, const v16f& em, const v16f& er, const float4& ecp, int esbuf) __attribute__((always_inline)) {
+        constexpr int SUB = decltype(sub_c)::value, hf = decltype(hf_c)::value, NW = decltype(nw_c)::value;
+        constexpr bool EPI = decltype(epi_c)::value;
+        const _Float16* row = reinterpret_cast<const _Float16*>(hbuf + (32 * SUB + j) * HLD) + 8 * hh;
+        float hv[4], cv[4];
+        v8h bt = *reinterpret_cast<const v8h*>(row), br = *reinterpret_cast<const v8h*>(row + PH);
+        float2 sb = make_float2(0.f, 0.f);
+        if constexpr (EPI) sb = gtab[0];
+        static_for<16>([&](auto s_c) __attribute__((always_inline)) {
+          constexpr int sidx = decltype(s_c)::value;
+          constexpr int qq = 16 * hf + sidx;
+          constexpr bool first = hf == 0 && sidx == 0;
+          v8h nt = bt, nr = br;
+          float2 nsb = sb;
+          if constexpr (sidx + 1 < 16) {
+            nt = *reinterpret_cast<const v8h*>(row + 16 * (sidx + 1));
+            nr = *reinterpret_cast<const v8h*>(row + PH + 16 * (sidx + 1));
+            if constexpr (EPI) nsb = gtab[sidx + 1];
+          }
+          // top x top in one accumulator; top x rest and rest x top, both 2^-11 of a product, share the other
+          am = __builtin_amdgcn_mfma_f32_32x32x16_f16(whi[qq], bt, first ? zero16 : am, 0, 0, 0);
+          ar = __builtin_amdgcn_mfma_f32_32x32x16_f16(whi[qq], br, first ? zero16 : ar, 0, 0, 0);
+          ar = __builtin_amdgcn_mfma_f32_32x32x16_f16(wlo[qq], bt, ar, 0, 0, 0);
+          if constexpr (EPI) {
+            pair_piece(em, er, ecp, hv, cv, sb, s_c);
+            // the piece's results are pinned to this step: left alone, the compiler moves every piece behind the last
+            // step, next to the only place that reads them
+            if constexpr ((sidx & 3) == 0) asm volatile("" : "+v"(eg_i));
+            if constexpr ((sidx & 3) == 1) asm volatile("" : "+v"(eg_f));
+            if constexpr ((sidx & 3) == 2) asm volatile("" : "+v"(eg_o));
+            if constexpr ((sidx & 3) == 3) asm volatile("" : "+v"(hv[sidx >> 2]), "+v"(cv[sidx >> 2]));
+          }
+          // the order within the step: next step's fragments (and the piece's table entry) first, then the MFMAs
+          // with the piece's vector instructions between them
+          __builtin_amdgcn_sched_group_barrier(0x100, EPI ? 3 : 2, 0);
+          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+          if constexpr (EPI) __builtin_amdgcn_sched_group_barrier(0x002, 10, 0);
+          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+          if constexpr (EPI) __builtin_amdgcn_sched_group_barrier(0x002, 10, 0);
+          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+          if constexpr (NW == 16) {
+            if (sidx < 8 ? w.lo.on : w.hi.on) copy_row(sidx < 8 ? w.lo : w.hi, IC<(sidx & 7)>{});
+          } else if constexpr (NW == 8 && (sidx & 1) == 0) {
+            if (w.lo.on) copy_row(w.lo, IC<(sidx >> 1)>{});
+          }
+          bt = nt; br = nr; sb = nsb;
+        });
+        if constexpr (EPI) stage_results(hv, cv, esbuf);
+      };
+      const float4 zero4 = make_float4(0.f, 0.f, 0.f, 0.f);
+      v16f am0, ar0, am1, ar1;
+
+      // item 0 is a first step: no h columns
+      Pair cur = pair_at(0, 0), prev = cur;
+      alive = wait_below(cur);
+      if (alive) {
+        copy_ratios(cur);
+        if (cur.on0) copy_block(x_rows(0), cur.rb0, xa_lds, 0);
+        if (cur.on1) copy_block(x_rows(0), cur.rb1, xa_lds, 1);
+      }
+      float4 cp0 = zero4, cp1 = zero4;
+      __builtin_amdgcn_s_waitcnt(0);
+      __syncthreads();
+      bool b_pending = false;    // block b of item p-1 waits for its activations (they run under Xa of item p)
+      bool a_stored = false, b_stored = false;   // stores of item p-1's blocks are on their way, not yet published
+      for (int p = 0; p < n_pairs; ++p) {
+        if (tracing) a.trace[TS * p + 0] = wall_clock64();
+        const bool more = p + 1 < n_pairs;
+        const Pair nxt = more ? pair_after(cur) : cur;
+        const bool has_prev = cur.t >= d;
+        const bool on0 = alive && cur.on0, on1 = alive && cur.on1;
+        float ratio0 = 1.0f, ratio1 = 1.0f;
+        if (x_rescaled) {
+          const float* rr = reinterpret_cast<const float*>(reinterpret_cast<const unsigned char*>(tile) + kRatioOffset);
+          ratio0 = rr[j];
+          ratio1 = rr[64 + j];
+        }
+        const int fo = look(l, cur.t - d, cur);       // this layer's flags for the item's h columns
+        const int fb = look(l - 1, nxt.t, nxt);       // the layer below's for the next item's x columns
+        // ---- Xa with Eb of the item before; one block only: its h columns are woven here
+        const char* hsrc = h_rows(has_prev ? cur.t : d);
+        Weave wh{rows_of(hsrc, cur.rb0, hb_lds, 0, false), rows_of(hsrc, cur.rb1, hb_lds, 1, false)};
+        if (on0 && !on1 && has_prev) {
+          if (!all_set(fo)) alive = wait_own(cur);
+          asm volatile("" ::: "memory");
+          wh.lo.on = alive;
+        }
+        if (on0) {
+          if (b_pending) block_products(xa, IC<0>{}, IC<0>{}, am0, ar0, IC<8>{}, wh, std::true_type{}, am1, ar1, cp1, 1);
+          else block_products(xa, IC<0>{}, IC<0>{}, am0, ar0, IC<8>{}, wh, std::false_type{}, am1, ar1, cp1, 1);
+          if (x_rescaled) {
+#pragma unroll
+            for (int r = 0; r < 16; ++r) { am0[r] *= ratio0; ar0[r] *= ratio0; }
+          }
+        } else if (b_pending) {
+          activations_alone(am1, ar1, cp1, 1);
+        }
+        b_pending = false;
+        if (tracing) a.trace[TS * p + 1] = wall_clock64();
+        // ---- Xb | h columns of both blocks -> HB
+        if (on1) {
+          if (has_prev) {
+            if (!all_set(fo)) alive = wait_own(cur);
+            asm volatile("" ::: "memory");
+            wh.lo.on = wh.hi.on = alive;
+          }
+          block_products(xa, IC<1>{}, IC<0>{}, am1, ar1, IC<16>{}, wh, std::false_type{}, am1, ar1, cp1, 1);
+          if (x_rescaled) {
+#pragma unroll
+            for (int r = 0; r < 16; ++r) { am1[r] *= ratio1; ar1[r] *= ratio1; }
+          }
+        }
+        if (tracing) a.trace[TS * p + 2] = wall_clock64();
+        wait_all();
+        if (a_stored) publish_block(prev.t, prev.rb0, prev.on0);
+        a_stored = false;
+        barrier();   // 1: HB and staging 1 complete, XA free
+        if (tracing) a.trace[TS * p + 3] = wall_clock64();
+        if (p > 0) { store_block(prev.t, prev.rb1, prev.on1, 1); b_stored = true; }
+        cp1 = load_cprev_of(cur.t, cur.rb1, cur.on1);
+        // ---- Ha, Hb with Ea | x columns of the next item -> XA
+        const bool x_ok = more && alive && (l == 0 || all_set(fb));
+        asm volatile("" ::: "memory");
+        if (x_ok) copy_ratios(nxt);
+        const char* xsrc = x_rows(nxt.t);
+        Weave wx{rows_of(xsrc, nxt.rb0, xa_lds, 0, x_ok && nxt.on0), rows_of(xsrc, nxt.rb1, xa_lds, 1, x_ok && nxt.on1)};
+        if (on0 && has_prev) {
+          block_products(hb, IC<0>{}, IC<1>{}, am0, ar0, IC<8>{}, wx, std::false_type{}, am0, ar0, cp0, 0);
+          wx.lo = wx.hi;
+          if (tracing) a.trace[TS * p + 4] = wall_clock64();
+          if (on1) block_products(hb, IC<1>{}, IC<1>{}, am1, ar1, IC<8>{}, wx, std::true_type{}, am0, ar0, cp0, 0);
+          else {
+            if (wx.lo.on) copy_block(xsrc, nxt.rb1, xa_lds, 1);
+            activations_alone(am0, ar0, cp0, 0);
+          }
+        } else {
+          if (x_ok && nxt.on0) copy_block(xsrc, nxt.rb0, xa_lds, 0);
+          if (x_ok && nxt.on1) copy_block(xsrc, nxt.rb1, xa_lds, 1);
+          if (tracing) a.trace[TS * p + 4] = wall_clock64();
+          if (on0) activations_alone(am0, ar0, cp0, 0);
+        }
+        b_pending = on1;
+        if (tracing) a.trace[TS * p + 5] = wall_clock64();
+        if (more && !x_ok) {   // the layer below was not ready at barrier 1
+          if (alive) alive = wait_below(nxt);
+          if (alive) {
+            copy_ratios(nxt);
+            if (nxt.on0) copy_block(xsrc, nxt.rb0, xa_lds, 0);
+            if (nxt.on1) copy_block(xsrc, nxt.rb1, xa_lds, 1);
+          }
+        }
+        wait_all();
+        if (b_stored) publish_block(prev.t, prev.rb1, prev.on1);
+        b_stored = false;
+        barrier();   // 2: XA and staging 0 complete, HB free
+        if (tracing) a.trace[TS * p + 6] = wall_clock64();
+        store_block(cur.t, cur.rb0, cur.on0, 0);
+        a_stored = true;
+        if (more) cp0 = load_cprev_of(nxt.t, nxt.rb0, nxt.on0);
+        if (tracing) a.trace[TS * p + 7] = wall_clock64();
+        prev = cur;
+        cur = nxt;
+      }
+      // the last item's second block
+      if (b_pending) activations_alone(am1, ar1, cp1, 1);
+      wait_all();
+      if (a_stored) publish_block(prev.t, prev.rb0, prev.on0);
+      barrier();
+      store_block(prev.t, prev.rb1, prev.on1, 1);
+      wait_all();
+      publish_block(prev.t, prev.rb1, prev.on1);
+      return;
+    }
   }
 
   // ---- pipelined schedule.  Per item n:
@@ -904,7 +1225,11 @@ __global__ void fill_zero_kernel(int* p, size_t n) {
 
 // Split mode, before the persistent kernel: every input row as its two fp16
 // planes, with the row's own power-of-two scale.  One wave per row of 256.
-__global__ __launch_bounds__(256) void lstm_split_rows_kernel(const float* xs, _Float16* xsp, float* xratio, int rows) {
+// Input rows -> their two fp16 planes and the factor that takes their products to h's scale.  A row whose largest
+// magnitude is zero or in [2^-24, 2^4 (1 - 2^-11)] takes the common scale 2^kSplitCommon: its largest element stays
+// finite in fp16 and the planes keep 22 bits of it, as with a scale of the row's own.  Any other row gets a scale of
+// its own, and *own_scales says that there is one.
+__global__ __launch_bounds__(256) void lstm_split_rows_kernel(const float* xs, _Float16* xsp, float* xratio, int* own_scales, int rows) {
   const int lane = threadIdx.x & 63;
   const int row = blockIdx.x * 4 + (threadIdx.x >> 6);
   if (row >= rows) return;
@@ -912,7 +1237,10 @@ __global__ __launch_bounds__(256) void lstm_split_rows_kernel(const float* xs, _
   float m = fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w)));
 #pragma unroll
   for (int o = 32; o > 0; o >>= 1) m = fmaxf(m, __shfl_xor(m, o));
-  const int eb = min(max((int)((__float_as_uint(m) >> 23) & 0xff), 15), 254);
+  int eb = min(max((int)((__float_as_uint(m) >> 23) & 0xff), 15), 254);
+  const bool common = m == 0.0f || (m >= 0x1p-24f && m <= 16.0f * (1.0f - 0x1p-11f));
+  if (common) eb = 127 + kSplitTop - kSplitCommon;   // the exponent whose own scale is the common one
+  else if (lane == 0) __hip_atomic_store(own_scales, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   const float scale = __uint_as_float((unsigned)(127 + kSplitTop + 127 - eb) << 23);
   const float vs[4] = {v.x * scale, v.y * scale, v.z * scale, v.w * scale};
   v4h top, rest;
@@ -1106,6 +1434,9 @@ static int run_persistent(int mode, const void* xs, const void* WU, const float*
   }
   const int grid = a.groups;
   a.xcd_remap = (grid % 8 == 0) ? 1 : 0;
+  // FTK_LSTM_PAIRS=0: pipelined layers of the split-product kernel walk single row blocks (the older schedule)
+  static const bool pairs_off = getenv("FTK_LSTM_PAIRS") && atoi(getenv("FTK_LSTM_PAIRS")) == 0;
+  a.paired = (split && !pairs_off && B % 8 == 0) ? 1 : 0;
 
   // flags and status block start from zero; a later launch of a stack that runs as several keeps the error word
   // of the earlier ones (it then drains at its first long wait, and the call reports the time-out)
@@ -1117,7 +1448,7 @@ static int run_persistent(int mode, const void* xs, const void* WU, const float*
 
   if (split) {
     const int rows = T * B;
-    hipLaunchKernelGGL(lstm_split_rows_kernel, dim3((rows + 3) / 4), dim3(256), 0, s, a.xs, xsp, xratio, rows);
+    hipLaunchKernelGGL(lstm_split_rows_kernel, dim3((rows + 3) / 4), dim3(256), 0, s, a.xs, xsp, xratio, a.status + 2, rows);
     rc = check_launch("lstm_split_rows_kernel");
     if (rc) return rc;
   }
