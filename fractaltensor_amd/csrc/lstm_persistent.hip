@@ -179,6 +179,18 @@ __device__ __forceinline__ void lds_dma16(const void* gbase, unsigned byte_off, 
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2 offset:%3"
                  :: "s"(lds_addr), "v"(byte_off), "s"(gbase), "n"(OFF) : "memory", "m0");
 }
+// The same with the LDS address formed in the instruction stream, base + DELTA: a caller with many destinations at
+// fixed distances keeps one scalar register instead of one per destination (sixteen of them per phase would be
+// spilled into a vector register's lanes and read back one by one in front of every copy).
+template <int OFF, bool COHERENT, int DELTA>
+__device__ __forceinline__ void lds_dma16_at(const void* gbase, unsigned byte_off, unsigned lds_base) {
+  if constexpr (COHERENT)
+    asm volatile("s_add_u32 m0, %0, %4\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2 offset:%3 sc1"
+                 :: "s"(lds_base), "v"(byte_off), "s"(gbase), "n"(OFF), "n"(DELTA - OFF) : "memory", "m0", "scc");
+  else
+    asm volatile("s_add_u32 m0, %0, %4\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2 offset:%3"
+                 :: "s"(lds_base), "v"(byte_off), "s"(gbase), "n"(OFF), "n"(DELTA - OFF) : "memory", "m0", "scc");
+}
 // 4 bytes per lane, through the caches: used to touch cache lines ahead of time.
 __device__ __forceinline__ void lds_dma4(const void* gbase, unsigned byte_off, unsigned lds_addr) {
   asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, %2"
@@ -308,6 +320,27 @@ void lstm_persistent_kernel(PersistArgs a) {
       }
 #pragma unroll
     for (int r = 0; r < 16; ++r) ginv[r] = __shfl(winv, (r & 3) + 8 * (r >> 2) + 4 * hh) * (1.0f / kSplitAct);
+    // Seven eighths of the fragments move to the accumulation registers, by hand.  The matrix instructions read
+    // their operands from either register file; the vector ALU, which everything else here goes through, only from
+    // the architectural one, whose 256 registers the weights alone would fill.  Left to itself the compiler parks
+    // fragments in accumulation registers too, but as spills: four moves back and a wait state in front of every
+    // MFMA that uses one, in loops where the issue slots beside an MFMA are what is scarce.
+    auto to_acc = [](v8h v) __attribute__((always_inline)) -> v8h {
+      typedef unsigned v4u __attribute__((ext_vector_type(4)));
+      const v4u u = __builtin_bit_cast(v4u, v);
+      unsigned a0, a1, a2, a3;
+      asm("v_accvgpr_write_b32 %0, %1" : "=a"(a0) : "v"(u[0]));
+      asm("v_accvgpr_write_b32 %0, %1" : "=a"(a1) : "v"(u[1]));
+      asm("v_accvgpr_write_b32 %0, %1" : "=a"(a2) : "v"(u[2]));
+      asm("v_accvgpr_write_b32 %0, %1" : "=a"(a3) : "v"(u[3]));
+      const v4u r = {a0, a1, a2, a3};
+      return __builtin_bit_cast(v8h, r);
+    };
+#pragma unroll
+    for (int s = 0; s < PK / 16; ++s) {
+      whi[s] = to_acc(whi[s]);
+      if (s % 4 != 3) wlo[s] = to_acc(wlo[s]);
+    }
   }
   const int u0 = 32 * pc + 8 * wave + 4 * hh;  // first of this lane's 4 units
   // sigmoid(v) = 1 / (1 + 2^(-v log2 e)): the -log2 e of the gates i, f, o (accumulator register r holds gate r / 4
@@ -850,7 +883,7 @@ void lstm_persistent_kernel(PersistArgs a) {
       };
       auto copy_row = [&](const Rows& x, auto r_c) __attribute__((always_inline)) {
         constexpr int r = decltype(r_c)::value;
-        lds_dma16<(r & 3) * 1024, kCoherentTiles>(x.g + (r >> 2) * 4096, lane16, x.lds + (unsigned)(r * HLD));
+        lds_dma16_at<(r & 3) * 1024, kCoherentTiles, r * HLD>(x.g + (r >> 2) * 4096, lane16, x.lds);
       };
       auto copy_block = [&](const char* src, int rb, unsigned half_lds, int sub) __attribute__((always_inline)) {
         const Rows x = rows_of(src, rb, half_lds, sub, true);
