@@ -852,17 +852,44 @@ void lstm_persistent_kernel(PersistArgs a) {
       const unsigned xa_lds = tile_lds, hb_lds = tile_lds + 64u * HLD;
       // The per-register factors and biases of the gate sums move to a table in LDS, one set per wave and lane half,
       // in the order the activations take them: with four accumulators per lane the registers are needed elsewhere.
+      // (a unit's four entries: gate i, the candidate, gates f and o -- the first part of a unit's activations takes
+      // the first two with one read)
       float2* const gtab = reinterpret_cast<float2*>(reinterpret_cast<unsigned char*>(tile) + kGateTableOffset) + 16 * (2 * wave + hh);
       if (j == 0) {
 #pragma unroll
-        for (int m = 0; m < 16; ++m) gtab[m] = make_float2(esc[4 * (m & 3) + (m >> 2)], ebias[4 * (m & 3) + (m >> 2)]);
+        for (int m = 0; m < 16; ++m) {
+          constexpr int gate_of[4] = {0, 3, 1, 2};
+          const int reg = 4 * gate_of[m & 3] + (m >> 2);
+          gtab[m] = make_float2(esc[reg], ebias[reg]);
+        }
       }
+      // what part m of the activations needs from the table
+      auto gate_entry = [&](auto mc) __attribute__((always_inline)) -> float4 {
+        constexpr int m = decltype(mc)::value;
+        if constexpr ((m & 3) == 0) return *reinterpret_cast<const float4*>(gtab + m);
+        else if constexpr ((m & 3) == 3) return make_float4(0.f, 0.f, 0.f, 0.f);
+        else { const float2 e = gtab[m + 1]; return make_float4(e.x, e.y, 0.f, 0.f); }
+      };
+      // Every per-layer array here has 1 KB per batch row (256 fp32, or the two fp16 planes of 256), and a flag is
+      // kFlagStride bytes.  With one wave per SIMD the scalar arithmetic of an item has nothing to hide behind, so
+      // an item's addresses are not multiplied out of (layer, step, row) each time: an item carries the byte offset
+      // of its time step in those arrays (tO) and in a layer's flags (tF), the next item's follow by addition, and
+      // the layer's bases are formed once.  (tF fits 32 bits: a layer's flags are 1/512 the size of its h.)
+      const size_t stepO = (size_t)B * 1024, dO = (size_t)d * stepO;
+      const unsigned stepF = (unsigned)a.nrb * kFlagStride, dF = (unsigned)d * stepF;
+      const char* const xbase = reinterpret_cast<const char*>((l == 0) ? xin : hin + (size_t)(l - 1) * T * cell);
+      const char* const hbase = reinterpret_cast<const char*>(hin + (size_t)l * T * cell);
+      char* const pbase = reinterpret_cast<char*>(a.hsp) + (size_t)l * T * stepO;
+      char* const cbase = reinterpret_cast<char*>(a.csss + (size_t)l * T * cell);
+      char* const obase = reinterpret_cast<char*>(a.hsss + (size_t)l * T * cell);
+      unsigned char* const fown = flag_of(l, 0, 0);
+      unsigned char* const fbelow = flag_of(max(l - 1, 0), 0, 0);
       // an item: time step t, row blocks rb0 and rb1 = rb0 + pr; on0 / on1: the block exists and is live at t.  Rows
       // are sorted by length, so a live second block has a live first one.
-      struct Pair { int t, i, rb0, rb1; bool on0, on1; };
-      auto pair_at = [&](int t, int i) __attribute__((always_inline)) -> Pair {
+      struct Pair { int t, i, rb0, rb1; size_t tO; unsigned tF; int on0, on1; };
+      auto pair_at = [&](int t, int i, size_t tO, unsigned tF) __attribute__((always_inline)) -> Pair {
         Pair x;
-        x.t = t; x.i = i;
+        x.t = t; x.i = i; x.tO = tO; x.tF = tF;
         x.rb0 = prs + pr * (2 * i);
         x.rb1 = x.rb0 + pr;
         x.on0 = !a.ragged || t < a.steps_of[x.rb0];
@@ -870,16 +897,14 @@ void lstm_persistent_kernel(PersistArgs a) {
         return x;
       };
       auto pair_after = [&](const Pair& x) __attribute__((always_inline)) -> Pair {
-        return x.i + 1 < ppt ? pair_at(x.t, x.i + 1) : pair_at(x.t + 1, 0);
+        return x.i + 1 < ppt ? pair_at(x.t, x.i + 1, x.tO, x.tF) : pair_at(x.t + 1, 0, x.tO + stepO, x.tF + stepF);
       };
-      auto x_rows = [&](int t) { return reinterpret_cast<const char*>((l == 0) ? xin + (size_t)t * cell : hin + ((size_t)(l - 1) * T + t) * cell); };
-      auto h_rows = [&](int t) { return reinterpret_cast<const char*>(hin + ((size_t)l * T + (t - d)) * cell); };
       // A wave's 8 rows of a row block: where the first of them lies in global memory (the rows are 1 KB apart) and
       // where it goes in LDS.  The batch is a multiple of 8 rows here, so the 8 rows are all inside it or all beyond
       // its end; those beyond are copied from the batch's last 8 rows instead (nobody stores what comes of them).
       struct Rows { bool on; const char* g; unsigned lds; };
       auto rows_of = [&](const char* src, int rb, unsigned half_lds, int sub, bool on) __attribute__((always_inline)) -> Rows {
-        return Rows{on, src + (size_t)min(rb * 32 + 8 * wave_u, B - 8) * 1024, half_lds + (unsigned)((32 * sub + 8 * wave_u) * HLD)};
+        return Rows{on, src + ((unsigned)min(rb * 32 + 8 * wave_u, B - 8) << 10), half_lds + (unsigned)((32 * sub + 8 * wave_u) * HLD)};
       };
       auto copy_row = [&](const Rows& x, auto r_c) __attribute__((always_inline)) {
         constexpr int r = decltype(r_c)::value;
@@ -899,10 +924,10 @@ void lstm_persistent_kernel(PersistArgs a) {
       // and its address always valid, so that nothing makes the compiler wait for it where it is issued: the wave
       // asks, works, and reads the answer later.  Callers ignore the answer where there is no such dependency.
       static_assert(FLAG_TARGET == 32, "one half of the wave per row block");
-      auto look = [&](int ll, int t, const Pair& x) __attribute__((always_inline)) -> int {
-        const unsigned char* f = flag_of(max(ll, 0), max(t, 0), x.rb0) + (lane & 31);
-        if (lane >= 32 && x.on1) f += (x.rb1 - x.rb0) * kFlagStride;
-        return __hip_atomic_load(f, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      auto look = [&](const unsigned char* layer_flags, unsigned tF, const Pair& x) __attribute__((always_inline)) -> int {
+        unsigned off = tF + (unsigned)x.rb0 * kFlagStride + (lane & 31);
+        if (lane >= 32 && x.on1) off += (unsigned)(x.rb1 - x.rb0) * kFlagStride;
+        return __hip_atomic_load(layer_flags + off, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       };
       auto wait_pair = [&](const Pair& x, int ll, int t) __attribute__((always_inline)) -> bool {
         bool ok = true;
@@ -914,33 +939,71 @@ void lstm_persistent_kernel(PersistArgs a) {
       auto wait_below = [&](const Pair& x) __attribute__((always_inline)) -> bool { return l == 0 || wait_pair(x, l - 1, x.t); };
       auto wait_own = [&](const Pair& x) __attribute__((always_inline)) -> bool { return x.t < d || wait_pair(x, l, x.t - d); };
       // a wave publishes its part of one row block of an item; its stores have been waited for
-      auto publish_block = [&](int t, int rb, bool on) __attribute__((always_inline)) {
+      auto publish_block = [&](unsigned tF, int rb, bool on) __attribute__((always_inline)) {
         if (lane == 0 && alive && on)
-          __hip_atomic_store(flag_of(l, t, rb) + 4 * pc + wave, (unsigned char)1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          __hip_atomic_store(fown + (tF + (unsigned)rb * kFlagStride + 4 * pc + wave), (unsigned char)1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      };
+      // store_block / load_cprev_of on the offsets an item carries
+      auto store_rows = [&](size_t tO, int rb, bool is_live, int sbuf) __attribute__((always_inline)) {
+        const int rl = 8 * wave + (lane >> 3), cc = lane & 7;
+        const int rg = rb * 32 + rl;
+        if (alive && rg < B && is_live) {
+          const unsigned char* sb = stage + sbuf * kStageBytes;
+          const size_t at = tO + (((unsigned)rg << 10) + 16u * (unsigned)(8 * pc + cc));
+          *reinterpret_cast<float4*>(cbase + at) = *reinterpret_cast<const float4*>(sb + kStageC + rl * kStageRow32 + 16 * cc);
+          *reinterpret_cast<float4*>(obase + at) = *reinterpret_cast<const float4*>(sb + kStageH + rl * kStageRow32 + 16 * cc);
+          _Float16* pdst = reinterpret_cast<_Float16*>(pbase + tO + (((unsigned)rg << 10) + 8u * (unsigned)(8 * pc + cc)));
+          coherent_store8h(pdst, *reinterpret_cast<const v4h*>(sb + kStageTop + rl * kStageRow16 + 8 * cc));
+          coherent_store8h(pdst + PH, *reinterpret_cast<const v4h*>(sb + kStageRest + rl * kStageRow16 + 8 * cc));
+        }
+      };
+      auto cprev_rows = [&](size_t tO_prev, int rb, bool has) __attribute__((always_inline)) -> float4 {
+        float4 cp = make_float4(0.f, 0.f, 0.f, 0.f);
+        if (alive && has)
+          cp = *reinterpret_cast<const float4*>(cbase + tO_prev + (((unsigned)min(rb * 32 + j, B - 1) << 10) + 4u * (unsigned)u0));
+        return cp;
       };
       auto wait_all = [&]() __attribute__((always_inline)) {
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
         __builtin_amdgcn_s_waitcnt(0);
       };
-      // piece m (0..15) of a block's activations, straight from the two accumulators: gate m & 3 of unit m >> 2
-      auto pair_piece = [&](const v16f& em, const v16f& er, const float4& cp, float (&hv)[4], float (&cv)[4], const float2 sb, auto mc) __attribute__((always_inline)) {
+      // piece m (0..15) of a block's activations, straight from the two accumulators: unit m >> 2, part m & 3.  With
+      // one wave per SIMD a chain of dependent vector instructions runs at its latency, not at the issue rate, so a
+      // piece carries two chains that do not depend on each other: parts 0..2 hold a sigmoid (gates i, f, o) beside a
+      // third of the candidate's tanh, part 3 the tanh of the new c, whose exponential and polynomial are independent.
+      float tc_v = 0.f, tc_e = 0.f, tc_x2 = 0.f, tc_p = 0.f, tc_r = 0.f;   // the candidate's tanh between the parts
+      auto pair_piece = [&](const v16f& em, const v16f& er, const float4& cp, float (&hv)[4], float (&cv)[4], const float4 sb, auto mc) __attribute__((always_inline)) {
         constexpr int m = decltype(mc)::value;
         constexpr int r = m >> 2, g = m & 3, reg = 4 * g + r;
         const float cpv[4] = {cp.x, cp.y, cp.z, cp.w};
         auto inv1p = [](float e) { return __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(e)); };
-        const float v = sb.x * (em[reg] + (1.0f / kSplitRest) * er[reg]) + sb.y;
-        if constexpr (g == 0) eg_i = inv1p(v);
-        if constexpr (g == 1) eg_f = inv1p(v);
-        if constexpr (g == 2) eg_o = inv1p(v);
-        if constexpr (g == 3) {
-          const float cand = tanh_f(v);
-          cv[r] = eg_f * cpv[r] + eg_i * cand;
+        if constexpr (g < 3) {
+          const float v = sb.x * (em[reg] + (1.0f / kSplitRest) * er[reg]) + sb.y;
+          if constexpr (g == 0) {
+            eg_i = inv1p(v);
+            tc_v = sb.z * (em[12 + r] + (1.0f / kSplitRest) * er[12 + r]) + sb.w;
+            tc_e = fast_exp(2.0f * tc_v);
+            tc_x2 = tc_v * tc_v;
+          }
+          if constexpr (g == 1) {
+            eg_f = inv1p(v);
+            tc_p = -0.33333333333f + tc_x2 * (0.13333333333f + tc_x2 * (-0.05396825397f + tc_x2 * 0.02186948854f));
+            tc_r = __builtin_amdgcn_rcpf(1.0f + tc_e);
+          }
+          if constexpr (g == 2) {
+            eg_o = inv1p(v);
+            const float big = 1.0f - 2.0f * tc_r;
+            const float small = tc_v * (1.0f + tc_x2 * tc_p);
+            const float cand = fabsf(tc_v) < 0.25f ? small : big;   // tanh_f, in three parts
+            cv[r] = eg_f * cpv[r] + eg_i * cand;
+          }
+        } else {
           hv[r] = eg_o * tanh_f(cv[r]);
         }
       };
       auto activations_alone = [&](const v16f& em, const v16f& er, const float4& cp, int sbuf) __attribute__((always_inline)) {
         float hv[4], cv[4];
-        static_for<16>([&](auto mc) __attribute__((always_inline)) { pair_piece(em, er, cp, hv, cv, gtab[decltype(mc)::value], mc); });
+        static_for<16>([&](auto mc) __attribute__((always_inline)) { pair_piece(em, er, cp, hv, cv, gate_entry(mc), mc); });
         stage_results(hv, cv, sbuf);
       };
       // Copies dealt out over a phase's 16 steps.  NW = 16: one per step, rows 0..7 of group lo, then of group hi;
@@ -950,24 +1013,24 @@ void lstm_persistent_kernel(PersistArgs a) {
       // am / ar.  EPI: the activations of ANOTHER block, from em / er, cp, are dealt out over the steps as well and
       // end in staging buffer esbuf.  A step's fragments are requested a step ahead.
       auto block_products = [&](const unsigned char* hbuf, auto sub_c, auto hf_c, v16f& am, v16f& ar, auto nw_c, const Weave& w,
-                                auto epi_c, const v16f& em, const v16f& er, const float4& ecp, int esbuf) __attribute__((always_inline)) {
+                                auto epi_c, const v16f& em, const v16f& er, const float4& ecp, int esbuf, auto&& late) __attribute__((always_inline)) {
         constexpr int SUB = decltype(sub_c)::value, hf = decltype(hf_c)::value, NW = decltype(nw_c)::value;
         constexpr bool EPI = decltype(epi_c)::value;
         const _Float16* row = reinterpret_cast<const _Float16*>(hbuf + (32 * SUB + j) * HLD) + 8 * hh;
         float hv[4], cv[4];
         v8h bt = *reinterpret_cast<const v8h*>(row), br = *reinterpret_cast<const v8h*>(row + PH);
-        float2 sb = make_float2(0.f, 0.f);
-        if constexpr (EPI) sb = gtab[0];
+        float4 sb = make_float4(0.f, 0.f, 0.f, 0.f);
+        if constexpr (EPI) sb = gate_entry(IC<0>{});
         static_for<16>([&](auto s_c) __attribute__((always_inline)) {
           constexpr int sidx = decltype(s_c)::value;
           constexpr int qq = 16 * hf + sidx;
           constexpr bool first = hf == 0 && sidx == 0;
           v8h nt = bt, nr = br;
-          float2 nsb = sb;
+          float4 nsb = sb;
           if constexpr (sidx + 1 < 16) {
             nt = *reinterpret_cast<const v8h*>(row + 16 * (sidx + 1));
             nr = *reinterpret_cast<const v8h*>(row + PH + 16 * (sidx + 1));
-            if constexpr (EPI) nsb = gtab[sidx + 1];
+            if constexpr (EPI) nsb = gate_entry(IC<sidx + 1>{});
           }
           // top x top in one accumulator; top x rest and rest x top, both 2^-11 of a product, share the other
           am = __builtin_amdgcn_mfma_f32_32x32x16_f16(whi[qq], bt, first ? zero16 : am, 0, 0, 0);
@@ -977,10 +1040,10 @@ void lstm_persistent_kernel(PersistArgs a) {
             pair_piece(em, er, ecp, hv, cv, sb, s_c);
             // the piece's results are pinned to this step: left alone, the compiler moves every piece behind the last
             // step, next to the only place that reads them
-            if constexpr ((sidx & 3) == 0) asm volatile("" : "+v"(eg_i));
-            if constexpr ((sidx & 3) == 1) asm volatile("" : "+v"(eg_f));
-            if constexpr ((sidx & 3) == 2) asm volatile("" : "+v"(eg_o));
-            if constexpr ((sidx & 3) == 3) asm volatile("" : "+v"(hv[sidx >> 2]), "+v"(cv[sidx >> 2]));
+            if constexpr ((sidx & 3) == 0) asm volatile("" : "+v"(eg_i), "+v"(tc_e), "+v"(tc_x2));
+            if constexpr ((sidx & 3) == 1) asm volatile("" : "+v"(eg_f), "+v"(tc_p), "+v"(tc_r));
+            if constexpr ((sidx & 3) == 2) asm volatile("" : "+v"(eg_o), "+v"(cv[sidx >> 2]));
+            if constexpr ((sidx & 3) == 3) asm volatile("" : "+v"(hv[sidx >> 2]));
           }
           // the order within the step: next step's fragments (and the piece's table entry) first, then the MFMAs
           // with the piece's vector instructions between them
@@ -990,6 +1053,7 @@ void lstm_persistent_kernel(PersistArgs a) {
           __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
           if constexpr (EPI) __builtin_amdgcn_sched_group_barrier(0x002, 10, 0);
           __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+          if constexpr (sidx == 13) late();   // something the caller wants issued near the end of the phase
           if constexpr (NW == 16) {
             if (sidx < 8 ? w.lo.on : w.hi.on) copy_row(sidx < 8 ? w.lo : w.hi, IC<(sidx & 7)>{});
           } else if constexpr (NW == 8 && (sidx & 1) == 0) {
@@ -1001,14 +1065,15 @@ void lstm_persistent_kernel(PersistArgs a) {
       };
       const float4 zero4 = make_float4(0.f, 0.f, 0.f, 0.f);
       v16f am0, ar0, am1, ar1;
+      auto nothing = []() {};
 
       // item 0 is a first step: no h columns
-      Pair cur = pair_at(0, 0), prev = cur;
+      Pair cur = pair_at(0, 0, 0, 0u), prev = cur;
       alive = wait_below(cur);
       if (alive) {
         copy_ratios(cur);
-        if (cur.on0) copy_block(x_rows(0), cur.rb0, xa_lds, 0);
-        if (cur.on1) copy_block(x_rows(0), cur.rb1, xa_lds, 1);
+        if (cur.on0) copy_block(xbase, cur.rb0, xa_lds, 0);
+        if (cur.on1) copy_block(xbase, cur.rb1, xa_lds, 1);
       }
       float4 cp0 = zero4, cp1 = zero4;
       __builtin_amdgcn_s_waitcnt(0);
@@ -1027,10 +1092,14 @@ void lstm_persistent_kernel(PersistArgs a) {
           ratio0 = rr[j];
           ratio1 = rr[64 + j];
         }
-        const int fo = look(l, cur.t - d, cur);       // this layer's flags for the item's h columns
-        const int fb = look(l - 1, nxt.t, nxt);       // the layer below's for the next item's x columns
+        const int fo = look(fown, has_prev ? cur.tF - dF : cur.tF, cur);   // this layer's flags for the item's h columns
+        // (the layer below's flags for the next item's x columns are looked at as late as their use allows: near the
+        // end of Xb, for the test behind barrier 1.  How far a layer runs behind the one below is set by how early it
+        // has to see those flags.)
+        int fb = 0;
+        auto look_below = [&]() __attribute__((always_inline)) { fb = look(fbelow, nxt.tF, nxt); };
         // ---- Xa with Eb of the item before; one block only: its h columns are woven here
-        const char* hsrc = h_rows(has_prev ? cur.t : d);
+        const char* hsrc = hbase + (has_prev ? cur.tO - dO : 0);
         Weave wh{rows_of(hsrc, cur.rb0, hb_lds, 0, false), rows_of(hsrc, cur.rb1, hb_lds, 1, false)};
         if (on0 && !on1 && has_prev) {
           if (!all_set(fo)) alive = wait_own(cur);
@@ -1038,8 +1107,8 @@ void lstm_persistent_kernel(PersistArgs a) {
           wh.lo.on = alive;
         }
         if (on0) {
-          if (b_pending) block_products(xa, IC<0>{}, IC<0>{}, am0, ar0, IC<8>{}, wh, std::true_type{}, am1, ar1, cp1, 1);
-          else block_products(xa, IC<0>{}, IC<0>{}, am0, ar0, IC<8>{}, wh, std::false_type{}, am1, ar1, cp1, 1);
+          if (b_pending) block_products(xa, IC<0>{}, IC<0>{}, am0, ar0, IC<8>{}, wh, std::true_type{}, am1, ar1, cp1, 1, nothing);
+          else block_products(xa, IC<0>{}, IC<0>{}, am0, ar0, IC<8>{}, wh, std::false_type{}, am1, ar1, cp1, 1, nothing);
           if (x_rescaled) {
 #pragma unroll
             for (int r = 0; r < 16; ++r) { am0[r] *= ratio0; ar0[r] *= ratio0; }
@@ -1056,31 +1125,33 @@ void lstm_persistent_kernel(PersistArgs a) {
             asm volatile("" ::: "memory");
             wh.lo.on = wh.hi.on = alive;
           }
-          block_products(xa, IC<1>{}, IC<0>{}, am1, ar1, IC<16>{}, wh, std::false_type{}, am1, ar1, cp1, 1);
+          block_products(xa, IC<1>{}, IC<0>{}, am1, ar1, IC<16>{}, wh, std::false_type{}, am1, ar1, cp1, 1, look_below);
           if (x_rescaled) {
 #pragma unroll
             for (int r = 0; r < 16; ++r) { am1[r] *= ratio1; ar1[r] *= ratio1; }
           }
+        } else {
+          look_below();
         }
         if (tracing) a.trace[TS * p + 2] = wall_clock64();
         wait_all();
-        if (a_stored) publish_block(prev.t, prev.rb0, prev.on0);
+        if (a_stored) publish_block(prev.tF, prev.rb0, prev.on0);
         a_stored = false;
         barrier();   // 1: HB and staging 1 complete, XA free
         if (tracing) a.trace[TS * p + 3] = wall_clock64();
-        if (p > 0) { store_block(prev.t, prev.rb1, prev.on1, 1); b_stored = true; }
-        cp1 = load_cprev_of(cur.t, cur.rb1, cur.on1);
+        if (p > 0) { store_rows(prev.tO, prev.rb1, prev.on1, 1); b_stored = true; }
+        cp1 = cprev_rows(cur.tO - dO, cur.rb1, cur.on1 && has_prev);
         // ---- Ha, Hb with Ea | x columns of the next item -> XA
         const bool x_ok = more && alive && (l == 0 || all_set(fb));
         asm volatile("" ::: "memory");
         if (x_ok) copy_ratios(nxt);
-        const char* xsrc = x_rows(nxt.t);
+        const char* xsrc = xbase + nxt.tO;
         Weave wx{rows_of(xsrc, nxt.rb0, xa_lds, 0, x_ok && nxt.on0), rows_of(xsrc, nxt.rb1, xa_lds, 1, x_ok && nxt.on1)};
         if (on0 && has_prev) {
-          block_products(hb, IC<0>{}, IC<1>{}, am0, ar0, IC<8>{}, wx, std::false_type{}, am0, ar0, cp0, 0);
+          block_products(hb, IC<0>{}, IC<1>{}, am0, ar0, IC<8>{}, wx, std::false_type{}, am0, ar0, cp0, 0, nothing);
           wx.lo = wx.hi;
           if (tracing) a.trace[TS * p + 4] = wall_clock64();
-          if (on1) block_products(hb, IC<1>{}, IC<1>{}, am1, ar1, IC<8>{}, wx, std::true_type{}, am0, ar0, cp0, 0);
+          if (on1) block_products(hb, IC<1>{}, IC<1>{}, am1, ar1, IC<8>{}, wx, std::true_type{}, am0, ar0, cp0, 0, nothing);
           else {
             if (wx.lo.on) copy_block(xsrc, nxt.rb1, xa_lds, 1);
             activations_alone(am0, ar0, cp0, 0);
@@ -1102,13 +1173,13 @@ void lstm_persistent_kernel(PersistArgs a) {
           }
         }
         wait_all();
-        if (b_stored) publish_block(prev.t, prev.rb1, prev.on1);
+        if (b_stored) publish_block(prev.tF, prev.rb1, prev.on1);
         b_stored = false;
         barrier();   // 2: XA and staging 0 complete, HB free
         if (tracing) a.trace[TS * p + 6] = wall_clock64();
-        store_block(cur.t, cur.rb0, cur.on0, 0);
+        store_rows(cur.tO, cur.rb0, cur.on0, 0);
         a_stored = true;
-        if (more) cp0 = load_cprev_of(nxt.t, nxt.rb0, nxt.on0);
+        if (more) cp0 = cprev_rows(nxt.tO - dO, nxt.rb0, nxt.on0 && nxt.t >= d);
         if (tracing) a.trace[TS * p + 7] = wall_clock64();
         prev = cur;
         cur = nxt;
@@ -1116,11 +1187,11 @@ void lstm_persistent_kernel(PersistArgs a) {
       // the last item's second block
       if (b_pending) activations_alone(am1, ar1, cp1, 1);
       wait_all();
-      if (a_stored) publish_block(prev.t, prev.rb0, prev.on0);
+      if (a_stored) publish_block(prev.tF, prev.rb0, prev.on0);
       barrier();
-      store_block(prev.t, prev.rb1, prev.on1, 1);
+      store_rows(prev.tO, prev.rb1, prev.on1, 1);
       wait_all();
-      publish_block(prev.t, prev.rb1, prev.on1);
+      publish_block(prev.tF, prev.rb1, prev.on1);
       return;
     }
   }
