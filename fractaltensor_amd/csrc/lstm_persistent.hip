@@ -828,7 +828,8 @@ void lstm_persistent_kernel(PersistArgs a) {
   // is not busy and does not hold the wave at issue.  Per item p, with X / H the halves of the products and E the
   // activations (which also split h into its planes and leave everything in a staging area):
   //   Xa(p) with Eb(p-1) -> staging 1    | the own layer's flags for item p are on their way
-  //   Xb(p)                              | this wave's rows of item p's h columns -> HB
+  //   Xb(p)                              | this wave's rows of item p's h columns -> HB; near its end, a look at the
+  //                                        layer below's flags for item p+1
   //   wait for everything outstanding (the stores of block a of item p-1 among it: that block is published)
   //   barrier 1: HB and staging 1 complete, XA free
   //   stores of block b of item p-1 from staging 1
