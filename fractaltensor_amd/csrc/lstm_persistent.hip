@@ -846,6 +846,10 @@ void lstm_persistent_kernel(PersistArgs a) {
   if constexpr (SPLIT) {
     const int ppt = (my_rbs + 1) / 2;            // pair items per time step
     if (a.paired && my_rbs >= 2 && (long long)d * ppt >= 2) {
+      // PLAIN: every item has both its blocks at every step (no ragged batch, an even number of row blocks): the
+      // tests for a block that is missing or past its rows' end then fold away, at the item's top most of all.
+      auto paired_schedule = [&](auto plain_c) __attribute__((always_inline)) {
+      constexpr bool PLAIN = decltype(plain_c)::value;
       constexpr int HLD = 1040;                  // bytes per row of a half buffer: 16 more than the row's two planes
       const int n_pairs = T * ppt;
       unsigned char* const xa = reinterpret_cast<unsigned char*>(tile);
@@ -893,8 +897,8 @@ void lstm_persistent_kernel(PersistArgs a) {
         x.t = t; x.i = i; x.tO = tO; x.tF = tF;
         x.rb0 = prs + pr * (2 * i);
         x.rb1 = x.rb0 + pr;
-        x.on0 = !a.ragged || t < a.steps_of[x.rb0];
-        x.on1 = 2 * i + 1 < my_rbs && (!a.ragged || t < a.steps_of[min(x.rb1, kMaxBlocks - 1)]);
+        x.on0 = PLAIN || !a.ragged || t < a.steps_of[x.rb0];
+        x.on1 = PLAIN || (2 * i + 1 < my_rbs && (!a.ragged || t < a.steps_of[min(x.rb1, kMaxBlocks - 1)]));
         return x;
       };
       auto pair_after = [&](const Pair& x) __attribute__((always_inline)) -> Pair {
@@ -1217,6 +1221,9 @@ void lstm_persistent_kernel(PersistArgs a) {
       store_rows(prev.tO, prev.rb1, prev.on1, 1);
       wait_all();
       publish_block(prev.tF, prev.rb1, prev.on1);
+      };
+      if (!a.ragged && my_rbs % 2 == 0) paired_schedule(std::true_type{});
+      else paired_schedule(std::false_type{});
       return;
     }
   }
