@@ -846,10 +846,15 @@ void lstm_persistent_kernel(PersistArgs a) {
   if constexpr (SPLIT) {
     const int ppt = (my_rbs + 1) / 2;            // pair items per time step
     if (a.paired && my_rbs >= 2 && (long long)d * ppt >= 2) {
-      // PLAIN: every item has both its blocks at every step (no ragged batch, an even number of row blocks): the
-      // tests for a block that is missing or past its rows' end then fold away, at the item's top most of all.
-      auto paired_schedule = [&](auto plain_c) __attribute__((always_inline)) {
+      // PLAIN: every item has both its blocks at every step (no ragged batch, an even number of row blocks), and no
+      // input row carries a scale of its own: the tests for a block that is missing or past its rows' end then fold
+      // away, at the item's top most of all, and so does the rescaling of the x products, whose mere presence behind a
+      // branch makes the compiler move both accumulators of a block out of and back into the accumulation registers
+      // at every item.  Only the
+      // workgroup that leaves time stamps carries the code for them.
+      auto paired_schedule = [&](auto plain_c, auto traced_c) __attribute__((always_inline)) {
       constexpr bool PLAIN = decltype(plain_c)::value;
+      constexpr bool TRACED = decltype(traced_c)::value;   // this workgroup leaves time stamps
       constexpr int HLD = 1040;                  // bytes per row of a half buffer: 16 more than the row's two planes
       const int n_pairs = T * ppt;
       unsigned char* const xa = reinterpret_cast<unsigned char*>(tile);
@@ -920,7 +925,7 @@ void lstm_persistent_kernel(PersistArgs a) {
         static_for<8>([&](auto r_c) __attribute__((always_inline)) { copy_row(x, r_c); });
       };
       auto copy_ratios = [&](const Pair& x) __attribute__((always_inline)) {   // first layer: the rows' scale ratios travel with their x columns
-        if (!x_rescaled || wave_u != 0) return;
+        if (PLAIN || !x_rescaled || wave_u != 0) return;
         if (x.on0) lds_dma4(a.xratio + (size_t)x.t * B, 4u * (unsigned)min(x.rb0 * 32 + (lane & 31), B - 1), tile_lds + (unsigned)kRatioOffset);
         if (x.on1) lds_dma4(a.xratio + (size_t)x.t * B, 4u * (unsigned)min(x.rb1 * 32 + (lane & 31), B - 1), tile_lds + (unsigned)kRatioOffset + 256u);
       };
@@ -1102,13 +1107,13 @@ void lstm_persistent_kernel(PersistArgs a) {
       bool b_pending = false;    // block b of item p-1 waits for its activations (they run under Xa of item p)
       bool a_stored = false, b_stored = false;   // stores of item p-1's blocks are on their way, not yet published
       for (int p = 0; p < n_pairs; ++p) {
-        if (tracing) a.trace[TS * p + 0] = wall_clock64();
+        if (TRACED && tracing) a.trace[TS * p + 0] = wall_clock64();
         const bool more = p + 1 < n_pairs;
         const Pair nxt = more ? pair_after(cur) : cur;
         const bool has_prev = cur.t >= d;
         const bool on0 = alive && cur.on0, on1 = alive && cur.on1;
         float ratio0 = 1.0f, ratio1 = 1.0f;
-        if (x_rescaled) {
+        if (!PLAIN && x_rescaled) {
           const float* rr = reinterpret_cast<const float*>(reinterpret_cast<const unsigned char*>(tile) + kRatioOffset);
           ratio0 = rr[j];
           ratio1 = rr[64 + j];
@@ -1130,7 +1135,7 @@ void lstm_persistent_kernel(PersistArgs a) {
         if (on0) {
           if (b_pending) block_products(xa, IC<0>{}, IC<0>{}, am0, ar0, IC<8>{}, wh, std::true_type{}, am1, ar1, cp1, 1, nothing);
           else block_products(xa, IC<0>{}, IC<0>{}, am0, ar0, IC<8>{}, wh, std::false_type{}, am1, ar1, cp1, 1, nothing);
-          if (x_rescaled) {
+          if (!PLAIN && x_rescaled) {
 #pragma unroll
             for (int r = 0; r < 16; ++r) { am0[r] *= ratio0; ar0[r] *= ratio0; }
           }
@@ -1138,7 +1143,7 @@ void lstm_persistent_kernel(PersistArgs a) {
           activations_alone(am1, ar1, cp1, 1);
         }
         b_pending = false;
-        if (tracing) a.trace[TS * p + 1] = wall_clock64();
+        if (TRACED && tracing) a.trace[TS * p + 1] = wall_clock64();
         // ---- Xb | h columns of both blocks -> HB
         if (on1) {
           if (has_prev) {
@@ -1147,19 +1152,19 @@ void lstm_persistent_kernel(PersistArgs a) {
             wh.lo.on = wh.hi.on = alive;
           }
           block_products(xa, IC<1>{}, IC<0>{}, am1, ar1, IC<16>{}, wh, std::false_type{}, am1, ar1, cp1, 1, look_below);
-          if (x_rescaled) {
+          if (!PLAIN && x_rescaled) {
 #pragma unroll
             for (int r = 0; r < 16; ++r) { am1[r] *= ratio1; ar1[r] *= ratio1; }
           }
         } else {
           look_below();
         }
-        if (tracing) a.trace[TS * p + 2] = wall_clock64();
+        if (TRACED && tracing) a.trace[TS * p + 2] = wall_clock64();
         wait_all();
         if (a_stored) publish_block(prev.tF, prev.rb0, prev.on0);
         a_stored = false;
         barrier();   // 1: HB and staging 1 complete, XA free
-        if (tracing) a.trace[TS * p + 3] = wall_clock64();
+        if (TRACED && tracing) a.trace[TS * p + 3] = wall_clock64();
         if (p > 0) { store_rows(prev.tO, prev.rb1, prev.on1, 1); b_stored = true; }
         const bool cp1_loads = alive && cur.on1 && has_prev;
         cp1 = cprev_rows(cur.tO - dO, cur.rb1, cur.on1 && has_prev);
@@ -1179,7 +1184,7 @@ void lstm_persistent_kernel(PersistArgs a) {
             b_stored = false;
           }
           wx.lo = wx.hi;
-          if (tracing) a.trace[TS * p + 4] = wall_clock64();
+          if (TRACED && tracing) a.trace[TS * p + 4] = wall_clock64();
           if (on1) block_products(hb, IC<1>{}, IC<1>{}, am1, ar1, IC<8>{}, wx, std::true_type{}, am0, ar0, cp0, 0, nothing);
           else {
             if (wx.lo.on) copy_block(xsrc, nxt.rb1, xa_lds, 1);
@@ -1188,11 +1193,11 @@ void lstm_persistent_kernel(PersistArgs a) {
         } else {
           if (x_ok && nxt.on0) copy_block(xsrc, nxt.rb0, xa_lds, 0);
           if (x_ok && nxt.on1) copy_block(xsrc, nxt.rb1, xa_lds, 1);
-          if (tracing) a.trace[TS * p + 4] = wall_clock64();
+          if (TRACED && tracing) a.trace[TS * p + 4] = wall_clock64();
           if (on0) activations_alone(am0, ar0, cp0, 0);
         }
         b_pending = on1;
-        if (tracing) a.trace[TS * p + 5] = wall_clock64();
+        if (TRACED && tracing) a.trace[TS * p + 5] = wall_clock64();
         if (more && !x_ok) {   // the layer below was not ready at barrier 1
           if (alive) alive = wait_below(nxt);
           if (alive) {
@@ -1205,11 +1210,11 @@ void lstm_persistent_kernel(PersistArgs a) {
         if (b_stored) publish_block(prev.tF, prev.rb1, prev.on1);
         b_stored = false;
         barrier();   // 2: XA and staging 0 complete, HB free
-        if (tracing) a.trace[TS * p + 6] = wall_clock64();
+        if (TRACED && tracing) a.trace[TS * p + 6] = wall_clock64();
         store_rows(cur.tO, cur.rb0, cur.on0, 0);
         a_stored = true;
         if (more) cp0 = cprev_rows(nxt.tO - dO, nxt.rb0, nxt.on0 && nxt.t >= d);
-        if (tracing) a.trace[TS * p + 7] = wall_clock64();
+        if (TRACED && tracing) a.trace[TS * p + 7] = wall_clock64();
         prev = cur;
         cur = nxt;
       }
@@ -1222,8 +1227,9 @@ void lstm_persistent_kernel(PersistArgs a) {
       wait_all();
       publish_block(prev.tF, prev.rb1, prev.on1);
       };
-      if (!a.ragged && my_rbs % 2 == 0) paired_schedule(std::true_type{});
-      else paired_schedule(std::false_type{});
+      if (a.ragged || my_rbs % 2 != 0 || x_rescaled) paired_schedule(std::false_type{}, std::true_type{});
+      else if (q == a.trace_q) paired_schedule(std::true_type{}, std::true_type{});
+      else paired_schedule(std::true_type{}, std::false_type{});
       return;
     }
   }
