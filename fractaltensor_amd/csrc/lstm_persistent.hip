@@ -1184,8 +1184,9 @@ void lstm_persistent_kernel(PersistArgs a) {
             b_stored = false;
           }
           wx.lo = wx.hi;
+          wx.hi.on = false;   // block b's rows on the first eight steps: they have landed when the phase ends
           if (TRACED && tracing) a.trace[TS * p + 4] = wall_clock64();
-          if (on1) block_products(hb, IC<1>{}, IC<1>{}, am1, ar1, IC<8>{}, wx, std::true_type{}, am0, ar0, cp0, 0, nothing);
+          if (on1) block_products(hb, IC<1>{}, IC<1>{}, am1, ar1, IC<16>{}, wx, std::true_type{}, am0, ar0, cp0, 0, nothing);
           else {
             if (wx.lo.on) copy_block(xsrc, nxt.rb1, xa_lds, 1);
             activations_alone(am0, ar0, cp0, 0);
