@@ -791,8 +791,13 @@ void lstm_persistent_kernel(PersistArgs a) {
       }
       const float4 cp = load_cprev(n);
       if (lane == 0) votes[wave] = xnext ? 1 : 0;
-      __builtin_amdgcn_s_waitcnt(0);
-      __syncthreads();
+      // This item needs its own tile, not the next one's x columns: those were requested behind it (eight copies,
+      // four with two batch rows per tile row), the counter of outstanding copies runs in issue order, and the
+      // barrier behind the activations waits for the rest.
+      if (xnext && PAIR) asm volatile("s_waitcnt vmcnt(4) lgkmcnt(0)" ::: "memory");
+      else if (xnext) asm volatile("s_waitcnt vmcnt(8) lgkmcnt(0)" ::: "memory");
+      else asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+      barrier();
       const int4 vote = *reinterpret_cast<const int4*>(votes);
       const bool xall = (vote.x & vote.y & vote.z & vote.w) != 0;   // the whole of tile n+1's x columns has landed
       if (live(n)) {
