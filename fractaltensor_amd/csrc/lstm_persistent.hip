@@ -106,7 +106,8 @@ struct PersistArgs {
   int pr_of[kMaxLayers];        // row slices of layer l (its workgroups: column slices x row slices)
   int first_q[kMaxLayers + 1];  // first logical workgroup of layer l; [L] = all
   int groups;      // workgroups that take part (= first_q[L])
-  int xcd_remap;   // 1: grid is a multiple of 8, map workgroups so a layer shares an XCD
+  int xcd_remap;   // 1: grid is a multiple of 8, map workgroups so a layer shares an XCD; w > 1: layers of w workgroups
+                   // each, layer l on XCD l % 8
   int spin_limit;
   int trace_q;            // logical workgroup whose item timeline is recorded, or -1
   long long* trace;       // [items][8] 100 MHz clock stamps of that workgroup
@@ -247,7 +248,12 @@ void lstm_persistent_kernel(PersistArgs a) {
   const int jb = MODE == kHalfData256 ? 2 * (j & 15) + (j >> 4) : j;
 
   int q = blockIdx.x;
-  if (a.xcd_remap) q = (blockIdx.x & 7) * (gridDim.x >> 3) + (blockIdx.x >> 3);
+  if (a.xcd_remap == 1) q = (blockIdx.x & 7) * (gridDim.x >> 3) + (blockIdx.x >> 3);
+  if (a.xcd_remap > 1) {   // the i-th layer of XCD x is the stack's layer 8 i + x; slots beyond the last layer stay empty
+    const int slot = blockIdx.x >> 3, w = a.xcd_remap;
+    const int layer = (slot / w) * 8 + (int)(blockIdx.x & 7);
+    q = layer < a.L ? layer * w + slot % w : a.groups;
+  }
   if (q >= a.groups) return;
   if (q == a.trace_q && tid == 0) reinterpret_cast<long long*>(a.status + 16)[0] = wall_clock64();
   int l = 0;
@@ -1580,8 +1586,24 @@ static int run_persistent(int mode, const void* xs, const void* WU, const float*
     }
     a.steps_of[rb] = steps;
   }
-  const int grid = a.groups;
+  int grid = a.groups;
   a.xcd_remap = (grid % 8 == 0) ? 1 : 0;
+  // Deep stacks of equal layers: consecutive layers go to different XCDs (layer l to XCD l % 8) instead of four in a
+  // row to the same one.  The layers at the bottom of a stack never wait and set the pace of all the others, which
+  // wait a little in every item; an XCD that holds only layers of the first kind runs every phase about 8 % slower
+  // than one that holds only layers of the second (measured: the clock follows what the XCD does), so the pacing
+  // layers are better spread, each beside layers that leave the XCD some slack.  (FTK_LSTM_LAYER_BLOCKS=1: the
+  // older placement.)
+  {
+    bool uniform = true;
+    for (int l = 1; l < L; ++l) uniform = uniform && a.pr_of[l] == a.pr_of[0];
+    const int w = npc * a.pr_of[0], per_xcd = ((L + 7) / 8) * w;
+    static const bool blocks = getenv("FTK_LSTM_LAYER_BLOCKS") && atoi(getenv("FTK_LSTM_LAYER_BLOCKS")) != 0;
+    if (uniform && L >= 8 && w > 1 && 8 * per_xcd <= slots && !blocks) {
+      a.xcd_remap = w;
+      grid = 8 * per_xcd;
+    }
+  }
   // FTK_LSTM_PAIRS=0: pipelined layers of the split-product kernel walk single row blocks (the older schedule)
   static const bool pairs_off = getenv("FTK_LSTM_PAIRS") && atoi(getenv("FTK_LSTM_PAIRS")) == 0;
   a.paired = (split && !pairs_off && B % 8 == 0) ? 1 : 0;
