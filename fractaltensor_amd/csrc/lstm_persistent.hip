@@ -799,7 +799,7 @@ void lstm_persistent_kernel(PersistArgs a) {
       if (lane == 0) votes[wave] = xnext ? 1 : 0;
       // This item needs its own tile, not the next one's x columns: those were requested behind it (eight copies,
       // four with two batch rows per tile row), the counter of outstanding copies runs in issue order, and the
-      // barrier behind the activations waits for the rest.
+      // rest is waited for in front of the barrier behind the activations.
       if (xnext && PAIR) asm volatile("s_waitcnt vmcnt(4) lgkmcnt(0)" ::: "memory");
       else if (xnext) asm volatile("s_waitcnt vmcnt(8) lgkmcnt(0)" ::: "memory");
       else asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
@@ -814,7 +814,10 @@ void lstm_persistent_kernel(PersistArgs a) {
         if (item_t(n) >= d) mfma_range(buf, IC<1>{}, IC<0>{}, IC<16>{});
         epilogue_to_lds(gate_sums(), cp, 0);
       }
-      __syncthreads();  // results staged; the tile may be rewritten by the item after the next
+      // the next item's x columns, requested above, are waited for here, by hand: the compiler does not count those
+      // copies, so the barrier's own fence waits for none of them
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+      __syncthreads();  // results staged; the next item's x columns complete; the tile may be rewritten by the item after the next
       store_item(n, 0);
       xdone = false;
       if (xall) {           // while the stores are acknowledged
