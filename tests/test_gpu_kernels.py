@@ -536,6 +536,38 @@ def test_stacked_lstm_f16(core, H, L, T, B, dil, bias, ragged):
     assert same > (0.6 if L * T > 250 else 0.7 if L * T > 150 else 0.9 if H <= 512 else 0.8), same
 
 
+def test_hand_over_with_fp16_data_gives_the_same_bits_every_launch(core):
+    """The same soak as for the fp32 kernel, on the fp16 flavours of the persistent kernel (whole rows of 512 fp16 per
+    tile row, and two batch rows of 256 per tile row).  Layers on the serial schedule request the next item's x columns
+    behind the tile that the current item needs and wait for the two separately; a product formed before the second
+    wait would show here as a launch that differs from the first (it did, once, in a launch of the first case)."""
+    cases = [
+        (512, 3, 8, 96, [1, 2, 4], 40),
+        (512, 4, 24, 64, None, 30),
+        (256, 3, 8, 96, [1, 2, 4], 40),
+        (256, 8, 24, 64, None, 30),
+    ]
+    for ci, (H, L, T, B, dil, launches) in enumerate(cases):
+        print(f'fp16 soak case {ci}: H{H} L{L} T{T} B{B} dil {dil}', flush=True)
+        rng = np.random.default_rng(40 + ci)
+        xs = rng.standard_normal((T, B, H)).astype(np.float16)
+        WU = rng.uniform(-1, 1, (L, 2 * H, 4 * H)).astype(np.float16) / np.float16(np.sqrt(H))
+        x_d, w_d = dev(xs), dev(WU)
+        first = None
+        for i in range(launches):
+            hsss, csss = core.stacked_lstm_f16(x_d, w_d, None, dilations=dil)
+            torch.cuda.synchronize()
+            if first is None:
+                first = (hsss.clone(), csss.clone())
+                hr, cr = ko.stacked_lstm_f16(xs, WU, None, dil)
+                assert ko.max_rel_err(first[0].float().cpu().numpy(), hr.astype(np.float32)) <= F16_TOL
+                assert ko.max_rel_err(first[1].float().cpu().numpy(), cr.astype(np.float32)) <= F16_TOL
+                continue
+            assert torch.equal(hsss, first[0]) and torch.equal(csss, first[1]), f'fp16 case {ci}, launch {i} differs from launch 0'
+        del first, x_d, w_d
+        torch.cuda.empty_cache()
+
+
 def test_stacked_lstm_f16_rejects_other_hidden_sizes(core):
     xs = torch.zeros((2, 32, 80), dtype=torch.float16, device='cuda')
     WU = torch.zeros((1, 160, 320), dtype=torch.float16, device='cuda')
