@@ -106,8 +106,8 @@ struct PersistArgs {
   int pr_of[kMaxLayers];        // row slices of layer l (its workgroups: column slices x row slices)
   int first_q[kMaxLayers + 1];  // first logical workgroup of layer l; [L] = all
   int groups;      // workgroups that take part (= first_q[L])
-  int xcd_remap;   // 1: grid is a multiple of 8, map workgroups so a layer shares an XCD; w > 1: layers of w workgroups
-                   // each, layer l on XCD l % 8
+  int xcd_remap;   // 1: grid is a multiple of 8, workgroups in order, grid / 8 per XCD; w > 1: units of w workgroups
+                   // (a layer's column slices of one row slice), unit u on XCD u % 8
   int spin_limit;
   int trace_q;            // logical workgroup whose item timeline is recorded, or -1
   long long* trace;       // [items][8] 100 MHz clock stamps of that workgroup
@@ -249,10 +249,9 @@ void lstm_persistent_kernel(PersistArgs a) {
 
   int q = blockIdx.x;
   if (a.xcd_remap == 1) q = (blockIdx.x & 7) * (gridDim.x >> 3) + (blockIdx.x >> 3);
-  if (a.xcd_remap > 1) {   // the i-th layer of XCD x is the stack's layer 8 i + x; slots beyond the last layer stay empty
+  if (a.xcd_remap > 1) {   // the i-th unit of XCD x is unit 8 i + x of the launch; slots beyond the last unit stay empty
     const int slot = blockIdx.x >> 3, w = a.xcd_remap;
-    const int layer = (slot / w) * 8 + (int)(blockIdx.x & 7);
-    q = layer < a.L ? layer * w + slot % w : a.groups;
+    q = ((slot / w) * 8 + (int)(blockIdx.x & 7)) * w + slot % w;
   }
   if (q >= a.groups) return;
   if (q == a.trace_q && tid == 0) reinterpret_cast<long long*>(a.status + 16)[0] = wall_clock64();
@@ -1591,19 +1590,19 @@ static int run_persistent(int mode, const void* xs, const void* WU, const float*
   }
   int grid = a.groups;
   a.xcd_remap = (grid % 8 == 0) ? 1 : 0;
-  // Deep stacks of equal layers: consecutive layers go to different XCDs (layer l to XCD l % 8) instead of four in a
-  // row to the same one.  The layers at the bottom of a stack never wait and set the pace of all the others, which
-  // wait a little in every item; an XCD that holds only layers of the first kind runs every phase about 8 % slower
-  // than one that holds only layers of the second (measured: the clock follows what the XCD does), so the pacing
-  // layers are better spread, each beside layers that leave the XCD some slack.  (FTK_LSTM_LAYER_BLOCKS=1: the
-  // older placement.)
+  // Placement.  A unit is the npc workgroups that share a layer's rows (its column slices): they exchange h at every
+  // step, and a unit stays on one XCD.  Units go to the XCDs in turn, unit u to XCD u % 8, so that consecutive layers
+  // of a deep stack sit on different XCDs: the
+  // layers at the bottom of a stack never wait and set the pace of all the others, which wait a little in every
+  // item, and an XCD that holds only layers of the first kind runs every phase about 8 % slower than one that holds
+  // only layers of the second (the clock follows what the XCD does), so the pacing layers are better spread, each
+  // beside layers that leave the XCD some slack.  The grid is rounded up to whole units per XCD; workgroups beyond the
+  // last unit leave at once.  (FTK_LSTM_LAYER_BLOCKS=1: the older placement, workgroups in order, grid / 8 per XCD.)
   {
-    bool uniform = true;
-    for (int l = 1; l < L; ++l) uniform = uniform && a.pr_of[l] == a.pr_of[0];
-    const int w = npc * a.pr_of[0], per_xcd = ((L + 7) / 8) * w;
+    const int units = a.groups / npc, per_xcd = ((units + 7) / 8) * npc;
     static const bool blocks = getenv("FTK_LSTM_LAYER_BLOCKS") && atoi(getenv("FTK_LSTM_LAYER_BLOCKS")) != 0;
-    if (uniform && L >= 8 && w > 1 && 8 * per_xcd <= slots && !blocks) {
-      a.xcd_remap = w;
+    if (npc > 1 && 8 * per_xcd <= slots && !blocks) {
+      a.xcd_remap = npc;
       grid = 8 * per_xcd;
     }
   }
