@@ -1262,10 +1262,10 @@ void lstm_persistent_kernel(PersistArgs a) {
   //     after counting item n itself, which is what the layer above is waiting for while the wavefront
   //     fills;
   //   barrier: tile n+1 is complete.
-  // Loads and stores share one counter of outstanding operations and may complete out of order with
-  // respect to each other, so the result of a load is only known to have arrived when nothing at all is
-  // outstanding: a look at completion counts less than about 2 us after an item's stores have left waits
-  // for their acknowledgement.  Hence the order above: what is asked for before the barrier costs no
+  // Loads and stores share one counter of outstanding operations, and completion is reported in issue
+  // order: the result of a load is known to have arrived only once everything issued before it, stores
+  // included, has completed, so a look at completion counts less than about 2 us after an item's stores
+  // have left waits for their acknowledgement.  Hence the order above: what is asked for before the barrier costs no
   // wait of its own, and an item that finds its successor's tile already requested touches no load
   // result until its MFMAs are done.  With split
   // products an item's MFMAs take less than those 2 us, so the only look inside an item is the one after
