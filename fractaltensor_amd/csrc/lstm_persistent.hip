@@ -856,7 +856,7 @@ void lstm_persistent_kernel(PersistArgs a) {
   // wave reached after such a wait.  Flags stay per 32-row block, so layers on the other schedules hand over to this
   // one and back.  The h columns of item p need this layer's item p - (own distance >= 2), whose second block was
   // published before barrier 2 of item p-1.
-  if constexpr (SPLIT) {
+  if constexpr (SPLIT || MODE == kHalfData256) {
     const int ppt = (my_rbs + 1) / 2;            // pair items per time step
     if (a.paired && my_rbs >= 2 && (long long)d * ppt >= 2) {
       // PLAIN: every item has both its blocks at every step (no ragged batch, an even number of row blocks), and no
@@ -868,11 +868,18 @@ void lstm_persistent_kernel(PersistArgs a) {
       auto paired_schedule = [&](auto plain_c, auto traced_c) __attribute__((always_inline)) {
       constexpr bool PLAIN = decltype(plain_c)::value;
       constexpr bool TRACED = decltype(traced_c)::value;   // this workgroup leaves time stamps
-      constexpr int HLD = 1040;                  // bytes per row of a half buffer: 16 more than the row's two planes
+      // fp16 data at H = 256 walks the same schedule: a batch row is 512 bytes there, a tile row of a half buffer holds
+      // two of them (a copy instruction carries 1 KB), a contraction step is one MFMA instead of three, and h and c
+      // leave as fp16.
+      constexpr bool P16 = MODE == kHalfData256;
+      constexpr int RB = P16 ? 512 : 1024;       // bytes of a batch row in a layer's arrays
+      constexpr int TR = P16 ? 16 : 32;          // tile rows of a row block in a half buffer
+      constexpr int NC = TR / 4;                 // copies per wave and block half: one tile row each
+      constexpr int HLD = 1040;                  // bytes per row of a half buffer: 16 more than the 1 KB it holds
       const int n_pairs = T * ppt;
       unsigned char* const xa = reinterpret_cast<unsigned char*>(tile);
-      unsigned char* const hb = xa + 64 * HLD;
-      const unsigned xa_lds = tile_lds, hb_lds = tile_lds + 64u * HLD;
+      unsigned char* const hb = xa + 2 * TR * HLD;
+      const unsigned xa_lds = tile_lds, hb_lds = tile_lds + 2u * TR * HLD;
       // The per-register factors and biases of the gate sums move to a table in LDS, one set per wave and lane half,
       // in the order the activations take them: with four accumulators per lane the registers are needed elsewhere.
       // (a unit's four entries: gate i, the candidate, gates f and o -- the first part of a unit's activations takes
@@ -883,7 +890,9 @@ void lstm_persistent_kernel(PersistArgs a) {
         for (int m = 0; m < 16; ++m) {
           constexpr int gate_of[4] = {0, 3, 1, 2};
           const int reg = 4 * gate_of[m & 3] + (m >> 2);
-          gtab[m] = make_float2(esc[reg], ebias[reg]);
+          float factor = (reg >> 2) == 3 ? 1.0f : -kLog2e;
+          if constexpr (SPLIT) factor = esc[SPLIT ? reg : 0];
+          gtab[m] = make_float2(factor, ebias[reg]);
         }
       }
       // what part m of the activations needs from the table
@@ -898,7 +907,7 @@ void lstm_persistent_kernel(PersistArgs a) {
       // an item's addresses are not multiplied out of (layer, step, row) each time: an item carries the byte offset
       // of its time step in those arrays (tO) and in a layer's flags (tF), the next item's follow by addition, and
       // the layer's bases are formed once.  (tF fits 32 bits: a layer's flags are 1/512 the size of its h.)
-      const size_t stepO = (size_t)B * 1024, dO = (size_t)d * stepO;
+      const size_t stepO = (size_t)B * RB, dO = (size_t)d * stepO;
       const unsigned stepF = (unsigned)a.nrb * kFlagStride, dF = (unsigned)d * stepF;
       const char* const xbase = reinterpret_cast<const char*>((l == 0) ? xin : hin + (size_t)(l - 1) * T * cell);
       const char* const hbase = reinterpret_cast<const char*>(hin + (size_t)l * T * cell);
@@ -927,7 +936,7 @@ void lstm_persistent_kernel(PersistArgs a) {
       // its end; those beyond are copied from the batch's last 8 rows instead (nobody stores what comes of them).
       struct Rows { bool on; const char* g; unsigned lds; };
       auto rows_of = [&](const char* src, int rb, unsigned half_lds, int sub, bool on) __attribute__((always_inline)) -> Rows {
-        return Rows{on, src + ((unsigned)min(rb * 32 + 8 * wave_u, B - 8) << 10), half_lds + (unsigned)((32 * sub + 8 * wave_u) * HLD)};
+        return Rows{on, src + (unsigned)min(rb * 32 + 8 * wave_u, B - 8) * (unsigned)RB, half_lds + (unsigned)((TR * sub + NC * wave_u) * HLD)};
       };
       auto copy_row = [&](const Rows& x, auto r_c) __attribute__((always_inline)) {
         constexpr int r = decltype(r_c)::value;
@@ -935,7 +944,7 @@ void lstm_persistent_kernel(PersistArgs a) {
       };
       auto copy_block = [&](const char* src, int rb, unsigned half_lds, int sub) __attribute__((always_inline)) {
         const Rows x = rows_of(src, rb, half_lds, sub, true);
-        static_for<8>([&](auto r_c) __attribute__((always_inline)) { copy_row(x, r_c); });
+        static_for<NC>([&](auto r_c) __attribute__((always_inline)) { copy_row(x, r_c); });
       };
       auto copy_ratios = [&](const Pair& x) __attribute__((always_inline)) {   // first layer: the rows' scale ratios travel with their x columns
         if (PLAIN || !x_rescaled || wave_u != 0) return;
@@ -967,7 +976,8 @@ void lstm_persistent_kernel(PersistArgs a) {
           __hip_atomic_store(fown + (tF + (unsigned)rb * kFlagStride + 4 * pc + wave), (unsigned char)1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       };
       // store_block / load_cprev_of on the offsets an item carries
-      auto store_rows = [&](size_t tO, int rb, bool is_live, int sbuf) __attribute__((always_inline)) {
+      auto store_rows = [&](int t, size_t tO, int rb, bool is_live, int sbuf) __attribute__((always_inline)) {
+        if constexpr (P16) { store_block(t, rb, is_live, sbuf); return; }
         const int rl = 8 * wave + (lane >> 3), cc = lane & 7;
         const int rg = rb * 32 + rl;
         if (alive && rg < B && is_live) {
@@ -980,7 +990,8 @@ void lstm_persistent_kernel(PersistArgs a) {
           coherent_store8h(pdst + PH, *reinterpret_cast<const v4h*>(sb + kStageRest + rl * kStageRow16 + 8 * cc));
         }
       };
-      auto cprev_rows = [&](size_t tO_prev, int rb, bool has) __attribute__((always_inline)) -> float4 {
+      auto cprev_rows = [&](int t, size_t tO_prev, int rb, bool has) __attribute__((always_inline)) -> float4 {
+        if constexpr (P16) return load_cprev_of(t, rb, has);
         float4 cp = make_float4(0.f, 0.f, 0.f, 0.f);
         if (alive && has)
           cp = *reinterpret_cast<const float4*>(cbase + tO_prev + (((unsigned)min(rb * 32 + j, B - 1) << 10) + 4u * (unsigned)u0));
@@ -991,7 +1002,10 @@ void lstm_persistent_kernel(PersistArgs a) {
       // no more operations are outstanding than were issued behind them.  `loads` (0 or 1) and `copies` (0 or 8) are
       // what the caller knows was issued behind the stores; more than that only makes the wait longer.
       auto wait_stores_behind = [&](bool one_load, bool eight_copies) __attribute__((always_inline)) {
-        if (eight_copies) {
+        if (eight_copies && P16) {   // (four copies carry a block half there)
+          if (one_load) asm volatile("s_waitcnt vmcnt(5)" ::: "memory");
+          else asm volatile("s_waitcnt vmcnt(4)" ::: "memory");
+        } else if (eight_copies) {
           if (one_load) asm volatile("s_waitcnt vmcnt(9)" ::: "memory");
           else asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
         } else {
@@ -1008,16 +1022,19 @@ void lstm_persistent_kernel(PersistArgs a) {
       // piece carries two chains that do not depend on each other: parts 0..2 hold a sigmoid (gates i, f, o) beside a
       // third of the candidate's tanh, part 3 the tanh of the new c, whose exponential and polynomial are independent.
       float tc_v = 0.f, tc_e = 0.f, tc_x2 = 0.f, tc_p = 0.f, tc_r = 0.f;   // the candidate's tanh between the parts
+      // (split products: the second accumulator holds the cross terms, 2^-11 of a product; fp16 data: the two
+      // accumulators are two chains of the same sum)
+      constexpr float kRestFactor = SPLIT ? 1.0f / kSplitRest : 1.0f;
       auto pair_piece = [&](const v16f& em, const v16f& er, const float4& cp, float (&hv)[4], float (&cv)[4], const float4 sb, auto mc) __attribute__((always_inline)) {
         constexpr int m = decltype(mc)::value;
         constexpr int r = m >> 2, g = m & 3, reg = 4 * g + r;
         const float cpv[4] = {cp.x, cp.y, cp.z, cp.w};
         auto inv1p = [](float e) { return __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(e)); };
         if constexpr (g < 3) {
-          const float v = sb.x * (em[reg] + (1.0f / kSplitRest) * er[reg]) + sb.y;
+          const float v = sb.x * (em[reg] + kRestFactor * er[reg]) + sb.y;
           if constexpr (g == 0) {
             eg_i = inv1p(v);
-            tc_v = sb.z * (em[12 + r] + (1.0f / kSplitRest) * er[12 + r]) + sb.w;
+            tc_v = sb.z * (em[12 + r] + kRestFactor * er[12 + r]) + sb.w;
             tc_e = fast_exp(2.0f * tc_v);
             tc_x2 = tc_v * tc_v;
           }
@@ -1052,10 +1069,13 @@ void lstm_persistent_kernel(PersistArgs a) {
                                 auto epi_c, const v16f& em, const v16f& er, const float4& ecp, int esbuf, auto&& late) __attribute__((always_inline)) {
         constexpr int SUB = decltype(sub_c)::value, hf = decltype(hf_c)::value, NW = decltype(nw_c)::value;
         constexpr bool EPI = decltype(epi_c)::value;
-        const _Float16* row = reinterpret_cast<const _Float16*>(hbuf + (32 * SUB + j) * HLD) + 8 * hh;
+        // (fp16 data: batch row jb of the block is half jb & 1 of tile row jb >> 1, and has no second plane)
+        const _Float16* row = P16 ? reinterpret_cast<const _Float16*>(hbuf + (TR * SUB + (jb >> 1)) * HLD + (jb & 1) * RB) + 8 * hh
+                                  : reinterpret_cast<const _Float16*>(hbuf + (TR * SUB + j) * HLD) + 8 * hh;
+        constexpr int RO = P16 ? 0 : PH;   // where a row's second plane starts (fp16 elements)
         float hv[4], cv[4];
-        v8h bt = *reinterpret_cast<const v8h*>(row), br = *reinterpret_cast<const v8h*>(row + PH);
-        v8h nt = *reinterpret_cast<const v8h*>(row + 16), nr = *reinterpret_cast<const v8h*>(row + PH + 16);
+        v8h bt = *reinterpret_cast<const v8h*>(row), br = *reinterpret_cast<const v8h*>(row + RO);
+        v8h nt = *reinterpret_cast<const v8h*>(row + 16), nr = *reinterpret_cast<const v8h*>(row + RO + 16);
         float4 sb = make_float4(0.f, 0.f, 0.f, 0.f);
         if constexpr (EPI) sb = gate_entry(IC<0>{});
         static_for<16>([&](auto s_c) __attribute__((always_inline)) {
@@ -1066,15 +1086,21 @@ void lstm_persistent_kernel(PersistArgs a) {
           float4 nsb = sb;
           if constexpr (sidx + 2 < 16) {
             n2t = *reinterpret_cast<const v8h*>(row + 16 * (sidx + 2));
-            n2r = *reinterpret_cast<const v8h*>(row + PH + 16 * (sidx + 2));
+            if constexpr (!P16) n2r = *reinterpret_cast<const v8h*>(row + RO + 16 * (sidx + 2));
           }
           if constexpr (sidx + 1 < 16) {
             if constexpr (EPI) nsb = gate_entry(IC<sidx + 1>{});
           }
           // top x top in one accumulator; top x rest and rest x top, both 2^-11 of a product, share the other
-          am = __builtin_amdgcn_mfma_f32_32x32x16_f16(whi[qq], bt, first ? zero16 : am, 0, 0, 0);
-          ar = __builtin_amdgcn_mfma_f32_32x32x16_f16(whi[qq], br, first ? zero16 : ar, 0, 0, 0);
-          ar = __builtin_amdgcn_mfma_f32_32x32x16_f16(wlo[qq], bt, ar, 0, 0, 0);
+          if constexpr (P16) {   // one product per step, the steps dealt to two accumulation chains
+            constexpr bool first2 = hf == 0 && sidx < 2;
+            if constexpr ((sidx & 1) == 0) am = __builtin_amdgcn_mfma_f32_32x32x16_f16(wh[P16 ? qq : 0], bt, first2 ? zero16 : am, 0, 0, 0);
+            else ar = __builtin_amdgcn_mfma_f32_32x32x16_f16(wh[P16 ? qq : 0], bt, first2 ? zero16 : ar, 0, 0, 0);
+          } else {
+            am = __builtin_amdgcn_mfma_f32_32x32x16_f16(whi[SPLIT ? qq : 0], bt, first ? zero16 : am, 0, 0, 0);
+            ar = __builtin_amdgcn_mfma_f32_32x32x16_f16(whi[SPLIT ? qq : 0], br, first ? zero16 : ar, 0, 0, 0);
+            ar = __builtin_amdgcn_mfma_f32_32x32x16_f16(wlo[SPLIT ? qq : 0], bt, ar, 0, 0, 0);
+          }
           if constexpr (EPI) {
             pair_piece(em, er, ecp, hv, cv, sb, s_c);
             // the piece's results are pinned to this step: left alone, the compiler moves every piece behind the last
@@ -1086,16 +1112,24 @@ void lstm_persistent_kernel(PersistArgs a) {
           }
           // the order within the step: next step's fragments (and the piece's table entry) first, then the MFMAs
           // with the piece's vector instructions between them
-          __builtin_amdgcn_sched_group_barrier(0x100, EPI ? 3 : 2, 0);
-          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-          if constexpr (EPI) __builtin_amdgcn_sched_group_barrier(0x002, 10, 0);
-          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-          if constexpr (EPI) __builtin_amdgcn_sched_group_barrier(0x002, 10, 0);
-          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+          if constexpr (P16) {
+            __builtin_amdgcn_sched_group_barrier(0x100, EPI ? 2 : 1, 0);
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+            if constexpr (EPI) __builtin_amdgcn_sched_group_barrier(0x002, 20, 0);
+          } else {
+            __builtin_amdgcn_sched_group_barrier(0x100, EPI ? 3 : 2, 0);
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+            if constexpr (EPI) __builtin_amdgcn_sched_group_barrier(0x002, 10, 0);
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+            if constexpr (EPI) __builtin_amdgcn_sched_group_barrier(0x002, 10, 0);
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+          }
           if constexpr (sidx == 13) late();   // something the caller wants issued near the end of the phase
-          if constexpr (NW == 16) {
+          // (a group is NC copies: NW == 16 puts group lo on the first steps of the phase's first half and group hi on
+          // the first of its second half, NW == 8 group lo on the even steps)
+          if constexpr (NW == 16 && (sidx & 7) < NC) {
             if (sidx < 8 ? w.lo.on : w.hi.on) copy_row(sidx < 8 ? w.lo : w.hi, IC<(sidx & 7)>{});
-          } else if constexpr (NW == 8 && (sidx & 1) == 0) {
+          } else if constexpr (NW == 8 && (sidx & 1) == 0 && (sidx >> 1) < NC) {
             if (w.lo.on) copy_row(w.lo, IC<(sidx >> 1)>{});
           }
           bt = nt; br = nr; nt = n2t; nr = n2r; sb = nsb;
@@ -1178,9 +1212,9 @@ void lstm_persistent_kernel(PersistArgs a) {
         a_stored = false;
         barrier();   // 1: HB and staging 1 complete, XA free
         if (TRACED && tracing) a.trace[TS * p + 3] = wall_clock64();
-        if (p > 0) { store_rows(prev.tO, prev.rb1, prev.on1, 1); b_stored = true; }
+        if (p > 0) { store_rows(prev.t, prev.tO, prev.rb1, prev.on1, 1); b_stored = true; }
         const bool cp1_loads = alive && cur.on1 && has_prev;
-        cp1 = cprev_rows(cur.tO - dO, cur.rb1, cur.on1 && has_prev);
+        cp1 = cprev_rows(cur.t, cur.tO - dO, cur.rb1, cur.on1 && has_prev);
         // ---- Ha, Hb with Ea | x columns of the next item -> XA
         const bool x_ok = more && alive && (l == 0 || all_set(fb));
         asm volatile("" ::: "memory");
@@ -1225,9 +1259,9 @@ void lstm_persistent_kernel(PersistArgs a) {
         b_stored = false;
         barrier();   // 2: XA and staging 0 complete, HB free
         if (TRACED && tracing) a.trace[TS * p + 6] = wall_clock64();
-        store_rows(cur.tO, cur.rb0, cur.on0, 0);
+        store_rows(cur.t, cur.tO, cur.rb0, cur.on0, 0);
         a_stored = true;
-        if (more) cp0 = cprev_rows(nxt.tO - dO, nxt.rb0, nxt.on0 && nxt.t >= d);
+        if (more) cp0 = cprev_rows(nxt.t, nxt.tO - dO, nxt.rb0, nxt.on0 && nxt.t >= d);
         if (TRACED && tracing) a.trace[TS * p + 7] = wall_clock64();
         prev = cur;
         cur = nxt;
@@ -1237,7 +1271,7 @@ void lstm_persistent_kernel(PersistArgs a) {
       wait_all();
       if (a_stored) publish_block(prev.tF, prev.rb0, prev.on0);
       barrier();
-      store_rows(prev.tO, prev.rb1, prev.on1, 1);
+      store_rows(prev.t, prev.tO, prev.rb1, prev.on1, 1);
       wait_all();
       publish_block(prev.tF, prev.rb1, prev.on1);
       };
@@ -1608,7 +1642,7 @@ static int run_persistent(int mode, const void* xs, const void* WU, const float*
   }
   // FTK_LSTM_PAIRS=0: pipelined layers of the split-product kernel walk single row blocks (the older schedule)
   static const bool pairs_off = getenv("FTK_LSTM_PAIRS") && atoi(getenv("FTK_LSTM_PAIRS")) == 0;
-  a.paired = (split && !pairs_off && B % 8 == 0) ? 1 : 0;
+  a.paired = ((split || mode == kHalfData256) && !pairs_off && B % 8 == 0) ? 1 : 0;
 
   // flags and status block start from zero; a later launch of a stack that runs as several keeps the error word
   // of the earlier ones (it then drains at its first long wait, and the call reports the time-out)

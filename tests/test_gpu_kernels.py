@@ -509,6 +509,11 @@ def test_stacked_lstm_ragged_rejects_unsorted_rows(core):
     (512, 6, 50, 16, [1, 2, 4, 8, 16, 32], False, False),
     (32, 4, 4, 8, [1, 2, 4, 8], False, False),      # test_dilated_lstm_region.cu:125-148
     (32, 4, 4, 32, [1, 2, 4, 8], False, False),
+    (256, 4, 12, 256, None, True, False),           # eight row blocks per workgroup: items of two row blocks (the paired schedule)
+    (256, 3, 10, 128, None, False, False),          # ... four
+    (256, 3, 12, 256, None, True, True),            # ... with rows that stop after 4 steps
+    (256, 2, 6, 96, None, True, False),             # ... an odd number of row blocks: the last item has one
+    (256, 3, 8, 128, [1, 2, 4], False, False),      # ... dilated
 ])
 def test_stacked_lstm_f16(core, H, L, T, B, dil, bias, ragged):
     rng = np.random.default_rng(13)
@@ -546,6 +551,7 @@ def test_hand_over_with_fp16_data_gives_the_same_bits_every_launch(core):
         (512, 4, 24, 64, None, 30),
         (256, 3, 8, 96, [1, 2, 4], 40),
         (256, 8, 24, 64, None, 30),
+        (256, 12, 16, 256, None, 30),                   # items of two row blocks
     ]
     for ci, (H, L, T, B, dil, launches) in enumerate(cases):
         print(f'fp16 soak case {ci}: H{H} L{L} T{T} B{B} dil {dil}', flush=True)
