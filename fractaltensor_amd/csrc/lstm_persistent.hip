@@ -831,7 +831,8 @@ void lstm_persistent_kernel(PersistArgs a) {
     return;
   }
 
-  // ---- paired schedule (split products): an item is TWO row blocks (a, b) of one time step, 64 batch rows.
+  // ---- paired schedule (split products, and fp16 data at H = 256): an item is TWO row blocks (a, b) of one time
+  // step, 64 batch rows.
   // What an item costs beyond its MFMAs -- the looks at the producers' flags, the waits for the stores'
   // acknowledgement, the barriers -- is paid once per hand-over whatever the number of rows, and with two blocks in
   // flight the activations of one block run on the vector pipeline while the matrix pipeline forms the other block's
@@ -846,10 +847,12 @@ void lstm_persistent_kernel(PersistArgs a) {
   //   wait for everything outstanding (the stores of block a of item p-1 among it: that block is published)
   //   barrier 1: HB and staging 1 complete, XA free
   //   stores of block b of item p-1 from staging 1
-  //   Ha(p)                              | rows of item p+1's x columns -> XA, if the layer below was seen ready
-  //   Hb(p) with Ea(p) -> staging 0      | the same, second block
+  //   Ha(p)                              | block a's rows of item p+1's x columns -> XA, if the layer below was seen
+  //                                        ready
+  //   wait for those stores alone: block b of item p-1 is published (split products)
+  //   Hb(p) with Ea(p) -> staging 0      | block b's rows, on the phase's first steps
   //   (a wave that could not request its x rows waits for the layer below and requests them now)
-  //   wait for everything outstanding (block b of item p-1 is published)
+  //   wait for everything outstanding (fp16 data: block b of item p-1 is published here)
   //   barrier 2: XA and staging 0 complete, HB free
   //   stores of block a of item p from staging 0
   // A wave only ever waits for the copies it issued itself, and fragment reads of a half follow a barrier that every
