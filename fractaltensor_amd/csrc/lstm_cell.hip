@@ -1097,6 +1097,12 @@ int run_wavefront_split(const float* xs, const float* WU, const float* bias, con
 
 }  // namespace ftk
 
+namespace ftk {
+// gemm_f16.hip: the product for shapes made of whole 256 x 256 tiles
+bool gemm_f16_tiles_fit(int M, int N, int K);
+int launch_gemm_f16_tiles(const void* A, const void* Bm, void* C, int G, int M, int N, int K, hipStream_t s);
+}  // namespace ftk
+
 extern "C" {
 
 int ftk_lstm_cell_f32(const float* x, const float* h_prev, const float* c_prev, const float* WU, const float* bias,
@@ -1212,6 +1218,8 @@ static int gemm_f16(const char* who, const void* A, const void* Bm, void* C, int
   if (!A || !Bm || !C) return ftk::fail(FTK_ERR_INVALID_ARGUMENT, "%s: A, B, C must be non-NULL", who);
   if (G <= 0 || M <= 0 || N <= 0 || K <= 0) return ftk::fail(FTK_ERR_INVALID_ARGUMENT, "%s: G, M, N, K must be positive", who);
   if (N % 128 || K % 32) return ftk::fail(FTK_ERR_UNSUPPORTED_SHAPE, "%s: N=%d must be a multiple of 128 and K=%d of 32", who, N, K);
+  // N a multiple of 256: the kernel built for the product (gemm_f16.hip); otherwise the cell kernel without the cell
+  if (ftk::gemm_f16_tiles_fit(M, N, K)) return ftk::launch_gemm_f16_tiles(A, Bm, C, G, M, N, K, s);
   if ((long long)M * std::max(K, N) >= (1ll << 30)) return ftk::fail(FTK_ERR_UNSUPPORTED_SHAPE, "%s: M=%d too large", who, M);
   const int Hq = N / 4;  // a column quarter
   const _Float16* a = (const _Float16*)A;

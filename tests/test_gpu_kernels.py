@@ -812,6 +812,12 @@ def test_b2b_gemm_rowmajor(core, G, M, N, K, P):
     (0, 1, 256, 32),            # one row, one k chunk
     (3, 257, 384, 96),          # batched; 96 columns per quarter
     (45, 64, 256, 128),         # more problems than one launch takes
+    (0, 256, 256, 32),          # whole 256 x 256 tiles: the tile kernel; one k chunk
+    (0, 256, 512, 96),          # fewer chunks than LDS stages
+    (2, 512, 256, 160),         # batched; one chunk more than stages
+    (0, 768, 1024, 1056),       # many chunks
+    (0, 700, 512, 288),         # the tile kernel with a ragged last row block
+    (3, 130, 256, 64),          # ... batched, fewer rows than one wave's share of a tile
 ])
 def test_gemm_f16(core, G, M, N, K):
     rng = np.random.default_rng(4)
