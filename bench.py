@@ -562,7 +562,7 @@ def bench_windowed_attention(torch, core, steps, warmup, cpu):
 
 
 def bench_gemm(torch, core, steps, warmup, cpu):
-    """The plain fp16 product that the streaming kernels are built around, on its own: 8192^3, beside torch.mm."""
+    """The plain fp16 product (ftk_gemm_f16) on its own: 8192^3, beside torch.mm."""
     M = N = K = 8192
     gen = torch.Generator(device='cpu').manual_seed(1234)
     A = (torch.randn((M, K), generator=gen) / K ** 0.5).half().cuda()
@@ -577,7 +577,7 @@ def bench_gemm(torch, core, steps, warmup, cpu):
         'config': {'workload': 'plain GEMM building block (ftk_gemm_f16), row-major A, B, C', 'M': M, 'N': N, 'K': K, 'accumulate': 'f32'},
         'roofline': {'bound': 'mfma', 'achieved': flop / ms / 1e9, 'peak': PEAK_F16_TFLOPS, 'unit': 'TFLOP/s',
                      'frac': flop / ms / 1e9 / PEAK_F16_TFLOPS, 'traffic': MEASURED_TRAFFIC_BYTES.get('gemm_8192'),
-                     'kernel': 'lstm_cell_f16_kernel<false, 8, false, true>'},
+                     'kernel': 'gemm_f16_tile_kernel'},
         'torch_mm': {'ms_per_step': ms_t, 'tflops': flop / ms_t / 1e9,
                      'max_rel_diff': float((C.float() - ref.float()).abs().max() / ref.float().abs().max())},
     }

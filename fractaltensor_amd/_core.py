@@ -501,6 +501,7 @@ def gemm(A, B, out: Optional[torch.Tensor] = None) -> torch.Tensor:
     C = out if out is not None else torch.empty((*A.shape[:-1], N), dtype=f16, device=A.device)
     _req_out(C, f16, (*A.shape[:-1], N), 'C')
     ci = ctypes.c_int
+    _count('gemm')
     if batched:
         _check(lib.ftk_batched_gemm_f16(_ptr(A), _ptr(B), _ptr(C), ci(G), ci(M), ci(N), ci(K), _stream()))
     else:

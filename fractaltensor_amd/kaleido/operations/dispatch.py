@@ -51,7 +51,7 @@ from ..tensor import Tensor
 
 enabled = os.environ.get('FTK_DISPATCH', '1') != '0'
 allow_half_attention = False
-stats = {'stacked_lstm': 0, 'dilated_lstm': 0, 'lstm_scan': 0, 'flash_attention': 0, 'b2b_gemm': 0, 'probes': 0, 'declined': 0,
+stats = {'stacked_lstm': 0, 'dilated_lstm': 0, 'lstm_scan': 0, 'flash_attention': 0, 'b2b_gemm': 0, 'gemm': 0, 'probes': 0, 'declined': 0,
          'weight_cache_hits': 0, 'repeated_on_f32_products': 0}
 
 _verdicts: dict = {}
@@ -871,6 +871,25 @@ def _b2b_candidate(t: torch.Tensor) -> bool:
     return t is not None and t.is_cuda and t.dtype == torch.float16 and t.dim() == 2 and t.is_contiguous()
 
 
+_cu_count: dict = {}
+
+
+def _try_own_gemm(a: torch.Tensor, b: torch.Tensor):
+    """a @ b through the library's product kernel (ftk_gemm_f16) where it is the faster of the two: N a multiple of 256,
+    K of 32, and at least one 256 x 256 output tile per compute unit; NotImplemented (torch's product) otherwise."""
+    M, K = a.shape
+    N = b.shape[1]
+    if N % 256 or K % 32 or M < 1:
+        return NotImplemented
+    dev = a.device.index if a.device.index is not None else torch.cuda.current_device()
+    if dev not in _cu_count:
+        _cu_count[dev] = torch.cuda.get_device_properties(dev).multi_processor_count
+    if -(-M // 256) * (N // 256) < _cu_count[dev]:
+        return NotImplemented
+    stats['gemm'] += 1
+    return Tensor.from_tensor(_core().gemm(a, b))
+
+
 def try_mm(x, y):
     """x @ y: the fused back-to-back GEMM when x is a pending a @ b, a pending product when x @ y could be the
     first half of one, NotImplemented otherwise."""
@@ -896,7 +915,7 @@ def try_mm(x, y):
     if not (_b2b_candidate(a) and _b2b_candidate(b)) or a.shape[1] != b.shape[0]:
         return NotImplemented
     if a.shape[1] not in (32, 64, 96, 128) or b.shape[1] % 32 or a.shape[0] < 32:
-        return NotImplemented                           # not a first product the fused kernels take
+        return _try_own_gemm(a, b)                      # not a first product the fused kernels take
     if not _core().b2b_gemm_supported(b.shape[1], a.shape[1], 32):
         return NotImplemented                           # N beyond what any of the kernels holds (whatever P turns out to be)
     return Tensor.pending_product(a, b)

@@ -219,8 +219,9 @@ def b2b_gemm(a, b, c):
 
 def mm(a: Tensor, b: Tensor) -> Tensor:
     """a @ b for fp16 Tensors on the GPU through the library's own MFMA product (ftk_gemm_f16): a [M,K], b [K,N],
-    N a multiple of 128, K of 32.  `ops.mm` itself stays with torch (hipBLASLt), which is the faster of the two
-    for a plain product; this is the building block the fused kernels are made of, callable on its own."""
+    N a multiple of 128, K of 32, whatever the size.  `ops.mm` routes a product here by itself when it is large enough
+    for this kernel to be the faster one (N a multiple of 256 and a 256 x 256 tile per compute unit) and leaves the
+    rest with torch; this calls it on any shape the kernel takes."""
     for x, name in ((a, 'a'), (b, 'b')):
         if not isinstance(x, Tensor):
             raise TypeError(f'{name} should be a Tensor.')

@@ -84,7 +84,7 @@ def cross_entropy(x, y):
 # ---- contractions and broadcasts ------------------------------------------------
 
 def mm(x, y):
-    routed = dispatch.try_mm(x, y)       # (a @ b) @ c on fp16 GPU tensors: one back-to-back GEMM
+    routed = dispatch.try_mm(x, y)       # fp16 GPU tensors: (a @ b) @ c as one back-to-back GEMM; a large a @ b on ftk_gemm_f16
     if routed is not NotImplemented:
         return routed
     require_tensor(x, 'x'); require_tensor(y, 'y')

@@ -423,10 +423,11 @@ int ftk_b2b_gemm_rowmajor_f16(const void* A, const void* B, const void* C,
 /*
  * C = A @ B, fp16 storage, fp32 accumulation, every operand row-major:
  * A [M,K], B [K,N], C [M,N]; the batched form takes G independent problems
- * A [G,M,K], B [G,K,N], C [G,M,N].  Needs N%128==0, K%32==0.  The product of
- * the streaming LSTM cell kernel without the cell (256 rows x 256 columns per
- * workgroup, k chunks of 32 through a ring of LDS stages, B transposed between
- * LDS and the matrix unit), offered as a building block.  Stands in for
+ * A [G,M,K], B [G,K,N], C [G,M,N].  Needs N%128==0, K%32==0.  N%256==0 runs
+ * on a kernel built for the product (256 x 256 outputs per workgroup, one wave
+ * per SIMD with 128 x 128 of them, k chunks of 32 through four LDS stages, B
+ * transposed between LDS and the matrix unit; any M); other widths on the
+ * streaming LSTM cell kernel without the cell.  Stands in for
  * KeCuteGemm / KeBatchedCuteGemm / KeGemmPipelined
  * (kaleido/core/device/kernels/cutlass_wmma.h:116,186,259; functors CuteGemm,
  * GemmPipelined gemm.h:152,201 and batched_gemm.h:84) behind ops.mm (MatMul,

@@ -572,6 +572,27 @@ def test_chained_matmul_beyond_the_fused_kernels_runs_as_two_products():
     assert ko.max_rel_err(d2.data.float().cpu().numpy(), ref) <= 1e-2
 
 
+def test_a_large_plain_product_runs_on_the_library_kernel():
+    """ops.mm on fp16 GPU operands: the library's product kernel when there is a 256 x 256 tile for every compute unit
+    (N % 256 == 0, K % 32 == 0), torch's otherwise; the same values either way."""
+    core = _core()
+    rng = np.random.default_rng(53)
+    M, K, N = 4000, 160, 4096                       # 16 x 16 tiles, the last row block ragged
+    a = torch.from_numpy((rng.standard_normal((M, K)) / np.sqrt(K)).astype(np.float16)).cuda()
+    b = torch.from_numpy(rng.standard_normal((K, N)).astype(np.float16)).cuda()
+    before = core.launch_counts.get('gemm', 0)
+    d = Tensor.from_tensor(a) @ Tensor.from_tensor(b)
+    assert dispatch.stats['gemm'] == 1 and core.launch_counts.get('gemm', 0) == before + 1
+    ref = a.double() @ b.double()
+    assert d.shape == (M, N) and d.data.dtype == torch.float16
+    assert float((d.data.double() - ref).abs().max() / ref.abs().max()) <= 1e-3
+    assert float((d.data == ref.half()).float().mean()) > 0.98        # fp32 sums of exact products, rounded once
+    # few tiles, a width that is no multiple of 256, fp32 operands: torch's product, bit for bit
+    for aa, bb in ((a[:512].contiguous(), b), (a, b[:, :4000].contiguous()), (a.float(), b.float())):
+        d = Tensor.from_tensor(aa) @ Tensor.from_tensor(bb)
+        assert dispatch.stats['gemm'] == 1 and torch.equal(d.data, aa @ bb)
+
+
 def test_a_pending_product_is_formed_by_any_other_use():
     rng = np.random.default_rng(51)
     a, b = (torch.from_numpy((rng.standard_normal(s) / 8).astype(np.float16)).cuda() for s in ((64, 64), (64, 96)))
