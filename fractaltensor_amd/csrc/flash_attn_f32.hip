@@ -8,15 +8,19 @@
 // top * top in one accumulator, top * rest and rest * top in a second one that is folded in with 2^-11;
 // rest * rest, 2^-22 of a product, is dropped.  What shares a power-of-two scale 2^e (its largest magnitude
 // lands in [2^14, 2^15)): a row of Q, all of K of one (batch, head), all of V of one (batch, head), and the
-// fixed 2^14 for the softmax weights p in [0, 1].  An element keeps 22 significant bits of its own as long as it
-// is within 2^-28 of its group's largest; smaller ones lose bits, of products that are that much smaller too.
+// fixed 2^7 for the softmax weights p in [0, 2^8).  An element keeps 22 significant bits of its own as long as it
+// is within 2^-28 of its group's largest (a weight: down to 2^-21, and an absolute 2^-43 below that, the remainder
+// plane holding what the value plane's subnormals drop); smaller ones lose bits, of products that are that much
+// smaller too.
 //
 // Three launches: the largest |K| and |V| per (batch, head); the split of Q (times scale * log2 e), K and V into
 // planes [row][top D | rest D] in the workspace; the attention kernel.  A plane row is an fp16 row of 2 D
 // elements, so tiles, copies and fragment reads are those of the fp16 kernel at twice the head dimension
 // (fa_common.h), and the contractions are its transposed ones: S^T = K Q^T, O^T += V^T P^T, a lane owns one query
-// row, the running maximum and sum are lane-local.  The maximum is tracked per 32-key half tile, exactly (fp32
-// results leave no room for the fp16 kernel's lazily moved reference).
+// row, the running maximum and sum are lane-local.  The reference that the weights are taken against follows the
+// running maximum lazily: it moves only when a score exceeds it by more than 8 bits (kLazyBits), so weights reach
+// 2^8 at most and O's accumulators, 256 registers behind the matrix unit, are rescaled once per row block on
+// ordinary data rather than whenever one of a wave's 32 rows finds a new maximum (every other half tile).
 #include <algorithm>
 #include <type_traits>
 
@@ -26,7 +30,10 @@ namespace ftk {
 
 constexpr int kF32Top = 14;             // a scale group's largest magnitude lands in [2^14, 2^15)
 constexpr float kF32Rest = 2048.0f;     // 2^11
-constexpr float kF32P = 16384.0f;       // 2^14: the scale of the softmax weights
+constexpr float kF32P = 128.0f;         // 2^7: the scale of the softmax weights in their fp16 planes
+constexpr float kLazyBits = 7.99f;      // how far a score may exceed the softmax reference: weights below 2^8, below 65504 in their plane
+// s_waitcnt immediate: at most n vector memory operations outstanding (n < 64), the other counters left alone
+constexpr int vmcnt_at_most(int n) { return 0x0F70 | (n & 15) | ((n >> 4) << 14); }
 
 // the power of two that brings a largest magnitude with these float bits into [2^14, 2^15), and its inverse
 __device__ __forceinline__ void split_scale(unsigned max_bits, float* scale, float* inv) {
@@ -43,15 +50,23 @@ __global__ void attn_f32_clear_kernel(unsigned* p, int n) {
 // largest |x| of every (batch, head) of K and V, as float bits (which order like the magnitudes): grid
 // (chunks, BH, 2), per_bh a multiple of 4
 __global__ __launch_bounds__(256) void attn_f32_absmax_kernel(const float* K, const float* V, unsigned* bits, size_t per_bh, int BH) {
+  __shared__ unsigned wave_max[4];
   const float* x = (blockIdx.z ? V : K) + (size_t)blockIdx.y * per_bh;
   unsigned m = 0;
+#pragma unroll 4
   for (size_t i = ((size_t)blockIdx.x * 256 + threadIdx.x) * 4; i < per_bh; i += (size_t)gridDim.x * 1024) {
     const float4 v = *reinterpret_cast<const float4*>(x + i);
     m = max(max(m, __float_as_uint(fabsf(v.x))), max(__float_as_uint(fabsf(v.y)), max(__float_as_uint(fabsf(v.z)), __float_as_uint(fabsf(v.w)))));
   }
 #pragma unroll
   for (int o = 32; o > 0; o >>= 1) m = max(m, (unsigned)__shfl_xor((int)m, o));
-  if ((threadIdx.x & 63) == 0 && m) atomicMax(bits + blockIdx.z * BH + blockIdx.y, m);
+  if ((threadIdx.x & 63) == 0) wave_max[threadIdx.x >> 6] = m;
+  __syncthreads();
+  // one atomic per workgroup: thousands of them on one word take longer than the reading
+  if (threadIdx.x == 0) {
+    m = max(max(wave_max[0], wave_max[1]), max(wave_max[2], wave_max[3]));
+    if (m) atomicMax(bits + blockIdx.z * BH + blockIdx.y, m);
+  }
 }
 
 // One wave per row of D floats: planes [top D | rest D] of the row times `mul`, under the row's own scale
@@ -165,7 +180,7 @@ __global__ __launch_bounds__(256, 1) void flash_attn_f32_kernel(const _Float16* 
     const int row = min(x / VRS, FA_KT - 1), col = x % VRS;
     v_src[i] = row * RB + (col < RB ? col : 0);
   }
-  auto copy_tile = [&](int kt, int buf) __attribute__((always_inline)) {
+  auto copy_k = [&](int kt, int buf) __attribute__((always_inline)) {
     const int key0 = kt * FA_KT;
     const bool tail = key0 + FA_KT > Skv;   // rows past the end re-read the last key; their scores are masked
     static_for<KCP>([&](auto i_c) __attribute__((always_inline)) {
@@ -179,6 +194,10 @@ __global__ __launch_bounds__(256, 1) void flash_attn_f32_kernel(const _Float16* 
         lds_dma16(Kg + (size_t)key0 * (2 * D), off, Kb + buf * KTB + 1024 * (wave + WAVES * i));
       }
     });
+  };
+  auto copy_v = [&](int kt, int buf) __attribute__((always_inline)) {
+    const int key0 = kt * FA_KT;
+    const bool tail = key0 + FA_KT > Skv;
     static_for<VCP>([&](auto i_c) __attribute__((always_inline)) {
       constexpr int i = decltype(i_c)::value;
       if (wave + WAVES * i < VTB / 1024) {
@@ -191,6 +210,8 @@ __global__ __launch_bounds__(256, 1) void flash_attn_f32_kernel(const _Float16* 
       }
     });
   };
+  // every wave issues at least this many copies of a K tile, of a V tile (wave 0 may issue one more)
+  constexpr int KC_MIN = KTB / 1024 / WAVES, VC_MIN = VTB / 1024 / WAVES;
 
   const int k_lane = j * KRS + 16 * hh;
   const int v_lane = (4 * hh + ((lane & 15) >> 2)) * VRS + 32 * ((lane >> 4) & 1) + 8 * (lane & 3);
@@ -205,76 +226,183 @@ __global__ __launch_bounds__(256, 1) void flash_attn_f32_kernel(const _Float16* 
     return __builtin_bit_cast(v8h, both);
   };
 
-  const int ntiles = (Skv + FA_KT - 1) / FA_KT;
-  copy_tile(0, 0);
-  __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
-  __syncthreads();
+  const v16f zero16 = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+  // The scores of 32 keys (one half of a tile): value x value, and the two mixed products at 2^-11.  A step's K
+  // fragments are requested two steps ahead, behind the first MFMA of the step (three sets of registers in turn).
+  // (the two mixed products have a chain of accumulators each: an MFMA that adds to the result of the one before it waits for it)
+  auto scores = [&](const unsigned char* kbase, v16f& am, v16f& ar, v16f& a2) __attribute__((always_inline)) {
+    v8h kf_t[3], kf_r[3];
+#pragma unroll
+    for (int s = 0; s < 2; ++s) {
+      kf_t[s] = *reinterpret_cast<const v8h*>(kbase + 32 * s);
+      kf_r[s] = *reinterpret_cast<const v8h*>(kbase + 2 * D + 32 * s);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    static_for<DS>([&](auto s_c) __attribute__((always_inline)) {
+      constexpr int s = decltype(s_c)::value, b = s % 3;
+      am = __builtin_amdgcn_mfma_f32_32x32x16_f16(kf_t[b], qt[s], s == 0 ? zero16 : am, 0, 0, 0);
+      __builtin_amdgcn_sched_barrier(0);
+      if constexpr (s + 2 < DS) {
+        kf_t[(s + 2) % 3] = *reinterpret_cast<const v8h*>(kbase + 32 * (s + 2));
+        kf_r[(s + 2) % 3] = *reinterpret_cast<const v8h*>(kbase + 2 * D + 32 * (s + 2));
+        __builtin_amdgcn_sched_barrier(0);
+      }
+      ar = __builtin_amdgcn_mfma_f32_32x32x16_f16(kf_t[b], qr[s], s == 0 ? zero16 : ar, 0, 0, 0);
+      a2 = __builtin_amdgcn_mfma_f32_32x32x16_f16(kf_r[b], qt[s], s == 0 ? zero16 : a2, 0, 0, 0);
+      __builtin_amdgcn_sched_barrier(0);
+    });
+  };
 
-  for (int kt = 0; kt < ntiles; ++kt) {
-    const int buf = kt & 1;
-    if (kt + 1 < ntiles) copy_tile(kt + 1, buf ^ 1);   // its buffers were last read before the barrier that ended tile kt - 1
+  // The softmax of one half's scores, dealt out over the MFMAs of the P V product of the half BEFORE (HAS_PV; weights
+  // ppt / ppr, V rows at pvbase): the one wave of a SIMD has nothing else to put beside its vector instructions.
+  // Slot i holds MFMA i of the product and a share of the softmax: the first third of the slots the scores and their
+  // maximum, the rest the weights.  V fragments of a group (key step, d tile: 3 MFMAs) are requested two groups ahead.
+  // HAS_SM false: the product alone (behind the last half).
+  float alpha = 1.0f;
+  auto weights_and_pv = [&](auto has_pv_c, auto has_sm_c, const unsigned char* pvbase, const v8h (&ppt)[2], const v8h (&ppr)[2],
+                            const v16f& am, const v16f& ar, const v16f& a2, int key0, v8h (&npt)[2], v8h (&npr)[2]) __attribute__((always_inline)) {
+    constexpr bool HAS_PV = decltype(has_pv_c)::value, HAS_SM = decltype(has_sm_c)::value;
+    constexpr int NG = 2 * DT, NM = 3 * NG, N1 = NM / 3, N2 = NM - N1;
+    // groups are taken two at a time, their six MFMAs in an order in which none adds to the result of the one before
+    // it (two d tiles; at D = 32, with its one d tile, the two key steps)
+    v8h vf_t[4], vf_r[4];
+    if constexpr (HAS_PV) {
 #pragma unroll
-    for (int half = 0; half < 2; ++half) {
-      const int key0 = kt * FA_KT + 32 * half;
-      if (key0 >= Skv) break;
-      const unsigned char* kbase = Kb + buf * KTB + k_lane + 32 * half * KRS;
-      const unsigned char* vbase = Vb + buf * VTB + v_lane + 32 * half * VRS;
-      // scores of 32 keys: value x value, and the two mixed products at 2^-11
-      v16f am, ar;
-#pragma unroll
-      for (int r = 0; r < 16; ++r) { am[r] = 0.0f; ar[r] = 0.0f; }
-#pragma unroll
-      for (int s = 0; s < DS; ++s) {
-        const v8h kt_ = *reinterpret_cast<const v8h*>(kbase + 32 * s);
-        const v8h kr_ = *reinterpret_cast<const v8h*>(kbase + 2 * D + 32 * s);
-        am = __builtin_amdgcn_mfma_f32_32x32x16_f16(kt_, qt[s], am, 0, 0, 0);
-        ar = __builtin_amdgcn_mfma_f32_32x32x16_f16(kt_, qr[s], ar, 0, 0, 0);
-        ar = __builtin_amdgcn_mfma_f32_32x32x16_f16(kr_, qt[s], ar, 0, 0, 0);
+      for (int g = 0; g < 2; ++g) {
+        vf_t[g] = read_v(pvbase, g / DT, g % DT, 0);
+        vf_r[g] = read_v(pvbase, g / DT, g % DT, 1);
       }
-      float sc[16];
-      float mx = -INFINITY;
-#pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        sc[r] = (am[r] + (1.0f / kF32Rest) * ar[r]) * s_mul;
-        if (key0 + 8 * (r >> 2) + 4 * hh + (r & 3) >= Skv) sc[r] = -INFINITY;
-        mx = fmaxf(mx, sc[r]);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    float sc[16];
+    float mx = -INFINITY, m_new = 0.0f, lsum = 0.0f;
+    unsigned nptu[8], npru[8];
+    static_for<NM>([&](auto i_c) __attribute__((always_inline)) {
+      constexpr int i = decltype(i_c)::value, pair = i / 6, k = i % 6, g0 = 2 * pair, g1 = g0 + 1;
+      constexpr int b0 = (pair & 1) * 2, b1 = b0 + 1, nb = ((pair + 1) & 1) * 2;
+      constexpr int sk0 = g0 / DT, dt0 = g0 % DT, sk1 = g1 / DT, dt1 = g1 % DT;
+      if constexpr (HAS_PV) {
+        if constexpr ((k == 1 || k == 3) && g0 + 2 < NG) {   // the next pair's fragments
+          constexpr int g = g0 + 2 + (k == 3);
+          vf_t[nb + (k == 3)] = read_v(pvbase, g / DT, g % DT, 0);
+          vf_r[nb + (k == 3)] = read_v(pvbase, g / DT, g % DT, 1);
+        }
+        if constexpr (k == 0) om[dt0] = __builtin_amdgcn_mfma_f32_32x32x16_f16(vf_t[b0], ppt[sk0], om[dt0], 0, 0, 0);
+        if constexpr (k == 1) oc[dt0] = __builtin_amdgcn_mfma_f32_32x32x16_f16(vf_t[b0], ppr[sk0], oc[dt0], 0, 0, 0);
+        if constexpr (k == 2) om[dt1] = __builtin_amdgcn_mfma_f32_32x32x16_f16(vf_t[b1], ppt[sk1], om[dt1], 0, 0, 0);
+        if constexpr (k == 3) oc[dt1] = __builtin_amdgcn_mfma_f32_32x32x16_f16(vf_t[b1], ppr[sk1], oc[dt1], 0, 0, 0);
+        if constexpr (k == 4) oc[dt0] = __builtin_amdgcn_mfma_f32_32x32x16_f16(vf_r[b0], ppt[sk0], oc[dt0], 0, 0, 0);
+        if constexpr (k == 5) oc[dt1] = __builtin_amdgcn_mfma_f32_32x32x16_f16(vf_r[b1], ppt[sk1], oc[dt1], 0, 0, 0);
       }
-      mx = max_with_other_half(mx);
-      const float m_new = fmaxf(m_run, mx);   // finite: the half holds at least one key
-      const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);   // 0 the first time (m_run = -inf)
-      m_run = m_new;
-      float lsum = 0.0f;
-      v8h pt[2], pr[2];
+      if constexpr (HAS_SM) {
+        if constexpr (i < N1) {
 #pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        const float p = __builtin_amdgcn_exp2f(sc[r] - m_new);
-        lsum += p;
-        const float ps = p * kF32P;
-        const _Float16 top = (_Float16)ps;
-        pt[r >> 3][r & 7] = top;
-        pr[r >> 3][r & 7] = (_Float16)((ps - (float)top) * kF32Rest);
+          for (int r = 16 * i / N1; r < 16 * (i + 1) / N1; ++r) {
+            sc[r] = (am[r] + (1.0f / kF32Rest) * (ar[r] + a2[r])) * s_mul;
+            if (key0 + 8 * (r >> 2) + 4 * hh + (r & 3) >= Skv) sc[r] = -INFINITY;
+            mx = fmaxf(mx, sc[r]);
+          }
+        } else {
+          if constexpr (i == N1) {
+            // the reference that the weights are taken against follows the running maximum lazily: it moves only when
+            // a score exceeds it by more than kLazyBits, so a weight is at most 2^kLazyBits and O is rescaled rarely
+            mx = max_with_other_half(mx);   // finite: the half holds at least one key
+            const bool moves = mx > m_run + kLazyBits;
+            m_new = moves ? mx : m_run;
+            alpha = moves ? __builtin_amdgcn_exp2f(m_run - m_new) : 1.0f;   // 0 the first time (m_run = -inf)
+            m_run = m_new;
+          }
+          // weights in pairs: two fp16 values share a register of their plane
+#pragma unroll
+          for (int k = 8 * (i - N1) / N2; k < 8 * (i - N1 + 1) / N2; ++k) {
+            const float p0 = __builtin_amdgcn_exp2f(sc[2 * k] - m_new), p1 = __builtin_amdgcn_exp2f(sc[2 * k + 1] - m_new);
+            lsum += p0 + p1;
+            const float s0 = p0 * kF32P, s1 = p1 * kF32P;
+            const v2h top = {(_Float16)s0, (_Float16)s1};
+            const v2h rest = {(_Float16)((s0 - (float)top[0]) * kF32Rest), (_Float16)((s1 - (float)top[1]) * kF32Rest)};
+            unsigned tu = __builtin_bit_cast(unsigned, top), ru = __builtin_bit_cast(unsigned, rest);
+            // pinned to this slot: left alone, the compiler moves the arithmetic to where the weights are next read,
+            // behind the barrier and out from under the MFMAs
+            asm volatile("" : "+v"(tu), "+v"(ru), "+v"(lsum));
+            nptu[k] = tu;
+            npru[k] = ru;
+          }
+        }
+      }
+      __builtin_amdgcn_sched_barrier(0);
+    });
+    if constexpr (HAS_SM) {
+#pragma unroll
+      for (int h = 0; h < 2; ++h) {
+        npt[h] = __builtin_bit_cast(v8h, v4u{nptu[4 * h], nptu[4 * h + 1], nptu[4 * h + 2], nptu[4 * h + 3]});
+        npr[h] = __builtin_bit_cast(v8h, v4u{npru[4 * h], npru[4 * h + 1], npru[4 * h + 2], npru[4 * h + 3]});
       }
       l_run = l_run * alpha + lsum;
+      // (the product above belongs to the half before: it is in O before O is brought to this half's maximum)
       if (__builtin_amdgcn_ballot_w64(alpha != 1.0f) != 0) {
 #pragma unroll
         for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
           for (int r = 0; r < 16; ++r) { om[dt][r] *= alpha; oc[dt][r] *= alpha; }
       }
-#pragma unroll
-      for (int s = 0; s < 2; ++s)
-#pragma unroll
-        for (int dt = 0; dt < DT; ++dt) {
-          const v8h vt_ = read_v(vbase, s, dt, 0);
-          const v8h vr_ = read_v(vbase, s, dt, 1);
-          om[dt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(vt_, pt[s], om[dt], 0, 0, 0);
-          oc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(vt_, pr[s], oc[dt], 0, 0, 0);
-          oc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(vr_, pt[s], oc[dt], 0, 0, 0);
-        }
     }
-    __builtin_amdgcn_s_waitcnt(0x0F70);  // this wave's copies of tile kt + 1 have landed
+  };
+
+  // A tile's K rows are last read by the scores of its second half and its V rows one half later, beside the next
+  // tile's first softmax: K of tile kt + 1 is requested when tile kt begins, V of tile kt + 1 behind the barrier in
+  // the middle of tile kt.  Copies complete in the order of their issue, so each of the two barriers waits for the
+  // older of the two requests only.
+  const int ntiles = (Skv + FA_KT - 1) / FA_KT;
+  copy_k(0, 0);
+  copy_v(0, 0);
+  __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
+  __syncthreads();
+
+  // the weights of the half whose P V product is still to come, and its V rows (in front of the first half: weights
+  // of zero on the first tile's rows)
+  v8h pt[2], pr[2];
+#pragma unroll
+  for (int s = 0; s < 2; ++s)
+#pragma unroll
+    for (int e = 0; e < 8; ++e) { pt[s][e] = (_Float16)0.0f; pr[s][e] = (_Float16)0.0f; }
+  const unsigned char* pend_v = Vb + v_lane;
+  for (int kt = 0; kt < ntiles; ++kt) {
+    const int buf = kt & 1;
+    const bool more = kt + 1 < ntiles;
+    if (more) copy_k(kt + 1, buf ^ 1);   // K[buf ^ 1] was last read before the barrier that ended tile kt - 1
+    {   // first half
+      v16f am, ar, a2;
+      scores(Kb + buf * KTB + k_lane, am, ar, a2);
+      v8h npt[2], npr[2];
+      weights_and_pv(std::true_type{}, std::true_type{}, pend_v, pt, pr, am, ar, a2, kt * FA_KT, npt, npr);
+#pragma unroll
+      for (int s = 0; s < 2; ++s) { pt[s] = npt[s]; pr[s] = npr[s]; }
+      pend_v = Vb + buf * VTB + v_lane;
+    }
+    // V of tile kt has landed in every wave (asked for half a tile ago or more); V[buf ^ 1] has been read for the last time
+    if (more) __builtin_amdgcn_s_waitcnt(vmcnt_at_most(KC_MIN));
+    else __builtin_amdgcn_s_waitcnt(0x0F70);
+    __syncthreads();
+    if (more) copy_v(kt + 1, buf ^ 1);
+    if (kt * FA_KT + 32 < Skv) {   // second half
+      v16f am, ar, a2;
+      scores(Kb + buf * KTB + k_lane + 32 * KRS, am, ar, a2);
+      v8h npt[2], npr[2];
+      weights_and_pv(std::true_type{}, std::true_type{}, pend_v, pt, pr, am, ar, a2, kt * FA_KT + 32, npt, npr);
+#pragma unroll
+      for (int s = 0; s < 2; ++s) { pt[s] = npt[s]; pr[s] = npr[s]; }
+      pend_v = Vb + buf * VTB + v_lane + 32 * VRS;
+    }
+    // K of tile kt + 1 has landed; K[buf] has been read for the last time
+    if (more) __builtin_amdgcn_s_waitcnt(vmcnt_at_most(VC_MIN));
     __syncthreads();
   }
+  {   // the last half's product
+    const v16f none = zero16;
+    v8h npt[2], npr[2];
+    weights_and_pv(std::true_type{}, std::false_type{}, pend_v, pt, pr, none, none, none, 0, npt, npr);
+  }
+  __syncthreads();   // LDS is reused below
 
   // ---- normalise and store: the wave turns its 32 x D tile round through the LDS nobody reads any more (the
   // barrier above ended the last tile), so that whole rows leave as consecutive bytes
@@ -334,7 +462,7 @@ static int launch_fa_f32(const float* Q, const float* K, const float* V, float* 
   int rc = check_launch("attn_f32_clear_kernel");
   if (rc) return rc;
   const size_t per_bh = (size_t)Skv * D;
-  const int chunks = (int)std::min<size_t>(64, (per_bh + 4095) / 4096);
+  const int chunks = (int)std::min<size_t>(std::max(1, 4096 / (2 * BH)), (per_bh + 4095) / 4096);   // some 4096 workgroups in all
   hipLaunchKernelGGL(attn_f32_absmax_kernel, dim3(chunks, BH, 2), dim3(256), 0, s, K, V, bits, per_bh, BH);
   rc = check_launch("attn_f32_absmax_kernel");
   if (rc) return rc;
