@@ -30,7 +30,7 @@ namespace ftk {
 
 constexpr int kF32Top = 14;             // a scale group's largest magnitude lands in [2^14, 2^15)
 constexpr float kF32Rest = 2048.0f;     // 2^11
-constexpr float kF32P = 128.0f;         // 2^7: the scale of the softmax weights in their fp16 planes
+constexpr float kF32PBits = 7.0f;        // 2^7: the scale of the softmax weights in their fp16 planes
 constexpr float kLazyBits = 7.99f;      // how far a score may exceed the softmax reference: weights below 2^8, below 65504 in their plane
 // s_waitcnt immediate: at most n vector memory operations outstanding (n < 64), the other counters left alone
 constexpr int vmcnt_at_most(int n) { return 0x0F70 | (n & 15) | ((n >> 4) << 14); }
@@ -110,9 +110,10 @@ __global__ __launch_bounds__(256) void attn_f32_split_kernel(const float* X, _Fl
 }
 
 // 4 waves x 32 query rows per workgroup, one workgroup per compute unit (the accumulators of O, both planes of Q
-// and the scores take more than 256 registers at D = 128).  K and V tiles of 64 keys, both double buffered; the
-// tile after the current one is requested when the current one's products begin and waited for at the barrier
-// that ends them.
+// and the scores take more than 256 registers at D = 128).  K and V tiles of 64 keys, both double buffered.  A wave
+// works through the tiles in halves of 32 keys, and with one wave per SIMD the softmax of a half has no other
+// wave's MFMAs to run beside: it is cut in two, the maxima under the P V MFMAs of the half before and the weights
+// under the score MFMAs of the half after (the comments in the kernel give the order).
 template <int D>
 __global__ __launch_bounds__(256, 1) void flash_attn_f32_kernel(const _Float16* __restrict__ Qp, const _Float16* __restrict__ Kp,
                                                                 const _Float16* __restrict__ Vp, const float* __restrict__ q_inv,
@@ -164,7 +165,6 @@ __global__ __launch_bounds__(256, 1) void flash_attn_f32_kernel(const _Float16* 
   for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
     for (int r = 0; r < 16; ++r) { om[dt][r] = 0.0f; oc[dt][r] = 0.0f; }
-  float m_run = -INFINITY, l_run = 0.0f;
 
   // copies: as in the fp16 kernel, copy c of a tile fills LDS bytes [1024 c, 1024 c + 1024) of the padded tile
   unsigned k_src[KCP], v_src[VCP];
@@ -180,35 +180,34 @@ __global__ __launch_bounds__(256, 1) void flash_attn_f32_kernel(const _Float16* 
     const int row = min(x / VRS, FA_KT - 1), col = x % VRS;
     v_src[i] = row * RB + (col < RB ? col : 0);
   }
-  auto copy_k = [&](int kt, int buf) __attribute__((always_inline)) {
-    const int key0 = kt * FA_KT;
-    const bool tail = key0 + FA_KT > Skv;   // rows past the end re-read the last key; their scores are masked
-    static_for<KCP>([&](auto i_c) __attribute__((always_inline)) {
-      constexpr int i = decltype(i_c)::value;
-      if (wave + WAVES * i < KTB / 1024) {
-        unsigned off = k_src[i];
-        if (tail) {
-          const unsigned last = (unsigned)(Skv - 1 - key0), row = off / RB;
+  // (a whole tile takes the copies' offsets as they are; the last tile of a ragged row of keys clamps each)
+  auto copy_rows = [&](auto n_c, auto bytes_c, const unsigned (&src)[decltype(n_c)::value], const _Float16* rows, int key0,
+                       unsigned char* dst) __attribute__((always_inline)) {
+    constexpr int N = decltype(n_c)::value, COPIES = decltype(bytes_c)::value / 1024;
+    if (key0 + FA_KT <= Skv) {
+      static_for<N>([&](auto i_c) __attribute__((always_inline)) {
+        constexpr int i = decltype(i_c)::value;
+        if (WAVES * i + WAVES - 1 < COPIES || wave + WAVES * i < COPIES) lds_dma16(rows, src[i], dst + 1024 * (wave + WAVES * i));
+      });
+    } else {
+      static_for<N>([&](auto i_c) __attribute__((always_inline)) {
+        constexpr int i = decltype(i_c)::value;
+        if (wave + WAVES * i < COPIES) {
+          unsigned off = src[i];
+          const unsigned last = (unsigned)(Skv - 1 - key0), row = off / RB;   // rows past the end re-read the last key; their scores are masked
           if (row > last) off -= (row - last) * RB;
+          lds_dma16(rows, off, dst + 1024 * (wave + WAVES * i));
         }
-        lds_dma16(Kg + (size_t)key0 * (2 * D), off, Kb + buf * KTB + 1024 * (wave + WAVES * i));
-      }
-    });
+      });
+    }
+  };
+  auto copy_k = [&](int kt, int buf) __attribute__((always_inline)) {
+    copy_rows(std::integral_constant<int, KCP>{}, std::integral_constant<int, KTB>{}, k_src, Kg + (size_t)kt * FA_KT * (2 * D), kt * FA_KT,
+              Kb + buf * KTB);
   };
   auto copy_v = [&](int kt, int buf) __attribute__((always_inline)) {
-    const int key0 = kt * FA_KT;
-    const bool tail = key0 + FA_KT > Skv;
-    static_for<VCP>([&](auto i_c) __attribute__((always_inline)) {
-      constexpr int i = decltype(i_c)::value;
-      if (wave + WAVES * i < VTB / 1024) {
-        unsigned off = v_src[i];
-        if (tail) {
-          const unsigned last = (unsigned)(Skv - 1 - key0), row = off / RB;
-          if (row > last) off -= (row - last) * RB;
-        }
-        lds_dma16(Vg + (size_t)key0 * (2 * D), off, Vb + buf * VTB + 1024 * (wave + WAVES * i));
-      }
-    });
+    copy_rows(std::integral_constant<int, VCP>{}, std::integral_constant<int, VTB>{}, v_src, Vg + (size_t)kt * FA_KT * (2 * D), kt * FA_KT,
+              Vb + buf * VTB);
   };
   // every wave issues at least this many copies of a K tile, of a V tile (wave 0 may issue one more)
   constexpr int KC_MIN = KTB / 1024 / WAVES, VC_MIN = VTB / 1024 / WAVES;
@@ -227,119 +226,141 @@ __global__ __launch_bounds__(256, 1) void flash_attn_f32_kernel(const _Float16* 
   };
 
   const v16f zero16 = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-  // The scores of 32 keys (one half of a tile): value x value, and the two mixed products at 2^-11.  A step's K
-  // fragments are requested two steps ahead, behind the first MFMA of the step (three sets of registers in turn).
-  // (the two mixed products have a chain of accumulators each: an MFMA that adds to the result of the one before it waits for it)
-  auto scores = [&](const unsigned char* kbase, v16f& am, v16f& ar, v16f& a2) __attribute__((always_inline)) {
+  // One wave per SIMD has only its own vector instructions to put beside its MFMAs, so the softmax of a half is cut in
+  // two and each part runs under the MFMAs of another product:
+  //   the scores of half h                  beside  the weights of half h - 1 (exp2, the split into planes)
+  //   the P V product of half h - 1         beside  the raw scores and the maximum of half h
+  // and then the reference moves if it has to (rarely, see kLazyBits) and O is rescaled.
+  //
+  // State between the two: raw[], the scores of the half before in the matrix unit's units (times s_mul: exponent
+  // units), and m_ref, the reference they are taken against; pt / pr, the weights whose product is still to come.
+  float raw[16];
+  float m_ref = -INFINITY, l_run = 0.0f;   // l_run: the sum of the weights, in their planes' scale
+  v8h pt[2], pr[2];
+#pragma unroll
+  for (int s = 0; s < 2; ++s)
+#pragma unroll
+    for (int e = 0; e < 8; ++e) { pt[s][e] = (_Float16)0.0f; pr[s][e] = (_Float16)0.0f; }
+#pragma unroll
+  for (int r = 0; r < 16; ++r) raw[r] = -INFINITY;   // in front of the first half: weights of zero
+
+  // weights of pair k (two neighbouring scores) of the half before: p * 2^7 = exp2(raw * s_mul - m_ref + kF32PBits), its two planes
+  float lsum = 0.0f;
+  unsigned ptu[8], pru[8];
+  auto weight_pair = [&](auto k_c, float bias) __attribute__((always_inline)) {
+    constexpr int k = decltype(k_c)::value;
+    const float s0 = __builtin_amdgcn_exp2f(fmaf(raw[2 * k], s_mul, bias)), s1 = __builtin_amdgcn_exp2f(fmaf(raw[2 * k + 1], s_mul, bias));
+    lsum += s0 + s1;
+    const v2h top = {(_Float16)s0, (_Float16)s1};
+    const v2h rest = {(_Float16)((s0 - (float)top[0]) * kF32Rest), (_Float16)((s1 - (float)top[1]) * kF32Rest)};
+    unsigned tu = __builtin_bit_cast(unsigned, top), ru = __builtin_bit_cast(unsigned, rest);
+    // pinned to its place: left alone, the compiler moves the arithmetic to where the weights are read, out from under the MFMAs
+    asm volatile("" : "+v"(tu), "+v"(ru), "+v"(lsum));
+    ptu[k] = tu;
+    pru[k] = ru;
+  };
+  auto weights_done = [&]() __attribute__((always_inline)) {
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+      pt[h] = __builtin_bit_cast(v8h, v4u{ptu[4 * h], ptu[4 * h + 1], ptu[4 * h + 2], ptu[4 * h + 3]});
+      pr[h] = __builtin_bit_cast(v8h, v4u{pru[4 * h], pru[4 * h + 1], pru[4 * h + 2], pru[4 * h + 3]});
+    }
+    l_run += lsum;
+  };
+
+  // The scores of 32 keys (one half of a tile): value x value in am, the two mixed products, 2^-11 of it, in ar.  A
+  // step's K fragments are requested two steps ahead (three sets of registers in turn).  WEIGHTS: the weights of the
+  // half before are formed beside them, a share with every step.
+  auto scores = [&](auto weights_c, const unsigned char* kbase, v16f& am, v16f& ar) __attribute__((always_inline)) {
+    constexpr bool WEIGHTS = decltype(weights_c)::value;
     v8h kf_t[3], kf_r[3];
 #pragma unroll
     for (int s = 0; s < 2; ++s) {
       kf_t[s] = *reinterpret_cast<const v8h*>(kbase + 32 * s);
       kf_r[s] = *reinterpret_cast<const v8h*>(kbase + 2 * D + 32 * s);
     }
+    // (before the first half there is no reference, and every raw score is -inf: weights of zero)
+    const float bias = m_ref > -INFINITY ? kF32PBits - m_ref : 0.0f;
+    lsum = 0.0f;
     __builtin_amdgcn_sched_barrier(0);
     static_for<DS>([&](auto s_c) __attribute__((always_inline)) {
       constexpr int s = decltype(s_c)::value, b = s % 3;
       am = __builtin_amdgcn_mfma_f32_32x32x16_f16(kf_t[b], qt[s], s == 0 ? zero16 : am, 0, 0, 0);
-      __builtin_amdgcn_sched_barrier(0);
       if constexpr (s + 2 < DS) {
         kf_t[(s + 2) % 3] = *reinterpret_cast<const v8h*>(kbase + 32 * (s + 2));
         kf_r[(s + 2) % 3] = *reinterpret_cast<const v8h*>(kbase + 2 * D + 32 * (s + 2));
-        __builtin_amdgcn_sched_barrier(0);
       }
       ar = __builtin_amdgcn_mfma_f32_32x32x16_f16(kf_t[b], qr[s], s == 0 ? zero16 : ar, 0, 0, 0);
-      a2 = __builtin_amdgcn_mfma_f32_32x32x16_f16(kf_r[b], qt[s], s == 0 ? zero16 : a2, 0, 0, 0);
+      ar = __builtin_amdgcn_mfma_f32_32x32x16_f16(kf_r[b], qt[s], ar, 0, 0, 0);
+      if constexpr (WEIGHTS) {
+        static_for<8 * (s + 1) / DS - 8 * s / DS>([&](auto j_c) __attribute__((always_inline)) {
+          weight_pair(std::integral_constant<int, 8 * s / DS + decltype(j_c)::value>{}, bias);
+        });
+      }
+      // the order within the step: MFMA, the reads, and the vector instructions in three shares behind the three MFMAs
+      // (the first share holds the two exp2, four issue slots each)
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+      __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+      __builtin_amdgcn_sched_group_barrier(0x002, 4, 0);
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+      __builtin_amdgcn_sched_group_barrier(0x002, 6, 0);
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+      __builtin_amdgcn_sched_group_barrier(0x002, 6, 0);
       __builtin_amdgcn_sched_barrier(0);
     });
+    if constexpr (WEIGHTS) weights_done();
   };
 
-  // The softmax of one half's scores, dealt out over the MFMAs of the P V product of the half BEFORE (HAS_PV; weights
-  // ppt / ppr, V rows at pvbase): the one wave of a SIMD has nothing else to put beside its vector instructions.
-  // Slot i holds MFMA i of the product and a share of the softmax: the first third of the slots the scores and their
-  // maximum, the rest the weights.  V fragments of a group (key step, d tile: 3 MFMAs) are requested two groups ahead.
-  // HAS_SM false: the product alone (behind the last half).
-  float alpha = 1.0f;
-  auto weights_and_pv = [&](auto has_pv_c, auto has_sm_c, const unsigned char* pvbase, const v8h (&ppt)[2], const v8h (&ppr)[2],
-                            const v16f& am, const v16f& ar, const v16f& a2, int key0, v8h (&npt)[2], v8h (&npr)[2]) __attribute__((always_inline)) {
-    constexpr bool HAS_PV = decltype(has_pv_c)::value, HAS_SM = decltype(has_sm_c)::value;
-    constexpr int NG = 2 * DT, NM = 3 * NG, N1 = NM / 3, N2 = NM - N1;
-    // groups are taken two at a time, their six MFMAs in an order in which none adds to the result of the one before
-    // it (two d tiles; at D = 32, with its one d tile, the two key steps)
+  // The P V product of the half whose weights are in pt / pr (V rows at pvbase), and beside it (MAXIMA) the raw
+  // scores and the maximum of the half whose products are in am / ar; then the reference moves if a score exceeds it
+  // by more than kLazyBits, and O and the sum are brought to the new one.  Groups (key step, d tile: 3 MFMAs) are
+  // taken two at a time, in an order in which no MFMA adds to the result of the one before it; a pair's V fragments are
+  // requested under the pair before.
+  auto pv_and_maxima = [&](auto maxima_c, const unsigned char* pvbase, const v16f& am, const v16f& ar, int key0) __attribute__((always_inline)) {
+    constexpr bool MAXIMA = decltype(maxima_c)::value;
+    constexpr int NG = 2 * DT, NM = 3 * NG;
     v8h vf_t[4], vf_r[4];
-    if constexpr (HAS_PV) {
 #pragma unroll
-      for (int g = 0; g < 2; ++g) {
-        vf_t[g] = read_v(pvbase, g / DT, g % DT, 0);
-        vf_r[g] = read_v(pvbase, g / DT, g % DT, 1);
-      }
-      __builtin_amdgcn_sched_barrier(0);
+    for (int g = 0; g < 2; ++g) {
+      vf_t[g] = read_v(pvbase, g / DT, g % DT, 0);
+      vf_r[g] = read_v(pvbase, g / DT, g % DT, 1);
     }
-    float sc[16];
-    float mx = -INFINITY, m_new = 0.0f, lsum = 0.0f;
-    unsigned nptu[8], npru[8];
+    __builtin_amdgcn_sched_barrier(0);
+    float mx = -INFINITY;
+    const int lim = Skv - key0 - 4 * hh;   // score r belongs to a key past the end when 8 (r >> 2) + (r & 3) >= lim
     static_for<NM>([&](auto i_c) __attribute__((always_inline)) {
       constexpr int i = decltype(i_c)::value, pair = i / 6, k = i % 6, g0 = 2 * pair, g1 = g0 + 1;
       constexpr int b0 = (pair & 1) * 2, b1 = b0 + 1, nb = ((pair + 1) & 1) * 2;
       constexpr int sk0 = g0 / DT, dt0 = g0 % DT, sk1 = g1 / DT, dt1 = g1 % DT;
-      if constexpr (HAS_PV) {
-        if constexpr ((k == 1 || k == 3) && g0 + 2 < NG) {   // the next pair's fragments
-          constexpr int g = g0 + 2 + (k == 3);
-          vf_t[nb + (k == 3)] = read_v(pvbase, g / DT, g % DT, 0);
-          vf_r[nb + (k == 3)] = read_v(pvbase, g / DT, g % DT, 1);
-        }
-        if constexpr (k == 0) om[dt0] = __builtin_amdgcn_mfma_f32_32x32x16_f16(vf_t[b0], ppt[sk0], om[dt0], 0, 0, 0);
-        if constexpr (k == 1) oc[dt0] = __builtin_amdgcn_mfma_f32_32x32x16_f16(vf_t[b0], ppr[sk0], oc[dt0], 0, 0, 0);
-        if constexpr (k == 2) om[dt1] = __builtin_amdgcn_mfma_f32_32x32x16_f16(vf_t[b1], ppt[sk1], om[dt1], 0, 0, 0);
-        if constexpr (k == 3) oc[dt1] = __builtin_amdgcn_mfma_f32_32x32x16_f16(vf_t[b1], ppr[sk1], oc[dt1], 0, 0, 0);
-        if constexpr (k == 4) oc[dt0] = __builtin_amdgcn_mfma_f32_32x32x16_f16(vf_r[b0], ppt[sk0], oc[dt0], 0, 0, 0);
-        if constexpr (k == 5) oc[dt1] = __builtin_amdgcn_mfma_f32_32x32x16_f16(vf_r[b1], ppt[sk1], oc[dt1], 0, 0, 0);
+      if constexpr ((k == 1 || k == 3) && g0 + 2 < NG) {   // the next pair's fragments
+        constexpr int g = g0 + 2 + (k == 3);
+        vf_t[nb + (k == 3)] = read_v(pvbase, g / DT, g % DT, 0);
+        vf_r[nb + (k == 3)] = read_v(pvbase, g / DT, g % DT, 1);
       }
-      if constexpr (HAS_SM) {
-        if constexpr (i < N1) {
+      if constexpr (k == 0) om[dt0] = __builtin_amdgcn_mfma_f32_32x32x16_f16(vf_t[b0], pt[sk0], om[dt0], 0, 0, 0);
+      if constexpr (k == 1) oc[dt0] = __builtin_amdgcn_mfma_f32_32x32x16_f16(vf_t[b0], pr[sk0], oc[dt0], 0, 0, 0);
+      if constexpr (k == 2) om[dt1] = __builtin_amdgcn_mfma_f32_32x32x16_f16(vf_t[b1], pt[sk1], om[dt1], 0, 0, 0);
+      if constexpr (k == 3) oc[dt1] = __builtin_amdgcn_mfma_f32_32x32x16_f16(vf_t[b1], pr[sk1], oc[dt1], 0, 0, 0);
+      if constexpr (k == 4) oc[dt0] = __builtin_amdgcn_mfma_f32_32x32x16_f16(vf_r[b0], pt[sk0], oc[dt0], 0, 0, 0);
+      if constexpr (k == 5) oc[dt1] = __builtin_amdgcn_mfma_f32_32x32x16_f16(vf_r[b1], pt[sk1], oc[dt1], 0, 0, 0);
+      if constexpr (MAXIMA) {
 #pragma unroll
-          for (int r = 16 * i / N1; r < 16 * (i + 1) / N1; ++r) {
-            sc[r] = (am[r] + (1.0f / kF32Rest) * (ar[r] + a2[r])) * s_mul;
-            if (key0 + 8 * (r >> 2) + 4 * hh + (r & 3) >= Skv) sc[r] = -INFINITY;
-            mx = fmaxf(mx, sc[r]);
-          }
-        } else {
-          if constexpr (i == N1) {
-            // the reference that the weights are taken against follows the running maximum lazily: it moves only when
-            // a score exceeds it by more than kLazyBits, so a weight is at most 2^kLazyBits and O is rescaled rarely
-            mx = max_with_other_half(mx);   // finite: the half holds at least one key
-            const bool moves = mx > m_run + kLazyBits;
-            m_new = moves ? mx : m_run;
-            alpha = moves ? __builtin_amdgcn_exp2f(m_run - m_new) : 1.0f;   // 0 the first time (m_run = -inf)
-            m_run = m_new;
-          }
-          // weights in pairs: two fp16 values share a register of their plane
-#pragma unroll
-          for (int k = 8 * (i - N1) / N2; k < 8 * (i - N1 + 1) / N2; ++k) {
-            const float p0 = __builtin_amdgcn_exp2f(sc[2 * k] - m_new), p1 = __builtin_amdgcn_exp2f(sc[2 * k + 1] - m_new);
-            lsum += p0 + p1;
-            const float s0 = p0 * kF32P, s1 = p1 * kF32P;
-            const v2h top = {(_Float16)s0, (_Float16)s1};
-            const v2h rest = {(_Float16)((s0 - (float)top[0]) * kF32Rest), (_Float16)((s1 - (float)top[1]) * kF32Rest)};
-            unsigned tu = __builtin_bit_cast(unsigned, top), ru = __builtin_bit_cast(unsigned, rest);
-            // pinned to this slot: left alone, the compiler moves the arithmetic to where the weights are next read,
-            // behind the barrier and out from under the MFMAs
-            asm volatile("" : "+v"(tu), "+v"(ru), "+v"(lsum));
-            nptu[k] = tu;
-            npru[k] = ru;
-          }
+        for (int r = 16 * i / NM; r < 16 * (i + 1) / NM; ++r) {
+          raw[r] = fmaf(ar[r], 1.0f / kF32Rest, am[r]);
+          if (8 * (r >> 2) + (r & 3) >= lim) raw[r] = -INFINITY;
+          mx = fmaxf(mx, raw[r]);
         }
       }
       __builtin_amdgcn_sched_barrier(0);
     });
-    if constexpr (HAS_SM) {
-#pragma unroll
-      for (int h = 0; h < 2; ++h) {
-        npt[h] = __builtin_bit_cast(v8h, v4u{nptu[4 * h], nptu[4 * h + 1], nptu[4 * h + 2], nptu[4 * h + 3]});
-        npr[h] = __builtin_bit_cast(v8h, v4u{npru[4 * h], npru[4 * h + 1], npru[4 * h + 2], npru[4 * h + 3]});
-      }
-      l_run = l_run * alpha + lsum;
-      // (the product above belongs to the half before: it is in O before O is brought to this half's maximum)
-      if (__builtin_amdgcn_ballot_w64(alpha != 1.0f) != 0) {
+    if constexpr (MAXIMA) {
+      mx = max_with_other_half(mx) * s_mul;   // finite: the half holds at least one key; s_mul > 0
+      if (__builtin_amdgcn_ballot_w64(mx > m_ref + kLazyBits) != 0) {   // a row of the wave moves its reference
+        const bool moves = mx > m_ref + kLazyBits;
+        const float m_new = moves ? mx : m_ref;
+        const float alpha = moves ? __builtin_amdgcn_exp2f(m_ref - m_new) : 1.0f;   // 0 the first time (m_ref = -inf)
+        m_ref = m_new;
+        l_run *= alpha;
 #pragma unroll
         for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
@@ -349,7 +370,7 @@ __global__ __launch_bounds__(256, 1) void flash_attn_f32_kernel(const _Float16* 
   };
 
   // A tile's K rows are last read by the scores of its second half and its V rows one half later, beside the next
-  // tile's first softmax: K of tile kt + 1 is requested when tile kt begins, V of tile kt + 1 behind the barrier in
+  // tile's first maxima: K of tile kt + 1 is requested when tile kt begins, V of tile kt + 1 behind the barrier in
   // the middle of tile kt.  Copies complete in the order of their issue, so each of the two barriers waits for the
   // older of the two requests only.
   const int ntiles = (Skv + FA_KT - 1) / FA_KT;
@@ -358,25 +379,15 @@ __global__ __launch_bounds__(256, 1) void flash_attn_f32_kernel(const _Float16* 
   __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
   __syncthreads();
 
-  // the weights of the half whose P V product is still to come, and its V rows (in front of the first half: weights
-  // of zero on the first tile's rows)
-  v8h pt[2], pr[2];
-#pragma unroll
-  for (int s = 0; s < 2; ++s)
-#pragma unroll
-    for (int e = 0; e < 8; ++e) { pt[s][e] = (_Float16)0.0f; pr[s][e] = (_Float16)0.0f; }
-  const unsigned char* pend_v = Vb + v_lane;
+  const unsigned char* pend_v = Vb + v_lane;   // the V rows of the half whose product is still to come (first: zero weights on tile 0)
   for (int kt = 0; kt < ntiles; ++kt) {
     const int buf = kt & 1;
     const bool more = kt + 1 < ntiles;
     if (more) copy_k(kt + 1, buf ^ 1);   // K[buf ^ 1] was last read before the barrier that ended tile kt - 1
     {   // first half
-      v16f am, ar, a2;
-      scores(Kb + buf * KTB + k_lane, am, ar, a2);
-      v8h npt[2], npr[2];
-      weights_and_pv(std::true_type{}, std::true_type{}, pend_v, pt, pr, am, ar, a2, kt * FA_KT, npt, npr);
-#pragma unroll
-      for (int s = 0; s < 2; ++s) { pt[s] = npt[s]; pr[s] = npr[s]; }
+      v16f am, ar;
+      scores(std::true_type{}, Kb + buf * KTB + k_lane, am, ar);
+      pv_and_maxima(std::true_type{}, pend_v, am, ar, kt * FA_KT);
       pend_v = Vb + buf * VTB + v_lane;
     }
     // V of tile kt has landed in every wave (asked for half a tile ago or more); V[buf ^ 1] has been read for the last time
@@ -385,22 +396,22 @@ __global__ __launch_bounds__(256, 1) void flash_attn_f32_kernel(const _Float16* 
     __syncthreads();
     if (more) copy_v(kt + 1, buf ^ 1);
     if (kt * FA_KT + 32 < Skv) {   // second half
-      v16f am, ar, a2;
-      scores(Kb + buf * KTB + k_lane + 32 * KRS, am, ar, a2);
-      v8h npt[2], npr[2];
-      weights_and_pv(std::true_type{}, std::true_type{}, pend_v, pt, pr, am, ar, a2, kt * FA_KT + 32, npt, npr);
-#pragma unroll
-      for (int s = 0; s < 2; ++s) { pt[s] = npt[s]; pr[s] = npr[s]; }
+      v16f am, ar;
+      scores(std::true_type{}, Kb + buf * KTB + k_lane + 32 * KRS, am, ar);
+      pv_and_maxima(std::true_type{}, pend_v, am, ar, kt * FA_KT + 32);
       pend_v = Vb + buf * VTB + v_lane + 32 * VRS;
     }
     // K of tile kt + 1 has landed; K[buf] has been read for the last time
     if (more) __builtin_amdgcn_s_waitcnt(vmcnt_at_most(VC_MIN));
     __syncthreads();
   }
-  {   // the last half's product
+  {   // the last half's weights, then its product
+    const float bias = kF32PBits - m_ref;
+    lsum = 0.0f;
+    static_for<8>([&](auto k_c) __attribute__((always_inline)) { weight_pair(k_c, bias); });
+    weights_done();
     const v16f none = zero16;
-    v8h npt[2], npr[2];
-    weights_and_pv(std::true_type{}, std::false_type{}, pend_v, pt, pr, none, none, none, 0, npt, npr);
+    pv_and_maxima(std::false_type{}, pend_v, none, none, 0);
   }
   __syncthreads();   // LDS is reused below
 
@@ -410,7 +421,7 @@ __global__ __launch_bounds__(256, 1) void flash_attn_f32_kernel(const _Float16* 
   constexpr int LPR = D / 4;   // 16-byte chunks per row
   unsigned char* const ot = smem + wave * (32 * ORS);
   const float l = l_run + __shfl_xor(l_run, 32);
-  const float fin = v_inv * (1.0f / kF32P) / l;
+  const float fin = v_inv / l;   // l in the scale of the weights' planes, as O's accumulators
 #pragma unroll
   for (int dt = 0; dt < DT; ++dt)
 #pragma unroll

@@ -1132,6 +1132,14 @@ def test_flash_attention_f32_closed_forms_and_scales(core):
     K[0, 0, 5, 7] = 50.0
     O = core.flash_attention_f32(dev(Q), dev(K), dev(V), 0.125).cpu().numpy()
     assert ko.max_rel_err(O, ko.attention(Q, K, V, 0.125)) <= F32_ATTN_TOL / 10
+    # the softmax reference follows the maximum lazily (it moves when a score exceeds it by 8 bits): scores that climb or
+    # fall by a few bits per half tile of 32 keys, so that weights reach 2^7 before it moves, or shrink to nothing
+    u = np.sign(Q.mean(axis=2, keepdims=True)) / np.abs(Q.mean(axis=2, keepdims=True)).clip(0.05)
+    for bits_per_half in (2.5, 7.5, -3.0, -20.0):
+        K = rng.standard_normal((B, Hd, S, D)).astype(np.float32) * 0.1
+        K += ((np.arange(S) // 32)[None, None, :, None] * bits_per_half * np.log(2.0) / 0.125 / D * u).astype(np.float32)
+        O = core.flash_attention_f32(dev(Q), dev(K), dev(V), 0.125).cpu().numpy()
+        assert ko.max_rel_err(O, ko.attention(Q, K, V, 0.125)) <= F32_ATTN_TOL / 10, bits_per_half
 
 
 def test_flash_attention_f32_config3_shape_properties(core):
