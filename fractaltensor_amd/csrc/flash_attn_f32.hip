@@ -4,14 +4,14 @@
 // The reference's attention program computes in fp32 (examples/flash_attention/flash_attention.py:14-91 with
 // kaleido.float32 blocks, flash_attention_utils.py:20-24).  fp32 MFMAs move two k per 16 passes where fp16
 // MFMAs move sixteen per 8, so, as in the stacked LSTM, an fp32 product is cheaper as three fp16 ones:
-//   v * 2^e = top + rest / 2^11,  top = fp16(v * 2^e),  rest = fp16((v * 2^e - top) * 2^11),
-// top * top in one accumulator, top * rest and rest * top in a second one that is folded in with 2^-11;
-// rest * rest, 2^-22 of a product, is dropped.  What shares a power-of-two scale 2^e (its largest magnitude
-// lands in [2^14, 2^15)): a row of Q, all of K of one (batch, head), all of V of one (batch, head), and the
-// fixed 2^7 for the softmax weights p in [0, 2^8).  An element keeps 22 significant bits of its own as long as it
-// is within 2^-28 of its group's largest (a weight: down to 2^-21, and an absolute 2^-43 below that, the remainder
-// plane holding what the value plane's subnormals drop); smaller ones lose bits, of products that are that much
-// smaller too.
+//   v * 2^e = top + rest,  top = fp16(v * 2^e),  rest = fp16(v * 2^e - top),
+// and top * top, top * rest and rest * top go into one fp32 accumulator; rest * rest, 2^-22 of a product, is
+// dropped.  What shares a power-of-two scale 2^e (its largest magnitude lands in [2^14, 2^15)): a row of Q, all
+// of K of one (batch, head), all of V of one (batch, head), and the fixed 2^7 for the softmax weights p in
+// [0, 2^8).  The two planes hold an element to within 2^-40 of its group's largest magnitude (2^-29 where the
+// matrix unit flushes an fp16 subnormal: the remainder of an element below 2^-17 of the largest is one), which is
+// what a sum of products is accurate to anyway: 22 significant bits of its own are kept by every element within
+// 2^-17 of the largest.
 //
 // Three launches: the largest |K| and |V| per (batch, head); the split of Q (times scale * log2 e), K and V into
 // planes [row][top D | rest D] in the workspace; the attention kernel.  A plane row is an fp16 row of 2 D
@@ -19,8 +19,9 @@
 // (fa_common.h), and the contractions are its transposed ones: S^T = K Q^T, O^T += V^T P^T, a lane owns one query
 // row, the running maximum and sum are lane-local.  The reference that the weights are taken against follows the
 // running maximum lazily: it moves only when a score exceeds it by more than 8 bits (kLazyBits), so weights reach
-// 2^8 at most and O's accumulators, 256 registers behind the matrix unit, are rescaled once per row block on
-// ordinary data rather than whenever one of a wave's 32 rows finds a new maximum (every other half tile).
+// 2^8 at most and O's accumulators (accumulation registers, which vector instructions reach only through moves)
+// are rescaled once per row block on ordinary data rather than whenever one of a wave's 32 rows finds a new
+// maximum (every other half tile).
 #include <algorithm>
 #include <type_traits>
 
@@ -28,8 +29,9 @@
 
 namespace ftk {
 
+typedef float v2f __attribute__((ext_vector_type(2)));
+
 constexpr int kF32Top = 14;             // a scale group's largest magnitude lands in [2^14, 2^15)
-constexpr float kF32Rest = 2048.0f;     // 2^11
 constexpr float kF32PBits = 7.0f;        // 2^7: the scale of the softmax weights in their fp16 planes
 constexpr float kLazyBits = 7.99f;      // how far a score may exceed the softmax reference: weights below 2^8, below 65504 in their plane
 // s_waitcnt immediate: at most n vector memory operations outstanding (n < 64), the other counters left alone
@@ -104,7 +106,7 @@ __global__ __launch_bounds__(256) void attn_f32_split_kernel(const float* X, _Fl
       const float s = v[e] * scale;
       const _Float16 top = (_Float16)s;
       dst[e] = top;
-      dst[D + e] = (_Float16)((s - (float)top) * kF32Rest);
+      dst[D + e] = (_Float16)(s - (float)top);
     }
   }
 }
@@ -160,11 +162,11 @@ __global__ __launch_bounds__(256, 1) void flash_attn_f32_kernel(const _Float16* 
   split_scale(kv_bits[BH + bh], &v_scale, &v_inv);
   const float s_mul = q_inv[(size_t)bh * Sq + qrow] * k_inv;
 
-  v16f om[DT], oc[DT];
+  v16f om[DT];
 #pragma unroll
   for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
-    for (int r = 0; r < 16; ++r) { om[dt][r] = 0.0f; oc[dt][r] = 0.0f; }
+    for (int r = 0; r < 16; ++r) om[dt][r] = 0.0f;
 
   // copies: as in the fp16 kernel, copy c of a tile fills LDS bytes [1024 c, 1024 c + 1024) of the padded tile
   unsigned k_src[KCP], v_src[VCP];
@@ -251,103 +253,144 @@ __global__ __launch_bounds__(256, 1) void flash_attn_f32_kernel(const _Float16* 
     constexpr int k = decltype(k_c)::value;
     const float s0 = __builtin_amdgcn_exp2f(fmaf(raw[2 * k], s_mul, bias)), s1 = __builtin_amdgcn_exp2f(fmaf(raw[2 * k + 1], s_mul, bias));
     lsum += s0 + s1;
-    const v2h top = {(_Float16)s0, (_Float16)s1};
-    const v2h rest = {(_Float16)((s0 - (float)top[0]) * kF32Rest), (_Float16)((s1 - (float)top[1]) * kF32Rest)};
-    unsigned tu = __builtin_bit_cast(unsigned, top), ru = __builtin_bit_cast(unsigned, rest);
+    const v2f sv = {s0, s1};
+    const v2h top = __builtin_convertvector(sv, v2h);
+    unsigned tu = __builtin_bit_cast(unsigned, top), ru;
+    // the remainders, s - top rounded to fp16: one mixed-precision fma each (the fp16 value read as fp32 times -1, plus
+    // s; the difference is exact in fp32) instead of a conversion back, a subtraction and a conversion
+    asm("v_fma_mixlo_f16 %0, %1, -1.0, %2 op_sel_hi:[1,0,0]\n\tv_fma_mixhi_f16 %0, %1, -1.0, %3 op_sel:[1,0,0] op_sel_hi:[1,0,0]"
+        : "=&v"(ru) : "v"(tu), "v"(s0), "v"(s1));
     // pinned to its place: left alone, the compiler moves the arithmetic to where the weights are read, out from under the MFMAs
     asm volatile("" : "+v"(tu), "+v"(ru), "+v"(lsum));
     ptu[k] = tu;
     pru[k] = ru;
   };
-  auto weights_done = [&]() __attribute__((always_inline)) {
-#pragma unroll
-    for (int h = 0; h < 2; ++h) {
-      pt[h] = __builtin_bit_cast(v8h, v4u{ptu[4 * h], ptu[4 * h + 1], ptu[4 * h + 2], ptu[4 * h + 3]});
-      pr[h] = __builtin_bit_cast(v8h, v4u{pru[4 * h], pru[4 * h + 1], pru[4 * h + 2], pru[4 * h + 3]});
-    }
-    l_run += lsum;
+  // the weights of key step h of the half (pairs 4 h .. 4 h + 3) as the P V product's fragments
+  auto weights_done = [&](int h) __attribute__((always_inline)) {
+    pt[h] = __builtin_bit_cast(v8h, v4u{ptu[4 * h], ptu[4 * h + 1], ptu[4 * h + 2], ptu[4 * h + 3]});
+    pr[h] = __builtin_bit_cast(v8h, v4u{pru[4 * h], pru[4 * h + 1], pru[4 * h + 2], pru[4 * h + 3]});
+  };
+  // With an even number of d tiles the P V product uses the weights of the first key step (pairs 0..3) alone for its
+  // first half: only those are formed beside the scores, pairs 4..7 beside the first half of the product itself, and
+  // the maxima of the next scores beside its second half -- a wave that is alone on its SIMD hides some four vector
+  // instructions per MFMA, so the vector work is dealt out as evenly as the order allows.
+  constexpr bool kDefer = DT % 2 == 0;
+  constexpr int kPairsBesideScores = kDefer ? 4 : 8;
+  float bias = 0.0f;   // what a raw score times s_mul is offset by in the weights' exponent (set where a half's weights begin)
+
+  // Fragments live across the two products: each requests the other's first ones before it ends, so that no product
+  // begins by waiting for LDS (a read takes some hundreds of cycles under this load).
+  v8h kf_t[4], kf_r[4];   // K fragments (values, remainders) of a k step, four sets in turn
+  v8h vf_t[4], vf_r[4];   // V fragments of a (key step, d tile) group, two pairs of groups in turn
+  auto read_k = [&](const unsigned char* kbase, int s, int set) __attribute__((always_inline)) {
+    kf_t[set] = *reinterpret_cast<const v8h*>(kbase + 32 * s);
+    kf_r[set] = *reinterpret_cast<const v8h*>(kbase + 2 * D + 32 * s);
+  };
+  auto read_group = [&](const unsigned char* pvbase, int g, int set) __attribute__((always_inline)) {
+    vf_t[set] = read_v(pvbase, g / DT, g % DT, 0);
+    vf_r[set] = read_v(pvbase, g / DT, g % DT, 1);
   };
 
-  // The scores of 32 keys (one half of a tile): value x value in am, the two mixed products, 2^-11 of it, in ar.  A
-  // step's K fragments are requested two steps ahead (three sets of registers in turn).  WEIGHTS: the weights of the
-  // half before are formed beside them, a share with every step.
-  auto scores = [&](auto weights_c, const unsigned char* kbase, v16f& am, v16f& ar) __attribute__((always_inline)) {
-    constexpr bool WEIGHTS = decltype(weights_c)::value;
-    v8h kf_t[3], kf_r[3];
-#pragma unroll
-    for (int s = 0; s < 2; ++s) {
-      kf_t[s] = *reinterpret_cast<const v8h*>(kbase + 32 * s);
-      kf_r[s] = *reinterpret_cast<const v8h*>(kbase + 2 * D + 32 * s);
+  // The scores of 32 keys (one half of a tile): value x value and the two mixed products, all into am.  A step's
+  // K fragments are requested three steps ahead; PRELOADED: those of steps 0 and 1 by the product before.
+  // Beside the MFMAs: the weights of the half before, a share with every step; the copies of a whole tile that is
+  // on its way (COPY 1: K of tile ckt, 2: V of tile ckt; 0: none), a share with every step and no branch among them;
+  // and at the end the first V fragments of the product that follows (rows at pvbase).
+  auto scores = [&](auto preloaded_c, auto copy_c, int ckt, int cbuf, const unsigned char* kbase, const unsigned char* pvbase,
+                    v16f& am) __attribute__((always_inline)) {
+    constexpr bool PRELOADED = decltype(preloaded_c)::value;
+    constexpr int COPY = decltype(copy_c)::value;
+    constexpr int NCOPY = COPY == 1 ? KCP : VCP;
+    if constexpr (!PRELOADED) {
+      read_k(kbase, 0, 0);
+      read_k(kbase, 1, 1);
     }
-    // (before the first half there is no reference, and every raw score is -inf: weights of zero)
-    const float bias = m_ref > -INFINITY ? kF32PBits - m_ref : 0.0f;
+    if constexpr (DS > 2) read_k(kbase, 2, 2);
+    bias = m_ref > -INFINITY ? kF32PBits - m_ref : 0.0f;   // (no reference before the first half: every raw score is -inf)
     lsum = 0.0f;
+    const _Float16* crows = (COPY == 1 ? Kg : Vg) + (size_t)ckt * FA_KT * (2 * D);
+    unsigned char* cdst = COPY == 1 ? Kb + cbuf * KTB : Vb + cbuf * VTB;
     __builtin_amdgcn_sched_barrier(0);
     static_for<DS>([&](auto s_c) __attribute__((always_inline)) {
-      constexpr int s = decltype(s_c)::value, b = s % 3;
+      constexpr int s = decltype(s_c)::value, b = s % 4;
       am = __builtin_amdgcn_mfma_f32_32x32x16_f16(kf_t[b], qt[s], s == 0 ? zero16 : am, 0, 0, 0);
-      if constexpr (s + 2 < DS) {
-        kf_t[(s + 2) % 3] = *reinterpret_cast<const v8h*>(kbase + 32 * (s + 2));
-        kf_r[(s + 2) % 3] = *reinterpret_cast<const v8h*>(kbase + 2 * D + 32 * (s + 2));
-      }
-      ar = __builtin_amdgcn_mfma_f32_32x32x16_f16(kf_t[b], qr[s], s == 0 ? zero16 : ar, 0, 0, 0);
-      ar = __builtin_amdgcn_mfma_f32_32x32x16_f16(kf_r[b], qt[s], ar, 0, 0, 0);
-      if constexpr (WEIGHTS) {
-        static_for<8 * (s + 1) / DS - 8 * s / DS>([&](auto j_c) __attribute__((always_inline)) {
-          weight_pair(std::integral_constant<int, 8 * s / DS + decltype(j_c)::value>{}, bias);
-        });
-      }
+      if constexpr (s + 3 < DS) read_k(kbase, s + 3, (s + 3) % 4);
+      if constexpr (s >= DS - 2) read_group(pvbase, s - (DS - 2), s - (DS - 2));
+      am = __builtin_amdgcn_mfma_f32_32x32x16_f16(kf_t[b], qr[s], am, 0, 0, 0);
+      am = __builtin_amdgcn_mfma_f32_32x32x16_f16(kf_r[b], qt[s], am, 0, 0, 0);
+      static_for<kPairsBesideScores * (s + 1) / DS - kPairsBesideScores * s / DS>([&](auto j_c) __attribute__((always_inline)) {
+        weight_pair(std::integral_constant<int, kPairsBesideScores * s / DS + decltype(j_c)::value>{}, bias);
+      });
       // the order within the step: MFMA, the reads, and the vector instructions in three shares behind the three MFMAs
       // (the first share holds the two exp2, four issue slots each)
       __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-      __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+      __builtin_amdgcn_sched_group_barrier(0x100, s >= DS - 2 ? 4 : 2, 0);
       __builtin_amdgcn_sched_group_barrier(0x002, 4, 0);
       __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
       __builtin_amdgcn_sched_group_barrier(0x002, 6, 0);
       __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
       __builtin_amdgcn_sched_group_barrier(0x002, 6, 0);
       __builtin_amdgcn_sched_barrier(0);
+      if constexpr (COPY != 0) {
+        static_for<NCOPY * (s + 1) / DS - NCOPY * s / DS>([&](auto j_c) __attribute__((always_inline)) {
+          constexpr int i = NCOPY * s / DS + decltype(j_c)::value, COPIES = (COPY == 1 ? KTB : VTB) / 1024;
+          const unsigned src = COPY == 1 ? k_src[i % KCP] : v_src[i % VCP];
+          if (WAVES * i + WAVES - 1 < COPIES || wave + WAVES * i < COPIES) lds_dma16(crows, src, cdst + 1024 * (wave + WAVES * i));
+        });
+        __builtin_amdgcn_sched_barrier(0);
+      }
     });
-    if constexpr (WEIGHTS) weights_done();
+    weights_done(0);
+    if constexpr (!kDefer) {
+      weights_done(1);
+      l_run += lsum;
+    }
   };
 
   // The P V product of the half whose weights are in pt / pr (V rows at pvbase), and beside it (MAXIMA) the raw
-  // scores and the maximum of the half whose products are in am / ar; then the reference moves if a score exceeds it
+  // scores and the maximum of the half whose products are in am; then the reference moves if a score exceeds it
   // by more than kLazyBits, and O and the sum are brought to the new one.  Groups (key step, d tile: 3 MFMAs) are
   // taken two at a time, in an order in which no MFMA adds to the result of the one before it; a pair's V fragments are
   // requested under the pair before.
-  auto pv_and_maxima = [&](auto maxima_c, const unsigned char* pvbase, const v16f& am, const v16f& ar, int key0) __attribute__((always_inline)) {
-    constexpr bool MAXIMA = decltype(maxima_c)::value;
+  auto pv_and_maxima = [&](auto maxima_c, auto next_k_c, auto mask_c, const unsigned char* pvbase, const unsigned char* next_kbase,
+                           const v16f& am, int key0) __attribute__((always_inline)) {
+    // MAXIMA false: the product alone, behind the last half, all of whose weights are there; MASK: the half is ragged
+    constexpr bool MAXIMA = decltype(maxima_c)::value, NEXT_K = decltype(next_k_c)::value, MASK = decltype(mask_c)::value;
+    constexpr bool DEFER = kDefer && MAXIMA;
     constexpr int NG = 2 * DT, NM = 3 * NG;
-    v8h vf_t[4], vf_r[4];
-#pragma unroll
-    for (int g = 0; g < 2; ++g) {
-      vf_t[g] = read_v(pvbase, g / DT, g % DT, 0);
-      vf_r[g] = read_v(pvbase, g / DT, g % DT, 1);
-    }
-    __builtin_amdgcn_sched_barrier(0);
+    constexpr int M0 = DEFER ? NM / 2 : 0, MN = NM - M0;   // the slots that hold the maxima
+    // (the first pair's fragments were requested by the scores before; NEXT_K: the last slots request the K fragments
+    // of steps 0 and 1 of the scores that follow, rows at next_kbase)
     float mx = -INFINITY;
-    const int lim = Skv - key0 - 4 * hh;   // score r belongs to a key past the end when 8 (r >> 2) + (r & 3) >= lim
+    [[maybe_unused]] const int lim = Skv - key0 - 4 * hh;   // score r belongs to a key past the end when 8 (r >> 2) + (r & 3) >= lim
     static_for<NM>([&](auto i_c) __attribute__((always_inline)) {
       constexpr int i = decltype(i_c)::value, pair = i / 6, k = i % 6, g0 = 2 * pair, g1 = g0 + 1;
       constexpr int b0 = (pair & 1) * 2, b1 = b0 + 1, nb = ((pair + 1) & 1) * 2;
       constexpr int sk0 = g0 / DT, dt0 = g0 % DT, sk1 = g1 / DT, dt1 = g1 % DT;
-      if constexpr ((k == 1 || k == 3) && g0 + 2 < NG) {   // the next pair's fragments
-        constexpr int g = g0 + 2 + (k == 3);
-        vf_t[nb + (k == 3)] = read_v(pvbase, g / DT, g % DT, 0);
-        vf_r[nb + (k == 3)] = read_v(pvbase, g / DT, g % DT, 1);
-      }
+      if constexpr ((k == 1 || k == 3) && g0 + 2 < NG) read_group(pvbase, g0 + 2 + (k == 3), nb + (k == 3));   // the next pair's fragments
+      if constexpr (NEXT_K && g0 + 2 >= NG && (k == 1 || k == 3)) read_k(next_kbase, k == 3, k == 3);
       if constexpr (k == 0) om[dt0] = __builtin_amdgcn_mfma_f32_32x32x16_f16(vf_t[b0], pt[sk0], om[dt0], 0, 0, 0);
-      if constexpr (k == 1) oc[dt0] = __builtin_amdgcn_mfma_f32_32x32x16_f16(vf_t[b0], pr[sk0], oc[dt0], 0, 0, 0);
-      if constexpr (k == 2) om[dt1] = __builtin_amdgcn_mfma_f32_32x32x16_f16(vf_t[b1], pt[sk1], om[dt1], 0, 0, 0);
-      if constexpr (k == 3) oc[dt1] = __builtin_amdgcn_mfma_f32_32x32x16_f16(vf_t[b1], pr[sk1], oc[dt1], 0, 0, 0);
-      if constexpr (k == 4) oc[dt0] = __builtin_amdgcn_mfma_f32_32x32x16_f16(vf_r[b0], pt[sk0], oc[dt0], 0, 0, 0);
-      if constexpr (k == 5) oc[dt1] = __builtin_amdgcn_mfma_f32_32x32x16_f16(vf_r[b1], pt[sk1], oc[dt1], 0, 0, 0);
-      if constexpr (MAXIMA) {
+      if constexpr (k == 1) om[dt1] = __builtin_amdgcn_mfma_f32_32x32x16_f16(vf_t[b1], pt[sk1], om[dt1], 0, 0, 0);
+      if constexpr (k == 2) om[dt0] = __builtin_amdgcn_mfma_f32_32x32x16_f16(vf_t[b0], pr[sk0], om[dt0], 0, 0, 0);
+      if constexpr (k == 3) om[dt1] = __builtin_amdgcn_mfma_f32_32x32x16_f16(vf_t[b1], pr[sk1], om[dt1], 0, 0, 0);
+      if constexpr (k == 4) om[dt0] = __builtin_amdgcn_mfma_f32_32x32x16_f16(vf_r[b0], pt[sk0], om[dt0], 0, 0, 0);
+      if constexpr (k == 5) om[dt1] = __builtin_amdgcn_mfma_f32_32x32x16_f16(vf_r[b1], pt[sk1], om[dt1], 0, 0, 0);
+      if constexpr (DEFER && i < M0) {   // the weights of the second key step (pairs 4..7), wanted by this product's second half
+        static_for<4 * (i + 1) / M0 - 4 * i / M0>([&](auto j_c) __attribute__((always_inline)) {
+          weight_pair(std::integral_constant<int, 4 + 4 * i / M0 + decltype(j_c)::value>{}, bias);
+        });
+        if constexpr (i == M0 - 1) {
+          weights_done(1);
+          l_run += lsum;
+        }
+      }
+      if constexpr (MAXIMA && i >= M0) {
 #pragma unroll
-        for (int r = 16 * i / NM; r < 16 * (i + 1) / NM; ++r) {
-          raw[r] = fmaf(ar[r], 1.0f / kF32Rest, am[r]);
-          if (8 * (r >> 2) + (r & 3) >= lim) raw[r] = -INFINITY;
+        for (int r = 16 * (i - M0) / MN; r < 16 * (i - M0 + 1) / MN; ++r) {
+          raw[r] = am[r];
+          if constexpr (MASK) {
+            if (8 * (r >> 2) + (r & 3) >= lim) raw[r] = -INFINITY;
+          }
           mx = fmaxf(mx, raw[r]);
         }
       }
@@ -364,14 +407,14 @@ __global__ __launch_bounds__(256, 1) void flash_attn_f32_kernel(const _Float16* 
 #pragma unroll
         for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
-          for (int r = 0; r < 16; ++r) { om[dt][r] *= alpha; oc[dt][r] *= alpha; }
+          for (int r = 0; r < 16; ++r) om[dt][r] *= alpha;
       }
     }
   };
 
   // A tile's K rows are last read by the scores of its second half and its V rows one half later, beside the next
-  // tile's first maxima: K of tile kt + 1 is requested when tile kt begins, V of tile kt + 1 behind the barrier in
-  // the middle of tile kt.  Copies complete in the order of their issue, so each of the two barriers waits for the
+  // tile's first maxima: K of tile kt + 1 is requested beside the scores of tile kt's first half, V of tile kt + 1
+  // beside those of its second half, behind the barrier in the middle of the tile.  Copies complete in the order of their issue, so each of the two barriers waits for the
   // older of the two requests only.
   const int ntiles = (Skv + FA_KT - 1) / FA_KT;
   copy_k(0, 0);
@@ -383,22 +426,35 @@ __global__ __launch_bounds__(256, 1) void flash_attn_f32_kernel(const _Float16* 
   for (int kt = 0; kt < ntiles; ++kt) {
     const int buf = kt & 1;
     const bool more = kt + 1 < ntiles;
-    if (more) copy_k(kt + 1, buf ^ 1);   // K[buf ^ 1] was last read before the barrier that ended tile kt - 1
-    {   // first half
-      v16f am, ar;
-      scores(std::true_type{}, Kb + buf * KTB + k_lane, am, ar);
-      pv_and_maxima(std::true_type{}, pend_v, am, ar, kt * FA_KT);
+    const bool whole_next = (kt + 2) * FA_KT <= Skv;   // a tile follows and all of its 64 keys exist
+    {   // first half; beside its scores, K of tile kt + 1 is requested (K[buf ^ 1] was last read before the barrier that ended tile kt - 1)
+      v16f am;
+      const unsigned char* kbase = Kb + buf * KTB + k_lane;
+      if (whole_next) {
+        scores(std::false_type{}, std::integral_constant<int, 1>{}, kt + 1, buf ^ 1, kbase, pend_v, am);
+      } else {
+        if (more) copy_k(kt + 1, buf ^ 1);   // the last, ragged tile: each copy clamps its rows
+        scores(std::false_type{}, std::integral_constant<int, 0>{}, 0, 0, kbase, pend_v, am);
+      }
+      if (kt * FA_KT + 32 <= Skv) pv_and_maxima(std::true_type{}, std::true_type{}, std::false_type{}, pend_v, kbase + 32 * KRS, am, kt * FA_KT);
+      else pv_and_maxima(std::true_type{}, std::true_type{}, std::true_type{}, pend_v, kbase + 32 * KRS, am, kt * FA_KT);
       pend_v = Vb + buf * VTB + v_lane;
     }
     // V of tile kt has landed in every wave (asked for half a tile ago or more); V[buf ^ 1] has been read for the last time
     if (more) __builtin_amdgcn_s_waitcnt(vmcnt_at_most(KC_MIN));
     else __builtin_amdgcn_s_waitcnt(0x0F70);
     __syncthreads();
-    if (more) copy_v(kt + 1, buf ^ 1);
-    if (kt * FA_KT + 32 < Skv) {   // second half
-      v16f am, ar;
-      scores(std::true_type{}, Kb + buf * KTB + k_lane + 32 * KRS, am, ar);
-      pv_and_maxima(std::true_type{}, pend_v, am, ar, kt * FA_KT + 32);
+    if (kt * FA_KT + 32 < Skv) {   // second half (a tile that is followed by another has one); beside its scores, V of tile kt + 1 is requested
+      v16f am;
+      const unsigned char* kbase = Kb + buf * KTB + k_lane + 32 * KRS;
+      if (whole_next) {
+        scores(std::true_type{}, std::integral_constant<int, 2>{}, kt + 1, buf ^ 1, kbase, pend_v, am);
+      } else {
+        if (more) copy_v(kt + 1, buf ^ 1);
+        scores(std::true_type{}, std::integral_constant<int, 0>{}, 0, 0, kbase, pend_v, am);
+      }
+      if (kt * FA_KT + 64 <= Skv) pv_and_maxima(std::true_type{}, std::false_type{}, std::false_type{}, pend_v, nullptr, am, kt * FA_KT + 32);
+      else pv_and_maxima(std::true_type{}, std::false_type{}, std::true_type{}, pend_v, nullptr, am, kt * FA_KT + 32);
       pend_v = Vb + buf * VTB + v_lane + 32 * VRS;
     }
     // K of tile kt + 1 has landed; K[buf] has been read for the last time
@@ -406,12 +462,16 @@ __global__ __launch_bounds__(256, 1) void flash_attn_f32_kernel(const _Float16* 
     __syncthreads();
   }
   {   // the last half's weights, then its product
-    const float bias = kF32PBits - m_ref;
+    bias = kF32PBits - m_ref;
     lsum = 0.0f;
     static_for<8>([&](auto k_c) __attribute__((always_inline)) { weight_pair(k_c, bias); });
-    weights_done();
+    weights_done(0);
+    weights_done(1);
+    l_run += lsum;
+    read_group(pend_v, 0, 0);
+    read_group(pend_v, 1, 1);
     const v16f none = zero16;
-    pv_and_maxima(std::false_type{}, pend_v, none, none, 0);
+    pv_and_maxima(std::false_type{}, std::false_type{}, std::false_type{}, pend_v, nullptr, none, 0);
   }
   __syncthreads();   // LDS is reused below
 
@@ -427,10 +487,10 @@ __global__ __launch_bounds__(256, 1) void flash_attn_f32_kernel(const _Float16* 
 #pragma unroll
     for (int g = 0; g < 4; ++g) {
       float4 o;
-      o.x = (om[dt][4 * g + 0] + (1.0f / kF32Rest) * oc[dt][4 * g + 0]) * fin;
-      o.y = (om[dt][4 * g + 1] + (1.0f / kF32Rest) * oc[dt][4 * g + 1]) * fin;
-      o.z = (om[dt][4 * g + 2] + (1.0f / kF32Rest) * oc[dt][4 * g + 2]) * fin;
-      o.w = (om[dt][4 * g + 3] + (1.0f / kF32Rest) * oc[dt][4 * g + 3]) * fin;
+      o.x = om[dt][4 * g + 0] * fin;
+      o.y = om[dt][4 * g + 1] * fin;
+      o.z = om[dt][4 * g + 2] * fin;
+      o.w = om[dt][4 * g + 3] * fin;
       *reinterpret_cast<float4*>(ot + j * ORS + 4 * (32 * dt + 8 * g + 4 * hh)) = o;
     }
 #pragma unroll
