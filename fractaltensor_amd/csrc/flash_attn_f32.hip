@@ -13,8 +13,9 @@
 // what a sum of products is accurate to anyway: 22 significant bits of its own are kept by every element within
 // 2^-17 of the largest.
 //
-// Three launches: the largest |K| and |V| per (batch, head); the split of Q (times scale * log2 e), K and V into
-// planes [row][top D | rest D] in the workspace; the attention kernel.  A plane row is an fp16 row of 2 D
+// Three launches besides a clear: the largest |K| and |V| per (batch, head); the split of K and V into planes
+// [row][top D | rest D] in the workspace; the attention kernel, which splits its rows of Q (times scale * log2 e)
+// itself, in registers.  A plane row is an fp16 row of 2 D
 // elements, so tiles, copies and fragment reads are those of the fp16 kernel at twice the head dimension
 // (fa_common.h), and the contractions are its transposed ones: S^T = K Q^T, O^T += V^T P^T, a lane owns one query
 // row, the running maximum and sum are lane-local.  The reference that the weights are taken against follows the
@@ -71,39 +72,25 @@ __global__ __launch_bounds__(256) void attn_f32_absmax_kernel(const float* K, co
   }
 }
 
-// One wave per row of D floats: planes [top D | rest D] of the row times `mul`, under the row's own scale
-// (row_inv != nullptr: Q; the inverse scale goes to row_inv[row]) or under the (batch, head)'s (K, V).
+// One wave per row of D floats of K (blockIdx.y 0) or V (1): planes [top D | rest D] of the row under its (batch,
+// head)'s scale.
 template <int D>
-__global__ __launch_bounds__(256) void attn_f32_split_kernel(const float* X, _Float16* planes, float* row_inv, const unsigned* group_bits,
-                                                            int rows_per_bh, long long rows, float mul) {
-  constexpr int PER = D / 32;   // floats per lane: 1, 2, 3 or 4; lanes 32..63 idle for D = 32 only when PER * 64 > D
+__global__ __launch_bounds__(256) void attn_f32_split_kernel(const float* K, const float* V, _Float16* kplanes, _Float16* vplanes,
+                                                            const unsigned* group_bits, int rows_per_bh, long long rows, int BH) {
+  constexpr int PER = D / 32;   // floats per lane: 1, 2, 3 or 4
   const int lane = threadIdx.x & 63;
   const long long row = (long long)blockIdx.x * 4 + (threadIdx.x >> 6);
   if (row >= rows) return;
+  const float* X = blockIdx.y ? V : K;
+  _Float16* planes = blockIdx.y ? vplanes : kplanes;
   constexpr int LANES = D / PER > 64 ? 64 : D / PER;   // 32 lanes x PER floats cover a row
-  float v[PER];
-  unsigned m = 0;
-  if (lane < LANES) {
-#pragma unroll
-    for (int e = 0; e < PER; ++e) {
-      v[e] = X[row * D + lane * PER + e] * mul;
-      m = max(m, __float_as_uint(fabsf(v[e])));
-    }
-  }
   float scale, inv;
-  if (row_inv) {
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) m = max(m, (unsigned)__shfl_xor((int)m, o));
-    split_scale(m, &scale, &inv);
-    if (lane == 0) row_inv[row] = inv;
-  } else {
-    split_scale(group_bits[row / rows_per_bh], &scale, &inv);
-  }
+  split_scale(group_bits[blockIdx.y * BH + row / rows_per_bh], &scale, &inv);
   if (lane < LANES) {
     _Float16* dst = planes + row * (2 * D) + lane * PER;
 #pragma unroll
     for (int e = 0; e < PER; ++e) {
-      const float s = v[e] * scale;
+      const float s = X[row * D + lane * PER + e] * scale;
       const _Float16 top = (_Float16)s;
       dst[e] = top;
       dst[D + e] = (_Float16)(s - (float)top);
@@ -117,8 +104,8 @@ __global__ __launch_bounds__(256) void attn_f32_split_kernel(const float* X, _Fl
 // wave's MFMAs to run beside: it is cut in two, the maxima under the P V MFMAs of the half before and the weights
 // under the score MFMAs of the half after (the comments in the kernel give the order).
 template <int D>
-__global__ __launch_bounds__(256, 1) void flash_attn_f32_kernel(const _Float16* __restrict__ Qp, const _Float16* __restrict__ Kp,
-                                                                const _Float16* __restrict__ Vp, const float* __restrict__ q_inv,
+__global__ __launch_bounds__(256, 1) void flash_attn_f32_kernel(const float* __restrict__ Q, const _Float16* __restrict__ Kp,
+                                                                const _Float16* __restrict__ Vp, float q_mul,
                                                                 const unsigned* __restrict__ kv_bits, float* __restrict__ O,
                                                                 int Sq, int Skv, int nqb, int BH) {
   using L = FaLayout<2 * D>;          // a plane row is an fp16 row of 2 D elements
@@ -144,23 +131,54 @@ __global__ __launch_bounds__(256, 1) void flash_attn_f32_kernel(const _Float16* 
   const int qb = id - bh * nqb;
   const int q_base = qb * (WAVES * 32) + wave * 32;
 
-  const _Float16* Qg = Qp + (size_t)bh * Sq * (2 * D);
   const _Float16* Kg = Kp + (size_t)bh * Skv * (2 * D);
   const _Float16* Vg = Vp + (size_t)bh * Skv * (2 * D);
   float* Og = O + (size_t)bh * Sq * D;
 
-  // the lane's query row: both planes of its fragments, and what a score is multiplied by to undo the scales
+  // The lane's query row: the fp32 row is read, multiplied by q_mul (scale * log2 e: a score leaves the matrix unit in
+  // exponent units), brought under the row's own power-of-two scale and split into the two planes here, in registers
+  // (a lane and its partner 32 lanes on hold the row's two halves of every 16 columns).
   const int qrow = min(q_base + j, Sq - 1);
   v8h qt[DS], qr[DS];
+  float s_mul;
+  {
+    const float* qsrc = Q + ((size_t)bh * Sq + qrow) * D + 8 * hh;
+    float4 x[DS][2];
 #pragma unroll
-  for (int s = 0; s < DS; ++s) {
-    qt[s] = *reinterpret_cast<const v8h*>(Qg + (size_t)qrow * (2 * D) + 16 * s + 8 * hh);
-    qr[s] = *reinterpret_cast<const v8h*>(Qg + (size_t)qrow * (2 * D) + D + 16 * s + 8 * hh);
+    for (int s = 0; s < DS; ++s) {
+      x[s][0] = *reinterpret_cast<const float4*>(qsrc + 16 * s);
+      x[s][1] = *reinterpret_cast<const float4*>(qsrc + 16 * s + 4);
+    }
+    unsigned m = 0;
+#pragma unroll
+    for (int s = 0; s < DS; ++s)
+#pragma unroll
+      for (int h = 0; h < 2; ++h) {
+        x[s][h].x *= q_mul; x[s][h].y *= q_mul; x[s][h].z *= q_mul; x[s][h].w *= q_mul;
+        m = max(max(m, __float_as_uint(fabsf(x[s][h].x))), max(__float_as_uint(fabsf(x[s][h].y)),
+                                                               max(__float_as_uint(fabsf(x[s][h].z)), __float_as_uint(fabsf(x[s][h].w)))));
+      }
+    m = max(m, (unsigned)__shfl_xor((int)m, 32));   // the row's largest magnitude, as float bits
+    float q_scale, q_inv;
+    split_scale(m, &q_scale, &q_inv);
+#pragma unroll
+    for (int s = 0; s < DS; ++s)
+#pragma unroll
+      for (int h = 0; h < 2; ++h) {
+        const float v[4] = {x[s][h].x * q_scale, x[s][h].y * q_scale, x[s][h].z * q_scale, x[s][h].w * q_scale};
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          const _Float16 top = (_Float16)v[e];
+          qt[s][4 * h + e] = top;
+          qr[s][4 * h + e] = (_Float16)(v[e] - (float)top);
+        }
+      }
+    float k_scale, k_inv;
+    split_scale(kv_bits[bh], &k_scale, &k_inv);
+    s_mul = q_inv * k_inv;   // what a score is multiplied by to undo the scales
   }
-  float k_scale, k_inv, v_scale, v_inv;
-  split_scale(kv_bits[bh], &k_scale, &k_inv);
+  float v_scale, v_inv;
   split_scale(kv_bits[BH + bh], &v_scale, &v_inv);
-  const float s_mul = q_inv[(size_t)bh * Sq + qrow] * k_inv;
 
   v16f om[DT];
 #pragma unroll
@@ -505,14 +523,12 @@ __global__ __launch_bounds__(256, 1) void flash_attn_f32_kernel(const _Float16* 
 static size_t round256f(size_t v) { return (v + 255) / 256 * 256; }
 
 struct F32Layout {
-  size_t bits, qinv, qp, kp, vp, total;
+  size_t bits, kp, vp, total;
 };
-static F32Layout f32_layout(long long bh, int Sq, int Skv, int D) {
+static F32Layout f32_layout(long long bh, int Skv, int D) {
   F32Layout w;
   w.bits = 0;
-  w.qinv = round256f((size_t)2 * bh * sizeof(unsigned));
-  w.qp = w.qinv + round256f((size_t)bh * Sq * sizeof(float));
-  w.kp = w.qp + round256f((size_t)bh * Sq * 2 * D * sizeof(_Float16));
+  w.kp = round256f((size_t)2 * bh * sizeof(unsigned));
   w.vp = w.kp + round256f((size_t)bh * Skv * 2 * D * sizeof(_Float16));
   w.total = w.vp + round256f((size_t)bh * Skv * 2 * D * sizeof(_Float16));
   return w;
@@ -525,8 +541,6 @@ static int launch_fa_f32(const float* Q, const float* K, const float* V, float* 
   const size_t lds = std::max((size_t)2 * (L::KTB + L::VTB), (size_t)4 * 32 * (4 * D + 16));
   if ((int)lds > lds_max) return fail(FTK_ERR_DEVICE, "ftk_flash_attn_f32: D=%d needs %zu bytes of LDS, the device offers %d", D, lds, lds_max);
   unsigned* bits = reinterpret_cast<unsigned*>(ws + w.bits);
-  float* qinv = reinterpret_cast<float*>(ws + w.qinv);
-  _Float16* qp = reinterpret_cast<_Float16*>(ws + w.qp);
   _Float16* kp = reinterpret_cast<_Float16*>(ws + w.kp);
   _Float16* vp = reinterpret_cast<_Float16*>(ws + w.vp);
   hipLaunchKernelGGL(attn_f32_clear_kernel, dim3((2 * BH + 255) / 256), dim3(256), 0, s, bits, 2 * BH);
@@ -537,13 +551,9 @@ static int launch_fa_f32(const float* Q, const float* K, const float* V, float* 
   hipLaunchKernelGGL(attn_f32_absmax_kernel, dim3(chunks, BH, 2), dim3(256), 0, s, K, V, bits, per_bh, BH);
   rc = check_launch("attn_f32_absmax_kernel");
   if (rc) return rc;
-  const long long qrows = (long long)BH * Sq, krows = (long long)BH * Skv;
-  hipLaunchKernelGGL(attn_f32_split_kernel<D>, dim3((unsigned)((qrows + 3) / 4)), dim3(256), 0, s, Q, qp, qinv, (const unsigned*)nullptr, Sq,
-                     qrows, scale * 1.4426950408889634f);
-  hipLaunchKernelGGL(attn_f32_split_kernel<D>, dim3((unsigned)((krows + 3) / 4)), dim3(256), 0, s, K, kp, (float*)nullptr, (const unsigned*)bits,
-                     Skv, krows, 1.0f);
-  hipLaunchKernelGGL(attn_f32_split_kernel<D>, dim3((unsigned)((krows + 3) / 4)), dim3(256), 0, s, V, vp, (float*)nullptr,
-                     (const unsigned*)(bits + BH), Skv, krows, 1.0f);
+  const long long krows = (long long)BH * Skv;
+  hipLaunchKernelGGL(attn_f32_split_kernel<D>, dim3((unsigned)((krows + 3) / 4), 2), dim3(256), 0, s, K, V, kp, vp, (const unsigned*)bits, Skv, krows,
+                     BH);
   rc = check_launch("attn_f32_split_kernel");
   if (rc) return rc;
   const int nqb = (Sq + 127) / 128;
@@ -555,7 +565,7 @@ static int launch_fa_f32(const float* Q, const float* K, const float* V, float* 
     FTK_HIP(hipFuncSetAttribute((const void*)flash_attn_f32_kernel<D>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
     attr_once.done(attr_bit);
   }
-  hipLaunchKernelGGL(flash_attn_f32_kernel<D>, dim3((unsigned)blocks), dim3(256), lds, s, qp, kp, vp, qinv, bits, O, Sq, Skv, nqb, BH);
+  hipLaunchKernelGGL(flash_attn_f32_kernel<D>, dim3((unsigned)blocks), dim3(256), lds, s, Q, kp, vp, scale * 1.4426950408889634f, bits, O, Sq, Skv, nqb, BH);
   return check_launch("flash_attn_f32_kernel");
 }
 
@@ -563,7 +573,7 @@ static int launch_fa_f32(const float* Q, const float* K, const float* V, float* 
 
 extern "C" size_t ftk_flash_attn_f32_workspace_bytes(int B, int Hd, int Sq, int Skv, int D) {
   if (B <= 0 || Hd <= 0 || Sq <= 0 || Skv <= 0 || D <= 0) return 0;
-  return ftk::f32_layout((long long)B * Hd, Sq, Skv, D).total;
+  return ftk::f32_layout((long long)B * Hd, Skv, D).total;
 }
 
 extern "C" int ftk_flash_attn_f32(const float* Q, const float* K, const float* V, float* O, int B, int Hd, int Sq, int Skv, int D,
@@ -577,7 +587,7 @@ extern "C" int ftk_flash_attn_f32(const float* Q, const float* K, const float* V
   const long long bh = (long long)B * Hd;
   if (bh > (1LL << 16)) return fail(FTK_ERR_UNSUPPORTED_SHAPE, "%s: B*Hd=%lld too large", who, bh);
   if ((long long)Skv * D >= (1LL << 31) || (long long)Sq * D >= (1LL << 31)) return fail(FTK_ERR_UNSUPPORTED_SHAPE, "%s: a head is too large", who);
-  const F32Layout w = f32_layout(bh, Sq, Skv, D);
+  const F32Layout w = f32_layout(bh, Skv, D);
   if (!workspace || workspace_bytes < w.total)
     return fail(FTK_ERR_WORKSPACE, "%s: workspace of %zu bytes needed, %zu given", who, w.total, workspace ? workspace_bytes : (size_t)0);
   if (reinterpret_cast<uintptr_t>(workspace) % 256) return fail(FTK_ERR_INVALID_ARGUMENT, "%s: workspace must be 256-byte aligned", who);

@@ -481,9 +481,10 @@ int ftk_flash_attn_ws_f16(const void* Q, const void* K, const void* V, void* O,
  * a (batch, head) each share a power-of-two scale), the softmax state is fp32:
  * results agree with a float64 evaluation to a few 1e-6 of the largest |O|.
  * Non-finite inputs give NaN.  The workspace (ftk_flash_attn_f32_workspace_bytes,
- * about the size of Q, K and V together, 256-byte aligned) holds the split
- * operands; three small launches precede the attention kernel.  The reference
- * has no device kernel for this program.
+ * about the size of K and V together, 256-byte aligned) holds their split
+ * planes (Q is split in the attention kernel's registers); three small
+ * launches precede the attention kernel.  The reference has no device kernel
+ * for this program.
  */
 size_t ftk_flash_attn_f32_workspace_bytes(int B, int Hd, int Sq, int Skv, int D);
 int ftk_flash_attn_f32(const float* Q, const float* K, const float* V, float* O,
