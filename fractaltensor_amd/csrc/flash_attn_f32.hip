@@ -583,6 +583,8 @@ extern "C" int ftk_flash_attn_f32(const float* Q, const float* K, const float* V
   if (!Q || !K || !V || !O) return fail(FTK_ERR_INVALID_ARGUMENT, "%s: Q, K, V, O must be non-NULL", who);
   if (B <= 0 || Hd <= 0 || Sq <= 0 || Skv <= 0 || D <= 0) return fail(FTK_ERR_INVALID_ARGUMENT, "%s: B, Hd, Sq, Skv, D must be positive", who);
   if (D != 32 && D != 64 && D != 96 && D != 128) return fail(FTK_ERR_UNSUPPORTED_SHAPE, "%s: D=%d must be 32, 64, 96 or 128", who, D);
+  if ((reinterpret_cast<uintptr_t>(Q) | reinterpret_cast<uintptr_t>(K) | reinterpret_cast<uintptr_t>(V) | reinterpret_cast<uintptr_t>(O)) % 16)
+    return fail(FTK_ERR_INVALID_ARGUMENT, "%s: Q, K, V, O must be 16-byte aligned", who);   // rows are read and written 16 bytes at a time
   if (!(scale > 0.0f) || !(scale < INFINITY)) return fail(FTK_ERR_INVALID_ARGUMENT, "%s: scale must be positive and finite", who);
   const long long bh = (long long)B * Hd;
   if (bh > (1LL << 16)) return fail(FTK_ERR_UNSUPPORTED_SHAPE, "%s: B*Hd=%lld too large", who, bh);

@@ -1218,6 +1218,8 @@ static int gemm_f16(const char* who, const void* A, const void* Bm, void* C, int
   if (!A || !Bm || !C) return ftk::fail(FTK_ERR_INVALID_ARGUMENT, "%s: A, B, C must be non-NULL", who);
   if (G <= 0 || M <= 0 || N <= 0 || K <= 0) return ftk::fail(FTK_ERR_INVALID_ARGUMENT, "%s: G, M, N, K must be positive", who);
   if (N % 128 || K % 32) return ftk::fail(FTK_ERR_UNSUPPORTED_SHAPE, "%s: N=%d must be a multiple of 128 and K=%d of 32", who, N, K);
+  if ((reinterpret_cast<uintptr_t>(A) | reinterpret_cast<uintptr_t>(Bm) | reinterpret_cast<uintptr_t>(C)) % 16)
+    return ftk::fail(FTK_ERR_INVALID_ARGUMENT, "%s: A, B, C must be 16-byte aligned", who);   // rows are copied and stored 16 bytes at a time
   // N a multiple of 256: the kernel built for the product (gemm_f16.hip); otherwise the cell kernel without the cell
   if (ftk::gemm_f16_tiles_fit(M, N, K)) return ftk::launch_gemm_f16_tiles(A, Bm, C, G, M, N, K, s);
   if ((long long)M * std::max(K, N) >= (1ll << 30)) return ftk::fail(FTK_ERR_UNSUPPORTED_SHAPE, "%s: M=%d too large", who, M);

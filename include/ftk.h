@@ -14,7 +14,9 @@
  *   - no entry point allocates device memory: kernels that need scratch take
  *     a caller-provided workspace whose size the matching
  *     *_workspace_bytes() function reports;
- *   - matrices are dense row-major with the last index contiguous.
+ *   - matrices are dense row-major with the last index contiguous, and start
+ *     at a 16-byte boundary (every device allocator's do); the entry points
+ *     that say so return FTK_ERR_INVALID_ARGUMENT for one that does not.
  *
  * The reference (microsoft/FractalTensor) has no C ABI of its own: its
  * kernels are compile-time-shaped C++ functors called from gtest/benchmark
@@ -423,7 +425,8 @@ int ftk_b2b_gemm_rowmajor_f16(const void* A, const void* B, const void* C,
 /*
  * C = A @ B, fp16 storage, fp32 accumulation, every operand row-major:
  * A [M,K], B [K,N], C [M,N]; the batched form takes G independent problems
- * A [G,M,K], B [G,K,N], C [G,M,N].  Needs N%128==0, K%32==0.  N%256==0 runs
+ * A [G,M,K], B [G,K,N], C [G,M,N].  Needs N%128==0, K%32==0 and 16-byte
+ * aligned A, B, C.  N%256==0 runs
  * on a kernel built for the product (256 x 256 outputs per workgroup, one wave
  * per SIMD with 128 x 128 of them, k chunks of 32 through four LDS stages, B
  * transposed between LDS and the matrix unit; any M); other widths on the
@@ -480,7 +483,7 @@ int ftk_flash_attn_ws_f16(const void* Q, const void* K, const void* V, void* O,
  * split operands with fp32 accumulation (a row of Q, all of K and all of V of
  * a (batch, head) each share a power-of-two scale), the softmax state is fp32:
  * results agree with a float64 evaluation to a few 1e-6 of the largest |O|.
- * Non-finite inputs give NaN.  The workspace (ftk_flash_attn_f32_workspace_bytes,
+ * Q, K, V, O 16-byte aligned.  Non-finite inputs give NaN.  The workspace (ftk_flash_attn_f32_workspace_bytes,
  * about the size of K and V together, 256-byte aligned) holds their split
  * planes (Q is split in the attention kernel's registers); three small
  * launches precede the attention kernel.  The reference has no device kernel

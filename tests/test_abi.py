@@ -44,11 +44,13 @@ def test_argument_errors_come_back_as_codes_not_crashes():
     assert lib.ftk_b2b_gemm_rowmajor_f16(one, one, one, one, ci(1), ci(64), ci(64), ci(96), ci(128), nul) == -2
     assert lib.ftk_b2b_gemm_rowmajor_f16(one, nul, one, one, ci(1), ci(64), ci(64), ci(64), ci(128), nul) == -1
     assert lib.ftk_gemm_f16(one, one, one, ci(64), ci(96), ci(64), nul) == -2
+    assert lib.ftk_gemm_f16(one, ctypes.c_void_p(18), one, ci(64), ci(256), ci(64), nul) == -1 and b'aligned' in lib.ftk_last_error()
     assert lib.ftk_batched_gemm_f16(one, one, nul, ci(2), ci(64), ci(128), ci(64), nul) == -1
     assert lib.ftk_flash_attn_f16(one, one, one, one, ci(1), ci(1), ci(64), ci(64), ci(48), ctypes.c_float(1), nul) == -2
     cf = ctypes.c_float
     assert lib.ftk_flash_attn_f32(one, nul, one, one, ci(1), ci(1), ci(64), ci(64), ci(64), cf(1), one, ctypes.c_size_t(1 << 30), nul) == -1
     assert lib.ftk_flash_attn_f32(one, one, one, one, ci(1), ci(1), ci(64), ci(64), ci(48), cf(1), one, ctypes.c_size_t(1 << 30), nul) == -2
+    assert lib.ftk_flash_attn_f32(ctypes.c_void_p(20), one, one, one, ci(1), ci(1), ci(64), ci(64), ci(64), cf(1), one, ctypes.c_size_t(1 << 30), nul) == -1
     assert lib.ftk_flash_attn_f32(one, one, one, one, ci(1), ci(1), ci(64), ci(64), ci(64), cf(0), one, ctypes.c_size_t(1 << 30), nul) == -1
     assert lib.ftk_flash_attn_f32(one, one, one, one, ci(1), ci(1), ci(64), ci(64), ci(64), cf(1), nul, ctypes.c_size_t(0), nul) == -3
     assert lib.ftk_flash_attn_f32_workspace_bytes(ci(2), ci(3), ci(100), ci(77), ci(64)) >= 4 * 6 * (2 * 77) * 64   # K's and V's planes
