@@ -348,8 +348,8 @@ def stacked_lstm_check(workspace: Optional[torch.Tensor]) -> None:
 
 def stacked_lstm_small_states(workspace: torch.Tensor) -> bool:
     """Waits for the current stream; True if the last fp32 stacked-LSTM call given this workspace ran on split
-    products and wrote hidden states too small for the fixed scale of their fp16 planes (non-zero |h| below 2^-37
-    at H = 256, 2^-26 at other hidden sizes): such values reach the cells that read them with fewer than 13 bits.
+    products and wrote hidden states too small for the fixed scale of their fp16 planes (four neighbouring units of a
+    row all below 2^-26 and not all zero): such values reach the cells that read them with fewer than 13 bits.
     The whole output is still accurate relative to its largest value; layers that faded that far are not accurate
     relative to themselves.  stacked_lstm(..., exact_small_states=True) repeats such a call on fp32 products."""
     _req_workspace(workspace)

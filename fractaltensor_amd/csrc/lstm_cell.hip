@@ -234,12 +234,14 @@ struct CellDescH {
 struct CellListH {
   int n;
   int packed;  // 1: WU of every cell is in the packed layout; 2, 3: packed split weights (three / two planes per chunk)
-  int* small_states = nullptr;  // split flavour: set to 1 when a non-zero |h| below 2^-26 is written (may be nullptr)
+  int* small_states = nullptr;  // split flavour: set to 1 when four neighbouring units of a row are written whose largest non-zero |h| is below 2^-26 (may be nullptr)
   CellDescH cells[kMaxCellsPerLaunch];
 };
 
 // The split flavour writes h as fp16(h * 2^14) plus the fp16 of what that leaves, unscaled: below h * 2^14 = 2^-12
-// (|h| < 2^-26, 1.5e-8) the two planes hold fewer than 13 bits of a value.
+// (|h| < 2^-26, 1.5e-8) the two planes hold fewer than 13 bits of a value.  One such value among larger ones is exact
+// enough for the sums it enters; what is reported is a lane's four neighbouring units all being that small (and not
+// all zero): a row, or a layer, that has faded.
 constexpr unsigned kSmallStateStreamedBits = (127u - 12u) << 23;
 constexpr int HK = 32;                       // k chunk
 constexpr int HROWS = 256;                   // batch rows per workgroup
@@ -542,15 +544,15 @@ __global__ __launch_bounds__(WAVES * 64, 8 / WAVES) void lstm_cell_f16_kernel(Ce
         *reinterpret_cast<v4f*>(reinterpret_cast<float*>(cd.c) + (size_t)row_g * H + u0) = cn;
         *reinterpret_cast<v4f*>(reinterpret_cast<float*>(cd.h) + (size_t)row_g * H + u0) = hn;
         v4h top, rest;
-        unsigned smallest = 0xffffffffu;
+        unsigned largest = 0;   // of the lane's four neighbouring units
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
           const float hs = hn[r] * 16384.0f;  // |h| < 1: 2^14 keeps the value plane below 2^14
           top[r] = (_Float16)hs;
           rest[r] = (_Float16)(hs - (float)top[r]);
-          smallest = min(smallest, (__float_as_uint(hs) & 0x7fffffffu) - 1u);
+          largest = max(largest, __float_as_uint(hs) & 0x7fffffffu);
         }
-        if (smallest < kSmallStateStreamedBits - 1u && list.small_states) *list.small_states = 1;   // same word, same value: one transaction per wave
+        if (largest - 1u < kSmallStateStreamedBits - 1u && list.small_states) *list.small_states = 1;   // same word, same value: one transaction per wave
         _Float16* hp = cd.h_planes + (size_t)row_g * 2 * H + u0;
         *reinterpret_cast<v4h*>(hp) = top;
         *reinterpret_cast<v4h*>(hp + H) = rest;
@@ -738,7 +740,7 @@ __global__ __launch_bounds__(512, 1) void lstm_cell_split4_kernel(CellListH list
       const v4f sg = *reinterpret_cast<const v4f*>(cd.wscale + 3 * H + u0);
       v4f hn, cn;
       v4h top, rest;
-      unsigned smallest = 0xffffffffu;
+      unsigned largest = 0;   // of the lane's four neighbouring units
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
         const float ig = sigmoid_f(acc[rt][u2][r] * si[r] + bi[r]);
@@ -750,9 +752,9 @@ __global__ __launch_bounds__(512, 1) void lstm_cell_split4_kernel(CellListH list
         const float hs = hn[r] * 16384.0f;
         top[r] = (_Float16)hs;
         rest[r] = (_Float16)(hs - (float)top[r]);
-        smallest = min(smallest, (__float_as_uint(hs) & 0x7fffffffu) - 1u);
+        largest = max(largest, __float_as_uint(hs) & 0x7fffffffu);
       }
-      if (smallest < kSmallStateStreamedBits - 1u && list.small_states) *list.small_states = 1;   // same word, same value: one transaction per wave
+      if (largest - 1u < kSmallStateStreamedBits - 1u && list.small_states) *list.small_states = 1;   // same word, same value: one transaction per wave
       *reinterpret_cast<v4f*>(reinterpret_cast<float*>(cd.c) + (size_t)row_g * H + u0) = cn;
       *reinterpret_cast<v4f*>(reinterpret_cast<float*>(cd.h) + (size_t)row_g * H + u0) = hn;
       _Float16* hp = cd.h_planes + (size_t)row_g * 2 * H + u0;

@@ -74,20 +74,21 @@ constexpr int kMaxBlocks = 64;     // 32-row blocks a ragged batch may have (B <
 // Split products.  v_mfma_f32_32x32x16_f16 moves sixteen k per 8 passes where
 // v_mfma_f32_32x32x2_f32 moves two per 16, so a product of two fp32 numbers is
 // cheaper as three fp16 products than as one fp32 product, if each number is
-// first cut in two: v * 2^e = top + rest / 2^11 with top = fp16(v * 2^e) and
-// rest = fp16((v * 2^e - top) * 2^11).  The cut is exact up to the rounding of
-// rest: 22 significant bits relative to the largest magnitude that shares the
-// scale 2^e (a weight column, an input row, or the fixed 2^14 of h in (-1, 1)),
-// where fp32 keeps 24.  top*top, top*rest and rest*top are accumulated in fp32
-// (the last two in accumulators of their own, folded in with 2^-11 at the end);
-// rest*rest, 2^-22 of the product, is dropped.
+// first cut in two: v * 2^e = top + rest with top = fp16(v * 2^e) and
+// rest = fp16(v * 2^e - top).  The cut is exact up to the rounding of rest: 22
+// significant bits for values within 2^-17 of the largest magnitude that shares
+// the scale 2^e (a weight column, an input row, or the fixed 2^14 of h in
+// (-1, 1)), where fp32 keeps 24, and 2^-40 of that magnitude below (the
+// remainder is then an fp16 subnormal) -- what a sum of products needs.
+// top*top, top*rest and rest*top are accumulated in fp32, in one accumulator
+// where nothing waits for the sum and in two chains where a layer waits for
+// its own results; rest*rest, 2^-22 of the product, is dropped.
 constexpr int kSplitTop = 14;          // a scale group's largest magnitude lands in [2^14, 2^15)
-constexpr float kSplitRest = 2048.0f;  // 2^11: what the remainder is multiplied by before it is rounded
 constexpr float kSplitAct = 16384.0f;  // 2^14: the scale of h
 constexpr int kSplitCommon = 12;       // input rows whose largest magnitude is below 2^(16 - 12) take the scale 2^12
-// h * 2^14 below 2^-23 (|h| < 2^-37, 7e-12): the remainder plane is an fp16 subnormal there and value plus remainder
-// keep fewer than 13 bits
-constexpr unsigned kSmallStateBits = (127u - 23u) << 23;
+// h * 2^14 below 2^-12 (|h| < 2^-26, 1.5e-8): the remainder plane, an fp16 subnormal from 2^-3 down, resolves 2^-24,
+// and value plus remainder keep fewer than 13 bits
+constexpr unsigned kSmallStateBits = (127u - 12u) << 23;
 
 struct PersistArgs {
   const float* xs;
@@ -321,7 +322,7 @@ void lstm_persistent_kernel(PersistArgs a) {
         const float w = wl[(size_t)(16 * s + 8 * hh + e) * PN] * (s < PK / 32 ? xfold * wscale : wscale);
         const _Float16 top = (_Float16)w;
         whi[s][e] = top;
-        wlo[s][e] = (_Float16)((w - (float)top) * kSplitRest);
+        wlo[s][e] = (_Float16)(w - (float)top);
       }
 #pragma unroll
     for (int r = 0; r < 16; ++r) ginv[r] = __shfl(winv, (r & 3) + 8 * (r >> 2) + 4 * hh) * (1.0f / kSplitAct);
@@ -545,7 +546,8 @@ void lstm_persistent_kernel(PersistArgs a) {
     for (int qq = q0; qq < q1; ++qq) {
       v8h btn = bt, brn = br;
       if (qq + 1 < q1) { btn = top_of(qq + 1); brn = rest_of(qq + 1); }
-      // top x top in one accumulator; top x rest and rest x top, both 2^-11 of a product, share the other
+      // top x top in one accumulator; top x rest and rest x top share the other (two chains:
+      // where a layer waits for its own results, an MFMA that adds to the one before it would lengthen the wait)
       am = __builtin_amdgcn_mfma_f32_32x32x16_f16(whi[qq], bt, first && qq == q0 ? zero16 : am, 0, 0, 0);
       ar = __builtin_amdgcn_mfma_f32_32x32x16_f16(whi[qq], br, first && qq == q0 ? zero16 : ar, 0, 0, 0);
       ar = __builtin_amdgcn_mfma_f32_32x32x16_f16(wlo[qq], bt, ar, 0, 0, 0);
@@ -621,7 +623,7 @@ void lstm_persistent_kernel(PersistArgs a) {
     v16f acc;
 #pragma unroll
     for (int r = 0; r < 16; ++r) {
-      if constexpr (SPLIT) acc[r] = esc[r] * (acc0[r] + (1.0f / kSplitRest) * acc1[r]) + ebias[r];
+      if constexpr (SPLIT) acc[r] = esc[r] * (acc0[r] + acc1[r]) + ebias[r];
       else acc[r] = ((r >> 2) == 3 ? 1.0f : -kLog2e) * (acc0[r] + acc1[r]) + ebias[r];
     }
     return acc;
@@ -667,22 +669,24 @@ void lstm_persistent_kernel(PersistArgs a) {
     *reinterpret_cast<float4*>(sb + kStageH + j * kStageRow32 + 4 * c4) = make_float4(hv[0], hv[1], hv[2], hv[3]);
     if constexpr (SPLIT) {
       v4h top, rest;
-      unsigned smallest = 0xffffffffu;  // bit pattern of the smallest non-zero |h * 2^14|, less one (zero wraps to the top)
+      unsigned largest = 0;  // bit pattern of the largest |h * 2^14| of the lane's four neighbouring units
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
         const float v = hv[r] * kSplitAct;
         top[r] = (_Float16)v;
-        rest[r] = (_Float16)((v - (float)top[r]) * kSplitRest);
-        smallest = min(smallest, (__float_as_uint(v) & 0x7fffffffu) - 1u);
+        rest[r] = (_Float16)(v - (float)top[r]);
+        largest = max(largest, __float_as_uint(v) & 0x7fffffffu);
       }
       *reinterpret_cast<v4h*>(sb + kStageTop + j * kStageRow16 + 2 * c4) = top;
       *reinterpret_cast<v4h*>(sb + kStageRest + j * kStageRow16 + 2 * c4) = rest;
-      // the planes have a fixed scale: below kSmallState the two of them hold fewer than 13 bits of a value, and the
-      // cells that read it see it less accurately than 1e-4 of ITS size (the fp32 h and c in hsss / csss are exact
-      // either way).  The status block's second word tells the caller that this happened.
+      // the planes have a fixed scale: below kSmallState the two of them hold fewer than 13 bits of a value.  One such
+      // value beside larger ones is exact enough for the sums it enters (2^-38 in absolute terms); where four
+      // neighbouring units of a row are all that small (and not all zero) the row or the layer has faded, and the cells
+      // that read it see it less accurately than 1e-4 of ITS size (the fp32 h and c in hsss / csss are exact either
+      // way).  The status block's second word tells the caller that this happened.
       // (once per wave: a store per item to one word from every compute unit of a faded layer queues up behind
       // itself, and the wait for an item's stores then waits for it)
-      if (!small_reported && __builtin_amdgcn_ballot_w64(smallest < kSmallStateBits - 1u) != 0) {
+      if (!small_reported && __builtin_amdgcn_ballot_w64(largest - 1u < kSmallStateBits - 1u) != 0) {
         small_reported = true;
         if (lane == 0) __hip_atomic_store(a.status + 1, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       }
@@ -1035,9 +1039,8 @@ void lstm_persistent_kernel(PersistArgs a) {
       // piece carries two chains that do not depend on each other: parts 0..2 hold a sigmoid (gates i, f, o) beside a
       // third of the candidate's tanh, part 3 the tanh of the new c, whose exponential and polynomial are independent.
       float tc_v = 0.f, tc_e = 0.f, tc_x2 = 0.f, tc_p = 0.f, tc_r = 0.f;   // the candidate's tanh between the parts
-      // (split products: the second accumulator holds the cross terms, 2^-11 of a product; fp16 data: the two
-      // accumulators are two chains of the same sum)
-      constexpr float kRestFactor = SPLIT ? 1.0f / kSplitRest : 1.0f;
+      // (split products: one accumulator, em, holds all three products; fp16 data: the two accumulators are two chains
+      // of the same sum)
       auto pair_piece = [&](const v16f& em, const v16f& er, const float4& cp, float (&hv)[4], float (&cv)[4], const float4 sb, auto mc) __attribute__((always_inline)) {
         constexpr int m = decltype(mc)::value;
         constexpr int r = m >> 2, g = m & 3, reg = 4 * g + r;
@@ -1048,10 +1051,10 @@ void lstm_persistent_kernel(PersistArgs a) {
         }
         auto inv1p = [](float e) { return __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(e)); };
         if constexpr (g < 3) {
-          const float v = sb.x * (em[reg] + kRestFactor * er[reg]) + sb.y;
+          const float v = P16 ? sb.x * (em[reg] + er[reg]) + sb.y : sb.x * em[reg] + sb.y;
           if constexpr (g == 0) {
             eg_i = inv1p(v);
-            tc_v = sb.z * (em[12 + r] + kRestFactor * er[12 + r]) + sb.w;
+            tc_v = P16 ? sb.z * (em[12 + r] + er[12 + r]) + sb.w : sb.z * em[12 + r] + sb.w;
             tc_e = fast_exp(2.0f * tc_v);
             tc_x2 = tc_v * tc_v;
           }
@@ -1108,15 +1111,17 @@ void lstm_persistent_kernel(PersistArgs a) {
           if constexpr (sidx + 1 < 16) {
             if constexpr (EPI) nsb = gate_entry(IC<sidx + 1>{});
           }
-          // top x top in one accumulator; top x rest and rest x top, both 2^-11 of a product, share the other
           if constexpr (P16) {   // one product per step, the steps dealt to two accumulation chains
             constexpr bool first2 = hf == 0 && sidx < 2;
             if constexpr ((sidx & 1) == 0) am = __builtin_amdgcn_mfma_f32_32x32x16_f16(wh[P16 ? qq : 0], bt, first2 ? zero16 : am, 0, 0, 0);
             else ar = __builtin_amdgcn_mfma_f32_32x32x16_f16(wh[P16 ? qq : 0], bt, first2 ? zero16 : ar, 0, 0, 0);
           } else {
+            // (all three into one accumulator: the remainder planes are unscaled, and beside the activations of another
+            // block nothing waits for this sum, so a chain of MFMAs that add to one another costs nothing here and saves
+            // the activations a second accumulator to read and fold in)
             am = __builtin_amdgcn_mfma_f32_32x32x16_f16(whi[SPLIT ? qq : 0], bt, first ? zero16 : am, 0, 0, 0);
-            ar = __builtin_amdgcn_mfma_f32_32x32x16_f16(whi[SPLIT ? qq : 0], br, first ? zero16 : ar, 0, 0, 0);
-            ar = __builtin_amdgcn_mfma_f32_32x32x16_f16(wlo[SPLIT ? qq : 0], bt, ar, 0, 0, 0);
+            am = __builtin_amdgcn_mfma_f32_32x32x16_f16(whi[SPLIT ? qq : 0], br, am, 0, 0, 0);
+            am = __builtin_amdgcn_mfma_f32_32x32x16_f16(wlo[SPLIT ? qq : 0], bt, am, 0, 0, 0);
           }
           if constexpr (EPI) {
             pair_piece(em, er, ecp, hv, cv, sb, s_c);
@@ -1435,8 +1440,8 @@ __global__ void fill_zero_kernel(int* p, size_t n) {
 // Split mode, before the persistent kernel: every input row as its two fp16
 // planes, with the row's own power-of-two scale.  One wave per row of 256.
 // Input rows -> their two fp16 planes and the factor that takes their products to h's scale.  A row whose largest
-// magnitude is zero or in [2^-24, 2^4 (1 - 2^-11)] takes the common scale 2^kSplitCommon: its largest element stays
-// finite in fp16 and the planes keep 22 bits of it, as with a scale of the row's own.  Any other row gets a scale of
+// magnitude is zero or in [2^-15, 2^4 (1 - 2^-11)] takes the common scale 2^kSplitCommon: its largest element stays
+// finite in fp16 and the planes keep 22 bits of it (its remainder is no fp16 subnormal), as with a scale of the row's own.  Any other row gets a scale of
 // its own, and *own_scales says that there is one.
 __global__ __launch_bounds__(256) void lstm_split_rows_kernel(const float* xs, _Float16* xsp, float* xratio, int* own_scales, int rows) {
   const int lane = threadIdx.x & 63;
@@ -1447,7 +1452,7 @@ __global__ __launch_bounds__(256) void lstm_split_rows_kernel(const float* xs, _
 #pragma unroll
   for (int o = 32; o > 0; o >>= 1) m = fmaxf(m, __shfl_xor(m, o));
   int eb = min(max((int)((__float_as_uint(m) >> 23) & 0xff), 15), 254);
-  const bool common = m == 0.0f || (m >= 0x1p-24f && m <= 16.0f * (1.0f - 0x1p-11f));
+  const bool common = m == 0.0f || (m >= 0x1p-15f && m <= 16.0f * (1.0f - 0x1p-11f));
   if (common) eb = 127 + kSplitTop - kSplitCommon;   // the exponent whose own scale is the common one
   else if (lane == 0) __hip_atomic_store(own_scales, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   const float scale = __uint_as_float((unsigned)(127 + kSplitTop + 127 - eb) << 23);
@@ -1456,7 +1461,7 @@ __global__ __launch_bounds__(256) void lstm_split_rows_kernel(const float* xs, _
 #pragma unroll
   for (int r = 0; r < 4; ++r) {
     top[r] = (_Float16)vs[r];
-    rest[r] = (_Float16)((vs[r] - (float)top[r]) * kSplitRest);
+    rest[r] = (_Float16)(vs[r] - (float)top[r]);
   }
   _Float16* dst = xsp + (size_t)row * (2 * PH) + 4 * lane;
   *reinterpret_cast<v4h*>(dst) = top;

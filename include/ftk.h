@@ -278,10 +278,12 @@ int ftk_stacked_lstm_status(const void* workspace, ftk_stream_t stream);
  * states too small for them, 0 if not, negative on error.  Split products
  * hand h from cell to cell as two fp16 planes under a fixed scale (|h| < 1):
  * the results are accurate to a few 1e-7 of the LARGEST |h|, but a non-zero
- * |h| below 2^-37 (H = 256; 2^-26 at other hidden sizes) reaches the cells
- * that read it with fewer than 13 bits, and below about 2^-49 (2^-38) as zero.
- * A stack whose upper layers fade towards zero (small weights, no bias: the
- * benchmark configuration) is then exact relative to the whole output and
+ * |h| below 2^-26 reaches the cells that read it with fewer than 13 bits of
+ * its own, and below about 2^-38 as zero.  One such value beside larger ones
+ * is harmless (its error is 2^-38 in absolute terms); reported is a row in
+ * which four neighbouring units are all that small and not all zero.
+ * A stack whose upper layers fade towards zero (small weights, no bias)
+ * is then exact relative to the whole output and
  * inexact relative to those layers; a caller that needs every layer accurate
  * to its own size repeats the call with FTK_LSTM_PRODUCTS_F32 when this
  * returns 1.  No counterpart in the reference (its CuTe stack is fp16
