@@ -1039,8 +1039,8 @@ void lstm_persistent_kernel(PersistArgs a) {
       // piece carries two chains that do not depend on each other: parts 0..2 hold a sigmoid (gates i, f, o) beside a
       // third of the candidate's tanh, part 3 the tanh of the new c, whose exponential and polynomial are independent.
       float tc_v = 0.f, tc_e = 0.f, tc_x2 = 0.f, tc_p = 0.f, tc_r = 0.f;   // the candidate's tanh between the parts
-      // (split products: one accumulator, em, holds all three products; fp16 data: the two accumulators are two chains
-      // of the same sum)
+      // (one accumulator, em, holds a block's sums: all three products of the split mode, the one product of fp16 data;
+      // er is not used by this schedule)
       auto pair_piece = [&](const v16f& em, const v16f& er, const float4& cp, float (&hv)[4], float (&cv)[4], const float4 sb, auto mc) __attribute__((always_inline)) {
         constexpr int m = decltype(mc)::value;
         constexpr int r = m >> 2, g = m & 3, reg = 4 * g + r;
@@ -1051,10 +1051,10 @@ void lstm_persistent_kernel(PersistArgs a) {
         }
         auto inv1p = [](float e) { return __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(e)); };
         if constexpr (g < 3) {
-          const float v = P16 ? sb.x * (em[reg] + er[reg]) + sb.y : sb.x * em[reg] + sb.y;
+          const float v = sb.x * em[reg] + sb.y;
           if constexpr (g == 0) {
             eg_i = inv1p(v);
-            tc_v = P16 ? sb.z * (em[12 + r] + er[12 + r]) + sb.w : sb.z * em[12 + r] + sb.w;
+            tc_v = sb.z * em[12 + r] + sb.w;
             tc_e = fast_exp(2.0f * tc_v);
             tc_x2 = tc_v * tc_v;
           }
@@ -1111,10 +1111,8 @@ void lstm_persistent_kernel(PersistArgs a) {
           if constexpr (sidx + 1 < 16) {
             if constexpr (EPI) nsb = gate_entry(IC<sidx + 1>{});
           }
-          if constexpr (P16) {   // one product per step, the steps dealt to two accumulation chains
-            constexpr bool first2 = hf == 0 && sidx < 2;
-            if constexpr ((sidx & 1) == 0) am = __builtin_amdgcn_mfma_f32_32x32x16_f16(wh[P16 ? qq : 0], bt, first2 ? zero16 : am, 0, 0, 0);
-            else ar = __builtin_amdgcn_mfma_f32_32x32x16_f16(wh[P16 ? qq : 0], bt, first2 ? zero16 : ar, 0, 0, 0);
+          if constexpr (P16) {   // one product per step, all into one accumulator (see below)
+            am = __builtin_amdgcn_mfma_f32_32x32x16_f16(wh[P16 ? qq : 0], bt, first ? zero16 : am, 0, 0, 0);
           } else {
             // (all three into one accumulator: the remainder planes are unscaled, and beside the activations of another
             // block nothing waits for this sum, so a chain of MFMAs that add to one another costs nothing here and saves
