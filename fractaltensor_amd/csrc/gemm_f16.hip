@@ -103,10 +103,6 @@ __global__ __launch_bounds__(256, 1) void gemm_f16_tile_kernel(const _Float16* _
                    :: "s"(lds_wave), "n"(ST * G_STAGE + within), "v"(voff), "s"(base) : "memory", "m0", "scc");
     }
   };
-  auto chunk_copied = [&]() __attribute__((always_inline)) {
-    a_next += GK * 2;
-    b_next += b_chunk;
-  };
 
   // fragment addresses within a stage; and, for stages known to the compiler, within each pair of stages (a read's
   // immediate offset reaches 64 KB: two stages)
@@ -176,46 +172,57 @@ __global__ __launch_bounds__(256, 1) void gemm_f16_tile_kernel(const _Float16* _
   };
 
   // One k step: 16 MFMAs on (af, bf); under them the 12 fragment reads of the step after (stage nst, k step nks)
-  // into (naf, nbf) and, mode 1, the wave's 8 copies of the next chunk to copy into stage cst.
-  auto k_step = [&](v8h (&af)[4], v8h (&bf)[4], auto nst, int nks, v8h (&naf)[4], v8h (&nbf)[4], auto mode_c, auto cst)
+  // into (naf, nbf) and four of the wave's copies into stage cst: SET 1 the A rows of the chunk that a_next points at,
+  // SET 2 the Bm rows of the chunk that b_next points at (0: none).
+  auto k_step = [&](v8h (&af)[4], v8h (&bf)[4], auto nst, int nks, v8h (&naf)[4], v8h (&nbf)[4], auto set_c, auto cst)
                     __attribute__((always_inline)) {
-    constexpr bool COPY = decltype(mode_c)::value == 1;
+    constexpr int SET = decltype(set_c)::value;
     static_for<16>([&](auto s_c) __attribute__((always_inline)) {
       constexpr int s = decltype(s_c)::value;
       constexpr int rt = s >> 2, nt = s & 3;
       if constexpr (s < 12) frag_read(nst, nks, s_c, naf, nbf);
       acc[rt][nt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(bf[nt], af[rt], acc[rt][nt], 0, 0, 0);
-      if constexpr (COPY && s < 12 && s % 3 != 0) copy(cst, GIC<(s - 1 - s / 3)>{});   // steps 1 2 4 5 7 8 10 11
+      if constexpr (SET != 0 && s < 12 && s % 3 == 1) copy(cst, GIC<(4 * (SET - 1) + s / 3)>{});   // steps 1 4 7 10
       if constexpr (s < 12) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
       __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
     });
-    if constexpr (COPY) chunk_copied();
+    if constexpr (SET == 1) a_next += GK * 2;
+    if constexpr (SET == 2) b_next += b_chunk;
     __builtin_amdgcn_sched_barrier(0);   // the step's last MFMAs stay in front of what follows
   };
 
-  // ---- prologue: the first stages on their way, chunk 0 landed, its first k step's fragments read
-  const int ahead = min(GS, nch);
+  // ---- prologue: the first stages on their way, chunk 0 landed, its first k step's fragments read.  A chunk's A rows
+  // are copied half a chunk before its Bm rows (below): of chunk 3 only the A rows are requested here.
+  const int ahead = min(GS - 1, nch);
   for (int c = 0; c < ahead; ++c) {
     static_for<G_COPIES>([&](auto i_c) __attribute__((always_inline)) { copy(c, i_c); });
     a_next += GK * 2;
     b_next += b_chunk;
   }
-  switch (ahead - 1) {
+  if (nch >= GS) {
+    static_for<4>([&](auto i_c) __attribute__((always_inline)) { copy(GS - 1, i_c); });
+    a_next += GK * 2;
+  }
+  switch (ahead - 1) {   // copies issued behind chunk 0's
     case 0: __builtin_amdgcn_s_waitcnt(gemm_vmcnt(0)); break;
     case 1: __builtin_amdgcn_s_waitcnt(gemm_vmcnt(G_COPIES)); break;
-    case 2: __builtin_amdgcn_s_waitcnt(gemm_vmcnt(2 * G_COPIES)); break;
-    default: __builtin_amdgcn_s_waitcnt(gemm_vmcnt(3 * G_COPIES)); break;
+    default:
+      if (nch >= GS) __builtin_amdgcn_s_waitcnt(gemm_vmcnt(2 * G_COPIES + 4));
+      else __builtin_amdgcn_s_waitcnt(gemm_vmcnt(2 * G_COPIES));
+      break;
   }
   __builtin_amdgcn_s_barrier();
   static_for<12>([&](auto n_c) __attribute__((always_inline)) { frag_read(0, 0, n_c, af0, bf0); });
 
-  // chunk ch, in stage `stage` (an int, or a GIC in the loop that is unrolled over the stages)
-  auto chunk = [&](int ch, auto stage, auto nstage, auto mode_c) __attribute__((always_inline)) {
-    constexpr int mode = decltype(mode_c)::value;
-    k_step(af0, bf0, stage, 1, af1, bf1, GIC<0>{}, 0);
+  // chunk ch, in stage `stage` (an int, or a GIC in the loop that is unrolled over the stages); pstage: the stage of
+  // chunk ch - 1.  Beside the first k step the Bm rows of chunk ch + 3 go into pstage (BROWS), beside the second the
+  // A rows of chunk ch + 4 into `stage` (AROWS): eight copies in one k step left the other with issue slots to spare.
+  auto chunk = [&](int ch, auto pstage, auto stage, auto nstage, auto brows_c, auto arows_c) __attribute__((always_inline)) {
+    constexpr bool BROWS = decltype(brows_c)::value, AROWS = decltype(arows_c)::value;
+    k_step(af0, bf0, stage, 1, af1, bf1, GIC<(BROWS ? 2 : 0)>{}, pstage);
     // chunk ch + 1 landed (copies complete in the order of their issue: as many may be outstanding as were issued
-    // behind it); this wave's reads of chunk ch complete
-    if constexpr (mode == 1) {
+    // behind it: the A rows of chunks ch + 2 and ch + 3 and the Bm rows of the same); this wave's reads of chunk ch complete
+    if constexpr (BROWS) {
       __builtin_amdgcn_s_waitcnt(gemm_vmcnt((GS - 2) * G_COPIES) & 0xC07F);   // and lgkmcnt(0)
     } else {
       switch (min(GS - 2, nch - 2 - ch)) {
@@ -225,25 +232,31 @@ __global__ __launch_bounds__(256, 1) void gemm_f16_tile_kernel(const _Float16* _
       }
     }
     __builtin_amdgcn_s_barrier();   // every wave has chunk ch in registers: its stage takes chunk ch + GS
-    k_step(af1, bf1, nstage, 0, af0, bf0, mode_c, stage);
+    k_step(af1, bf1, nstage, 0, af0, bf0, GIC<(AROWS ? 1 : 0)>{}, stage);
   };
   static_assert(GS == 4, "the unrolled loop and the wait counts");
   int ch = 0;
   for (; ch + GS + 3 < nch; ch += 4) {
-    chunk(ch, GIC<0>{}, GIC<1>{}, GIC<1>{});
-    chunk(ch + 1, GIC<1>{}, GIC<2>{}, GIC<1>{});
-    chunk(ch + 2, GIC<2>{}, GIC<3>{}, GIC<1>{});
-    chunk(ch + 3, GIC<3>{}, GIC<0>{}, GIC<1>{});
+    chunk(ch, GIC<3>{}, GIC<0>{}, GIC<1>{}, std::true_type{}, std::true_type{});
+    chunk(ch + 1, GIC<0>{}, GIC<1>{}, GIC<2>{}, std::true_type{}, std::true_type{});
+    chunk(ch + 2, GIC<1>{}, GIC<2>{}, GIC<3>{}, std::true_type{}, std::true_type{});
+    chunk(ch + 3, GIC<2>{}, GIC<3>{}, GIC<0>{}, std::true_type{}, std::true_type{});
   }
   int stage = 0;
   for (; ch + GS < nch; ++ch) {
     const int nstage = (stage + 1) & 3;
-    chunk(ch, stage, nstage, GIC<1>{});
+    chunk(ch, (stage + 3) & 3, stage, nstage, std::true_type{}, std::true_type{});
     stage = nstage;
+  }
+  if (ch + GS - 1 < nch) {   // the last chunk's Bm rows are still to be requested
+    const int nstage = (stage + 1) & 3;
+    chunk(ch, (stage + 3) & 3, stage, nstage, std::true_type{}, std::false_type{});
+    stage = nstage;
+    ++ch;
   }
   for (; ch < nch; ++ch) {
     const int nstage = (stage + 1) & 3;
-    chunk(ch, stage, nstage, GIC<0>{});
+    chunk(ch, (stage + 3) & 3, stage, nstage, std::false_type{}, std::false_type{});
     stage = nstage;
   }
 
