@@ -8,7 +8,8 @@
 // leaves none it can avoid: the fragments of a k step are read while the MFMAs of the step before run, across
 // the chunk boundary as well -- the barrier sits in the MIDDLE of a chunk, between its two k steps, where the
 // second step's fragments are already in registers (the chunk's stage is then free for the copy of chunk
-// ch + 4) and the first step's fragments of the next chunk can be read behind it.
+// ch + 4: its A rows beside the second k step, its Bm rows beside the next chunk's first) and the first step's
+// fragments of the next chunk can be read behind it.
 #include <algorithm>
 
 #include "ftk_common.h"
