@@ -818,10 +818,12 @@ def test_b2b_gemm_rowmajor(core, G, M, N, K, P):
     (0, 768, 1024, 1056),       # many chunks
     (0, 700, 512, 288),         # the tile kernel with a ragged last row block
     (3, 130, 256, 64),          # ... batched, fewer rows than one wave's share of a tile
-    (0, 256, 256, 128),         # as many chunks as stages: the last one's Bm rows are requested in the main loop
-    (0, 512, 256, 224),         # seven chunks: the loop over runtime stages only
-    (0, 256, 512, 256),         # eight: once through the loop unrolled over the stages
-    (0, 300, 256, 352),         # eleven: unrolled loop, runtime-stage loop and tail
+    (0, 256, 256, 128),         # as many chunks as Bm stages
+    (0, 512, 256, 224),         # seven chunks: ends on half a pair of chunks
+    (0, 256, 512, 256),         # eight
+    (0, 300, 256, 352),         # eleven
+    (0, 256, 256, 608),         # nineteen: the fewest that enter the loop unrolled over twelve; ends on half a pair
+    (2, 256, 256, 1280),        # forty: twice through that loop, sixteen behind it
 ])
 def test_gemm_f16(core, G, M, N, K):
     rng = np.random.default_rng(4)
