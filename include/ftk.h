@@ -430,8 +430,9 @@ int ftk_b2b_gemm_rowmajor_f16(const void* A, const void* B, const void* C,
  * A [G,M,K], B [G,K,N], C [G,M,N].  Needs N%128==0, K%32==0 and 16-byte
  * aligned A, B, C.  N%256==0 runs
  * on a kernel built for the product (256 x 256 outputs per workgroup, one wave
- * per SIMD with 128 x 128 of them, k chunks of 32 through four LDS stages, B
- * transposed between LDS and the matrix unit; any M); other widths on the
+ * per SIMD with 128 x 128 of them, k chunks of 32 through all 160 KB of LDS,
+ * A a whole cache line per row at a time, B transposed between LDS and the
+ * matrix unit; any M); other widths on the
  * streaming LSTM cell kernel without the cell.  Stands in for
  * KeCuteGemm / KeBatchedCuteGemm / KeGemmPipelined
  * (kaleido/core/device/kernels/cutlass_wmma.h:116,186,259; functors CuteGemm,
